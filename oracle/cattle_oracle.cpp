@@ -1,0 +1,677 @@
+/*
+ * cattle_oracle.cpp — CPU restatement of C-ATTL3's kernel-layer algorithms.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE. It exists so that the HIP kernels can be checked
+ * against the algorithm of the reference on identical inputs, and so that the benchmark can time
+ * a CPU baseline next to the GPU. Nothing in the product path may link or call it.
+ *
+ * The reference (ViktorC/C-ATTL3) delegates its arithmetic to Eigen, which is an un-vendored git
+ * submodule and is absent; the reference therefore cannot be compiled. Every function below is a
+ * plain-loop restatement of one reference function and cites it (paths relative to the reference
+ * root, C-ATTL3/...). Buffers use the reference's memory layout: column-major tensors whose
+ * index order is (N,H,W,C), so the offset of (n,h,w,c) is n + N*(h + H*(w + W*c))
+ * (core/EigenProxy.hpp:43-64); matrices are column-major as well.
+ *
+ * Parity status of each function (what pins it is in tests/test_oracle_*.py):
+ *   conv/dense fwd+bwd  pinned: 7-loop definitional cross-correlation, torch float64 conv2d,
+ *                       adjoint identities, delta/box kernels, index-ordering probes.
+ *   batch norm          pinned: closed-form invariants + torch float64 batch_norm.
+ *   activations         pinned: libm/numpy closed forms and derivative-at-zero conventions.
+ *   max/mean pool       pinned: brute force incl. crafted ties, NaN/-inf windows, overlaps.
+ * What stays unpinned is only the bit pattern of Eigen's own summation order and of its
+ * vectorised exp/tanh/log, which the reference's tests do not pin either (they hold no golden
+ * vectors: test/gradient_test.cpp, test/training_test.cpp).
+ */
+#include <cmath>
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <vector>
+#include <algorithm>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef long long i64;
+
+namespace {
+
+/* ---------------------------------------------------------------------------------------------
+ * Dense column-major GEMMs. Eigen's product kernels are replaced by cache-blocked loops; the
+ * row-block loop is OpenMP-parallel to mirror Eigen's OpenMP GEMM (Makefile:7, -fopenmp).
+ * ------------------------------------------------------------------------------------------- */
+const i64 ROW_BLOCK = 256;
+
+/* C[M x F] = A[M x K] * B[K x F]  (+ bias[f] broadcast over rows if bias != nullptr) */
+template<typename T>
+void gemm_nn(i64 M, i64 K, i64 F, const T* A, const T* B, const T* bias, T* C) {
+	#pragma omp parallel for schedule(static)
+	for (i64 m0 = 0; m0 < M; m0 += ROW_BLOCK) {
+		const i64 mb = std::min(ROW_BLOCK, M - m0);
+		for (i64 f = 0; f < F; ++f) {
+			T* c = C + m0 + M * f;
+			const T b0 = bias ? bias[f] : (T) 0;
+			for (i64 i = 0; i < mb; ++i)
+				c[i] = 0;
+			for (i64 k = 0; k < K; ++k) {
+				const T w = B[k + K * f];
+				const T* a = A + m0 + M * k;
+				for (i64 i = 0; i < mb; ++i)
+					c[i] += a[i] * w;
+			}
+			if (bias)
+				for (i64 i = 0; i < mb; ++i)
+					c[i] += b0;
+		}
+	}
+}
+
+/* C[K x F] += A^T[K x M] * G[M x F] */
+template<typename T>
+void gemm_tn_acc(i64 M, i64 K, i64 F, const T* A, const T* G, T* C) {
+	std::vector<T> prod((size_t) (K * F), (T) 0);
+	#pragma omp parallel for schedule(static)
+	for (i64 k = 0; k < K; ++k) {
+		for (i64 m0 = 0; m0 < M; m0 += ROW_BLOCK) {
+			const i64 mb = std::min(ROW_BLOCK, M - m0);
+			const T* a = A + m0 + M * k;
+			for (i64 f = 0; f < F; ++f) {
+				const T* g = G + m0 + M * f;
+				T s = 0;
+				for (i64 i = 0; i < mb; ++i)
+					s += a[i] * g[i];
+				prod[(size_t) (k + K * f)] += s;
+			}
+		}
+	}
+	for (i64 i = 0; i < K * F; ++i)
+		C[i] += prod[(size_t) i];
+}
+
+/* D[M x K] = G[M x F] * W^T[F x K], W stored [K x F] */
+template<typename T>
+void gemm_nt(i64 M, i64 K, i64 F, const T* G, const T* W, T* D) {
+	#pragma omp parallel for schedule(static)
+	for (i64 m0 = 0; m0 < M; m0 += ROW_BLOCK) {
+		const i64 mb = std::min(ROW_BLOCK, M - m0);
+		for (i64 k = 0; k < K; ++k) {
+			T* d = D + m0 + M * k;
+			for (i64 i = 0; i < mb; ++i)
+				d[i] = 0;
+			for (i64 f = 0; f < F; ++f) {
+				const T w = W[k + K * f];
+				const T* g = G + m0 + M * f;
+				for (i64 i = 0; i < mb; ++i)
+					d[i] += g[i] * w;
+			}
+		}
+	}
+}
+
+/* colsum: out[f] += sum_m G[m,f]  (Eigen colwise().sum()); pairwise to keep fp32 error small */
+template<typename T>
+T pairwise_sum(const T* v, i64 n) {
+	if (n <= 64) {
+		T s = 0;
+		for (i64 i = 0; i < n; ++i)
+			s += v[i];
+		return s;
+	}
+	const i64 h = n / 2;
+	return pairwise_sum(v, h) + pairwise_sum(v + h, n - h);
+}
+
+template<typename T>
+void colsum_acc(i64 M, i64 F, const T* G, T* out) {
+	for (i64 f = 0; f < F; ++f)
+		out[f] += pairwise_sum(G + M * f, M);
+}
+
+struct ConvGeom {
+	i64 N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh;
+	i64 PH, PW, DRH, DRW, OH, OW, M, K;
+	void derive() {
+		PH = H + 2 * pv;                       /* layer/kernel/ConvKernelLayer.hpp:69 */
+		PW = W + 2 * ph;                       /* :70 */
+		DRH = RH + (RH - 1) * dv;              /* :71 (dilation 0 = dense receptor) */
+		DRW = RW + (RW - 1) * dh;              /* :72 */
+		OH = (H - RH - (RH - 1) * dv + 2 * pv) / sv + 1;   /* :194-197 */
+		OW = (W - RW - (RW - 1) * dh + 2 * ph) / sh + 1;
+		M = N * OH * OW;
+		K = RH * RW * C;
+	}
+};
+
+/* layer/kernel/ConvKernelLayer.hpp:117-118 — zero padding on the H and W ranks only. */
+template<typename T>
+void pad_input(const ConvGeom& g, const T* x, std::vector<T>& xp) {
+	xp.assign((size_t) (g.N * g.PH * g.PW * g.C), (T) 0);
+	for (i64 c = 0; c < g.C; ++c)
+		for (i64 w = 0; w < g.W; ++w)
+			for (i64 h = 0; h < g.H; ++h)
+				std::memcpy(&xp[(size_t) (g.N * ((h + g.pv) + g.PH * ((w + g.ph) + g.PW * c)))],
+						x + g.N * (h + g.H * (w + g.W * c)), sizeof(T) * (size_t) g.N);
+}
+
+/* layer/kernel/ConvKernelLayer.hpp:125-142 — the materialised patch matrix [M x K]; patches are
+ * enumerated with the horizontal offset in the outer loop and the vertical one in the inner loop,
+ * each patch contributes N consecutive rows, and a patch tensor (N,RH,RW,C) viewed as an
+ * N x (RH*RW*C) matrix gives column index rh + RH*(rw + RW*c). */
+template<typename T>
+void im2col(const ConvGeom& g, const T* xp, T* cache) {
+	i64 patch_ind = 0;
+	for (i64 i = 0; i <= g.PW - g.DRW; i += g.sh) {
+		for (i64 j = 0; j <= g.PH - g.DRH; j += g.sv) {
+			for (i64 c = 0; c < g.C; ++c)
+				for (i64 rw = 0; rw < g.RW; ++rw)
+					for (i64 rh = 0; rh < g.RH; ++rh) {
+						const i64 col = rh + g.RH * (rw + g.RW * c);
+						const T* src = xp + g.N * ((j + rh * (g.dv + 1)) +
+								g.PH * ((i + rw * (g.dh + 1)) + g.PW * c));
+						std::memcpy(cache + patch_ind + g.M * col, src, sizeof(T) * (size_t) g.N);
+					}
+			patch_ind += g.N;
+		}
+	}
+}
+
+/* layer/kernel/ConvKernelLayer.hpp:115-148 */
+template<typename T>
+int conv_forward(ConvGeom g, const T* x, const T* w, const T* b, T* out, T* cache) {
+	g.derive();
+	std::vector<T> xp;
+	const T* src = x;
+	if (g.pv > 0 || g.ph > 0) {
+		pad_input(g, x, xp);
+		src = xp.data();
+	}
+	std::vector<T> own;
+	if (!cache) {
+		own.resize((size_t) (g.M * g.K));
+		cache = own.data();
+	}
+	im2col(g, src, cache);
+	gemm_nn(g.M, g.K, g.F, cache, w, b, out);                /* :144-145 */
+	return 0;
+}
+
+/* layer/kernel/ConvKernelLayer.hpp:149-189. wgrad and bgrad accumulate (StandardParameters.hpp:119).
+ * in_grad == nullptr reproduces the input-layer early-out (:156-157). */
+template<typename T>
+int conv_backward(ConvGeom g, const T* cache, const T* w, const T* out_grad, T* wgrad, T* bgrad, T* in_grad) {
+	g.derive();
+	gemm_tn_acc(g.M, g.K, g.F, cache, out_grad, wgrad);       /* :154 */
+	colsum_acc(g.M, g.F, out_grad, bgrad);                    /* :155 */
+	if (!in_grad)
+		return 0;
+	std::vector<T> D((size_t) (g.M * g.K));
+	gemm_nt(g.M, g.K, g.F, out_grad, w, D.data());            /* :159 */
+	std::vector<T> pg((size_t) (g.N * g.PH * g.PW * g.C), (T) 0);   /* :162-163 */
+	i64 patch_ind = 0;
+	for (i64 i = 0; i <= g.PW - g.DRW; i += g.sh) {           /* :166-181, col2im in the same patch order */
+		for (i64 j = 0; j <= g.PH - g.DRH; j += g.sv) {
+			for (i64 c = 0; c < g.C; ++c)
+				for (i64 rw = 0; rw < g.RW; ++rw)
+					for (i64 rh = 0; rh < g.RH; ++rh) {
+						const i64 col = rh + g.RH * (rw + g.RW * c);
+						T* dst = &pg[(size_t) (g.N * ((j + rh * (g.dv + 1)) +
+								g.PH * ((i + rw * (g.dh + 1)) + g.PW * c)))];
+						const T* s = &D[(size_t) (patch_ind + g.M * col)];
+						for (i64 n = 0; n < g.N; ++n)
+							dst[n] += s[n];
+					}
+			patch_ind += g.N;
+		}
+	}
+	for (i64 c = 0; c < g.C; ++c)                               /* :183-188, crop the padding */
+		for (i64 wv = 0; wv < g.W; ++wv)
+			for (i64 h = 0; h < g.H; ++h)
+				std::memcpy(in_grad + g.N * (h + g.H * (wv + g.W * c)),
+						&pg[(size_t) (g.N * ((h + g.pv) + g.PH * ((wv + g.ph) + g.PW * c)))],
+						sizeof(T) * (size_t) g.N);
+	return 0;
+}
+
+/* layer/kernel/DenseKernelLayer.hpp:92-102 */
+template<typename T>
+int dense_forward(i64 N, i64 V, i64 O, const T* x, const T* w, const T* b, T* out) {
+	gemm_nn(N, V, O, x, w, b, out);
+	return 0;
+}
+
+/* layer/kernel/DenseKernelLayer.hpp:103-115 */
+template<typename T>
+int dense_backward(i64 N, i64 V, i64 O, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad, T* in_grad) {
+	gemm_tn_acc(N, V, O, x, out_grad, wgrad);                   /* :108 */
+	colsum_acc(N, O, out_grad, bgrad);                          /* :109 */
+	if (in_grad)
+		gemm_nt(N, V, O, out_grad, w, in_grad);                 /* :113 */
+	return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Batch normalisation.
+ * groups = number of statistics groups, L = elements per group.
+ *   per-channel (layer/BatchNormLayer.hpp:170-262): group i is the contiguous slab
+ *     [i*L, (i+1)*L), L = N*H*W; params are per-channel scalars.
+ *   per-activation (:411-456): group i is column i of the N x vol matrix, L = N; it is the same
+ *     memory pattern (contiguous column), so one routine serves both.
+ * stats_init != 0 means the running statistics already hold values (avgs_init, :234-243).
+ * ------------------------------------------------------------------------------------------- */
+template<typename T>
+int bn_forward(i64 groups, i64 L, const T* x, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd,
+		int stats_init, int training, T decay, T eps, T* out, T* std_cache, T* inv_sd_cache) {
+	std::vector<T> tmp((size_t) L);
+	for (i64 gidx = 0; gidx < groups; ++gidx) {
+		const T* xs = x + gidx * L;
+		T* ys = out + gidx * L;
+		if (training) {
+			const T mean = pairwise_sum(xs, L) / (T) L;                       /* :229 */
+			for (i64 i = 0; i < L; ++i) {
+				const T d = xs[i] - mean;                                     /* :230 */
+				tmp[(size_t) i] = d * d;
+			}
+			const T inv_sd = (T) 1 / std::sqrt(pairwise_sum(tmp.data(), L) / (T) L + eps);   /* :231 */
+			inv_sd_cache[gidx] = inv_sd;
+			T* sc = std_cache + gidx * L;
+			for (i64 i = 0; i < L; ++i)
+				sc[i] = (xs[i] - mean) * inv_sd;                              /* :232 */
+			if (stats_init) {                                                 /* :234-238 */
+				avg_mean[gidx] = ((T) 1 - decay) * avg_mean[gidx] + decay * mean;
+				avg_inv_sd[gidx] = ((T) 1 - decay) * avg_inv_sd[gidx] + decay * inv_sd;
+			} else {                                                          /* :239-243 */
+				avg_mean[gidx] = mean;
+				avg_inv_sd[gidx] = inv_sd;
+			}
+			for (i64 i = 0; i < L; ++i)
+				ys[i] = sc[i] * gamma[gidx] + beta[gidx];                     /* :248 */
+		} else {
+			for (i64 i = 0; i < L; ++i)                                       /* :246, :248 */
+				ys[i] = ((xs[i] - avg_mean[gidx]) * avg_inv_sd[gidx]) * gamma[gidx] + beta[gidx];
+		}
+	}
+	return 0;
+}
+
+/* layer/BatchNormLayer.hpp:250-262 (per-channel) and :441-456 (per-activation). */
+template<typename T>
+int bn_backward(i64 groups, i64 L, const T* out_grad, const T* gamma, const T* std_cache, const T* inv_sd_cache,
+		T* gamma_grad, T* beta_grad, T* in_grad) {
+	std::vector<T> tmp((size_t) L);
+	for (i64 gidx = 0; gidx < groups; ++gidx) {
+		const T* g = out_grad + gidx * L;
+		const T* sc = std_cache + gidx * L;
+		for (i64 i = 0; i < L; ++i)
+			tmp[(size_t) i] = g[i] * sc[i];
+		gamma_grad[gidx] += pairwise_sum(tmp.data(), L);                      /* :252-253 */
+		beta_grad[gidx] += pairwise_sum(g, L);                                /* :254 */
+		if (!in_grad)
+			continue;
+		/* std_in_grad = g * gamma (:256); sums of it and of std_in * std_in_grad (:257-259) */
+		for (i64 i = 0; i < L; ++i)
+			tmp[(size_t) i] = g[i] * gamma[gidx];
+		const T sum_sg = pairwise_sum(tmp.data(), L);
+		std::vector<T> tmp2((size_t) L);
+		for (i64 i = 0; i < L; ++i)
+			tmp2[(size_t) i] = sc[i] * tmp[(size_t) i];
+		const T sum_ssg = pairwise_sum(tmp2.data(), L);
+		const T scale = ((T) 1 / (T) L) * inv_sd_cache[gidx];                 /* :260-261 */
+		T* dx = in_grad + gidx * L;
+		for (i64 i = 0; i < L; ++i)
+			dx[i] = (((T) L * tmp[(size_t) i] - sum_sg) - sc[i] * sum_ssg) * scale;
+	}
+	return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Activations. kind codes are shared with the C-ABI of the HIP library.
+ * fwd produces out and up to two caches exactly as the reference layers keep them.
+ * ------------------------------------------------------------------------------------------- */
+enum ActKind {
+	ACT_IDENTITY = 0, ACT_SCALED = 1, ACT_BINARY_STEP = 2, ACT_SIGMOID = 3, ACT_TANH = 4, ACT_SOFTSIGN = 5,
+	ACT_SOFTPLUS = 6, ACT_RELU = 7, ACT_LEAKY_RELU = 8, ACT_ELU = 9, ACT_SWISH = 10
+};
+
+template<typename T>
+int act_forward(int kind, i64 n, T p, const T* x, T* y) {
+	switch (kind) {
+	case ACT_IDENTITY:      /* layer/activation/IdentityActivationLayer.hpp:37-42 */
+		for (i64 i = 0; i < n; ++i) y[i] = x[i];
+		break;
+	case ACT_SCALED:        /* ScaledActivationLayer.hpp:38-43 */
+		for (i64 i = 0; i < n; ++i) y[i] = x[i] * p;
+		break;
+	case ACT_BINARY_STEP:   /* BinaryStepActivationLayer.hpp:42-47 */
+		for (i64 i = 0; i < n; ++i) y[i] = (T) (x[i] >= 0);
+		break;
+	case ACT_SIGMOID:       /* SigmoidActivationLayer.hpp:38-43 */
+		for (i64 i = 0; i < n; ++i) y[i] = (T) 1 / (std::exp(-x[i]) + (T) 1);
+		break;
+	case ACT_TANH:          /* TanhActivationLayer.hpp:38-43 */
+		for (i64 i = 0; i < n; ++i) y[i] = std::tanh(x[i]);
+		break;
+	case ACT_SOFTSIGN:      /* SoftsignActivationLayer.hpp:39-44 */
+		for (i64 i = 0; i < n; ++i) y[i] = x[i] / ((T) 1 + std::abs(x[i]));
+		break;
+	case ACT_SOFTPLUS:      /* SoftplusActivationLayer.hpp:40-45 (no overflow guard in the reference) */
+		for (i64 i = 0; i < n; ++i) y[i] = std::log(std::exp(x[i]) + (T) 1);
+		break;
+	case ACT_RELU:          /* ReLUActivationLayer.hpp:45-50 */
+		for (i64 i = 0; i < n; ++i) y[i] = std::max(x[i], (T) 0);
+		break;
+	case ACT_LEAKY_RELU:    /* LeakyReLUActivationLayer.hpp:50-55: max(x, alpha*x) */
+		for (i64 i = 0; i < n; ++i) y[i] = std::max(x[i], x[i] * p);
+		break;
+	case ACT_ELU:           /* ELUActivationLayer.hpp:55-64 */
+		for (i64 i = 0; i < n; ++i) y[i] = x[i] >= 0 ? x[i] : p * (std::exp(x[i]) - (T) 1);
+		break;
+	case ACT_SWISH:         /* SwishActivationLayer.hpp:45-51 */
+		for (i64 i = 0; i < n; ++i) y[i] = x[i] * ((T) 1 / (std::exp(-p * x[i]) + (T) 1));
+		break;
+	default:
+		return 1;
+	}
+	return 0;
+}
+
+/* x = forward input, y = forward output (both are given; each kind reads what its reference
+ * layer caches). */
+template<typename T>
+int act_backward(int kind, i64 n, T p, const T* x, const T* y, const T* g, T* dx) {
+	switch (kind) {
+	case ACT_IDENTITY:      /* IdentityActivationLayer.hpp:43-49 */
+		for (i64 i = 0; i < n; ++i) dx[i] = g[i];
+		break;
+	case ACT_SCALED:        /* ScaledActivationLayer.hpp:44-50 */
+		for (i64 i = 0; i < n; ++i) dx[i] = g[i] * p;
+		break;
+	case ACT_BINARY_STEP:   /* BinaryStepActivationLayer.hpp:48-54 */
+		for (i64 i = 0; i < n; ++i) dx[i] = 0;
+		break;
+	case ACT_SIGMOID:       /* SigmoidActivationLayer.hpp:44-50 */
+		for (i64 i = 0; i < n; ++i) dx[i] = (y[i] * ((T) 1 - y[i])) * g[i];
+		break;
+	case ACT_TANH:          /* TanhActivationLayer.hpp:44-50 */
+		for (i64 i = 0; i < n; ++i) dx[i] = ((T) 1 - y[i] * y[i]) * g[i];
+		break;
+	case ACT_SOFTSIGN: {    /* SoftsignActivationLayer.hpp:45-51 */
+		for (i64 i = 0; i < n; ++i) {
+			const T d = (T) 1 + std::abs(x[i]);
+			dx[i] = ((T) 1 / (d * d)) * g[i];
+		}
+		break;
+	}
+	case ACT_SOFTPLUS:      /* SoftplusActivationLayer.hpp:46-52 */
+		for (i64 i = 0; i < n; ++i) dx[i] = ((T) 1 / (std::exp(-x[i]) + (T) 1)) * g[i];
+		break;
+	case ACT_RELU:          /* ReLUActivationLayer.hpp:51-57: derivative 1 at x == 0 */
+		for (i64 i = 0; i < n; ++i) dx[i] = (T) (x[i] >= 0) * g[i];
+		break;
+	case ACT_LEAKY_RELU:    /* LeakyReLUActivationLayer.hpp:56-62 */
+		for (i64 i = 0; i < n; ++i) dx[i] = (x[i] >= 0 ? (T) 1 : p) * g[i];
+		break;
+	case ACT_ELU:           /* ELUActivationLayer.hpp:65-78 */
+		for (i64 i = 0; i < n; ++i) dx[i] = (x[i] >= 0 ? (T) 1 : (y[i] + p)) * g[i];
+		break;
+	case ACT_SWISH: {       /* SwishActivationLayer.hpp:52-59 */
+		for (i64 i = 0; i < n; ++i) {
+			const T s = (T) 1 / (std::exp(-p * x[i]) + (T) 1);
+			dx[i] = s * ((((T) 1 - s) * p) * x[i] + (T) 1) * g[i];
+		}
+		break;
+	}
+	default:
+		return 1;
+	}
+	return 0;
+}
+
+/* layer/activation/SoftmaxActivationLayer.hpp:49-62; rows = samples of the N x V matrix. */
+template<typename T>
+int softmax_forward(i64 N, i64 V, T eps, const T* x, T* y) {
+	for (i64 n = 0; n < N; ++n) {
+		T mx = x[n];
+		for (i64 v = 1; v < V; ++v)
+			mx = std::max(mx, x[n + N * v]);
+		T s = 0;
+		for (i64 v = 0; v < V; ++v) {
+			const T e = std::exp(x[n + N * v] - mx);
+			y[n + N * v] = e;
+			s += e;
+		}
+		for (i64 v = 0; v < V; ++v)
+			y[n + N * v] /= (s + eps);
+	}
+	return 0;
+}
+
+/* SoftmaxActivationLayer.hpp:63-78: dx_row = g_row * (diag(y) - y^T y) */
+template<typename T>
+int softmax_backward(i64 N, i64 V, const T* y, const T* g, T* dx) {
+	for (i64 n = 0; n < N; ++n) {
+		for (i64 j = 0; j < V; ++j) {
+			T s = 0;
+			for (i64 i = 0; i < V; ++i) {
+				const T jac = (i == j ? y[n + N * i] : (T) 0) - y[n + N * i] * y[n + N * j];
+				s += g[n + N * i] * jac;
+			}
+			dx[n + N * j] = s;
+		}
+	}
+	return 0;
+}
+
+/* layer/activation/PReLUActivationLayer.hpp:80-109; alpha is a 1 x V row vector. */
+template<typename T>
+int prelu_forward(i64 N, i64 V, const T* alpha, const T* x, T* y) {
+	for (i64 v = 0; v < V; ++v)
+		for (i64 n = 0; n < N; ++n)
+			y[n + N * v] = std::max(x[n + N * v], x[n + N * v] * alpha[v]);   /* :85 */
+	return 0;
+}
+
+template<typename T>
+int prelu_backward(i64 N, i64 V, const T* alpha, const T* x, const T* g, T* alpha_grad, T* dx) {
+	for (i64 v = 0; v < V; ++v) {
+		T ag = 0;
+		for (i64 n = 0; n < N; ++n) {
+			const T xi = x[n + N * v], gi = g[n + N * v];
+			if (xi >= 0) {
+				if (dx) dx[n + N * v] = gi;
+			} else {
+				if (dx) dx[n + N * v] = alpha[v] * gi;
+				ag += xi * gi;                                                /* :102 */
+			}
+		}
+		alpha_grad[v] += ag;
+	}
+	return 0;
+}
+
+/* layer/activation/PSwishActivationLayer.hpp:77-99; beta is a 1 x V row vector. */
+template<typename T>
+int pswish_forward(i64 N, i64 V, const T* beta, const T* x, T* y) {
+	for (i64 v = 0; v < V; ++v)
+		for (i64 n = 0; n < N; ++n) {
+			const T xi = x[n + N * v];
+			y[n + N * v] = xi * ((T) 1 / (std::exp(xi * (-beta[v])) + (T) 1));
+		}
+	return 0;
+}
+
+template<typename T>
+int pswish_backward(i64 N, i64 V, const T* beta, const T* x, const T* g, T* beta_grad, T* dx) {
+	std::vector<T> col((size_t) N);
+	for (i64 v = 0; v < V; ++v) {
+		for (i64 n = 0; n < N; ++n) {
+			const T xi = x[n + N * v], gi = g[n + N * v];
+			const T s = (T) 1 / (std::exp(xi * (-beta[v])) + (T) 1);
+			col[(size_t) n] = s * ((T) 1 - s) * xi * xi * gi;                /* :90-91 */
+			if (dx)
+				dx[n + N * v] = s * ((((T) 1 - s) * beta[v]) * xi + (T) 1) * gi;   /* :94-96 */
+		}
+		beta_grad[v] += pairwise_sum(col.data(), N);
+	}
+	return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Pooling. layer/PoolLayer.hpp:77-116 drives windows with the horizontal offset outer and the
+ * vertical one inner; there is no padding or dilation and windows that do not fit are dropped.
+ * ------------------------------------------------------------------------------------------- */
+struct PoolGeom {
+	i64 N, H, W, C, RH, RW, sv, sh, OH, OW;
+	void derive() {
+		OH = (H - RH) / sv + 1;               /* layer/PoolLayer.hpp:145-148 */
+		OW = (W - RW) / sh + 1;
+	}
+};
+
+/* layer/pool/MaxPoolLayer.hpp:38-64. inds has OH*OW rows of C*N entries: inds[patch][c*N + n] with
+ * patch = ow_idx*OH + oh_idx; value = w_in_window*RH + h_in_window. */
+template<typename T>
+int maxpool_forward(PoolGeom g, const T* x, T* out, unsigned* inds) {
+	g.derive();
+	i64 patch = 0;
+	for (i64 ow = 0; ow < g.OW; ++ow)
+		for (i64 oh = 0; oh < g.OH; ++oh, ++patch)
+			for (i64 c = 0; c < g.C; ++c)
+				for (i64 n = 0; n < g.N; ++n) {
+					T mx = std::numeric_limits<T>::lowest();      /* core/NumericUtils.hpp:26 */
+					unsigned mh = 0, mw = 0;
+					for (i64 k = 0; k < g.RW; ++k)
+						for (i64 l = 0; l < g.RH; ++l) {
+							const T v = x[n + g.N * ((oh * g.sv + l) + g.H * ((ow * g.sh + k) + g.W * c))];
+							if (v > mx) {
+								mx = v;
+								mh = (unsigned) l;
+								mw = (unsigned) k;
+							}
+						}
+					inds[patch * (g.C * g.N) + c * g.N + n] = mw * (unsigned) g.RH + mh;
+					out[n + g.N * (oh + g.OH * (ow + g.OW * c))] = mx;
+				}
+	return 0;
+}
+
+/* layer/pool/MaxPoolLayer.hpp:65-80 + layer/PoolLayer.hpp:96-116 (accumulation over overlaps). */
+template<typename T>
+int maxpool_backward(PoolGeom g, const T* out_grad, const unsigned* inds, T* in_grad) {
+	g.derive();
+	std::fill(in_grad, in_grad + g.N * g.H * g.W * g.C, (T) 0);
+	i64 patch = 0;
+	for (i64 ow = 0; ow < g.OW; ++ow)
+		for (i64 oh = 0; oh < g.OH; ++oh, ++patch)
+			for (i64 c = 0; c < g.C; ++c)
+				for (i64 n = 0; n < g.N; ++n) {
+					const unsigned ind = inds[patch * (g.C * g.N) + c * g.N + n];
+					const i64 mh = ind % (unsigned) g.RH, mw = ind / (unsigned) g.RH;
+					in_grad[n + g.N * ((oh * g.sv + mh) + g.H * ((ow * g.sh + mw) + g.W * c))] +=
+							out_grad[n + g.N * (oh + g.OH * (ow + g.OW * c))];
+				}
+	return 0;
+}
+
+/* layer/pool/MeanPoolLayer.hpp:35-38 */
+template<typename T>
+int meanpool_forward(PoolGeom g, const T* x, T* out) {
+	g.derive();
+	for (i64 c = 0; c < g.C; ++c)
+		for (i64 ow = 0; ow < g.OW; ++ow)
+			for (i64 oh = 0; oh < g.OH; ++oh)
+				for (i64 n = 0; n < g.N; ++n) {
+					T s = 0;
+					for (i64 k = 0; k < g.RW; ++k)
+						for (i64 l = 0; l < g.RH; ++l)
+							s += x[n + g.N * ((oh * g.sv + l) + g.H * ((ow * g.sh + k) + g.W * c))];
+					out[n + g.N * (oh + g.OH * (ow + g.OW * c))] = s / (T) (g.RH * g.RW);
+				}
+	return 0;
+}
+
+/* layer/pool/MeanPoolLayer.hpp:39-41 + layer/PoolLayer.hpp:96-116 */
+template<typename T>
+int meanpool_backward(PoolGeom g, const T* out_grad, T* in_grad) {
+	g.derive();
+	std::fill(in_grad, in_grad + g.N * g.H * g.W * g.C, (T) 0);
+	const T area = (T) (g.RH * g.RW);
+	for (i64 ow = 0; ow < g.OW; ++ow)
+		for (i64 oh = 0; oh < g.OH; ++oh)
+			for (i64 c = 0; c < g.C; ++c)
+				for (i64 k = 0; k < g.RW; ++k)
+					for (i64 l = 0; l < g.RH; ++l)
+						for (i64 n = 0; n < g.N; ++n)
+							in_grad[n + g.N * ((oh * g.sv + l) + g.H * ((ow * g.sh + k) + g.W * c))] +=
+									out_grad[n + g.N * (oh + g.OH * (ow + g.OW * c))] / area;
+	return 0;
+}
+
+} /* namespace */
+
+#define CONV_ARGS i64 N, i64 H, i64 W, i64 C, i64 F, i64 RH, i64 RW, i64 pv, i64 ph, i64 sv, i64 sh, i64 dv, i64 dh
+#define CONV_GEOM ConvGeom g = { N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh, 0, 0, 0, 0, 0, 0, 0, 0 }
+#define POOL_ARGS i64 N, i64 H, i64 W, i64 C, i64 RH, i64 RW, i64 sv, i64 sh
+#define POOL_GEOM PoolGeom g = { N, H, W, C, RH, RW, sv, sh, 0, 0 }
+
+#define ORACLE_INSTANTIATE(T, SFX) \
+extern "C" int oracle_conv_forward_##SFX(CONV_ARGS, const T* x, const T* w, const T* b, T* out, T* cache) { \
+	CONV_GEOM; return conv_forward<T>(g, x, w, b, out, cache); } \
+extern "C" int oracle_conv_backward_##SFX(CONV_ARGS, const T* cache, const T* w, const T* out_grad, T* wgrad, \
+		T* bgrad, T* in_grad) { CONV_GEOM; return conv_backward<T>(g, cache, w, out_grad, wgrad, bgrad, in_grad); } \
+extern "C" int oracle_dense_forward_##SFX(i64 N, i64 V, i64 O, const T* x, const T* w, const T* b, T* out) { \
+	return dense_forward<T>(N, V, O, x, w, b, out); } \
+extern "C" int oracle_dense_backward_##SFX(i64 N, i64 V, i64 O, const T* x, const T* w, const T* out_grad, \
+		T* wgrad, T* bgrad, T* in_grad) { return dense_backward<T>(N, V, O, x, w, out_grad, wgrad, bgrad, in_grad); } \
+extern "C" int oracle_bn_forward_##SFX(i64 groups, i64 L, const T* x, const T* gamma, const T* beta, T* avg_mean, \
+		T* avg_inv_sd, int stats_init, int training, double decay, double eps, T* out, T* std_cache, T* inv_sd_cache) { \
+	return bn_forward<T>(groups, L, x, gamma, beta, avg_mean, avg_inv_sd, stats_init, training, (T) decay, (T) eps, \
+			out, std_cache, inv_sd_cache); } \
+extern "C" int oracle_bn_backward_##SFX(i64 groups, i64 L, const T* out_grad, const T* gamma, const T* std_cache, \
+		const T* inv_sd_cache, T* gamma_grad, T* beta_grad, T* in_grad) { \
+	return bn_backward<T>(groups, L, out_grad, gamma, std_cache, inv_sd_cache, gamma_grad, beta_grad, in_grad); } \
+extern "C" int oracle_act_forward_##SFX(int kind, i64 n, double p, const T* x, T* y) { \
+	return act_forward<T>(kind, n, (T) p, x, y); } \
+extern "C" int oracle_act_backward_##SFX(int kind, i64 n, double p, const T* x, const T* y, const T* g, T* dx) { \
+	return act_backward<T>(kind, n, (T) p, x, y, g, dx); } \
+extern "C" int oracle_softmax_forward_##SFX(i64 N, i64 V, double eps, const T* x, T* y) { \
+	return softmax_forward<T>(N, V, (T) eps, x, y); } \
+extern "C" int oracle_softmax_backward_##SFX(i64 N, i64 V, const T* y, const T* g, T* dx) { \
+	return softmax_backward<T>(N, V, y, g, dx); } \
+extern "C" int oracle_prelu_forward_##SFX(i64 N, i64 V, const T* alpha, const T* x, T* y) { \
+	return prelu_forward<T>(N, V, alpha, x, y); } \
+extern "C" int oracle_prelu_backward_##SFX(i64 N, i64 V, const T* alpha, const T* x, const T* g, T* ag, T* dx) { \
+	return prelu_backward<T>(N, V, alpha, x, g, ag, dx); } \
+extern "C" int oracle_pswish_forward_##SFX(i64 N, i64 V, const T* beta, const T* x, T* y) { \
+	return pswish_forward<T>(N, V, beta, x, y); } \
+extern "C" int oracle_pswish_backward_##SFX(i64 N, i64 V, const T* beta, const T* x, const T* g, T* bg, T* dx) { \
+	return pswish_backward<T>(N, V, beta, x, g, bg, dx); } \
+extern "C" int oracle_maxpool_forward_##SFX(POOL_ARGS, const T* x, T* out, unsigned* inds) { \
+	POOL_GEOM; return maxpool_forward<T>(g, x, out, inds); } \
+extern "C" int oracle_maxpool_backward_##SFX(POOL_ARGS, const T* out_grad, const unsigned* inds, T* in_grad) { \
+	POOL_GEOM; return maxpool_backward<T>(g, out_grad, inds, in_grad); } \
+extern "C" int oracle_meanpool_forward_##SFX(POOL_ARGS, const T* x, T* out) { \
+	POOL_GEOM; return meanpool_forward<T>(g, x, out); } \
+extern "C" int oracle_meanpool_backward_##SFX(POOL_ARGS, const T* out_grad, T* in_grad) { \
+	POOL_GEOM; return meanpool_backward<T>(g, out_grad, in_grad); }
+
+ORACLE_INSTANTIATE(float, f32)
+ORACLE_INSTANTIATE(double, f64)
+
+extern "C" int oracle_num_threads(void) {
+#ifdef _OPENMP
+	return omp_get_max_threads();
+#else
+	return 1;
+#endif
+}
+
+extern "C" void oracle_set_num_threads(int n) {
+#ifdef _OPENMP
+	/* core/EigenProxy.hpp:102-105 clamps the requested count to [1, hardware concurrency]. */
+	const int hw = omp_get_num_procs();
+	omp_set_num_threads(n < 1 ? 1 : (n > hw ? hw : n));
+#else
+	(void) n;
+#endif
+}

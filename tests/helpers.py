@@ -1,0 +1,96 @@
+"""Shared test helpers: seeded inputs in the reference's memory layout, the error metric, and
+definitional (brute-force) versions of the layer maths used to pin the oracle."""
+import numpy as np
+
+# Conv geometries exercised by the reference's own gradient tests (test/gradient_test.cpp:166-185),
+# re-viewed as 4-D (H,W,C) problems the way ConvKernelLayer<Scalar,1|2> does
+# (layer/kernel/ConvKernelLayer.hpp:400-417, :494-508), plus the BASELINE-style 3x3 p1 case.
+#   (H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh)
+REFERENCE_CONV_CASES = [
+    (32, 1, 1, 5, 3, 1, 2, 0, 1, 1, 1, 0),    # rank 1: length 32, k3 p2 s1 d1
+    (30, 1, 5, 1, 3, 1, 1, 0, 1, 1, 0, 0),    # rank 1 second layer (as C=5 re-view)
+    (10, 10, 1, 5, 3, 2, 1, 2, 1, 2, 1, 0),   # rank 2: 3x2 receptor, pad (1,2), stride (1,2), dilation (1,0)
+    (8, 8, 2, 5, 3, 2, 1, 2, 1, 2, 1, 0),     # rank 3: same on 8x8x2
+    (6, 6, 5, 1, 2, 2, 1, 1, 1, 1, 0, 0),     # second layer: 2x2 p1 s1
+    (7, 6, 3, 4, 3, 3, 1, 1, 1, 1, 0, 0),     # BASELINE-style 3x3 p1 s1
+    (9, 11, 2, 3, 2, 3, 0, 1, 2, 3, 0, 1),    # strides (2,3), dilation (0,1), no vertical padding
+]
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def uniform(gen, shape, lo, hi, dtype):
+    return np.asfortranarray(gen.uniform(lo, hi, size=shape).astype(dtype))
+
+
+def normal(gen, shape, dtype, std=1.0):
+    return np.asfortranarray((gen.standard_normal(size=shape) * std).astype(dtype))
+
+
+def rel_err(a, b, floor_frac=0.1):
+    """max_i |a_i - b_i| / max(|b_i|, floor), floor = floor_frac * RMS(b) (tiny if b is all zero).
+
+    The absolute floor keeps the relative error meaningful for elements that are (near) zero by
+    cancellation: they are compared relative to a tenth of the tensor's RMS instead."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    if a.size == 0:
+        return 0.0
+    rms = float(np.sqrt(np.mean(b * b)))
+    floor = max(floor_frac * rms, 1e-30)
+    return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), floor)))
+
+
+def conv_dims(H, W, RH, RW, pv, ph, sv, sh, dv, dh):
+    OH = (H - RH - (RH - 1) * dv + 2 * pv) // sv + 1
+    OW = (W - RW - (RW - 1) * dh + 2 * ph) // sh + 1
+    return OH, OW
+
+
+def brute_conv_forward(x, w, b, RH, RW, pv, ph, sv, sh, dv, dh):
+    """Definitional cross-correlation in float64: the seven nested loops, no matrices."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(w, dtype=np.float64)
+    N, H, W, C = x.shape
+    F = w.shape[1]
+    OH, OW = conv_dims(H, W, RH, RW, pv, ph, sv, sh, dv, dh)
+    out = np.zeros((N, OH, OW, F))
+    for n in range(N):
+        for oh in range(OH):
+            for ow in range(OW):
+                for f in range(F):
+                    s = float(np.reshape(b, (-1,))[f])
+                    for c in range(C):
+                        for rw in range(RW):
+                            for rh in range(RH):
+                                h = oh * sv + rh * (dv + 1) - pv
+                                ww = ow * sh + rw * (dh + 1) - ph
+                                if 0 <= h < H and 0 <= ww < W:
+                                    s += x[n, h, ww, c] * w[rh + RH * (rw + RW * c), f]
+                    out[n, oh, ow, f] = s
+    return out
+
+
+def brute_maxpool(x, RH, RW, sv, sh):
+    x = np.asarray(x)
+    N, H, W, C = x.shape
+    OH, OW = (H - RH) // sv + 1, (W - RW) // sh + 1
+    out = np.empty((N, OH, OW, C), dtype=x.dtype)
+    inds = np.empty((OH * OW, C * N), dtype=np.uint32)
+    lowest = np.finfo(x.dtype).min
+    for ow in range(OW):
+        for oh in range(OH):
+            for c in range(C):
+                for n in range(N):
+                    best, bi = lowest, 0
+                    for k in range(RW):
+                        for l in range(RH):
+                            v = x[n, oh * sv + l, ow * sh + k, c]
+                            if v > best:
+                                best, bi = v, k * RH + l
+                    out[n, oh, ow, c] = best
+                    inds[ow * OH + oh, c * N + n] = bi
+    return out, inds
