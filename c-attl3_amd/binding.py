@@ -1,0 +1,405 @@
+"""ctypes binding of libcattle_hip.so plus thin layer classes that mirror cattle::Layer.
+
+The classes carry the reference's names and method names (pass_forward, pass_back, get_params,
+set_input_layer, empty_cache, clone, clone_with_shared_params: core/Layer.hpp:47-137) so that tests
+read like the reference's. Host tensors are numpy arrays of shape (N,H,W,C) in Fortran order, i.e.
+the reference's column-major Eigen buffers; DeviceTensor keeps a tensor resident in HBM between
+layers. There is no host fallback: without the built library or without an MI355X every call raises.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcattle_hip.so")
+
+F32, F64 = 0, 1
+HOST, DEVICE = 0, 1
+POOL_MAX, POOL_MEAN = 0, 1
+ACT = {
+    "identity": 0, "scaled": 1, "binary_step": 2, "sigmoid": 3, "tanh": 4, "softsign": 5, "softplus": 6,
+    "relu": 7, "leaky_relu": 8, "elu": 9, "swish": 10, "softmax": 11, "prelu": 12, "pswish": 13,
+}
+
+# every symbol include/cattle_hip.h declares
+EXPORTS = [
+    "cattle_hip_init", "cattle_hip_last_error", "cattle_hip_synchronize", "cattle_hip_alloc", "cattle_hip_free",
+    "cattle_hip_upload", "cattle_hip_download", "cattle_hip_fill_zero", "cattle_hip_timer_create",
+    "cattle_hip_timer_destroy", "cattle_hip_timer_start", "cattle_hip_timer_stop", "cattle_hip_conv_create",
+    "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
+    "cattle_hip_batchnorm_set_stats_initialized", "cattle_hip_activation_create", "cattle_hip_pool_create",
+    "cattle_hip_layer_clone", "cattle_hip_layer_destroy", "cattle_hip_layer_input_dims",
+    "cattle_hip_layer_output_dims", "cattle_hip_layer_is_input_layer", "cattle_hip_layer_set_input_layer",
+    "cattle_hip_layer_empty_cache", "cattle_hip_layer_forward", "cattle_hip_layer_backward",
+    "cattle_hip_layer_num_params", "cattle_hip_layer_param_shape", "cattle_hip_layer_set_param_values",
+    "cattle_hip_layer_get_param_values", "cattle_hip_layer_get_param_grad", "cattle_hip_layer_reset_param_grad",
+    "cattle_hip_maxpool_indices",
+]
+
+
+class CattleHipError(RuntimeError):
+    def __init__(self, code, message):
+        RuntimeError.__init__(self, "cattle_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+def build():
+    """Compile libcattle_hip.so for gfx950 with the package Makefile (hipcc cross-compiles)."""
+    subprocess.check_call(["make", "-s", "-j4", "-C", _HERE])
+
+
+_lib = None
+
+
+def lib():
+    """Loads the built library; raises if it has not been built (there is no other code path)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise CattleHipError(-1, "libcattle_hip.so is not built: run __graft_entry__.build() or make -C c-attl3_amd")
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.cattle_hip_last_error.restype = ctypes.c_char_p
+        for name in EXPORTS:
+            if name != "cattle_hip_last_error":
+                getattr(_lib, name).restype = ctypes.c_int
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise CattleHipError(rc, lib().cattle_hip_last_error().decode("utf-8", "replace"))
+
+
+def init(device=0):
+    _check(lib().cattle_hip_init(ctypes.c_int(device)))
+
+
+def synchronize():
+    _check(lib().cattle_hip_synchronize())
+
+
+def _dtype_code(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return F32
+    if dtype == np.float64:
+        return F64
+    raise TypeError("Scalar must be float32 or float64")
+
+
+def _sz(v):
+    return ctypes.c_size_t(int(v))
+
+
+class DeviceTensor(object):
+    """A tensor resident in device memory, in the reference's column-major layout."""
+
+    def __init__(self, shape, dtype):
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape)) * self.dtype.itemsize
+        p = ctypes.c_void_p()
+        _check(lib().cattle_hip_alloc(ctypes.byref(p), _sz(self.nbytes)))
+        self.ptr = p
+
+    @staticmethod
+    def from_host(a):
+        a = np.asfortranarray(a)
+        t = DeviceTensor(a.shape, a.dtype)
+        _check(lib().cattle_hip_upload(t.ptr, ctypes.c_void_p(a.ctypes.data), _sz(t.nbytes)))
+        return t
+
+    def to_host(self):
+        a = np.empty(self.shape, dtype=self.dtype, order="F")
+        _check(lib().cattle_hip_download(ctypes.c_void_p(a.ctypes.data), self.ptr, _sz(self.nbytes)))
+        return a
+
+    def free(self):
+        if self.ptr is not None and self.ptr.value:
+            _check(lib().cattle_hip_free(self.ptr))
+        self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Timer(object):
+    def __init__(self):
+        self.h = ctypes.c_void_p()
+        _check(lib().cattle_hip_timer_create(ctypes.byref(self.h)))
+
+    def start(self):
+        _check(lib().cattle_hip_timer_start(self.h))
+
+    def stop(self):
+        ms = ctypes.c_float()
+        _check(lib().cattle_hip_timer_stop(self.h, ctypes.byref(ms)))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            lib().cattle_hip_timer_destroy(self.h)
+        except Exception:
+            pass
+
+
+class Parameters(object):
+    """View of one parameter matrix of a layer (core/Parameters.hpp:15-95)."""
+
+    def __init__(self, layer, index):
+        self._layer, self._index = layer, index
+        r, c, o = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_int()
+        _check(lib().cattle_hip_layer_param_shape(layer._h, _sz(index), ctypes.byref(r), ctypes.byref(c), ctypes.byref(o)))
+        self._rows, self._cols, self._opt = int(r.value), int(c.value), bool(o.value)
+
+    def get_rows(self):
+        return self._rows
+
+    def get_cols(self):
+        return self._cols
+
+    def are_optimizable(self):
+        return self._opt
+
+    def get_values(self):
+        a = np.empty((self._rows, self._cols), dtype=self._layer.dtype, order="F")
+        _check(lib().cattle_hip_layer_get_param_values(self._layer._h, _sz(self._index), ctypes.c_void_p(a.ctypes.data), HOST))
+        return a
+
+    def set_values(self, values):
+        a = np.asfortranarray(values, dtype=self._layer.dtype)
+        if a.shape != (self._rows, self._cols):
+            raise ValueError("expected a %dx%d matrix" % (self._rows, self._cols))
+        _check(lib().cattle_hip_layer_set_param_values(self._layer._h, _sz(self._index), ctypes.c_void_p(a.ctypes.data), HOST))
+
+    def get_grad(self):
+        a = np.empty((self._rows, self._cols), dtype=self._layer.dtype, order="F")
+        _check(lib().cattle_hip_layer_get_param_grad(self._layer._h, _sz(self._index), ctypes.c_void_p(a.ctypes.data), HOST))
+        return a
+
+    def reset_grad(self):
+        _check(lib().cattle_hip_layer_reset_param_grad(self._layer._h, _sz(self._index)))
+
+
+class Layer(object):
+    """Base of the layer mirrors; subclasses create the handle."""
+
+    def __init__(self, handle, dtype, in_shape, out_shape):
+        self._h = handle
+        self.dtype = np.dtype(dtype)
+        self._in_shape = tuple(in_shape)        # per-sample shapes as the caller sees them
+        self._out_shape = tuple(out_shape)
+
+    # -- cattle::Layer ------------------------------------------------------------------------
+    def get_input_dims(self):
+        return self._in_shape
+
+    def get_output_dims(self):
+        return self._out_shape
+
+    def is_input_layer(self):
+        v = ctypes.c_int()
+        _check(lib().cattle_hip_layer_is_input_layer(self._h, ctypes.byref(v)))
+        return bool(v.value)
+
+    def set_input_layer(self, flag):
+        _check(lib().cattle_hip_layer_set_input_layer(self._h, ctypes.c_int(int(bool(flag)))))
+
+    def empty_cache(self):
+        _check(lib().cattle_hip_layer_empty_cache(self._h))
+
+    def get_params(self):
+        n = ctypes.c_size_t()
+        _check(lib().cattle_hip_layer_num_params(self._h, ctypes.byref(n)))
+        return [Parameters(self, i) for i in range(int(n.value))]
+
+    def _clone(self, share):
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_layer_clone(self._h, ctypes.c_int(int(share)), ctypes.byref(h)))
+        c = object.__new__(type(self))
+        c.__dict__.update(self.__dict__)
+        c._h = h
+        return c
+
+    def clone(self):
+        return self._clone(False)
+
+    def clone_with_shared_params(self):
+        return self._clone(True)
+
+    def pass_forward(self, x, training):
+        """x: numpy array (host path, returns numpy) or DeviceTensor (device path, returns DeviceTensor)."""
+        if isinstance(x, DeviceTensor):
+            batch = x.shape[0]
+            self._expect(x.shape[1:], self._in_shape, "input")
+            out = DeviceTensor((batch,) + self._out_shape, self.dtype)
+            _check(lib().cattle_hip_layer_forward(self._h, x.ptr, DEVICE, _sz(batch), ctypes.c_int(int(training)), out.ptr, DEVICE))
+            self._keep = (x, out)                 # borrowed by the layer until pass_back
+            return out
+        x = np.asfortranarray(x, dtype=self.dtype)
+        batch = x.shape[0]
+        self._expect(x.shape[1:], self._in_shape, "input")
+        out = np.empty((batch,) + self._out_shape, dtype=self.dtype, order="F")
+        _check(lib().cattle_hip_layer_forward(self._h, ctypes.c_void_p(x.ctypes.data), HOST, _sz(batch),
+                                              ctypes.c_int(int(training)), ctypes.c_void_p(out.ctypes.data), HOST))
+        return out
+
+    def pass_back(self, out_grad):
+        """Returns the input gradient, or None for an input layer (the reference's null tensor)."""
+        skip = self.is_input_layer() and not getattr(self, "_always_backprop", False)
+        if isinstance(out_grad, DeviceTensor):
+            batch = out_grad.shape[0]
+            self._expect(out_grad.shape[1:], self._out_shape, "output gradient")
+            dx = None if skip else DeviceTensor((batch,) + self._in_shape, self.dtype)
+            _check(lib().cattle_hip_layer_backward(self._h, out_grad.ptr, DEVICE, _sz(batch), None if skip else dx.ptr, DEVICE))
+            return dx
+        g = np.asfortranarray(out_grad, dtype=self.dtype)
+        batch = g.shape[0]
+        self._expect(g.shape[1:], self._out_shape, "output gradient")
+        dx = None if skip else np.empty((batch,) + self._in_shape, dtype=self.dtype, order="F")
+        _check(lib().cattle_hip_layer_backward(self._h, ctypes.c_void_p(g.ctypes.data), HOST, _sz(batch),
+                                               None if skip else ctypes.c_void_p(dx.ctypes.data), HOST))
+        return dx
+
+    @staticmethod
+    def _expect(got, want, what):
+        if tuple(got) != tuple(want):
+            raise ValueError("%s dimensions %s do not match the layer's %s" % (what, tuple(got), tuple(want)))
+
+    def __del__(self):
+        try:
+            if self._h is not None and self._h.value:
+                lib().cattle_hip_layer_destroy(self._h)
+        except Exception:
+            pass
+        self._h = None
+
+
+def _ext3(dims):
+    """Dimensions::extend<3 - Rank>() (core/Dimensions.hpp:63-103): pad with ones to rank 3."""
+    dims = tuple(int(d) for d in dims)
+    return dims + (1,) * (3 - len(dims))
+
+
+class ConvKernelLayer(Layer):
+    """layer/kernel/ConvKernelLayer.hpp:282-296; rank 1/2 inputs are re-viewed as in :400-417, :494-508."""
+
+    def __init__(self, dtype, input_dims, filters, receptor_height=3, receptor_width=3, vertical_padding=1,
+                 horizontal_padding=1, vertical_stride=1, horizontal_stride=1, vertical_dilation=0,
+                 horizontal_dilation=0):
+        rank = len(input_dims)
+        if rank == 1:       # ConvKernelLayer<Scalar,1>: (length) -> receptor (len,1), padding (p,0), stride (s,1)
+            receptor_width, horizontal_padding, horizontal_stride, horizontal_dilation = 1, 0, 1, 0
+        H, W, C = _ext3(input_dims)
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_conv_create(_dtype_code(dtype), _sz(H), _sz(W), _sz(C), _sz(filters), _sz(receptor_height),
+                                            _sz(receptor_width), _sz(vertical_padding), _sz(horizontal_padding),
+                                            _sz(vertical_stride), _sz(horizontal_stride), _sz(vertical_dilation),
+                                            _sz(horizontal_dilation), ctypes.byref(h)))
+        od = (ctypes.c_size_t * 3)()
+        _check(lib().cattle_hip_layer_output_dims(h, od))
+        OH, OW, F = int(od[0]), int(od[1]), int(od[2])
+        # calculate_adjusted_output_dims (:206-217): filters land on the last nominal rank
+        out = {3: (OH, OW, F), 2: (OH, OW * F), 1: (OH * F,)}[rank]
+        Layer.__init__(self, h, dtype, tuple(input_dims), out)
+
+
+class DenseKernelLayer(Layer):
+    """layer/kernel/DenseKernelLayer.hpp:61-77; output dims are (output_size, 1, ...) (:68)."""
+
+    def __init__(self, dtype, input_dims, output_size):
+        vol = int(np.prod(input_dims))
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_dense_create(_dtype_code(dtype), _sz(vol), _sz(output_size), ctypes.byref(h)))
+        Layer.__init__(self, h, dtype, tuple(input_dims), (int(output_size),) + (1,) * (len(input_dims) - 1))
+
+
+class BatchNormLayer(Layer):
+    """layer/BatchNormLayer.hpp:66-101 (per_last_rank=True) and :334-361 (False); default as in :28."""
+
+    def __init__(self, dtype, dims, norm_avg_decay=0.1, epsilon=1e-5, per_last_rank=None):
+        if per_last_rank is None:
+            per_last_rank = len(dims) == 3
+        # the statistics group is the last nominal rank: view it as the channel rank
+        dims = tuple(int(d) for d in dims)
+        lead = int(np.prod(dims[:-1])) if len(dims) > 1 else 1
+        H, W, C = (lead, 1, dims[-1]) if per_last_rank else _ext3(dims)
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_batchnorm_create(_dtype_code(dtype), _sz(H), _sz(W), _sz(C), ctypes.c_int(int(per_last_rank)),
+                                                 ctypes.c_double(norm_avg_decay), ctypes.c_double(epsilon), ctypes.byref(h)))
+        Layer.__init__(self, h, dtype, dims, dims)
+
+    def stats_initialized(self):
+        v = ctypes.c_int()
+        _check(lib().cattle_hip_batchnorm_get_stats_initialized(self._h, ctypes.byref(v)))
+        return bool(v.value)
+
+    def set_stats_initialized(self, flag):
+        _check(lib().cattle_hip_batchnorm_set_stats_initialized(self._h, ctypes.c_int(int(bool(flag)))))
+
+
+class ActivationLayer(Layer):
+    """layer/activation/<Name>ActivationLayer.hpp; kind is a key of ACT."""
+
+    def __init__(self, dtype, kind, dims, param=0.0):
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_activation_create(_dtype_code(dtype), ctypes.c_int(ACT[kind]), _sz(int(np.prod(dims))),
+                                                  ctypes.c_double(param), ctypes.byref(h)))
+        Layer.__init__(self, h, dtype, tuple(dims), tuple(dims))
+        self.kind = kind
+        self._always_backprop = kind == "prelu"
+
+
+def ReLUActivationLayer(dtype, dims):
+    return ActivationLayer(dtype, "relu", dims)
+
+
+def SigmoidActivationLayer(dtype, dims):
+    return ActivationLayer(dtype, "sigmoid", dims)
+
+
+def TanhActivationLayer(dtype, dims):
+    return ActivationLayer(dtype, "tanh", dims)
+
+
+class _PoolLayer(Layer):
+    def __init__(self, kind, dtype, input_dims, receptor_height, receptor_width, vertical_stride, horizontal_stride):
+        rank = len(input_dims)
+        if rank == 1:       # Max/MeanPoolLayer<Scalar,1>(dims, receptor_length, stride)
+            receptor_width, horizontal_stride = 1, 1
+        H, W, C = _ext3(input_dims)
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_pool_create(_dtype_code(dtype), ctypes.c_int(kind), _sz(H), _sz(W), _sz(C), _sz(receptor_height),
+                                            _sz(receptor_width), _sz(vertical_stride), _sz(horizontal_stride), ctypes.byref(h)))
+        od = (ctypes.c_size_t * 3)()
+        _check(lib().cattle_hip_layer_output_dims(h, od))
+        out = (int(od[0]), int(od[1]), int(od[2]))[:rank]
+        Layer.__init__(self, h, dtype, tuple(input_dims), out)
+
+
+class MaxPoolLayer(_PoolLayer):
+    """layer/pool/MaxPoolLayer.hpp:105-108 (defaults 2x2 stride 2)."""
+
+    def __init__(self, dtype, input_dims, receptor_height=2, receptor_width=2, vertical_stride=2, horizontal_stride=2):
+        _PoolLayer.__init__(self, POOL_MAX, dtype, input_dims, receptor_height, receptor_width, vertical_stride,
+                            horizontal_stride)
+
+    def max_indices(self, batch):
+        """The argmax cache, shape (OH*OW, C*batch), as layer/pool/MaxPoolLayer.hpp:58-62 stores it."""
+        od = _ext3(self._out_shape)
+        a = np.empty((od[0] * od[1], od[2] * batch), dtype=np.uint32)
+        _check(lib().cattle_hip_maxpool_indices(self._h, ctypes.c_void_p(a.ctypes.data), HOST))
+        return a
+
+
+class MeanPoolLayer(_PoolLayer):
+    """layer/pool/MeanPoolLayer.hpp:62-65."""
+
+    def __init__(self, dtype, input_dims, receptor_height=2, receptor_width=2, vertical_stride=2, horizontal_stride=2):
+        _PoolLayer.__init__(self, POOL_MEAN, dtype, input_dims, receptor_height, receptor_width, vertical_stride,
+                            horizontal_stride)

@@ -1,0 +1,115 @@
+/*
+ * common.hpp — shared declarations of the cattle_hip library internals (gfx950 only).
+ */
+#ifndef CATTLE_HIP_COMMON_HPP_
+#define CATTLE_HIP_COMMON_HPP_
+
+#include <hip/hip_runtime.h>
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+namespace cattle_hip {
+
+/* Error carrier used inside the library; the C-ABI layer turns it into a status code plus the
+ * thread-local message returned by cattle_hip_last_error(). */
+struct Error : public std::runtime_error {
+	int code;
+	Error(int code, const std::string& what) : std::runtime_error(what), code(code) { }
+};
+
+enum { ERR_INVALID = 1, ERR_STATE = 2, ERR_DEVICE = 3, ERR_OOM = 4 };
+
+#define CATTLE_HIP_CHECK(expr) do { \
+	hipError_t _e = (expr); \
+	if (_e != hipSuccess) \
+		throw ::cattle_hip::Error(_e == hipErrorOutOfMemory ? ::cattle_hip::ERR_OOM : ::cattle_hip::ERR_DEVICE, \
+				std::string(#expr) + ": " + hipGetErrorString(_e)); \
+} while (0)
+
+#define CATTLE_HIP_REQUIRE(cond, msg) do { \
+	if (!(cond)) \
+		throw ::cattle_hip::Error(::cattle_hip::ERR_INVALID, std::string(msg)); \
+} while (0)
+
+/* The stream every kernel and copy of the library is issued on. */
+hipStream_t stream();
+
+/* Geometry of a gathered GEMM  out[M x F] = A[M x K] * Wt[K x F]  whose A matrix is never
+ * materialised: A(m,k) is read from a column-major (N, LH, LW, LC) tensor.
+ *   m = n + N*(a + OA*b)           k = r + R*(s + S*ch)
+ *   ya = (a*SA + PA + r*RA) / DA   (must divide exactly and lie in [0, LH))
+ *   yb = (b*SB + PB + s*RB) / DB   (must divide exactly and lie in [0, LW))
+ *   A(m,k) = src[n + N*(ya + LH*(yb + LW*ch))], or 0 where the conditions fail (zero padding).
+ * The forward convolution uses SA = stride, RA = dilation + 1, PA = -padding, DA = 1; the input
+ * gradient uses SA = 1, RA = -(dilation + 1), PA = +padding, DA = stride on the output gradient. */
+struct GatherGeom {
+	int N, LH, LW, LC;
+	int OA, OB;
+	int R, S;
+	int SA, SB, RA, RB, PA, PB, DA, DB;
+	int M, K, F;
+	int ldw;        /* row stride of the prepared weight matrix Wt (elements) */
+};
+
+/* Convolution hyper-parameters in the reference's terms (dilation 0 = dense receptor). */
+struct ConvShape {
+	int H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh;
+	int OH() const { return (H - RH - (RH - 1) * dv + 2 * pv) / sv + 1; }
+	int OW() const { return (W - RW - (RW - 1) * dh + 2 * ph) / sh + 1; }
+	int K() const { return RH * RW * C; }
+};
+
+/* Sizes of the scratch buffers the GEMM launchers need for a batch of N (in elements of T). */
+struct ConvWorkspace {
+	size_t wt_fwd;      /* prepared forward weights  */
+	size_t wt_dgrad;    /* prepared input-gradient weights */
+	size_t partials;    /* split-M partial weight gradients + bias-gradient partials */
+};
+
+template<typename T> ConvWorkspace conv_workspace(const ConvShape& s, int N);
+
+/* Forward: out(N,OH,OW,F) = conv(x; w) + b. w is the reference's [K x F] column-major matrix.
+ * wt is scratch of conv_workspace().wt_fwd elements; if wt_ready is false it is (re)built from w. */
+template<typename T> void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out,
+		T* wt, bool wt_ready);
+
+/* Backward: wgrad[K x F] += A^T G, bgrad[F] += colsum(G), in_grad = dgrad (skipped if null). */
+template<typename T> void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad,
+		T* wgrad, T* bgrad, T* in_grad, T* wt_dgrad, bool wt_ready, T* partials);
+
+/* Element-wise / reduction kernels (pointwise_kernels.hip). */
+template<typename T> void act_forward(int kind, size_t n, T p, const T* x, T* y);
+template<typename T> void act_backward(int kind, size_t n, T p, const T* x, const T* y, const T* g, T* dx);
+template<typename T> void softmax_forward(int N, int V, T eps, const T* x, T* y);
+template<typename T> void softmax_backward(int N, int V, const T* y, const T* g, T* dx);
+template<typename T> void prelu_forward(int N, int V, const T* alpha, const T* x, T* y);
+template<typename T> void prelu_backward(int N, int V, const T* alpha, const T* x, const T* g, T* alpha_grad, T* dx);
+template<typename T> void pswish_forward(int N, int V, const T* beta, const T* x, T* y);
+template<typename T> void pswish_backward(int N, int V, const T* beta, const T* x, const T* g, T* beta_grad, T* dx);
+
+/* Batch norm over `groups` contiguous slabs of L elements (per-channel: slab = channel, L = N*H*W;
+ * per-activation: slab = one activation's column, L = N). ws needs bn_workspace() elements. */
+size_t bn_workspace(int groups, size_t L);
+template<typename T> void bn_forward(int groups, size_t L, const T* x, const T* gamma, const T* beta, T* avg_mean,
+		T* avg_inv_sd, bool stats_init, bool training, T decay, T eps, T* out, T* std_cache, T* inv_sd_cache, T* ws);
+template<typename T> void bn_backward(int groups, size_t L, const T* out_grad, const T* gamma, const T* std_cache,
+		const T* inv_sd_cache, T* gamma_grad, T* beta_grad, T* in_grad, T* ws);
+
+struct PoolShape {
+	int H, W, C, RH, RW, sv, sh;
+	int OH() const { return (H - RH) / sv + 1; }
+	int OW() const { return (W - RW) / sh + 1; }
+};
+template<typename T> void maxpool_forward(const PoolShape& s, int N, const T* x, T* out, unsigned* inds);
+template<typename T> void maxpool_backward(const PoolShape& s, int N, const T* out_grad, const unsigned* inds, T* in_grad);
+template<typename T> void meanpool_forward(const PoolShape& s, int N, const T* x, T* out);
+template<typename T> void meanpool_backward(const PoolShape& s, int N, const T* out_grad, T* in_grad);
+
+/* dst[i] += src[i] */
+template<typename T> void axpy_one(size_t n, const T* src, T* dst);
+
+} /* namespace cattle_hip */
+
+#endif /* CATTLE_HIP_COMMON_HPP_ */

@@ -1,0 +1,854 @@
+/*
+ * layers.hip — layer objects behind the C ABI declared in include/cattle_hip.h.
+ *
+ * Each handle mirrors one cattle::Layer object (core/Layer.hpp:30-155): it keeps what the
+ * reference layer caches between pass_forward and pass_back, device copies of the parameters and
+ * accumulating gradient buffers, and forwards the arithmetic to the kernels in gemm_kernels.hip
+ * and pointwise_kernels.hip. There is no host implementation of any operation here.
+ */
+#include "common.hpp"
+#include "../../include/cattle_hip.h"
+
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <vector>
+
+namespace cattle_hip {
+
+namespace {
+
+std::recursive_mutex g_mutex;
+thread_local std::string g_last_error;
+bool g_ready = false;
+hipStream_t g_stream = nullptr;
+
+void ensure_init(int device) {
+	if (g_ready)
+		return;
+	int count = 0;
+	hipError_t e = hipGetDeviceCount(&count);
+	if (e != hipSuccess || count <= 0)
+		throw Error(ERR_DEVICE, "no HIP device is available; cattle_hip has no host fallback");
+	CATTLE_HIP_REQUIRE(device >= 0 && device < count, "device index out of range");
+	CATTLE_HIP_CHECK(hipSetDevice(device));
+	hipDeviceProp_t prop;
+	CATTLE_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+	if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+		throw Error(ERR_DEVICE, std::string("cattle_hip is built for gfx950 only, found ") + prop.gcnArchName);
+	CATTLE_HIP_CHECK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+	g_ready = true;
+}
+
+/* Grow-only device buffer. */
+struct DevBuf {
+	void* p = nullptr;
+	size_t cap = 0;
+	DevBuf() { }
+	DevBuf(const DevBuf&) = delete;
+	DevBuf& operator=(const DevBuf&) = delete;
+	~DevBuf() {
+		release();
+	}
+	void release() {
+		if (p)
+			(void) hipFree(p);
+		p = nullptr;
+		cap = 0;
+	}
+	void* ensure(size_t bytes) {
+		if (bytes > cap) {
+			release();
+			const size_t want = (bytes + 255) / 256 * 256;
+			CATTLE_HIP_CHECK(hipMalloc(&p, want));
+			cap = want;
+		}
+		return p;
+	}
+};
+
+void copy_in(void* dst_dev, const void* src, int space, size_t bytes) {
+	if (bytes == 0)
+		return;
+	CATTLE_HIP_CHECK(hipMemcpyAsync(dst_dev, src, bytes, space == CATTLE_HIP_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice,
+			stream()));
+	if (space == CATTLE_HIP_HOST)
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));    /* the pageable source may be freed on return */
+}
+
+void copy_out(void* dst, int space, const void* src_dev, size_t bytes) {
+	if (bytes == 0)
+		return;
+	CATTLE_HIP_CHECK(hipMemcpyAsync(dst, src_dev, bytes, space == CATTLE_HIP_HOST ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice,
+			stream()));
+	if (space == CATTLE_HIP_HOST)
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+}
+
+void fill_zero(void* dst_dev, size_t bytes) {
+	if (bytes)
+		CATTLE_HIP_CHECK(hipMemsetAsync(dst_dev, 0, bytes, stream()));
+}
+
+/* Device twin of a Parameters object (core/Parameters.hpp:15-95): values plus accumulated gradient.
+ * `derived` holds kernel-friendly re-layouts of the values, rebuilt when `version` moves on. */
+struct Param {
+	size_t rows, cols;
+	bool optimizable;
+	size_t esize;
+	DevBuf values, grad;
+	uint64_t version = 1;
+	DevBuf derived[2];
+	uint64_t derived_version[2] = { 0, 0 };
+	Param(size_t rows, size_t cols, bool optimizable, size_t esize) : rows(rows), cols(cols), optimizable(optimizable), esize(esize) {
+		values.ensure(bytes());
+		grad.ensure(bytes());
+		fill_zero(values.p, bytes());
+		fill_zero(grad.p, bytes());
+	}
+	size_t bytes() const {
+		return rows * cols * esize;
+	}
+	std::shared_ptr<Param> deep_copy() const {
+		std::shared_ptr<Param> c = std::make_shared<Param>(rows, cols, optimizable, esize);
+		copy_in(c->values.p, values.p, CATTLE_HIP_DEVICE, bytes());
+		copy_in(c->grad.p, grad.p, CATTLE_HIP_DEVICE, bytes());
+		return c;
+	}
+};
+
+typedef std::shared_ptr<Param> ParamPtr;
+
+template<typename T>
+void fill_constant(Param& p, T v) {
+	std::vector<T> host(p.rows * p.cols, v);
+	copy_in(p.values.p, host.data(), CATTLE_HIP_HOST, p.bytes());
+	++p.version;
+}
+
+struct LayerBase {
+	int dtype;
+	size_t in_dims[3], out_dims[3];
+	bool input_layer = false;
+	bool always_backprop = false;      /* PReLU ignores the input-layer flag */
+	std::vector<ParamPtr> params;
+	DevBuf in_stage, out_stage, og_stage, ig_stage;
+	size_t batch = 0;
+	bool have_forward = false;
+
+	LayerBase(int dtype) : dtype(dtype) { }
+	virtual ~LayerBase() { }
+	size_t esize() const {
+		return dtype == CATTLE_HIP_F32 ? 4 : 8;
+	}
+	size_t in_volume() const {
+		return in_dims[0] * in_dims[1] * in_dims[2];
+	}
+	size_t out_volume() const {
+		return out_dims[0] * out_dims[1] * out_dims[2];
+	}
+	void copy_base(const LayerBase& o, bool share) {
+		std::memcpy(in_dims, o.in_dims, sizeof(in_dims));
+		std::memcpy(out_dims, o.out_dims, sizeof(out_dims));
+		input_layer = o.input_layer;
+		always_backprop = o.always_backprop;
+		params.clear();
+		for (const ParamPtr& p : o.params)
+			params.push_back(share ? p : p->deep_copy());
+	}
+	virtual LayerBase* clone(bool share) const = 0;
+	/* in/out are device pointers; `out` persists until the next forward when it is a stage buffer
+	 * or for as long as the caller keeps it (borrowed) */
+	virtual void forward(const void* in, size_t N, bool training, void* out) = 0;
+	virtual void backward(const void* out_grad, size_t N, void* in_grad) = 0;
+	virtual void empty_cache() {
+		have_forward = false;
+	}
+};
+
+int checked_int(size_t v, const char* what) {
+	CATTLE_HIP_REQUIRE(v <= 2147483647u, std::string(what) + " exceeds 2^31-1");
+	return (int) v;
+}
+
+/* ConvKernelLayer and DenseKernelLayer (a dense layer is the 1x1 case on a 1x1 image whose
+ * channels are the input volume: X = Map(in.data(), N, volume), DenseKernelLayer.hpp:98). */
+template<typename T>
+struct ConvLayer : LayerBase {
+	ConvShape shape;
+	const T* x_cache = nullptr;
+	DevBuf partials;
+
+	ConvLayer(int dtype, const ConvShape& s, bool dense) : LayerBase(dtype), shape(s) {
+		if (dense) {
+			in_dims[0] = (size_t) s.C; in_dims[1] = 1; in_dims[2] = 1;
+			out_dims[0] = (size_t) s.F; out_dims[1] = 1; out_dims[2] = 1;
+		} else {
+			in_dims[0] = (size_t) s.H; in_dims[1] = (size_t) s.W; in_dims[2] = (size_t) s.C;
+			out_dims[0] = (size_t) s.OH(); out_dims[1] = (size_t) s.OW(); out_dims[2] = (size_t) s.F;
+		}
+		params.push_back(std::make_shared<Param>((size_t) s.K(), (size_t) s.F, true, sizeof(T)));
+		params.push_back(std::make_shared<Param>(1, (size_t) s.F, true, sizeof(T)));
+	}
+	ConvLayer(const ConvLayer& o, bool share) : LayerBase(o.dtype), shape(o.shape) {
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new ConvLayer(*this, share);
+	}
+	void forward(const void* in, size_t N, bool, void* out) override {
+		const int n = checked_int(N, "batch size");
+		const ConvWorkspace ws = conv_workspace<T>(shape, n);
+		Param& w = *params[0];
+		T* wt = (T*) w.derived[0].ensure(ws.wt_fwd * sizeof(T));
+		const bool ready = w.derived_version[0] == w.version;
+		conv_forward<T>(shape, n, (const T*) in, (const T*) w.values.p, (const T*) params[1]->values.p, (T*) out, wt, ready);
+		w.derived_version[0] = w.version;
+		x_cache = (const T*) in;       /* the reference caches the patch matrix (ConvKernelLayer.hpp:127); the input suffices */
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		CATTLE_HIP_REQUIRE(x_cache != nullptr, "pass_back without a cached forward input");
+		const int n = checked_int(N, "batch size");
+		const ConvWorkspace ws = conv_workspace<T>(shape, n);
+		Param& w = *params[0];
+		T* wt = (T*) w.derived[1].ensure(ws.wt_dgrad * sizeof(T));
+		const bool ready = w.derived_version[1] == w.version;
+		T* part = (T*) partials.ensure(ws.partials * sizeof(T));
+		conv_backward<T>(shape, n, x_cache, (const T*) w.values.p, (const T*) out_grad, (T*) w.grad.p, (T*) params[1]->grad.p,
+				(T*) in_grad, wt, ready, part);
+		if (in_grad)
+			w.derived_version[1] = w.version;
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		x_cache = nullptr;
+	}
+};
+
+template<typename T>
+struct BatchNormLayer : LayerBase {
+	bool per_last_rank;
+	T decay, eps;
+	bool stats_init = false;
+	DevBuf std_cache, inv_sd_cache, ws;
+	bool cache_valid = false;
+
+	BatchNormLayer(int dtype, size_t H, size_t W, size_t C, bool per_last_rank, T decay, T eps) :
+			LayerBase(dtype), per_last_rank(per_last_rank), decay(decay), eps(eps) {
+		in_dims[0] = out_dims[0] = H;
+		in_dims[1] = out_dims[1] = W;
+		in_dims[2] = out_dims[2] = C;
+		const size_t g = groups();
+		params.push_back(std::make_shared<Param>(1, g, false, sizeof(T)));     /* running means */
+		params.push_back(std::make_shared<Param>(1, g, false, sizeof(T)));     /* running inverse sds */
+		params.push_back(std::make_shared<Param>(1, g, true, sizeof(T)));      /* gammas, OneParameterInitialization */
+		params.push_back(std::make_shared<Param>(1, g, true, sizeof(T)));      /* betas, ZeroParameterInitialization */
+		fill_constant<T>(*params[2], (T) 1);
+	}
+	BatchNormLayer(const BatchNormLayer& o, bool share) : LayerBase(o.dtype), per_last_rank(o.per_last_rank), decay(o.decay),
+			eps(o.eps), stats_init(o.stats_init) {
+		copy_base(o, share);
+	}
+	size_t groups() const {
+		return per_last_rank ? in_dims[2] : in_volume();
+	}
+	LayerBase* clone(bool share) const override {
+		return new BatchNormLayer(*this, share);
+	}
+	void forward(const void* in, size_t N, bool training, void* out) override {
+		const int g = checked_int(groups(), "statistics groups");
+		const size_t L = N * in_volume() / groups();
+		CATTLE_HIP_REQUIRE(training || stats_init, "inference before any training pass: running statistics unset");
+		T* sc = nullptr;
+		T* isd = nullptr;
+		if (training) {
+			sc = (T*) std_cache.ensure(N * in_volume() * sizeof(T));
+			isd = (T*) inv_sd_cache.ensure(groups() * sizeof(T));
+		}
+		T* w = (T*) ws.ensure(bn_workspace(g, L) * sizeof(T));
+		bn_forward<T>(g, L, (const T*) in, (const T*) params[2]->values.p, (const T*) params[3]->values.p,
+				(T*) params[0]->values.p, (T*) params[1]->values.p, stats_init, training, decay, eps, (T*) out, sc, isd, w);
+		if (training) {
+			stats_init = true;
+			cache_valid = true;
+			++params[0]->version;
+			++params[1]->version;
+		}
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		CATTLE_HIP_REQUIRE(cache_valid, "pass_back without a training-mode forward pass");
+		const int g = checked_int(groups(), "statistics groups");
+		const size_t L = N * in_volume() / groups();
+		T* w = (T*) ws.ensure(bn_workspace(g, L) * sizeof(T));
+		bn_backward<T>(g, L, (const T*) out_grad, (const T*) params[2]->values.p, (const T*) std_cache.p,
+				(const T*) inv_sd_cache.p, (T*) params[2]->grad.p, (T*) params[3]->grad.p, (T*) in_grad, w);
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		cache_valid = false;
+		std_cache.release();
+	}
+};
+
+template<typename T>
+struct ActivationLayer : LayerBase {
+	int kind;
+	T p;
+	const T* x_cache = nullptr;
+	const T* y_cache = nullptr;
+
+	ActivationLayer(int dtype, int kind, size_t volume, T p) : LayerBase(dtype), kind(kind), p(p) {
+		in_dims[0] = out_dims[0] = volume;
+		in_dims[1] = out_dims[1] = 1;
+		in_dims[2] = out_dims[2] = 1;
+		if (kind == CATTLE_HIP_ACT_PRELU || kind == CATTLE_HIP_ACT_PSWISH) {
+			params.push_back(std::make_shared<Param>(1, volume, true, sizeof(T)));   /* ConstantParameterInitialization(p) */
+			fill_constant<T>(*params[0], p);
+		}
+		always_backprop = kind == CATTLE_HIP_ACT_PRELU;
+	}
+	ActivationLayer(const ActivationLayer& o, bool share) : LayerBase(o.dtype), kind(o.kind), p(o.p) {
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new ActivationLayer(*this, share);
+	}
+	void forward(const void* in, size_t N, bool, void* out) override {
+		const size_t total = N * in_volume();
+		const int n = checked_int(N, "batch size"), v = checked_int(in_volume(), "volume");
+		switch (kind) {
+		case CATTLE_HIP_ACT_SOFTMAX:
+			softmax_forward<T>(n, v, p, (const T*) in, (T*) out);
+			break;
+		case CATTLE_HIP_ACT_PRELU:
+			prelu_forward<T>(n, v, (const T*) params[0]->values.p, (const T*) in, (T*) out);
+			break;
+		case CATTLE_HIP_ACT_PSWISH:
+			pswish_forward<T>(n, v, (const T*) params[0]->values.p, (const T*) in, (T*) out);
+			break;
+		default:
+			act_forward<T>(kind, total, p, (const T*) in, (T*) out);
+		}
+		x_cache = (const T*) in;
+		y_cache = (const T*) out;
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		CATTLE_HIP_REQUIRE(x_cache != nullptr, "pass_back without a cached forward pass");
+		const size_t total = N * in_volume();
+		const int n = checked_int(N, "batch size"), v = checked_int(in_volume(), "volume");
+		switch (kind) {
+		case CATTLE_HIP_ACT_SOFTMAX:
+			if (in_grad)
+				softmax_backward<T>(n, v, y_cache, (const T*) out_grad, (T*) in_grad);
+			break;
+		case CATTLE_HIP_ACT_PRELU:
+			prelu_backward<T>(n, v, (const T*) params[0]->values.p, x_cache, (const T*) out_grad, (T*) params[0]->grad.p,
+					(T*) in_grad);
+			break;
+		case CATTLE_HIP_ACT_PSWISH:
+			pswish_backward<T>(n, v, (const T*) params[0]->values.p, x_cache, (const T*) out_grad, (T*) params[0]->grad.p,
+					(T*) in_grad);
+			break;
+		default:
+			if (in_grad)
+				act_backward<T>(kind, total, p, x_cache, y_cache, (const T*) out_grad, (T*) in_grad);
+		}
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		x_cache = y_cache = nullptr;
+	}
+};
+
+template<typename T>
+struct PoolLayer : LayerBase {
+	int kind;
+	PoolShape shape;
+	DevBuf inds;
+	size_t inds_count = 0;
+
+	PoolLayer(int dtype, int kind, const PoolShape& s) : LayerBase(dtype), kind(kind), shape(s) {
+		in_dims[0] = (size_t) s.H; in_dims[1] = (size_t) s.W; in_dims[2] = (size_t) s.C;
+		out_dims[0] = (size_t) s.OH(); out_dims[1] = (size_t) s.OW(); out_dims[2] = (size_t) s.C;
+	}
+	PoolLayer(const PoolLayer& o, bool share) : LayerBase(o.dtype), kind(o.kind), shape(o.shape) {
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new PoolLayer(*this, share);
+	}
+	void forward(const void* in, size_t N, bool, void* out) override {
+		const int n = checked_int(N, "batch size");
+		checked_int(N * in_volume(), "tensor size");
+		if (kind == CATTLE_HIP_POOL_MAX) {
+			inds_count = N * out_volume();
+			unsigned* ip = (unsigned*) inds.ensure(inds_count * sizeof(unsigned));
+			maxpool_forward<T>(shape, n, (const T*) in, (T*) out, ip);
+		} else {
+			meanpool_forward<T>(shape, n, (const T*) in, (T*) out);
+		}
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		if (!in_grad)
+			return;
+		const int n = checked_int(N, "batch size");
+		if (kind == CATTLE_HIP_POOL_MAX) {
+			CATTLE_HIP_REQUIRE(inds_count == N * out_volume(), "pass_back without cached max indices");
+			maxpool_backward<T>(shape, n, (const T*) out_grad, (const unsigned*) inds.p, (T*) in_grad);
+		} else {
+			meanpool_backward<T>(shape, n, (const T*) out_grad, (T*) in_grad);
+		}
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		inds_count = 0;
+		inds.release();
+	}
+};
+
+struct Timer {
+	hipEvent_t start = nullptr, stop = nullptr;
+};
+
+LayerBase* as_layer(cattle_hip_layer_t h) {
+	CATTLE_HIP_REQUIRE(h != nullptr, "null layer handle");
+	return reinterpret_cast<LayerBase*>(h);
+}
+
+Param& param_at(LayerBase* l, size_t index) {
+	CATTLE_HIP_REQUIRE(index < l->params.size(), "parameter index out of range");
+	return *l->params[index];
+}
+
+void check_dtype(int dtype) {
+	CATTLE_HIP_REQUIRE(dtype == CATTLE_HIP_F32 || dtype == CATTLE_HIP_F64, "dtype must be CATTLE_HIP_F32 or CATTLE_HIP_F64");
+}
+
+void check_space(int space) {
+	CATTLE_HIP_REQUIRE(space == CATTLE_HIP_HOST || space == CATTLE_HIP_DEVICE, "memspace must be HOST or DEVICE");
+}
+
+template<typename Fn>
+int guarded(Fn fn) {
+	std::lock_guard<std::recursive_mutex> lock(g_mutex);
+	try {
+		ensure_init(0);
+		fn();
+		return CATTLE_HIP_OK;
+	} catch (const Error& e) {
+		g_last_error = e.what();
+		return e.code;
+	} catch (const std::bad_alloc&) {
+		g_last_error = "host allocation failed";
+		return CATTLE_HIP_ERR_OOM;
+	} catch (const std::exception& e) {
+		g_last_error = e.what();
+		return CATTLE_HIP_ERR_INVALID;
+	}
+}
+
+} /* namespace */
+
+hipStream_t stream() {
+	return g_stream;
+}
+
+} /* namespace cattle_hip */
+
+using namespace cattle_hip;
+
+extern "C" {
+
+int cattle_hip_init(int device) {
+	std::lock_guard<std::recursive_mutex> lock(g_mutex);
+	try {
+		ensure_init(device);
+		return CATTLE_HIP_OK;
+	} catch (const Error& e) {
+		g_last_error = e.what();
+		return e.code;
+	}
+}
+
+const char* cattle_hip_last_error(void) {
+	return g_last_error.c_str();
+}
+
+int cattle_hip_synchronize(void) {
+	return guarded([&] { CATTLE_HIP_CHECK(hipStreamSynchronize(stream())); });
+}
+
+int cattle_hip_alloc(void** device_ptr, size_t bytes) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(device_ptr != nullptr, "null output pointer");
+		*device_ptr = nullptr;
+		CATTLE_HIP_CHECK(hipMalloc(device_ptr, bytes ? bytes : 1));
+	});
+}
+
+int cattle_hip_free(void* device_ptr) {
+	return guarded([&] {
+		if (device_ptr) {
+			CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+			CATTLE_HIP_CHECK(hipFree(device_ptr));
+		}
+	});
+}
+
+int cattle_hip_upload(void* dst_device, const void* src_host, size_t bytes) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(bytes == 0 || (dst_device && src_host), "null buffer");
+		copy_in(dst_device, src_host, CATTLE_HIP_HOST, bytes);
+	});
+}
+
+int cattle_hip_download(void* dst_host, const void* src_device, size_t bytes) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(bytes == 0 || (dst_host && src_device), "null buffer");
+		copy_out(dst_host, CATTLE_HIP_HOST, src_device, bytes);
+	});
+}
+
+int cattle_hip_fill_zero(void* dst_device, size_t bytes) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(bytes == 0 || dst_device, "null buffer");
+		fill_zero(dst_device, bytes);
+	});
+}
+
+int cattle_hip_timer_create(cattle_hip_timer_t* timer) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(timer != nullptr, "null output pointer");
+		std::unique_ptr<Timer> t(new Timer());
+		CATTLE_HIP_CHECK(hipEventCreate(&t->start));
+		CATTLE_HIP_CHECK(hipEventCreate(&t->stop));
+		*timer = reinterpret_cast<cattle_hip_timer_t>(t.release());
+	});
+}
+
+int cattle_hip_timer_destroy(cattle_hip_timer_t timer) {
+	return guarded([&] {
+		Timer* t = reinterpret_cast<Timer*>(timer);
+		if (t) {
+			(void) hipEventDestroy(t->start);
+			(void) hipEventDestroy(t->stop);
+			delete t;
+		}
+	});
+}
+
+int cattle_hip_timer_start(cattle_hip_timer_t timer) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(timer != nullptr, "null timer");
+		CATTLE_HIP_CHECK(hipEventRecord(reinterpret_cast<Timer*>(timer)->start, stream()));
+	});
+}
+
+int cattle_hip_timer_stop(cattle_hip_timer_t timer, float* elapsed_ms) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(timer != nullptr && elapsed_ms != nullptr, "null timer or output");
+		Timer* t = reinterpret_cast<Timer*>(timer);
+		CATTLE_HIP_CHECK(hipEventRecord(t->stop, stream()));
+		CATTLE_HIP_CHECK(hipEventSynchronize(t->stop));
+		CATTLE_HIP_CHECK(hipEventElapsedTime(elapsed_ms, t->start, t->stop));
+	});
+}
+
+int cattle_hip_conv_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, size_t filters,
+		size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
+		cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr, "null output pointer");
+		/* the constructor assertions of layer/kernel/ConvKernelLayer.hpp:82-87 */
+		CATTLE_HIP_REQUIRE(height > 0 && width > 0 && channels > 0, "input dimensions must be positive");
+		CATTLE_HIP_REQUIRE(filters > 0, "filters must be positive");
+		CATTLE_HIP_REQUIRE(receptor_height > 0 && receptor_width > 0, "receptor dimensions must be positive");
+		CATTLE_HIP_REQUIRE(vertical_stride > 0 && horizontal_stride > 0, "strides must be positive");
+		const size_t lim = 1u << 20;
+		CATTLE_HIP_REQUIRE(height < lim && width < lim && channels < lim && filters < lim && receptor_height < lim &&
+				receptor_width < lim && vertical_padding < lim && horizontal_padding < lim && vertical_stride < lim &&
+				horizontal_stride < lim && vertical_dilation < lim && horizontal_dilation < lim, "dimension too large");
+		const size_t drh = receptor_height + (receptor_height - 1) * vertical_dilation;
+		const size_t drw = receptor_width + (receptor_width - 1) * horizontal_dilation;
+		CATTLE_HIP_REQUIRE(height + 2 * vertical_padding >= drh && width + 2 * horizontal_padding >= drw,
+				"dilated receptor larger than the padded input");
+		CATTLE_HIP_REQUIRE(receptor_height * receptor_width * channels <= 2147483647u / 2 &&
+				receptor_height * receptor_width * filters <= 2147483647u / 2, "receptor volume too large");
+		ConvShape s = { (int) height, (int) width, (int) channels, (int) filters, (int) receptor_height, (int) receptor_width,
+				(int) vertical_padding, (int) horizontal_padding, (int) vertical_stride, (int) horizontal_stride,
+				(int) vertical_dilation, (int) horizontal_dilation };
+		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new ConvLayer<float>(dtype, s, false) :
+				(LayerBase*) new ConvLayer<double>(dtype, s, false);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_dense_create(cattle_hip_dtype dtype, size_t input_volume, size_t output_size, cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr, "null output pointer");
+		CATTLE_HIP_REQUIRE(input_volume > 0 && output_size > 0, "dense layer sizes must be positive");
+		CATTLE_HIP_REQUIRE(input_volume <= 2147483647u / 2 && output_size <= 2147483647u / 2, "dense layer too large");
+		ConvShape s = { 1, 1, (int) input_volume, (int) output_size, 1, 1, 0, 0, 1, 1, 0, 0 };
+		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new ConvLayer<float>(dtype, s, true) :
+				(LayerBase*) new ConvLayer<double>(dtype, s, true);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_batchnorm_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, int per_last_rank,
+		double norm_avg_decay, double epsilon, cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr, "null output pointer");
+		CATTLE_HIP_REQUIRE(height > 0 && width > 0 && channels > 0, "dimensions must be positive");
+		/* layer/BatchNormLayer.hpp:80-82 */
+		CATTLE_HIP_REQUIRE(norm_avg_decay >= 0 && norm_avg_decay <= 1, "norm avg decay must not be less than 0 or greater than 1");
+		CATTLE_HIP_REQUIRE(epsilon > 0, "epsilon must be greater than 0");
+		LayerBase* l = dtype == CATTLE_HIP_F32 ?
+				(LayerBase*) new BatchNormLayer<float>(dtype, height, width, channels, per_last_rank != 0, (float) norm_avg_decay,
+						(float) epsilon) :
+				(LayerBase*) new BatchNormLayer<double>(dtype, height, width, channels, per_last_rank != 0, norm_avg_decay, epsilon);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_batchnorm_get_stats_initialized(cattle_hip_layer_t layer, int* initialized) {
+	return guarded([&] {
+		LayerBase* l = as_layer(layer);
+		CATTLE_HIP_REQUIRE(initialized != nullptr, "null output pointer");
+		if (BatchNormLayer<float>* b = dynamic_cast<BatchNormLayer<float>*>(l))
+			*initialized = b->stats_init;
+		else if (BatchNormLayer<double>* b = dynamic_cast<BatchNormLayer<double>*>(l))
+			*initialized = b->stats_init;
+		else
+			throw Error(ERR_INVALID, "not a batch norm layer");
+	});
+}
+
+int cattle_hip_batchnorm_set_stats_initialized(cattle_hip_layer_t layer, int initialized) {
+	return guarded([&] {
+		LayerBase* l = as_layer(layer);
+		if (BatchNormLayer<float>* b = dynamic_cast<BatchNormLayer<float>*>(l))
+			b->stats_init = initialized != 0;
+		else if (BatchNormLayer<double>* b = dynamic_cast<BatchNormLayer<double>*>(l))
+			b->stats_init = initialized != 0;
+		else
+			throw Error(ERR_INVALID, "not a batch norm layer");
+	});
+}
+
+int cattle_hip_activation_create(cattle_hip_dtype dtype, cattle_hip_activation kind, size_t volume, double param,
+		cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr, "null output pointer");
+		CATTLE_HIP_REQUIRE(volume > 0, "volume must be positive");
+		CATTLE_HIP_REQUIRE((int) kind >= 0 && (int) kind <= CATTLE_HIP_ACT_PSWISH, "unknown activation kind");
+		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new ActivationLayer<float>(dtype, kind, volume, (float) param) :
+				(LayerBase*) new ActivationLayer<double>(dtype, kind, volume, param);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t height, size_t width, size_t channels,
+		size_t receptor_height, size_t receptor_width, size_t vertical_stride, size_t horizontal_stride,
+		cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr, "null output pointer");
+		CATTLE_HIP_REQUIRE(kind == CATTLE_HIP_POOL_MAX || kind == CATTLE_HIP_POOL_MEAN, "unknown pool kind");
+		/* layer/PoolLayer.hpp:73-75 */
+		CATTLE_HIP_REQUIRE(receptor_height > 0 && receptor_width > 0, "receptor dimensions must be positive");
+		CATTLE_HIP_REQUIRE(vertical_stride > 0 && horizontal_stride > 0, "strides must be positive");
+		CATTLE_HIP_REQUIRE(channels > 0 && height >= receptor_height && width >= receptor_width, "receptor larger than the input");
+		const size_t lim = 1u << 20;
+		CATTLE_HIP_REQUIRE(height < lim && width < lim && channels < lim && vertical_stride < lim && horizontal_stride < lim,
+				"dimension too large");
+		CATTLE_HIP_REQUIRE(receptor_height * receptor_width < 65536, "receptor area too large");
+		PoolShape s = { (int) height, (int) width, (int) channels, (int) receptor_height, (int) receptor_width,
+				(int) vertical_stride, (int) horizontal_stride };
+		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new PoolLayer<float>(dtype, kind, s) :
+				(LayerBase*) new PoolLayer<double>(dtype, kind, s);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_layer_clone(cattle_hip_layer_t layer, int share_params, cattle_hip_layer_t* clone) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(clone != nullptr, "null output pointer");
+		*clone = reinterpret_cast<cattle_hip_layer_t>(as_layer(layer)->clone(share_params != 0));
+	});
+}
+
+int cattle_hip_layer_destroy(cattle_hip_layer_t layer) {
+	return guarded([&] {
+		if (layer) {
+			CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+			delete reinterpret_cast<LayerBase*>(layer);
+		}
+	});
+}
+
+int cattle_hip_layer_input_dims(cattle_hip_layer_t layer, size_t dims[3]) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(dims != nullptr, "null output pointer");
+		std::memcpy(dims, as_layer(layer)->in_dims, 3 * sizeof(size_t));
+	});
+}
+
+int cattle_hip_layer_output_dims(cattle_hip_layer_t layer, size_t dims[3]) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(dims != nullptr, "null output pointer");
+		std::memcpy(dims, as_layer(layer)->out_dims, 3 * sizeof(size_t));
+	});
+}
+
+int cattle_hip_layer_is_input_layer(cattle_hip_layer_t layer, int* is_input_layer) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(is_input_layer != nullptr, "null output pointer");
+		*is_input_layer = as_layer(layer)->input_layer ? 1 : 0;
+	});
+}
+
+int cattle_hip_layer_set_input_layer(cattle_hip_layer_t layer, int is_input_layer) {
+	return guarded([&] { as_layer(layer)->input_layer = is_input_layer != 0; });
+}
+
+int cattle_hip_layer_empty_cache(cattle_hip_layer_t layer) {
+	return guarded([&] {
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+		as_layer(layer)->empty_cache();
+	});
+}
+
+int cattle_hip_layer_forward(cattle_hip_layer_t layer, const void* in, cattle_hip_memspace in_space, size_t batch,
+		int training, void* out, cattle_hip_memspace out_space) {
+	return guarded([&] {
+		LayerBase* l = as_layer(layer);
+		check_space(in_space);
+		check_space(out_space);
+		CATTLE_HIP_REQUIRE(in != nullptr && out != nullptr, "null tensor buffer");
+		CATTLE_HIP_REQUIRE(batch > 0, "batch size must be positive");            /* assert(in.dimension(0) > 0) */
+		const size_t in_bytes = batch * l->in_volume() * l->esize(), out_bytes = batch * l->out_volume() * l->esize();
+		CATTLE_HIP_REQUIRE(batch * l->in_volume() <= 2147483647u && batch * l->out_volume() <= 2147483647u,
+				"tensor exceeds 2^31-1 elements");
+		const void* in_dev = in;
+		if (in_space == CATTLE_HIP_HOST) {
+			copy_in(l->in_stage.ensure(in_bytes), in, CATTLE_HIP_HOST, in_bytes);
+			in_dev = l->in_stage.p;
+		}
+		void* out_dev = out_space == CATTLE_HIP_HOST ? l->out_stage.ensure(out_bytes) : out;
+		l->have_forward = false;
+		l->forward(in_dev, batch, training != 0, out_dev);
+		if (out_space == CATTLE_HIP_HOST)
+			copy_out(out, CATTLE_HIP_HOST, out_dev, out_bytes);
+		l->batch = batch;
+		l->have_forward = true;
+	});
+}
+
+int cattle_hip_layer_backward(cattle_hip_layer_t layer, const void* out_grad, cattle_hip_memspace grad_space, size_t batch,
+		void* in_grad, cattle_hip_memspace in_grad_space) {
+	return guarded([&] {
+		LayerBase* l = as_layer(layer);
+		check_space(grad_space);
+		check_space(in_grad_space);
+		CATTLE_HIP_REQUIRE(out_grad != nullptr, "null gradient buffer");
+		if (!l->have_forward)
+			throw Error(ERR_STATE, "pass_back without a preceding pass_forward");
+		CATTLE_HIP_REQUIRE(batch > 0 && batch == l->batch, "batch size differs from the forward pass");   /* e.g. ConvKernelLayer.hpp:314 */
+		CATTLE_HIP_REQUIRE(in_grad != nullptr || l->input_layer, "in_grad may be NULL only for an input layer");
+		const size_t in_bytes = batch * l->in_volume() * l->esize(), out_bytes = batch * l->out_volume() * l->esize();
+		const void* og_dev = out_grad;
+		if (grad_space == CATTLE_HIP_HOST) {
+			copy_in(l->og_stage.ensure(out_bytes), out_grad, CATTLE_HIP_HOST, out_bytes);
+			og_dev = l->og_stage.p;
+		}
+		const bool want_in_grad = in_grad != nullptr && (!l->input_layer || l->always_backprop);
+		void* ig_dev = nullptr;
+		if (want_in_grad)
+			ig_dev = in_grad_space == CATTLE_HIP_HOST ? l->ig_stage.ensure(in_bytes) : in_grad;
+		l->backward(og_dev, batch, ig_dev);
+		if (want_in_grad && in_grad_space == CATTLE_HIP_HOST)
+			copy_out(in_grad, CATTLE_HIP_HOST, ig_dev, in_bytes);
+	});
+}
+
+int cattle_hip_layer_num_params(cattle_hip_layer_t layer, size_t* count) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(count != nullptr, "null output pointer");
+		*count = as_layer(layer)->params.size();
+	});
+}
+
+int cattle_hip_layer_param_shape(cattle_hip_layer_t layer, size_t index, size_t* rows, size_t* cols, int* optimizable) {
+	return guarded([&] {
+		Param& p = param_at(as_layer(layer), index);
+		if (rows)
+			*rows = p.rows;
+		if (cols)
+			*cols = p.cols;
+		if (optimizable)
+			*optimizable = p.optimizable ? 1 : 0;
+	});
+}
+
+int cattle_hip_layer_set_param_values(cattle_hip_layer_t layer, size_t index, const void* values, cattle_hip_memspace space) {
+	return guarded([&] {
+		check_space(space);
+		CATTLE_HIP_REQUIRE(values != nullptr, "null buffer");
+		Param& p = param_at(as_layer(layer), index);
+		copy_in(p.values.p, values, space, p.bytes());
+		++p.version;
+	});
+}
+
+int cattle_hip_layer_get_param_values(cattle_hip_layer_t layer, size_t index, void* values, cattle_hip_memspace space) {
+	return guarded([&] {
+		check_space(space);
+		CATTLE_HIP_REQUIRE(values != nullptr, "null buffer");
+		Param& p = param_at(as_layer(layer), index);
+		copy_out(values, space, p.values.p, p.bytes());
+	});
+}
+
+int cattle_hip_layer_get_param_grad(cattle_hip_layer_t layer, size_t index, void* grad, cattle_hip_memspace space) {
+	return guarded([&] {
+		check_space(space);
+		CATTLE_HIP_REQUIRE(grad != nullptr, "null buffer");
+		Param& p = param_at(as_layer(layer), index);
+		copy_out(grad, space, p.grad.p, p.bytes());
+	});
+}
+
+int cattle_hip_layer_reset_param_grad(cattle_hip_layer_t layer, size_t index) {
+	return guarded([&] {
+		Param& p = param_at(as_layer(layer), index);
+		fill_zero(p.grad.p, p.bytes());
+	});
+}
+
+int cattle_hip_maxpool_indices(cattle_hip_layer_t layer, unsigned* indices, cattle_hip_memspace space) {
+	return guarded([&] {
+		check_space(space);
+		CATTLE_HIP_REQUIRE(indices != nullptr, "null buffer");
+		LayerBase* l = as_layer(layer);
+		DevBuf* buf = nullptr;
+		size_t count = 0;
+		if (PoolLayer<float>* p = dynamic_cast<PoolLayer<float>*>(l)) {
+			buf = &p->inds;
+			count = p->kind == CATTLE_HIP_POOL_MAX ? p->inds_count : 0;
+		} else if (PoolLayer<double>* p = dynamic_cast<PoolLayer<double>*>(l)) {
+			buf = &p->inds;
+			count = p->kind == CATTLE_HIP_POOL_MAX ? p->inds_count : 0;
+		}
+		if (!buf || count == 0)
+			throw Error(ERR_STATE, "no max-pool index cache (not a max pool layer, or no forward pass yet)");
+		copy_out(indices, space, buf->p, count * sizeof(unsigned));
+	});
+}
+
+} /* extern "C" */

@@ -1,0 +1,702 @@
+/*
+ * pointwise_kernels.hip — HBM-bound kernels: activations, softmax, batch norm, pooling (gfx950).
+ *
+ * Every tensor is the reference's column-major (N,H,W,C) buffer. Consecutive threads always walk
+ * the contiguous N (then H) direction, element-wise kernels use 16-byte accesses, and every
+ * reduction is a fixed-order two-stage sum (wavefront shuffles + LDS, then partials in ascending
+ * order), so results are reproducible run to run; no atomics are used anywhere.
+ */
+#include "common.hpp"
+
+#include <algorithm>
+#include <limits>
+#include <type_traits>
+
+namespace cattle_hip {
+
+namespace {
+
+enum ActKind {
+	ACT_IDENTITY = 0, ACT_SCALED = 1, ACT_BINARY_STEP = 2, ACT_SIGMOID = 3, ACT_TANH = 4, ACT_SOFTSIGN = 5,
+	ACT_SOFTPLUS = 6, ACT_RELU = 7, ACT_LEAKY_RELU = 8, ACT_ELU = 9, ACT_SWISH = 10
+};
+
+__device__ __forceinline__ float dev_exp(float v) { return expf(v); }
+__device__ __forceinline__ double dev_exp(double v) { return exp(v); }
+__device__ __forceinline__ float dev_log(float v) { return logf(v); }
+__device__ __forceinline__ double dev_log(double v) { return log(v); }
+__device__ __forceinline__ float dev_tanh(float v) { return tanhf(v); }
+__device__ __forceinline__ double dev_tanh(double v) { return tanh(v); }
+__device__ __forceinline__ float dev_sqrt(float v) { return sqrtf(v); }
+__device__ __forceinline__ double dev_sqrt(double v) { return sqrt(v); }
+
+/* Forward functions; each cites the reference layer whose formula it evaluates. */
+template<typename T, int KIND>
+__device__ __forceinline__ T act_f(T x, T p) {
+	switch (KIND) {
+	case ACT_IDENTITY: return x;                                        /* IdentityActivationLayer.hpp:37-42 */
+	case ACT_SCALED: return x * p;                                      /* ScaledActivationLayer.hpp:38-43 */
+	case ACT_BINARY_STEP: return (T) (x >= (T) 0);                      /* BinaryStepActivationLayer.hpp:42-47 */
+	case ACT_SIGMOID: return (T) 1 / (dev_exp(-x) + (T) 1);             /* SigmoidActivationLayer.hpp:38-43 */
+	case ACT_TANH: return dev_tanh(x);                                  /* TanhActivationLayer.hpp:38-43 */
+	case ACT_SOFTSIGN: return x / ((T) 1 + (x < (T) 0 ? -x : x));       /* SoftsignActivationLayer.hpp:39-44 */
+	case ACT_SOFTPLUS: return dev_log(dev_exp(x) + (T) 1);              /* SoftplusActivationLayer.hpp:40-45 */
+	case ACT_RELU: return x > (T) 0 ? x : (x == x ? (T) 0 : x);         /* ReLUActivationLayer.hpp:45-50 */
+	case ACT_LEAKY_RELU: { const T ax = x * p; return x > ax ? x : (ax == ax ? ax : x); }   /* LeakyReLU :50-55 */
+	case ACT_ELU: return x >= (T) 0 ? x : p * (dev_exp(x) - (T) 1);     /* ELUActivationLayer.hpp:55-64 */
+	case ACT_SWISH: return x * ((T) 1 / (dev_exp(-p * x) + (T) 1));     /* SwishActivationLayer.hpp:45-51 */
+	}
+	return x;
+}
+
+/* Backward functions of (input x, output y, upstream gradient g). */
+template<typename T, int KIND>
+__device__ __forceinline__ T act_b(T x, T y, T g, T p) {
+	switch (KIND) {
+	case ACT_IDENTITY: return g;                                        /* IdentityActivationLayer.hpp:43-49 */
+	case ACT_SCALED: return g * p;                                      /* ScaledActivationLayer.hpp:44-50 */
+	case ACT_BINARY_STEP: return (T) 0;                                 /* BinaryStepActivationLayer.hpp:48-54 */
+	case ACT_SIGMOID: return (y * ((T) 1 - y)) * g;                     /* SigmoidActivationLayer.hpp:44-50 */
+	case ACT_TANH: return ((T) 1 - y * y) * g;                          /* TanhActivationLayer.hpp:44-50 */
+	case ACT_SOFTSIGN: { const T d = (T) 1 + (x < (T) 0 ? -x : x); return ((T) 1 / (d * d)) * g; }   /* :45-51 */
+	case ACT_SOFTPLUS: return ((T) 1 / (dev_exp(-x) + (T) 1)) * g;      /* SoftplusActivationLayer.hpp:46-52 */
+	case ACT_RELU: return (T) (x >= (T) 0) * g;                         /* ReLUActivationLayer.hpp:51-57 */
+	case ACT_LEAKY_RELU: return (x >= (T) 0 ? (T) 1 : p) * g;           /* LeakyReLUActivationLayer.hpp:56-62 */
+	case ACT_ELU: return (x >= (T) 0 ? (T) 1 : (y + p)) * g;            /* ELUActivationLayer.hpp:65-78 */
+	case ACT_SWISH: {                                                   /* SwishActivationLayer.hpp:52-59 */
+		const T s = (T) 1 / (dev_exp(-p * x) + (T) 1);
+		return s * ((((T) 1 - s) * p) * x + (T) 1) * g;
+	}
+	}
+	return g;
+}
+
+/* Which cached operands the backward of a kind actually reads (the others may be null). */
+__host__ __device__ constexpr bool act_needs_x(int k) {
+	return k == ACT_SOFTSIGN || k == ACT_SOFTPLUS || k == ACT_RELU || k == ACT_LEAKY_RELU || k == ACT_ELU || k == ACT_SWISH;
+}
+__host__ __device__ constexpr bool act_needs_y(int k) {
+	return k == ACT_SIGMOID || k == ACT_TANH || k == ACT_ELU;
+}
+
+template<typename T> struct Pack { static constexpr int V = 16 / (int) sizeof(T); typedef T type __attribute__((ext_vector_type(16 / sizeof(T)))); };
+
+template<typename T, int KIND, bool VECTOR>
+__global__ __launch_bounds__(256)
+void act_forward_kernel(size_t n, T p, const T* __restrict__ x, T* __restrict__ y) {
+	constexpr int V = VECTOR ? Pack<T>::V : 1;
+	typedef typename Pack<T>::type vt;
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	const size_t nv = n / V;
+	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+		if constexpr (VECTOR) {
+			vt a = reinterpret_cast<const vt*>(x)[i], o;
+			#pragma unroll
+			for (int e = 0; e < V; ++e)
+				o[e] = act_f<T, KIND>(a[e], p);
+			reinterpret_cast<vt*>(y)[i] = o;
+		} else {
+			y[i] = act_f<T, KIND>(x[i], p);
+		}
+	}
+	if (VECTOR && blockIdx.x == 0 && threadIdx.x < n - nv * V) {
+		const size_t i = nv * V + threadIdx.x;
+		y[i] = act_f<T, KIND>(x[i], p);
+	}
+}
+
+template<typename T, int KIND, bool VECTOR>
+__global__ __launch_bounds__(256)
+void act_backward_kernel(size_t n, T p, const T* __restrict__ x, const T* __restrict__ y, const T* __restrict__ g,
+		T* __restrict__ dx) {
+	constexpr int V = VECTOR ? Pack<T>::V : 1;
+	typedef typename Pack<T>::type vt;
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	const size_t nv = n / V;
+	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+		if constexpr (VECTOR) {
+			vt xv = {0}, yv = {0}, o;
+			if (act_needs_x(KIND))
+				xv = reinterpret_cast<const vt*>(x)[i];
+			if (act_needs_y(KIND))
+				yv = reinterpret_cast<const vt*>(y)[i];
+			const vt gv = reinterpret_cast<const vt*>(g)[i];
+			#pragma unroll
+			for (int e = 0; e < V; ++e)
+				o[e] = act_b<T, KIND>(xv[e], yv[e], gv[e], p);
+			reinterpret_cast<vt*>(dx)[i] = o;
+		} else {
+			dx[i] = act_b<T, KIND>(act_needs_x(KIND) ? x[i] : (T) 0, act_needs_y(KIND) ? y[i] : (T) 0, g[i], p);
+		}
+	}
+	if (VECTOR && blockIdx.x == 0 && threadIdx.x < n - nv * V) {
+		const size_t i = nv * V + threadIdx.x;
+		dx[i] = act_b<T, KIND>(act_needs_x(KIND) ? x[i] : (T) 0, act_needs_y(KIND) ? y[i] : (T) 0, g[i], p);
+	}
+}
+
+bool aligned16(const void* p) {
+	return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
+unsigned stream_grid(size_t work_items) {
+	const size_t blocks = (work_items + 255) / 256;
+	return (unsigned) std::max<size_t>(1, std::min<size_t>(blocks, 256 * 16));
+}
+
+template<typename T, int KIND>
+void act_forward_kind(size_t n, T p, const T* x, T* y) {
+	if (aligned16(x) && aligned16(y))
+		act_forward_kernel<T, KIND, true><<<stream_grid(n / Pack<T>::V), 256, 0, stream()>>>(n, p, x, y);
+	else
+		act_forward_kernel<T, KIND, false><<<stream_grid(n), 256, 0, stream()>>>(n, p, x, y);
+}
+
+template<typename T, int KIND>
+void act_backward_kind(size_t n, T p, const T* x, const T* y, const T* g, T* dx) {
+	CATTLE_HIP_REQUIRE(!act_needs_x(KIND) || x, "activation backward needs the cached input");
+	CATTLE_HIP_REQUIRE(!act_needs_y(KIND) || y, "activation backward needs the cached output");
+	const bool al = aligned16(g) && aligned16(dx) && (!act_needs_x(KIND) || aligned16(x)) && (!act_needs_y(KIND) || aligned16(y));
+	if (al)
+		act_backward_kernel<T, KIND, true><<<stream_grid(n / Pack<T>::V), 256, 0, stream()>>>(n, p, x, y, g, dx);
+	else
+		act_backward_kernel<T, KIND, false><<<stream_grid(n), 256, 0, stream()>>>(n, p, x, y, g, dx);
+}
+
+/* Sum over the 64 lanes of a wavefront; the result is valid in lane 0. */
+template<typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+	#pragma unroll
+	for (int off = 32; off > 0; off >>= 1)
+		v += __shfl_down(v, off, 64);
+	return v;
+}
+
+/* Sum over a 256-thread block (4 wavefronts); the result is returned to every thread. */
+template<typename T>
+__device__ __forceinline__ T block_sum_256(T v, T* lds) {
+	v = wave_sum(v);
+	__syncthreads();
+	if (threadIdx.x % 64 == 0)
+		lds[threadIdx.x / 64] = v;
+	__syncthreads();
+	return ((lds[0] + lds[1]) + lds[2]) + lds[3];
+}
+
+/* ----------------------------------------------------------------------------------------------
+ * Softmax over the columns of an N x V column-major matrix, one thread per row
+ * (layer/activation/SoftmaxActivationLayer.hpp:49-78).
+ * -------------------------------------------------------------------------------------------- */
+template<typename T>
+__global__ void softmax_forward_kernel(int N, int V, T eps, const T* __restrict__ x, T* __restrict__ y) {
+	const int n = blockIdx.x * blockDim.x + threadIdx.x;
+	if (n >= N)
+		return;
+	T mx = x[n];
+	for (int v = 1; v < V; ++v) {
+		const T e = x[n + (size_t) N * v];
+		mx = e > mx ? e : mx;
+	}
+	T s = (T) 0;
+	for (int v = 0; v < V; ++v) {
+		const T e = dev_exp(x[n + (size_t) N * v] - mx);
+		y[n + (size_t) N * v] = e;
+		s += e;
+	}
+	const T d = s + eps;
+	for (int v = 0; v < V; ++v)
+		y[n + (size_t) N * v] /= d;
+}
+
+/* dx_j = sum_i g_i (delta_ij y_i - y_i y_j) = y_j (g_j - sum_i g_i y_i) */
+template<typename T>
+__global__ void softmax_backward_kernel(int N, int V, const T* __restrict__ y, const T* __restrict__ g, T* __restrict__ dx) {
+	const int n = blockIdx.x * blockDim.x + threadIdx.x;
+	if (n >= N)
+		return;
+	T dot = (T) 0;
+	for (int v = 0; v < V; ++v)
+		dot += g[n + (size_t) N * v] * y[n + (size_t) N * v];
+	for (int v = 0; v < V; ++v) {
+		const size_t i = n + (size_t) N * v;
+		dx[i] = y[i] * g[i] - y[i] * dot;
+	}
+}
+
+/* ----------------------------------------------------------------------------------------------
+ * PReLU / PSwish: per-activation parameter (1 x V), gradients are column sums over the batch
+ * (layer/activation/PReLUActivationLayer.hpp:80-109, PSwishActivationLayer.hpp:77-99).
+ * One wavefront per column for the backward pass.
+ * -------------------------------------------------------------------------------------------- */
+template<typename T, bool SWISH>
+__global__ __launch_bounds__(256)
+void param_act_forward_kernel(size_t total, int N, const T* __restrict__ param, const T* __restrict__ x, T* __restrict__ y) {
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		const T p = param[i / N], xi = x[i];
+		if (SWISH) {
+			y[i] = xi * ((T) 1 / (dev_exp(xi * (-p)) + (T) 1));
+		} else {
+			const T ax = xi * p;
+			y[i] = xi > ax ? xi : (ax == ax ? ax : xi);
+		}
+	}
+}
+
+template<typename T, bool SWISH>
+__global__ __launch_bounds__(256)
+void param_act_backward_kernel(int N, int V, const T* __restrict__ param, const T* __restrict__ x, const T* __restrict__ g,
+		T* __restrict__ param_grad, T* __restrict__ dx) {
+	const int v = blockIdx.x * 4 + threadIdx.x / 64;
+	if (v >= V)
+		return;
+	const int lane = threadIdx.x % 64;
+	const T p = param[v];
+	T acc = (T) 0;
+	for (int n = lane; n < N; n += 64) {
+		const size_t i = n + (size_t) N * v;
+		const T xi = x[i], gi = g[i];
+		if (SWISH) {
+			const T s = (T) 1 / (dev_exp(xi * (-p)) + (T) 1);
+			acc += s * ((T) 1 - s) * xi * xi * gi;
+			if (dx)
+				dx[i] = s * ((((T) 1 - s) * p) * xi + (T) 1) * gi;
+		} else {
+			if (xi >= (T) 0) {
+				if (dx)
+					dx[i] = gi;
+			} else {
+				if (dx)
+					dx[i] = p * gi;
+				acc += xi * gi;
+			}
+		}
+	}
+	acc = wave_sum(acc);
+	if (lane == 0)
+		param_grad[v] += acc;
+}
+
+/* ----------------------------------------------------------------------------------------------
+ * Batch norm (layer/BatchNormLayer.hpp:225-262 per channel, :411-456 per activation).
+ * A statistics group is a contiguous slab of L elements. grid = (groups, splits); split s covers
+ * [s*span, (s+1)*span) of the slab. Mean and variance are two separate passes (the variance is the
+ * mean of squared *centred* values, as in the reference), each a shuffle + LDS block reduction
+ * followed by an ascending sum of the per-split partials.
+ * -------------------------------------------------------------------------------------------- */
+template<typename T>
+__global__ __launch_bounds__(256)
+void bn_sum_kernel(size_t L, size_t span, const T* __restrict__ x, T* __restrict__ ws_sum) {
+	__shared__ T lds[4];
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
+	const T* xs = x + (size_t) blockIdx.x * L;
+	T s = (T) 0;
+	for (size_t i = begin + threadIdx.x; i < end; i += 256)
+		s += xs[i];
+	s = block_sum_256(s, lds);
+	if (threadIdx.x == 0)
+		ws_sum[(size_t) blockIdx.x * gridDim.y + blockIdx.y] = s;
+}
+
+template<typename T>
+__device__ __forceinline__ T sum_partials(const T* ws, int splits) {
+	T s = (T) 0;
+	for (int p = 0; p < splits; ++p)
+		s += ws[p];
+	return s;
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void bn_sqdev_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __restrict__ ws_sum, T* __restrict__ ws_sq) {
+	__shared__ T lds[4];
+	const int splits = gridDim.y;
+	const T mean = sum_partials(ws_sum + (size_t) blockIdx.x * splits, splits) / (T) L;
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
+	const T* xs = x + (size_t) blockIdx.x * L;
+	T s = (T) 0;
+	for (size_t i = begin + threadIdx.x; i < end; i += 256) {
+		const T d = xs[i] - mean;
+		s += d * d;
+	}
+	s = block_sum_256(s, lds);
+	if (threadIdx.x == 0)
+		ws_sq[(size_t) blockIdx.x * splits + blockIdx.y] = s;
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void bn_train_apply_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __restrict__ gamma,
+		const T* __restrict__ beta, T* __restrict__ avg_mean, T* __restrict__ avg_inv_sd, bool stats_init, T decay, T eps,
+		const T* __restrict__ ws_sum, const T* __restrict__ ws_sq, T* __restrict__ out, T* __restrict__ std_cache,
+		T* __restrict__ inv_sd_cache) {
+	const int splits = gridDim.y;
+	const int grp = blockIdx.x;
+	const T mean = sum_partials(ws_sum + (size_t) grp * splits, splits) / (T) L;
+	const T inv_sd = (T) 1 / dev_sqrt(sum_partials(ws_sq + (size_t) grp * splits, splits) / (T) L + eps);
+	const T ga = gamma[grp], be = beta[grp];
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
+	const T* xs = x + (size_t) grp * L;
+	T* ys = out + (size_t) grp * L;
+	T* sc = std_cache + (size_t) grp * L;
+	for (size_t i = begin + threadIdx.x; i < end; i += 256) {
+		const T sv = (xs[i] - mean) * inv_sd;
+		sc[i] = sv;
+		ys[i] = sv * ga + be;
+	}
+	if (blockIdx.y == 0 && threadIdx.x == 0) {
+		inv_sd_cache[grp] = inv_sd;
+		if (stats_init) {       /* running average (BatchNormLayer.hpp:234-238) */
+			avg_mean[grp] = ((T) 1 - decay) * avg_mean[grp] + decay * mean;
+			avg_inv_sd[grp] = ((T) 1 - decay) * avg_inv_sd[grp] + decay * inv_sd;
+		} else {                /* first call assigns (:239-243) */
+			avg_mean[grp] = mean;
+			avg_inv_sd[grp] = inv_sd;
+		}
+	}
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void bn_infer_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
+		const T* __restrict__ avg_mean, const T* __restrict__ avg_inv_sd, T* __restrict__ out) {
+	const int grp = blockIdx.x;
+	const T mean = avg_mean[grp], inv_sd = avg_inv_sd[grp], ga = gamma[grp], be = beta[grp];
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
+	const T* xs = x + (size_t) grp * L;
+	T* ys = out + (size_t) grp * L;
+	for (size_t i = begin + threadIdx.x; i < end; i += 256)
+		ys[i] = ((xs[i] - mean) * inv_sd) * ga + be;
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void bn_backward_sums_kernel(size_t L, size_t span, const T* __restrict__ g, const T* __restrict__ std_cache,
+		T* __restrict__ ws_g, T* __restrict__ ws_gs) {
+	__shared__ T lds[4];
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
+	const T* gs = g + (size_t) blockIdx.x * L;
+	const T* sc = std_cache + (size_t) blockIdx.x * L;
+	T s1 = (T) 0, s2 = (T) 0;
+	for (size_t i = begin + threadIdx.x; i < end; i += 256) {
+		const T gi = gs[i];
+		s1 += gi;
+		s2 += gi * sc[i];
+	}
+	s1 = block_sum_256(s1, lds);
+	s2 = block_sum_256(s2, lds);
+	if (threadIdx.x == 0) {
+		ws_g[(size_t) blockIdx.x * gridDim.y + blockIdx.y] = s1;
+		ws_gs[(size_t) blockIdx.x * gridDim.y + blockIdx.y] = s2;
+	}
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void bn_backward_apply_kernel(size_t L, size_t span, const T* __restrict__ g, const T* __restrict__ gamma,
+		const T* __restrict__ std_cache, const T* __restrict__ inv_sd_cache, const T* __restrict__ ws_g,
+		const T* __restrict__ ws_gs, T* __restrict__ gamma_grad, T* __restrict__ beta_grad, T* __restrict__ in_grad) {
+	const int splits = gridDim.y;
+	const int grp = blockIdx.x;
+	const T sum_g = sum_partials(ws_g + (size_t) grp * splits, splits);
+	const T sum_gs = sum_partials(ws_gs + (size_t) grp * splits, splits);
+	if (blockIdx.y == 0 && threadIdx.x == 0) {
+		gamma_grad[grp] += sum_gs;          /* BatchNormLayer.hpp:252-253 */
+		beta_grad[grp] += sum_g;            /* :254 */
+	}
+	if (!in_grad)
+		return;
+	const T ga = gamma[grp];
+	const T sum_sg = sum_g * ga, sum_ssg = sum_gs * ga;       /* sums of g*gamma and of std_in * g*gamma */
+	const T scale = ((T) 1 / (T) L) * inv_sd_cache[grp];      /* :260-261 */
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
+	const T* gs = g + (size_t) grp * L;
+	const T* sc = std_cache + (size_t) grp * L;
+	T* dx = in_grad + (size_t) grp * L;
+	for (size_t i = begin + threadIdx.x; i < end; i += 256)
+		dx[i] = (((T) L * (gs[i] * ga) - sum_sg) - sc[i] * sum_ssg) * scale;
+}
+
+constexpr int BN_MAX_SPLITS = 64;
+
+int bn_splits(int groups, size_t L) {
+	const size_t by_len = std::max<size_t>(1, L / 2048);
+	const size_t by_fill = std::max<size_t>(1, (size_t) 2048 / (size_t) std::max(1, groups));
+	return (int) std::min<size_t>(BN_MAX_SPLITS, std::min(by_len, by_fill));
+}
+
+/* ----------------------------------------------------------------------------------------------
+ * Pooling (layer/PoolLayer.hpp:77-116, layer/pool/MaxPoolLayer.hpp:38-80, MeanPoolLayer.hpp:35-41).
+ * One thread per output element (forward) or per input element (backward, gather form: each
+ * input sums the windows that cover it in the reference's patch order, so overlapping windows
+ * accumulate without atomics and in the reference's order of additions).
+ * -------------------------------------------------------------------------------------------- */
+template<typename T, bool MAX>
+__global__ __launch_bounds__(256)
+void pool_forward_kernel(PoolShape s, int N, int OH, int OW, const T* __restrict__ x, T* __restrict__ out,
+		unsigned* __restrict__ inds) {
+	const size_t total = (size_t) N * OH * OW * s.C;
+	const size_t idx = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+	if (idx >= total)
+		return;
+	const int n = (int) (idx % N);
+	size_t t = idx / N;
+	const int oh = (int) (t % OH);
+	t /= OH;
+	const int ow = (int) (t % OW);
+	const int c = (int) (t / OW);
+	const T* base = x + n + (size_t) N * ((size_t) oh * s.sv + (size_t) s.H * ((size_t) ow * s.sh + (size_t) s.W * c));
+	if (MAX) {
+		/* strict '>' from lowest(): first maximum in (width-major, height-minor) order wins and NaN
+		 * is never selected (MaxPoolLayer.hpp:45-56) */
+		T best = std::numeric_limits<T>::lowest();
+		unsigned bh = 0, bw = 0;
+		for (int k = 0; k < s.RW; ++k)
+			for (int l = 0; l < s.RH; ++l) {
+				const T v = base[(size_t) N * (l + (size_t) s.H * k)];
+				if (v > best) {
+					best = v;
+					bh = (unsigned) l;
+					bw = (unsigned) k;
+				}
+			}
+		out[idx] = best;
+		inds[((size_t) ow * OH + oh) * ((size_t) s.C * N) + (size_t) c * N + n] = bw * (unsigned) s.RH + bh;
+	} else {
+		T sum = (T) 0;
+		for (int k = 0; k < s.RW; ++k)
+			for (int l = 0; l < s.RH; ++l)
+				sum += base[(size_t) N * (l + (size_t) s.H * k)];
+		out[idx] = sum / (T) (s.RH * s.RW);
+	}
+}
+
+template<typename T, bool MAX>
+__global__ __launch_bounds__(256)
+void pool_backward_kernel(PoolShape s, int N, int OH, int OW, const T* __restrict__ g, const unsigned* __restrict__ inds,
+		T* __restrict__ dx) {
+	const size_t total = (size_t) N * s.H * s.W * s.C;
+	const size_t idx = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+	if (idx >= total)
+		return;
+	const int n = (int) (idx % N);
+	size_t t = idx / N;
+	const int h = (int) (t % s.H);
+	t /= s.H;
+	const int w = (int) (t % s.W);
+	const int c = (int) (t / s.W);
+	/* windows [o*stride, o*stride + R) containing the coordinate */
+	const int ow_lo = w >= s.RW ? (w - s.RW + s.sh) / s.sh : 0;
+	const int ow_hi = min(w / s.sh, OW - 1);
+	const int oh_lo = h >= s.RH ? (h - s.RH + s.sv) / s.sv : 0;
+	const int oh_hi = min(h / s.sv, OH - 1);
+	const T area = (T) (s.RH * s.RW);
+	T sum = (T) 0;
+	for (int ow = ow_lo; ow <= ow_hi; ++ow)
+		for (int oh = oh_lo; oh <= oh_hi; ++oh) {
+			const T gv = g[n + (size_t) N * (oh + (size_t) OH * (ow + (size_t) OW * c))];
+			if (MAX) {
+				const unsigned ind = inds[((size_t) ow * OH + oh) * ((size_t) s.C * N) + (size_t) c * N + n];
+				const unsigned mine = (unsigned) (w - ow * s.sh) * (unsigned) s.RH + (unsigned) (h - oh * s.sv);
+				sum += ind == mine ? gv : (T) 0;
+			} else {
+				sum += gv / area;
+			}
+		}
+	dx[idx] = sum;
+}
+
+template<typename T>
+__global__ void axpy_one_kernel(size_t n, const T* __restrict__ src, T* __restrict__ dst) {
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+		dst[i] += src[i];
+}
+
+void check_launch() {
+	CATTLE_HIP_CHECK(hipGetLastError());
+}
+
+} /* namespace */
+
+template<typename T>
+void act_forward(int kind, size_t n, T p, const T* x, T* y) {
+	if (n == 0)
+		return;
+	switch (kind) {
+	case ACT_IDENTITY: act_forward_kind<T, ACT_IDENTITY>(n, p, x, y); break;
+	case ACT_SCALED: act_forward_kind<T, ACT_SCALED>(n, p, x, y); break;
+	case ACT_BINARY_STEP: act_forward_kind<T, ACT_BINARY_STEP>(n, p, x, y); break;
+	case ACT_SIGMOID: act_forward_kind<T, ACT_SIGMOID>(n, p, x, y); break;
+	case ACT_TANH: act_forward_kind<T, ACT_TANH>(n, p, x, y); break;
+	case ACT_SOFTSIGN: act_forward_kind<T, ACT_SOFTSIGN>(n, p, x, y); break;
+	case ACT_SOFTPLUS: act_forward_kind<T, ACT_SOFTPLUS>(n, p, x, y); break;
+	case ACT_RELU: act_forward_kind<T, ACT_RELU>(n, p, x, y); break;
+	case ACT_LEAKY_RELU: act_forward_kind<T, ACT_LEAKY_RELU>(n, p, x, y); break;
+	case ACT_ELU: act_forward_kind<T, ACT_ELU>(n, p, x, y); break;
+	case ACT_SWISH: act_forward_kind<T, ACT_SWISH>(n, p, x, y); break;
+	default: throw Error(ERR_INVALID, "unknown activation kind");
+	}
+	check_launch();
+}
+
+template<typename T>
+void act_backward(int kind, size_t n, T p, const T* x, const T* y, const T* g, T* dx) {
+	if (n == 0)
+		return;
+	switch (kind) {
+	case ACT_IDENTITY: act_backward_kind<T, ACT_IDENTITY>(n, p, x, y, g, dx); break;
+	case ACT_SCALED: act_backward_kind<T, ACT_SCALED>(n, p, x, y, g, dx); break;
+	case ACT_BINARY_STEP: act_backward_kind<T, ACT_BINARY_STEP>(n, p, x, y, g, dx); break;
+	case ACT_SIGMOID: act_backward_kind<T, ACT_SIGMOID>(n, p, x, y, g, dx); break;
+	case ACT_TANH: act_backward_kind<T, ACT_TANH>(n, p, x, y, g, dx); break;
+	case ACT_SOFTSIGN: act_backward_kind<T, ACT_SOFTSIGN>(n, p, x, y, g, dx); break;
+	case ACT_SOFTPLUS: act_backward_kind<T, ACT_SOFTPLUS>(n, p, x, y, g, dx); break;
+	case ACT_RELU: act_backward_kind<T, ACT_RELU>(n, p, x, y, g, dx); break;
+	case ACT_LEAKY_RELU: act_backward_kind<T, ACT_LEAKY_RELU>(n, p, x, y, g, dx); break;
+	case ACT_ELU: act_backward_kind<T, ACT_ELU>(n, p, x, y, g, dx); break;
+	case ACT_SWISH: act_backward_kind<T, ACT_SWISH>(n, p, x, y, g, dx); break;
+	default: throw Error(ERR_INVALID, "unknown activation kind");
+	}
+	check_launch();
+}
+
+template<typename T>
+void softmax_forward(int N, int V, T eps, const T* x, T* y) {
+	softmax_forward_kernel<T><<<(unsigned) ((N + 63) / 64), 64, 0, stream()>>>(N, V, eps, x, y);
+	check_launch();
+}
+
+template<typename T>
+void softmax_backward(int N, int V, const T* y, const T* g, T* dx) {
+	softmax_backward_kernel<T><<<(unsigned) ((N + 63) / 64), 64, 0, stream()>>>(N, V, y, g, dx);
+	check_launch();
+}
+
+template<typename T>
+void prelu_forward(int N, int V, const T* alpha, const T* x, T* y) {
+	const size_t total = (size_t) N * V;
+	param_act_forward_kernel<T, false><<<stream_grid(total), 256, 0, stream()>>>(total, N, alpha, x, y);
+	check_launch();
+}
+
+template<typename T>
+void prelu_backward(int N, int V, const T* alpha, const T* x, const T* g, T* alpha_grad, T* dx) {
+	param_act_backward_kernel<T, false><<<(unsigned) ((V + 3) / 4), 256, 0, stream()>>>(N, V, alpha, x, g, alpha_grad, dx);
+	check_launch();
+}
+
+template<typename T>
+void pswish_forward(int N, int V, const T* beta, const T* x, T* y) {
+	const size_t total = (size_t) N * V;
+	param_act_forward_kernel<T, true><<<stream_grid(total), 256, 0, stream()>>>(total, N, beta, x, y);
+	check_launch();
+}
+
+template<typename T>
+void pswish_backward(int N, int V, const T* beta, const T* x, const T* g, T* beta_grad, T* dx) {
+	param_act_backward_kernel<T, true><<<(unsigned) ((V + 3) / 4), 256, 0, stream()>>>(N, V, beta, x, g, beta_grad, dx);
+	check_launch();
+}
+
+size_t bn_workspace(int groups, size_t L) {
+	(void) L;
+	return (size_t) 2 * groups * BN_MAX_SPLITS;
+}
+
+template<typename T>
+void bn_forward(int groups, size_t L, const T* x, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd,
+		bool stats_init, bool training, T decay, T eps, T* out, T* std_cache, T* inv_sd_cache, T* ws) {
+	const int splits = bn_splits(groups, L);
+	const size_t span = (L + splits - 1) / splits;
+	dim3 grid((unsigned) groups, (unsigned) splits);
+	if (training) {
+		T* ws_sum = ws;
+		T* ws_sq = ws + (size_t) groups * BN_MAX_SPLITS;
+		bn_sum_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, ws_sum);
+		check_launch();
+		bn_sqdev_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, ws_sum, ws_sq);
+		check_launch();
+		bn_train_apply_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, gamma, beta, avg_mean, avg_inv_sd, stats_init, decay,
+				eps, ws_sum, ws_sq, out, std_cache, inv_sd_cache);
+		check_launch();
+	} else {
+		bn_infer_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, gamma, beta, avg_mean, avg_inv_sd, out);
+		check_launch();
+	}
+}
+
+template<typename T>
+void bn_backward(int groups, size_t L, const T* out_grad, const T* gamma, const T* std_cache, const T* inv_sd_cache,
+		T* gamma_grad, T* beta_grad, T* in_grad, T* ws) {
+	const int splits = bn_splits(groups, L);
+	const size_t span = (L + splits - 1) / splits;
+	dim3 grid((unsigned) groups, (unsigned) splits);
+	T* ws_g = ws;
+	T* ws_gs = ws + (size_t) groups * BN_MAX_SPLITS;
+	bn_backward_sums_kernel<T><<<grid, 256, 0, stream()>>>(L, span, out_grad, std_cache, ws_g, ws_gs);
+	check_launch();
+	bn_backward_apply_kernel<T><<<grid, 256, 0, stream()>>>(L, span, out_grad, gamma, std_cache, inv_sd_cache, ws_g, ws_gs,
+			gamma_grad, beta_grad, in_grad);
+	check_launch();
+}
+
+template<typename T>
+void maxpool_forward(const PoolShape& s, int N, const T* x, T* out, unsigned* inds) {
+	const size_t total = (size_t) N * s.OH() * s.OW() * s.C;
+	pool_forward_kernel<T, true><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), x, out, inds);
+	check_launch();
+}
+
+template<typename T>
+void maxpool_backward(const PoolShape& s, int N, const T* out_grad, const unsigned* inds, T* in_grad) {
+	const size_t total = (size_t) N * s.H * s.W * s.C;
+	pool_backward_kernel<T, true><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), out_grad, inds,
+			in_grad);
+	check_launch();
+}
+
+template<typename T>
+void meanpool_forward(const PoolShape& s, int N, const T* x, T* out) {
+	const size_t total = (size_t) N * s.OH() * s.OW() * s.C;
+	pool_forward_kernel<T, false><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), x, out, nullptr);
+	check_launch();
+}
+
+template<typename T>
+void meanpool_backward(const PoolShape& s, int N, const T* out_grad, T* in_grad) {
+	const size_t total = (size_t) N * s.H * s.W * s.C;
+	pool_backward_kernel<T, false><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), out_grad,
+			nullptr, in_grad);
+	check_launch();
+}
+
+template<typename T>
+void axpy_one(size_t n, const T* src, T* dst) {
+	if (n == 0)
+		return;
+	axpy_one_kernel<T><<<stream_grid(n), 256, 0, stream()>>>(n, src, dst);
+	check_launch();
+}
+
+#define CATTLE_HIP_INSTANTIATE(T) \
+template void act_forward<T>(int, size_t, T, const T*, T*); \
+template void act_backward<T>(int, size_t, T, const T*, const T*, const T*, T*); \
+template void softmax_forward<T>(int, int, T, const T*, T*); \
+template void softmax_backward<T>(int, int, const T*, const T*, T*); \
+template void prelu_forward<T>(int, int, const T*, const T*, T*); \
+template void prelu_backward<T>(int, int, const T*, const T*, const T*, T*, T*); \
+template void pswish_forward<T>(int, int, const T*, const T*, T*); \
+template void pswish_backward<T>(int, int, const T*, const T*, const T*, T*, T*); \
+template void bn_forward<T>(int, size_t, const T*, const T*, const T*, T*, T*, bool, bool, T, T, T*, T*, T*, T*); \
+template void bn_backward<T>(int, size_t, const T*, const T*, const T*, const T*, T*, T*, T*, T*); \
+template void maxpool_forward<T>(const PoolShape&, int, const T*, T*, unsigned*); \
+template void maxpool_backward<T>(const PoolShape&, int, const T*, const unsigned*, T*); \
+template void meanpool_forward<T>(const PoolShape&, int, const T*, T*); \
+template void meanpool_backward<T>(const PoolShape&, int, const T*, T*); \
+template void axpy_one<T>(size_t, const T*, T*);
+
+CATTLE_HIP_INSTANTIATE(float)
+CATTLE_HIP_INSTANTIATE(double)
+
+} /* namespace cattle_hip */

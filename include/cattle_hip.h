@@ -1,0 +1,184 @@
+/*
+ * cattle_hip.h — C ABI of libcattle_hip.so: MI355X (gfx950) kernels for C-ATTL3's kernel-layer
+ * hot path behind the contract of cattle::Layer<Scalar,Rank>.
+ *
+ * A layer handle is the device-side twin of one cattle::Layer object: it owns the forward caches
+ * the reference layer keeps, device copies of the layer's parameters and an accumulating gradient
+ * buffer per parameter. Citations name the reference interface each entry point stands in for
+ * (paths relative to the reference's C-ATTL3/ directory).
+ *
+ * Data layout: every tensor is the reference's column-major buffer whose index order is
+ * (N, H, W, C): offset(n,h,w,c) = n + N*(h + H*(w + W*c)) (core/EigenProxy.hpp:43-64). Rank-1 and
+ * rank-2 layers pass their data re-viewed as (N,H,1,1) / (N,H,W,1) exactly as the reference does
+ * (layer/kernel/ConvKernelLayer.hpp:400-417, :494-508). Matrices are column-major.
+ *
+ * Every function returns CATTLE_HIP_OK or an error code; cattle_hip_last_error() then returns a
+ * message for the calling thread. Calls are serialised internally, so distinct layers may be
+ * driven from different host threads (neural_network/ParallelNeuralNetwork.hpp:158-171); a single
+ * layer is not re-entrant, as in the reference. No entry point falls back to host computation: if
+ * no MI355X is usable, cattle_hip_init() fails and so does everything after it.
+ */
+#ifndef CATTLE_HIP_H_
+#define CATTLE_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cattle_hip_layer_s* cattle_hip_layer_t;
+typedef struct cattle_hip_timer_s* cattle_hip_timer_t;
+
+enum {
+	CATTLE_HIP_OK = 0,
+	CATTLE_HIP_ERR_INVALID = 1,   /* bad argument or dimension mismatch (the reference asserts) */
+	CATTLE_HIP_ERR_STATE = 2,     /* e.g. backward without a matching forward */
+	CATTLE_HIP_ERR_DEVICE = 3,    /* HIP runtime failure */
+	CATTLE_HIP_ERR_OOM = 4        /* device allocation failed */
+};
+
+/* Scalar of Layer<Scalar,Rank> (core/Layer.hpp:32). */
+typedef enum { CATTLE_HIP_F32 = 0, CATTLE_HIP_F64 = 1 } cattle_hip_dtype;
+
+/* Where a buffer argument lives. HOST buffers are pageable host memory (an Eigen tensor's data());
+ * they are staged through device buffers owned by the layer. DEVICE buffers are used in place;
+ * a DEVICE input that a layer caches for its backward pass (the layer input of conv, dense, ReLU,
+ * ..., or the output of sigmoid/tanh) is borrowed, not copied: it must stay valid and unmodified
+ * until the matching backward call or cattle_hip_layer_empty_cache(). */
+typedef enum { CATTLE_HIP_HOST = 0, CATTLE_HIP_DEVICE = 1 } cattle_hip_memspace;
+
+/* Activation layers of layer/activation/<Name>ActivationLayer.hpp. */
+typedef enum {
+	CATTLE_HIP_ACT_IDENTITY = 0, CATTLE_HIP_ACT_SCALED = 1, CATTLE_HIP_ACT_BINARY_STEP = 2,
+	CATTLE_HIP_ACT_SIGMOID = 3, CATTLE_HIP_ACT_TANH = 4, CATTLE_HIP_ACT_SOFTSIGN = 5,
+	CATTLE_HIP_ACT_SOFTPLUS = 6, CATTLE_HIP_ACT_RELU = 7, CATTLE_HIP_ACT_LEAKY_RELU = 8,
+	CATTLE_HIP_ACT_ELU = 9, CATTLE_HIP_ACT_SWISH = 10, CATTLE_HIP_ACT_SOFTMAX = 11,
+	CATTLE_HIP_ACT_PRELU = 12, CATTLE_HIP_ACT_PSWISH = 13
+} cattle_hip_activation;
+
+typedef enum { CATTLE_HIP_POOL_MAX = 0, CATTLE_HIP_POOL_MEAN = 1 } cattle_hip_pool;
+
+/* ---- library ---------------------------------------------------------------------------- */
+
+/* Selects the device and creates the library's stream. Fails unless the device is a gfx950. */
+int cattle_hip_init(int device);
+const char* cattle_hip_last_error(void);
+/* Waits for all work issued by the library. */
+int cattle_hip_synchronize(void);
+
+/* Plain device memory for callers that keep activations resident between layers (the idea of
+ * core/gpu/GPULayer.hpp:31-58: device-tensor overloads next to the host-tensor virtuals). */
+int cattle_hip_alloc(void** device_ptr, size_t bytes);
+int cattle_hip_free(void* device_ptr);
+int cattle_hip_upload(void* dst_device, const void* src_host, size_t bytes);
+int cattle_hip_download(void* dst_host, const void* src_device, size_t bytes);
+int cattle_hip_fill_zero(void* dst_device, size_t bytes);
+
+/* Event timers on the library's stream (for benchmarks: kernel time with data resident). */
+int cattle_hip_timer_create(cattle_hip_timer_t* timer);
+int cattle_hip_timer_destroy(cattle_hip_timer_t timer);
+int cattle_hip_timer_start(cattle_hip_timer_t timer);
+int cattle_hip_timer_stop(cattle_hip_timer_t timer, float* elapsed_ms);   /* synchronises */
+
+/* ---- layer construction ------------------------------------------------------------------ */
+
+/* ConvKernelLayer<Scalar,Rank>(input_dims, filters, init, receptor_height, receptor_width,
+ * vertical_padding, horizontal_padding, vertical_stride, horizontal_stride, vertical_dilation,
+ * horizontal_dilation) — layer/kernel/ConvKernelLayer.hpp:282-296 (rank 2 :342-357, rank 1
+ * :441-456). Dilation 0 means a dense receptor (:71-72). Parameters: 0 = weights
+ * [receptor_height*receptor_width*channels x filters] with row index rh + RH*(rw + RW*c)
+ * (:138-139), 1 = bias [1 x filters] (:48-55). */
+int cattle_hip_conv_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, size_t filters,
+		size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
+		cattle_hip_layer_t* layer);
+
+/* DenseKernelLayer<Scalar,Rank>(input_dims, output_size, init) — layer/kernel/DenseKernelLayer.hpp:61-77.
+ * input_volume = input_dims.get_volume(). Parameters: 0 = weights [input_volume x output_size],
+ * 1 = bias [1 x output_size]. */
+int cattle_hip_dense_create(cattle_hip_dtype dtype, size_t input_volume, size_t output_size, cattle_hip_layer_t* layer);
+
+/* BatchNormLayer<Scalar,Rank,PerLastRank>(dims, norm_avg_decay, epsilon) — layer/BatchNormLayer.hpp:66-101
+ * (per_last_rank != 0: one statistics group per channel) and :334-361 (per_last_rank == 0: one per
+ * activation). Parameters, each [1 x groups]: 0 = running means, 1 = running inverse standard
+ * deviations (both not optimizable), 2 = gammas, 3 = betas — the order of get_params() (:263-272,
+ * :399-406); the per-channel reference layer holds them as `groups` separate 1x1 matrices. */
+int cattle_hip_batchnorm_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, int per_last_rank,
+		double norm_avg_decay, double epsilon, cattle_hip_layer_t* layer);
+/* The avgs_init flag of the reference layer (BatchNormLayer.hpp:234-243): whether the running
+ * statistics hold values yet. A fresh layer starts at 0; clones copy it. */
+int cattle_hip_batchnorm_get_stats_initialized(cattle_hip_layer_t layer, int* initialized);
+int cattle_hip_batchnorm_set_stats_initialized(cattle_hip_layer_t layer, int initialized);
+
+/* <Name>ActivationLayer<Scalar,Rank>(dims[, param]) — layer/activation/<Name>ActivationLayer.hpp; volume =
+ * dims.get_volume(). param is the scale (Scaled), alpha (LeakyReLU, ELU), beta (Swish), epsilon
+ * (Softmax), or the initial alpha / beta of PReLU / PSwish, whose parameter 0 is [1 x volume]
+ * (PReLUActivationLayer.hpp:62-65, PSwishActivationLayer.hpp:59-62); ignored otherwise. */
+int cattle_hip_activation_create(cattle_hip_dtype dtype, cattle_hip_activation kind, size_t volume, double param,
+		cattle_hip_layer_t* layer);
+
+/* MaxPoolLayer / MeanPoolLayer<Scalar,Rank>(input_dims, receptor_height, receptor_width,
+ * vertical_stride, horizontal_stride) — layer/pool/MaxPoolLayer.hpp:105-108,
+ * layer/pool/MeanPoolLayer.hpp:62-65, geometry in layer/PoolLayer.hpp:53-76, :145-155. */
+int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t height, size_t width, size_t channels,
+		size_t receptor_height, size_t receptor_width, size_t vertical_stride, size_t horizontal_stride,
+		cattle_hip_layer_t* layer);
+
+/* ---- the cattle::Layer contract (core/Layer.hpp:47-137) ------------------------------------- */
+
+/* Layer::clone() (:47) when share_params == 0: deep copy including parameter values and gradients;
+ * Layer::clone_with_shared_params() (:56) otherwise: the clone refers to the same device parameter
+ * and gradient buffers (layer/KernelLayer.hpp:71-77). Forward caches are not copied. */
+int cattle_hip_layer_clone(cattle_hip_layer_t layer, int share_params, cattle_hip_layer_t* clone);
+int cattle_hip_layer_destroy(cattle_hip_layer_t layer);
+
+/* Layer::get_input_dims() / get_output_dims() (:73, :80), always as (height, width, channels). */
+int cattle_hip_layer_input_dims(cattle_hip_layer_t layer, size_t dims[3]);
+int cattle_hip_layer_output_dims(cattle_hip_layer_t layer, size_t dims[3]);
+
+/* Layer::is_input_layer() / set_input_layer() (:90, :96). An input layer skips the input gradient. */
+int cattle_hip_layer_is_input_layer(cattle_hip_layer_t layer, int* is_input_layer);
+int cattle_hip_layer_set_input_layer(cattle_hip_layer_t layer, int is_input_layer);
+
+/* Layer::empty_cache() (:101). */
+int cattle_hip_layer_empty_cache(cattle_hip_layer_t layer);
+
+/* Layer::pass_forward(Data in, bool training) (:126). in holds batch * volume(input dims) scalars,
+ * out receives batch * volume(output dims) scalars. */
+int cattle_hip_layer_forward(cattle_hip_layer_t layer, const void* in, cattle_hip_memspace in_space, size_t batch,
+		int training, void* out, cattle_hip_memspace out_space);
+
+/* Layer::pass_back(Data out_grad) (:137). Must follow a forward call with the same batch size.
+ * Parameter gradients ACCUMULATE into the layer's gradient buffers, as Parameters::accumulate_grad
+ * does (parameters/StandardParameters.hpp:115-123). in_grad may be NULL exactly when the layer is
+ * an input layer (the reference then returns a null tensor); it is never written in that case.
+ * Exception kept from the reference: PReLU computes the input gradient even as an input layer
+ * (PReLUActivationLayer.hpp:87-109), so it requires in_grad unless it is NULL by choice. */
+int cattle_hip_layer_backward(cattle_hip_layer_t layer, const void* out_grad, cattle_hip_memspace grad_space, size_t batch,
+		void* in_grad, cattle_hip_memspace in_grad_space);
+
+/* ---- Parameters (core/Parameters.hpp:15-95) ------------------------------------------------- */
+
+/* Layer::get_params().size() (core/Layer.hpp:107-113). */
+int cattle_hip_layer_num_params(cattle_hip_layer_t layer, size_t* count);
+/* Parameters::get_rows() / get_cols() / are_optimizable(). */
+int cattle_hip_layer_param_shape(cattle_hip_layer_t layer, size_t index, size_t* rows, size_t* cols, int* optimizable);
+/* Parameters::set_values(Matrix) / get_values(): column-major rows x cols scalars. */
+int cattle_hip_layer_set_param_values(cattle_hip_layer_t layer, size_t index, const void* values, cattle_hip_memspace space);
+int cattle_hip_layer_get_param_values(cattle_hip_layer_t layer, size_t index, void* values, cattle_hip_memspace space);
+/* Parameters::get_grad(): the gradient accumulated by backward calls since the last reset. */
+int cattle_hip_layer_get_param_grad(cattle_hip_layer_t layer, size_t index, void* grad, cattle_hip_memspace space);
+/* Parameters::reset_grad(). */
+int cattle_hip_layer_reset_param_grad(cattle_hip_layer_t layer, size_t index);
+
+/* The argmax cache of MaxPoolLayer (layer/pool/MaxPoolLayer.hpp:58-62, :82): OH*OW rows of
+ * channels*batch unsigned entries, row = ow*OH + oh, column = c*batch + n, value =
+ * w_in_window*receptor_height + h_in_window. Valid after a forward call. */
+int cattle_hip_maxpool_indices(cattle_hip_layer_t layer, unsigned* indices, cattle_hip_memspace space);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CATTLE_HIP_H_ */
