@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Benchmark of the kernel-layer hot path on one MI355X.
+
+Workload (BASELINE.json configs[3], the shape north_star's target is stated on):
+ConvKernelLayer<float,3> forward + backward (weight, bias and input gradients), batch 256, input
+NHWC 56x56x64 drawn from N(0,1), 128 filters 3x3, stride 1, padding 1, He-normal weights, upstream
+gradient N(0,1). One step = one pass_forward + one pass_back on tensors already resident in HBM.
+
+Prints one JSON line: whole-step throughput in GFLOP/s (algorithmic FLOP = 6*M*K*F per step),
+samples/s, the MFMA roofline of the slowest GEMM kernel (measured with HIP events on the library's
+stream) and the CPU baseline (the oracle's restatement of the reference algorithm on the host
+cores, on a bounded sample of the same workload).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}      # MI355X dense matrix peaks (no sparsity)
+SHAPE = dict(H=56, W=56, C=64, F=128, RH=3, RW=3)
+
+
+def he_normal(gen, rows, cols, dtype):
+    # parameter_initialization/HeParameterInitialization.hpp:34-36: sd = sqrt(2 / fan_in), fan_in = rows
+    return np.asfortranarray((gen.standard_normal((rows, cols)) * np.sqrt(2.0 / rows)).astype(dtype))
+
+
+def gpu_run(args, dtype):
+    ch = importlib.import_module("c-attl3_amd")
+    ch.init(0)
+    N, H, W, C, F = args.batch, SHAPE["H"], SHAPE["W"], SHAPE["C"], SHAPE["F"]
+    K = SHAPE["RH"] * SHAPE["RW"] * C
+    M = N * H * W
+    gen = np.random.default_rng(0xC0FFEE04)
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F)
+    layer.get_params()[0].set_values(he_normal(gen, K, F, dtype))
+    x = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H, W, C)).astype(dtype)))
+    go = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H, W, F)).astype(dtype)))
+    out = ch.DeviceTensor((N, H, W, F), dtype)
+    dx = ch.DeviceTensor((N, H, W, C), dtype)
+
+    def step():
+        layer.forward_into(x, out, True)
+        layer.backward_into(go, dx)
+
+    for _ in range(args.warmup):
+        step()
+    ch.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ch.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-kernel durations with HIP events on the library's stream
+    timer = ch.Timer()
+    reps = max(3, args.steps)
+
+    def timed(fn):
+        fn()
+        timer.start()
+        for _ in range(reps):
+            fn()
+        return timer.stop() / reps
+
+    t_fwd = timed(lambda: layer.forward_into(x, out, True))
+    t_bwd = timed(lambda: layer.backward_into(go, dx))
+    layer.set_input_layer(True)
+    t_wgrad = timed(lambda: layer.backward_into(go, None))         # weight + bias gradient only
+    layer.set_input_layer(False)
+    t_dgrad = max(t_bwd - t_wgrad, 1e-6)
+    gemm_flop = 2.0 * M * K * F
+    kernels = {
+        "gather_gemm_kernel (forward)": t_fwd,
+        "wgrad_kernel (+ reduce, bias column sums)": t_wgrad,
+        "gather_gemm_kernel (input gradient)": t_dgrad,
+    }
+    if args.copy_calibration:
+        # a plain copy kernel of known size (identity activation: reads and writes x.nbytes) so that
+        # FETCH_SIZE / WRITE_SIZE counter readings of the same profile can be scaled to bytes
+        ident = ch.ActivationLayer(dtype, "identity", (H, W, C))
+        for _ in range(3):
+            ident.forward_into(x, dx, True)
+        ch.synchronize()
+    return dict(wall_ms=wall_ms, M=M, K=K, F=F, gemm_flop=gemm_flop, kernels=kernels)
+
+
+def cpu_baseline(args, dtype):
+    """Times the oracle (the restatement of the reference algorithm: explicit patch matrix + GEMMs +
+    col2im, OpenMP GEMMs) on a bounded sample: the same layer at a smaller batch."""
+    from oracle import oracle
+    N = args.cpu_batch
+    H, W, C, F = SHAPE["H"], SHAPE["W"], SHAPE["C"], SHAPE["F"]
+    K = 9 * C
+    gen = np.random.default_rng(0xC0FFEE04)
+    w = he_normal(gen, K, F, dtype)
+    b = np.zeros((1, F), dtype)
+    x = np.asfortranarray(gen.standard_normal((N, H, W, C)).astype(dtype))
+    go = np.asfortranarray(gen.standard_normal((N, H, W, F)).astype(dtype))
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        _, cache = oracle.conv_forward(x, w, b, return_cache=True)
+        oracle.conv_backward(x.shape, cache, w, go)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    flop = 6.0 * N * H * W * K * F
+    return {
+        "value": round(flop / best / 1e9, 2), "unit": "GFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+        "sample": "same layer at batch %d (1/%d of the workload), best of 3, %.2f s per fwd+bwd, %.1f samples/s"
+                  % (N, max(1, args.batch // N), best, N / best),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=256)
+    ap.add_argument("--dtype", choices=["f32", "f64"], default="f32")
+    ap.add_argument("--cpu-batch", type=int, default=256)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain copy kernel of x's size (for scaling rocprof byte counters)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
+    dtype = np.float32 if args.dtype == "f32" else np.float64
+
+    r = gpu_run(args, dtype)
+    step_flop = 3.0 * r["gemm_flop"]
+    gflops = step_flop / (r["wall_ms"] * 1e-3) / 1e9
+    peak = PEAK_TFLOPS[args.dtype]
+    name, t_ms = max(r["kernels"].items(), key=lambda kv: kv[1])
+    achieved = r["gemm_flop"] / (t_ms * 1e-3) / 1e12
+    line = {
+        "metric": "conv_fwd_bwd_gflops", "value": round(gflops, 1), "unit": "GFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r["wall_ms"], 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "ConvKernelLayer<%s,3> fwd+bwd, batch %d, NHWC 56x56x64 -> 128 filters 3x3 s1 p1 "
+                               "(BASELINE configs[3])" % ("float" if args.dtype == "f32" else "double", args.batch),
+                   "M": r["M"], "K": r["K"], "F": r["F"], "flop_per_step": step_flop},
+        "samples_per_s": round(args.batch / (r["wall_ms"] * 1e-3), 1),
+        "frac_of_mfma_peak": round(gflops / 1e3 / peak, 4),
+        "roofline": {"bound": "mfma", "kernel": name, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "flop_per_launch": r["gemm_flop"], "ms_per_launch": round(t_ms, 4)},
+        "kernel_ms": {k: round(v, 4) for k, v in r["kernels"].items()},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args, dtype)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

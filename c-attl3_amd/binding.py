@@ -249,6 +249,16 @@ class Layer(object):
                                               ctypes.c_int(int(training)), ctypes.c_void_p(out.ctypes.data), HOST))
         return out
 
+    def forward_into(self, x, out, training=True):
+        """Device path without allocation: x and out are DeviceTensors owned by the caller."""
+        _check(lib().cattle_hip_layer_forward(self._h, x.ptr, DEVICE, _sz(x.shape[0]), ctypes.c_int(int(training)), out.ptr,
+                                              DEVICE))
+
+    def backward_into(self, out_grad, in_grad):
+        """Device path without allocation; in_grad may be None for an input layer."""
+        _check(lib().cattle_hip_layer_backward(self._h, out_grad.ptr, DEVICE, _sz(out_grad.shape[0]),
+                                               None if in_grad is None else in_grad.ptr, DEVICE))
+
     def pass_back(self, out_grad):
         """Returns the input gradient, or None for an input layer (the reference's null tensor)."""
         skip = self.is_input_layer() and not getattr(self, "_always_backprop", False)
