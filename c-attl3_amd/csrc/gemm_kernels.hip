@@ -8,8 +8,8 @@
  *
  *   gather_gemm_kernel   out[M x F] = A[M x K] * Wt[K x F] (+ bias)     forward and input gradient
  *   wgrad_kernel         P_s[K x F] = A_s^T * G_s over a slice s of M    weight gradient partials
- *   reduce_partials      dW += sum_s P_s in fixed order                 deterministic, no atomics
- *   colsum kernels       db += column sums of G                         bias gradient
+ *                        (+ bias-gradient partials: column sums of G from the tile already in LDS)
+ *   reduce_partials      dW += sum_s P_s, db += sum_s p_s in fixed order    deterministic, no atomics
  *
  * MFMA operand convention used throughout: the matrix instruction computes D[i][j] += A[i][k]*B[k][j]
  * with lane l holding A[i = l % TL][k = l / TL] and B[k = l / TL][j = l % TL]; accumulator register r
@@ -19,6 +19,8 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <cstdlib>
+#include <string>
 #include <type_traits>
 
 namespace cattle_hip {
@@ -223,20 +225,30 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		const int buf = c & 1;
 		if (c + 1 < nchunks)
 			load_tiles((c + 1) * KC);
+		/* operand fragments are fetched one reduction step ahead of the MFMAs that use them */
+		T xa[2][MB], wb[2][FB];
 		#pragma unroll
-		for (int kk = 0; kk < KC; kk += KS) {
-			T xa[MB], wb[FB];
-			#pragma unroll
-			for (int j = 0; j < MB; ++j)
-				xa[j] = As[buf][kk + lk][wm * WT_M + j * TL + lc];
-			#pragma unroll
-			for (int i = 0; i < FB; ++i)
-				wb[i] = Bs[buf][kk + lk][wf * WT_F + i * TL + lc];
+		for (int j = 0; j < MB; ++j)
+			xa[0][j] = As[buf][lk][wm * WT_M + j * TL + lc];
+		#pragma unroll
+		for (int i = 0; i < FB; ++i)
+			wb[0][i] = Bs[buf][lk][wf * WT_F + i * TL + lc];
+		#pragma unroll
+		for (int st = 0; st < KC / KS; ++st) {
+			const int cur = st & 1, nxt = cur ^ 1;
+			if (st + 1 < KC / KS) {
+				#pragma unroll
+				for (int j = 0; j < MB; ++j)
+					xa[nxt][j] = As[buf][(st + 1) * KS + lk][wm * WT_M + j * TL + lc];
+				#pragma unroll
+				for (int i = 0; i < FB; ++i)
+					wb[nxt][i] = Bs[buf][(st + 1) * KS + lk][wf * WT_F + i * TL + lc];
+			}
 			#pragma unroll
 			for (int i = 0; i < FB; ++i)
 				#pragma unroll
 				for (int j = 0; j < MB; ++j)
-					acc[i][j] = MF::mma(wb[i], xa[j], acc[i][j]);
+					acc[i][j] = MF::mma(wb[cur][i], xa[cur][j], acc[i][j]);
 		}
 		if (c + 1 < nchunks)
 			store_tiles(buf ^ 1);
@@ -263,16 +275,20 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 }
 
 /* ------------------------------------------------------------------------------------------------
- * Weight-gradient partials: P[k + K*f] = sum over this block's slice of m of A(m,k) * G(m,f).
+ * Weight-gradient partials: P[k + K*f] = sum over this block's slice of m of A(m,k) * G(m,f), plus the
+ * bias-gradient partials (column sums of G over the same slice) from the G tile already in LDS.
  * The reduction index m is the contiguous one, so both operand tiles are staged as [row][m] and a
  * lane fetches VR consecutive m with one 16-byte LDS read; since a sum may be taken in any order,
  * MFMA step e pairs reduction slot lk with m = mm + lk*VR + e for both operands.
- * grid = (ktiles * ftiles, splits).
+ * The LDS tile is single-buffered: the global loads of the next chunk are in flight in registers
+ * while the current chunk is multiplied, and two to three blocks per CU cover the barriers.
+ * grid = (ktiles * ftiles, splits). Bias rows are dealt out over the k tiles (row f belongs to the
+ * block with f % ktiles == k-tile index) so that every block does the same amount of extra work.
  * ---------------------------------------------------------------------------------------------- */
 template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC>
 __global__ __launch_bounds__(64 * WAVES_K * WAVES_F)
 void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
-		const GatherGeom g, const int ktiles, const int chunks_per_split) {
+		T* __restrict__ bias_partials, const GatherGeom g, const int ktiles, const int chunks_per_split) {
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_K * WAVES_F;
 	constexpr int BK = WAVES_K * WT_K, BF = WAVES_F * WT_F;
@@ -281,16 +297,20 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	constexpr int TL = MF::TL, KS = MF::KS;
 	constexpr int KB = WT_K / TL, FB = WT_F / TL;
 	constexpr int COLS = MC / VEC, RP = THREADS / COLS;
-	constexpr int XSLOTS = BK / RP, GSLOTS = BF / RP;
-	static_assert(THREADS % COLS == 0 && BK % RP == 0 && BF % RP == 0, "loader mapping");
+	constexpr int XSLOTS = (BK + RP - 1) / RP, GSLOTS = (BF + RP - 1) / RP;
+	constexpr int Q = MC / VR;                               /* 16-byte groups per tile row */
+	constexpr int BIAS_IT = (BF * Q + THREADS - 1) / THREADS;
+	static_assert(THREADS % COLS == 0, "loader mapping");
 	static_assert(MC % (VR * KS) == 0, "reduction chunk");
+	static_assert(BK * LDM >= BF * Q, "bias reduction reuses the X tile");
 
-	__shared__ __attribute__((aligned(16))) T Xs[2][BK][LDM];
-	__shared__ __attribute__((aligned(16))) T Gs[2][BF][LDM];
+	__shared__ __attribute__((aligned(16))) T Xs[BK][LDM];
+	__shared__ __attribute__((aligned(16))) T Gs[BF][LDM];
 	__shared__ int4 ktab[BK];      /* per k row: ya term, yb term, channel offset, valid */
 
 	const int tid = threadIdx.x;
-	const int k0 = (blockIdx.x % ktiles) * BK;
+	const int kt = blockIdx.x % ktiles;
+	const int k0 = kt * BK;
 	const int f0 = (blockIdx.x / ktiles) * BF;
 	const int chunk_begin = blockIdx.y * chunks_per_split;
 	const int total_chunks = (g.M + MC - 1) / MC;
@@ -321,11 +341,17 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		const int ya0 = a * g.SA + g.PA, yb0 = b * g.SB + g.PB;
 		#pragma unroll
 		for (int s = 0; s < XSLOTS; ++s) {
-			const int4 ke = ktab[row0 + s * RP];
-			const int ya = ya0 + ke.x, yb = yb0 + ke.y;
-			const bool ok = mvalid && ke.w && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
+			const int row = row0 + s * RP;
+			bool ok = false;
+			int off = 0;
+			if (BK % RP == 0 || row < BK) {
+				const int4 ke = ktab[row];
+				const int ya = ya0 + ke.x, yb = yb0 + ke.y;
+				ok = mvalid && ke.w && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
+				off = n + g.N * (ya + g.LH * yb) + ke.z;
+			}
 			if (ok) {
-				vec_load<T, VEC>(xreg[s], src + (n + g.N * (ya + g.LH * yb) + ke.z));
+				vec_load<T, VEC>(xreg[s], src + off);
 			} else {
 				#pragma unroll
 				for (int v = 0; v < VEC; ++v)
@@ -334,8 +360,9 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		}
 		#pragma unroll
 		for (int s = 0; s < GSLOTS; ++s) {
-			const int f = f0 + row0 + s * RP;
-			if (mvalid && f < g.F) {
+			const int row = row0 + s * RP;
+			const int f = f0 + row;
+			if (mvalid && f < g.F && (BF % RP == 0 || row < BF)) {
 				vec_load<T, VEC>(greg[s], og + ((size_t) m + (size_t) g.M * f));
 			} else {
 				#pragma unroll
@@ -353,13 +380,15 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		a -= c2 ? g.OA : 0;
 		b += eB + c2;
 	};
-	auto store_tiles = [&](int buf) {
+	auto store_tiles = [&]() {
 		#pragma unroll
 		for (int s = 0; s < XSLOTS; ++s)
-			vec_store<T, VEC>(&Xs[buf][row0 + s * RP][col * VEC], xreg[s]);
+			if (BK % RP == 0 || row0 + s * RP < BK)
+				vec_store<T, VEC>(&Xs[row0 + s * RP][col * VEC], xreg[s]);
 		#pragma unroll
 		for (int s = 0; s < GSLOTS; ++s)
-			vec_store<T, VEC>(&Gs[buf][row0 + s * RP][col * VEC], greg[s]);
+			if (BF % RP == 0 || row0 + s * RP < BF)
+				vec_store<T, VEC>(&Gs[row0 + s * RP][col * VEC], greg[s]);
 	};
 
 	const int lane = tid % 64, wave = tid / 64;
@@ -375,36 +404,62 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 			for (int r = 0; r < MF::NACC; ++r)
 				acc[i][j][r] = (T) 0;
 
+	/* bias partial sums: item p = tid + it*THREADS covers 16-byte group p % Q of local row
+	 * (p / Q) * ktiles + kt */
+	T bacc[BIAS_IT];
+	#pragma unroll
+	for (int it = 0; it < BIAS_IT; ++it)
+		bacc[it] = (T) 0;
+
 	__syncthreads();                  /* ktab visible */
-	if (chunk_begin < chunk_end) {
+	if (chunk_begin < chunk_end)
 		load_tiles();
-		store_tiles(0);
-	}
-	__syncthreads();
 	for (int c = chunk_begin; c < chunk_end; ++c) {
-		const int buf = (c - chunk_begin) & 1;
+		__syncthreads();              /* every wave is done reading the previous chunk */
+		store_tiles();
+		__syncthreads();
 		if (c + 1 < chunk_end)
 			load_tiles();
+		/* operand fragments are fetched one group of VR reduction steps ahead of the MFMAs */
+		T ga[2][FB][VR], xb[2][KB][VR];
 		#pragma unroll
-		for (int mm = 0; mm < MC; mm += VR * KS) {
-			T ga[FB][VR], xb[KB][VR];
-			#pragma unroll
-			for (int i = 0; i < FB; ++i)
-				vec_load<T, VR>(ga[i], &Gs[buf][wf * WT_F + i * TL + lc][mm + lk * VR]);
-			#pragma unroll
-			for (int j = 0; j < KB; ++j)
-				vec_load<T, VR>(xb[j], &Xs[buf][wk * WT_K + j * TL + lc][mm + lk * VR]);
+		for (int i = 0; i < FB; ++i)
+			vec_load<T, VR>(ga[0][i], &Gs[wf * WT_F + i * TL + lc][lk * VR]);
+		#pragma unroll
+		for (int j = 0; j < KB; ++j)
+			vec_load<T, VR>(xb[0][j], &Xs[wk * WT_K + j * TL + lc][lk * VR]);
+		#pragma unroll
+		for (int st = 0; st < MC / (VR * KS); ++st) {
+			const int cur = st & 1, nxt = cur ^ 1;
+			if (st + 1 < MC / (VR * KS)) {
+				const int mm = (st + 1) * VR * KS;
+				#pragma unroll
+				for (int i = 0; i < FB; ++i)
+					vec_load<T, VR>(ga[nxt][i], &Gs[wf * WT_F + i * TL + lc][mm + lk * VR]);
+				#pragma unroll
+				for (int j = 0; j < KB; ++j)
+					vec_load<T, VR>(xb[nxt][j], &Xs[wk * WT_K + j * TL + lc][mm + lk * VR]);
+			}
 			#pragma unroll
 			for (int e = 0; e < VR; ++e)
 				#pragma unroll
 				for (int i = 0; i < FB; ++i)
 					#pragma unroll
 					for (int j = 0; j < KB; ++j)
-						acc[i][j] = MF::mma(ga[i][e], xb[j][e], acc[i][j]);
+						acc[i][j] = MF::mma(ga[cur][i][e], xb[cur][j][e], acc[i][j]);
 		}
-		if (c + 1 < chunk_end)
-			store_tiles(buf ^ 1);
-		__syncthreads();
+		#pragma unroll
+		for (int it = 0; it < BIAS_IT; ++it) {
+			const int p = tid + it * THREADS;
+			const int frow = (p / Q) * ktiles + kt;
+			if (frow < BF) {
+				T v[VR];
+				vec_load<T, VR>(v, &Gs[frow][(p % Q) * VR]);
+				#pragma unroll
+				for (int e = 0; e < VR; ++e)
+					bacc[it] += v[e];
+			}
+		}
 	}
 
 	T* dst = partials + (size_t) blockIdx.y * ((size_t) g.K * g.F);
@@ -423,65 +478,44 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 			}
 		}
 	}
-}
 
-/* dst[i] += sum_s partials[s][i], s ascending: the order is fixed, so results are reproducible. */
-template<typename T>
-__global__ void reduce_partials_kernel(const T* __restrict__ partials, T* __restrict__ dst, size_t count, int splits) {
-	const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
-	if (i >= count)
-		return;
-	T s = (T) 0;
-	for (int p = 0; p < splits; ++p)
-		s += partials[(size_t) p * count + i];
-	dst[i] += s;
-}
-
-/* Block-wide sum with wavefront shuffles then LDS; every thread of the block must call it. */
-template<typename T>
-__device__ __forceinline__ T block_sum(T v, T* lds) {
-	#pragma unroll
-	for (int off = 32; off > 0; off >>= 1)
-		v += __shfl_down(v, off, 64);
-	const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-	if (lane == 0)
-		lds[wave] = v;
+	/* finish the bias partials: Q group sums per row, added in ascending group order */
 	__syncthreads();
-	T total = (T) 0;
-	if (threadIdx.x == 0) {
-		const int nw = (blockDim.x + 63) / 64;
-		for (int w = 0; w < nw; ++w)
-			total += lds[w];
+	T* bred = &Xs[0][0];
+	#pragma unroll
+	for (int it = 0; it < BIAS_IT; ++it) {
+		const int p = tid + it * THREADS;
+		const int frow = (p / Q) * ktiles + kt;
+		if (frow < BF)
+			bred[frow * Q + p % Q] = bacc[it];
 	}
 	__syncthreads();
-	return total;        /* valid in thread 0 */
+	if (tid < BF && tid % ktiles == kt && f0 + tid < g.F) {
+		T s = (T) 0;
+		#pragma unroll
+		for (int q = 0; q < Q; ++q)
+			s += bred[tid * Q + q];
+		bias_partials[(size_t) blockIdx.y * g.F + f0 + tid] = s;
+	}
 }
 
-/* Column sums of G[M x F]: grid (splits, F); block (s, f) sums rows [s*span, (s+1)*span). */
+/* dst[i] += sum_s partials[s][i]. A block covers 64 outputs with four groups of threads; group j adds
+ * the partials s = j, j+4, j+8, ... in ascending order and the four group sums are then added in
+ * ascending order, so the summation order is fixed and results are reproducible. */
 template<typename T>
 __global__ __launch_bounds__(256)
-void colsum_partial_kernel(const T* __restrict__ G, T* __restrict__ ws, size_t M, size_t span) {
-	__shared__ T lds[4];
-	const size_t begin = (size_t) blockIdx.x * span;
-	const size_t end = begin + span < M ? begin + span : M;
-	const T* col = G + M * blockIdx.y;
+void reduce_partials_kernel(const T* __restrict__ partials, T* __restrict__ dst, size_t count, int splits) {
+	__shared__ T lds[4][64];
+	const int ox = threadIdx.x % 64, grp = threadIdx.x / 64;
+	const size_t i = (size_t) blockIdx.x * 64 + ox;
 	T s = (T) 0;
-	for (size_t i = begin + threadIdx.x; i < end; i += 256)
-		s += col[i];
-	const T total = block_sum(s, lds);
-	if (threadIdx.x == 0)
-		ws[(size_t) blockIdx.y * gridDim.x + blockIdx.x] = total;
-}
-
-template<typename T>
-__global__ void colsum_final_kernel(const T* __restrict__ ws, T* __restrict__ dst, int F, int splits) {
-	const int f = blockIdx.x * blockDim.x + threadIdx.x;
-	if (f >= F)
-		return;
-	T s = (T) 0;
-	for (int p = 0; p < splits; ++p)
-		s += ws[(size_t) f * splits + p];
-	dst[f] += s;
+	if (i < count)
+		for (int p = grp; p < splits; p += 4)
+			s += partials[(size_t) p * count + i];
+	lds[grp][ox] = s;
+	__syncthreads();
+	if (grp == 0 && i < count)
+		dst[i] += ((lds[0][ox] + lds[1][ox]) + lds[2][ox]) + lds[3][ox];
 }
 
 /* Forward weights: wt[k][f] = w[k + K*f], zero-padded to Kp rows x ldw columns. */
@@ -512,46 +546,106 @@ int round_up(int v, int to) {
 
 constexpr int WT_ROW_PAD = 16;     /* >= every KC */
 constexpr int WT_COL_PAD = 128;    /* >= every BF */
+constexpr int NUM_CUS = 256;
+constexpr int LDS_PER_CU = 160 * 1024;
+constexpr int MAX_WAVES_PER_CU = 16;   /* four per SIMD: every kernel here stays within 128 registers per lane */
 
 template<typename T> struct GemmCfg;
-template<> struct GemmCfg<float> { static constexpr int KC = 16, VEC = 4; };
-template<> struct GemmCfg<double> { static constexpr int KC = 8, VEC = 2; };
+template<> struct GemmCfg<float> { static constexpr int KC = 16, VEC = 4, PAD = 32; };
+template<> struct GemmCfg<double> { static constexpr int KC = 8, VEC = 2, PAD = 16; };
+
+/* One instantiation of gather_gemm_kernel and what the tile chooser needs to know about it. */
+template<typename T>
+struct GatherVariant {
+	int bm, bf, waves, lds_bytes;
+	void (*launch)(dim3 grid, size_t dyn_lds, const T*, const T*, const T*, T*, const GatherGeom&, int mtiles, bool vec, bool divs);
+};
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F>
-void launch_gather_variant(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, bool vec, bool divs) {
+void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g,
+		int mtiles, bool vec, bool divs) {
 	constexpr int KC = GemmCfg<T>::KC, VEC = GemmCfg<T>::VEC;
-	constexpr int BM = WAVES_M * WT_M, BF = WAVES_F * WT_F;
-	const int mtiles = (g.M + BM - 1) / BM;
-	dim3 grid((unsigned) round_up(mtiles, 8), (unsigned) ((g.F + BF - 1) / BF));
 	dim3 block(64 * WAVES_M * WAVES_F);
 	if (vec && !divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, 0, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
 	else if (vec && divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, 0, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
 	else if (!divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, 0, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
 	else
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, 0, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F>
+GatherVariant<T> gather_variant() {
+	typedef GemmCfg<T> C;
+	GatherVariant<T> v;
+	v.bm = WAVES_M * WT_M;
+	v.bf = WAVES_F * WT_F;
+	v.waves = WAVES_M * WAVES_F;
+	v.lds_bytes = 2 * C::KC * (v.bm + C::PAD + v.bf + C::PAD) * (int) sizeof(T);
+	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F>;
+	return v;
+}
+
+template<typename T> struct GatherVariants;
+template<> struct GatherVariants<float> {
+	static constexpr int COUNT = 3;
+	static const GatherVariant<float>* get() {
+		static const GatherVariant<float> v[COUNT] = {
+			gather_variant<float, 4, 2, 64, 64>(),      /* 256 x 128 */
+			gather_variant<float, 4, 1, 64, 64>(),      /* 256 x 64 */
+			gather_variant<float, 4, 1, 64, 32>(),      /* 256 x 32 */
+		};
+		return v;
+	}
+};
+template<> struct GatherVariants<double> {
+	static constexpr int COUNT = 2;
+	static const GatherVariant<double>* get() {
+		static const GatherVariant<double> v[COUNT] = {
+			gather_variant<double, 4, 2, 64, 32>(),     /* 256 x 64 */
+			gather_variant<double, 4, 1, 64, 32>(),     /* 256 x 32 */
+		};
+		return v;
+	}
+};
+
+/* Picks the tile shape: the narrowest F tile that covers all output columns in one block column (so
+ * the gathered A operand, the expensive one, is read once), else the widest. Blocks run at the
+ * occupancy their LDS and register use allows; measured on MI355X, more co-resident blocks beat
+ * fewer blocks even when the last round of blocks is mostly idle. */
 template<typename T>
 void launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g) {
 	const bool vec = g.N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
 	const bool divs = g.DA != 1 || g.DB != 1;
-	if (std::is_same<T, float>::value) {
-		if (g.F > 64)
-			launch_gather_variant<T, 4, 2, 64, 64>(src, wt, bias, out, g, vec, divs);
-		else if (g.F > 32)
-			launch_gather_variant<T, 4, 1, 64, 64>(src, wt, bias, out, g, vec, divs);
-		else
-			launch_gather_variant<T, 4, 1, 64, 32>(src, wt, bias, out, g, vec, divs);
-	} else {
-		if (g.F > 32)
-			launch_gather_variant<T, 4, 2, 64, 32>(src, wt, bias, out, g, vec, divs);
-		else
-			launch_gather_variant<T, 4, 1, 64, 32>(src, wt, bias, out, g, vec, divs);
+	const GatherVariant<T>* vars = GatherVariants<T>::get();
+	int best_v = 0;                     /* the table is ordered from the widest F tile to the narrowest */
+	for (int i = 1; i < GatherVariants<T>::COUNT; ++i)
+		if (vars[i].bf >= g.F)
+			best_v = i;
+	/* tuning overrides for experiments, keyed by the number of output columns F of the GEMM:
+	 * CATTLE_HIP_GATHER_VARIANT_F<F> = index into the variant table, CATTLE_HIP_GATHER_OCC_F<F> = blocks per CU
+	 * (enforced by reserving dynamic LDS) */
+	int occ = 0;
+	const std::string suffix = "_F" + std::to_string(g.F);
+	if (const char* e = std::getenv(("CATTLE_HIP_GATHER_VARIANT" + suffix).c_str())) {
+		const int i = std::atoi(e);
+		if (i >= 0 && i < GatherVariants<T>::COUNT)
+			best_v = i;
 	}
+	if (const char* e = std::getenv(("CATTLE_HIP_GATHER_OCC" + suffix).c_str()))
+		occ = std::atoi(e);
+	const GatherVariant<T>& v = vars[best_v];
+	size_t dyn = 0;
+	if (occ >= 1 && occ <= 8) {
+		const int want_bytes = LDS_PER_CU / (occ + 1) + 256;
+		dyn = want_bytes > v.lds_bytes ? (size_t) (want_bytes - v.lds_bytes) : 0;
+	}
+	const int mtiles = (g.M + v.bm - 1) / v.bm;
+	dim3 grid((unsigned) round_up(mtiles, 8), (unsigned) ((g.F + v.bf - 1) / v.bf));
+	v.launch(grid, dyn, src, wt, bias, out, g, mtiles, vec, divs);
 }
 
 GatherGeom forward_geom(const ConvShape& s, int N) {
@@ -583,36 +677,106 @@ void check_sizes(const ConvShape& s, int N) {
 	CATTLE_HIP_REQUIRE(in_elems <= lim && out_elems <= lim, "tensor exceeds 2^31-1 elements");
 }
 
-/* Split plan of the weight-gradient reduction over M. */
-template<typename T> struct WgradCfg;
-template<> struct WgradCfg<float> { static constexpr int WK = 2, WF = 2, TK = 64, TF = 64, MC = 32, VEC = 4; };
-template<> struct WgradCfg<double> { static constexpr int WK = 2, WF = 2, TK = 32, TF = 32, MC = 32, VEC = 2; };
-
-struct WgradPlan {
-	int ktiles, ftiles, splits, chunks_per_split;
-};
+/* Weight-gradient tile shapes (K rows x F columns of the gradient per block) and the split of M. */
+constexpr int WGRAD_MC = 32;
 
 template<typename T>
+struct WgradVariant {
+	int bk, bf, waves, lds_bytes;
+	void (*launch)(dim3 grid, const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom&, int ktiles,
+			int chunks_per_split, bool vec);
+};
+
+template<typename T, int WK, int WF, int TK, int TF>
+void launch_wgrad_variant(dim3 grid, const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom& g, int ktiles,
+		int chunks_per_split, bool vec) {
+	constexpr int VEC = GemmCfg<T>::VEC;
+	dim3 block(64 * WK * WF);
+	if (vec)
+		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, VEC><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, ktiles,
+				chunks_per_split);
+	else
+		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, ktiles,
+				chunks_per_split);
+	CATTLE_HIP_CHECK(hipGetLastError());
+}
+
+template<typename T, int WK, int WF, int TK, int TF>
+WgradVariant<T> wgrad_variant() {
+	WgradVariant<T> v;
+	v.bk = WK * TK;
+	v.bf = WF * TF;
+	v.waves = WK * WF;
+	v.lds_bytes = (v.bk + v.bf) * (WGRAD_MC + 16 / (int) sizeof(T)) * (int) sizeof(T) + v.bk * 16;
+	v.launch = &launch_wgrad_variant<T, WK, WF, TK, TF>;
+	return v;
+}
+
+template<typename T> struct WgradVariants;
+template<> struct WgradVariants<float> {
+	static constexpr int COUNT = 4;
+	static const WgradVariant<float>* get() {
+		static const WgradVariant<float> v[COUNT] = {
+			wgrad_variant<float, 2, 4, 96, 32>(),       /* 192 x 128 */
+			wgrad_variant<float, 2, 2, 64, 64>(),       /* 128 x 128 */
+			wgrad_variant<float, 1, 4, 32, 32>(),       /*  32 x 128 */
+			wgrad_variant<float, 1, 4, 64, 32>(),       /*  64 x 128 */
+		};
+		return v;
+	}
+};
+template<> struct WgradVariants<double> {
+	static constexpr int COUNT = 3;
+	static const WgradVariant<double>* get() {
+		static const WgradVariant<double> v[COUNT] = {
+			wgrad_variant<double, 2, 4, 48, 16>(),      /* 96 x 64 */
+			wgrad_variant<double, 2, 2, 32, 32>(),      /* 64 x 64 */
+			wgrad_variant<double, 1, 4, 32, 16>(),      /* 32 x 64 */
+		};
+		return v;
+	}
+};
+
+struct WgradPlan {
+	int variant, ktiles, ftiles, splits, chunks_per_split;
+};
+
+/* The tile shape with the least padding wins (larger tile on ties: it re-reads G less often); the
+ * M range is then cut into as many slices as fill the chip once (blocks = tiles * splits <= slots),
+ * so that no block runs in a second, mostly idle round. The plan depends on the shape only, which
+ * keeps the summation order, and with it the result, reproducible. */
+template<typename T>
 WgradPlan wgrad_plan(int M, int K, int F) {
-	typedef WgradCfg<T> C;
+	const WgradVariant<T>* vars = WgradVariants<T>::get();
 	WgradPlan p;
-	p.ktiles = (K + C::WK * C::TK - 1) / (C::WK * C::TK);
-	p.ftiles = (F + C::WF * C::TF - 1) / (C::WF * C::TF);
-	const int chunks = (M + C::MC - 1) / C::MC;
+	p.variant = 0;
+	long best = -1;
+	for (int i = 0; i < WgradVariants<T>::COUNT; ++i) {
+		const long padded = (long) round_up(K, vars[i].bk) * round_up(F, vars[i].bf);
+		if (best < 0 || padded < best) {
+			best = padded;
+			p.variant = i;
+		}
+	}
+	if (const char* e = std::getenv("CATTLE_HIP_WGRAD_VARIANT")) {
+		const int i = std::atoi(e);
+		if (i >= 0 && i < WgradVariants<T>::COUNT)
+			p.variant = i;
+	}
+	const WgradVariant<T>& v = vars[p.variant];
+	p.ktiles = (K + v.bk - 1) / v.bk;
+	p.ftiles = (F + v.bf - 1) / v.bf;
+	const int occ = std::max(1, std::min(std::min(LDS_PER_CU / v.lds_bytes, MAX_WAVES_PER_CU / v.waves), 3));
+	const int slots = NUM_CUS * occ;
 	const int tiles = p.ktiles * p.ftiles;
-	int want = std::max(1, (1024 + tiles - 1) / tiles);      /* about four blocks per CU */
-	want = std::min(want, std::max(1, chunks / 8));           /* at least 8 chunks per block */
+	const int chunks = (M + WGRAD_MC - 1) / WGRAD_MC;
+	int want = std::max(1, slots / tiles);
+	if (const char* e = std::getenv("CATTLE_HIP_WGRAD_SPLITS"))
+		want = std::max(1, std::atoi(e));
+	want = std::min(want, std::max(1, chunks / 4));           /* at least four chunks per block */
 	p.chunks_per_split = (chunks + want - 1) / want;
 	p.splits = (chunks + p.chunks_per_split - 1) / p.chunks_per_split;
 	return p;
-}
-
-constexpr int COLSUM_MAX_SPLITS = 64;
-
-int colsum_splits(size_t M, int F) {
-	const size_t by_rows = std::max<size_t>(1, M / 4096);
-	const size_t by_fill = std::max<size_t>(1, (size_t) 1024 / (size_t) std::max(1, F));
-	return (int) std::min<size_t>(COLSUM_MAX_SPLITS, std::min(by_rows, by_fill));
 }
 
 } /* namespace */
@@ -625,7 +789,7 @@ ConvWorkspace conv_workspace(const ConvShape& s, int N) {
 	ws.wt_dgrad = (size_t) round_up(s.RH * s.RW * s.F, WT_ROW_PAD) * round_up(s.C, WT_COL_PAD);
 	const int M = N * s.OH() * s.OW();
 	const WgradPlan p = wgrad_plan<T>(M, s.K(), s.F);
-	ws.partials = (size_t) p.splits * s.K() * s.F + (size_t) COLSUM_MAX_SPLITS * s.F;
+	ws.partials = (size_t) p.splits * ((size_t) s.K() * s.F + (size_t) s.F);
 	return ws;
 }
 
@@ -646,32 +810,20 @@ template<typename T>
 void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad,
 		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials) {
 	check_sizes(s, N);
-	typedef WgradCfg<T> C;
 	const GatherGeom g = forward_geom(s, N);
-	/* weight gradient: split-M partials, then a fixed-order reduction that accumulates into wgrad */
+	/* weight and bias gradients: split-M partials, then a fixed-order reduction that accumulates */
 	{
 		const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F);
-		dim3 grid((unsigned) (p.ktiles * p.ftiles), (unsigned) p.splits);
-		dim3 block(64 * C::WK * C::WF);
-		const bool vec = N % C::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-				(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
-		if (vec)
-			wgrad_kernel<T, C::WK, C::WF, C::TK, C::TF, C::MC, C::VEC><<<grid, block, 0, stream()>>>(x, out_grad, partials, g,
-					p.ktiles, p.chunks_per_split);
-		else
-			wgrad_kernel<T, C::WK, C::WF, C::TK, C::TF, C::MC, 1><<<grid, block, 0, stream()>>>(x, out_grad, partials, g,
-					p.ktiles, p.chunks_per_split);
-		CATTLE_HIP_CHECK(hipGetLastError());
+		const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
 		const size_t count = (size_t) g.K * g.F;
-		reduce_partials_kernel<T><<<(unsigned) ((count + 255) / 256), 256, 0, stream()>>>(partials, wgrad, count, p.splits);
+		T* bias_partials = partials + (size_t) p.splits * count;
+		dim3 grid((unsigned) (p.ktiles * p.ftiles), (unsigned) p.splits);
+		const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+				(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
+		v.launch(grid, x, out_grad, partials, bias_partials, g, p.ktiles, p.chunks_per_split, vec);
+		reduce_partials_kernel<T><<<(unsigned) ((count + 63) / 64), 256, 0, stream()>>>(partials, wgrad, count, p.splits);
 		CATTLE_HIP_CHECK(hipGetLastError());
-		/* bias gradient */
-		T* bws = partials + (size_t) p.splits * count;
-		const int cs = colsum_splits((size_t) g.M, g.F);
-		const size_t span = ((size_t) g.M + cs - 1) / cs;
-		colsum_partial_kernel<T><<<dim3((unsigned) cs, (unsigned) g.F), 256, 0, stream()>>>(out_grad, bws, (size_t) g.M, span);
-		CATTLE_HIP_CHECK(hipGetLastError());
-		colsum_final_kernel<T><<<(unsigned) ((g.F + 255) / 256), 256, 0, stream()>>>(bws, bgrad, g.F, cs);
+		reduce_partials_kernel<T><<<(unsigned) ((g.F + 63) / 64), 256, 0, stream()>>>(bias_partials, bgrad, (size_t) g.F, p.splits);
 		CATTLE_HIP_CHECK(hipGetLastError());
 	}
 	if (!in_grad)
