@@ -13,7 +13,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libcattle_hip.so")
+# CATTLE_HIP_LIBRARY overrides the location of the built library (e.g. an experimental build)
+LIB_PATH = os.environ.get("CATTLE_HIP_LIBRARY") or os.path.join(_HERE, "libcattle_hip.so")
 
 F32, F64 = 0, 1
 HOST, DEVICE = 0, 1

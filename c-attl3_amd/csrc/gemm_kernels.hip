@@ -96,10 +96,22 @@ __device__ __forceinline__ int xcd_tile(int bid, int ntiles) {
 	return (bid % XCDS) * per + bid / XCDS;
 }
 
+/* Where gathered loads that fall into the zero padding are pointed at. */
+__device__ __attribute__((aligned(16))) const unsigned g_zero_block[4] = { 0u, 0u, 0u, 0u };
+
 /* ------------------------------------------------------------------------------------------------
  * out[M x F] = gather(src)[M x K] * wt[K x F] (+ bias).
  * Block tile BM x BF, wave tile WT_M x WT_F, reduction chunks of KC staged through double-buffered
  * LDS: As[k][m] (m fastest, exactly as it lies in memory) and Bs[k][f].
+ *
+ * Keeping the MFMA pipe fed means keeping other vector instructions out of the loop, so:
+ *  - the per-k part of the gather (element offset, row/column displacement) comes from a small
+ *    table in LDS that one wave keeps three chunks ahead; a thread only adds its own base;
+ *  - loads that fall into the zero padding are redirected to a 16-byte block of zeros in device
+ *    memory (a pointer select), so the load itself is unconditional: no branch, no zero fill;
+ *  - a lane's MB column blocks are interleaved (column = MB*lane + j) so that its operand values
+ *    are adjacent in LDS and in the output: one LDS read per operand and reduction step with an
+ *    immediate offset, and one vector store per output row.
  * VEC = elements per global load along m (needs N % VEC == 0 and a 16-byte aligned src).
  * DIVS = the gather has divisors (strided input gradient).
  * ---------------------------------------------------------------------------------------------- */
@@ -117,11 +129,14 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	constexpr int ACOLS = BM / VEC, ARP = THREADS / ACOLS, ASLOTS = KC / ARP;
 	constexpr int VB = 16 / (int) sizeof(T);
 	constexpr int BCOLS = BF / VB, BVECS = KC * BCOLS, BITER = (BVECS + THREADS - 1) / THREADS;
+	constexpr int INVALID = -(1 << 30);
 	static_assert(THREADS % ACOLS == 0 && KC % ARP == 0 && ASLOTS >= 1, "A loader mapping");
 	static_assert(KC % KS == 0 && WT_M % TL == 0 && WT_F % TL == 0, "tile shape");
+	static_assert(THREADS >= KC, "table writers");
 
-	__shared__ T As[2][KC][LDA];
-	__shared__ T Bs[2][KC][LDB];
+	__shared__ __attribute__((aligned(32))) T As[2][KC][LDA];
+	__shared__ __attribute__((aligned(32))) T Bs[2][KC][LDB];
+	__shared__ int4 ktab[3][KC];     /* per reduction index: element offset, ya term, yb term, channel offset */
 
 	const int tile = xcd_tile(blockIdx.x, mtiles);
 	if (tile >= mtiles)
@@ -129,8 +144,34 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	const int tid = threadIdx.x;
 	const int m0 = tile * BM;
 	const int f0 = blockIdx.y * BF;
+	const int nchunks = (g.K + KC - 1) / KC;
 
-	/* --- per-thread gather state: a fixed group of VEC rows m, and a walking k row --- */
+	/* --- table writer state: thread t < KC walks k = t, t + KC, t + 2 KC, ... --- */
+	int tr = tid % g.R, ts, tch;
+	{
+		const int t = tid / g.R;
+		ts = t % g.S;
+		tch = t / g.S;
+	}
+	const int eR = KC % g.R, eS = (KC / g.R) % g.S, eCh = (KC / g.R) / g.S;
+	const int plane = g.N * g.LH * g.LW;
+	auto write_table = [&](int slot) {
+		if (tid < KC) {
+			const bool kv = tch < g.LC;
+			const int dya = tr * g.RA, dyb = ts * g.RB;
+			const int choff = kv ? plane * tch : 0;
+			ktab[slot][tid] = make_int4(kv ? g.N * (dya + g.LH * dyb) + choff : 0, kv ? dya : INVALID, dyb, choff);
+			tr += eR;
+			const int c1 = tr >= g.R;
+			tr -= c1 ? g.R : 0;
+			ts += eS + c1;
+			const int c2 = ts >= g.S;
+			ts -= c2 ? g.S : 0;
+			tch += eCh + c2;
+		}
+	};
+
+	/* --- per-thread gather state: a fixed group of VEC rows m --- */
 	const int acol = tid % ACOLS, arow0 = tid / ACOLS;
 	const int m = m0 + acol * VEC;
 	const bool mvalid = m < g.M;
@@ -142,51 +183,43 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		ya0 = a * g.SA + g.PA;
 		yb0 = b * g.SB + g.PB;
 	}
-	int kr = arow0 % g.R, ks, kch;
-	{
-		const int t = arow0 / g.R;
-		ks = t % g.S;
-		kch = t / g.S;
+	const int base_m = n + g.N * (ya0 + g.LH * yb0);      /* may be negative; only used when in range */
+	const T* const zeros = reinterpret_cast<const T*>(g_zero_block);
+	const T* bptr[BITER];
+	#pragma unroll
+	for (int it = 0; it < BITER; ++it) {
+		const int idx = tid + it * THREADS;
+		bptr[it] = wt + ((size_t) (idx / BCOLS) * g.ldw + f0 + (idx % BCOLS) * VB);
 	}
-	const int eR = ARP % g.R, eS = (ARP / g.R) % g.S, eCh = (ARP / g.R) / g.S;
+	const size_t bstep = (size_t) KC * g.ldw;
 
 	T areg[ASLOTS][VEC];
 	T breg[BITER][VB];
 
-	auto load_tiles = [&](int k0) {
+	auto load_tiles = [&](int slot) {
 		#pragma unroll
 		for (int s = 0; s < ASLOTS; ++s) {
-			int ya = ya0 + kr * g.RA, yb = yb0 + ks * g.RB;
-			bool ok = mvalid && kch < g.LC;
+			const int4 e = ktab[slot][arow0 + s * ARP];
+			int ya = ya0 + e.y, yb = yb0 + e.z;
+			int ok = mvalid;                 /* bitwise, not short-circuit: keep this branch-free */
+			int off;
 			if (DIVS) {
 				const int qa = ya / g.DA, qb = yb / g.DB;
-				ok = ok && qa * g.DA == ya && qb * g.DB == yb;
+				ok &= (qa * g.DA == ya) & (qb * g.DB == yb);
 				ya = qa;
 				yb = qb;
-			}
-			ok = ok && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
-			if (ok) {
-				vec_load<T, VEC>(areg[s], src + (n + g.N * (ya + g.LH * (yb + g.LW * kch))));
+				off = n + g.N * (ya + g.LH * yb) + e.w;
 			} else {
-				#pragma unroll
-				for (int v = 0; v < VEC; ++v)
-					areg[s][v] = (T) 0;
+				off = base_m + e.x;
 			}
-			/* advance the k row by ARP with carries */
-			kr += eR;
-			const int c1 = kr >= g.R;
-			kr -= c1 ? g.R : 0;
-			ks += eS + c1;
-			const int c2 = ks >= g.S;
-			ks -= c2 ? g.S : 0;
-			kch += eCh + c2;
+			ok &= ((unsigned) ya < (unsigned) g.LH) & ((unsigned) yb < (unsigned) g.LW);
+			vec_load<T, VEC>(areg[s], ok ? src + off : zeros);
 		}
 		#pragma unroll
 		for (int it = 0; it < BITER; ++it) {
-			const int idx = tid + it * THREADS;
-			if (BVECS % THREADS == 0 || idx < BVECS) {
-				const int brow = idx / BCOLS, bcol = idx % BCOLS;
-				vec_load<T, VB>(breg[it], wt + ((size_t) (k0 + brow) * g.ldw + f0 + bcol * VB));
+			if (BVECS % THREADS == 0 || tid + it * THREADS < BVECS) {
+				vec_load<T, VB>(breg[it], bptr[it]);
+				bptr[it] += bstep;
 			}
 		}
 	};
@@ -217,57 +250,75 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			for (int r = 0; r < MF::NACC; ++r)
 				acc[i][j][r] = (T) 0;
 
-	const int nchunks = (g.K + KC - 1) / KC;
+	write_table(0);
+	write_table(1);
+	__syncthreads();
 	load_tiles(0);
 	store_tiles(0);
 	__syncthreads();
+	int slot_next = 1, slot_write = 2;       /* table slots of chunk c + 1 and c + 2 */
 	for (int c = 0; c < nchunks; ++c) {
 		const int buf = c & 1;
+		write_table(slot_write);
 		if (c + 1 < nchunks)
-			load_tiles((c + 1) * KC);
+			load_tiles(slot_next);
+		slot_next = slot_next == 2 ? 0 : slot_next + 1;
+		slot_write = slot_write == 2 ? 0 : slot_write + 1;
 		/* operand fragments are fetched one reduction step ahead of the MFMAs that use them */
 		T xa[2][MB], wb[2][FB];
-		#pragma unroll
-		for (int j = 0; j < MB; ++j)
-			xa[0][j] = As[buf][lk][wm * WT_M + j * TL + lc];
-		#pragma unroll
-		for (int i = 0; i < FB; ++i)
-			wb[0][i] = Bs[buf][lk][wf * WT_F + i * TL + lc];
+		vec_load<T, MB>(xa[0], &As[buf][lk][wm * WT_M + MB * lc]);
+		vec_load<T, FB>(wb[0], &Bs[buf][lk][wf * WT_F + FB * lc]);
 		#pragma unroll
 		for (int st = 0; st < KC / KS; ++st) {
 			const int cur = st & 1, nxt = cur ^ 1;
 			if (st + 1 < KC / KS) {
-				#pragma unroll
-				for (int j = 0; j < MB; ++j)
-					xa[nxt][j] = As[buf][(st + 1) * KS + lk][wm * WT_M + j * TL + lc];
-				#pragma unroll
-				for (int i = 0; i < FB; ++i)
-					wb[nxt][i] = Bs[buf][(st + 1) * KS + lk][wf * WT_F + i * TL + lc];
+				vec_load<T, MB>(xa[nxt], &As[buf][(st + 1) * KS + lk][wm * WT_M + MB * lc]);
+				vec_load<T, FB>(wb[nxt], &Bs[buf][(st + 1) * KS + lk][wf * WT_F + FB * lc]);
 			}
+			/* issue order matters (a wave issues in order and stalls on a busy MFMA pipe): the LDS reads
+			 * of the next step must go out before this step's MFMAs, so pin the schedule here */
+			__builtin_amdgcn_sched_barrier(0);
 			#pragma unroll
 			for (int i = 0; i < FB; ++i)
 				#pragma unroll
 				for (int j = 0; j < MB; ++j)
 					acc[i][j] = MF::mma(wb[cur][i], xa[cur][j], acc[i][j]);
+			__builtin_amdgcn_sched_barrier(0);
 		}
 		if (c + 1 < nchunks)
 			store_tiles(buf ^ 1);
 		__syncthreads();
 	}
 
-	/* epilogue: D rows are filters, D columns are m (contiguous in memory) */
+	/* epilogue: D rows are filters (row rr of block i is filter FB*rr + i), D columns are m
+	 * (column lc of block j is row MB*lc + j of the tile), so a lane owns MB adjacent outputs */
+	constexpr int VS = MB * (int) sizeof(T) > 16 ? 16 / (int) sizeof(T) : MB;
+	const bool vec_out = g.M % MB == 0 && (reinterpret_cast<uintptr_t>(out) & (VS * sizeof(T) - 1)) == 0;
+	const int mm = m0 + wm * WT_M + MB * lc;
 	#pragma unroll
 	for (int i = 0; i < FB; ++i) {
 		#pragma unroll
 		for (int r = 0; r < MF::NACC; ++r) {
-			const int f = f0 + wf * WT_F + i * TL + acc_row<T>(r, lk);
+			const int f = f0 + wf * WT_F + FB * acc_row<T>(r, lk) + i;
 			if (f < g.F) {
 				const T bv = bias ? bias[f] : (T) 0;
-				#pragma unroll
-				for (int j = 0; j < MB; ++j) {
-					const int mm = m0 + wm * WT_M + j * TL + lc;
-					if (mm < g.M)
-						out[(size_t) mm + (size_t) g.M * f] = acc[i][j][r] + bv;
+				T* dst = out + ((size_t) mm + (size_t) g.M * f);
+				if (vec_out) {
+					if (mm < g.M) {
+						#pragma unroll
+						for (int j0 = 0; j0 < MB; j0 += VS) {
+							T v[VS];
+							#pragma unroll
+							for (int j = 0; j < VS; ++j)
+								v[j] = acc[i][j0 + j][r] + bv;
+							vec_store<T, VS>(dst + j0, v);
+						}
+					}
+				} else {
+					#pragma unroll
+					for (int j = 0; j < MB; ++j)
+						if (mm + j < g.M)
+							dst[j] = acc[i][j][r] + bv;
 				}
 			}
 		}
@@ -440,6 +491,7 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 				for (int j = 0; j < KB; ++j)
 					vec_load<T, VR>(xb[nxt][j], &Xs[wk * WT_K + j * TL + lc][mm + lk * VR]);
 			}
+			__builtin_amdgcn_sched_barrier(0);       /* next group's LDS reads go out before these MFMAs */
 			#pragma unroll
 			for (int e = 0; e < VR; ++e)
 				#pragma unroll
@@ -447,6 +499,7 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 					#pragma unroll
 					for (int j = 0; j < KB; ++j)
 						acc[i][j] = MF::mma(ga[cur][i][e], xb[cur][j][e], acc[i][j]);
+			__builtin_amdgcn_sched_barrier(0);
 		}
 		#pragma unroll
 		for (int it = 0; it < BIAS_IT; ++it) {
@@ -584,7 +637,7 @@ GatherVariant<T> gather_variant() {
 	v.bm = WAVES_M * WT_M;
 	v.bf = WAVES_F * WT_F;
 	v.waves = WAVES_M * WAVES_F;
-	v.lds_bytes = 2 * C::KC * (v.bm + C::PAD + v.bf + C::PAD) * (int) sizeof(T);
+	v.lds_bytes = 2 * C::KC * (v.bm + C::PAD + v.bf + C::PAD) * (int) sizeof(T) + 3 * C::KC * 16;
 	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F>;
 	return v;
 }
@@ -675,6 +728,10 @@ void check_sizes(const ConvShape& s, int N) {
 	const double lim = 2147483647.0;
 	const double in_elems = (double) N * s.H * s.W * s.C, out_elems = (double) N * s.OH() * s.OW() * s.F;
 	CATTLE_HIP_REQUIRE(in_elems <= lim && out_elems <= lim, "tensor exceeds 2^31-1 elements");
+	/* gather offsets are formed in 32-bit arithmetic relative to positions inside the padding */
+	const double padded = (double) N * (s.H + 2.0 * s.pv + s.RH * (s.dv + 1.0)) * (s.W + 2.0 * s.ph + s.RW * (s.dh + 1.0)) *
+			std::max(s.C, s.F);
+	CATTLE_HIP_REQUIRE(padded <= lim, "padded tensor exceeds 2^31-1 elements");
 }
 
 /* Weight-gradient tile shapes (K rows x F columns of the gradient per block) and the split of M. */
