@@ -93,6 +93,54 @@ def gpu_run(args, dtype):
     return dict(wall_ms=wall_ms, M=M, K=K, F=F, gemm_flop=gemm_flop, kernels=kernels)
 
 
+def pointwise_run(args, dtype):
+    """HBM-bound layers at the cfg4 activation shape (N x 56 x 56 x 64): achieved GB/s against the
+    algorithmic bytes per element of each pass (read x, write y, ...)."""
+    ch = importlib.import_module("c-attl3_amd")
+    ch.init(0)
+    N, H, W, C = args.batch, SHAPE["H"], SHAPE["W"], SHAPE["C"]
+    es = np.dtype(dtype).itemsize
+    gen = np.random.default_rng(7)
+    x = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H, W, C)).astype(dtype)))
+    y = ch.DeviceTensor((N, H, W, C), dtype)
+    g = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H, W, C)).astype(dtype)))
+    dx = ch.DeviceTensor((N, H, W, C), dtype)
+    yp = ch.DeviceTensor((N, H // 2, W // 2, C), dtype)
+    gp = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H // 2, W // 2, C)).astype(dtype)))
+    elems = N * H * W * C
+    timer = ch.Timer()
+    reps = max(3, args.steps)
+
+    def timed(fn):
+        fn()
+        timer.start()
+        for _ in range(reps):
+            fn()
+        return timer.stop() / reps
+
+    rows = []
+
+    def add(name, ms, bytes_per_elem):
+        gbs = elems * bytes_per_elem / (ms * 1e-3) / 1e9
+        rows.append({"kernel": name, "ms": round(ms, 4), "bytes_per_elem": bytes_per_elem, "GB/s": round(gbs, 1),
+                     "frac_of_8TB/s": round(gbs / 8000.0, 4)})
+
+    for kind in ("identity", "relu", "sigmoid", "tanh"):
+        layer = ch.ActivationLayer(dtype, kind, (H, W, C))
+        add(kind + " forward", timed(lambda: layer.forward_into(x, y, True)), 2 * es)
+        add(kind + " backward", timed(lambda: layer.backward_into(g, dx)), (2 if kind == "identity" else 3) * es)
+    mx = ch.MaxPoolLayer(dtype, (H, W, C))
+    add("maxpool 2x2 forward", timed(lambda: mx.forward_into(x, yp, True)), es + (es + 4) / 4.0)
+    add("maxpool 2x2 backward", timed(lambda: mx.backward_into(gp, dx)), es + (es + 4) / 4.0)
+    mn = ch.MeanPoolLayer(dtype, (H, W, C))
+    add("meanpool 2x2 forward", timed(lambda: mn.forward_into(x, yp, True)), es + es / 4.0)
+    add("meanpool 2x2 backward", timed(lambda: mn.backward_into(gp, dx)), es + es / 4.0)
+    bn = ch.BatchNormLayer(dtype, (H, W, C))
+    add("batchnorm forward (training)", timed(lambda: bn.forward_into(x, y, True)), 5 * es)
+    add("batchnorm backward", timed(lambda: bn.backward_into(g, dx)), 5 * es)
+    return rows
+
+
 def cpu_baseline(args, dtype):
     """Times the oracle (the restatement of the reference algorithm: explicit patch matrix + GEMMs +
     col2im, OpenMP GEMMs) on a bounded sample: the same layer at a smaller batch."""
@@ -131,10 +179,19 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel of x's size (for scaling rocprof byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", choices=["conv", "pointwise"], default="conv",
+                    help="conv: the headline benchmark; pointwise: HBM-bound layers, one line of per-kernel GB/s")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
     dtype = np.float32 if args.dtype == "f32" else np.float64
+    if args.workload == "pointwise":
+        rows = pointwise_run(args, dtype)
+        print(json.dumps({"metric": "pointwise_layer_hbm_bandwidth", "unit": "GB/s", "n_gpus": 1, "dtype": args.dtype,
+                          "data": "synthetic", "config": {"workload": "activation / pool / batch-norm layers on a %d x 56 x 56 x 64 "
+                                                                      "tensor resident in HBM" % args.batch},
+                          "roofline": {"bound": "hbm", "peak": 8000.0, "unit": "GB/s"}, "kernels": rows}))
+        return
 
     r = gpu_run(args, dtype)
     step_flop = 3.0 * r["gemm_flop"]

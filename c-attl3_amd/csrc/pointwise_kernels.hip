@@ -431,79 +431,175 @@ int bn_splits(int groups, size_t L) {
  * input sums the windows that cover it in the reference's patch order, so overlapping windows
  * accumulate without atomics and in the reference's order of additions).
  * -------------------------------------------------------------------------------------------- */
-template<typename T, bool MAX>
-__global__ __launch_bounds__(256)
-void pool_forward_kernel(PoolShape s, int N, int OH, int OW, const T* __restrict__ x, T* __restrict__ out,
-		unsigned* __restrict__ inds) {
-	const size_t total = (size_t) N * OH * OW * s.C;
-	const size_t idx = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
-	if (idx >= total)
-		return;
-	const int n = (int) (idx % N);
-	size_t t = idx / N;
-	const int oh = (int) (t % OH);
-	t /= OH;
-	const int ow = (int) (t % OW);
-	const int c = (int) (t / OW);
-	const T* base = x + n + (size_t) N * ((size_t) oh * s.sv + (size_t) s.H * ((size_t) ow * s.sh + (size_t) s.W * c));
-	if (MAX) {
-		/* strict '>' from lowest(): first maximum in (width-major, height-minor) order wins and NaN
-		 * is never selected (MaxPoolLayer.hpp:45-56) */
-		T best = std::numeric_limits<T>::lowest();
-		unsigned bh = 0, bw = 0;
-		for (int k = 0; k < s.RW; ++k)
-			for (int l = 0; l < s.RH; ++l) {
-				const T v = base[(size_t) N * (l + (size_t) s.H * k)];
-				if (v > best) {
-					best = v;
-					bh = (unsigned) l;
-					bw = (unsigned) k;
-				}
-			}
-		out[idx] = best;
-		inds[((size_t) ow * OH + oh) * ((size_t) s.C * N) + (size_t) c * N + n] = bw * (unsigned) s.RH + bh;
+/* Thread layout of the pooling kernels: a thread owns VN consecutive samples (one 16-byte access when
+ * the batch allows it) of POOL_ROWS rows; a block is TX such threads wide and 256/TX tall. Rows are
+ * output rows in the forward pass and input rows in the backward pass. The block index carries
+ * (channel, column, row block, sample block), decoded with block-uniform scalar arithmetic. */
+constexpr int POOL_ROWS = 4;
+
+struct PoolLaunch {
+	int tx, ty, nblks, rblks;
+};
+
+template<typename T, int VN>
+__device__ __forceinline__ void pool_load(T (&dst)[VN], const T* p) {
+	if constexpr (VN == 1) {
+		dst[0] = *p;
 	} else {
-		T sum = (T) 0;
-		for (int k = 0; k < s.RW; ++k)
-			for (int l = 0; l < s.RH; ++l)
-				sum += base[(size_t) N * (l + (size_t) s.H * k)];
-		out[idx] = sum / (T) (s.RH * s.RW);
+		typedef T vt __attribute__((ext_vector_type(VN)));
+		const vt v = *reinterpret_cast<const vt*>(p);
+		#pragma unroll
+		for (int i = 0; i < VN; ++i)
+			dst[i] = v[i];
 	}
 }
 
-template<typename T, bool MAX>
+template<typename T, int VN>
+__device__ __forceinline__ void pool_store(T* p, const T (&src)[VN]) {
+	if constexpr (VN == 1) {
+		*p = src[0];
+	} else {
+		typedef T vt __attribute__((ext_vector_type(VN)));
+		vt v;
+		#pragma unroll
+		for (int i = 0; i < VN; ++i)
+			v[i] = src[i];
+		*reinterpret_cast<vt*>(p) = v;
+	}
+}
+
+template<typename T, bool MAX, int VN>
 __global__ __launch_bounds__(256)
-void pool_backward_kernel(PoolShape s, int N, int OH, int OW, const T* __restrict__ g, const unsigned* __restrict__ inds,
-		T* __restrict__ dx) {
-	const size_t total = (size_t) N * s.H * s.W * s.C;
-	const size_t idx = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
-	if (idx >= total)
+void pool_forward_kernel(PoolShape s, int N, int OH, int OW, PoolLaunch pl, const T* __restrict__ x, T* __restrict__ out,
+		unsigned* __restrict__ inds) {
+	unsigned b = blockIdx.x;
+	const int nb = (int) (b % (unsigned) pl.nblks);
+	b /= (unsigned) pl.nblks;
+	const int rb = (int) (b % (unsigned) pl.rblks);
+	b /= (unsigned) pl.rblks;
+	const int ow = (int) (b % (unsigned) OW);
+	const int c = (int) (b / (unsigned) OW);
+	const int n = (nb * pl.tx + (int) threadIdx.x % pl.tx) * VN;
+	if (n >= N)
 		return;
-	const int n = (int) (idx % N);
-	size_t t = idx / N;
-	const int h = (int) (t % s.H);
-	t /= s.H;
-	const int w = (int) (t % s.W);
-	const int c = (int) (t / s.W);
-	/* windows [o*stride, o*stride + R) containing the coordinate */
+	const int row0 = rb * pl.ty * POOL_ROWS + (int) threadIdx.x / pl.tx;
+	#pragma unroll
+	for (int j = 0; j < POOL_ROWS; ++j) {
+		const int oh = row0 + j * pl.ty;
+		if (oh >= OH)
+			break;
+		const T* base = x + n + (size_t) N * ((size_t) oh * s.sv + (size_t) s.H * ((size_t) ow * s.sh + (size_t) s.W * c));
+		const size_t oidx = n + (size_t) N * (oh + (size_t) OH * (ow + (size_t) OW * c));
+		T res[VN];
+		if (MAX) {
+			/* strict '>' from lowest(): first maximum in (width-major, height-minor) order wins and NaN
+			 * is never selected (MaxPoolLayer.hpp:45-56) */
+			unsigned bi[VN];
+			#pragma unroll
+			for (int v = 0; v < VN; ++v) {
+				res[v] = std::numeric_limits<T>::lowest();
+				bi[v] = 0;
+			}
+			for (int k = 0; k < s.RW; ++k)
+				for (int l = 0; l < s.RH; ++l) {
+					T val[VN];
+					pool_load<T, VN>(val, base + (size_t) N * (l + (size_t) s.H * k));
+					#pragma unroll
+					for (int v = 0; v < VN; ++v)
+						if (val[v] > res[v]) {
+							res[v] = val[v];
+							bi[v] = (unsigned) (k * s.RH + l);
+						}
+				}
+			pool_store<unsigned, VN>(inds + (((size_t) ow * OH + oh) * ((size_t) s.C * N) + (size_t) c * N + n), bi);
+		} else {
+			#pragma unroll
+			for (int v = 0; v < VN; ++v)
+				res[v] = (T) 0;
+			for (int k = 0; k < s.RW; ++k)
+				for (int l = 0; l < s.RH; ++l) {
+					T val[VN];
+					pool_load<T, VN>(val, base + (size_t) N * (l + (size_t) s.H * k));
+					#pragma unroll
+					for (int v = 0; v < VN; ++v)
+						res[v] += val[v];
+				}
+			#pragma unroll
+			for (int v = 0; v < VN; ++v)
+				res[v] = res[v] / (T) (s.RH * s.RW);
+		}
+		pool_store<T, VN>(out + oidx, res);
+	}
+}
+
+template<typename T, bool MAX, int VN>
+__global__ __launch_bounds__(256)
+void pool_backward_kernel(PoolShape s, int N, int OH, int OW, PoolLaunch pl, const T* __restrict__ g,
+		const unsigned* __restrict__ inds, T* __restrict__ dx) {
+	unsigned b = blockIdx.x;
+	const int nb = (int) (b % (unsigned) pl.nblks);
+	b /= (unsigned) pl.nblks;
+	const int rb = (int) (b % (unsigned) pl.rblks);
+	b /= (unsigned) pl.rblks;
+	const int w = (int) (b % (unsigned) s.W);
+	const int c = (int) (b / (unsigned) s.W);
+	const int n = (nb * pl.tx + (int) threadIdx.x % pl.tx) * VN;
+	if (n >= N)
+		return;
+	/* windows [o*stride, o*stride + R) containing the coordinate; the column range is block-uniform */
 	const int ow_lo = w >= s.RW ? (w - s.RW + s.sh) / s.sh : 0;
 	const int ow_hi = min(w / s.sh, OW - 1);
-	const int oh_lo = h >= s.RH ? (h - s.RH + s.sv) / s.sv : 0;
-	const int oh_hi = min(h / s.sv, OH - 1);
 	const T area = (T) (s.RH * s.RW);
-	T sum = (T) 0;
-	for (int ow = ow_lo; ow <= ow_hi; ++ow)
-		for (int oh = oh_lo; oh <= oh_hi; ++oh) {
-			const T gv = g[n + (size_t) N * (oh + (size_t) OH * (ow + (size_t) OW * c))];
-			if (MAX) {
-				const unsigned ind = inds[((size_t) ow * OH + oh) * ((size_t) s.C * N) + (size_t) c * N + n];
-				const unsigned mine = (unsigned) (w - ow * s.sh) * (unsigned) s.RH + (unsigned) (h - oh * s.sv);
-				sum += ind == mine ? gv : (T) 0;
-			} else {
-				sum += gv / area;
+	const int row0 = rb * pl.ty * POOL_ROWS + (int) threadIdx.x / pl.tx;
+	#pragma unroll
+	for (int j = 0; j < POOL_ROWS; ++j) {
+		const int h = row0 + j * pl.ty;
+		if (h >= s.H)
+			break;
+		const int oh_lo = h >= s.RH ? (h - s.RH + s.sv) / s.sv : 0;
+		const int oh_hi = min(h / s.sv, OH - 1);
+		T sum[VN];
+		#pragma unroll
+		for (int v = 0; v < VN; ++v)
+			sum[v] = (T) 0;
+		for (int ow = ow_lo; ow <= ow_hi; ++ow)
+			for (int oh = oh_lo; oh <= oh_hi; ++oh) {
+				T gv[VN];
+				pool_load<T, VN>(gv, g + (n + (size_t) N * (oh + (size_t) OH * (ow + (size_t) OW * c))));
+				if (MAX) {
+					unsigned ind[VN];
+					pool_load<unsigned, VN>(ind, inds + (((size_t) ow * OH + oh) * ((size_t) s.C * N) + (size_t) c * N + n));
+					const unsigned mine = (unsigned) (w - ow * s.sh) * (unsigned) s.RH + (unsigned) (h - oh * s.sv);
+					#pragma unroll
+					for (int v = 0; v < VN; ++v)
+						sum[v] += ind[v] == mine ? gv[v] : (T) 0;
+				} else {
+					#pragma unroll
+					for (int v = 0; v < VN; ++v)
+						sum[v] += gv[v] / area;
+				}
 			}
-		}
-	dx[idx] = sum;
+		pool_store<T, VN>(dx + (n + (size_t) N * (h + (size_t) s.H * (w + (size_t) s.W * c))), sum);
+	}
+}
+
+/* vn = samples per thread */
+PoolLaunch pool_launch(int N, int rows, int vn) {
+	const int nthreads = (N + vn - 1) / vn;
+	PoolLaunch pl;
+	pl.tx = 256;
+	while (pl.tx > 1 && pl.tx / 2 >= nthreads)
+		pl.tx /= 2;
+	pl.ty = 256 / pl.tx;
+	pl.nblks = (nthreads + pl.tx - 1) / pl.tx;
+	pl.rblks = (rows + pl.ty * POOL_ROWS - 1) / (pl.ty * POOL_ROWS);
+	return pl;
+}
+
+unsigned pool_grid(const PoolLaunch& pl, int cols, int channels) {
+	const double blocks = (double) pl.nblks * pl.rblks * cols * channels;
+	CATTLE_HIP_REQUIRE(blocks < 2147483647.0, "pooling launch exceeds the grid limit");
+	return (unsigned) blocks;
 }
 
 template<typename T>
@@ -641,34 +737,53 @@ void bn_backward(int groups, size_t L, const T* out_grad, const T* gamma, const 
 	check_launch();
 }
 
+/* float tensors use 4 samples per thread (16-byte accesses) when possible; doubles use 2 */
+template<typename T, bool MAX>
+void pool_forward_launch(const PoolShape& s, int N, const T* x, T* out, unsigned* inds) {
+	constexpr int VN = 16 / (int) sizeof(T);
+	if (N % 4 == 0 && aligned16(x) && aligned16(out) && (!inds || aligned16(inds))) {
+		const PoolLaunch pl = pool_launch(N, s.OH(), VN);
+		pool_forward_kernel<T, MAX, VN><<<pool_grid(pl, s.OW(), s.C), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), pl, x, out, inds);
+	} else {
+		const PoolLaunch pl = pool_launch(N, s.OH(), 1);
+		pool_forward_kernel<T, MAX, 1><<<pool_grid(pl, s.OW(), s.C), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), pl, x, out, inds);
+	}
+	check_launch();
+}
+
+template<typename T, bool MAX>
+void pool_backward_launch(const PoolShape& s, int N, const T* out_grad, const unsigned* inds, T* in_grad) {
+	constexpr int VN = 16 / (int) sizeof(T);
+	if (N % 4 == 0 && aligned16(out_grad) && aligned16(in_grad) && (!inds || aligned16(inds))) {
+		const PoolLaunch pl = pool_launch(N, s.H, VN);
+		pool_backward_kernel<T, MAX, VN><<<pool_grid(pl, s.W, s.C), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), pl, out_grad, inds,
+				in_grad);
+	} else {
+		const PoolLaunch pl = pool_launch(N, s.H, 1);
+		pool_backward_kernel<T, MAX, 1><<<pool_grid(pl, s.W, s.C), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), pl, out_grad, inds,
+				in_grad);
+	}
+	check_launch();
+}
+
 template<typename T>
 void maxpool_forward(const PoolShape& s, int N, const T* x, T* out, unsigned* inds) {
-	const size_t total = (size_t) N * s.OH() * s.OW() * s.C;
-	pool_forward_kernel<T, true><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), x, out, inds);
-	check_launch();
+	pool_forward_launch<T, true>(s, N, x, out, inds);
 }
 
 template<typename T>
 void maxpool_backward(const PoolShape& s, int N, const T* out_grad, const unsigned* inds, T* in_grad) {
-	const size_t total = (size_t) N * s.H * s.W * s.C;
-	pool_backward_kernel<T, true><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), out_grad, inds,
-			in_grad);
-	check_launch();
+	pool_backward_launch<T, true>(s, N, out_grad, inds, in_grad);
 }
 
 template<typename T>
 void meanpool_forward(const PoolShape& s, int N, const T* x, T* out) {
-	const size_t total = (size_t) N * s.OH() * s.OW() * s.C;
-	pool_forward_kernel<T, false><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), x, out, nullptr);
-	check_launch();
+	pool_forward_launch<T, false>(s, N, x, out, nullptr);
 }
 
 template<typename T>
 void meanpool_backward(const PoolShape& s, int N, const T* out_grad, T* in_grad) {
-	const size_t total = (size_t) N * s.H * s.W * s.C;
-	pool_backward_kernel<T, false><<<(unsigned) ((total + 255) / 256), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), out_grad,
-			nullptr, in_grad);
-	check_launch();
+	pool_backward_launch<T, false>(s, N, out_grad, nullptr, in_grad);
 }
 
 template<typename T>
