@@ -96,6 +96,21 @@ __device__ __forceinline__ int xcd_tile(int bid, int ntiles) {
 	return (bid % XCDS) * per + bid / XCDS;
 }
 
+/* The M tiles of a convolution form a grid of `rows` tiles per output column times `cols` columns
+ * (tile = r + rows*col) when a column is a whole number of tiles. Walking that grid column by
+ * column makes the ~64 tiles an XCD runs at a time one or two tall columns, and the halo they
+ * share with the next column is long gone from L2 when that column's turn comes (each input
+ * element was fetched about three times). Walking it in bands of SWIZZLE_COLS columns, row by row,
+ * makes the running set a compact block instead. Returns the tile for position q of the walk. */
+constexpr int SWIZZLE_COLS = 8;
+__device__ __forceinline__ int swizzle_tile(int q, int rows, int cols) {
+	const int band = q / (rows * SWIZZLE_COLS);
+	const int rem = q - band * rows * SWIZZLE_COLS;
+	const int width = min(SWIZZLE_COLS, cols - band * SWIZZLE_COLS);
+	const int r = rem / width;
+	return r + rows * (band * SWIZZLE_COLS + rem - r * width);
+}
+
 /* Where gathered loads that fall into the zero padding are pointed at. */
 __device__ __attribute__((aligned(16))) const unsigned g_zero_block[4] = { 0u, 0u, 0u, 0u };
 
@@ -118,7 +133,7 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero_block[4] = { 0u, 0
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
 void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom g, const int mtiles) {
+		T* __restrict__ out, const GatherGeom g, const int mtiles, const int tile_rows) {
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_M * WAVES_F;
 	constexpr int BM = WAVES_M * WT_M, BF = WAVES_F * WT_F;
@@ -138,9 +153,11 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	__shared__ __attribute__((aligned(32))) T Bs[2][KC][LDB];
 	__shared__ int4 ktab[3][KC];     /* per reduction index: element offset, ya term, yb term, channel offset */
 
-	const int tile = xcd_tile(blockIdx.x, mtiles);
+	int tile = xcd_tile(blockIdx.x, mtiles);
 	if (tile >= mtiles)
 		return;
+	if (tile_rows > 0)
+		tile = swizzle_tile(tile, tile_rows, mtiles / tile_rows);
 	const int tid = threadIdx.x;
 	const int m0 = tile * BM;
 	const int f0 = blockIdx.y * BF;
@@ -325,6 +342,11 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	}
 }
 
+/* How the weight-gradient launch is cut: tiles = ktiles * ftiles blocks per slice, `splits` slices. */
+struct WgradSplit {
+	int ktiles, tiles, splits, chunks_per_split, pixel_mode;
+};
+
 /* ------------------------------------------------------------------------------------------------
  * Weight-gradient partials: P[k + K*f] = sum over this block's slice of m of A(m,k) * G(m,f), plus the
  * bias-gradient partials (column sums of G over the same slice) from the G tile already in LDS.
@@ -333,13 +355,13 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
  * MFMA step e pairs reduction slot lk with m = mm + lk*VR + e for both operands.
  * The LDS tile is single-buffered: the global loads of the next chunk are in flight in registers
  * while the current chunk is multiplied, and two to three blocks per CU cover the barriers.
- * grid = (ktiles * ftiles, splits). Bias rows are dealt out over the k tiles (row f belongs to the
+ * grid = tiles * splits blocks (1-D). Bias rows are dealt out over the k tiles (row f belongs to the
  * block with f % ktiles == k-tile index) so that every block does the same amount of extra work.
  * ---------------------------------------------------------------------------------------------- */
 template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC>
 __global__ __launch_bounds__(64 * WAVES_K * WAVES_F)
 void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
-		T* __restrict__ bias_partials, const GatherGeom g, const int ktiles, const int chunks_per_split) {
+		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan) {
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_K * WAVES_F;
 	constexpr int BK = WAVES_K * WT_K, BF = WAVES_F * WT_F;
@@ -360,12 +382,32 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	__shared__ int4 ktab[BK];      /* per k row: ya term, yb term, channel offset, valid */
 
 	const int tid = threadIdx.x;
-	const int kt = blockIdx.x % ktiles;
+	/* blocks of one slice (its k and f tiles) get consecutive positions on one XCD: they read the same
+	 * rows of G, which then come out of that XCD's L2 instead of HBM */
+	const int pos = xcd_tile(blockIdx.x, plan.tiles * plan.splits);
+	if (pos >= plan.tiles * plan.splits)
+		return;
+	const int split = pos / plan.tiles, tile = pos - split * plan.tiles;
+	const int ktiles = plan.ktiles;
+	const int kt = tile % ktiles;
 	const int k0 = kt * BK;
-	const int f0 = (blockIdx.x / ktiles) * BF;
-	const int chunk_begin = blockIdx.y * chunks_per_split;
-	const int total_chunks = (g.M + MC - 1) / MC;
-	const int chunk_end = min(chunk_begin + chunks_per_split, total_chunks);
+	const int f0 = (tile / ktiles) * BF;
+	/* The slice of M. Pixel mode (N a multiple of MC): the slice is a range of output positions and is
+	 * walked sample block by sample block (32 samples of every position, then the next 32), so the
+	 * input rows that neighbouring positions share are reused while still in L2. Linear mode: a
+	 * range of 32-row chunks of M in memory order. */
+	const bool pixel_mode = plan.pixel_mode != 0;
+	int chunk_count, pix0 = 0, npix = 1;
+	if (pixel_mode) {
+		const long positions = (long) g.OA * g.OB;
+		pix0 = (int) (positions * split / plan.splits);
+		npix = (int) (positions * (split + 1) / plan.splits) - pix0;
+		chunk_count = npix * (g.N / MC);
+	} else {
+		const int total_chunks = (g.M + MC - 1) / MC;
+		const int begin = split * plan.chunks_per_split;
+		chunk_count = max(0, min(begin + plan.chunks_per_split, total_chunks) - begin);
+	}
 
 	for (int i = tid; i < BK; i += THREADS) {
 		const int k = k0 + i;
@@ -375,20 +417,26 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	}
 
 	const int col = tid % COLS, row0 = tid / COLS;
-	/* m state of this thread's vector: starts at the first chunk of the slice, advances by MC */
-	int m = chunk_begin * MC + col * VEC;
-	int n = m % g.N, a, b;
-	{
+	/* (n, a, b) of this thread's vector for the next chunk to load */
+	int n, a, b, a0, b0, pleft = npix;
+	if (pixel_mode) {
+		n = col * VEC;
+		a0 = a = pix0 % g.OA;
+		b0 = b = pix0 / g.OA;
+	} else {
+		const int m = split * plan.chunks_per_split * MC + col * VEC;
+		n = m % g.N;
 		const int t = m / g.N;
-		a = t % g.OA;
-		b = t / g.OA;
+		a0 = a = t % g.OA;
+		b0 = b = t / g.OA;
 	}
 	const int eN = MC % g.N, eA = (MC / g.N) % g.OA, eB = (MC / g.N) / g.OA;
 
 	T xreg[XSLOTS][VEC], greg[GSLOTS][VEC];
 
 	auto load_tiles = [&]() {
-		const bool mvalid = m < g.M;
+		const int m = n + g.N * (a + g.OA * b);
+		const bool mvalid = b < g.OB;
 		const int ya0 = a * g.SA + g.PA, yb0 = b * g.SB + g.PB;
 		#pragma unroll
 		for (int s = 0; s < XSLOTS; ++s) {
@@ -421,15 +469,28 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 					greg[s][v] = (T) 0;
 			}
 		}
-		/* advance m by MC with carries into (a, b) */
-		m += MC;
-		n += eN;
-		const int c1 = n >= g.N;
-		n -= c1 ? g.N : 0;
-		a += eA + c1;
-		const int c2 = a >= g.OA;
-		a -= c2 ? g.OA : 0;
-		b += eB + c2;
+		if (pixel_mode) {
+			/* next position of the slice; after the last one, back to the first with the next samples */
+			a += 1;
+			const int c1 = a >= g.OA;
+			a -= c1 ? g.OA : 0;
+			b += c1;
+			if (--pleft == 0) {
+				pleft = npix;
+				a = a0;
+				b = b0;
+				n += MC;
+			}
+		} else {
+			/* advance m by MC with carries into (a, b) */
+			n += eN;
+			const int c1 = n >= g.N;
+			n -= c1 ? g.N : 0;
+			a += eA + c1;
+			const int c2 = a >= g.OA;
+			a -= c2 ? g.OA : 0;
+			b += eB + c2;
+		}
 	};
 	auto store_tiles = [&]() {
 		#pragma unroll
@@ -463,13 +524,13 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		bacc[it] = (T) 0;
 
 	__syncthreads();                  /* ktab visible */
-	if (chunk_begin < chunk_end)
+	if (chunk_count > 0)
 		load_tiles();
-	for (int c = chunk_begin; c < chunk_end; ++c) {
+	for (int c = 0; c < chunk_count; ++c) {
 		__syncthreads();              /* every wave is done reading the previous chunk */
 		store_tiles();
 		__syncthreads();
-		if (c + 1 < chunk_end)
+		if (c + 1 < chunk_count)
 			load_tiles();
 		/* operand fragments are fetched one group of VR reduction steps ahead of the MFMAs */
 		T ga[2][FB][VR], xb[2][KB][VR];
@@ -515,7 +576,7 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		}
 	}
 
-	T* dst = partials + (size_t) blockIdx.y * ((size_t) g.K * g.F);
+	T* dst = partials + (size_t) split * ((size_t) g.K * g.F);
 	#pragma unroll
 	for (int i = 0; i < FB; ++i) {
 		#pragma unroll
@@ -548,7 +609,7 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		#pragma unroll
 		for (int q = 0; q < Q; ++q)
 			s += bred[tid * Q + q];
-		bias_partials[(size_t) blockIdx.y * g.F + f0 + tid] = s;
+		bias_partials[(size_t) split * g.F + f0 + tid] = s;
 	}
 }
 
@@ -619,14 +680,19 @@ void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, con
 		int mtiles, bool vec, bool divs) {
 	constexpr int KC = GemmCfg<T>::KC, VEC = GemmCfg<T>::VEC;
 	dim3 block(64 * WAVES_M * WAVES_F);
+	/* tiles per output column, if a column (N * OA rows of M) is a whole number of tiles and there are
+	 * several columns; 0 switches the 2-D walk off */
+	constexpr int BM = WAVES_M * WT_M;
+	const long column = (long) g.N * g.OA;
+	int tile_rows = (column % BM == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE")) ? (int) (column / BM) : 0;
 	if (vec && !divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
 	else if (vec && divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
 	else if (!divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
 	else
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
@@ -740,21 +806,18 @@ constexpr int WGRAD_MC = 32;
 template<typename T>
 struct WgradVariant {
 	int bk, bf, waves, lds_bytes;
-	void (*launch)(dim3 grid, const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom&, int ktiles,
-			int chunks_per_split, bool vec);
+	void (*launch)(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom&, const WgradSplit&, bool vec);
 };
 
 template<typename T, int WK, int WF, int TK, int TF>
-void launch_wgrad_variant(dim3 grid, const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom& g, int ktiles,
-		int chunks_per_split, bool vec) {
+void launch_wgrad_variant(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom& g, const WgradSplit& plan,
+		bool vec) {
 	constexpr int VEC = GemmCfg<T>::VEC;
-	dim3 block(64 * WK * WF);
+	dim3 block(64 * WK * WF), grid((unsigned) round_up(plan.tiles * plan.splits, 8));
 	if (vec)
-		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, VEC><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, ktiles,
-				chunks_per_split);
+		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, VEC><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
 	else
-		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, ktiles,
-				chunks_per_split);
+		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
@@ -795,7 +858,7 @@ template<> struct WgradVariants<double> {
 };
 
 struct WgradPlan {
-	int variant, ktiles, ftiles, splits, chunks_per_split;
+	int variant, ktiles, ftiles, splits, chunks_per_split, pixel_mode;
 };
 
 /* The tile shape with the least padding wins (larger tile on ties: it re-reads G less often); the
@@ -803,7 +866,7 @@ struct WgradPlan {
  * so that no block runs in a second, mostly idle round. The plan depends on the shape only, which
  * keeps the summation order, and with it the result, reproducible. */
 template<typename T>
-WgradPlan wgrad_plan(int M, int K, int F) {
+WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	const WgradVariant<T>* vars = WgradVariants<T>::get();
 	WgradPlan p;
 	p.variant = 0;
@@ -833,6 +896,12 @@ WgradPlan wgrad_plan(int M, int K, int F) {
 	want = std::min(want, std::max(1, chunks / 4));           /* at least four chunks per block */
 	p.chunks_per_split = (chunks + want - 1) / want;
 	p.splits = (chunks + p.chunks_per_split - 1) / p.chunks_per_split;
+	/* pixel mode: slices are ranges of output positions (each at least one), walked sample block by
+	 * sample block; needs chunks that do not straddle positions */
+	const int positions = M / N;
+	p.pixel_mode = N % WGRAD_MC == 0 && positions >= 2 && !std::getenv("CATTLE_HIP_WGRAD_LINEAR");
+	if (p.pixel_mode)
+		p.splits = std::max(1, std::min(want, positions));
 	return p;
 }
 
@@ -845,7 +914,7 @@ ConvWorkspace conv_workspace(const ConvShape& s, int N) {
 	ws.wt_fwd = (size_t) round_up(s.K(), WT_ROW_PAD) * round_up(s.F, WT_COL_PAD);
 	ws.wt_dgrad = (size_t) round_up(s.RH * s.RW * s.F, WT_ROW_PAD) * round_up(s.C, WT_COL_PAD);
 	const int M = N * s.OH() * s.OW();
-	const WgradPlan p = wgrad_plan<T>(M, s.K(), s.F);
+	const WgradPlan p = wgrad_plan<T>(M, s.K(), s.F, N);
 	ws.partials = (size_t) p.splits * ((size_t) s.K() * s.F + (size_t) s.F);
 	return ws;
 }
@@ -870,14 +939,14 @@ void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* o
 	const GatherGeom g = forward_geom(s, N);
 	/* weight and bias gradients: split-M partials, then a fixed-order reduction that accumulates */
 	{
-		const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F);
+		const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N);
 		const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
 		const size_t count = (size_t) g.K * g.F;
 		T* bias_partials = partials + (size_t) p.splits * count;
-		dim3 grid((unsigned) (p.ktiles * p.ftiles), (unsigned) p.splits);
+		const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode };
 		const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
 				(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
-		v.launch(grid, x, out_grad, partials, bias_partials, g, p.ktiles, p.chunks_per_split, vec);
+		v.launch(x, out_grad, partials, bias_partials, g, split, vec);
 		reduce_partials_kernel<T><<<(unsigned) ((count + 63) / 64), 256, 0, stream()>>>(partials, wgrad, count, p.splits);
 		CATTLE_HIP_CHECK(hipGetLastError());
 		reduce_partials_kernel<T><<<(unsigned) ((g.F + 63) / 64), 256, 0, stream()>>>(bias_partials, bgrad, (size_t) g.F, p.splits);
