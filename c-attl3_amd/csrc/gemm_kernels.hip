@@ -49,6 +49,19 @@ template<> struct Mfma<double> {
 	}
 };
 
+/* Reduction chunk, global-load vector width and LDS row padding of the gather GEMM. The padding
+ * keeps the two (f32) or four (f64) reduction slots of a wave on different banks; the 512-row
+ * tile uses the smaller padding that still does, so that two blocks fit the 160 KB of LDS. */
+template<typename T> struct GemmCfg;
+template<> struct GemmCfg<float> {
+	static constexpr int KC = 16, VEC = 4;
+	static constexpr int pad(int bm) { return bm >= 512 ? 16 : 32; }
+};
+template<> struct GemmCfg<double> {
+	static constexpr int KC = 8, VEC = 2;
+	static constexpr int pad(int) { return 16; }
+};
+
 /* Row (i index) of accumulator register r for a lane in reduction slot lk (= lane / TL), as measured
  * on gfx950: 32x32x2 f32 packs rows in groups of four per slot, 16x16x4 f64 interleaves the slots. */
 template<typename T>
@@ -137,7 +150,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_M * WAVES_F;
 	constexpr int BM = WAVES_M * WT_M, BF = WAVES_F * WT_F;
-	constexpr int PAD = std::is_same<T, float>::value ? 32 : 16;
+	constexpr int PAD = GemmCfg<T>::pad(BM);
 	constexpr int LDA = BM + PAD, LDB = BF + PAD;
 	constexpr int TL = MF::TL, KS = MF::KS;
 	constexpr int MB = WT_M / TL, FB = WT_F / TL;
@@ -664,9 +677,6 @@ constexpr int NUM_CUS = 256;
 constexpr int LDS_PER_CU = 160 * 1024;
 constexpr int MAX_WAVES_PER_CU = 16;   /* four per SIMD: every kernel here stays within 128 registers per lane */
 
-template<typename T> struct GemmCfg;
-template<> struct GemmCfg<float> { static constexpr int KC = 16, VEC = 4, PAD = 32; };
-template<> struct GemmCfg<double> { static constexpr int KC = 8, VEC = 2, PAD = 16; };
 
 /* One instantiation of gather_gemm_kernel and what the tile chooser needs to know about it. */
 template<typename T>
@@ -703,7 +713,7 @@ GatherVariant<T> gather_variant() {
 	v.bm = WAVES_M * WT_M;
 	v.bf = WAVES_F * WT_F;
 	v.waves = WAVES_M * WAVES_F;
-	v.lds_bytes = 2 * C::KC * (v.bm + C::PAD + v.bf + C::PAD) * (int) sizeof(T) + 3 * C::KC * 16;
+	v.lds_bytes = 2 * C::KC * (v.bm + v.bf + 2 * C::pad(v.bm)) * (int) sizeof(T) + 3 * C::KC * 16;
 	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F>;
 	return v;
 }
@@ -740,10 +750,14 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	const bool vec = g.N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
 	const bool divs = g.DA != 1 || g.DB != 1;
 	const GatherVariant<T>* vars = GatherVariants<T>::get();
-	int best_v = 0;                     /* the table is ordered from the widest F tile to the narrowest */
-	for (int i = 1; i < GatherVariants<T>::COUNT; ++i)
-		if (vars[i].bf >= g.F)
+	int best_v = 0;
+	for (int i = 1; i < GatherVariants<T>::COUNT; ++i) {
+		const bool narrower = vars[i].bf >= g.F && vars[i].bf < vars[best_v].bf;
+		/* same width, taller tile: half the A-operand loads per MFMA; worth it once it still fills the chip */
+		const bool taller = vars[i].bf == vars[best_v].bf && vars[i].bm > vars[best_v].bm && g.M >= vars[i].bm * NUM_CUS * 4;
+		if (narrower || taller)
 			best_v = i;
+	}
 	/* tuning overrides for experiments, keyed by the number of output columns F of the GEMM:
 	 * CATTLE_HIP_GATHER_VARIANT_F<F> = index into the variant table, CATTLE_HIP_GATHER_OCC_F<F> = blocks per CU
 	 * (enforced by reserving dynamic LDS) */
