@@ -1,0 +1,442 @@
+"""Host-side counterparts of the reference's callers, used by the parity tests to
+drive the layers the way C-ATTL3's networks and optimizers do. Nothing here is product code; the
+same orchestration runs on two back ends with one interface:
+
+  * the HIP layers of libcattle_hip (through the Python binding), and
+  * `Oracle*` layers that wrap the CPU oracle's functions and keep the caches the reference keeps.
+
+Cited reference files are relative to C-ATTL3/.
+"""
+import importlib
+
+import numpy as np
+
+from oracle import oracle
+
+
+# ------------------------------------------------------------------------------------------------
+# Oracle-backed layers with the cattle::Layer interface (pass_forward / pass_back / get_params)
+# ------------------------------------------------------------------------------------------------
+class HostParams(object):
+    """parameters/StandardParameters.hpp:37-191 at default constraints: values + accumulated gradient."""
+
+    def __init__(self, rows, cols, dtype, optimizable=True, init=0.0):
+        self.values = np.full((rows, cols), init, dtype=dtype, order="F")
+        self.grad = np.zeros((rows, cols), dtype=dtype, order="F")
+        self.optimizable = optimizable
+
+    def get_values(self):
+        return self.values
+
+    def set_values(self, v):
+        self.values = np.asfortranarray(v, dtype=self.values.dtype).reshape(self.values.shape, order="F")
+
+    def get_grad(self):
+        return self.grad
+
+    def accumulate_grad(self, g):
+        if self.optimizable:
+            self.grad += np.reshape(g, self.grad.shape, order="F")
+
+    def reset_grad(self):
+        self.grad[...] = 0
+
+    def are_optimizable(self):
+        return self.optimizable
+
+
+class OracleLayer(object):
+    def __init__(self, dtype):
+        self.dtype = np.dtype(dtype)
+        self.input_layer = False
+        self.params = []
+
+    def set_input_layer(self, flag):
+        self.input_layer = bool(flag)
+
+    def is_input_layer(self):
+        return self.input_layer
+
+    def get_params(self):
+        return self.params
+
+    def clone_with_shared_params(self):
+        c = object.__new__(type(self))
+        c.__dict__.update(self.__dict__)        # same HostParams objects, own caches from now on
+        return c
+
+
+class OracleConv(OracleLayer):
+    """layer/kernel/ConvKernelLayer.hpp:115-189"""
+
+    def __init__(self, dtype, input_dims, filters, RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0):
+        OracleLayer.__init__(self, dtype)
+        H, W, C = input_dims
+        self.geom = dict(RH=RH, RW=RW, pv=pv, ph=ph, sv=sv, sh=sh, dv=dv, dh=dh)
+        self.params = [HostParams(RH * RW * C, filters, dtype), HostParams(1, filters, dtype)]
+        OH, OW = oracle.conv_out_dims(H, W, RH, RW, pv, ph, sv, sh, dv, dh)
+        self.out_dims = (OH, OW, filters)
+
+    def get_output_dims(self):
+        return self.out_dims
+
+    def pass_forward(self, x, training):
+        self.x_shape = x.shape
+        out, self.cache = oracle.conv_forward(np.asarray(x, self.dtype), self.params[0].values, self.params[1].values,
+                                              return_cache=True, **self.geom)
+        return out
+
+    def pass_back(self, g):
+        dx, dw, db = oracle.conv_backward(self.x_shape, self.cache, self.params[0].values, np.asarray(g, self.dtype),
+                                          input_layer=self.input_layer, **self.geom)
+        self.params[0].accumulate_grad(dw)
+        self.params[1].accumulate_grad(db)
+        return dx
+
+
+class OracleDense(OracleLayer):
+    """layer/kernel/DenseKernelLayer.hpp:92-115"""
+
+    def __init__(self, dtype, input_dims, output_size):
+        OracleLayer.__init__(self, dtype)
+        self.in_dims = tuple(input_dims)
+        V = int(np.prod(input_dims))
+        self.params = [HostParams(V, output_size, dtype), HostParams(1, output_size, dtype)]
+        self.out_dims = (output_size,) + (1,) * (len(input_dims) - 1)
+
+    def get_output_dims(self):
+        return self.out_dims
+
+    def pass_forward(self, x, training):
+        self.x = np.asarray(x, self.dtype)
+        out = oracle.dense_forward(self.x, self.params[0].values, self.params[1].values)
+        return out.reshape((x.shape[0],) + self.out_dims, order="F")
+
+    def pass_back(self, g):
+        N = self.x.shape[0]
+        dx, dw, db = oracle.dense_backward(self.x, self.params[0].values, np.asarray(g, self.dtype).reshape((N, -1), order="F"),
+                                           input_layer=self.input_layer)
+        self.params[0].accumulate_grad(dw)
+        self.params[1].accumulate_grad(db)
+        return dx
+
+
+class OracleActivation(OracleLayer):
+    def __init__(self, dtype, kind, dims, param=0.0):
+        OracleLayer.__init__(self, dtype)
+        self.kind, self.p, self.dims = kind, float(np.dtype(dtype).type(param)), tuple(dims)
+
+    def get_output_dims(self):
+        return self.dims
+
+    def pass_forward(self, x, training):
+        self.x = np.asarray(x, self.dtype)
+        self.y = oracle.act_forward(self.kind, self.x, self.p)
+        return self.y
+
+    def pass_back(self, g):
+        if self.input_layer:
+            return None
+        return oracle.act_backward(self.kind, self.x, self.y, np.asarray(g, self.dtype), self.p)
+
+
+class OracleBatchNorm(OracleLayer):
+    """layer/BatchNormLayer.hpp:170-272 (per last rank)."""
+
+    def __init__(self, dtype, dims, norm_avg_decay=0.1, epsilon=1e-5):
+        OracleLayer.__init__(self, dtype)
+        self.dims = tuple(dims)
+        C = dims[-1]
+        self.params = [HostParams(1, C, dtype, False), HostParams(1, C, dtype, False), HostParams(1, C, dtype, True, 1.0),
+                       HostParams(1, C, dtype)]
+        self.decay, self.eps, self.stats_init = float(np.dtype(dtype).type(norm_avg_decay)), float(np.dtype(dtype).type(epsilon)), False
+
+    def get_output_dims(self):
+        return self.dims
+
+    def pass_forward(self, x, training):
+        am = np.ascontiguousarray(self.params[0].values.reshape(-1))
+        ais = np.ascontiguousarray(self.params[1].values.reshape(-1))
+        y, self.std, self.isd = oracle.bn_forward(np.asarray(x, self.dtype), self.params[2].values.reshape(-1),
+                                                  self.params[3].values.reshape(-1), am, ais, self.stats_init, training,
+                                                  decay=self.decay, eps=self.eps)
+        if training:
+            self.params[0].set_values(am.reshape(1, -1))
+            self.params[1].set_values(ais.reshape(1, -1))
+            self.stats_init = True
+        return y
+
+    def pass_back(self, g):
+        dx, dg, db = oracle.bn_backward(np.asarray(g, self.dtype), self.params[2].values.reshape(-1), self.std, self.isd,
+                                        input_layer=self.input_layer)
+        self.params[2].accumulate_grad(dg)
+        self.params[3].accumulate_grad(db)
+        return dx
+
+
+class OracleMaxPool(OracleLayer):
+    """layer/pool/MaxPoolLayer.hpp:38-80 + layer/PoolLayer.hpp:77-116"""
+
+    def __init__(self, dtype, input_dims, RH=2, RW=2, sv=2, sh=2):
+        OracleLayer.__init__(self, dtype)
+        self.g = (RH, RW, sv, sh)
+        OH, OW = oracle.pool_out_dims(input_dims[0], input_dims[1], RH, RW, sv, sh)
+        self.out_dims = (OH, OW, input_dims[2])
+
+    def get_output_dims(self):
+        return self.out_dims
+
+    def pass_forward(self, x, training):
+        self.x_shape = x.shape
+        out, self.inds = oracle.maxpool_forward(np.asarray(x, self.dtype), *self.g)
+        return out
+
+    def max_indices(self, batch):
+        return self.inds
+
+    def pass_back(self, g):
+        if self.input_layer:
+            return None
+        return oracle.maxpool_backward(self.x_shape, np.asarray(g, self.dtype), self.inds, *self.g)
+
+
+class OracleBackend(object):
+    name = "oracle"
+
+    def __init__(self, dtype):
+        self.dtype = np.dtype(dtype)
+
+    def conv(self, dims, filters, **kw):
+        return OracleConv(self.dtype, dims, filters, **kw)
+
+    def dense(self, dims, out):
+        return OracleDense(self.dtype, dims, out)
+
+    def act(self, kind, dims, param=0.0):
+        return OracleActivation(self.dtype, kind, dims, param)
+
+    def batchnorm(self, dims):
+        return OracleBatchNorm(self.dtype, dims)
+
+    def maxpool(self, dims):
+        return OracleMaxPool(self.dtype, dims)
+
+
+class HipBackend(object):
+    name = "hip"
+
+    def __init__(self, dtype):
+        self.dtype = np.dtype(dtype)
+        self.ch = importlib.import_module("c-attl3_amd")
+
+    def conv(self, dims, filters, RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0):
+        return self.ch.ConvKernelLayer(self.dtype, dims, filters, RH, RW, pv, ph, sv, sh, dv, dh)
+
+    def dense(self, dims, out):
+        return self.ch.DenseKernelLayer(self.dtype, dims, out)
+
+    def act(self, kind, dims, param=0.0):
+        return self.ch.ActivationLayer(self.dtype, kind, dims, param)
+
+    def batchnorm(self, dims):
+        return self.ch.BatchNormLayer(self.dtype, dims)
+
+    def maxpool(self, dims):
+        return self.ch.MaxPoolLayer(self.dtype, dims)
+
+
+# ------------------------------------------------------------------------------------------------
+# Callers: feed-forward network, losses, optimizers
+# ------------------------------------------------------------------------------------------------
+class FeedforwardNet(object):
+    """neural_network/FeedforwardNeuralNetwork.hpp:38-53 (layer 0 is the input layer), :112-127."""
+
+    def __init__(self, layers, foremost=True):
+        self.layers = layers
+        layers[0].set_input_layer(foremost)
+
+    def propagate(self, x, training, keep=None):
+        for l in self.layers:
+            x = l.pass_forward(x, training)
+            if keep is not None:
+                keep.append(x)
+        return x
+
+    def backpropagate(self, g, keep=None):
+        for l in reversed(self.layers):
+            g = l.pass_back(g)
+            if keep is not None:
+                keep.append(g)
+        return g
+
+    def params(self):
+        out = []
+        for l in self.layers:
+            out.extend(l.get_params())
+        return out
+
+
+def softmax_ce_grad(out, obj, eps=1e-5):
+    """loss/SoftmaxCrossEntropyLoss.hpp:41-50: softmax with epsilon in the denominator minus the objective."""
+    N = out.shape[0]
+    o = np.asarray(out).reshape((N, -1), order="F")
+    e = np.exp(o - o.max(axis=1, keepdims=True))
+    g = e / (e.sum(axis=1, keepdims=True) + o.dtype.type(eps)) - np.asarray(obj, o.dtype).reshape((N, -1), order="F")
+    return np.asfortranarray(g.astype(o.dtype)).reshape(out.shape, order="F")
+
+
+def squared_loss_grad(out, obj):
+    """loss/SquaredLoss.hpp:30-34"""
+    return np.asfortranarray((2 * (np.asarray(out) - np.asarray(obj, out.dtype))).astype(out.dtype))
+
+
+def train_step_gradients(net, x, obj, loss_grad, keep_fwd=None, keep_bwd=None):
+    """optimizer/SGDOptimizer.hpp:44-56: propagate, loss gradient divided by the batch size, backpropagate."""
+    out = net.propagate(x, True, keep_fwd)
+    g = loss_grad(out, obj) / out.dtype.type(x.shape[0])
+    net.backpropagate(np.asfortranarray(g.astype(out.dtype)), keep_bwd)
+    return out
+
+
+def vanilla_sgd_update(params, lr=1e-3):
+    """optimizer/VanillaSGDOptimizer.hpp:38-43"""
+    for p in params:
+        if p.are_optimizable():
+            v = p.get_values()
+            p.set_values(v - v.dtype.type(lr) * p.get_grad())
+
+
+class Adam(object):
+    """optimizer/AdamOptimizer.hpp:55-82 (the reference's variant: decays 0.1 / 1e-3, epsilon inside both the
+    bias corrections and the square root)."""
+
+    def __init__(self, params, lr=1e-3, l1_decay=1e-1, l2_decay=1e-3, eps=1e-5):
+        self.lr, self.d1, self.d2, self.eps = lr, l1_decay, l2_decay, eps
+        self.state = [(np.zeros_like(p.get_values()), np.zeros_like(p.get_values())) for p in params if p.are_optimizable()]
+
+    def update(self, params, timestep=0):
+        i = 0
+        for p in params:
+            if not p.are_optimizable():
+                continue
+            v = p.get_values()
+            t = v.dtype.type
+            c1 = t(1) / t(1 - (1 - self.d1) ** (timestep + 1) + self.eps)
+            c2 = t(1) / t(1 - (1 - self.d2) ** (timestep + 1) + self.eps)
+            g = p.get_grad()
+            m, s = self.state[i]
+            m = m * t(1 - self.d1) + g * t(self.d1)
+            s = s * t(1 - self.d2) + g * g * t(self.d2)
+            self.state[i] = (m, s)
+            i += 1
+            p.set_values(v - (m * t(self.lr * c1)) / np.sqrt(s * c2 + t(self.eps)))
+
+
+# ------------------------------------------------------------------------------------------------
+# BASELINE configs 2, 3 and 5
+# ------------------------------------------------------------------------------------------------
+def he_normal(gen, rows, cols, dtype):
+    return np.asfortranarray((gen.standard_normal((rows, cols)) * np.sqrt(2.0 / rows)).astype(dtype))
+
+
+def build_mlp(backend):
+    """Config 2: DenseKernelLayer<float,1> 784 -> 512 -> 256 -> 10 with ReLU between."""
+    b = backend
+    return FeedforwardNet([b.dense((784,), 512), b.act("relu", (512,)), b.dense((512,), 256), b.act("relu", (256,)),
+                           b.dense((256,), 10)])
+
+
+def build_convnet(backend):
+    """Config 3: conv 3x3x32 p1 -> ReLU -> maxpool 2x2 -> conv 3x3x64 p1 -> BatchNorm -> ReLU -> maxpool 2x2 -> dense 10."""
+    b = backend
+    return FeedforwardNet([b.conv((32, 32, 3), 32), b.act("relu", (32, 32, 32)), b.maxpool((32, 32, 32)),
+                           b.conv((16, 16, 32), 64), b.batchnorm((16, 16, 64)), b.act("relu", (16, 16, 64)),
+                           b.maxpool((16, 16, 64)), b.dense((8, 8, 64), 10)])
+
+
+def init_kernel_weights(net, seed, dtype):
+    """He-normal weights for every kernel layer (parameter_initialization/HeParameterInitialization.hpp:34-36),
+    zero bias; identical values for any back end."""
+    gen = np.random.default_rng(seed)
+    for l in net.layers:
+        ps = l.get_params()
+        if len(ps) == 2:
+            v = ps[0].get_values()
+            ps[0].set_values(he_normal(gen, v.shape[0], v.shape[1], dtype))
+
+
+class ConvLSTM(object):
+    """neural_network/LSTMNeuralNetwork.hpp:236-503 with ConvKernelLayer kernels, no multiplicative
+    integration, not stateful, foremost (input kernels are input layers, :193-199), unrolled with
+    shared-parameter clones (:536-573). Output schedule (1, T-1): the last hidden state."""
+
+    GATES = ("forget", "write", "candidate", "read")
+
+    def __init__(self, backend, dims=(16, 16, 8), hidden=32, steps=10):
+        b = backend
+        self.T = steps
+        hdims = (dims[0], dims[1], hidden)
+        self.hdims = hdims
+        self.main = {}
+        for gate in self.GATES:
+            self.main["in_" + gate] = b.conv(dims, hidden)
+            self.main["out_" + gate] = b.conv(hdims, hidden)
+            self.main["in_" + gate].set_input_layer(True)
+        for gate, kind in (("forget", "sigmoid"), ("write", "sigmoid"), ("candidate", "tanh"), ("read", "sigmoid"), ("state", "tanh")):
+            self.main["act_" + gate] = b.act(kind, hdims)
+        self.cells = [self.main]
+        for _ in range(steps - 1):
+            self.cells.append({k: v.clone_with_shared_params() for k, v in self.main.items()})
+
+    def kernel_params(self):
+        out = []
+        for gate in self.GATES:
+            out.append(("in_" + gate, self.main["in_" + gate].get_params()))
+            out.append(("out_" + gate, self.main["out_" + gate].get_params()))
+        return out
+
+    def propagate(self, x):
+        """x: (N, T, H, W, C), Fortran order; returns the hidden output of the last step (N, H, W, hidden)."""
+        N = x.shape[0]
+        dt = x.dtype
+        state = np.zeros((N,) + self.hdims, dtype=dt, order="F")
+        hidden = None
+        for i in range(self.T):
+            c = self.cells[i]
+            xi = np.asfortranarray(x[:, i])
+            pre = {}
+            for gate in self.GATES:
+                w = c["in_" + gate].pass_forward(xi, True)
+                if i > 0:
+                    w = w + c["out_" + gate].pass_forward(hidden, True)
+                pre[gate] = np.asfortranarray(w)
+            c["forget_f"] = c["act_forget"].pass_forward(pre["forget"], True)
+            c["prev_state"] = state
+            state = c["forget_f"] * c["prev_state"]
+            c["write_f"] = c["act_write"].pass_forward(pre["write"], True)
+            c["cand"] = c["act_candidate"].pass_forward(pre["candidate"], True)
+            state = state + c["write_f"] * c["cand"]
+            c["read_f"] = c["act_read"].pass_forward(pre["read"], True)
+            c["act_state_v"] = c["act_state"].pass_forward(np.asfortranarray(state), True)
+            hidden = np.asfortranarray(c["read_f"] * c["act_state_v"])
+        return hidden
+
+    def backpropagate(self, out_grad):
+        state_grad = np.zeros_like(out_grad)
+        hidden_grad = np.zeros_like(out_grad)
+        F = np.asfortranarray
+        for i in range(self.T - 1, -1, -1):
+            c = self.cells[i]
+            if i == self.T - 1:
+                hidden_grad = hidden_grad + out_grad
+            state_grad = state_grad + c["act_state"].pass_back(F(c["read_f"] * hidden_grad))
+            g_read = c["act_read"].pass_back(F(c["act_state_v"] * hidden_grad))
+            g_cand = c["act_candidate"].pass_back(F(c["write_f"] * state_grad))
+            g_write = c["act_write"].pass_back(F(c["cand"] * state_grad))
+            g_forget = c["act_forget"].pass_back(F(c["prev_state"] * state_grad))
+            state_grad = state_grad * c["forget_f"]
+            if i != 0:
+                hidden_grad = (c["out_read"].pass_back(g_read) + c["out_candidate"].pass_back(g_cand) +
+                               c["out_write"].pass_back(g_write) + c["out_forget"].pass_back(g_forget))
+            for gate, g in (("read", g_read), ("candidate", g_cand), ("write", g_write), ("forget", g_forget)):
+                c["in_" + gate].pass_back(g)
