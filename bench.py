@@ -27,6 +27,18 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}      # MI355X dense matrix peaks (no sparsity)
 SHAPE = dict(H=56, W=56, C=64, F=128, RH=3, RW=3)
 
+# HBM bytes per launch (read + written) of the three GEMM kernels on the default workload (f32, batch 256):
+# rocprofv3 FETCH_SIZE and WRITE_SIZE readings of `bench.py --copy-calibration`, each scaled by what the same
+# counter reads for the calibration copy of known size (FETCH_SIZE x2.0, WRITE_SIZE x1.0). Counters cannot be
+# read while timing, so these are constants of the measured build; other shapes report null.
+MEASURED_TRAFFIC = {
+    ("f32", 256): {
+        "gather_gemm_kernel (forward)": 389.9e6 + 411.0e6,
+        "wgrad_kernel (+ reduce, bias column sums)": 945.7e6 + 50.3e6 + 2 * 12.6e6 + 0.3e6,
+        "gather_gemm_kernel (input gradient)": 726.6e6 + 205.5e6,
+    },
+}
+
 
 def he_normal(gen, rows, cols, dtype):
     # parameter_initialization/HeParameterInitialization.hpp:34-36: sd = sqrt(2 / fan_in), fan_in = rows
@@ -83,6 +95,13 @@ def gpu_run(args, dtype):
         "wgrad_kernel (+ reduce, bias column sums)": t_wgrad,
         "gather_gemm_kernel (input gradient)": t_dgrad,
     }
+    es = np.dtype(dtype).itemsize
+    in_b, out_b, w_b = N * H * W * C * es, N * H * W * F * es, K * F * es
+    nbytes = {
+        "gather_gemm_kernel (forward)": in_b + w_b + out_b,
+        "wgrad_kernel (+ reduce, bias column sums)": in_b + out_b + w_b,
+        "gather_gemm_kernel (input gradient)": out_b + w_b + in_b,
+    }
     if args.copy_calibration:
         # a plain copy kernel of known size (identity activation: reads and writes x.nbytes) so that
         # FETCH_SIZE / WRITE_SIZE counter readings of the same profile can be scaled to bytes
@@ -90,7 +109,7 @@ def gpu_run(args, dtype):
         for _ in range(3):
             ident.forward_into(x, dx, True)
         ch.synchronize()
-    return dict(wall_ms=wall_ms, M=M, K=K, F=F, gemm_flop=gemm_flop, kernels=kernels)
+    return dict(wall_ms=wall_ms, M=M, K=K, F=F, gemm_flop=gemm_flop, kernels=kernels, bytes=nbytes)
 
 
 def pointwise_run(args, dtype):
@@ -209,7 +228,9 @@ def main():
         "samples_per_s": round(args.batch / (r["wall_ms"] * 1e-3), 1),
         "frac_of_mfma_peak": round(gflops / 1e3 / peak, 4),
         "roofline": {"bound": "mfma", "kernel": name, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "frac": round(achieved / peak, 4),
+                     "traffic": MEASURED_TRAFFIC.get((args.dtype, args.batch), {}).get(name),
+                     "algorithmic_bytes": r["bytes"][name],
                      "flop_per_launch": r["gemm_flop"], "ms_per_launch": round(t_ms, 4)},
         "kernel_ms": {k: round(v, 4) for k, v in r["kernels"].items()},
     }
