@@ -36,7 +36,9 @@ EXPORTS = [
     "cattle_hip_layer_empty_cache", "cattle_hip_layer_forward", "cattle_hip_layer_backward",
     "cattle_hip_layer_num_params", "cattle_hip_layer_param_shape", "cattle_hip_layer_set_param_values",
     "cattle_hip_layer_get_param_values", "cattle_hip_layer_get_param_grad", "cattle_hip_layer_reset_param_grad",
-    "cattle_hip_maxpool_indices",
+    "cattle_hip_maxpool_indices", "cattle_hip_loss_function", "cattle_hip_loss_d_function",
+    "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
+    "cattle_hip_layer_param_reset_optimizer_state",
 ]
 
 
@@ -185,6 +187,64 @@ class Parameters(object):
 
     def reset_grad(self):
         _check(lib().cattle_hip_layer_reset_param_grad(self._layer._h, _sz(self._index)))
+
+    def sgd_update(self, learning_rate=1e-3):
+        """VanillaSGDOptimizer::_update_params on the device (optimizer/VanillaSGDOptimizer.hpp:38-43)."""
+        _check(lib().cattle_hip_layer_param_sgd_update(self._layer._h, _sz(self._index), ctypes.c_double(learning_rate)))
+
+    def adam_update(self, timestep, learning_rate=1e-3, l1_decay=1e-1, l2_decay=1e-3, epsilon=1e-5):
+        """AdamOptimizer::_update_params on the device; defaults of optimizer/AdamOptimizer.hpp:40-42."""
+        _check(lib().cattle_hip_layer_param_adam_update(self._layer._h, _sz(self._index), ctypes.c_double(learning_rate),
+                                                        ctypes.c_double(l1_decay), ctypes.c_double(l2_decay),
+                                                        ctypes.c_double(epsilon), _sz(timestep)))
+
+    def reset_optimizer_state(self):
+        """AdamOptimizer::_fit: zero the moving averages."""
+        _check(lib().cattle_hip_layer_param_reset_optimizer_state(self._layer._h, _sz(self._index)))
+
+
+LOSS = {"squared": 0, "softmax_cross_entropy": 1}
+
+
+def _loss_args(out, obj, sequential):
+    if isinstance(out, DeviceTensor) != isinstance(obj, DeviceTensor):
+        raise TypeError("out and obj must both be numpy arrays or both DeviceTensors")
+    if not isinstance(out, DeviceTensor):
+        out = np.asfortranarray(out)
+        obj = np.asfortranarray(obj, dtype=out.dtype)
+    if tuple(out.shape) != tuple(obj.shape):
+        raise ValueError("out and obj dimensions differ")          # assert(out.dimensions() == obj.dimensions())
+    batch = out.shape[0]
+    steps = out.shape[1] if sequential else 1
+    size = int(np.prod(out.shape[1:])) // steps
+    dev = isinstance(out, DeviceTensor)
+    ptr = (lambda t: t.ptr) if dev else (lambda a: ctypes.c_void_p(a.ctypes.data))
+    return out, obj, batch, steps, size, (DEVICE if dev else HOST), ptr
+
+
+def loss_function(kind, out, obj, epsilon=1e-5, sequential=False):
+    """Loss::function: the per-sample losses of a batch as a numpy vector (loss/UniversalLoss.hpp:37-41, :99-110).
+    out/obj are numpy arrays or DeviceTensors of shape (N, ...) or, if sequential, (N, T, ...)."""
+    out, obj, batch, steps, size, space, ptr = _loss_args(out, obj, sequential)
+    losses = np.empty((batch,), dtype=out.dtype)
+    _check(lib().cattle_hip_loss_function(_dtype_code(out.dtype), ctypes.c_int(LOSS[kind]), ptr(out), space, ptr(obj), space,
+                                          _sz(batch), _sz(steps), _sz(size), ctypes.c_double(epsilon),
+                                          ctypes.c_void_p(losses.ctypes.data), HOST))
+    return losses
+
+
+def loss_d_function(kind, out, obj, epsilon=1e-5, scale=1.0, sequential=False):
+    """Loss::d_function times scale (loss/UniversalLoss.hpp:42-46, :111-125); returns what it was given
+    (numpy array or DeviceTensor) in the shape of out."""
+    out, obj, batch, steps, size, space, ptr = _loss_args(out, obj, sequential)
+    if space == DEVICE:
+        grad = DeviceTensor(out.shape, out.dtype)
+    else:
+        grad = np.empty(out.shape, dtype=out.dtype, order="F")
+    _check(lib().cattle_hip_loss_d_function(_dtype_code(out.dtype), ctypes.c_int(LOSS[kind]), ptr(out), space, ptr(obj), space,
+                                            _sz(batch), _sz(steps), _sz(size), ctypes.c_double(epsilon),
+                                            ctypes.c_double(scale), ptr(grad), space))
+    return grad
 
 
 class Layer(object):

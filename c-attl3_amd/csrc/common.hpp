@@ -5,6 +5,8 @@
 #define CATTLE_HIP_COMMON_HPP_
 
 #include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <stdexcept>
@@ -109,6 +111,16 @@ template<typename T> void meanpool_backward(const PoolShape& s, int N, const T* 
 
 /* dst[i] += src[i] */
 template<typename T> void axpy_one(size_t n, const T* src, T* dst);
+
+/* Losses and optimizer updates (train_kernels.hip). A batch is N samples x T_steps x V elements,
+ * column-major with the sample index fastest. */
+enum { LOSS_SQUARED = 0, LOSS_SOFTMAX_CROSS_ENTROPY = 1 };
+template<typename T> void loss_function(int kind, int N, int T_steps, int V, T eps, const T* out, const T* obj, T* losses);
+template<typename T> void loss_d_function(int kind, int N, int T_steps, int V, T eps, T scale, const T* out, const T* obj,
+		T* grad);
+template<typename T> void sgd_update(size_t n, T lr, const T* grad, T* values);
+template<typename T> void adam_update(size_t n, T lr, T l1_decay, T l2_decay, T eps, size_t timestep, const T* grad, T* m,
+		T* v, T* values);
 
 } /* namespace cattle_hip */
 

@@ -100,6 +100,8 @@ struct Param {
 	uint64_t version = 1;
 	DevBuf derived[2];
 	uint64_t derived_version[2] = { 0, 0 };
+	DevBuf moments[2];                 /* optimizer moving averages, allocated on first use */
+	bool moments_ready = false;
 	Param(size_t rows, size_t cols, bool optimizable, size_t esize) : rows(rows), cols(cols), optimizable(optimizable), esize(esize) {
 		values.ensure(bytes());
 		grad.ensure(bytes());
@@ -446,6 +448,62 @@ int guarded(Fn fn) {
 		return CATTLE_HIP_ERR_INVALID;
 	}
 }
+
+/* Staging for the loss entry points when the caller's buffers are host memory. */
+struct LossStage {
+	DevBuf out, obj, dst;
+};
+LossStage g_loss_stage;
+
+template<typename T>
+void run_loss(bool grad_pass, int kind, const void* out, int out_space, const void* obj, int obj_space, size_t batch,
+		size_t time_steps, size_t sample_size, double epsilon, double scale, void* dst, int dst_space) {
+	const size_t count = batch * time_steps * sample_size;
+	CATTLE_HIP_REQUIRE(count <= 2147483647u, "tensor exceeds 2^31-1 elements");
+	const size_t bytes = count * sizeof(T), dst_bytes = grad_pass ? bytes : batch * sizeof(T);
+	const T* out_dev = static_cast<const T*>(out);
+	const T* obj_dev = static_cast<const T*>(obj);
+	if (out_space == CATTLE_HIP_HOST) {
+		copy_in(g_loss_stage.out.ensure(bytes), out, CATTLE_HIP_HOST, bytes);
+		out_dev = static_cast<const T*>(g_loss_stage.out.p);
+	}
+	if (obj_space == CATTLE_HIP_HOST) {
+		copy_in(g_loss_stage.obj.ensure(bytes), obj, CATTLE_HIP_HOST, bytes);
+		obj_dev = static_cast<const T*>(g_loss_stage.obj.p);
+	}
+	T* dst_dev = dst_space == CATTLE_HIP_HOST ? static_cast<T*>(g_loss_stage.dst.ensure(dst_bytes)) : static_cast<T*>(dst);
+	if (grad_pass)
+		loss_d_function<T>(kind, (int) batch, (int) time_steps, (int) sample_size, (T) epsilon, (T) scale, out_dev, obj_dev,
+				dst_dev);
+	else
+		loss_function<T>(kind, (int) batch, (int) time_steps, (int) sample_size, (T) epsilon, out_dev, obj_dev, dst_dev);
+	if (dst_space == CATTLE_HIP_HOST)
+		copy_out(dst, CATTLE_HIP_HOST, dst_dev, dst_bytes);
+}
+
+void loss_entry(bool grad_pass, int dtype, int kind, const void* out, int out_space, const void* obj, int obj_space,
+		size_t batch, size_t time_steps, size_t sample_size, double epsilon, double scale, void* dst, int dst_space) {
+	check_dtype(dtype);
+	check_space(out_space);
+	check_space(obj_space);
+	check_space(dst_space);
+	CATTLE_HIP_REQUIRE(kind == CATTLE_HIP_LOSS_SQUARED || kind == CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY, "unknown loss kind");
+	CATTLE_HIP_REQUIRE(out != nullptr && obj != nullptr && dst != nullptr, "null tensor buffer");
+	CATTLE_HIP_REQUIRE(batch > 0 && time_steps > 0 && sample_size > 0, "batch, time steps and sample size must be positive");
+	if (dtype == CATTLE_HIP_F32)
+		run_loss<float>(grad_pass, kind, out, out_space, obj, obj_space, batch, time_steps, sample_size, epsilon, scale, dst,
+				dst_space);
+	else
+		run_loss<double>(grad_pass, kind, out, out_space, obj, obj_space, batch, time_steps, sample_size, epsilon, scale, dst,
+				dst_space);
+}
+
+Param& optimizable_param(cattle_hip_layer_t layer, size_t index) {
+	Param& p = param_at(as_layer(layer), index);
+	CATTLE_HIP_REQUIRE(p.optimizable, "the parameters are not optimizable");
+	return p;
+}
+
 
 } /* namespace */
 
@@ -828,6 +886,71 @@ int cattle_hip_layer_reset_param_grad(cattle_hip_layer_t layer, size_t index) {
 	return guarded([&] {
 		Param& p = param_at(as_layer(layer), index);
 		fill_zero(p.grad.p, p.bytes());
+	});
+}
+
+int cattle_hip_loss_function(cattle_hip_dtype dtype, cattle_hip_loss kind, const void* out, cattle_hip_memspace out_space,
+		const void* obj, cattle_hip_memspace obj_space, size_t batch, size_t time_steps, size_t sample_size,
+		double epsilon, void* losses, cattle_hip_memspace losses_space) {
+	return guarded([&] {
+		loss_entry(false, dtype, kind, out, out_space, obj, obj_space, batch, time_steps, sample_size, epsilon, 1.0, losses,
+				losses_space);
+	});
+}
+
+int cattle_hip_loss_d_function(cattle_hip_dtype dtype, cattle_hip_loss kind, const void* out, cattle_hip_memspace out_space,
+		const void* obj, cattle_hip_memspace obj_space, size_t batch, size_t time_steps, size_t sample_size,
+		double epsilon, double scale, void* grad, cattle_hip_memspace grad_space) {
+	return guarded([&] {
+		loss_entry(true, dtype, kind, out, out_space, obj, obj_space, batch, time_steps, sample_size, epsilon, scale, grad,
+				grad_space);
+	});
+}
+
+int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate) {
+	return guarded([&] {
+		Param& p = optimizable_param(layer, index);
+		CATTLE_HIP_REQUIRE(learning_rate > 0, "learning rate must be positive");
+		const size_t n = p.rows * p.cols;
+		if (p.esize == sizeof(float))
+			sgd_update<float>(n, (float) learning_rate, static_cast<const float*>(p.grad.p), static_cast<float*>(p.values.p));
+		else
+			sgd_update<double>(n, learning_rate, static_cast<const double*>(p.grad.p), static_cast<double*>(p.values.p));
+		++p.version;
+	});
+}
+
+int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, double learning_rate, double l1_decay,
+		double l2_decay, double epsilon, size_t timestep) {
+	return guarded([&] {
+		Param& p = optimizable_param(layer, index);
+		CATTLE_HIP_REQUIRE(learning_rate > 0, "learning rate must be positive");
+		CATTLE_HIP_REQUIRE(l1_decay >= 0 && l1_decay <= 1 && l2_decay >= 0 && l2_decay <= 1, "decay rates must lie in [0,1]");
+		CATTLE_HIP_REQUIRE(epsilon > 0, "epsilon must be positive");
+		if (!p.moments_ready) {
+			for (int i = 0; i < 2; ++i)
+				fill_zero(p.moments[i].ensure(p.bytes()), p.bytes());
+			p.moments_ready = true;
+		}
+		const size_t n = p.rows * p.cols;
+		if (p.esize == sizeof(float))
+			adam_update<float>(n, (float) learning_rate, (float) l1_decay, (float) l2_decay, (float) epsilon, timestep,
+					static_cast<const float*>(p.grad.p), static_cast<float*>(p.moments[0].p),
+					static_cast<float*>(p.moments[1].p), static_cast<float*>(p.values.p));
+		else
+			adam_update<double>(n, learning_rate, l1_decay, l2_decay, epsilon, timestep, static_cast<const double*>(p.grad.p),
+					static_cast<double*>(p.moments[0].p), static_cast<double*>(p.moments[1].p),
+					static_cast<double*>(p.values.p));
+		++p.version;
+	});
+}
+
+int cattle_hip_layer_param_reset_optimizer_state(cattle_hip_layer_t layer, size_t index) {
+	return guarded([&] {
+		Param& p = param_at(as_layer(layer), index);
+		if (p.moments_ready)
+			for (int i = 0; i < 2; ++i)
+				fill_zero(p.moments[i].p, p.bytes());
 	});
 }
 

@@ -177,6 +177,41 @@ int cattle_hip_layer_reset_param_grad(cattle_hip_layer_t layer, size_t index);
  * w_in_window*receptor_height + h_in_window. Valid after a forward call. */
 int cattle_hip_maxpool_indices(cattle_hip_layer_t layer, unsigned* indices, cattle_hip_memspace space);
 
+/* ---- Device-resident training step: losses and optimizer updates ------------------------------
+ * With these a whole step (propagate, loss, backpropagate, update, reset) runs on buffers that
+ * never leave HBM; only the per-sample losses come back if the caller asks for them. */
+
+typedef enum cattle_hip_loss {
+	CATTLE_HIP_LOSS_SQUARED = 0,                 /* loss/SquaredLoss.hpp:25-34 */
+	CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY = 1    /* loss/SoftmaxCrossEntropyLoss.hpp:33-50 */
+} cattle_hip_loss;
+
+/* Loss::function (loss/UniversalLoss.hpp:37-41 non-sequential, :99-110 sequential): `losses`
+ * receives one value per sample, summed over the time steps. `out` and `obj` are
+ * (batch, time_steps, sample_size) column-major; pass time_steps = 1 for non-sequential data.
+ * `epsilon` is SoftmaxCrossEntropyLoss's constructor argument (ignored by the squared loss). */
+int cattle_hip_loss_function(cattle_hip_dtype dtype, cattle_hip_loss kind, const void* out, cattle_hip_memspace out_space,
+		const void* obj, cattle_hip_memspace obj_space, size_t batch, size_t time_steps, size_t sample_size,
+		double epsilon, void* losses, cattle_hip_memspace losses_space);
+/* Loss::d_function (loss/UniversalLoss.hpp:42-46, :111-125) times `scale`; scale = 1 / batch_size
+ * is the division SGDOptimizer::_train applies before backpropagating (optimizer/SGDOptimizer.hpp:54-55).
+ * `grad` has the shape of `out` and may alias it. */
+int cattle_hip_loss_d_function(cattle_hip_dtype dtype, cattle_hip_loss kind, const void* out, cattle_hip_memspace out_space,
+		const void* obj, cattle_hip_memspace obj_space, size_t batch, size_t time_steps, size_t sample_size,
+		double epsilon, double scale, void* grad, cattle_hip_memspace grad_space);
+
+/* VanillaSGDOptimizer::_update_params for one Parameters object (optimizer/VanillaSGDOptimizer.hpp:38-43):
+ * values -= grad * learning_rate, in place on the device. Non-optimizable parameters are rejected. */
+int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate);
+/* AdamOptimizer::_update_params for one Parameters object (optimizer/AdamOptimizer.hpp:66-82) with
+ * the reference's bias corrections 1 / (1 - (1 - decay)^(timestep + 1) + epsilon) and epsilon inside
+ * the square root. The two moving averages live with the parameter on the device (shared between
+ * layers that share the parameter) and start at zero. */
+int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, double learning_rate, double l1_decay,
+		double l2_decay, double epsilon, size_t timestep);
+/* AdamOptimizer::_fit (optimizer/AdamOptimizer.hpp:55-65): zero the moving averages. */
+int cattle_hip_layer_param_reset_optimizer_state(cattle_hip_layer_t layer, size_t index);
+
 #ifdef __cplusplus
 }
 #endif

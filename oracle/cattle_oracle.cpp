@@ -18,6 +18,10 @@
  *   batch norm          pinned: closed-form invariants + torch float64 batch_norm.
  *   activations         pinned: libm/numpy closed forms and derivative-at-zero conventions.
  *   max/mean pool       pinned: brute force incl. crafted ties, NaN/-inf windows, overlaps.
+ *   losses              pinned: torch float64 cross_entropy / mse (epsilon 0), numpy closed forms with
+ *                       the epsilon, central differences of the loss against its gradient.
+ *   SGD / Adam updates  pinned: numpy restatement in float64, first-step closed form, and torch's Adam
+ *                       in the limit where the two formulas coincide.
  * What stays unpinned is only the bit pattern of Eigen's own summation order and of its
  * vectorised exp/tanh/log, which the reference's tests do not pin either (they hold no golden
  * vectors: test/gradient_test.cpp, test/training_test.cpp).
@@ -607,6 +611,93 @@ int meanpool_backward(PoolGeom g, const T* out_grad, T* in_grad) {
 	return 0;
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * Losses (loss/SquaredLoss.hpp:25-34, loss/SoftmaxCrossEntropyLoss.hpp:33-50) under the
+ * UniversalLoss drivers (loss/UniversalLoss.hpp:37-46 non-sequential; :99-125 sequential: every time
+ * step is sliced out and treated as its own rows x cols matrix, losses add up over the steps).
+ * A batch is (N, T, V) column-major; T = 1 is the non-sequential case.
+ * ------------------------------------------------------------------------------------------- */
+template<typename T>
+int loss_function(int kind, i64 N, i64 Ts, i64 V, T eps, const T* out, const T* obj, T* losses) {
+	std::vector<T> e((size_t) V);
+	for (i64 n = 0; n < N; ++n)
+		losses[n] = 0;
+	for (i64 t = 0; t < Ts; ++t)
+		for (i64 n = 0; n < N; ++n) {
+			const T* o = out + n + N * t;
+			const T* y = obj + n + N * t;
+			const i64 cs = N * Ts;
+			T l = 0;
+			if (kind == 0) {
+				for (i64 j = 0; j < V; ++j)
+					l += (o[cs * j] - y[cs * j]) * (o[cs * j] - y[cs * j]);
+			} else {
+				T mx = o[0];
+				for (i64 j = 1; j < V; ++j)
+					mx = std::max(mx, o[cs * j]);
+				T sum = 0;
+				for (i64 j = 0; j < V; ++j) {
+					e[j] = std::exp(o[cs * j] - mx);
+					sum += e[j];
+				}
+				for (i64 j = 0; j < V; ++j)
+					l += std::log(e[j] / (sum + eps)) * y[cs * j];
+				l = -l;
+			}
+			losses[n] += l;
+		}
+	return 0;
+}
+
+/* grad = scale * d_function; scale = 1 / batch_size is SGDOptimizer::_train's division
+ * (optimizer/SGDOptimizer.hpp:54-55). */
+template<typename T>
+int loss_d_function(int kind, i64 N, i64 Ts, i64 V, T eps, T scale, const T* out, const T* obj, T* grad) {
+	std::vector<T> e((size_t) V);
+	const i64 cs = N * Ts;
+	for (i64 t = 0; t < Ts; ++t)
+		for (i64 n = 0; n < N; ++n) {
+			const i64 base = n + N * t;
+			if (kind == 0) {
+				for (i64 j = 0; j < V; ++j)
+					grad[base + cs * j] = scale * (2 * (out[base + cs * j] - obj[base + cs * j]));
+			} else {
+				T mx = out[base];
+				for (i64 j = 1; j < V; ++j)
+					mx = std::max(mx, out[base + cs * j]);
+				T sum = 0;
+				for (i64 j = 0; j < V; ++j) {
+					e[j] = std::exp(out[base + cs * j] - mx);
+					sum += e[j];
+				}
+				for (i64 j = 0; j < V; ++j)
+					grad[base + cs * j] = scale * (e[j] / (sum + eps) - obj[base + cs * j]);
+			}
+		}
+	return 0;
+}
+
+/* optimizer/VanillaSGDOptimizer.hpp:38-43 */
+template<typename T>
+int sgd_update(i64 n, T lr, const T* grad, T* values) {
+	for (i64 i = 0; i < n; ++i)
+		values[i] = values[i] - grad[i] * lr;
+	return 0;
+}
+
+/* optimizer/AdamOptimizer.hpp:66-82 (bias corrections carry the epsilon; epsilon sits inside the root) */
+template<typename T>
+int adam_update(i64 n, T lr, T d1, T d2, T eps, i64 timestep, const T* grad, T* m, T* v, T* values) {
+	const T l1_corr = (T) 1 / (1 - std::pow(1 - d1, (T) (timestep + 1)) + eps);
+	const T l2_corr = (T) 1 / (1 - std::pow(1 - d2, (T) (timestep + 1)) + eps);
+	for (i64 i = 0; i < n; ++i) {
+		m[i] = m[i] * (1 - d1) + grad[i] * d1;
+		v[i] = v[i] * (1 - d2) + grad[i] * grad[i] * d2;
+		values[i] = values[i] - (m[i] * (lr * l1_corr)) / std::sqrt(v[i] * l2_corr + eps);
+	}
+	return 0;
+}
+
 } /* namespace */
 
 #define CONV_ARGS i64 N, i64 H, i64 W, i64 C, i64 F, i64 RH, i64 RW, i64 pv, i64 ph, i64 sv, i64 sh, i64 dv, i64 dh
@@ -653,7 +744,15 @@ extern "C" int oracle_maxpool_backward_##SFX(POOL_ARGS, const T* out_grad, const
 extern "C" int oracle_meanpool_forward_##SFX(POOL_ARGS, const T* x, T* out) { \
 	POOL_GEOM; return meanpool_forward<T>(g, x, out); } \
 extern "C" int oracle_meanpool_backward_##SFX(POOL_ARGS, const T* out_grad, T* in_grad) { \
-	POOL_GEOM; return meanpool_backward<T>(g, out_grad, in_grad); }
+	POOL_GEOM; return meanpool_backward<T>(g, out_grad, in_grad); } \
+extern "C" int oracle_loss_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double eps, const T* out, const T* obj, T* losses) { \
+	return loss_function<T>(kind, N, Ts, V, (T) eps, out, obj, losses); } \
+extern "C" int oracle_loss_d_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double eps, double scale, const T* out, \
+		const T* obj, T* grad) { return loss_d_function<T>(kind, N, Ts, V, (T) eps, (T) scale, out, obj, grad); } \
+extern "C" int oracle_sgd_update_##SFX(i64 n, double lr, const T* grad, T* values) { \
+	return sgd_update<T>(n, (T) lr, grad, values); } \
+extern "C" int oracle_adam_update_##SFX(i64 n, double lr, double d1, double d2, double eps, i64 timestep, const T* grad, \
+		T* m, T* v, T* values) { return adam_update<T>(n, (T) lr, (T) d1, (T) d2, (T) eps, timestep, grad, m, v, values); }
 
 ORACLE_INSTANTIATE(float, f32)
 ORACLE_INSTANTIATE(double, f64)

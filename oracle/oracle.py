@@ -291,3 +291,52 @@ def meanpool_backward(x_shape, out_grad, RH=2, RW=2, sv=2, sh=2):
     dx = np.empty((N, H, W, C), dtype=dt, order="F")
     _call("meanpool_backward", dt, *_ll(N, H, W, C, RH, RW, sv, sh), _p(g), _p(dx))
     return dx
+
+
+LOSS_KINDS = {"squared": 0, "softmax_cross_entropy": 1}
+
+
+def _loss_dims(out, sequential):
+    N = out.shape[0]
+    Ts = out.shape[1] if sequential else 1
+    return N, Ts, out.size // (N * Ts)
+
+
+def loss_function(kind, out, obj, eps=1e-5, sequential=False):
+    """Per-sample losses (summed over time steps when sequential: out is then (N, T, ...))."""
+    dt = out.dtype
+    out, obj = _f(out, dt), _f(obj, dt)
+    N, Ts, V = _loss_dims(out, sequential)
+    losses = np.empty((N,), dtype=dt)
+    _call("loss_function", dt, ctypes.c_int(LOSS_KINDS[kind]), *_ll(N, Ts, V), ctypes.c_double(eps), _p(out), _p(obj),
+          _p(losses))
+    return losses
+
+
+def loss_d_function(kind, out, obj, eps=1e-5, scale=1.0, sequential=False):
+    dt = out.dtype
+    out, obj = _f(out, dt), _f(obj, dt)
+    N, Ts, V = _loss_dims(out, sequential)
+    grad = np.empty(out.shape, dtype=dt, order="F")
+    _call("loss_d_function", dt, ctypes.c_int(LOSS_KINDS[kind]), *_ll(N, Ts, V), ctypes.c_double(eps),
+          ctypes.c_double(scale), _p(out), _p(obj), _p(grad))
+    return grad
+
+
+def sgd_update(values, grad, lr=1e-3):
+    """Returns the updated values (the inputs are left alone)."""
+    dt = values.dtype
+    new = np.array(values, dtype=dt, order="F", copy=True)
+    grad = _f(grad, dt)
+    _call("sgd_update", dt, *_ll(new.size), ctypes.c_double(lr), _p(grad), _p(new))
+    return new
+
+
+def adam_update(values, grad, m, v, timestep, lr=1e-3, l1_decay=1e-1, l2_decay=1e-3, eps=1e-5):
+    """Returns (values, m, v) after one step; m and v are the moving averages before it."""
+    dt = values.dtype
+    new, m, v = (np.array(a, dtype=dt, order="F", copy=True) for a in (values, m, v))
+    grad = _f(grad, dt)
+    _call("adam_update", dt, *_ll(new.size), ctypes.c_double(lr), ctypes.c_double(l1_decay), ctypes.c_double(l2_decay),
+          ctypes.c_double(eps), *_ll(timestep), _p(grad), _p(m), _p(v), _p(new))
+    return new, m, v

@@ -1,0 +1,176 @@
+"""GPU parity of the device-resident ends of a training step: loss kernels and optimizer updates,
+called through the C ABI, against the CPU oracle on identical seeded inputs (fp32 1e-4, fp64 1e-10)."""
+import importlib
+
+import numpy as np
+import pytest
+
+import helpers as hp
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+ch = importlib.import_module("c-attl3_amd")
+
+TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-10}
+DTYPES = [np.float32, np.float64]
+KINDS = ["squared", "softmax_cross_entropy"]
+
+
+def _targets(gen, kind, shape, dtype):
+    if kind == "squared":
+        return hp.normal(gen, shape, dtype)
+    # one-hot over the flattened sample (the last axes), as a classifier's labels are
+    N = shape[0]
+    V = int(np.prod(shape[1:]))
+    y = np.zeros((N, V), dtype=dtype, order="F")
+    y[np.arange(N), gen.integers(0, V, N)] = 1
+    return np.asfortranarray(y.reshape(shape, order="F"))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("shape", [(256, 10), (37, 3, 5, 2), (1, 1), (70, 1000), (32, 16, 16, 32)])
+def test_losses(shape, kind, dtype):
+    g = hp.rng(1201)
+    out = hp.normal(g, shape, dtype, 2.0)
+    obj = _targets(g, kind, shape, dtype)
+    o64, y64 = np.asarray(out, np.float64), np.asarray(obj, np.float64)
+    eps = float(dtype(1e-5))
+    tol = TOL[np.dtype(dtype)]
+    # -log p of a probability p known to one ulp carries an absolute error of an ulp of 1 however small the
+    # loss is, so losses below 1 are compared absolutely (the reference's float arithmetic is no better)
+    l_ref = oracle.loss_function(kind, o64, y64, eps=eps)
+    assert np.max(np.abs(ch.loss_function(kind, out, obj) - l_ref) / np.maximum(np.abs(l_ref), 1.0)) < tol
+    scale = 1.0 / shape[0]
+    g_ref = oracle.loss_d_function(kind, o64, y64, eps=eps, scale=float(dtype(scale)))
+    # likewise p - y is a difference of numbers of size <= 1: its error is absolute, of the size of scale * ulp(1)
+    got = ch.loss_d_function(kind, out, obj, scale=scale)
+    floor = scale if kind == "softmax_cross_entropy" else 0.0
+    assert np.max(np.abs(got - g_ref) / np.maximum(np.abs(g_ref), floor + 1e-30)) < tol or hp.rel_err(got, g_ref) < tol
+    # the same through device-resident buffers
+    od, yd = ch.DeviceTensor.from_host(out), ch.DeviceTensor.from_host(obj)
+    assert np.array_equal(ch.loss_function(kind, od, yd), ch.loss_function(kind, out, obj))
+    assert np.array_equal(ch.loss_d_function(kind, od, yd, scale=scale).to_host(), ch.loss_d_function(kind, out, obj, scale=scale))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", KINDS)
+def test_sequential_losses(kind, dtype):
+    g = hp.rng(1202)
+    shape = (33, 5, 4, 3)              # (N, T, 4, 3)
+    out = hp.normal(g, shape, dtype)
+    obj = hp.uniform(g, shape, 0, 1, dtype)
+    o64, y64 = np.asarray(out, np.float64), np.asarray(obj, np.float64)
+    eps = float(dtype(1e-5))
+    tol = TOL[np.dtype(dtype)]
+    assert hp.rel_err(ch.loss_function(kind, out, obj, sequential=True),
+                      oracle.loss_function(kind, o64, y64, eps=eps, sequential=True)) < tol
+    assert hp.rel_err(ch.loss_d_function(kind, out, obj, scale=0.25, sequential=True),
+                      oracle.loss_d_function(kind, o64, y64, eps=eps, scale=0.25, sequential=True)) < tol
+
+
+def test_loss_errors():
+    a = np.zeros((4, 3), np.float32, order="F")
+    with pytest.raises(ValueError):
+        ch.loss_function("squared", a, np.zeros((4, 2), np.float32, order="F"))
+    lib = ch.lib()
+    import ctypes
+    rc = lib.cattle_hip_loss_function(0, 7, ctypes.c_void_p(a.ctypes.data), 0, ctypes.c_void_p(a.ctypes.data), 0,
+                                      ctypes.c_size_t(4), ctypes.c_size_t(1), ctypes.c_size_t(3), ctypes.c_double(1e-5),
+                                      ctypes.c_void_p(a.ctypes.data), 0)
+    assert rc != 0 and b"loss kind" in lib.cattle_hip_last_error()
+
+
+def _dense_with_grads(dtype, seed):
+    g = hp.rng(seed)
+    layer = ch.DenseKernelLayer(dtype, (24,), 17)
+    w = hp.normal(g, (24, 17), dtype, 0.3)
+    b = hp.normal(g, (1, 17), dtype, 0.1)
+    layer.get_params()[0].set_values(w)
+    layer.get_params()[1].set_values(b)
+    return layer, g, w, b
+
+
+def _accumulate(layer, g, dtype):
+    x = hp.normal(g, (9, 24), dtype)
+    go = hp.normal(g, (9, 17), dtype)
+    layer.pass_forward(x, True)
+    layer.pass_back(go)
+    return x
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sgd_update(dtype):
+    layer, g, w, b = _dense_with_grads(dtype, 1210)
+    _accumulate(layer, g, dtype)
+    tol = TOL[np.dtype(dtype)]
+    for prm, old in zip(layer.get_params(), (w, b)):
+        grad = prm.get_grad()
+        prm.sgd_update(0.05)
+        ref = oracle.sgd_update(np.asarray(old, np.float64), np.asarray(grad, np.float64), lr=float(dtype(0.05)))
+        assert hp.rel_err(prm.get_values(), ref) < tol
+        assert np.array_equal(prm.get_grad(), grad)            # the update leaves the gradient alone
+    # the forward pass uses the updated weights (kernel-side weight layouts are rebuilt)
+    x = hp.normal(g, (5, 24), dtype)
+    wn, bn = (np.asarray(p.get_values(), np.float64) for p in layer.get_params())
+    assert hp.rel_err(layer.pass_forward(x, False), oracle.dense_forward(np.asarray(x, np.float64), wn, bn)) < tol
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_adam_updates_over_steps(dtype):
+    layer, g, w, b = _dense_with_grads(dtype, 1211)
+    tol = TOL[np.dtype(dtype)]
+    state = [(np.asarray(v, np.float64), np.zeros(v.shape), np.zeros(v.shape)) for v in (w, b)]
+    hyper = dict(lr=2e-3, l1_decay=0.1, l2_decay=0.01, eps=1e-5)
+    for t in range(4):
+        for prm in layer.get_params():
+            prm.reset_grad()
+        _accumulate(layer, g, dtype)
+        for i, prm in enumerate(layer.get_params()):
+            grad = np.asarray(prm.get_grad(), np.float64)
+            prm.adam_update(t, learning_rate=hyper["lr"], l1_decay=hyper["l1_decay"], l2_decay=hyper["l2_decay"],
+                            epsilon=hyper["eps"])
+            state[i] = oracle.adam_update(state[i][0], grad, state[i][1], state[i][2], t,
+                                          **{k: float(dtype(v)) for k, v in hyper.items()})
+            # teacher-forced: the device continues from its own values, the oracle from the oracle's; compare, then
+            # hand the device values to the oracle so that rounding differences do not compound through 1/sqrt(v)
+            assert hp.rel_err(prm.get_values(), state[i][0]) < tol, (t, i)
+            state[i] = (np.asarray(prm.get_values(), np.float64), state[i][1], state[i][2])
+    # AdamOptimizer::_fit starts the averages again from zero
+    prm = layer.get_params()[0]
+    prm.reset_optimizer_state()
+    before = np.asarray(prm.get_values(), np.float64)
+    grad = np.asarray(prm.get_grad(), np.float64)
+    prm.adam_update(0)
+    ref, _, _ = oracle.adam_update(before, grad, np.zeros_like(before), np.zeros_like(before), 0,
+                                   lr=float(dtype(1e-3)), l1_decay=float(dtype(1e-1)), l2_decay=float(dtype(1e-3)),
+                                   eps=float(dtype(1e-5)))
+    assert hp.rel_err(prm.get_values(), ref) < tol
+
+
+def test_shared_parameters_share_the_update_and_its_state():
+    dtype = np.float32
+    layer, g, w, b = _dense_with_grads(dtype, 1212)
+    twin = layer.clone_with_shared_params()
+    _accumulate(layer, g, dtype)
+    _accumulate(twin, g, dtype)                       # both accumulate into the one gradient
+    layer.get_params()[0].adam_update(0)
+    assert np.array_equal(twin.get_params()[0].get_values(), layer.get_params()[0].get_values())
+    assert not np.array_equal(layer.get_params()[0].get_values(), w)
+    x = hp.normal(g, (3, 24), dtype)
+    assert np.array_equal(twin.pass_forward(x, False), layer.pass_forward(x, False))
+
+
+def test_updates_reject_what_the_reference_skips():
+    bn = ch.BatchNormLayer(np.float32, (4, 4, 3))
+    running_mean = bn.get_params()[0]                  # not optimizable: optimizers skip it (AdamOptimizer.hpp:72-73)
+    with pytest.raises(ch.CattleHipError):
+        running_mean.sgd_update(0.1)
+    with pytest.raises(ch.CattleHipError):
+        running_mean.adam_update(0)
+    gamma = bn.get_params()[2]
+    with pytest.raises(ch.CattleHipError):
+        gamma.sgd_update(0.0)                          # assert(learning_rate > 0)
+    with pytest.raises(ch.CattleHipError):
+        gamma.adam_update(0, l1_decay=1.5)             # assert(l1_decay >= 0 && l1_decay <= 1)

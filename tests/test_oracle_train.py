@@ -1,0 +1,167 @@
+"""Pins the oracle's loss functions and optimizer updates (the two ends of a training step around the
+layer stack) without the reference being compilable: torch float64 as an independent implementation
+where the formulas coincide, closed forms, central differences, and the time-step slicing property
+of the sequential losses. The reference's own tests hold no known answers for these either."""
+import numpy as np
+import pytest
+import torch
+
+import helpers as hp
+from oracle import oracle
+
+TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-10}
+DTYPES = [np.float32, np.float64]
+
+
+def _one_hot(gen, N, V, dtype):
+    y = np.zeros((N, V), dtype=dtype, order="F")
+    y[np.arange(N), gen.integers(0, V, N)] = 1
+    return y
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_softmax_cross_entropy_against_torch(dtype):
+    g = hp.rng(901)
+    N, V = 9, 10
+    out = hp.normal(g, (N, V), dtype, 3.0)
+    obj = _one_hot(g, N, V, dtype)
+    ot = torch.tensor(np.asarray(out, np.float64), requires_grad=True)
+    yt = torch.tensor(np.asarray(obj, np.float64))
+    lt = torch.nn.functional.cross_entropy(ot, yt, reduction="none")
+    lt.sum().backward()
+    # epsilon 0: the reference's formula is then exactly -sum y log softmax, and its gradient
+    # softmax - y is the true derivative because each row of y sums to one
+    assert hp.rel_err(oracle.loss_function("softmax_cross_entropy", out, obj, eps=0.0), lt.detach().numpy()) < TOL[np.dtype(dtype)]
+    assert hp.rel_err(oracle.loss_d_function("softmax_cross_entropy", out, obj, eps=0.0), ot.grad.numpy()) < TOL[np.dtype(dtype)]
+    # the scale multiplies the gradient (the optimizer's division by the batch size)
+    assert hp.rel_err(oracle.loss_d_function("softmax_cross_entropy", out, obj, eps=0.0, scale=1.0 / 128),
+                      ot.grad.numpy() / 128) < TOL[np.dtype(dtype)]
+
+
+def test_softmax_cross_entropy_epsilon_and_soft_targets():
+    """With the epsilon in the denominator and arbitrary targets: p = e / (sum e + eps), L = -sum log(p) y,
+    grad = p - y (not the derivative of L unless the targets sum to one: the reference's choice)."""
+    g = hp.rng(902)
+    N, V, eps = 6, 7, 1e-2          # a large epsilon so that a misplaced one shows
+    out = hp.normal(g, (N, V), np.float64, 2.0)
+    obj = hp.uniform(g, (N, V), 0, 1, np.float64)
+    e = np.exp(out - out.max(axis=1, keepdims=True))
+    p = e / (e.sum(axis=1, keepdims=True) + eps)
+    assert hp.rel_err(oracle.loss_function("softmax_cross_entropy", out, obj, eps=eps), -(np.log(p) * obj).sum(axis=1)) < 1e-12
+    assert hp.rel_err(oracle.loss_d_function("softmax_cross_entropy", out, obj, eps=eps), p - obj) < 1e-12
+    # shifting a row by a constant changes nothing (the max subtraction)
+    shifted = out + np.arange(N).reshape(N, 1) * 10.0
+    assert hp.rel_err(oracle.loss_function("softmax_cross_entropy", shifted, obj, eps=eps),
+                      oracle.loss_function("softmax_cross_entropy", out, obj, eps=eps)) < 1e-12
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_squared_loss_against_torch(dtype):
+    g = hp.rng(903)
+    N, dims = 5, (4, 3, 2)
+    out = hp.normal(g, (N,) + dims, dtype)
+    obj = hp.normal(g, (N,) + dims, dtype)
+    ot = torch.tensor(np.asarray(out, np.float64), requires_grad=True)
+    lt = torch.nn.functional.mse_loss(ot, torch.tensor(np.asarray(obj, np.float64)), reduction="none").reshape(N, -1).sum(dim=1)
+    lt.sum().backward()
+    assert hp.rel_err(oracle.loss_function("squared", out, obj), lt.detach().numpy()) < TOL[np.dtype(dtype)]
+    assert hp.rel_err(oracle.loss_d_function("squared", out, obj), ot.grad.numpy()) < TOL[np.dtype(dtype)]
+
+
+@pytest.mark.parametrize("kind", ["squared", "softmax_cross_entropy"])
+def test_loss_gradient_is_the_derivative(kind):
+    """Central differences of sum(function) against d_function (targets sum to one, tiny epsilon)."""
+    g = hp.rng(904)
+    N, V = 4, 6
+    out = hp.normal(g, (N, V), np.float64)
+    obj = _one_hot(g, N, V, np.float64) if kind != "squared" else hp.normal(g, (N, V), np.float64)
+    grad = oracle.loss_d_function(kind, out, obj, eps=1e-14)
+    h = 1e-6
+    for n in range(N):
+        for j in range(V):
+            up, dn = out.copy(order="F"), out.copy(order="F")
+            up[n, j] += h
+            dn[n, j] -= h
+            num = (oracle.loss_function(kind, up, obj, eps=1e-14).sum() - oracle.loss_function(kind, dn, obj, eps=1e-14).sum()) / (2 * h)
+            assert abs(num - grad[n, j]) < 1e-7
+
+
+@pytest.mark.parametrize("kind", ["squared", "softmax_cross_entropy"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sequential_losses_are_per_time_step(kind, dtype):
+    """loss/UniversalLoss.hpp:99-125: every time step is sliced out and handled as a non-sequential batch;
+    losses add up over the steps, gradients are written back into the step's slice."""
+    g = hp.rng(905)
+    N, Ts, dims = 5, 4, (3, 2)
+    out = hp.normal(g, (N, Ts) + dims, dtype)
+    obj = hp.uniform(g, (N, Ts) + dims, 0, 1, dtype)
+    total = oracle.loss_function(kind, out, obj, sequential=True)
+    grad = oracle.loss_d_function(kind, out, obj, scale=0.5, sequential=True)
+    acc = np.zeros(N)
+    for t in range(Ts):
+        o_t, y_t = np.asfortranarray(out[:, t]), np.asfortranarray(obj[:, t])
+        acc += oracle.loss_function(kind, o_t, y_t)
+        assert hp.rel_err(grad[:, t], oracle.loss_d_function(kind, o_t, y_t, scale=0.5)) < TOL[np.dtype(dtype)]
+    assert hp.rel_err(total, acc) < TOL[np.dtype(dtype)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sgd_update(dtype):
+    g = hp.rng(906)
+    w = hp.normal(g, (7, 5), dtype)
+    dw = hp.normal(g, (7, 5), dtype)
+    new = oracle.sgd_update(w, dw, lr=0.05)
+    assert hp.rel_err(new, np.asarray(w, np.float64) - 0.05 * np.asarray(dw, np.float64)) < TOL[np.dtype(dtype)]
+    assert np.array_equal(oracle.sgd_update(w, np.zeros_like(dw), lr=0.05), w)
+
+
+def test_adam_first_step_is_a_signed_step():
+    """From zero moving averages, step 0, epsilon -> 0: m = d1 g, v = d2 g^2, both corrections undo the
+    decay factors, so the update is lr * g / |g| whatever the decay rates are."""
+    g = hp.rng(907)
+    w = hp.normal(g, (6, 4), np.float64)
+    dw = hp.uniform(g, (6, 4), 0.5, 2.0, np.float64) * np.where(g.random((6, 4)) < 0.5, -1, 1)
+    z = np.zeros_like(w)
+    for d1, d2 in ((0.1, 0.001), (0.3, 0.05)):
+        new, m, v = oracle.adam_update(w, dw, z, z, 0, lr=0.01, l1_decay=d1, l2_decay=d2, eps=1e-30)
+        assert np.max(np.abs(new - (w - 0.01 * np.sign(dw)))) < 1e-12
+        assert hp.rel_err(m, d1 * dw) < 1e-12 and hp.rel_err(v, d2 * dw * dw) < 1e-12
+
+
+def test_adam_matches_torch_in_the_small_epsilon_limit():
+    """torch's Adam divides by sqrt(v_hat) + eps and corrects by 1 - beta^t; the reference divides by
+    sqrt(v_hat + eps) and corrects by 1 - beta^t + eps. For eps -> 0 they are the same recurrence with
+    beta = 1 - decay, so several steps with changing gradients must agree."""
+    g = hp.rng(908)
+    w0 = hp.normal(g, (5, 3), np.float64)
+    grads = [hp.uniform(g, (5, 3), 0.5, 2.0, np.float64) * np.where(g.random((5, 3)) < 0.5, -1, 1) for _ in range(6)]
+    d1, d2, lr = 0.1, 0.01, 0.02
+    pt = torch.tensor(w0.copy(), requires_grad=True)
+    opt = torch.optim.Adam([pt], lr=lr, betas=(1 - d1, 1 - d2), eps=1e-30)
+    w, m, v = w0, np.zeros_like(w0), np.zeros_like(w0)
+    for t, dw in enumerate(grads):
+        pt.grad = torch.tensor(dw.copy())
+        opt.step()
+        w, m, v = oracle.adam_update(w, dw, m, v, t, lr=lr, l1_decay=d1, l2_decay=d2, eps=1e-30)
+        assert np.max(np.abs(w - pt.detach().numpy())) < 1e-12, t
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_adam_reference_formula_with_default_epsilon(dtype):
+    """The reference's exact placement of epsilon (optimizer/AdamOptimizer.hpp:67-81), evaluated
+    independently in vectorised float64 over three steps."""
+    g = hp.rng(909)
+    w = hp.normal(g, (8, 3), dtype)
+    lr, d1, d2, eps = 1e-3, 1e-1, 1e-3, 1e-5
+    w64, m64, v64 = np.asarray(w, np.float64), np.zeros((8, 3)), np.zeros((8, 3))
+    m, v = np.zeros_like(w), np.zeros_like(w)
+    for t in range(3):
+        dw = hp.normal(g, (8, 3), dtype)
+        w, m, v = oracle.adam_update(w, dw, m, v, t, lr, d1, d2, eps)
+        c1 = 1.0 / (1 - (1 - d1) ** (t + 1) + eps)
+        c2 = 1.0 / (1 - (1 - d2) ** (t + 1) + eps)
+        m64 = (1 - d1) * m64 + d1 * dw
+        v64 = (1 - d2) * v64 + d2 * np.square(np.asarray(dw, np.float64))
+        w64 = w64 - lr * c1 * m64 / np.sqrt(c2 * v64 + eps)
+        assert hp.rel_err(w, w64) < TOL[np.dtype(dtype)]
+        assert hp.rel_err(m, m64) < TOL[np.dtype(dtype)] and hp.rel_err(v, v64) < TOL[np.dtype(dtype)]
