@@ -174,3 +174,64 @@ def test_updates_reject_what_the_reference_skips():
         gamma.sgd_update(0.0)                          # assert(learning_rate > 0)
     with pytest.raises(ch.CattleHipError):
         gamma.adam_update(0, l1_decay=1.5)             # assert(l1_decay >= 0 && l1_decay <= 1)
+
+
+def _one_hot_labels(gen, N, shape, dtype):
+    obj = np.zeros((N,) + shape, dtype, order="F")
+    obj.reshape((N, -1), order="F")[np.arange(N), gen.integers(0, int(np.prod(shape)), N)] = 1
+    return obj
+
+
+@pytest.mark.parametrize("config", ["mlp_sgd", "convnet_adam"])
+def test_whole_training_steps_stay_on_the_device(config):
+    """BASELINE configs 2 and 3 as SGDOptimizer::_train runs them (optimizer/SGDOptimizer.hpp:44-70), three steps
+    in a row: once with every tensor, the loss and the update on the device (only the per-sample losses come
+    back), once with the same HIP layers fed host tensors and the loss and optimizer done on the host by the
+    test harness. Both must tell the same story: same losses, same weights."""
+    import harness as hn
+    dt = np.float32
+    gen = hp.rng(0xC0FFEE20)
+    if config == "mlp_sgd":
+        N, in_shape, out_shape, build = 256, (784,), (10,), hn.build_mlp
+        x = np.asfortranarray(gen.uniform(0, 1, (N,) + in_shape).astype(dt))
+    else:
+        N, in_shape, out_shape, build = 128, (32, 32, 3), (10, 1, 1), hn.build_convnet
+        x = np.asfortranarray(gen.standard_normal((N,) + in_shape).astype(dt))
+    obj = _one_hot_labels(gen, N, out_shape, dt)
+    dev, host = build(hn.HipBackend(dt)), build(hn.HipBackend(dt))
+    hn.init_kernel_weights(dev, 20, dt)
+    for pd, ps in zip(dev.params(), host.params()):
+        ps.set_values(pd.get_values())
+    start = [p.get_values() for p in dev.params()]
+    host_adam = hn.Adam(host.params(), lr=1e-3)
+    xd, yd = ch.DeviceTensor.from_host(x), ch.DeviceTensor.from_host(obj)
+    for step in range(3):
+        # device-resident step
+        out = dev.propagate(xd, True)
+        loss_dev = ch.loss_function("softmax_cross_entropy", out, yd)
+        dev.backpropagate(ch.loss_d_function("softmax_cross_entropy", out, yd, scale=1.0 / N))
+        for p in dev.params():
+            if p.are_optimizable():
+                if config == "mlp_sgd":
+                    p.sgd_update(1e-3)
+                else:
+                    p.adam_update(step, learning_rate=1e-3)
+                p.reset_grad()
+        # host-orchestrated step on the twin network
+        out_h = hn.train_step_gradients(host, x, obj, hn.softmax_ce_grad)
+        loss_host = oracle.loss_function("softmax_cross_entropy", np.asarray(out_h, np.float64), np.asarray(obj, np.float64))
+        if config == "mlp_sgd":
+            hn.vanilla_sgd_update(host.params(), 1e-3)
+        else:
+            host_adam.update(host.params(), step)
+        for p in host.params():
+            p.reset_grad()
+        assert hp.rel_err(loss_dev, loss_host) < 1e-3, step
+    for pd, ps, w0 in zip(dev.params(), host.params(), start):
+        moved = np.max(np.abs(np.asarray(ps.get_values(), np.float64) - w0))
+        diff = np.max(np.abs(np.asarray(pd.get_values(), np.float64) - ps.get_values()))
+        # three steps move a weight by up to `moved`; both routes must agree on that movement to 1 % of the
+        # largest step (Adam turns rounding-level gradient differences near zero into sign flips of single
+        # entries, so entrywise relative agreement is not to be had) and on the values to 1e-4
+        assert diff <= 1e-2 * moved + 1e-7, (diff, moved)
+        assert np.allclose(pd.get_values(), ps.get_values(), rtol=1e-4, atol=1e-5)
