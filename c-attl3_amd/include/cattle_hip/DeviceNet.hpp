@@ -1,0 +1,418 @@
+/*
+ * DeviceNet.hpp — header-only C++11 view of libcattle_hip for callers that keep a whole training
+ * step on the MI355X: device tensors chained from layer to layer, parameters that never leave the
+ * device, loss and optimizer update as kernels.
+ *
+ * It plays the part that core/gpu/GPULayer.hpp:31-58, core/gpu/GPUNeuralNetwork.hpp:27-48 and
+ * parameters/gpu/StandardGPUParameters.hpp:50-120 sketch in the reference's unfinished CUDA tree
+ * (device-tensor overloads of pass_forward / pass_back / propagate / backpropagate, device-side
+ * values and gradients), and the training loop is SGDOptimizer::_train's batch body
+ * (optimizer/SGDOptimizer.hpp:44-70). It needs no C-ATTL3 header: only the C ABI.
+ *
+ * Tensors are the reference's column-major buffers with the sample index fastest; dims are
+ * (batch, height, width, channels) the way Dimensions::extend pads lower ranks with ones.
+ */
+#ifndef CATTLE_HIP_DEVICENET_HPP_
+#define CATTLE_HIP_DEVICENET_HPP_
+
+#include <array>
+#include <cassert>
+#include <cstddef>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "cattle_hip.h"
+
+namespace cattle {
+namespace hip {
+namespace device {
+
+inline void check(int status) {
+	if (status != CATTLE_HIP_OK)
+		throw std::runtime_error(std::string("cattle_hip: ") + cattle_hip_last_error());
+}
+
+template<typename Scalar> struct Code;
+template<> struct Code<float> { static constexpr cattle_hip_dtype value = CATTLE_HIP_F32; };
+template<> struct Code<double> { static constexpr cattle_hip_dtype value = CATTLE_HIP_F64; };
+
+/** A tensor in device memory; move-only owner of its buffer (the role of CuDNNTensor in the reference). */
+template<typename Scalar>
+class DeviceTensor {
+public:
+	typedef std::array<std::size_t,4> Dims;
+	inline DeviceTensor() : dims{ { 0, 0, 0, 0 } }, ptr(nullptr) { }
+	inline explicit DeviceTensor(const Dims& dims) : dims(dims), ptr(nullptr) {
+		if (size() > 0)
+			check(cattle_hip_alloc(&ptr, size() * sizeof(Scalar)));
+	}
+	/** Uploads a host buffer of the same layout (an Eigen tensor's data()). */
+	inline DeviceTensor(const Dims& dims, const Scalar* host) : DeviceTensor(dims) {
+		if (size() > 0)
+			check(cattle_hip_upload(ptr, host, size() * sizeof(Scalar)));
+	}
+	inline DeviceTensor(DeviceTensor&& other) : dims(other.dims), ptr(other.ptr) {
+		other.ptr = nullptr;
+		other.dims = Dims{ { 0, 0, 0, 0 } };
+	}
+	inline DeviceTensor& operator=(DeviceTensor&& other) {
+		if (this != &other) {
+			release();
+			dims = other.dims;
+			ptr = other.ptr;
+			other.ptr = nullptr;
+			other.dims = Dims{ { 0, 0, 0, 0 } };
+		}
+		return *this;
+	}
+	DeviceTensor(const DeviceTensor&) = delete;
+	DeviceTensor& operator=(const DeviceTensor&) = delete;
+	inline ~DeviceTensor() {
+		release();
+	}
+	inline std::size_t size() const {
+		return dims[0] * dims[1] * dims[2] * dims[3];
+	}
+	inline std::size_t batch() const {
+		return dims[0];
+	}
+	inline const Dims& dimensions() const {
+		return dims;
+	}
+	/** A null tensor, as pass_back of an input layer returns (core/Layer.hpp:131-137). */
+	inline bool is_null() const {
+		return ptr == nullptr;
+	}
+	inline Scalar* data() {
+		return static_cast<Scalar*>(ptr);
+	}
+	inline const Scalar* data() const {
+		return static_cast<const Scalar*>(ptr);
+	}
+	inline void download(Scalar* host) const {
+		if (size() > 0)
+			check(cattle_hip_download(host, ptr, size() * sizeof(Scalar)));
+	}
+	inline std::vector<Scalar> to_host() const {
+		std::vector<Scalar> out(size());
+		download(out.data());
+		return out;
+	}
+private:
+	inline void release() {
+		if (ptr)
+			cattle_hip_free(ptr);
+		ptr = nullptr;
+	}
+	Dims dims;
+	void* ptr;
+};
+
+/** One layer on the device: owner of a cattle_hip_layer_t, with the Layer contract on DeviceTensors. */
+template<typename Scalar>
+class DeviceLayer {
+public:
+	typedef std::array<std::size_t,3> Dims;
+	/* layer/kernel/ConvKernelLayer.hpp:282-296 */
+	inline static DeviceLayer conv(const Dims& input_dims, std::size_t filters, std::size_t receptor_height = 3,
+			std::size_t receptor_width = 3, std::size_t vertical_padding = 1, std::size_t horizontal_padding = 1,
+			std::size_t vertical_stride = 1, std::size_t horizontal_stride = 1, std::size_t vertical_dilation = 0,
+			std::size_t horizontal_dilation = 0) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_conv_create(Code<Scalar>::value, input_dims[0], input_dims[1], input_dims[2], filters,
+				receptor_height, receptor_width, vertical_padding, horizontal_padding, vertical_stride, horizontal_stride,
+				vertical_dilation, horizontal_dilation, &h));
+		return DeviceLayer(h);
+	}
+	/* layer/kernel/DenseKernelLayer.hpp:61-77 */
+	inline static DeviceLayer dense(const Dims& input_dims, std::size_t output_size) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_dense_create(Code<Scalar>::value, input_dims[0] * input_dims[1] * input_dims[2], output_size, &h));
+		return DeviceLayer(h, input_dims);
+	}
+	/* layer/BatchNormLayer.hpp:66-101 (per channel) / :334-361 (per activation) */
+	inline static DeviceLayer batch_norm(const Dims& dims, bool per_last_rank = true, Scalar norm_avg_decay = .1,
+			Scalar epsilon = 1e-5) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_batchnorm_create(Code<Scalar>::value, dims[0], dims[1], dims[2], per_last_rank ? 1 : 0,
+				(double) norm_avg_decay, (double) epsilon, &h));
+		return DeviceLayer(h);
+	}
+	/* layer/activation/<Name>ActivationLayer.hpp */
+	inline static DeviceLayer activation(cattle_hip_activation kind, const Dims& dims, Scalar param = 0) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_activation_create(Code<Scalar>::value, kind, dims[0] * dims[1] * dims[2], (double) param, &h));
+		return DeviceLayer(h, dims, dims);
+	}
+	/* layer/pool/MaxPoolLayer.hpp:105-108, layer/pool/MeanPoolLayer.hpp:62-65 */
+	inline static DeviceLayer pool(cattle_hip_pool kind, const Dims& input_dims, std::size_t receptor_height = 2,
+			std::size_t receptor_width = 2, std::size_t vertical_stride = 2, std::size_t horizontal_stride = 2) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_pool_create(Code<Scalar>::value, kind, input_dims[0], input_dims[1], input_dims[2], receptor_height,
+				receptor_width, vertical_stride, horizontal_stride, &h));
+		return DeviceLayer(h);
+	}
+	inline DeviceLayer(DeviceLayer&& other) : handle(other.handle), in_dims(other.in_dims), out_dims(other.out_dims),
+			cached_in(std::move(other.cached_in)), cached_out(std::move(other.cached_out)) {
+		other.handle = nullptr;
+	}
+	DeviceLayer(const DeviceLayer&) = delete;
+	DeviceLayer& operator=(const DeviceLayer&) = delete;
+	inline ~DeviceLayer() {
+		if (handle)
+			cattle_hip_layer_destroy(handle);
+	}
+	/* Layer::clone (core/Layer.hpp:47) / clone_with_shared_params (:56) */
+	inline DeviceLayer clone(bool share_params = false) const {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_layer_clone(handle, share_params ? 1 : 0, &h));
+		return DeviceLayer(h, in_dims, out_dims);
+	}
+	inline const Dims& get_input_dims() const {
+		return in_dims;
+	}
+	inline const Dims& get_output_dims() const {
+		return out_dims;
+	}
+	inline bool is_input_layer() const {
+		int flag = 0;
+		check(cattle_hip_layer_is_input_layer(handle, &flag));
+		return flag != 0;
+	}
+	inline void set_input_layer(bool input_layer) {
+		check(cattle_hip_layer_set_input_layer(handle, input_layer ? 1 : 0));
+	}
+	inline void empty_cache() {
+		check(cattle_hip_layer_empty_cache(handle));
+		cached_in = DeviceTensor<Scalar>();
+		cached_out = DeviceTensor<Scalar>();
+	}
+	/**
+	 * Layer::pass_forward on device tensors. The layer borrows its input (and, for layers whose backward
+	 * pass reads the output, its output) until pass_back, so the input is taken by value and kept here, and
+	 * the returned reference stays valid until the next pass_forward or empty_cache of this layer.
+	 */
+	inline const DeviceTensor<Scalar>& pass_forward(DeviceTensor<Scalar> in, bool training) {
+		assert(in.dimensions()[1] * in.dimensions()[2] * in.dimensions()[3] == in_dims[0] * in_dims[1] * in_dims[2]);
+		const std::size_t batch = in.batch();
+		DeviceTensor<Scalar> out(typename DeviceTensor<Scalar>::Dims{ { batch, out_dims[0], out_dims[1], out_dims[2] } });
+		check(cattle_hip_layer_forward(handle, in.data(), CATTLE_HIP_DEVICE, batch, training ? 1 : 0, out.data(),
+				CATTLE_HIP_DEVICE));
+		cached_in = std::move(in);
+		cached_out = std::move(out);
+		return cached_out;
+	}
+	/** Same, for an input the caller keeps alive and unmodified until pass_back (e.g. the training batch). */
+	inline const DeviceTensor<Scalar>& pass_forward_borrowed(const DeviceTensor<Scalar>& in, bool training) {
+		const std::size_t batch = in.batch();
+		DeviceTensor<Scalar> out(typename DeviceTensor<Scalar>::Dims{ { batch, out_dims[0], out_dims[1], out_dims[2] } });
+		check(cattle_hip_layer_forward(handle, in.data(), CATTLE_HIP_DEVICE, batch, training ? 1 : 0, out.data(),
+				CATTLE_HIP_DEVICE));
+		cached_in = DeviceTensor<Scalar>();
+		cached_out = std::move(out);
+		return cached_out;
+	}
+	/** Layer::pass_back: returns the input gradient, a null tensor for an input layer. */
+	inline DeviceTensor<Scalar> pass_back(const DeviceTensor<Scalar>& out_grad, bool needs_input_grad = true) {
+		const std::size_t batch = out_grad.batch();
+		DeviceTensor<Scalar> prev;
+		if (needs_input_grad)
+			prev = DeviceTensor<Scalar>(typename DeviceTensor<Scalar>::Dims{ { batch, in_dims[0], in_dims[1], in_dims[2] } });
+		check(cattle_hip_layer_backward(handle, out_grad.data(), CATTLE_HIP_DEVICE, batch,
+				needs_input_grad ? prev.data() : nullptr, CATTLE_HIP_DEVICE));
+		return prev;
+	}
+	/* ---- parameters (core/Parameters.hpp:15-95), resident on the device ---- */
+	inline std::size_t num_params() const {
+		std::size_t n = 0;
+		check(cattle_hip_layer_num_params(handle, &n));
+		return n;
+	}
+	inline void param_shape(std::size_t index, std::size_t& rows, std::size_t& cols, bool& optimizable) const {
+		int opt = 0;
+		check(cattle_hip_layer_param_shape(handle, index, &rows, &cols, &opt));
+		optimizable = opt != 0;
+	}
+	inline void set_param_values(std::size_t index, const Scalar* host_values) {
+		check(cattle_hip_layer_set_param_values(handle, index, host_values, CATTLE_HIP_HOST));
+	}
+	inline std::vector<Scalar> get_param_values(std::size_t index) const {
+		return fetch(index, &cattle_hip_layer_get_param_values);
+	}
+	inline std::vector<Scalar> get_param_grad(std::size_t index) const {
+		return fetch(index, &cattle_hip_layer_get_param_grad);
+	}
+	/** reset_grad of every parameter (optimizer/SGDOptimizer.hpp:68-70). */
+	inline void reset_grads() {
+		const std::size_t n = num_params();
+		for (std::size_t i = 0; i < n; ++i)
+			check(cattle_hip_layer_reset_param_grad(handle, i));
+	}
+	/** VanillaSGDOptimizer::_update_params over this layer's optimizable parameters. */
+	inline void sgd_update(Scalar learning_rate) {
+		for_each_optimizable([&](std::size_t i) {
+			check(cattle_hip_layer_param_sgd_update(handle, i, (double) learning_rate));
+		});
+	}
+	/** AdamOptimizer::_update_params over this layer's optimizable parameters (defaults of AdamOptimizer.hpp:40-42). */
+	inline void adam_update(std::size_t timestep, Scalar learning_rate = 1e-3, Scalar l1_decay = 1e-1,
+			Scalar l2_decay = 1e-3, Scalar epsilon = 1e-5) {
+		for_each_optimizable([&](std::size_t i) {
+			check(cattle_hip_layer_param_adam_update(handle, i, (double) learning_rate, (double) l1_decay, (double) l2_decay,
+					(double) epsilon, timestep));
+		});
+	}
+	/** AdamOptimizer::_fit. */
+	inline void reset_optimizer_state() {
+		const std::size_t n = num_params();
+		for (std::size_t i = 0; i < n; ++i)
+			check(cattle_hip_layer_param_reset_optimizer_state(handle, i));
+	}
+	inline cattle_hip_layer_t get() const {
+		return handle;
+	}
+private:
+	inline explicit DeviceLayer(cattle_hip_layer_t handle) : handle(handle) {
+		std::size_t d[3];
+		check(cattle_hip_layer_input_dims(handle, d));
+		in_dims = Dims{ { d[0], d[1], d[2] } };
+		check(cattle_hip_layer_output_dims(handle, d));
+		out_dims = Dims{ { d[0], d[1], d[2] } };
+	}
+	/* dense and activation layers are created from a volume: keep the caller's shape for the tensors */
+	inline DeviceLayer(cattle_hip_layer_t handle, const Dims& in) : DeviceLayer(handle) {
+		in_dims = in;
+	}
+	inline DeviceLayer(cattle_hip_layer_t handle, const Dims& in, const Dims& out) : handle(handle), in_dims(in),
+			out_dims(out) { }
+	template<typename Fn>
+	inline void for_each_optimizable(Fn fn) {
+		const std::size_t n = num_params();
+		for (std::size_t i = 0; i < n; ++i) {
+			std::size_t rows, cols;
+			bool optimizable;
+			param_shape(i, rows, cols, optimizable);
+			if (optimizable)
+				fn(i);
+		}
+	}
+	inline std::vector<Scalar> fetch(std::size_t index, int (*getter)(cattle_hip_layer_t, size_t, void*, cattle_hip_memspace)) const {
+		std::size_t rows, cols;
+		bool optimizable;
+		param_shape(index, rows, cols, optimizable);
+		std::vector<Scalar> out(rows * cols);
+		check(getter(handle, index, out.data(), CATTLE_HIP_HOST));
+		return out;
+	}
+	cattle_hip_layer_t handle;
+	Dims in_dims, out_dims;
+	DeviceTensor<Scalar> cached_in, cached_out;
+};
+
+/** Loss::function / d_function on device tensors (loss/UniversalLoss.hpp:27-55, non-sequential data). */
+template<typename Scalar>
+class DeviceLoss {
+public:
+	inline explicit DeviceLoss(cattle_hip_loss kind, Scalar epsilon = 1e-5) : kind(kind), epsilon(epsilon) { }
+	/** The per-sample losses, on the host (a column vector in the reference). */
+	inline std::vector<Scalar> function(const DeviceTensor<Scalar>& out, const DeviceTensor<Scalar>& obj) const {
+		assert(out.dimensions() == obj.dimensions());
+		std::vector<Scalar> losses(out.batch());
+		check(cattle_hip_loss_function(Code<Scalar>::value, kind, out.data(), CATTLE_HIP_DEVICE, obj.data(),
+				CATTLE_HIP_DEVICE, out.batch(), 1, out.size() / out.batch(), (double) epsilon, losses.data(),
+				CATTLE_HIP_HOST));
+		return losses;
+	}
+	/** scale * d_function; scale = 1 / batch_size is the optimizer's division (optimizer/SGDOptimizer.hpp:54-55). */
+	inline DeviceTensor<Scalar> d_function(const DeviceTensor<Scalar>& out, const DeviceTensor<Scalar>& obj,
+			Scalar scale = 1) const {
+		assert(out.dimensions() == obj.dimensions());
+		DeviceTensor<Scalar> grad(out.dimensions());
+		check(cattle_hip_loss_d_function(Code<Scalar>::value, kind, out.data(), CATTLE_HIP_DEVICE, obj.data(),
+				CATTLE_HIP_DEVICE, out.batch(), 1, out.size() / out.batch(), (double) epsilon, (double) scale, grad.data(),
+				CATTLE_HIP_DEVICE));
+		return grad;
+	}
+private:
+	cattle_hip_loss kind;
+	Scalar epsilon;
+};
+
+/**
+ * A stack of device layers (neural_network/FeedforwardNeuralNetwork.hpp:38-53, :112-127 on device
+ * tensors): layer 0 is the input layer when the network is foremost.
+ */
+template<typename Scalar>
+class DeviceFeedforwardNetwork {
+public:
+	inline explicit DeviceFeedforwardNetwork(std::vector<DeviceLayer<Scalar>> layers, bool foremost = true) :
+			layers(std::move(layers)),
+			foremost(foremost) {
+		assert(!this->layers.empty());
+		this->layers[0].set_input_layer(foremost);
+	}
+	inline std::vector<DeviceLayer<Scalar>>& get_layers() {
+		return layers;
+	}
+	/** propagate: `input` must stay alive and unmodified until backpropagate returns. */
+	inline const DeviceTensor<Scalar>& propagate(const DeviceTensor<Scalar>& input, bool training) {
+		const DeviceTensor<Scalar>* cur = &layers[0].pass_forward_borrowed(input, training);
+		for (std::size_t i = 1; i < layers.size(); ++i)
+			cur = &layers[i].pass_forward_borrowed(*cur, training);      /* the producer keeps its output alive */
+		return *cur;
+	}
+	inline DeviceTensor<Scalar> backpropagate(const DeviceTensor<Scalar>& out_grad) {
+		DeviceTensor<Scalar> grad;
+		for (std::size_t i = layers.size(); i-- > 0;) {
+			const bool needs = !(i == 0 && foremost);
+			grad = layers[i].pass_back(i + 1 == layers.size() ? out_grad : grad, needs);
+		}
+		return grad;
+	}
+	/**
+	 * One batch of SGDOptimizer::_train (optimizer/SGDOptimizer.hpp:44-70) with the vanilla SGD or the
+	 * Adam update: propagate, loss, gradient / batch size, backpropagate, update, reset. Returns the
+	 * sum of the per-sample losses of the batch.
+	 */
+	inline Scalar train_batch_sgd(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,
+			const DeviceLoss<Scalar>& loss, Scalar learning_rate) {
+		const Scalar total = forward_backward(input, obj, loss);
+		for (std::size_t i = 0; i < layers.size(); ++i) {
+			layers[i].sgd_update(learning_rate);
+			layers[i].reset_grads();
+		}
+		return total;
+	}
+	inline Scalar train_batch_adam(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,
+			const DeviceLoss<Scalar>& loss, std::size_t timestep, Scalar learning_rate = 1e-3, Scalar l1_decay = 1e-1,
+			Scalar l2_decay = 1e-3, Scalar epsilon = 1e-5) {
+		const Scalar total = forward_backward(input, obj, loss);
+		for (std::size_t i = 0; i < layers.size(); ++i) {
+			layers[i].adam_update(timestep, learning_rate, l1_decay, l2_decay, epsilon);
+			layers[i].reset_grads();
+		}
+		return total;
+	}
+private:
+	inline Scalar forward_backward(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,
+			const DeviceLoss<Scalar>& loss) {
+		const DeviceTensor<Scalar>& out = propagate(input, true);
+		const std::vector<Scalar> losses = loss.function(out, obj);
+		Scalar total = 0;
+		for (std::size_t i = 0; i < losses.size(); ++i)
+			total += losses[i];
+		backpropagate(loss.d_function(out, obj, (Scalar) 1 / (Scalar) input.batch()));
+		return total;
+	}
+	std::vector<DeviceLayer<Scalar>> layers;
+	bool foremost;
+};
+
+} /* namespace device */
+} /* namespace hip */
+} /* namespace cattle */
+
+#endif /* CATTLE_HIP_DEVICENET_HPP_ */

@@ -1,0 +1,170 @@
+/*
+ * device_net_test.cpp — drives cattle_hip/DeviceNet.hpp (device tensors chained between layers, loss and
+ * optimizer update on the device) through three training batches of two small networks and records the
+ * inputs, the initial parameters, the batch losses and the final parameters to a file that
+ * tests/test_gpu_device_net.py replays on the CPU oracle.
+ *
+ *   mlp:     dense 20 -> 16, ReLU, dense 16 -> 6, softmax cross-entropy, vanilla SGD
+ *   convnet: conv 8x8x3 -> 8 filters 3x3 p1, ReLU, max pool 2x2, batch norm, dense -> 5, softmax
+ *            cross-entropy, Adam
+ */
+#include "cattle_hip/DeviceNet.hpp"
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+using namespace cattle::hip::device;
+
+static FILE* g_out = nullptr;
+
+static void record(const std::string& name, std::size_t scalar_size, const std::vector<std::size_t>& dims, const void* data) {
+	std::uint32_t len = (std::uint32_t) name.size(), ss = (std::uint32_t) scalar_size, rank = (std::uint32_t) dims.size();
+	std::fwrite(&len, 4, 1, g_out);
+	std::fwrite(name.data(), 1, len, g_out);
+	std::fwrite(&ss, 4, 1, g_out);
+	std::fwrite(&rank, 4, 1, g_out);
+	std::size_t count = 1;
+	for (std::size_t d : dims) {
+		std::uint64_t v = d;
+		std::fwrite(&v, 8, 1, g_out);
+		count *= d;
+	}
+	std::fwrite(data, scalar_size, count, g_out);
+}
+
+/* deterministic inputs: a 64-bit LCG mapped to [-1, 1) */
+struct Lcg {
+	std::uint64_t s;
+	explicit Lcg(std::uint64_t seed) : s(seed * 2862933555777941757ULL + 3037000493ULL) { }
+	double next() {
+		s = s * 6364136223846793005ULL + 1442695040888963407ULL;
+		return (double) (s >> 11) / 9007199254740992.0 * 2.0 - 1.0;
+	}
+};
+
+template<typename Scalar>
+static std::vector<Scalar> random_values(std::size_t count, Lcg& g, double scale) {
+	std::vector<Scalar> v(count);
+	for (std::size_t i = 0; i < count; ++i)
+		v[i] = (Scalar) (g.next() * scale);
+	return v;
+}
+
+template<typename Scalar>
+static void init_and_record(const std::string& tag, DeviceFeedforwardNetwork<Scalar>& net, Lcg& g) {
+	std::vector<DeviceLayer<Scalar>>& layers = net.get_layers();
+	for (std::size_t l = 0; l < layers.size(); ++l)
+		for (std::size_t p = 0; p < layers[l].num_params(); ++p) {
+			std::size_t rows, cols;
+			bool opt;
+			layers[l].param_shape(p, rows, cols, opt);
+			if (opt && rows > 1) {      /* weight matrices; biases, gamma, beta keep their initial values */
+				std::vector<Scalar> w = random_values<Scalar>(rows * cols, g, std::sqrt(6.0 / (double) rows));
+				layers[l].set_param_values(p, w.data());
+			}
+			record(tag + ".init." + std::to_string(l) + "." + std::to_string(p), sizeof(Scalar), { rows, cols },
+					layers[l].get_param_values(p).data());
+		}
+}
+
+template<typename Scalar>
+static void record_final(const std::string& tag, DeviceFeedforwardNetwork<Scalar>& net) {
+	std::vector<DeviceLayer<Scalar>>& layers = net.get_layers();
+	for (std::size_t l = 0; l < layers.size(); ++l)
+		for (std::size_t p = 0; p < layers[l].num_params(); ++p) {
+			std::size_t rows, cols;
+			bool opt;
+			layers[l].param_shape(p, rows, cols, opt);
+			record(tag + ".final." + std::to_string(l) + "." + std::to_string(p), sizeof(Scalar), { rows, cols },
+					layers[l].get_param_values(p).data());
+			/* every step ends with reset_grad (optimizer/SGDOptimizer.hpp:68-70) */
+			std::vector<Scalar> grad = layers[l].get_param_grad(p);
+			for (Scalar v : grad)
+				if (v != 0)
+					throw std::runtime_error("gradient not reset after the step");
+		}
+}
+
+template<typename Scalar>
+static std::vector<Scalar> one_hot(std::size_t batch, std::size_t classes, Lcg& g) {
+	std::vector<Scalar> y(batch * classes, (Scalar) 0);
+	for (std::size_t n = 0; n < batch; ++n) {
+		std::size_t c = (std::size_t) ((g.next() + 1.0) / 2.0 * (double) classes);
+		y[n + batch * (c < classes ? c : classes - 1)] = 1;
+	}
+	return y;
+}
+
+template<typename Scalar>
+static void run(const std::string& tag) {
+	typedef DeviceTensor<Scalar> DT;
+	typedef DeviceLayer<Scalar> DL;
+	typedef typename DL::Dims Dims;
+	const std::size_t steps = 3;
+	DeviceLoss<Scalar> loss(CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY);
+	{
+		Lcg g(11);
+		const std::size_t batch = 24;
+		std::vector<DL> layers;
+		layers.push_back(DL::dense(Dims{ { 20, 1, 1 } }, 16));
+		layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+		layers.push_back(DL::dense(layers.back().get_output_dims(), 6));
+		DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
+		init_and_record<Scalar>(tag + ".mlp", net, g);
+		std::vector<Scalar> x = random_values<Scalar>(batch * 20, g, 1.0), y = one_hot<Scalar>(batch, 6, g);
+		record(tag + ".mlp.x", sizeof(Scalar), { batch, 20 }, x.data());
+		record(tag + ".mlp.y", sizeof(Scalar), { batch, 6 }, y.data());
+		DT xd(typename DT::Dims{ { batch, 20, 1, 1 } }, x.data()), yd(typename DT::Dims{ { batch, 6, 1, 1 } }, y.data());
+		std::vector<Scalar> totals;
+		for (std::size_t t = 0; t < steps; ++t)
+			totals.push_back(net.train_batch_sgd(xd, yd, loss, (Scalar) 0.05));
+		record(tag + ".mlp.losses", sizeof(Scalar), { steps }, totals.data());
+		record_final<Scalar>(tag + ".mlp", net);
+	}
+	{
+		Lcg g(12);
+		const std::size_t batch = 16;
+		std::vector<DL> layers;
+		layers.push_back(DL::conv(Dims{ { 8, 8, 3 } }, 8));
+		layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+		layers.push_back(DL::pool(CATTLE_HIP_POOL_MAX, layers.back().get_output_dims()));
+		layers.push_back(DL::batch_norm(layers.back().get_output_dims()));
+		layers.push_back(DL::dense(layers.back().get_output_dims(), 5));
+		DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
+		init_and_record<Scalar>(tag + ".convnet", net, g);
+		std::vector<Scalar> x = random_values<Scalar>(batch * 8 * 8 * 3, g, 1.0), y = one_hot<Scalar>(batch, 5, g);
+		record(tag + ".convnet.x", sizeof(Scalar), { batch, 8, 8, 3 }, x.data());
+		record(tag + ".convnet.y", sizeof(Scalar), { batch, 5 }, y.data());
+		DT xd(typename DT::Dims{ { batch, 8, 8, 3 } }, x.data()), yd(typename DT::Dims{ { batch, 5, 1, 1 } }, y.data());
+		std::vector<Scalar> totals;
+		for (std::size_t t = 0; t < steps; ++t)
+			totals.push_back(net.train_batch_adam(xd, yd, loss, t, (Scalar) 0.01));
+		record(tag + ".convnet.losses", sizeof(Scalar), { steps }, totals.data());
+		record_final<Scalar>(tag + ".convnet", net);
+		/* inference after training uses the running statistics */
+		const DT& out = net.propagate(xd, false);
+		record(tag + ".convnet.infer", sizeof(Scalar), { batch, 5 }, out.to_host().data());
+	}
+}
+
+int main(int argc, char** argv) {
+	if (argc != 2) {
+		std::fprintf(stderr, "usage: %s <records file>\n", argv[0]);
+		return 2;
+	}
+	try {
+		check(cattle_hip_init(0));
+		g_out = std::fopen(argv[1], "wb");
+		if (!g_out)
+			throw std::runtime_error("cannot open the records file");
+		run<float>("f32");
+		run<double>("f64");
+		std::fclose(g_out);
+	} catch (const std::exception& e) {
+		std::fprintf(stderr, "device_net_test: %s\n", e.what());
+		return 1;
+	}
+	return 0;
+}

@@ -1,0 +1,95 @@
+"""The device-resident C++ front end (c-attl3_amd/include/cattle_hip/DeviceNet.hpp) driven by
+tests/compat/device_net_test (built by __graft_entry__.build()): three training batches of an MLP with
+vanilla SGD and of a small convnet with Adam, every tensor staying on the GPU. The recorded inputs and
+initial parameters are replayed here on the CPU oracle with the host-side counterparts of the
+reference's callers (tests/harness.py), and batch losses, final parameters and the inference output
+are compared."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import harness as hn
+import helpers as hp
+from oracle import oracle
+from test_gpu_adapters import _read_records
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+BINARY = os.path.join(HERE, "compat", "device_net_test")
+
+
+def test_device_net_compiles_as_cpp11():
+    """CPU check: the header needs nothing but the C ABI and is valid C++11."""
+    subprocess.check_call(["g++", "-std=c++11", "-fsyntax-only", "-Wall", "-I" + os.path.join(HERE, "..", "include"),
+                           "-I" + os.path.join(HERE, "..", "c-attl3_amd", "include"),
+                           os.path.join(HERE, "compat", "device_net_test.cpp")])
+
+
+@pytest.fixture(scope="module")
+def records(tmp_path_factory):
+    if not os.path.exists(BINARY):
+        pytest.fail("tests/compat/device_net_test is not built: run __graft_entry__.build()")
+    out = str(tmp_path_factory.mktemp("device_net") / "records.bin")
+    subprocess.check_call([BINARY, out], timeout=120)
+    return _read_records(out)
+
+
+def _replay(r, net, lr, adam, steps=3):
+    """SGDOptimizer::_train's batch body on the oracle network, in float64."""
+    for li, layer in enumerate(net.layers):
+        for pi, p in enumerate(layer.get_params()):
+            p.set_values(np.asarray(r["init.%d.%d" % (li, pi)], np.float64))
+    x, y = np.asarray(r["x"], np.float64), np.asarray(r["y"], np.float64)
+    opt = hn.Adam(net.params(), lr=lr) if adam else None
+    losses = []
+    for t in range(steps):
+        out = hn.train_step_gradients(net, x, y.reshape((x.shape[0],) + out_shape(net), order="F"), hn.softmax_ce_grad)
+        losses.append(oracle.loss_function("softmax_cross_entropy", out, y.reshape(out.shape, order="F")).sum())
+        if adam:
+            opt.update(net.params(), t)
+        else:
+            hn.vanilla_sgd_update(net.params(), lr)
+        for p in net.params():
+            p.reset_grad()
+    return np.array(losses)
+
+
+def out_shape(net):
+    return tuple(net.layers[-1].get_output_dims())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-9)])
+def test_mlp_sgd_batches(records, tag, tol):
+    r = {k[len(tag) + 5:]: v for k, v in records.items() if k.startswith(tag + ".mlp.")}
+    be = hn.OracleBackend(np.float64)
+    net = hn.FeedforwardNet([be.dense((20,), 16), be.act("relu", (16,)), be.dense((16,), 6)])
+    lr = float(np.float32(0.05)) if tag == "f32" else 0.05
+    losses = _replay(r, net, lr, adam=False)
+    assert hp.rel_err(r["losses"], losses) < tol
+    assert losses[2] < losses[0]                                  # the steps do reduce the loss
+    for li, layer in enumerate(net.layers):
+        for pi, p in enumerate(layer.get_params()):
+            assert hp.rel_err(r["final.%d.%d" % (li, pi)], p.get_values()) < tol, (li, pi)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-9)])
+def test_convnet_adam_batches(records, tag, tol):
+    r = {k[len(tag) + 9:]: v for k, v in records.items() if k.startswith(tag + ".convnet.")}
+    be = hn.OracleBackend(np.float64)
+    net = hn.FeedforwardNet([be.conv((8, 8, 3), 8), be.act("relu", (8, 8, 8)), be.maxpool((8, 8, 8)),
+                             be.batchnorm((4, 4, 8)), be.dense((4, 4, 8), 5)])
+    lr = float(np.float32(0.01)) if tag == "f32" else 0.01
+    losses = _replay(r, net, lr, adam=True)
+    assert hp.rel_err(r["losses"], losses) < 10 * tol             # three Adam steps deep
+    for li, layer in enumerate(net.layers):
+        for pi, p in enumerate(layer.get_params()):
+            got, want = np.asarray(r["final.%d.%d" % (li, pi)], np.float64), p.get_values()
+            # an Adam step moves every weight by about lr whatever the gradient's size, so agreement is
+            # measured against the step (1 % of three steps of lr), not against the weight
+            assert np.max(np.abs(got - want)) < max(10 * tol, 1e-2 * 3 * lr if tag == "f32" else 1e-7), (li, pi)
+    x = np.asarray(r["x"], np.float64)
+    infer = net.propagate(x, False)
+    assert hp.rel_err(r["infer"], infer.reshape(r["infer"].shape, order="F")) < (1e-2 if tag == "f32" else 1e-6)
