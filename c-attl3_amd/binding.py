@@ -29,7 +29,7 @@ EXPORTS = [
     "cattle_hip_init", "cattle_hip_last_error", "cattle_hip_synchronize", "cattle_hip_alloc", "cattle_hip_free",
     "cattle_hip_upload", "cattle_hip_download", "cattle_hip_fill_zero", "cattle_hip_timer_create",
     "cattle_hip_timer_destroy", "cattle_hip_timer_start", "cattle_hip_timer_stop", "cattle_hip_conv_create",
-    "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
+    "cattle_hip_transconv_create", "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
     "cattle_hip_batchnorm_set_stats_initialized", "cattle_hip_activation_create", "cattle_hip_pool_create",
     "cattle_hip_layer_clone", "cattle_hip_layer_destroy", "cattle_hip_layer_input_dims",
     "cattle_hip_layer_output_dims", "cattle_hip_layer_is_input_layer", "cattle_hip_layer_set_input_layer",
@@ -376,6 +376,29 @@ class ConvKernelLayer(Layer):
         _check(lib().cattle_hip_layer_output_dims(h, od))
         OH, OW, F = int(od[0]), int(od[1]), int(od[2])
         # calculate_adjusted_output_dims (:206-217): filters land on the last nominal rank
+        out = {3: (OH, OW, F), 2: (OH, OW * F), 1: (OH * F,)}[rank]
+        Layer.__init__(self, h, dtype, tuple(input_dims), out)
+
+
+class TransConvKernelLayer(Layer):
+    """layer/kernel/TransConvKernelLayer.hpp:290-304; rank 1/2 inputs are re-viewed as in :404-417, :503-516 and the
+    filters land on the last nominal rank of the output (calculate_adjusted_output_dims, :241-251)."""
+
+    def __init__(self, dtype, input_dims, filters, receptor_height=3, receptor_width=3, vertical_padding=1,
+                 horizontal_padding=1, vertical_stride=1, horizontal_stride=1, vertical_dilation=0,
+                 horizontal_dilation=0):
+        rank = len(input_dims)
+        if rank == 1:       # TransConvKernelLayer<Scalar,1>(dims, filters, init, receptor_length, padding, stride, dilation)
+            receptor_width, horizontal_padding, horizontal_stride, horizontal_dilation = 1, 0, 1, 0
+        H, W, C = _ext3(input_dims)
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_transconv_create(_dtype_code(dtype), _sz(H), _sz(W), _sz(C), _sz(filters),
+                                                 _sz(receptor_height), _sz(receptor_width), _sz(vertical_padding),
+                                                 _sz(horizontal_padding), _sz(vertical_stride), _sz(horizontal_stride),
+                                                 _sz(vertical_dilation), _sz(horizontal_dilation), ctypes.byref(h)))
+        od = (ctypes.c_size_t * 3)()
+        _check(lib().cattle_hip_layer_output_dims(h, od))
+        OH, OW, F = int(od[0]), int(od[1]), int(od[2])
         out = {3: (OH, OW, F), 2: (OH, OW * F), 1: (OH * F,)}[rank]
         Layer.__init__(self, h, dtype, tuple(input_dims), out)
 

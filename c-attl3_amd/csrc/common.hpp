@@ -81,6 +81,13 @@ template<typename T> void conv_forward(const ConvShape& s, int N, const T* x, co
 template<typename T> void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad,
 		T* wgrad, T* bgrad, T* in_grad, T* wt_dgrad, bool wt_ready, T* partials);
 
+/* The two halves of conv_backward on their own (the transposed convolution uses them with the roles
+ * of input and output exchanged). bgrad may be null. */
+template<typename T> void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad,
+		T* partials);
+template<typename T> void conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad,
+		T* wt_dgrad, bool wt_ready);
+
 /* Element-wise / reduction kernels (pointwise_kernels.hip). */
 template<typename T> void act_forward(int kind, size_t n, T p, const T* x, T* y);
 template<typename T> void act_backward(int kind, size_t n, T p, const T* x, const T* y, const T* g, T* dx);
@@ -111,6 +118,12 @@ template<typename T> void meanpool_backward(const PoolShape& s, int N, const T* 
 
 /* dst[i] += src[i] */
 template<typename T> void axpy_one(size_t n, const T* src, T* dst);
+/* dst[c + cols*r] (+)= src[r + rows*c] for a column-major rows x cols matrix src */
+template<typename T> void transpose_matrix(int rows, int cols, const T* src, T* dst, bool accumulate);
+/* x[n + N*e] += row[e]  (a 1 x V row vector added to every row of an N x V matrix) */
+template<typename T> void add_row_vector(int N, size_t V, const T* row, T* x);
+/* row[e] += sum_n x[n + N*e]  (column sums of an N x V matrix, accumulated) */
+template<typename T> void accumulate_column_sums(int N, size_t V, const T* x, T* row);
 
 /* Losses and optimizer updates (train_kernels.hip). A batch is N samples x T_steps x V elements,
  * column-major with the sample index fastest. */

@@ -947,27 +947,29 @@ void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b,
 }
 
 template<typename T>
-void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad,
-		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials) {
+void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials) {
 	check_sizes(s, N);
 	const GatherGeom g = forward_geom(s, N);
-	/* weight and bias gradients: split-M partials, then a fixed-order reduction that accumulates */
-	{
-		const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N);
-		const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
-		const size_t count = (size_t) g.K * g.F;
-		T* bias_partials = partials + (size_t) p.splits * count;
-		const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode };
-		const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-				(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
-		v.launch(x, out_grad, partials, bias_partials, g, split, vec);
-		reduce_partials_kernel<T><<<(unsigned) ((count + 63) / 64), 256, 0, stream()>>>(partials, wgrad, count, p.splits);
-		CATTLE_HIP_CHECK(hipGetLastError());
+	/* split-M partials, then a fixed-order reduction that accumulates */
+	const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N);
+	const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
+	const size_t count = (size_t) g.K * g.F;
+	T* bias_partials = partials + (size_t) p.splits * count;
+	const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode };
+	const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
+	v.launch(x, out_grad, partials, bias_partials, g, split, vec);
+	reduce_partials_kernel<T><<<(unsigned) ((count + 63) / 64), 256, 0, stream()>>>(partials, wgrad, count, p.splits);
+	CATTLE_HIP_CHECK(hipGetLastError());
+	if (bgrad) {
 		reduce_partials_kernel<T><<<(unsigned) ((g.F + 63) / 64), 256, 0, stream()>>>(bias_partials, bgrad, (size_t) g.F, p.splits);
 		CATTLE_HIP_CHECK(hipGetLastError());
 	}
-	if (!in_grad)
-		return;
+}
+
+template<typename T>
+void conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad, T* wt_dgrad, bool wt_ready) {
+	check_sizes(s, N);
 	const GatherGeom d = dgrad_geom(s, N);
 	if (!wt_ready) {
 		const int Kp = round_up(d.K, WT_ROW_PAD);
@@ -979,6 +981,14 @@ void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* o
 	launch_gather<T>(out_grad, wt_dgrad, (const T*) nullptr, in_grad, d);
 }
 
+template<typename T>
+void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad,
+		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials) {
+	conv_weight_gradient<T>(s, N, x, out_grad, wgrad, bgrad, partials);
+	if (in_grad)
+		conv_input_gradient<T>(s, N, w, out_grad, in_grad, wt_dgrad, wt_ready);
+}
+
 template ConvWorkspace conv_workspace<float>(const ConvShape&, int);
 template ConvWorkspace conv_workspace<double>(const ConvShape&, int);
 template void conv_forward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, bool);
@@ -987,5 +997,9 @@ template void conv_backward<float>(const ConvShape&, int, const float*, const fl
 		float*, bool, float*);
 template void conv_backward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*,
 		double*, double*, bool, double*);
+template void conv_weight_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, float*);
+template void conv_weight_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, double*);
+template void conv_input_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, bool);
+template void conv_input_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, bool);
 
 } /* namespace cattle_hip */

@@ -98,8 +98,8 @@ struct Param {
 	size_t esize;
 	DevBuf values, grad;
 	uint64_t version = 1;
-	DevBuf derived[2];
-	uint64_t derived_version[2] = { 0, 0 };
+	DevBuf derived[3];
+	uint64_t derived_version[3] = { 0, 0, 0 };
 	DevBuf moments[2];                 /* optimizer moving averages, allocated on first use */
 	bool moments_ready = false;
 	Param(size_t rows, size_t cols, bool optimizable, size_t esize) : rows(rows), cols(cols), optimizable(optimizable), esize(esize) {
@@ -220,6 +220,77 @@ struct ConvLayer : LayerBase {
 				(T*) in_grad, wt, ready, part);
 		if (in_grad)
 			w.derived_version[1] = w.version;
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		x_cache = nullptr;
+	}
+};
+
+/* TransConvKernelLayer (layer/kernel/TransConvKernelLayer.hpp:143-216). Its forward pass scatters
+ * in * W into the output, which is the input gradient of the convolution that maps the output back
+ * to the input (same receptor, padding, stride, dilation; channels and filters exchanged) with
+ * weights W^T; its backward pass is that convolution's forward pass (input gradient) and weight
+ * gradient (transposed). So the three GEMM kernels are reused as they are:
+ *   weights W [C x RH*RW*F], column rh + RH*(rw + RW*f)   ->   Wc = W^T, the convolution's [K x C]
+ *   bias    [1 x OH*OW*F], one entry per output activation (:52-56). */
+template<typename T>
+struct TransConvLayer : LayerBase {
+	ConvShape conv;                   /* the equivalent convolution: output dims -> input dims */
+	const T* x_cache = nullptr;
+	DevBuf partials, wgrad_t;
+
+	TransConvLayer(int dtype, const ConvShape& c) : LayerBase(dtype), conv(c) {
+		in_dims[0] = (size_t) c.OH(); in_dims[1] = (size_t) c.OW(); in_dims[2] = (size_t) c.F;
+		out_dims[0] = (size_t) c.H; out_dims[1] = (size_t) c.W; out_dims[2] = (size_t) c.C;
+		params.push_back(std::make_shared<Param>((size_t) c.F, (size_t) c.K(), true, sizeof(T)));
+		params.push_back(std::make_shared<Param>(1, out_volume(), true, sizeof(T)));
+	}
+	TransConvLayer(const TransConvLayer& o, bool share) : LayerBase(o.dtype), conv(o.conv) {
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new TransConvLayer(*this, share);
+	}
+	/* Wc = W^T, rebuilt when the weights change */
+	const T* conv_weights() {
+		Param& w = *params[0];
+		T* wc = (T*) w.derived[2].ensure(w.bytes());
+		if (w.derived_version[2] != w.version) {
+			transpose_matrix<T>((int) w.rows, (int) w.cols, (const T*) w.values.p, wc, false);
+			w.derived_version[2] = w.version;
+		}
+		return wc;
+	}
+	void forward(const void* in, size_t N, bool, void* out) override {
+		const int n = checked_int(N, "batch size");
+		const ConvWorkspace ws = conv_workspace<T>(conv, n);
+		Param& w = *params[0];
+		const T* wc = conv_weights();
+		T* wt = (T*) w.derived[1].ensure(ws.wt_dgrad * sizeof(T));
+		conv_input_gradient<T>(conv, n, wc, (const T*) in, (T*) out, wt, w.derived_version[1] == w.version);
+		w.derived_version[1] = w.version;
+		add_row_vector<T>(n, out_volume(), (const T*) params[1]->values.p, (T*) out);
+		x_cache = (const T*) in;       /* in_mat_cache (:147) */
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		CATTLE_HIP_REQUIRE(x_cache != nullptr, "pass_back without a cached forward input");
+		const int n = checked_int(N, "batch size");
+		const ConvWorkspace ws = conv_workspace<T>(conv, n);
+		Param& w = *params[0];
+		accumulate_column_sums<T>(n, out_volume(), (const T*) out_grad, (T*) params[1]->grad.p);      /* :184-185 */
+		/* in_mat^T * patches(out_grad) (:208) is the transpose of the convolution's weight gradient */
+		T* part = (T*) partials.ensure(ws.partials * sizeof(T));
+		T* gt = (T*) wgrad_t.ensure(w.bytes());
+		fill_zero(gt, w.bytes());
+		conv_weight_gradient<T>(conv, n, (const T*) out_grad, x_cache, gt, (T*) nullptr, part);
+		transpose_matrix<T>((int) w.cols, (int) w.rows, gt, (T*) w.grad.p, true);
+		if (!in_grad)
+			return;
+		const T* wc = conv_weights();
+		T* wt = (T*) w.derived[0].ensure(ws.wt_fwd * sizeof(T));
+		conv_forward<T>(conv, n, (const T*) out_grad, wc, (const T*) nullptr, (T*) in_grad, wt, w.derived_version[0] == w.version);
+		w.derived_version[0] = w.version;
 	}
 	void empty_cache() override {
 		LayerBase::empty_cache();
@@ -639,6 +710,44 @@ int cattle_hip_conv_create(cattle_hip_dtype dtype, size_t height, size_t width, 
 				(int) vertical_dilation, (int) horizontal_dilation };
 		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new ConvLayer<float>(dtype, s, false) :
 				(LayerBase*) new ConvLayer<double>(dtype, s, false);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_transconv_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, size_t filters,
+		size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
+		cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr, "null output pointer");
+		/* the constructor assertions of layer/kernel/TransConvKernelLayer.hpp:84-89 */
+		CATTLE_HIP_REQUIRE(height > 0 && width > 0 && channels > 0, "input dimensions must be positive");
+		CATTLE_HIP_REQUIRE(filters > 0, "filters must be positive");
+		CATTLE_HIP_REQUIRE(receptor_height > 0 && receptor_width > 0, "receptor dimensions must be positive");
+		CATTLE_HIP_REQUIRE(vertical_stride > 0 && horizontal_stride > 0, "strides must be positive");
+		const size_t lim = 1u << 20;
+		CATTLE_HIP_REQUIRE(height < lim && width < lim && channels < lim && filters < lim && receptor_height < lim &&
+				receptor_width < lim && vertical_padding < lim && horizontal_padding < lim && vertical_stride < lim &&
+				horizontal_stride < lim && vertical_dilation < lim && horizontal_dilation < lim, "dimension too large");
+		/* calculate_spatial_output_dim (:226-229) */
+		const size_t drh = receptor_height + (receptor_height - 1) * vertical_dilation;
+		const size_t drw = receptor_width + (receptor_width - 1) * horizontal_dilation;
+		const size_t full_h = (height - 1) * vertical_stride + drh, full_w = (width - 1) * horizontal_stride + drw;
+		CATTLE_HIP_REQUIRE(full_h > 2 * vertical_padding && full_w > 2 * horizontal_padding,
+				"the padding cuts away the whole output");
+		const size_t out_h = full_h - 2 * vertical_padding, out_w = full_w - 2 * horizontal_padding;
+		CATTLE_HIP_REQUIRE(out_h < lim && out_w < lim, "dimension too large");
+		CATTLE_HIP_REQUIRE(receptor_height * receptor_width * channels <= 2147483647u / 2 &&
+				receptor_height * receptor_width * filters <= 2147483647u / 2, "receptor volume too large");
+		/* the equivalent convolution maps the output (out_h, out_w, filters) back to the input */
+		ConvShape c = { (int) out_h, (int) out_w, (int) filters, (int) channels, (int) receptor_height, (int) receptor_width,
+				(int) vertical_padding, (int) horizontal_padding, (int) vertical_stride, (int) horizontal_stride,
+				(int) vertical_dilation, (int) horizontal_dilation };
+		if ((size_t) c.OH() != height || (size_t) c.OW() != width)
+			throw Error(ERR_INVALID, "inconsistent transposed convolution geometry");
+		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new TransConvLayer<float>(dtype, c) :
+				(LayerBase*) new TransConvLayer<double>(dtype, c);
 		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
 	});
 }

@@ -609,6 +609,55 @@ __global__ void axpy_one_kernel(size_t n, const T* __restrict__ src, T* __restri
 		dst[i] += src[i];
 }
 
+/* ----------------------------------------------------------------------------------------------
+ * Small matrix helpers of the transposed convolution: its weight matrix is the transpose of the
+ * equivalent convolution's, and its bias has one entry per output activation
+ * (layer/kernel/TransConvKernelLayer.hpp:46-56, :143-144, :153-155).
+ * -------------------------------------------------------------------------------------------- */
+template<typename T, bool ACC>
+__global__ __launch_bounds__(256)
+void transpose_kernel(int rows, int cols, const T* __restrict__ src, T* __restrict__ dst) {
+	__shared__ T tile[32][33];
+	const int r0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+	const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+	for (int j = ty; j < 32; j += 8) {
+		const int r = r0 + tx, c = c0 + j;
+		tile[j][tx] = r < rows && c < cols ? src[(size_t) r + (size_t) rows * c] : (T) 0;
+	}
+	__syncthreads();
+	for (int j = ty; j < 32; j += 8) {
+		const int c = c0 + tx, r = r0 + j;
+		if (r < rows && c < cols) {
+			const size_t o = (size_t) c + (size_t) cols * r;
+			dst[o] = ACC ? dst[o] + tile[tx][j] : tile[tx][j];
+		}
+	}
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void add_row_vector_kernel(size_t total, int N, const T* __restrict__ row, T* __restrict__ x) {
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride)
+		x[i] += row[i / (size_t) N];
+}
+
+/* one wavefront per column: lanes stride over the N contiguous entries, fixed-order shuffle sum */
+template<typename T>
+__global__ __launch_bounds__(256)
+void column_sums_kernel(int N, size_t V, const T* __restrict__ x, T* __restrict__ row) {
+	const int lane = threadIdx.x % 64;
+	const size_t waves = (size_t) gridDim.x * 4;
+	for (size_t e = (size_t) blockIdx.x * 4 + threadIdx.x / 64; e < V; e += waves) {
+		T s = (T) 0;
+		for (int n = lane; n < N; n += 64)
+			s += x[(size_t) n + (size_t) N * e];
+		s = wave_sum(s);
+		if (lane == 0)
+			row[e] += s;
+	}
+}
+
 void check_launch() {
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
@@ -794,6 +843,36 @@ void axpy_one(size_t n, const T* src, T* dst) {
 	check_launch();
 }
 
+template<typename T>
+void transpose_matrix(int rows, int cols, const T* src, T* dst, bool accumulate) {
+	if (rows == 0 || cols == 0)
+		return;
+	const dim3 grid((unsigned) ((rows + 31) / 32), (unsigned) ((cols + 31) / 32));
+	if (accumulate)
+		transpose_kernel<T, true><<<grid, 256, 0, stream()>>>(rows, cols, src, dst);
+	else
+		transpose_kernel<T, false><<<grid, 256, 0, stream()>>>(rows, cols, src, dst);
+	check_launch();
+}
+
+template<typename T>
+void add_row_vector(int N, size_t V, const T* row, T* x) {
+	const size_t total = (size_t) N * V;
+	if (total == 0)
+		return;
+	add_row_vector_kernel<T><<<stream_grid(total), 256, 0, stream()>>>(total, N, row, x);
+	check_launch();
+}
+
+template<typename T>
+void accumulate_column_sums(int N, size_t V, const T* x, T* row) {
+	if (V == 0 || N == 0)
+		return;
+	const size_t blocks = std::min<size_t>((V + 3) / 4, 256 * 16);
+	column_sums_kernel<T><<<(unsigned) blocks, 256, 0, stream()>>>(N, V, x, row);
+	check_launch();
+}
+
 #define CATTLE_HIP_INSTANTIATE(T) \
 template void act_forward<T>(int, size_t, T, const T*, T*); \
 template void act_backward<T>(int, size_t, T, const T*, const T*, const T*, T*); \
@@ -809,7 +888,10 @@ template void maxpool_forward<T>(const PoolShape&, int, const T*, T*, unsigned*)
 template void maxpool_backward<T>(const PoolShape&, int, const T*, const unsigned*, T*); \
 template void meanpool_forward<T>(const PoolShape&, int, const T*, T*); \
 template void meanpool_backward<T>(const PoolShape&, int, const T*, T*); \
-template void axpy_one<T>(size_t, const T*, T*);
+template void axpy_one<T>(size_t, const T*, T*); \
+template void transpose_matrix<T>(int, int, const T*, T*, bool); \
+template void add_row_vector<T>(int, size_t, const T*, T*); \
+template void accumulate_column_sums<T>(int, size_t, const T*, T*);
 
 CATTLE_HIP_INSTANTIATE(float)
 CATTLE_HIP_INSTANTIATE(double)

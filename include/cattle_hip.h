@@ -94,6 +94,18 @@ int cattle_hip_conv_create(cattle_hip_dtype dtype, size_t height, size_t width, 
 		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
 		cattle_hip_layer_t* layer);
 
+/* TransConvKernelLayer<Scalar,Rank>(input_dims, filters, init, receptor_height, receptor_width,
+ * vertical_padding, horizontal_padding, vertical_stride, horizontal_stride, vertical_dilation,
+ * horizontal_dilation) — layer/kernel/TransConvKernelLayer.hpp:285-299 (rank 2 :345-360, rank 1
+ * :444-459). Output height = (height - 1) * stride + receptor + (receptor - 1) * dilation - 2 * padding
+ * (:226-229). Parameters: 0 = weights [channels x receptor_height*receptor_width*filters] with column
+ * index rh + RH*(rw + RW*f) (:46-48, :159-160), 1 = bias [1 x output volume], one entry per output
+ * activation (:52-56, :172-173). */
+int cattle_hip_transconv_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, size_t filters,
+		size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
+		cattle_hip_layer_t* layer);
+
 /* DenseKernelLayer<Scalar,Rank>(input_dims, output_size, init) — layer/kernel/DenseKernelLayer.hpp:61-77.
  * input_volume = input_dims.get_volume(). Parameters: 0 = weights [input_volume x output_size],
  * 1 = bias [1 x output_size]. */

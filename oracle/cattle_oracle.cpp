@@ -18,6 +18,8 @@
  *   batch norm          pinned: closed-form invariants + torch float64 batch_norm.
  *   activations         pinned: libm/numpy closed forms and derivative-at-zero conventions.
  *   max/mean pool       pinned: brute force incl. crafted ties, NaN/-inf windows, overlaps.
+ *   transposed conv     pinned: torch float64 conv_transpose2d with autograd, the adjoint identity with
+ *                       the (pinned) convolution, output-size formula on the reference's test geometries.
  *   losses              pinned: torch float64 cross_entropy / mse (epsilon 0), numpy closed forms with
  *                       the epsilon, central differences of the loss against its gradient.
  *   SGD / Adam updates  pinned: numpy restatement in float64, first-step closed form, and torch's Adam
@@ -612,6 +614,88 @@ int meanpool_backward(PoolGeom g, const T* out_grad, T* in_grad) {
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * TransConvKernelLayerBase::_pass_forward / _pass_back (layer/kernel/TransConvKernelLayer.hpp:143-216),
+ * restated with the reference's own staging: in_mat[(n, ih, iw) x C] * W[C x RH*RW*F], each row's
+ * receptor patch added into the zero-padded output (width-major / height-minor patch order, :153-169),
+ * padding cut off, per-activation bias added; backward gathers the same patches from the padded output
+ * gradient into a matrix and multiplies (:186-214).
+ * ------------------------------------------------------------------------------------------- */
+struct TransGeom {
+	i64 N, IH, IW, C, F, RH, RW, pv, ph, sv, sh, dv, dh;
+	i64 OH, OW, PH, PW, DRH, DRW;
+	void derive() {
+		DRH = RH + (RH - 1) * dv;
+		DRW = RW + (RW - 1) * dh;
+		OH = (IH - 1) * sv + DRH - 2 * pv;      /* calculate_spatial_output_dim :226-229 */
+		OW = (IW - 1) * sh + DRW - 2 * ph;
+		PH = OH + 2 * pv;
+		PW = OW + 2 * ph;
+	}
+};
+
+template<typename T>
+int transconv_forward(TransGeom g, const T* x, const T* w, const T* bias, T* out) {
+	g.derive();
+	const i64 M = g.N * g.IH * g.IW, RV = g.RH * g.RW * g.F;
+	std::vector<T> conv_mat((size_t) (M * RV));
+	gemm_nn<T>(M, g.C, RV, x, w, nullptr, conv_mat.data());
+	std::vector<T> padded((size_t) (g.N * g.PH * g.PW * g.F), (T) 0);
+	i64 patch = 0;
+	for (i64 i = 0; i + g.DRW <= g.PW; i += g.sh)
+		for (i64 j = 0; j + g.DRH <= g.PH; j += g.sv) {
+			for (i64 f = 0; f < g.F; ++f)
+				for (i64 rw = 0; rw < g.RW; ++rw)
+					for (i64 rh = 0; rh < g.RH; ++rh)
+						for (i64 n = 0; n < g.N; ++n)
+							padded[n + g.N * ((j + rh * (g.dv + 1)) + g.PH * ((i + rw * (g.dh + 1)) + g.PW * f))] +=
+									conv_mat[(patch + n) + M * (rh + g.RH * (rw + g.RW * f))];
+			patch += g.N;
+		}
+	if (patch != M)
+		return 1;
+	for (i64 f = 0; f < g.F; ++f)
+		for (i64 ow = 0; ow < g.OW; ++ow)
+			for (i64 oh = 0; oh < g.OH; ++oh)
+				for (i64 n = 0; n < g.N; ++n)
+					out[n + g.N * (oh + g.OH * (ow + g.OW * f))] =
+							padded[n + g.N * ((oh + g.pv) + g.PH * ((ow + g.ph) + g.PW * f))] + bias[oh + g.OH * (ow + g.OW * f)];
+	return 0;
+}
+
+template<typename T>
+int transconv_backward(TransGeom g, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad, T* in_grad) {
+	g.derive();
+	const i64 M = g.N * g.IH * g.IW, RV = g.RH * g.RW * g.F, OV = g.OH * g.OW * g.F;
+	for (i64 e = 0; e < OV; ++e) {
+		T s = 0;
+		for (i64 n = 0; n < g.N; ++n)
+			s += out_grad[n + g.N * e];
+		bgrad[e] += s;
+	}
+	std::vector<T> patches((size_t) (M * RV));
+	i64 patch = 0;
+	for (i64 i = 0; i + g.DRW <= g.PW; i += g.sh)
+		for (i64 j = 0; j + g.DRH <= g.PH; j += g.sv) {
+			for (i64 f = 0; f < g.F; ++f)
+				for (i64 rw = 0; rw < g.RW; ++rw)
+					for (i64 rh = 0; rh < g.RH; ++rh) {
+						const i64 oh = j + rh * (g.dv + 1) - g.pv, ow = i + rw * (g.dh + 1) - g.ph;
+						const bool inside = oh >= 0 && oh < g.OH && ow >= 0 && ow < g.OW;
+						for (i64 n = 0; n < g.N; ++n)
+							patches[(patch + n) + M * (rh + g.RH * (rw + g.RW * f))] =
+									inside ? out_grad[n + g.N * (oh + g.OH * (ow + g.OW * f))] : (T) 0;
+					}
+			patch += g.N;
+		}
+	if (patch != M)
+		return 1;
+	gemm_tn_acc<T>(M, g.C, RV, x, patches.data(), wgrad);          /* in_mat_cache^T * out_grad_conv_mat (:208) */
+	if (in_grad)
+		gemm_nt<T>(M, g.C, RV, patches.data(), w, in_grad);        /* out_grad_conv_mat * W^T (:211) */
+	return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
  * Losses (loss/SquaredLoss.hpp:25-34, loss/SoftmaxCrossEntropyLoss.hpp:33-50) under the
  * UniversalLoss drivers (loss/UniversalLoss.hpp:37-46 non-sequential; :99-125 sequential: every time
  * step is sliced out and treated as its own rows x cols matrix, losses add up over the steps).
@@ -745,6 +829,12 @@ extern "C" int oracle_meanpool_forward_##SFX(POOL_ARGS, const T* x, T* out) { \
 	POOL_GEOM; return meanpool_forward<T>(g, x, out); } \
 extern "C" int oracle_meanpool_backward_##SFX(POOL_ARGS, const T* out_grad, T* in_grad) { \
 	POOL_GEOM; return meanpool_backward<T>(g, out_grad, in_grad); } \
+extern "C" int oracle_transconv_forward_##SFX(CONV_ARGS, const T* x, const T* w, const T* b, T* out) { \
+	TransGeom g = { N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh, 0, 0, 0, 0, 0, 0 }; \
+	return transconv_forward<T>(g, x, w, b, out); } \
+extern "C" int oracle_transconv_backward_##SFX(CONV_ARGS, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad, \
+		T* in_grad) { TransGeom g = { N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh, 0, 0, 0, 0, 0, 0 }; \
+	return transconv_backward<T>(g, x, w, out_grad, wgrad, bgrad, in_grad); } \
 extern "C" int oracle_loss_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double eps, const T* out, const T* obj, T* losses) { \
 	return loss_function<T>(kind, N, Ts, V, (T) eps, out, obj, losses); } \
 extern "C" int oracle_loss_d_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double eps, double scale, const T* out, \

@@ -117,6 +117,39 @@ def conv_backward(x_shape, cache, w, out_grad, RH=3, RW=3, pv=1, ph=1, sv=1, sh=
     return in_grad, wgrad, bgrad
 
 
+def transconv_out_dims(IH, IW, RH, RW, pv, ph, sv, sh, dv, dh):
+    return ((IH - 1) * sv + RH + (RH - 1) * dv - 2 * pv, (IW - 1) * sh + RW + (RW - 1) * dh - 2 * ph)
+
+
+def transconv_forward(x, w, b, F, RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0):
+    """x (N,IH,IW,C); w [C x RH*RW*F]; b [1 x OH*OW*F]; returns (N,OH,OW,F)."""
+    dt = x.dtype
+    x = _f(x, dt)
+    N, IH, IW, C = x.shape
+    assert w.shape == (C, RH * RW * F)
+    OH, OW = transconv_out_dims(IH, IW, RH, RW, pv, ph, sv, sh, dv, dh)
+    w = _f(w, dt)
+    b = _f(np.reshape(b, (OH * OW * F,)), dt)
+    out = np.empty((N, OH, OW, F), dtype=dt, order="F")
+    _call("transconv_forward", dt, *_ll(N, IH, IW, C, F, RH, RW, pv, ph, sv, sh, dv, dh), _p(x), _p(w), _p(b), _p(out))
+    return out
+
+
+def transconv_backward(x, w, out_grad, RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0, input_layer=False, wgrad=None,
+                       bgrad=None):
+    """Returns (in_grad or None, wgrad, bgrad); wgrad/bgrad accumulate into the arrays passed in."""
+    dt = x.dtype
+    x, w, out_grad = _f(x, dt), _f(w, dt), _f(out_grad, dt)
+    N, IH, IW, C = x.shape
+    F = out_grad.shape[3]
+    wgrad = np.zeros(w.shape, dtype=dt, order="F") if wgrad is None else wgrad
+    bgrad = np.zeros((1, out_grad.size // N), dtype=dt, order="F") if bgrad is None else bgrad
+    in_grad = None if input_layer else np.empty(x.shape, dtype=dt, order="F")
+    _call("transconv_backward", dt, *_ll(N, IH, IW, C, F, RH, RW, pv, ph, sv, sh, dv, dh), _p(x), _p(w), _p(out_grad),
+          _p(wgrad), _p(bgrad), _p(in_grad))
+    return in_grad, wgrad, bgrad
+
+
 def dense_forward(x, w, b):
     dt = x.dtype
     N = x.shape[0]

@@ -16,6 +16,19 @@ REFERENCE_CONV_CASES = [
     (9, 11, 2, 3, 2, 3, 0, 1, 2, 3, 0, 1),    # strides (2,3), dilation (0,1), no vertical padding
 ]
 
+# Transposed-convolution geometries of the reference's gradient test (test/gradient_test.cpp:194-204), re-viewed as
+# 4-D problems the way TransConvKernelLayer<Scalar,1|2> does (layer/kernel/TransConvKernelLayer.hpp:404-417,
+# :503-516), plus an up-sampling case.   (IH, IW, C, F, RH, RW, pv, ph, sv, sh, dv, dh)
+REFERENCE_TRANSCONV_CASES = [
+    (16, 1, 1, 5, 4, 1, 1, 0, 1, 1, 1, 0),    # rank 1: length 16, receptor 4, padding 1, dilation 1
+    (100, 1, 1, 1, 1, 1, 1, 0, 1, 1, 0, 0),   # rank 1 second layer: receptor 1, padding 1 (cuts the border)
+    (4, 5, 1, 5, 5, 3, 1, 0, 1, 2, 0, 1),     # rank 2: 5x3 receptor, pad (1,0), stride (1,2), dilation (0,1)
+    (2, 3, 2, 5, 5, 3, 1, 0, 1, 2, 0, 1),     # rank 3: same on 2x3x2
+    (4, 9, 5, 1, 2, 2, 1, 1, 1, 1, 0, 0),     # second layer: 2x2 p1 s1
+    (5, 4, 3, 4, 3, 3, 1, 1, 1, 1, 0, 0),     # 3x3 p1 s1 (shape preserving)
+    (4, 3, 2, 3, 4, 4, 1, 1, 2, 2, 0, 0),     # 4x4 stride 2 padding 1: doubles the resolution
+]
+
 
 def rng(seed):
     return np.random.default_rng(seed)
