@@ -7,6 +7,7 @@
  * NeuralNetwork, Optimizer or GradientCheck of the library works on top of it unchanged:
  *
  *   cattle::ConvKernelLayer<S,R>        ->  cattle::hip::ConvKernelHIPLayer<S,R>
+ *   cattle::TransConvKernelLayer<S,R>   ->  cattle::hip::TransConvKernelHIPLayer<S,R>
  *   cattle::DenseKernelLayer<S,R>       ->  cattle::hip::DenseKernelHIPLayer<S,R>
  *   cattle::BatchNormLayer<S,R,P>       ->  cattle::hip::BatchNormHIPLayer<S,R,P>
  *   cattle::<Name>ActivationLayer<S,R>  ->  cattle::hip::<Name>ActivationHIPLayer<S,R>
@@ -131,20 +132,22 @@ inline Dims contracted(const std::array<std::size_t,3>& ext) {
 } /* namespace detail */
 
 /**
- * Drop-in for ConvKernelLayer<Scalar,Rank> (layer/kernel/ConvKernelLayer.hpp:232-512). For rank 2 the
- * input is viewed as single-channel, for rank 1 additionally as single-column, and the filters are
- * folded into the last nominal rank of the output, as in calculate_adjusted_output_dims (:206-217).
+ * Common body of the drop-ins for ConvKernelLayer<Scalar,Rank> (layer/kernel/ConvKernelLayer.hpp:232-512)
+ * and, with Transposed, TransConvKernelLayer<Scalar,Rank> (layer/kernel/TransConvKernelLayer.hpp:241-520).
+ * For rank 2 the input is viewed as single-channel, for rank 1 additionally as single-column, and the
+ * filters are folded into the last nominal rank of the output, as in calculate_adjusted_output_dims
+ * (ConvKernelLayer.hpp:206-217, TransConvKernelLayer.hpp:241-251).
  */
-template<typename Scalar, std::size_t Rank>
-class ConvKernelHIPLayerBase : public KernelLayer<Scalar,Rank> {
+template<typename Scalar, std::size_t Rank, bool Transposed>
+class ConvFamilyHIPLayerBase : public KernelLayer<Scalar,Rank> {
 	typedef Layer<Scalar,Rank> Root;
 	typedef KernelLayer<Scalar,Rank> Base;
 public:
 	inline Root* clone() const {
-		return new ConvKernelHIPLayerBase(*this, false);
+		return new ConvFamilyHIPLayerBase(*this, false);
 	}
 	inline Root* clone_with_shared_params() {
-		return new ConvKernelHIPLayerBase(*this, true);
+		return new ConvFamilyHIPLayerBase(*this, true);
 	}
 	inline void empty_cache() {
 		detail::check(cattle_hip_layer_empty_cache(device.get()));
@@ -179,14 +182,14 @@ protected:
 		std::size_t filters, receptor_height, receptor_width, vertical_padding, horizontal_padding, vertical_stride,
 				horizontal_stride, vertical_dilation, horizontal_dilation;
 	};
-	inline ConvKernelHIPLayerBase(const typename Root::Dims& input_dims, const Geometry& geom,
+	inline ConvFamilyHIPLayerBase(const typename Root::Dims& input_dims, const Geometry& geom,
 			ParamsSharedPtr<Scalar> weights, ParamsSharedPtr<Scalar> bias) :
 				Base(input_dims, output_dims_for(input_dims, geom), weights, bias),
 				geom(geom),
 				batch_size(0) {
 		create_device_layer();
 	}
-	inline ConvKernelHIPLayerBase(const ConvKernelHIPLayerBase<Scalar,Rank>& layer, bool share_params) :
+	inline ConvFamilyHIPLayerBase(const ConvFamilyHIPLayerBase<Scalar,Rank,Transposed>& layer, bool share_params) :
 			Base(layer, share_params),
 			geom(layer.geom),
 			batch_size(0) {
@@ -196,10 +199,11 @@ protected:
 			std::size_t receptor_width) {
 		return receptor_height * receptor_width * detail::extended<typename Root::Dims,Rank>(input_dims)[2];
 	}
-private:
 	inline static std::size_t spatial_output_dim(std::size_t input_dim, std::size_t receptor, std::size_t padding,
 			std::size_t dilation, std::size_t stride) {
-		return (input_dim - receptor - (receptor - 1) * dilation + 2 * padding) / stride + 1;
+		if (Transposed)         /* TransConvKernelLayer.hpp:226-229 */
+			return (input_dim - 1) * stride + receptor + (receptor - 1) * dilation - 2 * padding;
+		return (input_dim - receptor - (receptor - 1) * dilation + 2 * padding) / stride + 1;       /* ConvKernelLayer.hpp:194-197 */
 	}
 	inline static typename Root::Dims output_dims_for(const typename Root::Dims& input_dims, const Geometry& g) {
 		const std::array<std::size_t,3> in = detail::extended<typename Root::Dims,Rank>(input_dims);
@@ -210,16 +214,23 @@ private:
 		out[Rank - 1] *= g.filters;
 		return detail::contracted<typename Root::Dims,Rank>(out);
 	}
+private:
 	inline void create_device_layer() {
 		const std::array<std::size_t,3> in = detail::extended<typename Root::Dims,Rank>(Base::input_dims);
-		detail::check(cattle_hip_conv_create(detail::ScalarCode<Scalar>::value, in[0], in[1], in[2], geom.filters,
-				geom.receptor_height, geom.receptor_width, geom.vertical_padding, geom.horizontal_padding,
-				geom.vertical_stride, geom.horizontal_stride, geom.vertical_dilation, geom.horizontal_dilation, device.out()));
+		detail::check((Transposed ? cattle_hip_transconv_create : cattle_hip_conv_create)(detail::ScalarCode<Scalar>::value,
+				in[0], in[1], in[2], geom.filters, geom.receptor_height, geom.receptor_width, geom.vertical_padding,
+				geom.horizontal_padding, geom.vertical_stride, geom.horizontal_stride, geom.vertical_dilation,
+				geom.horizontal_dilation, device.out()));
 	}
 	const Geometry geom;
 	detail::Handle device;
 	std::size_t batch_size;
 };
+
+template<typename Scalar, std::size_t Rank>
+using ConvKernelHIPLayerBase = ConvFamilyHIPLayerBase<Scalar,Rank,false>;
+template<typename Scalar, std::size_t Rank>
+using TransConvKernelHIPLayerBase = ConvFamilyHIPLayerBase<Scalar,Rank,true>;
 
 /** Rank 3 and rank 2: the constructor of ConvKernelLayer<Scalar,3|2> (ConvKernelLayer.hpp:282-296, :375-389). */
 template<typename Scalar, std::size_t Rank = 3>
@@ -269,6 +280,64 @@ public:
 						std::make_shared<StandardParameters<Scalar>>(1, filters, true,
 								std::make_shared<ZeroParameterInitialization<Scalar>>(), bias_reg, bias_clip, bias_max_l1_norm,
 								bias_max_l2_norm, bias_grad_clip, bias_grad_max_l1_norm, bias_grad_max_l2_norm)) { }
+};
+
+/**
+ * Drop-in for TransConvKernelLayer<Scalar,3|2> (TransConvKernelLayer.hpp:290-304, :386-400): weights
+ * [channels x receptor_height*receptor_width*filters], one bias entry per output activation (:46-56).
+ */
+template<typename Scalar, std::size_t Rank = 3>
+class TransConvKernelHIPLayer : public TransConvKernelHIPLayerBase<Scalar,Rank> {
+	typedef Layer<Scalar,Rank> Root;
+	typedef TransConvKernelHIPLayerBase<Scalar,Rank> TransBase;
+public:
+	inline TransConvKernelHIPLayer(const typename Root::Dims& input_dims, std::size_t filters,
+			ParamInitSharedPtr<Scalar> weight_init, std::size_t receptor_height = 3, std::size_t receptor_width = 3,
+			std::size_t vertical_padding = 1, std::size_t horizontal_padding = 1, std::size_t vertical_stride = 1,
+			std::size_t horizontal_stride = 1, std::size_t vertical_dilation = 0, std::size_t horizontal_dilation = 0,
+			ParamRegSharedPtr<Scalar> weight_reg = nullptr, Scalar weight_clip = 0, Scalar weight_max_l1_norm = 0,
+			Scalar weight_max_l2_norm = 0, Scalar weight_grad_clip = 0, Scalar weight_grad_max_l1_norm = 0,
+			Scalar weight_grad_max_l2_norm = 0, ParamRegSharedPtr<Scalar> bias_reg = nullptr, Scalar bias_clip = 0,
+			Scalar bias_max_l1_norm = 0, Scalar bias_max_l2_norm = 0, Scalar bias_grad_clip = 0,
+			Scalar bias_grad_max_l1_norm = 0, Scalar bias_grad_max_l2_norm = 0) :
+				TransBase(input_dims, typename TransBase::Geometry{ filters, receptor_height, receptor_width, vertical_padding,
+						horizontal_padding, vertical_stride, horizontal_stride, vertical_dilation, horizontal_dilation },
+						std::make_shared<StandardParameters<Scalar>>(detail::extended<typename Root::Dims,Rank>(input_dims)[2],
+								receptor_height * receptor_width * filters, true, weight_init, weight_reg, weight_clip,
+								weight_max_l1_norm, weight_max_l2_norm, weight_grad_clip, weight_grad_max_l1_norm,
+								weight_grad_max_l2_norm),
+						std::make_shared<StandardParameters<Scalar>>(1, TransBase::output_dims_for(input_dims,
+								typename TransBase::Geometry{ filters, receptor_height, receptor_width, vertical_padding,
+										horizontal_padding, vertical_stride, horizontal_stride, vertical_dilation,
+										horizontal_dilation }).get_volume(), true,
+								std::make_shared<ZeroParameterInitialization<Scalar>>(), bias_reg, bias_clip, bias_max_l1_norm,
+								bias_max_l2_norm, bias_grad_clip, bias_grad_max_l1_norm, bias_grad_max_l2_norm)) {
+		static_assert(Rank == 2 || Rank == 3, "rank 1 has its own constructor");
+	}
+};
+
+/** Rank 1: the constructor of TransConvKernelLayer<Scalar,1> (TransConvKernelLayer.hpp:482-495). */
+template<typename Scalar>
+class TransConvKernelHIPLayer<Scalar,1> : public TransConvKernelHIPLayerBase<Scalar,1> {
+	typedef Layer<Scalar,1> Root;
+	typedef TransConvKernelHIPLayerBase<Scalar,1> TransBase;
+public:
+	inline TransConvKernelHIPLayer(const typename Root::Dims& input_dims, std::size_t filters,
+			ParamInitSharedPtr<Scalar> weight_init, std::size_t receptor_length = 3, std::size_t padding = 1,
+			std::size_t stride = 1, std::size_t dilation = 0, ParamRegSharedPtr<Scalar> weight_reg = nullptr,
+			Scalar weight_clip = 0, Scalar weight_max_l1_norm = 0, Scalar weight_max_l2_norm = 0,
+			Scalar weight_grad_clip = 0, Scalar weight_grad_max_l1_norm = 0, Scalar weight_grad_max_l2_norm = 0,
+			ParamRegSharedPtr<Scalar> bias_reg = nullptr, Scalar bias_clip = 0, Scalar bias_max_l1_norm = 0,
+			Scalar bias_max_l2_norm = 0, Scalar bias_grad_clip = 0, Scalar bias_grad_max_l1_norm = 0,
+			Scalar bias_grad_max_l2_norm = 0) :
+				TransBase(input_dims, typename TransBase::Geometry{ filters, receptor_length, 1, padding, 0, stride, 1, dilation, 0 },
+						std::make_shared<StandardParameters<Scalar>>(1, receptor_length * filters, true, weight_init, weight_reg,
+								weight_clip, weight_max_l1_norm, weight_max_l2_norm, weight_grad_clip, weight_grad_max_l1_norm,
+								weight_grad_max_l2_norm),
+						std::make_shared<StandardParameters<Scalar>>(1, TransBase::output_dims_for(input_dims,
+								typename TransBase::Geometry{ filters, receptor_length, 1, padding, 0, stride, 1, dilation, 0 })
+								.get_volume(), true, std::make_shared<ZeroParameterInitialization<Scalar>>(), bias_reg, bias_clip,
+								bias_max_l1_norm, bias_max_l2_norm, bias_grad_clip, bias_grad_max_l1_norm, bias_grad_max_l2_norm)) { }
 };
 
 /** Drop-in for DenseKernelLayer<Scalar,Rank> (layer/kernel/DenseKernelLayer.hpp:27-120). */

@@ -118,6 +118,35 @@ static void run(const std::string& tag) {
 		if (deep->is_shared_params_clone() || deep->get_params()[0] == conv.get_params()[0])
 			throw std::runtime_error("clone must copy the parameters");
 	}
+	/* 1b. transposed convolution, the rank-3 geometry of test/gradient_test.cpp:201, and its rank-1 form (:194) */
+	{
+		hip::TransConvKernelHIPLayer<Scalar,3> trans({ 2u, 3u, 2u }, 5, nullptr, 5, 3, 1, 0, 1, 2, 0, 1);
+		init_params(trans);
+		randomize(*trans.get_params()[0], g, 0.5);
+		randomize(*trans.get_params()[1], g, 0.5);
+		if (trans.get_output_dims()(0) != 4 || trans.get_output_dims()(1) != 9 || trans.get_output_dims()(2) != 5)
+			throw std::runtime_error("transposed convolution output dims");
+		auto x = random_tensor<Scalar,4>({ { N, 2, 3, 2 } }, g);
+		record(tag + "trans.x", x);
+		record(tag + "trans.w", trans.get_params()[0]->get_values());
+		record(tag + "trans.b", trans.get_params()[1]->get_values());
+		auto out = trans.pass_forward(x, true);
+		record(tag + "trans.out", out);
+		auto go = random_tensor<Scalar,4>(out.dimensions(), g);
+		record(tag + "trans.go", go);
+		record(tag + "trans.dx", trans.pass_back(go));
+		record(tag + "trans.dw", trans.get_params()[0]->get_grad());
+		record(tag + "trans.db", trans.get_params()[1]->get_grad());
+		hip::TransConvKernelHIPLayer<Scalar,1> trans1({ 16u }, 5, nullptr, 4, 1, 1, 1);
+		init_params(trans1);
+		randomize(*trans1.get_params()[0], g, 0.5);
+		if (trans1.get_output_dims()(0) != 100)
+			throw std::runtime_error("rank-1 transposed convolution output dims");
+		auto x1 = random_tensor<Scalar,2>({ { N, 16 } }, g);
+		record(tag + "trans1.x", x1);
+		record(tag + "trans1.w", trans1.get_params()[0]->get_values());
+		record(tag + "trans1.out", trans1.pass_forward(x1, true));
+	}
 	/* 2. dense on rank-3 data */
 	{
 		hip::DenseKernelHIPLayer<Scalar,3> dense({ 4u, 4u, 2u }, 16, nullptr);

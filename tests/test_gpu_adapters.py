@@ -62,6 +62,16 @@ def test_kernel_layers(records, tag):
     assert hp.rel_err(r["conv.out"], out) < tol and hp.rel_err(r["conv.dx"], dx) < tol
     assert hp.rel_err(r["conv.dw"], dw) < tol and hp.rel_err(r["conv.db"], db) < tol
     assert hp.rel_err(r["conv.dw3"], 3 * dw) < tol        # three pass_backs accumulated in the shared Parameters
+    # transposed convolution (rank 3 with full backward, rank 1 forward)
+    tg = dict(RH=5, RW=3, pv=1, ph=0, sv=1, sh=2, dv=0, dh=1)
+    out = oracle.transconv_forward(r["trans.x"], r["trans.w"], r["trans.b"], 5, **tg)
+    dx, dw, db = oracle.transconv_backward(r["trans.x"], r["trans.w"], r["trans.go"], **tg)
+    assert hp.rel_err(r["trans.out"], out) < tol and hp.rel_err(r["trans.dx"], dx) < tol
+    assert hp.rel_err(r["trans.dw"], dw) < tol and hp.rel_err(r["trans.db"], db) < tol
+    x1 = r["trans1.x"]
+    out1 = oracle.transconv_forward(x1.reshape(x1.shape + (1, 1)), r["trans1.w"], np.zeros((1, 100)), 5, RH=4, RW=1, pv=1, ph=0,
+                                    sv=1, sh=1, dv=1, dh=0)
+    assert hp.rel_err(r["trans1.out"], out1.reshape(r["trans1.out"].shape, order="F")) < tol
     X = r["dense.x"]
     out = oracle.dense_forward(X, r["dense.w"], r["dense.b"])
     dx, dw, db = oracle.dense_backward(X, r["dense.w"], r["dense.go"].reshape(out.shape, order="F"))
