@@ -38,7 +38,9 @@ EXPORTS = [
     "cattle_hip_layer_get_param_values", "cattle_hip_layer_get_param_grad", "cattle_hip_layer_reset_param_grad",
     "cattle_hip_maxpool_indices", "cattle_hip_loss_function", "cattle_hip_loss_d_function",
     "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
-    "cattle_hip_layer_param_reset_optimizer_state",
+    "cattle_hip_layer_param_reset_optimizer_state", "cattle_hip_convlstm_create", "cattle_hip_convlstm_propagate",
+    "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
+    "cattle_hip_convlstm_get_kernel_grad",
 ]
 
 
@@ -401,6 +403,111 @@ class TransConvKernelLayer(Layer):
         OH, OW, F = int(od[0]), int(od[1]), int(od[2])
         out = {3: (OH, OW, F), 2: (OH, OW * F), 1: (OH * F,)}[rank]
         Layer.__init__(self, h, dtype, tuple(input_dims), out)
+
+
+class _LstmKernelParameters(object):
+    """The weights or the bias of one of the eight kernels of a ConvLSTMNetwork: a block of columns of a fused parameter."""
+
+    def __init__(self, net, kernel, bias, rows, cols):
+        self._net, self._kernel, self._bias, self._rows, self._cols = net, kernel, int(bias), rows, cols
+
+    def get_rows(self):
+        return self._rows
+
+    def get_cols(self):
+        return self._cols
+
+    def are_optimizable(self):
+        return True
+
+    def _get(self, fn):
+        a = np.empty((self._rows, self._cols), dtype=self._net.dtype, order="F")
+        _check(fn(self._net._h, _sz(self._kernel), ctypes.c_int(self._bias), ctypes.c_void_p(a.ctypes.data), HOST))
+        return a
+
+    def get_values(self):
+        return self._get(lib().cattle_hip_convlstm_get_kernel_values)
+
+    def get_grad(self):
+        return self._get(lib().cattle_hip_convlstm_get_kernel_grad)
+
+    def set_values(self, values):
+        a = np.asfortranarray(values, dtype=self._net.dtype)
+        if a.shape != (self._rows, self._cols):
+            raise ValueError("expected a %dx%d matrix" % (self._rows, self._cols))
+        _check(lib().cattle_hip_convlstm_set_kernel_values(self._net._h, _sz(self._kernel), ctypes.c_int(self._bias),
+                                                           ctypes.c_void_p(a.ctypes.data), HOST))
+
+
+class ConvLSTMNetwork(Layer):
+    """LSTMNeuralNetwork<Scalar,3> over eight ConvKernelLayers with fused gates
+    (neural_network/LSTMNeuralNetwork.hpp:27-120, :236-503). activations: forget, write, candidate, state, read.
+    output_seq_size_func maps the input sequence length to (output length, output delay) (:60-63)."""
+
+    KERNELS = ("input_forget", "output_forget", "input_write", "output_write", "input_candidate", "output_candidate",
+               "input_read", "output_read")
+
+    def __init__(self, dtype, input_dims, hidden_channels, receptor_height=3, receptor_width=3, vertical_padding=1,
+                 horizontal_padding=1, vertical_dilation=0, horizontal_dilation=0,
+                 activations=("sigmoid", "sigmoid", "tanh", "tanh", "sigmoid"), activation_params=(0, 0, 0, 0, 0),
+                 output_seq_size_func=lambda input_seq_length: (input_seq_length, 0), foremost=True):
+        H, W, C = (int(d) for d in input_dims)
+        kinds = (ctypes.c_int * 5)(*[ACT[a] for a in activations])
+        params = (ctypes.c_double * 5)(*[float(p) for p in activation_params])
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_convlstm_create(_dtype_code(dtype), _sz(H), _sz(W), _sz(C), _sz(hidden_channels),
+                                                _sz(receptor_height), _sz(receptor_width), _sz(vertical_padding),
+                                                _sz(horizontal_padding), _sz(vertical_dilation), _sz(horizontal_dilation),
+                                                kinds, params, ctypes.c_int(int(foremost)), ctypes.byref(h)))
+        Layer.__init__(self, h, dtype, (H, W, C), (H, W, int(hidden_channels)))
+        self._seq = output_seq_size_func
+        self._foremost = bool(foremost)
+        self._rv = (receptor_height * receptor_width * C, receptor_height * receptor_width * int(hidden_channels))
+        self._hidden = int(hidden_channels)
+        self._in_seq_shape = None
+
+    def is_foremost(self):
+        return self._foremost
+
+    def kernel_params(self, kernel):
+        """(weights, bias) of kernel `kernel` (an index or a name of KERNELS)."""
+        k = self.KERNELS.index(kernel) if isinstance(kernel, str) else int(kernel)
+        return (_LstmKernelParameters(self, k, False, self._rv[k % 2], self._hidden),
+                _LstmKernelParameters(self, k, True, 1, self._hidden))
+
+    def propagate(self, x, training=True):
+        """x: (N, T, H, W, C) numpy array or DeviceTensor; returns the same kind, (N, T_out, H, W, hidden)."""
+        dev = isinstance(x, DeviceTensor)
+        if not dev:
+            x = np.asfortranarray(x, dtype=self.dtype)
+        self._expect(x.shape[2:], self._in_shape, "input")
+        N, T = x.shape[0], x.shape[1]
+        out_len, delay = self._seq(T)
+        shape = (N, out_len) + self._out_shape
+        out = DeviceTensor(shape, self.dtype) if dev else np.empty(shape, dtype=self.dtype, order="F")
+        ptr = (lambda t: t.ptr) if dev else (lambda a: ctypes.c_void_p(a.ctypes.data))
+        space = DEVICE if dev else HOST
+        _check(lib().cattle_hip_convlstm_propagate(self._h, ptr(x), space, _sz(N), _sz(T), _sz(out_len), _sz(delay),
+                                                   ctypes.c_int(int(training)), ptr(out), space))
+        self._in_seq_shape = tuple(x.shape)
+        self._keep = (x, out)
+        return out
+
+    def backpropagate(self, out_grad):
+        """Returns the input gradient (N, T, H, W, C), or None when the network is foremost."""
+        dev = isinstance(out_grad, DeviceTensor)
+        if not dev:
+            out_grad = np.asfortranarray(out_grad, dtype=self.dtype)
+        space = DEVICE if dev else HOST
+        ptr = (lambda t: t.ptr) if dev else (lambda a: ctypes.c_void_p(a.ctypes.data))
+        if self._foremost:
+            dx = None
+        elif dev:
+            dx = DeviceTensor(self._in_seq_shape, self.dtype)
+        else:
+            dx = np.empty(self._in_seq_shape, dtype=self.dtype, order="F")
+        _check(lib().cattle_hip_convlstm_backpropagate(self._h, ptr(out_grad), space, None if dx is None else ptr(dx), space))
+        return dx
 
 
 class DenseKernelLayer(Layer):

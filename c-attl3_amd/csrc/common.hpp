@@ -125,6 +125,17 @@ template<typename T> void add_row_vector(int N, size_t V, const T* row, T* x);
 /* row[e] += sum_n x[n + N*e]  (column sums of an N x V matrix, accumulated) */
 template<typename T> void accumulate_column_sums(int N, size_t V, const T* x, T* row);
 
+/* The element-wise part of an LSTM cell step between the kernel layers. kind/param index: 0 forget,
+ * 1 write, 2 candidate, 3 state, 4 read activation (element-wise kinds only). Per-step tensors hold
+ * the four gates as consecutive blocks of P elements; `*_all` tensors are (N, T, ...) over all steps. */
+template<typename T> struct LstmActs { int kind[5]; T param[5]; };
+template<typename T> void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int zx_T, int zx_t,
+		const T* zh, const T* prev_state, T* z, T* gates, T* state, T* act_state, T* hidden, T* hprev_all, int h_T, int h_t,
+		T* out, int out_T, int out_t);
+template<typename T> void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, const T* out_grad, int og_T,
+		int og_t, const T* z, const T* gates, const T* prev_state, const T* state, const T* act_state, T* state_grad, T* dz,
+		T* dzx_all, int x_T, int x_t, T* dzh_all, int h_T, int h_t);
+
 /* Losses and optimizer updates (train_kernels.hip). A batch is N samples x T_steps x V elements,
  * column-major with the sample index fastest. */
 enum { LOSS_SQUARED = 0, LOSS_SOFTMAX_CROSS_ENTROPY = 1 };

@@ -298,6 +298,160 @@ struct TransConvLayer : LayerBase {
 	}
 };
 
+/* A convolutional LSTM on the device: LSTMNeuralNetwork<Scalar,3,false,false>
+ * (neural_network/LSTMNeuralNetwork.hpp:236-503, no multiplicative integration, not stateful, not
+ * reversed) whose eight kernels are ConvKernelLayers of one receptor geometry that keep the spatial
+ * dimensions (stride 1, output dims = state dims as the constructor asserts, :88-101).
+ *
+ * The four kernels applied to the same tensor are run as ONE convolution with 4*hidden filters
+ * (weights [K x 4*hidden] = [forget | write | candidate | read]; channels are the slowest rank, so
+ * the four results are consecutive blocks of the output), and the input-side kernels of all time
+ * steps as one launch over a batch of N*T (the sequence tensor (N,T,H,W,C) is that batch as it
+ * lies in memory). Gate activations, state update and hidden output of a step are one kernel. The
+ * backward pass mirrors it: per step one element-wise kernel and one input-gradient launch for the
+ * recurrent kernels; the weight gradients of all steps in two launches at the end.
+ *
+ * params: 0 = input-side weights [9*C x 4*hidden], 1 = input-side bias [1 x 4*hidden],
+ *         2 = output-side (recurrent) weights [9*hidden x 4*hidden], 3 = output-side bias. */
+template<typename T>
+struct ConvLstm : LayerBase {
+	ConvShape sx, sh;               /* input-side and output-side fused convolutions */
+	int hidden;
+	LstmActs<T> acts;
+	bool foremost;
+	/* alignment of the last propagate (:398-401) */
+	size_t T_in = 0, T_out = 0, delay = 0, steps = 0;
+	const T* x_cache = nullptr;
+	DevBuf zx_all, zh, z, gates, state, act_state, hid, hprev_all, dzx_all, dzh_all, dz, dh, state_grad, partials;
+	DevBuf seq_in_stage, seq_out_stage, seq_og_stage, seq_ig_stage;
+
+	ConvLstm(int dtype, const ConvShape& x_shape, const ConvShape& h_shape, const LstmActs<T>& acts, bool foremost) :
+			LayerBase(dtype), sx(x_shape), sh(h_shape), hidden(x_shape.F / 4), acts(acts), foremost(foremost) {
+		in_dims[0] = (size_t) sx.H; in_dims[1] = (size_t) sx.W; in_dims[2] = (size_t) sx.C;
+		out_dims[0] = (size_t) sx.H; out_dims[1] = (size_t) sx.W; out_dims[2] = (size_t) hidden;
+		input_layer = foremost;
+		params.push_back(std::make_shared<Param>((size_t) sx.K(), (size_t) sx.F, true, sizeof(T)));
+		params.push_back(std::make_shared<Param>(1, (size_t) sx.F, true, sizeof(T)));
+		params.push_back(std::make_shared<Param>((size_t) sh.K(), (size_t) sh.F, true, sizeof(T)));
+		params.push_back(std::make_shared<Param>(1, (size_t) sh.F, true, sizeof(T)));
+	}
+	ConvLstm(const ConvLstm& o, bool share) : LayerBase(o.dtype), sx(o.sx), sh(o.sh), hidden(o.hidden), acts(o.acts),
+			foremost(o.foremost) {
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new ConvLstm(*this, share);
+	}
+	void forward(const void*, size_t, bool, void*) override {
+		throw Error(ERR_STATE, "a recurrent network takes sequences: use cattle_hip_convlstm_propagate");
+	}
+	void backward(const void*, size_t, void*) override {
+		throw Error(ERR_STATE, "a recurrent network takes sequences: use cattle_hip_convlstm_backpropagate");
+	}
+	size_t P(size_t N) const {            /* state elements of one step */
+		return N * out_volume();
+	}
+	T* step(DevBuf& b, size_t t, size_t per_step) {
+		return (T*) b.p + t * per_step;
+	}
+	/* propagate (:236-403): input (N, T_in, H, W, C) -> out (N, T_out, H, W, hidden), both on the device */
+	void propagate(const T* input, size_t N, size_t in_len, size_t out_len, size_t out_delay, T* out) {
+		const int n = checked_int(N, "batch size");
+		const size_t total = std::max(in_len, out_len + out_delay);      /* :245-246 */
+		const size_t p = P(N), e = sizeof(T);
+		checked_int(N * std::max(in_len, total), "batch size times sequence length");
+		T_in = in_len; T_out = out_len; delay = out_delay; steps = total;
+		/* all input-side kernels of all time steps: one convolution over a batch of N * T_in */
+		Param& wx = *params[0];
+		Param& wh = *params[2];
+		{
+			const ConvWorkspace ws = conv_workspace<T>(sx, (int) (N * in_len));
+			T* wt = (T*) wx.derived[0].ensure(ws.wt_fwd * e);
+			conv_forward<T>(sx, (int) (N * in_len), input, (const T*) wx.values.p, (const T*) params[1]->values.p,
+					(T*) zx_all.ensure(4 * p * in_len * e), wt, wx.derived_version[0] == wx.version);
+			wx.derived_version[0] = wx.version;
+		}
+		z.ensure(4 * p * total * e);
+		gates.ensure(4 * p * total * e);
+		state.ensure(p * total * e);
+		act_state.ensure(p * total * e);
+		hid.ensure(p * total * e);
+		zh.ensure(4 * p * e);
+		/* slab t of hprev_all is the hidden output of step t - 1 (slab 0 stays zero: no previous output) */
+		fill_zero(hprev_all.ensure(p * total * e), p * total * e);
+		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
+		T* wth = (T*) wh.derived[0].ensure(wsh.wt_fwd * e);
+		for (size_t t = 0; t < total; ++t) {
+			const bool has_in = t < in_len, has_prev = t > 0;
+			if (has_prev) {
+				conv_forward<T>(sh, n, step(hid, t - 1, p), (const T*) wh.values.p, (const T*) params[3]->values.p, (T*) zh.p,
+						wth, wh.derived_version[0] == wh.version);
+				wh.derived_version[0] = wh.version;
+			}
+			const bool emits = t >= out_delay && t < out_delay + out_len;      /* :386-393 */
+			lstm_gates_forward<T>(acts, n, p, has_in ? (const T*) zx_all.p : nullptr, (int) in_len, (int) t,
+					has_prev ? (const T*) zh.p : nullptr, has_prev ? step(state, t - 1, p) : nullptr, step(z, t, 4 * p),
+					step(gates, t, 4 * p), step(state, t, p), step(act_state, t, p), step(hid, t, p),
+					t + 1 < total ? (T*) hprev_all.p : nullptr, (int) total, (int) (t + 1), emits ? out : nullptr, (int) out_len,
+					(int) (t - out_delay));
+		}
+		x_cache = input;
+		batch = N;
+		have_forward = true;
+	}
+	/* backpropagate (:404-503): out_grad (N, T_out, H, W, hidden) -> in_grad (N, T_in, H, W, C), null if foremost */
+	void backpropagate(const T* out_grad, T* in_grad) {
+		CATTLE_HIP_REQUIRE(have_forward && x_cache != nullptr, "backpropagate without a matching propagate");
+		const size_t N = batch, p = P(N), e = sizeof(T), total = steps;
+		const int n = (int) N;
+		Param& wx = *params[0];
+		Param& wh = *params[2];
+		fill_zero(state_grad.ensure(p * e), p * e);                      /* :422-425 */
+		dz.ensure(4 * p * e);
+		dh.ensure(p * e);
+		dzx_all.ensure(4 * p * T_in * e);
+		fill_zero(dzh_all.ensure(4 * p * total * e), 4 * p * total * e);
+		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
+		T* wtd = (T*) wh.derived[1].ensure(wsh.wt_dgrad * e);
+		for (size_t t = total; t-- > 0;) {
+			const bool has_in = t < T_in, has_prev = t > 0;
+			const bool emitted = t >= delay && t < delay + T_out;
+			lstm_gates_backward<T>(acts, n, p, t + 1 < total ? (const T*) dh.p : nullptr, emitted ? out_grad : nullptr,
+					(int) T_out, (int) (t - delay), step(z, t, 4 * p), step(gates, t, 4 * p),
+					has_prev ? step(state, t - 1, p) : nullptr, step(state, t, p), step(act_state, t, p), (T*) state_grad.p,
+					(T*) dz.p, has_in ? (T*) dzx_all.p : nullptr, (int) T_in, (int) t, has_prev ? (T*) dzh_all.p : nullptr,
+					(int) total, (int) t);
+			if (has_prev) {
+				/* the four output-side kernels' pass_back, summed (:470-473, :491-494): one input-gradient launch */
+				conv_input_gradient<T>(sh, n, (const T*) wh.values.p, (const T*) dz.p, (T*) dh.p, wtd,
+						wh.derived_version[1] == wh.version);
+				wh.derived_version[1] = wh.version;
+			}
+		}
+		/* parameter gradients of all steps at once: slab 0 of dzh_all and of hprev_all is zero */
+		if (total > 1) {
+			const ConvWorkspace ws = conv_workspace<T>(sh, (int) (N * total));
+			conv_weight_gradient<T>(sh, (int) (N * total), (const T*) hprev_all.p, (const T*) dzh_all.p, (T*) wh.grad.p,
+					(T*) params[3]->grad.p, (T*) partials.ensure(ws.partials * e));
+		}
+		{
+			const ConvWorkspace ws = conv_workspace<T>(sx, (int) (N * T_in));
+			conv_weight_gradient<T>(sx, (int) (N * T_in), x_cache, (const T*) dzx_all.p, (T*) wx.grad.p, (T*) params[1]->grad.p,
+					(T*) partials.ensure(ws.partials * e));
+			if (in_grad) {
+				T* wt = (T*) wx.derived[1].ensure(ws.wt_dgrad * e);
+				conv_input_gradient<T>(sx, (int) (N * T_in), (const T*) wx.values.p, (const T*) dzx_all.p, in_grad, wt,
+						wx.derived_version[1] == wx.version);
+				wx.derived_version[1] = wx.version;
+			}
+		}
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		x_cache = nullptr;
+	}
+};
+
 template<typename T>
 struct BatchNormLayer : LayerBase {
 	bool per_last_rank;
@@ -576,6 +730,55 @@ Param& optimizable_param(cattle_hip_layer_t layer, size_t index) {
 }
 
 
+template<typename T>
+void convlstm_propagate(ConvLstm<T>* l, const void* input, int in_space, size_t batch, size_t in_len, size_t out_len,
+		size_t delay, void* out, int out_space) {
+	const size_t in_bytes = batch * in_len * l->in_volume() * sizeof(T), out_bytes = batch * out_len * l->out_volume() * sizeof(T);
+	const void* in_dev = input;
+	if (in_space == CATTLE_HIP_HOST) {
+		copy_in(l->seq_in_stage.ensure(in_bytes), input, CATTLE_HIP_HOST, in_bytes);
+		in_dev = l->seq_in_stage.p;
+	}
+	void* out_dev = out_space == CATTLE_HIP_HOST ? l->seq_out_stage.ensure(out_bytes) : out;
+	l->have_forward = false;
+	l->propagate((const T*) in_dev, batch, in_len, out_len, delay, (T*) out_dev);
+	if (out_space == CATTLE_HIP_HOST)
+		copy_out(out, CATTLE_HIP_HOST, out_dev, out_bytes);
+}
+
+template<typename T>
+void convlstm_backpropagate(ConvLstm<T>* l, const void* out_grad, int og_space, void* in_grad, int ig_space) {
+	if (!l->have_forward)
+		throw Error(ERR_STATE, "backpropagate without a matching propagate");
+	const size_t og_bytes = l->batch * l->T_out * l->out_volume() * sizeof(T), ig_bytes = l->batch * l->T_in * l->in_volume() * sizeof(T);
+	const void* og_dev = out_grad;
+	if (og_space == CATTLE_HIP_HOST) {
+		copy_in(l->seq_og_stage.ensure(og_bytes), out_grad, CATTLE_HIP_HOST, og_bytes);
+		og_dev = l->seq_og_stage.p;
+	}
+	void* ig_dev = nullptr;
+	if (in_grad)
+		ig_dev = ig_space == CATTLE_HIP_HOST ? l->seq_ig_stage.ensure(ig_bytes) : in_grad;
+	l->backpropagate((const T*) og_dev, (T*) ig_dev);
+	if (in_grad && ig_space == CATTLE_HIP_HOST)
+		copy_out(in_grad, CATTLE_HIP_HOST, ig_dev, ig_bytes);
+}
+
+/* kernel index in the order of LSTMNeuralNetwork::populate_layer_vector (:521-529): input_forget, output_forget,
+ * input_write, output_write, input_candidate, output_candidate, input_read, output_read; `bias` picks the bias.
+ * Returns the fused parameter and the byte range of the kernel's block of columns in it. */
+Param& lstm_kernel_param(cattle_hip_layer_t lstm, size_t kernel, int bias, size_t& offset, size_t& bytes) {
+	LayerBase* l = as_layer(lstm);
+	CATTLE_HIP_REQUIRE(dynamic_cast<ConvLstm<float>*>(l) || dynamic_cast<ConvLstm<double>*>(l), "not a ConvLSTM handle");
+	CATTLE_HIP_REQUIRE(kernel < 8, "kernel index out of range");
+	Param& p = *l->params[(kernel % 2) * 2 + (bias ? 1 : 0)];
+	const size_t gate = kernel / 2, block = p.rows * (p.cols / 4);
+	offset = gate * block * p.esize;
+	bytes = block * p.esize;
+	return p;
+}
+
+
 } /* namespace */
 
 hipStream_t stream() {
@@ -749,6 +952,129 @@ int cattle_hip_transconv_create(cattle_hip_dtype dtype, size_t height, size_t wi
 		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new TransConvLayer<float>(dtype, c) :
 				(LayerBase*) new TransConvLayer<double>(dtype, c);
 		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_convlstm_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, size_t hidden_channels,
+		size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_dilation, size_t horizontal_dilation, const int activation_kinds[5], const double activation_params[5],
+		int foremost, cattle_hip_layer_t* lstm) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(lstm != nullptr && activation_kinds != nullptr, "null pointer argument");
+		CATTLE_HIP_REQUIRE(height > 0 && width > 0 && channels > 0 && hidden_channels > 0, "dimensions must be positive");
+		CATTLE_HIP_REQUIRE(receptor_height > 0 && receptor_width > 0, "receptor dimensions must be positive");
+		const size_t lim = 1u << 20;
+		CATTLE_HIP_REQUIRE(height < lim && width < lim && channels < lim && hidden_channels < lim / 4 && receptor_height < lim &&
+				receptor_width < lim && vertical_padding < lim && horizontal_padding < lim && vertical_dilation < lim &&
+				horizontal_dilation < lim, "dimension too large");
+		CATTLE_HIP_REQUIRE(receptor_height * receptor_width * std::max(channels, hidden_channels) <= 2147483647u / 8,
+				"receptor volume too large");
+		for (int i = 0; i < 5; ++i)
+			CATTLE_HIP_REQUIRE(activation_kinds[i] >= CATTLE_HIP_ACT_IDENTITY && activation_kinds[i] <= CATTLE_HIP_ACT_SWISH,
+					"the cell's activations must be element-wise kinds");
+		ConvShape x = { (int) height, (int) width, (int) channels, (int) (4 * hidden_channels), (int) receptor_height,
+				(int) receptor_width, (int) vertical_padding, (int) horizontal_padding, 1, 1, (int) vertical_dilation,
+				(int) horizontal_dilation };
+		/* every kernel's output dims must be the state dims (LSTMNeuralNetwork.hpp:88-101) */
+		const size_t drh = receptor_height + (receptor_height - 1) * vertical_dilation;
+		const size_t drw = receptor_width + (receptor_width - 1) * horizontal_dilation;
+		CATTLE_HIP_REQUIRE(height + 2 * vertical_padding >= drh && width + 2 * horizontal_padding >= drw &&
+				(size_t) x.OH() == height && (size_t) x.OW() == width, "the kernels must keep the spatial dimensions");
+		ConvShape h = x;
+		h.C = (int) hidden_channels;
+		LayerBase* l;
+		if (dtype == CATTLE_HIP_F32) {
+			LstmActs<float> a;
+			for (int i = 0; i < 5; ++i) {
+				a.kind[i] = activation_kinds[i];
+				a.param[i] = activation_params ? (float) activation_params[i] : 0.0f;
+			}
+			l = new ConvLstm<float>(dtype, x, h, a, foremost != 0);
+		} else {
+			LstmActs<double> a;
+			for (int i = 0; i < 5; ++i) {
+				a.kind[i] = activation_kinds[i];
+				a.param[i] = activation_params ? activation_params[i] : 0.0;
+			}
+			l = new ConvLstm<double>(dtype, x, h, a, foremost != 0);
+		}
+		*lstm = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_convlstm_propagate(cattle_hip_layer_t lstm, const void* input, cattle_hip_memspace input_space, size_t batch,
+		size_t input_seq_length, size_t output_seq_length, size_t output_seq_delay, int training, void* out,
+		cattle_hip_memspace out_space) {
+	(void) training;        /* the caches a training pass needs are always kept */
+	return guarded([&] {
+		LayerBase* l = as_layer(lstm);
+		check_space(input_space);
+		check_space(out_space);
+		CATTLE_HIP_REQUIRE(input != nullptr && out != nullptr, "null tensor buffer");
+		CATTLE_HIP_REQUIRE(batch > 0 && input_seq_length > 0, "batch size and input sequence length must be positive");
+		CATTLE_HIP_REQUIRE(output_seq_length > 0, "output sequence length must be positive");          /* :244 */
+		if (ConvLstm<float>* f = dynamic_cast<ConvLstm<float>*>(l))
+			convlstm_propagate<float>(f, input, input_space, batch, input_seq_length, output_seq_length, output_seq_delay, out,
+					out_space);
+		else if (ConvLstm<double>* d = dynamic_cast<ConvLstm<double>*>(l))
+			convlstm_propagate<double>(d, input, input_space, batch, input_seq_length, output_seq_length, output_seq_delay, out,
+					out_space);
+		else
+			throw Error(ERR_INVALID, "not a ConvLSTM handle");
+	});
+}
+
+int cattle_hip_convlstm_backpropagate(cattle_hip_layer_t lstm, const void* out_grad, cattle_hip_memspace grad_space,
+		void* in_grad, cattle_hip_memspace in_grad_space) {
+	return guarded([&] {
+		LayerBase* l = as_layer(lstm);
+		check_space(grad_space);
+		check_space(in_grad_space);
+		CATTLE_HIP_REQUIRE(out_grad != nullptr, "null gradient buffer");
+		ConvLstm<float>* f = dynamic_cast<ConvLstm<float>*>(l);
+		ConvLstm<double>* d = dynamic_cast<ConvLstm<double>*>(l);
+		CATTLE_HIP_REQUIRE(f || d, "not a ConvLSTM handle");
+		const bool foremost = f ? f->foremost : d->foremost;
+		CATTLE_HIP_REQUIRE(foremost == (in_grad == nullptr),
+				"the input gradient buffer must be NULL exactly when the network is foremost");
+		if (f)
+			convlstm_backpropagate<float>(f, out_grad, grad_space, in_grad, in_grad_space);
+		else
+			convlstm_backpropagate<double>(d, out_grad, grad_space, in_grad, in_grad_space);
+	});
+}
+
+int cattle_hip_convlstm_set_kernel_values(cattle_hip_layer_t lstm, size_t kernel, int bias, const void* values,
+		cattle_hip_memspace space) {
+	return guarded([&] {
+		check_space(space);
+		CATTLE_HIP_REQUIRE(values != nullptr, "null buffer");
+		size_t offset, bytes;
+		Param& p = lstm_kernel_param(lstm, kernel, bias, offset, bytes);
+		copy_in((char*) p.values.p + offset, values, space, bytes);
+		++p.version;
+	});
+}
+
+int cattle_hip_convlstm_get_kernel_values(cattle_hip_layer_t lstm, size_t kernel, int bias, void* values,
+		cattle_hip_memspace space) {
+	return guarded([&] {
+		check_space(space);
+		CATTLE_HIP_REQUIRE(values != nullptr, "null buffer");
+		size_t offset, bytes;
+		Param& p = lstm_kernel_param(lstm, kernel, bias, offset, bytes);
+		copy_out(values, space, (const char*) p.values.p + offset, bytes);
+	});
+}
+
+int cattle_hip_convlstm_get_kernel_grad(cattle_hip_layer_t lstm, size_t kernel, int bias, void* grad, cattle_hip_memspace space) {
+	return guarded([&] {
+		check_space(space);
+		CATTLE_HIP_REQUIRE(grad != nullptr, "null buffer");
+		size_t offset, bytes;
+		Param& p = lstm_kernel_param(lstm, kernel, bias, offset, bytes);
+		copy_out(grad, space, (const char*) p.grad.p + offset, bytes);
 	});
 }
 

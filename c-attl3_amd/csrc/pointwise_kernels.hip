@@ -658,6 +658,120 @@ void column_sums_kernel(int N, size_t V, const T* __restrict__ x, T* __restrict_
 	}
 }
 
+/* ----------------------------------------------------------------------------------------------
+ * LSTM cell arithmetic between the kernel layers (neural_network/LSTMNeuralNetwork.hpp:283-394
+ * forward, :436-441 backward), one thread per state element. The four gates (forget, write,
+ * candidate, read) are the channel blocks of one tensor, so gate g of element e sits at g*P + e in a
+ * per-step tensor. Tensors that span all time steps are (N, T, ...) column-major: element e of step t
+ * is at n + N*(t + T*rest) with n = e % N, rest = e / N.
+ * -------------------------------------------------------------------------------------------- */
+template<typename T>
+__device__ __forceinline__ T act_f_rt(int kind, T x, T p) {
+	switch (kind) {
+	case ACT_IDENTITY: return act_f<T, ACT_IDENTITY>(x, p);
+	case ACT_SCALED: return act_f<T, ACT_SCALED>(x, p);
+	case ACT_BINARY_STEP: return act_f<T, ACT_BINARY_STEP>(x, p);
+	case ACT_SIGMOID: return act_f<T, ACT_SIGMOID>(x, p);
+	case ACT_TANH: return act_f<T, ACT_TANH>(x, p);
+	case ACT_SOFTSIGN: return act_f<T, ACT_SOFTSIGN>(x, p);
+	case ACT_SOFTPLUS: return act_f<T, ACT_SOFTPLUS>(x, p);
+	case ACT_RELU: return act_f<T, ACT_RELU>(x, p);
+	case ACT_LEAKY_RELU: return act_f<T, ACT_LEAKY_RELU>(x, p);
+	case ACT_ELU: return act_f<T, ACT_ELU>(x, p);
+	default: return act_f<T, ACT_SWISH>(x, p);
+	}
+}
+
+template<typename T>
+__device__ __forceinline__ T act_b_rt(int kind, T x, T y, T g, T p) {
+	switch (kind) {
+	case ACT_IDENTITY: return act_b<T, ACT_IDENTITY>(x, y, g, p);
+	case ACT_SCALED: return act_b<T, ACT_SCALED>(x, y, g, p);
+	case ACT_BINARY_STEP: return act_b<T, ACT_BINARY_STEP>(x, y, g, p);
+	case ACT_SIGMOID: return act_b<T, ACT_SIGMOID>(x, y, g, p);
+	case ACT_TANH: return act_b<T, ACT_TANH>(x, y, g, p);
+	case ACT_SOFTSIGN: return act_b<T, ACT_SOFTSIGN>(x, y, g, p);
+	case ACT_SOFTPLUS: return act_b<T, ACT_SOFTPLUS>(x, y, g, p);
+	case ACT_RELU: return act_b<T, ACT_RELU>(x, y, g, p);
+	case ACT_LEAKY_RELU: return act_b<T, ACT_LEAKY_RELU>(x, y, g, p);
+	case ACT_ELU: return act_b<T, ACT_ELU>(x, y, g, p);
+	default: return act_b<T, ACT_SWISH>(x, y, g, p);
+	}
+}
+
+__device__ __forceinline__ size_t seq_offset(size_t e, int N, int T_len, int t) {
+	const size_t n = e % (size_t) N, rest = e / (size_t) N;
+	return n + (size_t) N * ((size_t) t + (size_t) T_len * rest);
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void lstm_gates_forward_kernel(LstmActs<T> a, int N, size_t P, const T* __restrict__ zx, int zx_T, int zx_t,
+		const T* __restrict__ zh, const T* __restrict__ prev_state, T* __restrict__ z, T* __restrict__ gates,
+		T* __restrict__ state, T* __restrict__ act_state, T* __restrict__ hidden, T* __restrict__ hprev_all, int h_T, int h_t,
+		T* __restrict__ out, int out_T, int out_t) {
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < P; e += stride) {
+		T y[4];
+		#pragma unroll
+		for (int g = 0; g < 4; ++g) {
+			/* weighted input + weighted previous output (:312, :327, :342, :373) */
+			T v = (T) 0;
+			if (zx)
+				v = zx[seq_offset(e + g * P, N, zx_T, zx_t)];
+			if (zh)
+				v = zx ? v + zh[g * P + e] : zh[g * P + e];
+			z[g * P + e] = v;
+			const int which = g < 3 ? g : 4;                        /* kinds: forget, write, candidate, state, read */
+			y[g] = act_f_rt<T>(a.kind[which], v, a.param[which]);
+			gates[g * P + e] = y[g];
+		}
+		const T prev = prev_state ? prev_state[e] : (T) 0;
+		T s = y[0] * prev;                                          /* selective remembrance (:314) */
+		s += y[1] * y[2];                                           /* write filter * candidates (:345) */
+		state[e] = s;
+		const T as = act_f_rt<T>(a.kind[3], s, a.param[3]);
+		act_state[e] = as;
+		const T h = y[3] * as;                                      /* read filter * activated state (:383) */
+		hidden[e] = h;
+		if (hprev_all)
+			hprev_all[seq_offset(e, N, h_T, h_t)] = h;
+		if (out)
+			out[seq_offset(e, N, out_T, out_t)] = h;
+	}
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restrict__ dh, const T* __restrict__ out_grad,
+		int og_T, int og_t, const T* __restrict__ z, const T* __restrict__ gates, const T* __restrict__ prev_state,
+		const T* __restrict__ state, const T* __restrict__ act_state, T* __restrict__ state_grad, T* __restrict__ dz,
+		T* __restrict__ dzx_all, int x_T, int x_t, T* __restrict__ dzh_all, int h_T, int h_t) {
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < P; e += stride) {
+		T hg = dh ? dh[e] : (T) 0;
+		if (out_grad)
+			hg += out_grad[seq_offset(e, N, og_T, og_t)];           /* :431-438 */
+		const T f = gates[e], w = gates[P + e], c = gates[2 * P + e], r = gates[3 * P + e];
+		const T as = act_state[e];
+		const T sg = state_grad[e] + act_b_rt<T>(a.kind[3], state[e], as, r * hg, a.param[3]);      /* :440 */
+		T d[4];
+		d[3] = act_b_rt<T>(a.kind[4], z[3 * P + e], r, as * hg, a.param[4]);                       /* :441 */
+		d[2] = act_b_rt<T>(a.kind[2], z[2 * P + e], c, w * sg, a.param[2]);                        /* :442 */
+		d[1] = act_b_rt<T>(a.kind[1], z[P + e], w, c * sg, a.param[1]);                            /* :443 */
+		d[0] = act_b_rt<T>(a.kind[0], z[e], f, (prev_state ? prev_state[e] : (T) 0) * sg, a.param[0]);   /* :444 */
+		state_grad[e] = sg * f;                                                                    /* :445 */
+		#pragma unroll
+		for (int g = 0; g < 4; ++g) {
+			dz[g * P + e] = d[g];
+			if (dzx_all)
+				dzx_all[seq_offset(e + g * P, N, x_T, x_t)] = d[g];
+			if (dzh_all)
+				dzh_all[seq_offset(e + g * P, N, h_T, h_t)] = d[g];
+		}
+	}
+}
+
 void check_launch() {
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
@@ -873,6 +987,28 @@ void accumulate_column_sums(int N, size_t V, const T* x, T* row) {
 	check_launch();
 }
 
+template<typename T>
+void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int zx_T, int zx_t, const T* zh,
+		const T* prev_state, T* z, T* gates, T* state, T* act_state, T* hidden, T* hprev_all, int h_T, int h_t, T* out,
+		int out_T, int out_t) {
+	if (P == 0)
+		return;
+	lstm_gates_forward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, zx, zx_T, zx_t, zh, prev_state, z, gates, state,
+			act_state, hidden, hprev_all, h_T, h_t, out, out_T, out_t);
+	check_launch();
+}
+
+template<typename T>
+void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, const T* out_grad, int og_T, int og_t, const T* z,
+		const T* gates, const T* prev_state, const T* state, const T* act_state, T* state_grad, T* dz, T* dzx_all, int x_T,
+		int x_t, T* dzh_all, int h_T, int h_t) {
+	if (P == 0)
+		return;
+	lstm_gates_backward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, dh, out_grad, og_T, og_t, z, gates, prev_state,
+			state, act_state, state_grad, dz, dzx_all, x_T, x_t, dzh_all, h_T, h_t);
+	check_launch();
+}
+
 #define CATTLE_HIP_INSTANTIATE(T) \
 template void act_forward<T>(int, size_t, T, const T*, T*); \
 template void act_backward<T>(int, size_t, T, const T*, const T*, const T*, T*); \
@@ -891,7 +1027,11 @@ template void meanpool_backward<T>(const PoolShape&, int, const T*, T*); \
 template void axpy_one<T>(size_t, const T*, T*); \
 template void transpose_matrix<T>(int, int, const T*, T*, bool); \
 template void add_row_vector<T>(int, size_t, const T*, T*); \
-template void accumulate_column_sums<T>(int, size_t, const T*, T*);
+template void accumulate_column_sums<T>(int, size_t, const T*, T*); \
+template void lstm_gates_forward<T>(const LstmActs<T>&, int, size_t, const T*, int, int, const T*, const T*, T*, T*, T*, T*, T*, T*, int, int, \
+		T*, int, int); \
+template void lstm_gates_backward<T>(const LstmActs<T>&, int, size_t, const T*, const T*, int, int, const T*, const T*, const T*, const T*, \
+		const T*, T*, T*, T*, int, int, T*, int, int);
 
 CATTLE_HIP_INSTANTIATE(float)
 CATTLE_HIP_INSTANTIATE(double)

@@ -224,6 +224,46 @@ int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, d
 /* AdamOptimizer::_fit (optimizer/AdamOptimizer.hpp:55-65): zero the moving averages. */
 int cattle_hip_layer_param_reset_optimizer_state(cattle_hip_layer_t layer, size_t index);
 
+/* ---- Convolutional LSTM with fused gates ------------------------------------------------------
+ * LSTMNeuralNetwork<Scalar,3,false,false> (neural_network/LSTMNeuralNetwork.hpp:27-120 constructor,
+ * :236-403 propagate, :404-503 backpropagate; no multiplicative integration, not stateful, not
+ * reversed) whose eight kernels are ConvKernelLayers with `hidden_channels` filters and one receptor
+ * geometry that keeps the spatial dimensions (stride 1), and whose five activations are element-wise
+ * kinds (CATTLE_HIP_ACT_IDENTITY .. CATTLE_HIP_ACT_SWISH) given in the order forget, write, candidate,
+ * state, read with their scalar arguments (NULL = all zero). `foremost` as in the constructor (:81):
+ * a foremost network computes no input gradient.
+ *
+ * The handle is a cattle_hip_layer_t: clone/destroy, the parameter entry points and the optimizer
+ * updates work on it with FOUR fused parameters — 0: input-side weights
+ * [receptor_height*receptor_width*channels x 4*hidden_channels], column blocks forget | write |
+ * candidate | read; 1: input-side biases [1 x 4*hidden_channels]; 2, 3: the same for the
+ * output-side (recurrent) kernels, [receptor_height*receptor_width*hidden_channels x 4*hidden_channels].
+ * cattle_hip_layer_forward/backward are refused: sequences go through the two calls below. */
+int cattle_hip_convlstm_create(cattle_hip_dtype dtype, size_t height, size_t width, size_t channels, size_t hidden_channels,
+		size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_dilation, size_t horizontal_dilation, const int activation_kinds[5], const double activation_params[5],
+		int foremost, cattle_hip_layer_t* lstm);
+/* NeuralNetwork::propagate (:236-403). input is (batch, input_seq_length, height, width, channels), out
+ * (batch, output_seq_length, height, width, hidden_channels), column-major (core/NeuralNetwork.hpp:26);
+ * output_seq_length and output_seq_delay are what the network's OutputSeqSizeFunc returns for this input
+ * length (:241-243). A DEVICE input is borrowed until the matching backpropagate. */
+int cattle_hip_convlstm_propagate(cattle_hip_layer_t lstm, const void* input, cattle_hip_memspace input_space, size_t batch,
+		size_t input_seq_length, size_t output_seq_length, size_t output_seq_delay, int training, void* out,
+		cattle_hip_memspace out_space);
+/* NeuralNetwork::backpropagate (:404-503): out_grad has the shape of out; in_grad the shape of input, and is
+ * NULL exactly when the network is foremost. Kernel gradients accumulate. */
+int cattle_hip_convlstm_backpropagate(cattle_hip_layer_t lstm, const void* out_grad, cattle_hip_memspace grad_space,
+		void* in_grad, cattle_hip_memspace in_grad_space);
+/* The parameters of one of the eight kernels in the order of get_layers() (:521-529): 0 input_forget,
+ * 1 output_forget, 2 input_write, 3 output_write, 4 input_candidate, 5 output_candidate, 6 input_read,
+ * 7 output_read; bias = 0 selects the weights [receptor volume x hidden_channels], 1 the bias
+ * [1 x hidden_channels]: the kernel's block of columns of the fused parameter. */
+int cattle_hip_convlstm_set_kernel_values(cattle_hip_layer_t lstm, size_t kernel, int bias, const void* values,
+		cattle_hip_memspace space);
+int cattle_hip_convlstm_get_kernel_values(cattle_hip_layer_t lstm, size_t kernel, int bias, void* values,
+		cattle_hip_memspace space);
+int cattle_hip_convlstm_get_kernel_grad(cattle_hip_layer_t lstm, size_t kernel, int bias, void* grad, cattle_hip_memspace space);
+
 #ifdef __cplusplus
 }
 #endif

@@ -440,3 +440,94 @@ class ConvLSTM(object):
                                c["out_write"].pass_back(g_write) + c["out_forget"].pass_back(g_forget))
             for gate, g in (("read", g_read), ("candidate", g_cand), ("write", g_write), ("forget", g_forget)):
                 c["in_" + gate].pass_back(g)
+
+
+class SeqConvLSTM(object):
+    """neural_network/LSTMNeuralNetwork.hpp:236-503 in full generality of its sequence alignment: the input
+    has T_in steps, the output `out_len` steps starting after `delay` steps, the network runs
+    max(T_in, out_len + delay) steps; steps past the input run on the previous output only (:347-361), step 0
+    on the input only (:283-298). Built from per-layer objects of a backend (unrolled with shared-parameter
+    clones, :536-573), so on the oracle backend it is the CPU restatement the fused device network is checked
+    against. activations: forget, write, candidate, state, read."""
+
+    GATES = ("forget", "write", "candidate", "read")
+
+    def __init__(self, backend, dims, hidden, activations=(("sigmoid", 0), ("sigmoid", 0), ("tanh", 0), ("tanh", 0), ("sigmoid", 0)),
+                 conv_kw=None, foremost=True):
+        self.b, self.dims, self.hdims, self.foremost = backend, tuple(dims), (dims[0], dims[1], hidden), foremost
+        kw = conv_kw or {}
+        self.main = {}
+        for gate in self.GATES:
+            self.main["in_" + gate] = backend.conv(self.dims, hidden, **kw)
+            self.main["out_" + gate] = backend.conv(self.hdims, hidden, **kw)
+            self.main["in_" + gate].set_input_layer(foremost)          # :193-199
+        for gate, (kind, p) in zip(("forget", "write", "candidate", "state", "read"), activations):
+            self.main["act_" + gate] = backend.act(kind, self.hdims, p)
+        self.cells = [self.main]
+
+    def kernels(self):
+        """The eight kernels in the order of get_layers() (:521-529)."""
+        out = []
+        for gate in self.GATES:
+            out.append(self.main["in_" + gate])
+            out.append(self.main["out_" + gate])
+        return out
+
+    def propagate(self, x, out_len, delay):
+        N, T_in = x.shape[0], x.shape[1]
+        steps = max(T_in, out_len + delay)
+        while len(self.cells) < steps:
+            self.cells.append({k: v.clone_with_shared_params() for k, v in self.main.items()})
+        self.T_in, self.out_len, self.delay, self.steps = T_in, out_len, delay, steps
+        F = np.asfortranarray
+        state = np.zeros((N,) + self.hdims, dtype=x.dtype, order="F")
+        out = np.zeros((N, out_len) + self.hdims, dtype=x.dtype, order="F")
+        hidden = None
+        for i in range(steps):
+            c = self.cells[i]
+            pre = {}
+            for gate in self.GATES:
+                w = None
+                if i < T_in:
+                    w = c["in_" + gate].pass_forward(F(x[:, i]), True)
+                if i > 0:
+                    wo = c["out_" + gate].pass_forward(hidden, True)
+                    w = wo if w is None else w + wo
+                pre[gate] = F(w)
+            c["forget_f"] = c["act_forget"].pass_forward(pre["forget"], True)
+            c["prev_state"] = state
+            state = c["forget_f"] * c["prev_state"]
+            c["write_f"] = c["act_write"].pass_forward(pre["write"], True)
+            c["cand"] = c["act_candidate"].pass_forward(pre["candidate"], True)
+            state = state + c["write_f"] * c["cand"]
+            c["read_f"] = c["act_read"].pass_forward(pre["read"], True)
+            c["act_state_v"] = c["act_state"].pass_forward(F(state), True)
+            hidden = F(c["read_f"] * c["act_state_v"])
+            if delay <= i < delay + out_len:
+                out[:, i - delay] = hidden
+        return out
+
+    def backpropagate(self, out_grad):
+        F = np.asfortranarray
+        N = out_grad.shape[0]
+        state_grad = np.zeros((N,) + self.hdims, dtype=out_grad.dtype, order="F")
+        hidden_grad = np.zeros_like(state_grad)
+        in_grad = None if self.foremost else np.zeros((N, self.T_in) + self.dims, dtype=out_grad.dtype, order="F")
+        for i in range(self.steps - 1, -1, -1):
+            c = self.cells[i]
+            if self.delay <= i < self.delay + self.out_len:
+                hidden_grad = hidden_grad + out_grad[:, i - self.delay]
+            state_grad = state_grad + c["act_state"].pass_back(F(c["read_f"] * hidden_grad))
+            g_read = c["act_read"].pass_back(F(c["act_state_v"] * hidden_grad))
+            g_cand = c["act_candidate"].pass_back(F(c["write_f"] * state_grad))
+            g_write = c["act_write"].pass_back(F(c["cand"] * state_grad))
+            g_forget = c["act_forget"].pass_back(F(c["prev_state"] * state_grad))
+            state_grad = state_grad * c["forget_f"]
+            grads = (("read", g_read), ("candidate", g_cand), ("write", g_write), ("forget", g_forget))
+            if i != 0:
+                hidden_grad = sum(c["out_" + gate].pass_back(g) for gate, g in grads)
+            if i < self.T_in:
+                parts = [c["in_" + gate].pass_back(g) for gate, g in grads]
+                if not self.foremost:
+                    in_grad[:, i] = sum(parts)
+        return in_grad

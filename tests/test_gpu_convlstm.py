@@ -1,0 +1,125 @@
+"""The fused-gate convolutional LSTM on the device (one convolution per group of four kernels, all input-side
+kernels of all time steps in one launch, gate arithmetic in one kernel per step) against the per-layer
+restatement of LSTMNeuralNetwork on the CPU oracle (tests/harness.py, SeqConvLSTM), in float64 on identical
+inputs: output sequence, input gradient and all sixteen parameter gradients."""
+import importlib
+
+import numpy as np
+import pytest
+
+import harness as hn
+import helpers as hp
+
+pytestmark = pytest.mark.gpu
+
+ch = importlib.import_module("c-attl3_amd")
+
+TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-10}
+SMOOTH = (("sigmoid", 0), ("sigmoid", 0), ("tanh", 0), ("tanh", 0), ("sigmoid", 0))
+EXOTIC = (("softsign", 0), ("swish", 1.3), ("softplus", 0), ("elu", 0.7), ("scaled", 0.5))
+
+
+def _pair(dtype, dims, hidden, acts, foremost, seq, seed, conv_kw=None):
+    kw = conv_kw or {}
+    net = ch.ConvLSTMNetwork(dtype, dims, hidden, kw.get("RH", 3), kw.get("RW", 3), kw.get("pv", 1), kw.get("ph", 1),
+                             kw.get("dv", 0), kw.get("dh", 0), activations=[a for a, _ in acts],
+                             activation_params=[p for _, p in acts], output_seq_size_func=seq, foremost=foremost)
+    orc = hn.SeqConvLSTM(hn.OracleBackend(np.float64), dims, hidden, acts, conv_kw, foremost)
+    g = hp.rng(seed)
+    for k, layer in enumerate(orc.kernels()):
+        rows = layer.get_params()[0].get_values().shape[0]
+        w = hn.he_normal(g, rows, hidden, dtype)
+        b = hp.normal(g, (1, hidden), dtype, 0.1)
+        for host, dev, v in zip(layer.get_params(), net.kernel_params(k), (w, b)):
+            dev.set_values(v)
+            host.set_values(np.asarray(v, np.float64))
+            assert np.array_equal(dev.get_values(), v)
+    return net, orc, g
+
+
+def _check(dtype, N, T_in, dims, hidden, acts, foremost, seq, seed=7, conv_kw=None):
+    net, orc, g = _pair(dtype, dims, hidden, acts, foremost, seq, seed, conv_kw)
+    out_len, delay = seq(T_in)
+    x = hp.normal(g, (N, T_in) + tuple(dims), dtype)
+    go = hp.normal(g, (N, out_len, dims[0], dims[1], hidden), dtype)
+    tol = TOL[np.dtype(dtype)]
+    out = net.propagate(x)
+    ref = orc.propagate(np.asarray(x, np.float64), out_len, delay)
+    assert out.shape == ref.shape
+    assert hp.rel_err(out, ref) < tol, "output sequence"
+    dx = net.backpropagate(go)
+    dx_ref = orc.backpropagate(np.asarray(go, np.float64))
+    if foremost:
+        assert dx is None and dx_ref is None
+    else:
+        assert hp.rel_err(dx, dx_ref) < tol, "input gradient"
+    for k, layer in enumerate(orc.kernels()):
+        for which, (host, dev) in enumerate(zip(layer.get_params(), net.kernel_params(k))):
+            want = host.get_grad()
+            if np.all(want == 0):           # a kernel that never ran (no step used it)
+                assert np.all(dev.get_grad() == 0)
+            else:
+                assert hp.rel_err(dev.get_grad(), want) < tol, (net.KERNELS[k], "bias" if which else "weights")
+    return net, orc, (x, go)
+
+
+def test_config5_convlstm_fused():
+    """BASELINE config 5: T=10, batch 32, 16x16x8 input, 32 hidden channels, output = last hidden state."""
+    _check(np.float32, 32, 10, (16, 16, 8), 32, SMOOTH, True, lambda T: (1, T - 1))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("foremost", [True, False])
+def test_sequence_alignments(dtype, foremost):
+    dims, hidden = (6, 5, 3), 4
+    _check(dtype, 5, 4, dims, hidden, SMOOTH, foremost, lambda T: (T, 0))             # an output at every step
+    _check(dtype, 4, 3, dims, hidden, SMOOTH, foremost, lambda T: (4, 1))             # runs 2 steps past the input
+    _check(dtype, 4, 1, dims, hidden, SMOOTH, foremost, lambda T: (1, 0))             # a single step: no recurrent kernel runs
+    _check(dtype, 3, 5, dims, hidden, SMOOTH, foremost, lambda T: (2, 1))             # output in the middle of the sequence
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_other_activations_and_receptors(dtype):
+    _check(dtype, 4, 3, (7, 6, 2), 5, EXOTIC, False, lambda T: (T, 0), conv_kw=dict(RH=3, RW=1, pv=1, ph=0))
+    _check(dtype, 4, 3, (8, 8, 2), 3, SMOOTH, False, lambda T: (T, 0), conv_kw=dict(RH=3, RW=3, pv=2, ph=2, dv=1, dh=1))
+
+
+def test_gradients_accumulate_and_updates_apply():
+    net, orc, (x, go) = _check(np.float32, 4, 3, (6, 5, 3), 4, SMOOTH, True, lambda T: (T, 0))
+    w, b = net.kernel_params("output_write")
+    g1 = w.get_grad()
+    net.propagate(x)
+    net.backpropagate(go)
+    assert hp.rel_err(w.get_grad(), 2 * g1) < 1e-5                      # a second pass adds to the gradients
+    # the fused parameters are ordinary parameters of the handle: optimizer updates and resets work on them
+    fused = net.get_params()
+    assert [p.get_rows() for p in fused] == [27, 1, 36, 1] and all(p.get_cols() == 16 for p in fused)
+    before = w.get_values()
+    fused[2].sgd_update(0.1)
+    assert hp.rel_err(w.get_values(), np.asarray(before, np.float64) - float(np.float32(0.1)) * np.asarray(w.get_grad(), np.float64)) < 1e-5
+    for p in fused:
+        p.reset_grad()
+    assert np.all(w.get_grad() == 0) and np.all(b.get_grad() == 0)
+    # the next pass uses the updated recurrent weights (the fused update moved all four output-side kernels)
+    for k in (1, 3, 5, 7):
+        for host, dev in zip(orc.kernels()[k].get_params(), net.kernel_params(k)):
+            host.set_values(np.asarray(dev.get_values(), np.float64))
+    assert hp.rel_err(net.propagate(x), orc.propagate(np.asarray(x, np.float64), 3, 0)) < 1e-4
+
+
+def test_device_resident_sequences_and_errors():
+    net, orc, (x, go) = _check(np.float32, 4, 3, (6, 5, 3), 4, SMOOTH, False, lambda T: (T, 0))
+    host_out = net.propagate(x)
+    host_dx = net.backpropagate(go)
+    xd, gd = ch.DeviceTensor.from_host(x), ch.DeviceTensor.from_host(go)
+    assert np.array_equal(net.propagate(xd).to_host(), host_out)
+    assert np.array_equal(net.backpropagate(gd).to_host(), host_dx)
+    with pytest.raises(ch.CattleHipError):
+        net.pass_forward(x[:, 0], True)                                # sequences only
+    with pytest.raises(ch.CattleHipError):
+        ch.ConvLSTMNetwork(np.float32, (6, 5, 3), 4, 3, 3, 0, 0)       # the kernels must keep the spatial dimensions
+    with pytest.raises(ch.CattleHipError):
+        ch.ConvLSTMNetwork(np.float32, (6, 5, 3), 4, activations=("softmax", "sigmoid", "tanh", "tanh", "sigmoid"))
+    fresh = ch.ConvLSTMNetwork(np.float32, (6, 5, 3), 4)
+    with pytest.raises(ch.CattleHipError):
+        fresh.backpropagate(go)                                        # no propagate yet
