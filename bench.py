@@ -160,6 +160,42 @@ def pointwise_run(args, dtype):
     return rows
 
 
+def convlstm_run(args, dtype):
+    """BASELINE configs[4]: ConvLSTM, T=10, batch 32, 16x16x8 input, 32 hidden channels, 3x3 kernels, output = last
+    hidden state, full BPTT; one step = propagate + backpropagate on sequences resident in HBM."""
+    ch = importlib.import_module("c-attl3_amd")
+    ch.init(0)
+    N, T, H, W, C, hid = 32, 10, 16, 16, 8, 32
+    gen = np.random.default_rng(0xC0FFEE05)
+    net = ch.ConvLSTMNetwork(dtype, (H, W, C), hid, output_seq_size_func=lambda t: (1, t - 1))
+    for k in range(8):
+        w, _ = net.kernel_params(k)
+        w.set_values(he_normal(gen, w.get_rows(), hid, dtype))
+    x = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, T, H, W, C)).astype(dtype)))
+    go = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, 1, H, W, hid)).astype(dtype)))
+
+    def step():
+        net.propagate(x)
+        net.backpropagate(go)
+
+    for _ in range(args.warmup):
+        step()
+    ch.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ch.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    M = N * H * W
+    fwd = 2.0 * M * hid * 4 * (T * 9 * C + (T - 1) * 9 * hid)          # the 4+4 kernels of every step
+    flop = 2 * fwd + 2.0 * M * 4 * hid * 9 * hid * (T - 1)              # + weight gradients + recurrent input gradients
+    return {"metric": "convlstm_bptt_sequences_per_s", "value": round(N / (ms * 1e-3), 1), "unit": "sequences/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+            "dtype": args.dtype, "data": "synthetic", "gflops": round(flop / (ms * 1e-3) / 1e9, 1),
+            "config": {"workload": "ConvLSTM T=10 batch 32 16x16x8 -> 32 hidden, 3x3, propagate + BPTT (BASELINE configs[4])",
+                       "flop_per_step": flop}}
+
+
 def cpu_baseline(args, dtype):
     """Times the oracle (the restatement of the reference algorithm: explicit patch matrix + GEMMs +
     col2im, OpenMP GEMMs) on a bounded sample: the same layer at a smaller batch."""
@@ -198,8 +234,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel of x's size (for scaling rocprof byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", choices=["conv", "pointwise"], default="conv",
-                    help="conv: the headline benchmark; pointwise: HBM-bound layers, one line of per-kernel GB/s")
+    ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm"], default="conv",
+                    help="conv: the headline benchmark; pointwise: HBM-bound layers, one line of per-kernel GB/s; "
+                         "convlstm: the fused-gate ConvLSTM of BASELINE configs[4], sequences/s")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
@@ -210,6 +247,10 @@ def main():
                           "data": "synthetic", "config": {"workload": "activation / pool / batch-norm layers on a %d x 56 x 56 x 64 "
                                                                       "tensor resident in HBM" % args.batch},
                           "roofline": {"bound": "hbm", "peak": 8000.0, "unit": "GB/s"}, "kernels": rows}))
+        return
+
+    if args.workload == "convlstm":
+        print(json.dumps(convlstm_run(args, dtype)))
         return
 
     r = gpu_run(args, dtype)

@@ -671,7 +671,7 @@ int round_up(int v, int to) {
 	return (v + to - 1) / to * to;
 }
 
-constexpr int WT_ROW_PAD = 16;     /* >= every KC */
+constexpr int WT_ROW_PAD = 64;     /* a multiple of every KC: the last reduction chunk reads whole chunks of weight rows */
 constexpr int WT_COL_PAD = 128;    /* >= every BF */
 constexpr int NUM_CUS = 256;
 constexpr int LDS_PER_CU = 160 * 1024;
@@ -685,10 +685,10 @@ struct GatherVariant {
 	void (*launch)(dim3 grid, size_t dyn_lds, const T*, const T*, const T*, T*, const GatherGeom&, int mtiles, bool vec, bool divs);
 };
 
-template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F>
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
 void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g,
 		int mtiles, bool vec, bool divs) {
-	constexpr int KC = GemmCfg<T>::KC, VEC = GemmCfg<T>::VEC;
+	constexpr int VEC = GemmCfg<T>::VEC;
 	dim3 block(64 * WAVES_M * WAVES_F);
 	/* tiles per output column, if a column (N * OA rows of M) is a whole number of tiles and there are
 	 * several columns; 0 switches the 2-D walk off */
@@ -706,36 +706,43 @@ void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, con
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
-template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F>
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC = GemmCfg<T>::KC>
 GatherVariant<T> gather_variant() {
 	typedef GemmCfg<T> C;
+	static_assert(WT_ROW_PAD % KC == 0 && WAVES_F * WT_F <= WT_COL_PAD, "prepared weights are padded to whole tiles");
 	GatherVariant<T> v;
 	v.bm = WAVES_M * WT_M;
 	v.bf = WAVES_F * WT_F;
 	v.waves = WAVES_M * WAVES_F;
-	v.lds_bytes = 2 * C::KC * (v.bm + v.bf + 2 * C::pad(v.bm)) * (int) sizeof(T) + 3 * C::KC * 16;
-	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F>;
+	v.lds_bytes = 2 * KC * (v.bm + v.bf + 2 * C::pad(v.bm)) * (int) sizeof(T) + 3 * KC * 16;
+	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC>;
 	return v;
 }
 
 template<typename T> struct GatherVariants;
 template<> struct GatherVariants<float> {
-	static constexpr int COUNT = 3;
+	static constexpr int COUNT = 5, LARGE = 3;
 	static const GatherVariant<float>* get() {
 		static const GatherVariant<float> v[COUNT] = {
 			gather_variant<float, 4, 2, 64, 64>(),      /* 256 x 128 */
 			gather_variant<float, 4, 1, 64, 64>(),      /* 256 x 64 */
 			gather_variant<float, 4, 1, 64, 32>(),      /* 256 x 32 */
+			/* small problems (a few thousand rows): short tiles so that every CU gets a block, and long
+			 * reduction chunks because with one block per CU only the loads in flight hide memory latency */
+			gather_variant<float, 2, 2, 32, 32, 64>(),  /* 64 x 64 */
+			gather_variant<float, 2, 1, 32, 32, 64>(),  /* 64 x 32 */
 		};
 		return v;
 	}
 };
 template<> struct GatherVariants<double> {
-	static constexpr int COUNT = 2;
+	static constexpr int COUNT = 4, LARGE = 2;
 	static const GatherVariant<double>* get() {
 		static const GatherVariant<double> v[COUNT] = {
 			gather_variant<double, 4, 2, 64, 32>(),     /* 256 x 64 */
 			gather_variant<double, 4, 1, 64, 32>(),     /* 256 x 32 */
+			gather_variant<double, 2, 2, 32, 32, 32>(), /* 64 x 64, small problems */
+			gather_variant<double, 2, 1, 32, 32, 32>(), /* 64 x 32 */
 		};
 		return v;
 	}
@@ -751,12 +758,19 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	const bool divs = g.DA != 1 || g.DB != 1;
 	const GatherVariant<T>* vars = GatherVariants<T>::get();
 	int best_v = 0;
-	for (int i = 1; i < GatherVariants<T>::COUNT; ++i) {
+	for (int i = 1; i < GatherVariants<T>::LARGE; ++i) {
 		const bool narrower = vars[i].bf >= g.F && vars[i].bf < vars[best_v].bf;
 		/* same width, taller tile: half the A-operand loads per MFMA; worth it once it still fills the chip */
 		const bool taller = vars[i].bf == vars[best_v].bf && vars[i].bm > vars[best_v].bm && g.M >= vars[i].bm * NUM_CUS * 4;
 		if (narrower || taller)
 			best_v = i;
+	}
+	/* too few large tiles to give every CU one: take the short tiles (the narrowest that still covers F, else the widest) */
+	if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) < NUM_CUS) {
+		best_v = GatherVariants<T>::LARGE;
+		for (int i = GatherVariants<T>::LARGE + 1; i < GatherVariants<T>::COUNT; ++i)
+			if (vars[i].bf >= g.F && vars[i].bf < vars[best_v].bf)
+				best_v = i;
 	}
 	/* tuning overrides for experiments, keyed by the number of output columns F of the GEMM:
 	 * CATTLE_HIP_GATHER_VARIANT_F<F> = index into the variant table, CATTLE_HIP_GATHER_OCC_F<F> = blocks per CU
