@@ -411,6 +411,112 @@ private:
 	bool foremost;
 };
 
+/**
+ * LSTMNeuralNetwork<Scalar,3> over eight ConvKernelLayers with fused gates, on device tensors
+ * (neural_network/LSTMNeuralNetwork.hpp:27-120, :236-503; no multiplicative integration, not stateful, not
+ * reversed). Sequences are (batch, time, height, width, channels) column-major.
+ */
+template<typename Scalar>
+class DeviceConvLSTM {
+public:
+	typedef std::array<std::size_t,3> Dims;
+	/** (output sequence length, output delay) for an input sequence length: the OutputSeqSizeFunc (:60-63). */
+	typedef std::pair<std::size_t,std::size_t> (*OutputSeqSizeFunc)(std::size_t);
+	/** A sequence on the device: dims (batch, time, height, width, channels). */
+	struct Sequence {
+		std::array<std::size_t,5> dims;
+		DeviceTensor<Scalar> data;       /* stored as (batch * time, height, width, channels) */
+	};
+	/* kernels in the order of get_layers() (:521-529) */
+	enum Kernel { INPUT_FORGET = 0, OUTPUT_FORGET, INPUT_WRITE, OUTPUT_WRITE, INPUT_CANDIDATE, OUTPUT_CANDIDATE, INPUT_READ,
+		OUTPUT_READ };
+	inline DeviceConvLSTM(const Dims& input_dims, std::size_t hidden_channels, OutputSeqSizeFunc output_seq_size_func,
+			bool foremost = true, std::size_t receptor_height = 3, std::size_t receptor_width = 3,
+			std::size_t vertical_padding = 1, std::size_t horizontal_padding = 1, std::size_t vertical_dilation = 0,
+			std::size_t horizontal_dilation = 0, cattle_hip_activation forget_act = CATTLE_HIP_ACT_SIGMOID,
+			cattle_hip_activation write_act = CATTLE_HIP_ACT_SIGMOID, cattle_hip_activation candidate_act = CATTLE_HIP_ACT_TANH,
+			cattle_hip_activation state_act = CATTLE_HIP_ACT_TANH, cattle_hip_activation read_act = CATTLE_HIP_ACT_SIGMOID) :
+				handle(nullptr), input_dims(input_dims), hidden(hidden_channels), seq(output_seq_size_func), foremost(foremost),
+				batch(0), in_len(0) {
+		const int kinds[5] = { forget_act, write_act, candidate_act, state_act, read_act };
+		check(cattle_hip_convlstm_create(Code<Scalar>::value, input_dims[0], input_dims[1], input_dims[2], hidden_channels,
+				receptor_height, receptor_width, vertical_padding, horizontal_padding, vertical_dilation, horizontal_dilation,
+				kinds, nullptr, foremost ? 1 : 0, &handle));
+	}
+	DeviceConvLSTM(const DeviceConvLSTM&) = delete;
+	DeviceConvLSTM& operator=(const DeviceConvLSTM&) = delete;
+	inline ~DeviceConvLSTM() {
+		if (handle)
+			cattle_hip_layer_destroy(handle);
+	}
+	inline void set_kernel_values(Kernel kernel, bool bias, const Scalar* host_values) {
+		check(cattle_hip_convlstm_set_kernel_values(handle, (std::size_t) kernel, bias ? 1 : 0, host_values, CATTLE_HIP_HOST));
+	}
+	inline std::vector<Scalar> get_kernel_values(Kernel kernel, bool bias) const {
+		std::vector<Scalar> out(kernel_size(kernel, bias));
+		check(cattle_hip_convlstm_get_kernel_values(handle, (std::size_t) kernel, bias ? 1 : 0, out.data(), CATTLE_HIP_HOST));
+		return out;
+	}
+	inline std::vector<Scalar> get_kernel_grad(Kernel kernel, bool bias) const {
+		std::vector<Scalar> out(kernel_size(kernel, bias));
+		check(cattle_hip_convlstm_get_kernel_grad(handle, (std::size_t) kernel, bias ? 1 : 0, out.data(), CATTLE_HIP_HOST));
+		return out;
+	}
+	/** Rows of a kernel's weight matrix times hidden_channels, or hidden_channels for a bias. */
+	inline std::size_t kernel_size(Kernel kernel, bool bias) const {
+		std::size_t rows, cols;
+		int opt;
+		check(cattle_hip_layer_param_shape(handle, ((std::size_t) kernel % 2) * 2, &rows, &cols, &opt));
+		return bias ? hidden : rows * hidden;
+	}
+	/** propagate (:236-403): `input` must stay alive and unmodified until backpropagate returns. */
+	inline Sequence propagate(const Sequence& input, bool training) {
+		const std::pair<std::size_t,std::size_t> out_seq = seq(input.dims[1]);
+		Sequence out;
+		out.dims = { { input.dims[0], out_seq.first, input_dims[0], input_dims[1], hidden } };
+		out.data = DeviceTensor<Scalar>(typename DeviceTensor<Scalar>::Dims{ { input.dims[0] * out_seq.first, input_dims[0],
+				input_dims[1], hidden } });
+		check(cattle_hip_convlstm_propagate(handle, input.data.data(), CATTLE_HIP_DEVICE, input.dims[0], input.dims[1],
+				out_seq.first, out_seq.second, training ? 1 : 0, out.data.data(), CATTLE_HIP_DEVICE));
+		batch = input.dims[0];
+		in_len = input.dims[1];
+		return out;
+	}
+	/** backpropagate (:404-503): the input gradient, with a null tensor when the network is foremost. */
+	inline Sequence backpropagate(const Sequence& out_grad) {
+		Sequence grad;
+		grad.dims = { { batch, in_len, input_dims[0], input_dims[1], input_dims[2] } };
+		if (!foremost)
+			grad.data = DeviceTensor<Scalar>(typename DeviceTensor<Scalar>::Dims{ { batch * in_len, input_dims[0],
+					input_dims[1], input_dims[2] } });
+		check(cattle_hip_convlstm_backpropagate(handle, out_grad.data.data(), CATTLE_HIP_DEVICE,
+				foremost ? nullptr : grad.data.data(), CATTLE_HIP_DEVICE));
+		return grad;
+	}
+	/** Optimizer updates and gradient reset over the four fused parameters. */
+	inline void sgd_update(Scalar learning_rate) {
+		for (std::size_t i = 0; i < 4; ++i)
+			check(cattle_hip_layer_param_sgd_update(handle, i, (double) learning_rate));
+	}
+	inline void adam_update(std::size_t timestep, Scalar learning_rate = 1e-3, Scalar l1_decay = 1e-1,
+			Scalar l2_decay = 1e-3, Scalar epsilon = 1e-5) {
+		for (std::size_t i = 0; i < 4; ++i)
+			check(cattle_hip_layer_param_adam_update(handle, i, (double) learning_rate, (double) l1_decay, (double) l2_decay,
+					(double) epsilon, timestep));
+	}
+	inline void reset_grads() {
+		for (std::size_t i = 0; i < 4; ++i)
+			check(cattle_hip_layer_reset_param_grad(handle, i));
+	}
+private:
+	cattle_hip_layer_t handle;
+	Dims input_dims;
+	std::size_t hidden;
+	OutputSeqSizeFunc seq;
+	bool foremost;
+	std::size_t batch, in_len;
+};
+
 } /* namespace device */
 } /* namespace hip */
 } /* namespace cattle */

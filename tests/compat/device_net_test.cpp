@@ -149,6 +149,52 @@ static void run(const std::string& tag) {
 	}
 }
 
+static std::pair<std::size_t,std::size_t> last_two_steps(std::size_t input_seq_length) {
+	return std::make_pair((std::size_t) 2, input_seq_length - 2);
+}
+
+/* ConvLSTM: 4 steps of 5x4x3 input, 6 hidden channels, output = the last two hidden states, one SGD update. */
+template<typename Scalar>
+static void run_lstm(const std::string& tag) {
+	typedef DeviceConvLSTM<Scalar> Net;
+	Lcg g(13);
+	const std::size_t batch = 8, T = 4, H = 5, W = 4, C = 3, hid = 6;
+	Net net(typename Net::Dims{ { H, W, C } }, hid, &last_two_steps, false);
+	for (int k = 0; k < 8; ++k) {
+		const typename Net::Kernel kernel = (typename Net::Kernel) k;
+		const std::size_t rows = net.kernel_size(kernel, false) / hid;
+		std::vector<Scalar> w = random_values<Scalar>(rows * hid, g, std::sqrt(3.0 / (double) rows));
+		std::vector<Scalar> b = random_values<Scalar>(hid, g, 0.1);
+		net.set_kernel_values(kernel, false, w.data());
+		net.set_kernel_values(kernel, true, b.data());
+		record(tag + ".lstm.w" + std::to_string(k), sizeof(Scalar), { rows, hid }, w.data());
+		record(tag + ".lstm.b" + std::to_string(k), sizeof(Scalar), { 1, hid }, b.data());
+	}
+	std::vector<Scalar> x = random_values<Scalar>(batch * T * H * W * C, g, 1.0);
+	std::vector<Scalar> go = random_values<Scalar>(batch * 2 * H * W * hid, g, 1.0);
+	record(tag + ".lstm.x", sizeof(Scalar), { batch, T, H, W, C }, x.data());
+	record(tag + ".lstm.go", sizeof(Scalar), { batch, 2, H, W, hid }, go.data());
+	typename Net::Sequence in, og;
+	in.dims = { { batch, T, H, W, C } };
+	in.data = DeviceTensor<Scalar>(typename DeviceTensor<Scalar>::Dims{ { batch * T, H, W, C } }, x.data());
+	og.dims = { { batch, 2, H, W, hid } };
+	og.data = DeviceTensor<Scalar>(typename DeviceTensor<Scalar>::Dims{ { batch * 2, H, W, hid } }, go.data());
+	typename Net::Sequence out = net.propagate(in, true);
+	record(tag + ".lstm.out", sizeof(Scalar), { batch, 2, H, W, hid }, out.data.to_host().data());
+	typename Net::Sequence dx = net.backpropagate(og);
+	record(tag + ".lstm.dx", sizeof(Scalar), { batch, T, H, W, C }, dx.data.to_host().data());
+	for (int k = 0; k < 8; ++k) {
+		const typename Net::Kernel kernel = (typename Net::Kernel) k;
+		const std::size_t rows = net.kernel_size(kernel, false) / hid;
+		record(tag + ".lstm.dw" + std::to_string(k), sizeof(Scalar), { rows, hid }, net.get_kernel_grad(kernel, false).data());
+		record(tag + ".lstm.db" + std::to_string(k), sizeof(Scalar), { 1, hid }, net.get_kernel_grad(kernel, true).data());
+	}
+	net.sgd_update((Scalar) 0.05);
+	net.reset_grads();
+	record(tag + ".lstm.w3_updated", sizeof(Scalar), { net.kernel_size(Net::OUTPUT_WRITE, false) / hid, hid },
+			net.get_kernel_values(Net::OUTPUT_WRITE, false).data());
+}
+
 int main(int argc, char** argv) {
 	if (argc != 2) {
 		std::fprintf(stderr, "usage: %s <records file>\n", argv[0]);
@@ -161,6 +207,8 @@ int main(int argc, char** argv) {
 			throw std::runtime_error("cannot open the records file");
 		run<float>("f32");
 		run<double>("f64");
+		run_lstm<float>("f32");
+		run_lstm<double>("f64");
 		std::fclose(g_out);
 	} catch (const std::exception& e) {
 		std::fprintf(stderr, "device_net_test: %s\n", e.what());

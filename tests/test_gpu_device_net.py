@@ -93,3 +93,24 @@ def test_convnet_adam_batches(records, tag, tol):
     x = np.asarray(r["x"], np.float64)
     infer = net.propagate(x, False)
     assert hp.rel_err(r["infer"], infer.reshape(r["infer"].shape, order="F")) < (1e-2 if tag == "f32" else 1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-10)])
+def test_convlstm_sequence(records, tag, tol):
+    """DeviceConvLSTM: 4 input steps, the last two hidden states as output, not foremost; against the per-layer LSTM
+    on the oracle."""
+    r = {k[len(tag) + 6:]: np.asarray(v, np.float64) for k, v in records.items() if k.startswith(tag + ".lstm.")}
+    orc = hn.SeqConvLSTM(hn.OracleBackend(np.float64), (5, 4, 3), 6, foremost=False)
+    for k, layer in enumerate(orc.kernels()):
+        layer.get_params()[0].set_values(r["w%d" % k])
+        layer.get_params()[1].set_values(r["b%d" % k])
+    out = orc.propagate(np.asfortranarray(r["x"]), 2, 2)
+    assert hp.rel_err(r["out"], out) < tol
+    dx = orc.backpropagate(np.asfortranarray(r["go"]))
+    assert hp.rel_err(r["dx"], dx) < tol
+    for k, layer in enumerate(orc.kernels()):
+        assert hp.rel_err(r["dw%d" % k], layer.get_params()[0].get_grad()) < tol, k
+        assert hp.rel_err(r["db%d" % k], layer.get_params()[1].get_grad()) < tol, k
+    lr = float(np.float32(0.05)) if tag == "f32" else 0.05
+    assert hp.rel_err(r["w3_updated"], r["w3"] - lr * orc.kernels()[3].get_params()[0].get_grad()) < tol
