@@ -37,7 +37,7 @@ EXPORTS = [
     "cattle_hip_layer_num_params", "cattle_hip_layer_param_shape", "cattle_hip_layer_set_param_values",
     "cattle_hip_layer_get_param_values", "cattle_hip_layer_get_param_grad", "cattle_hip_layer_reset_param_grad",
     "cattle_hip_maxpool_indices", "cattle_hip_loss_function", "cattle_hip_loss_d_function",
-    "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
+    "cattle_hip_layer_param_optimizer_update", "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
     "cattle_hip_layer_param_reset_optimizer_state", "cattle_hip_convlstm_create", "cattle_hip_convlstm_propagate",
     "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
     "cattle_hip_convlstm_get_kernel_grad",
@@ -190,6 +190,13 @@ class Parameters(object):
     def reset_grad(self):
         _check(lib().cattle_hip_layer_reset_param_grad(self._layer._h, _sz(self._index)))
 
+    def optimizer_update(self, optimizer, hyper, epoch=0, timestep=0):
+        """<Name>Optimizer::_update_params on the device; optimizer is a key of OPTIMIZERS, hyper the reference
+        optimizer's constructor arguments in their order (see include/cattle_hip.h)."""
+        h = (ctypes.c_double * 4)(*(list(hyper) + [0.0] * (4 - len(hyper))))
+        _check(lib().cattle_hip_layer_param_optimizer_update(self._layer._h, _sz(self._index), ctypes.c_int(OPTIMIZERS[optimizer]),
+                                                             h, _sz(epoch), _sz(timestep)))
+
     def sgd_update(self, learning_rate=1e-3):
         """VanillaSGDOptimizer::_update_params on the device (optimizer/VanillaSGDOptimizer.hpp:38-43)."""
         _check(lib().cattle_hip_layer_param_sgd_update(self._layer._h, _sz(self._index), ctypes.c_double(learning_rate)))
@@ -206,6 +213,8 @@ class Parameters(object):
 
 
 LOSS = {"squared": 0, "softmax_cross_entropy": 1}
+OPTIMIZERS = {"vanilla_sgd": 0, "momentum_sgd": 1, "nesterov_momentum_sgd": 2, "adagrad": 3, "rmsprop": 4, "adadelta": 5,
+              "adam": 6, "adamax": 7, "nadam": 8, "amsgrad": 9}
 
 
 def _loss_args(out, obj, sequential):

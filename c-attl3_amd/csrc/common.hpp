@@ -142,9 +142,14 @@ enum { LOSS_SQUARED = 0, LOSS_SOFTMAX_CROSS_ENTROPY = 1 };
 template<typename T> void loss_function(int kind, int N, int T_steps, int V, T eps, const T* out, const T* obj, T* losses);
 template<typename T> void loss_d_function(int kind, int N, int T_steps, int V, T eps, T scale, const T* out, const T* obj,
 		T* grad);
-template<typename T> void sgd_update(size_t n, T lr, const T* grad, T* values);
-template<typename T> void adam_update(size_t n, T lr, T l1_decay, T l2_decay, T eps, size_t timestep, const T* grad, T* m,
-		T* v, T* values);
+/* Optimizer update rules; values equal cattle_hip_optimizer. hyper holds the constructor arguments of the
+ * reference optimizer in their order (learning rates, decays, epsilon; unused entries ignored). */
+enum { OPT_VANILLA_SGD = 0, OPT_MOMENTUM_SGD = 1, OPT_NESTEROV = 2, OPT_ADAGRAD = 3, OPT_RMSPROP = 4, OPT_ADADELTA = 5,
+	OPT_ADAM = 6, OPT_ADAMAX = 7, OPT_NADAM = 8, OPT_AMSGRAD = 9 };
+template<typename T> struct OptCoef { T c[8]; };
+int optimizer_state_count(int rule);
+template<typename T> void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n,
+		const T* grad, T* s0, T* s1, T* s2, T* values);
 
 } /* namespace cattle_hip */
 

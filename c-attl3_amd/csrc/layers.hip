@@ -100,8 +100,8 @@ struct Param {
 	uint64_t version = 1;
 	DevBuf derived[3];
 	uint64_t derived_version[3] = { 0, 0, 0 };
-	DevBuf moments[2];                 /* optimizer moving averages, allocated on first use */
-	bool moments_ready = false;
+	DevBuf moments[3];                 /* the optimizer's state matrices, allocated (zeroed) on first use */
+	int moments_ready = 0;             /* how many of them are */
 	Param(size_t rows, size_t cols, bool optimizable, size_t esize) : rows(rows), cols(cols), optimizable(optimizable), esize(esize) {
 		values.ensure(bytes());
 		grad.ensure(bytes());
@@ -1342,50 +1342,45 @@ int cattle_hip_loss_d_function(cattle_hip_dtype dtype, cattle_hip_loss kind, con
 	});
 }
 
-int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate) {
+int cattle_hip_layer_param_optimizer_update(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
+		const double hyper[4], size_t epoch, size_t timestep) {
 	return guarded([&] {
 		Param& p = optimizable_param(layer, index);
-		CATTLE_HIP_REQUIRE(learning_rate > 0, "learning rate must be positive");
+		CATTLE_HIP_REQUIRE(hyper != nullptr, "null hyper-parameter array");
+		const int states = optimizer_state_count((int) optimizer);
+		for (int i = p.moments_ready; i < states; ++i) {
+			fill_zero(p.moments[i].ensure(p.bytes()), p.bytes());
+			p.moments_ready = i + 1;
+		}
 		const size_t n = p.rows * p.cols;
 		if (p.esize == sizeof(float))
-			sgd_update<float>(n, (float) learning_rate, static_cast<const float*>(p.grad.p), static_cast<float*>(p.values.p));
+			optimizer_update<float>((int) optimizer, hyper, epoch, timestep, n, static_cast<const float*>(p.grad.p),
+					static_cast<float*>(p.moments[0].p), static_cast<float*>(p.moments[1].p), static_cast<float*>(p.moments[2].p),
+					static_cast<float*>(p.values.p));
 		else
-			sgd_update<double>(n, learning_rate, static_cast<const double*>(p.grad.p), static_cast<double*>(p.values.p));
+			optimizer_update<double>((int) optimizer, hyper, epoch, timestep, n, static_cast<const double*>(p.grad.p),
+					static_cast<double*>(p.moments[0].p), static_cast<double*>(p.moments[1].p),
+					static_cast<double*>(p.moments[2].p), static_cast<double*>(p.values.p));
 		++p.version;
 	});
 }
 
+int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate) {
+	const double hyper[4] = { learning_rate, 0, 0, 0 };
+	return cattle_hip_layer_param_optimizer_update(layer, index, CATTLE_HIP_OPT_VANILLA_SGD, hyper, 0, 0);
+}
+
 int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, double learning_rate, double l1_decay,
 		double l2_decay, double epsilon, size_t timestep) {
-	return guarded([&] {
-		Param& p = optimizable_param(layer, index);
-		CATTLE_HIP_REQUIRE(learning_rate > 0, "learning rate must be positive");
-		CATTLE_HIP_REQUIRE(l1_decay >= 0 && l1_decay <= 1 && l2_decay >= 0 && l2_decay <= 1, "decay rates must lie in [0,1]");
-		CATTLE_HIP_REQUIRE(epsilon > 0, "epsilon must be positive");
-		if (!p.moments_ready) {
-			for (int i = 0; i < 2; ++i)
-				fill_zero(p.moments[i].ensure(p.bytes()), p.bytes());
-			p.moments_ready = true;
-		}
-		const size_t n = p.rows * p.cols;
-		if (p.esize == sizeof(float))
-			adam_update<float>(n, (float) learning_rate, (float) l1_decay, (float) l2_decay, (float) epsilon, timestep,
-					static_cast<const float*>(p.grad.p), static_cast<float*>(p.moments[0].p),
-					static_cast<float*>(p.moments[1].p), static_cast<float*>(p.values.p));
-		else
-			adam_update<double>(n, learning_rate, l1_decay, l2_decay, epsilon, timestep, static_cast<const double*>(p.grad.p),
-					static_cast<double*>(p.moments[0].p), static_cast<double*>(p.moments[1].p),
-					static_cast<double*>(p.values.p));
-		++p.version;
-	});
+	const double hyper[4] = { learning_rate, l1_decay, l2_decay, epsilon };
+	return cattle_hip_layer_param_optimizer_update(layer, index, CATTLE_HIP_OPT_ADAM, hyper, 0, timestep);
 }
 
 int cattle_hip_layer_param_reset_optimizer_state(cattle_hip_layer_t layer, size_t index) {
 	return guarded([&] {
 		Param& p = param_at(as_layer(layer), index);
-		if (p.moments_ready)
-			for (int i = 0; i < 2; ++i)
-				fill_zero(p.moments[i].p, p.bytes());
+		for (int i = 0; i < p.moments_ready; ++i)
+			fill_zero(p.moments[i].p, p.bytes());
 	});
 }
 

@@ -124,30 +124,72 @@ void softmax_ce_kernel(int N, int T_steps, int V, T eps, T scale, const T* __res
 		dst[n] = total;
 }
 
-/* values -= grad * lr  (optimizer/VanillaSGDOptimizer.hpp:38-43) */
-template<typename T>
+/* The _update_params bodies of the reference's optimizers, one element per thread, in place. The
+ * scalars of a step (learning rate after annealing, bias corrections) come precomputed in `k`;
+ * s0..s2 are the optimizer's per-parameter state matrices (zero after _fit).
+ *   OPT_VANILLA_SGD   optimizer/VanillaSGDOptimizer.hpp:38-43        k: lr
+ *   OPT_MOMENTUM_SGD  optimizer/MomentumSGDOptimizer.hpp:54-63       k: lr, momentum
+ *   OPT_NESTEROV      optimizer/NesterovMomentumSGDOptimizer.hpp:43-55   k: lr, momentum
+ *   OPT_ADAGRAD       optimizer/AdaGradOptimizer.hpp:50-70           k: lr, eps
+ *   OPT_RMSPROP       optimizer/RMSPropOptimizer.hpp:43-47           k: lr, eps, l2_decay
+ *   OPT_ADADELTA      optimizer/AdaDeltaOptimizer.hpp:53-67          k: decay, eps
+ *   OPT_ADAM          optimizer/AdamOptimizer.hpp:66-82              k: d1, d2, lr * l1_corr, l2_corr, eps
+ *   OPT_ADAMAX        optimizer/AdaMaxOptimizer.hpp:44-60            k: d1, d2, lr * l1_corr, -, eps
+ *   OPT_NADAM         optimizer/NadamOptimizer.hpp:44-65             k: d1, d2, lr, l2_corr, eps, d1 * l1_corr, (1 - d1) * l1_next_corr
+ *   OPT_AMSGRAD       optimizer/AMSGradOptimizer.hpp:48-66           k: d1, d2, lr, -, eps */
+template<typename T, int RULE>
 __global__ __launch_bounds__(256)
-void sgd_update_kernel(size_t total, T lr, const T* __restrict__ grad, T* __restrict__ values) {
+void optimizer_update_kernel(size_t total, OptCoef<T> k, const T* __restrict__ grad, T* __restrict__ s0, T* __restrict__ s1,
+		T* __restrict__ s2, T* __restrict__ values) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
-	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride)
-		values[i] -= grad[i] * lr;
-}
-
-/* optimizer/AdamOptimizer.hpp:66-82:
- *   m = m (1 - d1) + g d1;  v = v (1 - d2) + g g d2;
- *   values -= (m * (lr * l1_corr)) / sqrt(v * l2_corr + eps)      (epsilon inside the root) */
-template<typename T>
-__global__ __launch_bounds__(256)
-void adam_update_kernel(size_t total, T d1, T d2, T lr_corr, T l2_corr, T eps, const T* __restrict__ grad,
-		T* __restrict__ m, T* __restrict__ v, T* __restrict__ values) {
-	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	const T one = (T) 1;
 	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
 		const T g = grad[i];
-		const T mi = m[i] * ((T) 1 - d1) + g * d1;
-		const T vi = v[i] * ((T) 1 - d2) + g * g * d2;
-		m[i] = mi;
-		v[i] = vi;
-		values[i] -= (mi * lr_corr) / dev_sqrt(vi * l2_corr + eps);
+		const T v = values[i];
+		if (RULE == OPT_VANILLA_SGD) {
+			values[i] = v - g * k.c[0];
+		} else if (RULE == OPT_MOMENTUM_SGD) {
+			const T s = s0[i] * k.c[1] + g * k.c[0];
+			s0[i] = s;
+			values[i] = v - s;
+		} else if (RULE == OPT_NESTEROV) {
+			const T old = s0[i];
+			const T s = old * k.c[1] - g * k.c[0];
+			s0[i] = s;
+			values[i] = v + old * -k.c[1] + s * (one + k.c[1]);
+		} else if (RULE == OPT_ADAGRAD || RULE == OPT_RMSPROP) {
+			const T a = RULE == OPT_ADAGRAD ? s0[i] + g * g : s0[i] * (one - k.c[2]) + g * g * k.c[2];
+			s0[i] = a;
+			values[i] = v - g * k.c[0] / (dev_sqrt(a) + k.c[1]);
+		} else if (RULE == OPT_ADADELTA) {
+			const T a = s0[i] * (one - k.c[0]) + g * g * k.c[0];
+			const T upd = -g * dev_sqrt(s1[i] + k.c[1]) / dev_sqrt(a + k.c[1]);
+			s0[i] = a;
+			values[i] = v + upd;
+			s1[i] = s1[i] * (one - k.c[0]) + upd * upd * k.c[0];
+		} else {
+			const T m = s0[i] * (one - k.c[0]) + g * k.c[0];
+			s0[i] = m;
+			if (RULE == OPT_ADAMAX) {
+				const T decayed = s1[i] * (one - k.c[1]), ag = g < (T) 0 ? -g : g;
+				const T u = decayed > ag ? decayed : ag;
+				s1[i] = u;
+				values[i] = v - (m * k.c[2]) / (u + k.c[4]);
+			} else {
+				const T sq = s1[i] * (one - k.c[1]) + g * g * k.c[1];
+				s1[i] = sq;
+				if (RULE == OPT_ADAM) {
+					values[i] = v - (m * k.c[2]) / dev_sqrt(sq * k.c[3] + k.c[4]);
+				} else if (RULE == OPT_NADAM) {
+					values[i] = v - ((g * k.c[5] + m * k.c[6]) * k.c[2]) / dev_sqrt(sq * k.c[3] + k.c[4]);
+				} else {        /* OPT_AMSGRAD */
+					const T prev = s2[i];
+					const T mx = sq > prev ? sq : prev;
+					s2[i] = mx;
+					values[i] = v - (m * k.c[2]) / dev_sqrt(mx + k.c[4]);
+				}
+			}
+		}
 	}
 }
 
@@ -200,32 +242,85 @@ void loss_d_function(int kind, int N, int T_steps, int V, T eps, T scale, const 
 	check_launch();
 }
 
-template<typename T>
-void sgd_update(size_t n, T lr, const T* grad, T* values) {
-	if (n == 0)
-		return;
-	sgd_update_kernel<T><<<flat_grid(n), 256, 0, stream()>>>(n, lr, grad, values);
-	check_launch();
+int optimizer_state_count(int rule) {
+	switch (rule) {
+	case OPT_VANILLA_SGD: return 0;
+	case OPT_MOMENTUM_SGD: case OPT_NESTEROV: case OPT_ADAGRAD: case OPT_RMSPROP: return 1;
+	case OPT_ADADELTA: case OPT_ADAM: case OPT_ADAMAX: case OPT_NADAM: return 2;
+	case OPT_AMSGRAD: return 3;
+	default: throw Error(ERR_INVALID, "unknown optimizer");
+	}
 }
 
 template<typename T>
-void adam_update(size_t n, T lr, T l1_decay, T l2_decay, T eps, size_t timestep, const T* grad, T* m, T* v,
-		T* values) {
+void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n, const T* grad, T* s0, T* s1,
+		T* s2, T* values) {
 	if (n == 0)
 		return;
-	/* the bias corrections are scalars of the step, computed in T as the reference does (:67-68) */
-	const T l1_corr = (T) 1 / ((T) 1 - (T) std::pow((T) 1 - l1_decay, (T) (timestep + 1)) + eps);
-	const T l2_corr = (T) 1 / ((T) 1 - (T) std::pow((T) 1 - l2_decay, (T) (timestep + 1)) + eps);
-	adam_update_kernel<T><<<flat_grid(n), 256, 0, stream()>>>(n, l1_decay, l2_decay, lr * l1_corr, l2_corr, eps,
-			grad, m, v, values);
+	OptCoef<T> k;
+	for (int i = 0; i < 8; ++i)
+		k.c[i] = (T) 0;
+	const T h0 = (T) hyper[0], h1 = (T) hyper[1], h2 = (T) hyper[2], h3 = (T) hyper[3];
+	const T one = (T) 1;
+	/* every scalar of the step is formed in T, as the reference forms it in Scalar */
+	switch (rule) {
+	case OPT_VANILLA_SGD:                /* hyper: learning_rate */
+		CATTLE_HIP_REQUIRE(h0 > 0, "learning rate must be positive");
+		k.c[0] = h0;
+		break;
+	case OPT_MOMENTUM_SGD: case OPT_NESTEROV:     /* hyper: init_learning_rate, annealing_rate, momentum */
+		CATTLE_HIP_REQUIRE(h0 > 0 && h1 >= 0 && h2 > 0 && h2 < 1, "momentum SGD: learning rate > 0, annealing rate >= 0, 0 < momentum < 1");
+		k.c[0] = h0 / (one + h1 * (T) epoch);       /* calculate_learning_rate (MomentumSGDOptimizer.hpp:70-72) */
+		k.c[1] = h2;
+		break;
+	case OPT_ADAGRAD:                    /* hyper: learning_rate, epsilon */
+		CATTLE_HIP_REQUIRE(h0 > 0 && h1 > 0, "AdaGrad: learning rate and epsilon must be positive");
+		k.c[0] = h0; k.c[1] = h1;
+		break;
+	case OPT_RMSPROP:                    /* hyper: learning_rate, l2_decay, epsilon */
+		CATTLE_HIP_REQUIRE(h0 > 0 && h1 >= 0 && h1 <= 1 && h2 > 0, "RMSProp: learning rate, epsilon > 0, decay in [0,1]");
+		k.c[0] = h0; k.c[1] = h2; k.c[2] = h1;
+		break;
+	case OPT_ADADELTA:                   /* hyper: decay, epsilon */
+		CATTLE_HIP_REQUIRE(h0 >= 0 && h0 <= 1 && h1 > 0, "AdaDelta: decay in [0,1], epsilon > 0");
+		k.c[0] = h0; k.c[1] = h1;
+		break;
+	case OPT_ADAM: case OPT_ADAMAX: case OPT_NADAM: case OPT_AMSGRAD: {      /* hyper: learning_rate, l1_decay, l2_decay, epsilon */
+		CATTLE_HIP_REQUIRE(h0 > 0, "learning rate must be positive");
+		CATTLE_HIP_REQUIRE(h1 >= 0 && h1 <= 1 && h2 >= 0 && h2 <= 1, "decay rates must lie in [0,1]");
+		CATTLE_HIP_REQUIRE(h3 > 0, "epsilon must be positive");
+		const T l1_corr = one / (one - (T) std::pow(one - h1, (T) (timestep + 1)) + h3);
+		const T l1_next_corr = one / (one - (T) std::pow(one - h1, (T) (timestep + 2)) + h3);
+		const T l2_corr = one / (one - (T) std::pow(one - h2, (T) (timestep + 1)) + h3);
+		k.c[0] = h1; k.c[1] = h2; k.c[3] = l2_corr; k.c[4] = h3;
+		k.c[2] = rule == OPT_ADAM || rule == OPT_ADAMAX ? h0 * l1_corr : h0;
+		k.c[5] = h1 * l1_corr;
+		k.c[6] = (one - h1) * l1_next_corr;
+		break;
+	}
+	default:
+		throw Error(ERR_INVALID, "unknown optimizer");
+	}
+	const unsigned grid = flat_grid(n);
+	switch (rule) {
+	case OPT_VANILLA_SGD: optimizer_update_kernel<T, OPT_VANILLA_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_MOMENTUM_SGD: optimizer_update_kernel<T, OPT_MOMENTUM_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_NESTEROV: optimizer_update_kernel<T, OPT_NESTEROV><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_ADAGRAD: optimizer_update_kernel<T, OPT_ADAGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_RMSPROP: optimizer_update_kernel<T, OPT_RMSPROP><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_ADADELTA: optimizer_update_kernel<T, OPT_ADADELTA><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_ADAM: optimizer_update_kernel<T, OPT_ADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_ADAMAX: optimizer_update_kernel<T, OPT_ADAMAX><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_NADAM: optimizer_update_kernel<T, OPT_NADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	default: optimizer_update_kernel<T, OPT_AMSGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	}
 	check_launch();
 }
 
 #define CATTLE_HIP_INSTANTIATE_TRAIN(T) \
 template void loss_function<T>(int, int, int, int, T, const T*, const T*, T*); \
 template void loss_d_function<T>(int, int, int, int, T, T, const T*, const T*, T*); \
-template void sgd_update<T>(size_t, T, const T*, T*); \
-template void adam_update<T>(size_t, T, T, T, T, size_t, const T*, T*, T*, T*);
+template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, const T*, T*, T*, T*, T*);
 
 CATTLE_HIP_INSTANTIATE_TRAIN(float)
 CATTLE_HIP_INSTANTIATE_TRAIN(double)

@@ -212,6 +212,30 @@ int cattle_hip_loss_d_function(cattle_hip_dtype dtype, cattle_hip_loss kind, con
 		const void* obj, cattle_hip_memspace obj_space, size_t batch, size_t time_steps, size_t sample_size,
 		double epsilon, double scale, void* grad, cattle_hip_memspace grad_space);
 
+/* The optimizers of the optimizer/ directory as in-place updates of one Parameters object on the device:
+ * <Name>Optimizer::_update_params for parameter `index` of `layer`, with the constructor arguments of
+ * the reference optimizer in `hyper` (unused entries are ignored):
+ *   VANILLA_SGD            learning_rate                                   VanillaSGDOptimizer.hpp:30-43
+ *   MOMENTUM_SGD           init_learning_rate, annealing_rate, momentum    MomentumSGDOptimizer.hpp:35-72
+ *   NESTEROV_MOMENTUM_SGD  init_learning_rate, annealing_rate, momentum    NesterovMomentumSGDOptimizer.hpp:37-55
+ *   ADAGRAD                learning_rate, epsilon                          AdaGradOptimizer.hpp:32-70
+ *   RMSPROP                learning_rate, l2_decay, epsilon                RMSPropOptimizer.hpp:34-47
+ *   ADADELTA               decay, epsilon                                  AdaDeltaOptimizer.hpp:33-67
+ *   ADAM, ADAMAX, NADAM, AMSGRAD   learning_rate, l1_decay, l2_decay, epsilon
+ *                          AdamOptimizer.hpp:40-82, AdaMaxOptimizer.hpp:39-60, NadamOptimizer.hpp:39-65, AMSGradOptimizer.hpp:39-66
+ * `epoch` is the zero-based epoch index SGDOptimizer::_train passes on (optimizer/SGDOptimizer.hpp:64: epoch - 1),
+ * used by the annealed learning rate; `timestep` the zero-based update count (:65-66), used by the bias corrections.
+ * The optimizer's state matrices (accumulated gradients, moving averages; up to three) live with the parameter
+ * on the device, start at zero and are shared between layers that share the parameter; switching optimizers
+ * calls for cattle_hip_layer_param_reset_optimizer_state (the optimizer's _fit). */
+typedef enum cattle_hip_optimizer {
+	CATTLE_HIP_OPT_VANILLA_SGD = 0, CATTLE_HIP_OPT_MOMENTUM_SGD = 1, CATTLE_HIP_OPT_NESTEROV_MOMENTUM_SGD = 2,
+	CATTLE_HIP_OPT_ADAGRAD = 3, CATTLE_HIP_OPT_RMSPROP = 4, CATTLE_HIP_OPT_ADADELTA = 5, CATTLE_HIP_OPT_ADAM = 6,
+	CATTLE_HIP_OPT_ADAMAX = 7, CATTLE_HIP_OPT_NADAM = 8, CATTLE_HIP_OPT_AMSGRAD = 9
+} cattle_hip_optimizer;
+int cattle_hip_layer_param_optimizer_update(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
+		const double hyper[4], size_t epoch, size_t timestep);
+
 /* VanillaSGDOptimizer::_update_params for one Parameters object (optimizer/VanillaSGDOptimizer.hpp:38-43):
  * values -= grad * learning_rate, in place on the device. Non-optimizable parameters are rejected. */
 int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate);
@@ -221,7 +245,7 @@ int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, do
  * layers that share the parameter) and start at zero. */
 int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, double learning_rate, double l1_decay,
 		double l2_decay, double epsilon, size_t timestep);
-/* AdamOptimizer::_fit (optimizer/AdamOptimizer.hpp:55-65): zero the moving averages. */
+/* The optimizer's _fit (e.g. optimizer/AdamOptimizer.hpp:55-65): zero the state matrices. */
 int cattle_hip_layer_param_reset_optimizer_state(cattle_hip_layer_t layer, size_t index);
 
 /* ---- Convolutional LSTM with fused gates ------------------------------------------------------

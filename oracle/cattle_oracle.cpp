@@ -22,6 +22,9 @@
  *                       the (pinned) convolution, output-size formula on the reference's test geometries.
  *   losses              pinned: torch float64 cross_entropy / mse (epsilon 0), numpy closed forms with
  *                       the epsilon, central differences of the loss against its gradient.
+ *   other optimizers    pinned: torch's SGD (momentum, Nesterov), Adagrad, RMSprop, Adadelta and Adamax where the
+ *                       recurrences coincide; first-step closed forms and the running-maximum property for
+ *                       Nadam and AMSGrad, whose reference formulas differ from torch's.
  *   SGD / Adam updates  pinned: numpy restatement in float64, first-step closed form, and torch's Adam
  *                       in the limit where the two formulas coincide.
  * What stays unpinned is only the bit pattern of Eigen's own summation order and of its
@@ -782,6 +785,78 @@ int adam_update(i64 n, T lr, T d1, T d2, T eps, i64 timestep, const T* grad, T* 
 	return 0;
 }
 
+/* The remaining optimizers' _update_params bodies (rule numbering as in the tests' front end):
+ * 1 MomentumSGDOptimizer.hpp:54-72, 2 NesterovMomentumSGDOptimizer.hpp:43-55, 3 AdaGradOptimizer.hpp:50-70,
+ * 4 RMSPropOptimizer.hpp:43-47, 5 AdaDeltaOptimizer.hpp:53-67, 7 AdaMaxOptimizer.hpp:44-60,
+ * 8 NadamOptimizer.hpp:44-65, 9 AMSGradOptimizer.hpp:48-66 (0 and 6 are the two functions above).
+ * h holds the optimizer's constructor arguments in their order; s0..s2 its state matrices. */
+template<typename T>
+int optimizer_update(int rule, const double* hd, i64 epoch, i64 timestep, i64 n, const T* grad, T* s0, T* s1, T* s2,
+		T* values) {
+	const T h0 = (T) hd[0], h1 = (T) hd[1], h2 = (T) hd[2], h3 = (T) hd[3];
+	if (rule == 0)
+		return sgd_update<T>(n, h0, grad, values);
+	if (rule == 6)
+		return adam_update<T>(n, h0, h1, h2, h3, timestep, grad, s0, s1, values);
+	if (rule == 1 || rule == 2) {
+		const T lr = h0 / (1 + h1 * epoch);
+		for (i64 i = 0; i < n; ++i) {
+			if (rule == 1) {
+				s0[i] = s0[i] * h2 + grad[i] * lr;
+				values[i] = values[i] - s0[i];
+			} else {
+				const T old = s0[i];
+				s0[i] = old * h2 - grad[i] * lr;
+				values[i] = values[i] + old * -h2 + s0[i] * (1 + h2);
+			}
+		}
+		return 0;
+	}
+	if (rule == 3 || rule == 4) {
+		const T eps = rule == 3 ? h1 : h2;
+		for (i64 i = 0; i < n; ++i) {
+			if (rule == 3)
+				s0[i] += grad[i] * grad[i];
+			else
+				s0[i] = s0[i] * (1 - h1) + grad[i] * grad[i] * h1;
+			values[i] = values[i] - grad[i] * h0 / (std::sqrt(s0[i]) + eps);
+		}
+		return 0;
+	}
+	if (rule == 5) {
+		for (i64 i = 0; i < n; ++i) {
+			s0[i] = s0[i] * (1 - h0) + grad[i] * grad[i] * h0;
+			const T upd = -grad[i] * std::sqrt(s1[i] + h1) / std::sqrt(s0[i] + h1);
+			values[i] = values[i] + upd;
+			s1[i] = s1[i] * (1 - h0) + upd * upd * h0;
+		}
+		return 0;
+	}
+	if (rule == 7 || rule == 8 || rule == 9) {
+		const T l1_corr = (T) 1 / (1 - std::pow(1 - h1, (T) (timestep + 1)) + h3);
+		const T l1_next_corr = (T) 1 / (1 - std::pow(1 - h1, (T) (timestep + 2)) + h3);
+		const T l2_corr = (T) 1 / (1 - std::pow(1 - h2, (T) (timestep + 1)) + h3);
+		for (i64 i = 0; i < n; ++i) {
+			s0[i] = s0[i] * (1 - h1) + grad[i] * h1;
+			if (rule == 7) {
+				s1[i] = std::max(s1[i] * (1 - h2), std::abs(grad[i]));
+				values[i] = values[i] - (s0[i] * (h0 * l1_corr)) / (s1[i] + h3);
+			} else {
+				s1[i] = s1[i] * (1 - h2) + grad[i] * grad[i] * h2;
+				if (rule == 8)
+					values[i] = values[i] - ((grad[i] * (h1 * l1_corr) + s0[i] * ((1 - h1) * l1_next_corr)) * h0) /
+							std::sqrt(s1[i] * l2_corr + h3);
+				else {
+					s2[i] = std::max(s1[i], s2[i]);
+					values[i] = values[i] - (s0[i] * h0) / std::sqrt(s2[i] + h3);
+				}
+			}
+		}
+		return 0;
+	}
+	return 1;
+}
+
 } /* namespace */
 
 #define CONV_ARGS i64 N, i64 H, i64 W, i64 C, i64 F, i64 RH, i64 RW, i64 pv, i64 ph, i64 sv, i64 sh, i64 dv, i64 dh
@@ -841,6 +916,8 @@ extern "C" int oracle_loss_d_function_##SFX(int kind, i64 N, i64 Ts, i64 V, doub
 		const T* obj, T* grad) { return loss_d_function<T>(kind, N, Ts, V, (T) eps, (T) scale, out, obj, grad); } \
 extern "C" int oracle_sgd_update_##SFX(i64 n, double lr, const T* grad, T* values) { \
 	return sgd_update<T>(n, (T) lr, grad, values); } \
+extern "C" int oracle_optimizer_update_##SFX(int rule, const double* h, i64 epoch, i64 timestep, i64 n, const T* grad, T* s0, \
+		T* s1, T* s2, T* values) { return optimizer_update<T>(rule, h, epoch, timestep, n, grad, s0, s1, s2, values); } \
 extern "C" int oracle_adam_update_##SFX(i64 n, double lr, double d1, double d2, double eps, i64 timestep, const T* grad, \
 		T* m, T* v, T* values) { return adam_update<T>(n, (T) lr, (T) d1, (T) d2, (T) eps, timestep, grad, m, v, values); }
 

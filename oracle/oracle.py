@@ -373,3 +373,20 @@ def adam_update(values, grad, m, v, timestep, lr=1e-3, l1_decay=1e-1, l2_decay=1
     _call("adam_update", dt, *_ll(new.size), ctypes.c_double(lr), ctypes.c_double(l1_decay), ctypes.c_double(l2_decay),
           ctypes.c_double(eps), *_ll(timestep), _p(grad), _p(m), _p(v), _p(new))
     return new, m, v
+
+
+OPTIMIZERS = {"vanilla_sgd": 0, "momentum_sgd": 1, "nesterov_momentum_sgd": 2, "adagrad": 3, "rmsprop": 4, "adadelta": 5,
+              "adam": 6, "adamax": 7, "nadam": 8, "amsgrad": 9}
+
+
+def optimizer_update(rule, values, grad, states, hyper, epoch=0, timestep=0):
+    """One _update_params of optimizer `rule` on one parameter matrix. states: three matrices (unused ones are
+    ignored); hyper: the optimizer's constructor arguments in their order. Returns (values, [s0, s1, s2])."""
+    dt = values.dtype
+    new = np.array(values, dtype=dt, order="F", copy=True)
+    st = [np.array(s, dtype=dt, order="F", copy=True) for s in states]
+    grad = _f(grad, dt)
+    h = (ctypes.c_double * 4)(*(list(hyper) + [0.0] * (4 - len(hyper))))
+    _call("optimizer_update", dt, ctypes.c_int(OPTIMIZERS[rule]), h, *_ll(epoch, timestep, new.size), _p(grad), _p(st[0]),
+          _p(st[1]), _p(st[2]), _p(new))
+    return new, st

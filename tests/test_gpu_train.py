@@ -235,3 +235,54 @@ def test_whole_training_steps_stay_on_the_device(config):
         # entries, so entrywise relative agreement is not to be had) and on the values to 1e-4
         assert diff <= 1e-2 * moved + 1e-7, (diff, moved)
         assert np.allclose(pd.get_values(), ps.get_values(), rtol=1e-4, atol=1e-5)
+
+
+ALL_OPTIMIZERS = [("vanilla_sgd", [1e-2]), ("momentum_sgd", [1e-2, 1e-3, 0.9]), ("nesterov_momentum_sgd", [1e-2, 1e-3, 0.9]),
+                  ("adagrad", [1e-2, 1e-5]), ("rmsprop", [1e-3, 1e-1, 1e-5]), ("adadelta", [5e-2, 1e-5]),
+                  ("adam", [1e-3, 1e-1, 1e-3, 1e-5]), ("adamax", [1e-3, 1e-1, 1e-3, 1e-5]), ("nadam", [1e-3, 1e-1, 1e-3, 1e-5]),
+                  ("amsgrad", [1e-3, 1e-1, 1e-3, 1e-5])]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rule,hyper", ALL_OPTIMIZERS)
+def test_every_optimizer_over_steps(rule, hyper, dtype):
+    """Each optimizer's _update_params on the device against the oracle, four steps with fresh gradients, epoch 2
+    (the annealed learning rate), default hyper-parameters of the reference. After each comparison the oracle
+    continues from the device's values and state estimate so that rounding does not compound through 1/sqrt(v)."""
+    layer, g, w, b = _dense_with_grads(dtype, 1220)
+    prm = layer.get_params()[0]
+    tol = TOL[np.dtype(dtype)]
+    hyper_t = [float(dtype(h)) for h in hyper]
+    values = np.asarray(w, np.float64)
+    states = [np.zeros_like(values) for _ in range(3)]
+    for t in range(4):
+        prm.reset_grad()
+        _accumulate(layer, g, dtype)
+        grad = np.asarray(prm.get_grad(), np.float64)
+        prm.optimizer_update(rule, hyper, epoch=2, timestep=t)
+        values, states = oracle.optimizer_update(rule, values, grad, states, hyper_t, epoch=2, timestep=t)
+        got = np.asarray(prm.get_values(), np.float64)
+        assert hp.rel_err(got, values) < tol, (rule, t)
+        values = got
+    # _fit: the state starts again from zero
+    prm.reset_optimizer_state()
+    before = np.asarray(prm.get_values(), np.float64)
+    grad = np.asarray(prm.get_grad(), np.float64)
+    prm.optimizer_update(rule, hyper, epoch=0, timestep=0)
+    ref, _ = oracle.optimizer_update(rule, before, grad, [np.zeros_like(before) for _ in range(3)], hyper_t, 0, 0)
+    assert hp.rel_err(prm.get_values(), ref) < tol
+
+
+def test_optimizer_argument_checks():
+    layer, g, w, b = _dense_with_grads(np.float32, 1221)
+    prm = layer.get_params()[0]
+    with pytest.raises(ch.CattleHipError):
+        prm.optimizer_update("momentum_sgd", [1e-2, 1e-3, 1.0])        # assert(momentum > 0 && momentum < 1)
+    with pytest.raises(ch.CattleHipError):
+        prm.optimizer_update("adadelta", [1.5, 1e-5])                   # assert(decay >= 0 && decay <= 1)
+    with pytest.raises(ch.CattleHipError):
+        prm.optimizer_update("rmsprop", [1e-3, 1e-1, 0.0])              # assert(epsilon > 0)
+    import ctypes
+    h = (ctypes.c_double * 4)(1e-3, 0, 0, 0)
+    assert ch.lib().cattle_hip_layer_param_optimizer_update(layer._h, ctypes.c_size_t(0), ctypes.c_int(17), h, ctypes.c_size_t(0),
+                                                            ctypes.c_size_t(0)) != 0

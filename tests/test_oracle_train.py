@@ -165,3 +165,126 @@ def test_adam_reference_formula_with_default_epsilon(dtype):
         w64 = w64 - lr * c1 * m64 / np.sqrt(c2 * v64 + eps)
         assert hp.rel_err(w, w64) < TOL[np.dtype(dtype)]
         assert hp.rel_err(m, m64) < TOL[np.dtype(dtype)] and hp.rel_err(v, v64) < TOL[np.dtype(dtype)]
+
+
+# ---------------------------------------------------------------------------------------------------------
+# The other optimizers (optimizer/*.hpp). torch's implementations are independent code; where the
+# reference's recurrence is the same one (possibly after mapping the hyper-parameters) several steps with
+# changing gradients must agree. Nadam and AMSGrad differ from torch's variants and are pinned by closed
+# forms instead.
+# ---------------------------------------------------------------------------------------------------------
+def _grads(seed, steps=5, shape=(6, 4)):
+    g = hp.rng(seed)
+    w0 = hp.normal(g, shape, np.float64)
+    return w0, [hp.uniform(g, shape, 0.5, 2.0, np.float64) * np.where(g.random(shape) < 0.5, -1, 1) for _ in range(steps)]
+
+
+def _run_oracle(rule, w0, grads, hyper, epoch=0):
+    w, st = w0, [np.zeros_like(w0) for _ in range(3)]
+    out = []
+    for t, dw in enumerate(grads):
+        w, st = oracle.optimizer_update(rule, w, dw, st, hyper, epoch=epoch, timestep=t)
+        out.append(w)
+    return out, st
+
+
+def _run_torch(make_opt, w0, grads):
+    pt = torch.tensor(w0.copy(), requires_grad=True)
+    opt = make_opt([pt])
+    out = []
+    for dw in grads:
+        pt.grad = torch.tensor(dw.copy())
+        opt.step()
+        out.append(pt.detach().numpy().copy())
+    return out
+
+
+@pytest.mark.parametrize("rule,hyper,make_opt", [
+    ("vanilla_sgd", [0.05], lambda p: torch.optim.SGD(p, lr=0.05)),
+    # s = momentum s + lr g, w -= s: torch's buffer times lr (annealing rate 0)
+    ("momentum_sgd", [0.05, 0.0, 0.9], lambda p: torch.optim.SGD(p, lr=0.05, momentum=0.9)),
+    # s = momentum s - lr g, w += -momentum s_old + (1 + momentum) s: torch's Nesterov step with s = -lr * buffer
+    ("nesterov_momentum_sgd", [0.05, 0.0, 0.8], lambda p: torch.optim.SGD(p, lr=0.05, momentum=0.8, nesterov=True)),
+    ("adagrad", [0.1, 1e-7], lambda p: torch.optim.Adagrad(p, lr=0.1, eps=1e-7)),
+    ("rmsprop", [0.02, 0.1, 1e-7], lambda p: torch.optim.RMSprop(p, lr=0.02, alpha=0.9, eps=1e-7)),
+    ("adadelta", [0.05, 1e-6], lambda p: torch.optim.Adadelta(p, lr=1.0, rho=0.95, eps=1e-6)),
+])
+def test_optimizers_that_coincide_with_torch(rule, hyper, make_opt):
+    w0, grads = _grads(920)
+    ours, _ = _run_oracle(rule, w0, grads, hyper)
+    theirs = _run_torch(make_opt, w0, grads)
+    for t, (a, b) in enumerate(zip(ours, theirs)):
+        assert np.max(np.abs(a - b)) < 1e-12, (rule, t)
+
+
+def test_adamax_matches_torch_in_the_small_epsilon_limit():
+    """torch: u = max(beta2 u, |g| + eps), w -= lr / (1 - beta1^t) * m / u; the reference: u = max((1 - d2) u, |g|),
+    w -= lr * m / (1 - (1 - d1)^t + eps) / (u + eps). Same recurrence for eps -> 0."""
+    w0, grads = _grads(921)
+    ours, _ = _run_oracle("adamax", w0, grads, [0.02, 0.1, 0.01, 1e-30])
+    theirs = _run_torch(lambda p: torch.optim.Adamax(p, lr=0.02, betas=(0.9, 0.99), eps=1e-30), w0, grads)
+    for a, b in zip(ours, theirs):
+        assert np.max(np.abs(a - b)) < 1e-12
+
+
+def test_annealed_learning_rate_of_the_momentum_optimizers():
+    """calculate_learning_rate (MomentumSGDOptimizer.hpp:70-72): lr = init / (1 + annealing * epoch); at zero
+    momentum-state the first step is w - lr g for both variants... Nesterov's is w - (1 + momentum) lr g."""
+    w0, grads = _grads(922, steps=1)
+    for epoch in (0, 3):
+        lr = 0.1 / (1 + 0.5 * epoch)
+        (w,), _ = _run_oracle("momentum_sgd", w0, grads, [0.1, 0.5, 0.9], epoch=epoch)
+        assert np.max(np.abs(w - (w0 - lr * grads[0]))) < 1e-13
+        (w,), _ = _run_oracle("nesterov_momentum_sgd", w0, grads, [0.1, 0.5, 0.9], epoch=epoch)
+        assert np.max(np.abs(w - (w0 - 1.9 * lr * grads[0]))) < 1e-13
+
+
+def test_nadam_first_step_closed_form_and_relation_to_adam():
+    """From zero state at step 0 with eps -> 0: m = d1 g, v = d2 g^2, l1_corr = 1/d1, l1_next_corr = 1/(1-(1-d1)^2),
+    l2_corr = 1/d2, so the step is lr sign(g) (1 + (1-d1)/(2-d1)). In general Nadam's numerator is
+    d1 l1_corr g + (1-d1) l1_next_corr m where Adam's is l1_corr m, over the same denominator."""
+    w0, grads = _grads(923, steps=3)
+    d1, d2, lr = 0.2, 0.05, 0.01
+    (w1, w2, w3), st = _run_oracle("nadam", w0, grads, [lr, d1, d2, 1e-30])
+    assert np.max(np.abs(w1 - (w0 - lr * np.sign(grads[0]) * (1 + (1 - d1) / (2 - d1))))) < 1e-12
+    # third step from the state after two steps, written out independently
+    m = np.zeros_like(w0)
+    v = np.zeros_like(w0)
+    for dw in grads:
+        m = (1 - d1) * m + d1 * dw
+        v = (1 - d2) * v + d2 * dw * dw
+    c1, c1n, c2 = 1 / (1 - (1 - d1) ** 3), 1 / (1 - (1 - d1) ** 4), 1 / (1 - (1 - d2) ** 3)
+    assert np.max(np.abs(w3 - (w2 - lr * (d1 * c1 * grads[2] + (1 - d1) * c1n * m) / np.sqrt(c2 * v)))) < 1e-12
+    assert hp.rel_err(st[0], m) < 1e-12 and hp.rel_err(st[1], v) < 1e-12
+
+
+def test_amsgrad_keeps_the_running_maximum_and_has_no_bias_correction():
+    """AMSGradOptimizer.hpp:48-66: w -= lr m / sqrt(max_t v_t + eps), m and v uncorrected. First step from zero
+    state: lr d1 g / sqrt(d2 g^2 + eps); after a large gradient the denominator never shrinks."""
+    shape = (5, 3)
+    g = hp.rng(924)
+    w0 = hp.normal(g, shape, np.float64)
+    big = hp.uniform(g, shape, 5, 6, np.float64)
+    small = [hp.uniform(g, shape, 0.1, 0.2, np.float64) for _ in range(4)]
+    d1, d2, lr, eps = 0.1, 0.2, 0.01, 1e-8
+    ws, st = _run_oracle("amsgrad", w0, [big] + small, [lr, d1, d2, eps])
+    assert np.max(np.abs(ws[0] - (w0 - lr * d1 * big / np.sqrt(d2 * big * big + eps)))) < 1e-13
+    vmax = d2 * big * big                      # v only decays from here on (small gradients): the maximum stays
+    assert hp.rel_err(st[2], vmax) < 1e-13
+    m = d1 * big
+    w = ws[0]
+    for t, dw in enumerate(small):
+        m = (1 - d1) * m + d1 * dw
+        w = w - lr * m / np.sqrt(vmax + eps)
+        assert np.max(np.abs(ws[t + 1] - w)) < 1e-13
+
+
+@pytest.mark.parametrize("rule,hyper", [("momentum_sgd", [1e-3, 1e-3, 0.9]), ("adagrad", [1e-2, 1e-5]), ("rmsprop", [1e-3, 1e-1, 1e-5]),
+                                        ("adadelta", [5e-2, 1e-5]), ("adamax", [1e-3, 1e-1, 1e-3, 1e-5]),
+                                        ("nadam", [1e-3, 1e-1, 1e-3, 1e-5]), ("amsgrad", [1e-3, 1e-1, 1e-3, 1e-5])])
+def test_float32_optimizer_steps_track_float64(rule, hyper):
+    """With the reference's default hyper-parameters, float32 steps stay within the float32 tolerance of float64 ones."""
+    w0, grads = _grads(925, steps=3)
+    w64, _ = _run_oracle(rule, w0, grads, hyper, epoch=2)
+    w32, _ = _run_oracle(rule, w0.astype(np.float32), [dw.astype(np.float32) for dw in grads], hyper, epoch=2)
+    assert hp.rel_err(w32[-1], w64[-1]) < 1e-4
