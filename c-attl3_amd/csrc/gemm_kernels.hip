@@ -143,10 +143,23 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero_block[4] = { 0u, 0
  * VEC = elements per global load along m (needs N % VEC == 0 and a 16-byte aligned src).
  * DIVS = the gather has divisors (strided input gradient).
  * ---------------------------------------------------------------------------------------------- */
+/* How a launch covers the M tiles, which are walked in the order swizzle_tile defines. The first
+ * main_count positions of the walk are whole tiles, one block each (blocks [0, main_blocks), dealt to the
+ * XCDs in contiguous ranges). The remaining split_count positions have their reduction cut into ksplit
+ * parts of chunks_per_part chunks, one block per part (blocks from main_blocks on, so they are dispatched
+ * last and fill the chip as the whole tiles drain): such a block writes its BM x BF partial sums, without
+ * bias, to `partials`, laid out [position - main_count][f block][part][f][m], and split_reduce_kernel adds
+ * the parts in a fixed order. */
+struct GatherLaunch {
+	int mtiles, tile_rows;
+	int main_count, main_blocks;
+	int split_count, ksplit, chunks_per_part;
+};
+
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
 void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom g, const int mtiles, const int tile_rows) {
+		T* __restrict__ out, const GatherGeom g, const GatherLaunch L, T* __restrict__ partials) {
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_M * WAVES_F;
 	constexpr int BM = WAVES_M * WT_M, BF = WAVES_F * WT_F;
@@ -166,20 +179,35 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	__shared__ __attribute__((aligned(32))) T Bs[2][KC][LDB];
 	__shared__ int4 ktab[3][KC];     /* per reduction index: element offset, ya term, yb term, channel offset */
 
-	int tile = xcd_tile(blockIdx.x, mtiles);
-	if (tile >= mtiles)
-		return;
-	if (tile_rows > 0)
-		tile = swizzle_tile(tile, tile_rows, mtiles / tile_rows);
+	int local, part = 0;
+	const bool split = (int) blockIdx.x >= L.main_blocks;
+	if (!split) {
+		local = xcd_tile(blockIdx.x, L.main_count);
+		if (local >= L.main_count)
+			return;
+	} else {
+		const int r = (int) blockIdx.x - L.main_blocks;
+		local = r / L.ksplit;
+		part = r - local * L.ksplit;
+		if (local >= L.split_count)
+			return;
+	}
+	int tile = split ? L.main_count + local : local;
+	if (L.tile_rows > 0)
+		tile = swizzle_tile(tile, L.tile_rows, L.mtiles / L.tile_rows);
 	const int tid = threadIdx.x;
 	const int m0 = tile * BM;
 	const int f0 = blockIdx.y * BF;
-	const int nchunks = (g.K + KC - 1) / KC;
+	/* this block's chunks of the reduction: all of them, or one part */
+	const int chunk0 = split ? part * L.chunks_per_part : 0;
+	const int nchunks = split ? min(L.chunks_per_part, (g.K + KC - 1) / KC - chunk0) : (g.K + KC - 1) / KC;
 
-	/* --- table writer state: thread t < KC walks k = t, t + KC, t + 2 KC, ... --- */
-	int tr = tid % g.R, ts, tch;
+	/* --- table writer state: thread t < KC walks k = k0 + t, k0 + t + KC, ... from the first chunk's k0 --- */
+	int tr, ts, tch;
 	{
-		const int t = tid / g.R;
+		const int k = chunk0 * KC + tid;
+		tr = k % g.R;
+		const int t = k / g.R;
 		ts = t % g.S;
 		tch = t / g.S;
 	}
@@ -219,7 +247,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	#pragma unroll
 	for (int it = 0; it < BITER; ++it) {
 		const int idx = tid + it * THREADS;
-		bptr[it] = wt + ((size_t) (idx / BCOLS) * g.ldw + f0 + (idx % BCOLS) * VB);
+		bptr[it] = wt + ((size_t) (chunk0 * KC + idx / BCOLS) * g.ldw + f0 + (idx % BCOLS) * VB);
 	}
 	const size_t bstep = (size_t) KC * g.ldw;
 
@@ -323,6 +351,25 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	/* epilogue: D rows are filters (row rr of block i is filter FB*rr + i), D columns are m
 	 * (column lc of block j is row MB*lc + j of the tile), so a lane owns MB adjacent outputs */
 	constexpr int VS = MB * (int) sizeof(T) > 16 ? 16 / (int) sizeof(T) : MB;
+	if (split) {
+		/* partial sums of this part: a dense BF x BM tile (m fastest), always whole and aligned */
+		T* ptile = partials + ((size_t) (local * (int) gridDim.y + (int) blockIdx.y) * L.ksplit + part) * (BM * BF);
+		#pragma unroll
+		for (int i = 0; i < FB; ++i)
+			#pragma unroll
+			for (int r = 0; r < MF::NACC; ++r) {
+				T* dst = ptile + (size_t) (wf * WT_F + FB * acc_row<T>(r, lk) + i) * BM + wm * WT_M + MB * lc;
+				#pragma unroll
+				for (int j0 = 0; j0 < MB; j0 += VS) {
+					T v[VS];
+					#pragma unroll
+					for (int j = 0; j < VS; ++j)
+						v[j] = acc[i][j0 + j][r];
+					vec_store<T, VS>(dst + j0, v);
+				}
+			}
+		return;
+	}
 	const bool vec_out = g.M % MB == 0 && (reinterpret_cast<uintptr_t>(out) & (VS * sizeof(T) - 1)) == 0;
 	const int mm = m0 + wm * WT_M + MB * lc;
 	#pragma unroll
@@ -678,31 +725,88 @@ constexpr int LDS_PER_CU = 160 * 1024;
 constexpr int MAX_WAVES_PER_CU = 16;   /* four per SIMD: every kernel here stays within 128 registers per lane */
 
 
+/* Grow-only device scratch for split reductions. Calls into the library are serialised and issued on
+ * one stream, so a later call may reuse (or, after hipFree's implicit synchronisation, replace) it. */
+void* split_workspace(size_t bytes) {
+	static void* ptr = nullptr;
+	static size_t cap = 0;
+	if (bytes > cap) {
+		if (ptr)
+			(void) hipFree(ptr);
+		ptr = nullptr;
+		cap = 0;
+		const size_t want = (bytes + 4095) / 4096 * 4096;
+		CATTLE_HIP_CHECK(hipMalloc(&ptr, want));
+		cap = want;
+	}
+	return ptr;
+}
+
+/* out tile = bias + sum over the parts of a split reduction, parts taken in ascending order (so the result
+ * does not depend on how blocks were scheduled). One block per (walk position, f block) tile. */
+template<typename T>
+__global__ __launch_bounds__(256)
+void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ bias, T* __restrict__ out, int M, int F,
+		const GatherLaunch L, int BM, int BF, int ftiles) {
+	constexpr int V = 16 / (int) sizeof(T);             /* consecutive m per thread: one 16-byte load per part */
+	const int groups = BM * BF / (256 * V);             /* blocks per tile; tiles are multiples of 64 x 32 */
+	const int t = blockIdx.x / groups, grp = blockIdx.x % groups;
+	const int local = t / ftiles, fb = t % ftiles;
+	int tile = L.main_count + local;
+	if (L.tile_rows > 0)
+		tile = swizzle_tile(tile, L.tile_rows, L.mtiles / L.tile_rows);
+	const size_t tile_elems = (size_t) BM * BF;
+	const int e = (grp * 256 + threadIdx.x) * V;
+	const T* base = partials + (size_t) t * L.ksplit * tile_elems + e;
+	T acc[V];
+	vec_load<T, V>(acc, base);
+	for (int z = 1; z < L.ksplit; ++z) {
+		T part[V];
+		vec_load<T, V>(part, base + (size_t) z * tile_elems);
+		#pragma unroll
+		for (int i = 0; i < V; ++i)
+			acc[i] += part[i];
+	}
+	const int m = tile * BM + e % BM, f = fb * BF + e / BM;
+	if (f >= F)
+		return;
+	const T bv = bias ? bias[f] : (T) 0;
+	T* dst = out + ((size_t) m + (size_t) M * f);
+	if (m + V <= M && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+		#pragma unroll
+		for (int i = 0; i < V; ++i)
+			acc[i] += bv;
+		vec_store<T, V>(dst, acc);
+	} else {
+		#pragma unroll
+		for (int i = 0; i < V; ++i)
+			if (m + i < M)
+				dst[i] = acc[i] + bv;
+	}
+}
+
 /* One instantiation of gather_gemm_kernel and what the tile chooser needs to know about it. */
 template<typename T>
 struct GatherVariant {
 	int bm, bf, waves, lds_bytes;
-	void (*launch)(dim3 grid, size_t dyn_lds, const T*, const T*, const T*, T*, const GatherGeom&, int mtiles, bool vec, bool divs);
+	int kc;
+	void (*launch)(dim3 grid, size_t dyn_lds, const T*, const T*, const T*, T*, const GatherGeom&, const GatherLaunch&,
+			T* partials, bool vec, bool divs);
 };
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
 void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g,
-		int mtiles, bool vec, bool divs) {
+		const GatherLaunch& L, T* partials, bool vec, bool divs) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	dim3 block(64 * WAVES_M * WAVES_F);
-	/* tiles per output column, if a column (N * OA rows of M) is a whole number of tiles and there are
-	 * several columns; 0 switches the 2-D walk off */
-	constexpr int BM = WAVES_M * WT_M;
-	const long column = (long) g.N * g.OA;
-	int tile_rows = (column % BM == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE")) ? (int) (column / BM) : 0;
 	if (vec && !divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
 	else if (vec && divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
 	else if (!divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
 	else
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, mtiles, tile_rows);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
@@ -715,6 +819,7 @@ GatherVariant<T> gather_variant() {
 	v.bf = WAVES_F * WT_F;
 	v.waves = WAVES_M * WAVES_F;
 	v.lds_bytes = 2 * KC * (v.bm + v.bf + 2 * C::pad(v.bm)) * (int) sizeof(T) + 3 * KC * 16;
+	v.kc = KC;
 	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC>;
 	return v;
 }
@@ -790,9 +895,51 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		const int want_bytes = LDS_PER_CU / (occ + 1) + 256;
 		dyn = want_bytes > v.lds_bytes ? (size_t) (want_bytes - v.lds_bytes) : 0;
 	}
-	const int mtiles = (g.M + v.bm - 1) / v.bm;
-	dim3 grid((unsigned) round_up(mtiles, 8), (unsigned) ((g.F + v.bf - 1) / v.bf));
-	v.launch(grid, dyn, src, wt, bias, out, g, mtiles, vec, divs);
+	const int mtiles = (g.M + v.bm - 1) / v.bm, ftiles = (g.F + v.bf - 1) / v.bf;
+	const int nchunks = (g.K + v.kc - 1) / v.kc;
+	/* tiles per output column, if a column (N * OA rows of M) is a whole number of tiles and there are
+	 * several columns; 0 switches the 2-D walk off */
+	const long column = (long) g.N * g.OA;
+	const int tile_rows = (column % v.bm == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE")) ? (int) (column / v.bm) : 0;
+	/* blocks the chip holds at once, by LDS and by waves (four per SIMD) */
+	const int per_cu = std::max(1, std::min(LDS_PER_CU / (v.lds_bytes + (int) dyn), MAX_WAVES_PER_CU / v.waves));
+	const int slots = NUM_CUS * per_cu;
+	const bool no_split = std::getenv("CATTLE_HIP_NO_SPLIT") != nullptr;
+
+	/* main_count whole tiles, the other mtiles - main_count with their reduction cut into about `ksplit` parts */
+	auto launch = [&](int main_count, int ksplit) {
+		GatherLaunch L = { mtiles, tile_rows, main_count, round_up(main_count, 8), mtiles - main_count, 1, nchunks };
+		T* partials = nullptr;
+		if (L.split_count > 0) {
+			L.chunks_per_part = (nchunks + ksplit - 1) / ksplit;
+			L.ksplit = (nchunks + L.chunks_per_part - 1) / L.chunks_per_part;       /* no empty part */
+			partials = static_cast<T*>(split_workspace((size_t) L.split_count * ftiles * L.ksplit * v.bm * v.bf * sizeof(T)));
+		}
+		dim3 grid((unsigned) (L.main_blocks + L.split_count * L.ksplit), (unsigned) ftiles);
+		v.launch(grid, dyn, src, wt, bias, out, g, L, partials, vec, divs);
+		if (L.split_count > 0) {
+			const int groups = v.bm * v.bf / (256 * (16 / (int) sizeof(T)));
+			split_reduce_kernel<T><<<dim3((unsigned) (L.split_count * ftiles * groups)), 256, 0, stream()>>>(partials, bias, out,
+					g.M, g.F, L, v.bm, v.bf, ftiles);
+			CATTLE_HIP_CHECK(hipGetLastError());
+		}
+	};
+
+	const long total = (long) mtiles * ftiles;
+	if (!no_split && total * 2 <= slots && nchunks >= 4) {
+		/* far fewer tiles than the chip holds blocks: cut every tile's reduction so that it fills up */
+		launch(0, (int) std::min<long>(std::min<long>(slots / total, nchunks / 2), 16));
+		return;
+	}
+	const int rem = mtiles % slots;
+	if (!no_split && ftiles == 1 && mtiles > slots && rem > 0 && rem * 2 <= slots && nchunks >= 8) {
+		/* The tiles left over after whole rounds would keep a fraction of the chip busy for a whole tile time.
+		 * Their reduction is cut into parts instead; the part blocks come last in the grid and fill the
+		 * chip as the last round of whole tiles drains. */
+		launch(mtiles - rem, (int) std::min<long>(std::min(slots / rem, nchunks / 4), 16));
+		return;
+	}
+	launch(mtiles, 1);
 }
 
 GatherGeom forward_geom(const ConvShape& s, int N) {
