@@ -841,9 +841,10 @@ template<> struct GatherVariants<float> {
 	}
 };
 template<> struct GatherVariants<double> {
-	static constexpr int COUNT = 4, LARGE = 2;
+	static constexpr int COUNT = 5, LARGE = 3;
 	static const GatherVariant<double>* get() {
 		static const GatherVariant<double> v[COUNT] = {
+			gather_variant<double, 8, 2, 32, 64>(),     /* 256 x 128, sixteen waves */
 			gather_variant<double, 4, 2, 64, 32>(),     /* 256 x 64 */
 			gather_variant<double, 4, 1, 64, 32>(),     /* 256 x 32 */
 			gather_variant<double, 2, 2, 32, 32, 32>(), /* 64 x 64, small problems */
