@@ -10,6 +10,7 @@
 #include "../../include/cattle_hip.h"
 
 #include <cstring>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <vector>
@@ -89,6 +90,61 @@ void fill_zero(void* dst_dev, size_t bytes) {
 	if (bytes)
 		CATTLE_HIP_CHECK(hipMemsetAsync(dst_dev, 0, bytes, stream()));
 }
+
+/* Device memory handed out through cattle_hip_alloc. Activations of a training step are allocated and
+ * released at every layer call; hipMalloc / hipFree would synchronise the device each time, so released
+ * blocks are kept, by size class, and handed out again. Everything the library does is ordered on one
+ * stream, so a block may be reused as soon as it has been given back: work that still reads it was issued
+ * earlier on that stream. Blocks return to the driver in trim() or at process exit. */
+struct DevicePool {
+	std::map<size_t, std::vector<void*>> idle;      /* size class -> blocks */
+	std::map<void*, size_t> live;                    /* block -> size class */
+	size_t idle_bytes = 0;
+	static size_t size_class(size_t bytes) {
+		/* powers of two up to 1 MiB, then multiples of 1 MiB: at most 2x / ~0 % over-allocation */
+		size_t c = 256;
+		while (c < bytes && c < (1u << 20))
+			c <<= 1;
+		return c >= bytes ? c : (bytes + (1u << 20) - 1) / (1u << 20) * (1u << 20);
+	}
+	void* take(size_t bytes) {
+		const size_t c = size_class(bytes ? bytes : 1);
+		std::vector<void*>& bucket = idle[c];
+		void* p = nullptr;
+		if (!bucket.empty()) {
+			p = bucket.back();
+			bucket.pop_back();
+			idle_bytes -= c;
+		} else {
+			hipError_t e = hipMalloc(&p, c);
+			if (e == hipErrorOutOfMemory && idle_bytes > 0) {       /* give the idle blocks back and try again */
+				(void) hipGetLastError();
+				(void) hipStreamSynchronize(stream());
+				trim();
+				e = hipMalloc(&p, c);
+			}
+			CATTLE_HIP_CHECK(e);
+		}
+		live[p] = c;
+		return p;
+	}
+	void give_back(void* p) {
+		std::map<void*, size_t>::iterator it = live.find(p);
+		CATTLE_HIP_REQUIRE(it != live.end(), "cattle_hip_free of a pointer that cattle_hip_alloc did not return");
+		idle[it->second].push_back(p);
+		idle_bytes += it->second;
+		live.erase(it);
+	}
+	void trim() {
+		for (std::map<size_t, std::vector<void*>>::iterator it = idle.begin(); it != idle.end(); ++it) {
+			for (void* p : it->second)
+				(void) hipFree(p);
+			it->second.clear();
+		}
+		idle_bytes = 0;
+	}
+};
+DevicePool g_pool;
 
 /* Device twin of a Parameters object (core/Parameters.hpp:15-95): values plus accumulated gradient.
  * `derived` holds kernel-friendly re-layouts of the values, rebuilt when `version` moves on. */
@@ -813,17 +869,21 @@ int cattle_hip_synchronize(void) {
 int cattle_hip_alloc(void** device_ptr, size_t bytes) {
 	return guarded([&] {
 		CATTLE_HIP_REQUIRE(device_ptr != nullptr, "null output pointer");
-		*device_ptr = nullptr;
-		CATTLE_HIP_CHECK(hipMalloc(device_ptr, bytes ? bytes : 1));
+		*device_ptr = g_pool.take(bytes);
 	});
 }
 
 int cattle_hip_free(void* device_ptr) {
 	return guarded([&] {
-		if (device_ptr) {
-			CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
-			CATTLE_HIP_CHECK(hipFree(device_ptr));
-		}
+		if (device_ptr)
+			g_pool.give_back(device_ptr);
+	});
+}
+
+int cattle_hip_trim(void) {
+	return guarded([&] {
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+		g_pool.trim();
 	});
 }
 

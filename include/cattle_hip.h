@@ -70,7 +70,10 @@ int cattle_hip_synchronize(void);
 /* Plain device memory for callers that keep activations resident between layers (the idea of
  * core/gpu/GPULayer.hpp:31-58: device-tensor overloads next to the host-tensor virtuals). */
 int cattle_hip_alloc(void** device_ptr, size_t bytes);
+/* Released blocks are kept by the library and handed out again (a hipFree would stall the device at every
+ * layer of a step); cattle_hip_trim returns the idle ones to the driver. */
 int cattle_hip_free(void* device_ptr);
+int cattle_hip_trim(void);
 int cattle_hip_upload(void* dst_device, const void* src_host, size_t bytes);
 int cattle_hip_download(void* dst_host, const void* src_device, size_t bytes);
 int cattle_hip_fill_zero(void* dst_device, size_t bytes);
