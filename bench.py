@@ -33,9 +33,10 @@ SHAPE = dict(H=56, W=56, C=64, F=128, RH=3, RW=3)
 # read while timing, so these are constants of the measured build; other shapes report null.
 MEASURED_TRAFFIC = {
     ("f32", 256): {
-        "gather_gemm_kernel (forward)": 389.9e6 + 411.0e6,
-        "wgrad_kernel (+ reduce, bias column sums)": 945.7e6 + 50.3e6 + 2 * 12.6e6 + 0.3e6,
-        "gather_gemm_kernel (input gradient)": 726.6e6 + 205.5e6,
+        # kernel read + written, then the reduce launches' read + written
+        "gather_gemm_kernel (forward)": 373.4e6 + 469.8e6 + 67.2e6 + 8.4e6,
+        "wgrad_kernel (+ reduce, bias column sums)": 956.7e6 + 50.3e6 + 50.5e6 + 0.3e6,
+        "gather_gemm_kernel (input gradient)": 730.6e6 + 234.9e6 + 33.6e6 + 4.2e6,
     },
 }
 
@@ -196,6 +197,69 @@ def convlstm_run(args, dtype):
                        "flop_per_step": flop}}
 
 
+def train_steps_run(args, dtype):
+    """BASELINE configs[1] and [2] as whole device-resident training steps (propagate, softmax cross-entropy gradient,
+    backpropagate, optimizer update, gradient reset): MLP 784-512-256-10 at batch 256 with vanilla SGD, and
+    conv32-ReLU-pool-conv64-BN-ReLU-pool-dense10 on 32x32x3 at batch 128 with Adam."""
+    ch = importlib.import_module("c-attl3_amd")
+    ch.init(0)
+    gen = np.random.default_rng(0xC0FFEE02)
+
+    def mlp():
+        return [ch.DenseKernelLayer(dtype, (784,), 512), ch.ActivationLayer(dtype, "relu", (512,)),
+                ch.DenseKernelLayer(dtype, (512,), 256), ch.ActivationLayer(dtype, "relu", (256,)),
+                ch.DenseKernelLayer(dtype, (256,), 10)]
+
+    def convnet():
+        return [ch.ConvKernelLayer(dtype, (32, 32, 3), 32), ch.ActivationLayer(dtype, "relu", (32, 32, 32)),
+                ch.MaxPoolLayer(dtype, (32, 32, 32)), ch.ConvKernelLayer(dtype, (16, 16, 32), 64),
+                ch.BatchNormLayer(dtype, (16, 16, 64)), ch.ActivationLayer(dtype, "relu", (16, 16, 64)),
+                ch.MaxPoolLayer(dtype, (16, 16, 64)), ch.DenseKernelLayer(dtype, (8, 8, 64), 10)]
+
+    rows = []
+    for name, build, N, in_shape, out_shape, adam, flop in (
+            ("MLP 784-512-256-10, batch 256, vanilla SGD (BASELINE configs[1])", mlp, 256, (784,), (10,), False, 616300544.0),
+            ("convnet 32x32x3, batch 128, Adam (BASELINE configs[2])", convnet, 128, (32, 32, 3), (10, 1, 1), True, 4.108e9)):
+        layers = build()
+        layers[0].set_input_layer(True)
+        params = [p for l in layers for p in l.get_params()]
+        for p in params:
+            if p.are_optimizable() and p.get_rows() > 1:
+                p.set_values(he_normal(gen, p.get_rows(), p.get_cols(), dtype))
+        x = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N,) + in_shape).astype(dtype)))
+        obj = np.zeros((N,) + out_shape, dtype, order="F")
+        obj.reshape((N, -1), order="F")[np.arange(N), gen.integers(0, 10, N)] = 1
+        y = ch.DeviceTensor.from_host(obj)
+
+        def step(t):
+            a = x
+            for l in layers:
+                a = l.pass_forward(a, True)
+            g = ch.loss_d_function("softmax_cross_entropy", a, y, scale=1.0 / N)
+            for l in reversed(layers):
+                g = l.pass_back(g)
+            for p in params:
+                if p.are_optimizable():
+                    if adam:
+                        p.adam_update(t)
+                    else:
+                        p.sgd_update(1e-3)
+                    p.reset_grad()
+
+        for t in range(args.warmup):
+            step(t)
+        ch.synchronize()
+        t0 = time.perf_counter()
+        for t in range(args.steps):
+            step(t)
+        ch.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        rows.append({"workload": name, "ms_per_step": round(ms, 4), "samples_per_s": round(N / (ms * 1e-3), 1),
+                     "gflops": round(flop / (ms * 1e-3) / 1e9, 1)})
+    return {"metric": "device_resident_training_step", "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "dtype": args.dtype, "data": "synthetic", "driver": "python (ctypes), one C-ABI call per layer pass", "steps_timed": rows}
+
+
 def cpu_baseline(args, dtype):
     """Times the oracle (the restatement of the reference algorithm: explicit patch matrix + GEMMs +
     col2im, OpenMP GEMMs) on a bounded sample: the same layer at a smaller batch."""
@@ -234,9 +298,10 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel of x's size (for scaling rocprof byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm"], default="conv",
+    ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm", "train_steps"], default="conv",
                     help="conv: the headline benchmark; pointwise: HBM-bound layers, one line of per-kernel GB/s; "
-                         "convlstm: the fused-gate ConvLSTM of BASELINE configs[4], sequences/s")
+                         "convlstm: the fused-gate ConvLSTM of BASELINE configs[4], sequences/s; "
+                         "train_steps: whole device-resident training steps of BASELINE configs[1] and [2]")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
@@ -249,6 +314,9 @@ def main():
                           "roofline": {"bound": "hbm", "peak": 8000.0, "unit": "GB/s"}, "kernels": rows}))
         return
 
+    if args.workload == "train_steps":
+        print(json.dumps(train_steps_run(args, dtype)))
+        return
     if args.workload == "convlstm":
         print(json.dumps(convlstm_run(args, dtype)))
         return
