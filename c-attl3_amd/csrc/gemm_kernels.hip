@@ -333,6 +333,11 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 				vec_load<T, MB>(xa[nxt], &As[buf][(st + 1) * KS + lk][wm * WT_M + MB * lc]);
 				vec_load<T, FB>(wb[nxt], &Bs[buf][(st + 1) * KS + lk][wf * WT_F + FB * lc]);
 			}
+			/* the next chunk goes into the other LDS buffer ahead of the last step's MFMAs rather than after
+			 * them: its stores (and the wait for its global loads) then overlap that MFMA work, and
+			 * only the barrier itself remains between the chunks */
+			if (KC / KS > 1 && st == KC / KS - 1 && c + 1 < nchunks)
+				store_tiles(buf ^ 1);
 			/* issue order matters (a wave issues in order and stalls on a busy MFMA pipe): the LDS reads
 			 * of the next step must go out before this step's MFMAs, so pin the schedule here */
 			__builtin_amdgcn_sched_barrier(0);
@@ -343,7 +348,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 					acc[i][j] = MF::mma(wb[cur][i], xa[cur][j], acc[i][j]);
 			__builtin_amdgcn_sched_barrier(0);
 		}
-		if (c + 1 < nchunks)
+		if (KC / KS <= 1 && c + 1 < nchunks)
 			store_tiles(buf ^ 1);
 		__syncthreads();
 	}
