@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the kernel-layer hot path on one MI355X.
 
-Workload (BASELINE.json configs[3], the shape north_star's target is stated on):
+Workload (BASELINE.json configs[3], the shape the performance target is stated on):
 ConvKernelLayer<float,3> forward + backward (weight, bias and input gradients), batch 256, input
 NHWC 56x56x64 drawn from N(0,1), 128 filters 3x3, stride 1, padding 1, He-normal weights, upstream
 gradient N(0,1). One step = one pass_forward + one pass_back on tensors already resident in HBM.

@@ -1,4 +1,4 @@
-"""Host-side counterparts of the reference's callers, used by the parity tests to
+"""Host-side counterparts of the reference's callers (networks, losses, optimizers), used by the parity tests to
 drive the layers the way C-ATTL3's networks and optimizers do. Nothing here is product code; the
 same orchestration runs on two back ends with one interface:
 

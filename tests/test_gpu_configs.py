@@ -13,7 +13,7 @@ import harness as hn
 import helpers as hp
 
 pytestmark = pytest.mark.gpu
-TOL = 1e-4          # fp32 max relative error (floor 0.1 RMS), north_star's bound
+TOL = 1e-4          # fp32 max relative error (floor 0.1 RMS), the bound the benchmark definition states
 
 
 def _sync_params(src_net, dst_net):

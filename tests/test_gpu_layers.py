@@ -1,5 +1,5 @@
 """GPU parity tests: the HIP layers, called through the C ABI, against the CPU oracle on identical
-seeded inputs. Tolerances are north_star's: fp32 max relative error 1e-4, fp64 1e-10 (metric and
+seeded inputs. Tolerances are those of the benchmark definition: fp32 max relative error 1e-4, fp64 1e-10 (metric and
 absolute floor in helpers.rel_err), max-pool indices bit-exact."""
 import importlib
 
