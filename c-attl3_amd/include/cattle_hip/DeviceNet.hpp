@@ -18,6 +18,7 @@
 #include <array>
 #include <cassert>
 #include <cstddef>
+#include <fstream>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -139,7 +140,9 @@ public:
 		cattle_hip_layer_t h = nullptr;
 		check(cattle_hip_batchnorm_create(Code<Scalar>::value, dims[0], dims[1], dims[2], per_last_rank ? 1 : 0,
 				(double) norm_avg_decay, (double) epsilon, &h));
-		return DeviceLayer(h);
+		DeviceLayer layer(h);
+		layer.params_per_column = per_last_rank;
+		return layer;
 	}
 	/* layer/activation/<Name>ActivationLayer.hpp */
 	inline static DeviceLayer activation(cattle_hip_activation kind, const Dims& dims, Scalar param = 0) {
@@ -156,7 +159,8 @@ public:
 		return DeviceLayer(h);
 	}
 	inline DeviceLayer(DeviceLayer&& other) : handle(other.handle), in_dims(other.in_dims), out_dims(other.out_dims),
-			cached_in(std::move(other.cached_in)), cached_out(std::move(other.cached_out)) {
+			cached_in(std::move(other.cached_in)), cached_out(std::move(other.cached_out)),
+			params_per_column(other.params_per_column) {
 		other.handle = nullptr;
 	}
 	DeviceLayer(const DeviceLayer&) = delete;
@@ -274,8 +278,71 @@ public:
 	inline cattle_hip_layer_t get() const {
 		return handle;
 	}
+	/**
+	 * The layer's parameter matrices the way the reference layer's get_params() lists them: a per-channel batch
+	 * norm holds four 1x1 matrices per channel (layer/BatchNormLayer.hpp:263-272) where the device holds four
+	 * 1 x channels rows; every other layer's lists coincide. Each entry is (rows, cols, values).
+	 */
+	struct HostMatrix {
+		std::size_t rows, cols;
+		std::vector<Scalar> values;
+	};
+	inline std::vector<HostMatrix> get_reference_params() const {
+		std::vector<HostMatrix> out;
+		const std::size_t n = num_params();
+		if (!params_per_column) {
+			for (std::size_t i = 0; i < n; ++i) {
+				HostMatrix m;
+				bool opt;
+				param_shape(i, m.rows, m.cols, opt);
+				m.values = get_param_values(i);
+				out.push_back(std::move(m));
+			}
+			return out;
+		}
+		std::vector<std::vector<Scalar>> rows(n);
+		for (std::size_t i = 0; i < n; ++i)
+			rows[i] = get_param_values(i);
+		for (std::size_t c = 0; c < rows[0].size(); ++c)
+			for (std::size_t i = 0; i < n; ++i)
+				out.push_back(HostMatrix{ 1, 1, std::vector<Scalar>(1, rows[i][c]) });
+		return out;
+	}
+	/** The inverse of get_reference_params(): consumes this layer's matrices from `mats` starting at `pos`. */
+	inline void set_reference_params(const std::vector<HostMatrix>& mats, std::size_t& pos) {
+		const std::size_t n = num_params();
+		for (std::size_t i = 0; i < n; ++i) {
+			std::size_t rows, cols;
+			bool opt;
+			param_shape(i, rows, cols, opt);
+			if (!params_per_column) {
+				if (pos >= mats.size() || mats[pos].rows != rows || mats[pos].cols != cols)
+					throw std::runtime_error("parameter matrix of unexpected dimensions");
+				set_param_values(i, mats[pos++].values.data());
+			}
+		}
+		if (params_per_column && n > 0) {
+			std::size_t rows, cols;
+			bool opt;
+			param_shape(0, rows, cols, opt);
+			if (pos + n * cols > mats.size())
+				throw std::runtime_error("too few parameter matrices");
+			std::vector<std::vector<Scalar>> vals(n, std::vector<Scalar>(cols));
+			for (std::size_t c = 0; c < cols; ++c)
+				for (std::size_t i = 0; i < n; ++i) {
+					const HostMatrix& m = mats[pos++];
+					if (m.rows != 1 || m.cols != 1)
+						throw std::runtime_error("parameter matrix of unexpected dimensions");
+					vals[i][c] = m.values[0];
+				}
+			for (std::size_t i = 0; i < n; ++i)
+				set_param_values(i, vals[i].data());
+			if (n == 4)       /* running statistics were loaded: the layer may infer (BatchNormLayer.hpp:234-243) */
+				check(cattle_hip_batchnorm_set_stats_initialized(handle, 1));
+		}
+	}
 private:
-	inline explicit DeviceLayer(cattle_hip_layer_t handle) : handle(handle) {
+	inline explicit DeviceLayer(cattle_hip_layer_t handle) : handle(handle), params_per_column(false) {
 		std::size_t d[3];
 		check(cattle_hip_layer_input_dims(handle, d));
 		in_dims = Dims{ { d[0], d[1], d[2] } };
@@ -287,7 +354,7 @@ private:
 		in_dims = in;
 	}
 	inline DeviceLayer(cattle_hip_layer_t handle, const Dims& in, const Dims& out) : handle(handle), in_dims(in),
-			out_dims(out) { }
+			out_dims(out), params_per_column(false) { }
 	template<typename Fn>
 	inline void for_each_optimizable(Fn fn) {
 		const std::size_t n = num_params();
@@ -310,6 +377,7 @@ private:
 	cattle_hip_layer_t handle;
 	Dims in_dims, out_dims;
 	DeviceTensor<Scalar> cached_in, cached_out;
+	bool params_per_column;
 };
 
 /** Loss::function / d_function on device tensors (loss/UniversalLoss.hpp:27-55, non-sequential data). */
@@ -356,6 +424,59 @@ public:
 	}
 	inline std::vector<DeviceLayer<Scalar>>& get_layers() {
 		return layers;
+	}
+	/**
+	 * NeuralNetwork::save_all_unique_params_values / load_all_unique_params_values in the binary format
+	 * (core/NeuralNetwork.hpp:195-223): one file <dir>/<prefix><i>.prms per parameter matrix in get_params() order,
+	 * each an unsigned short scalar size, unsigned rows, unsigned cols and the column-major coefficients
+	 * (core/EigenProxy.hpp:147-159, :212-224), so that networks trained by either side resume on the other.
+	 */
+	inline void save_all_unique_params_values(const std::string& dir_path,
+			const std::string& file_name_prefix = "c-attl3_neural_net_params_") const {
+		std::size_t index = 0;
+		for (std::size_t l = 0; l < layers.size(); ++l) {
+			const std::vector<typename DeviceLayer<Scalar>::HostMatrix> mats = layers[l].get_reference_params();
+			for (std::size_t i = 0; i < mats.size(); ++i) {
+				std::ofstream out(dir_path + "/" + file_name_prefix + std::to_string(index++) + ".prms", std::ios::binary);
+				if (!out.is_open())
+					throw std::runtime_error("cannot write a parameter file under " + dir_path);
+				const unsigned short scalar_size = (unsigned short) sizeof(Scalar);
+				const unsigned rows = (unsigned) mats[i].rows, cols = (unsigned) mats[i].cols;
+				out.write(reinterpret_cast<const char*>(&scalar_size), sizeof(scalar_size));
+				out.write(reinterpret_cast<const char*>(&rows), sizeof(rows));
+				out.write(reinterpret_cast<const char*>(&cols), sizeof(cols));
+				out.write(reinterpret_cast<const char*>(mats[i].values.data()), (std::streamsize) (mats[i].values.size() * sizeof(Scalar)));
+			}
+		}
+	}
+	inline void load_all_unique_params_values(const std::string& dir_path,
+			const std::string& file_name_prefix = "c-attl3_neural_net_params_") {
+		std::vector<typename DeviceLayer<Scalar>::HostMatrix> mats;
+		for (;;) {
+			std::ifstream in(dir_path + "/" + file_name_prefix + std::to_string(mats.size()) + ".prms", std::ios::binary);
+			if (!in.is_open())
+				break;
+			unsigned short scalar_size = 0;
+			unsigned rows = 0, cols = 0;
+			in.read(reinterpret_cast<char*>(&scalar_size), sizeof(scalar_size));
+			in.read(reinterpret_cast<char*>(&rows), sizeof(rows));
+			in.read(reinterpret_cast<char*>(&cols), sizeof(cols));
+			if (!in || scalar_size != sizeof(Scalar))          /* assert(scalar_size == sizeof(Scalar)) */
+				throw std::runtime_error("parameter file of another scalar type or truncated");
+			typename DeviceLayer<Scalar>::HostMatrix m;
+			m.rows = rows;
+			m.cols = cols;
+			m.values.resize((std::size_t) rows * cols);
+			in.read(reinterpret_cast<char*>(m.values.data()), (std::streamsize) (m.values.size() * sizeof(Scalar)));
+			if (!in)
+				throw std::runtime_error("truncated parameter file");
+			mats.push_back(std::move(m));
+		}
+		std::size_t pos = 0;
+		for (std::size_t l = 0; l < layers.size(); ++l)
+			layers[l].set_reference_params(mats, pos);
+		if (pos != mats.size())
+			throw std::runtime_error("more parameter files than the network has parameters");
 	}
 	/** propagate: `input` must stay alive and unmodified until backpropagate returns. */
 	inline const DeviceTensor<Scalar>& propagate(const DeviceTensor<Scalar>& input, bool training) {

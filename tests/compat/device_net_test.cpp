@@ -97,6 +97,8 @@ static std::vector<Scalar> one_hot(std::size_t batch, std::size_t classes, Lcg& 
 	return y;
 }
 
+static std::string g_dir;      /* scratch directory for parameter files */
+
 template<typename Scalar>
 static void run(const std::string& tag) {
 	typedef DeviceTensor<Scalar> DT;
@@ -146,6 +148,18 @@ static void run(const std::string& tag) {
 		/* inference after training uses the running statistics */
 		const DT& out = net.propagate(xd, false);
 		record(tag + ".convnet.infer", sizeof(Scalar), { batch, 5 }, out.to_host().data());
+		/* the reference's parameter files: written, then read back by a fresh network, which must infer alike */
+		net.save_all_unique_params_values(g_dir, tag + "_params_");
+		std::vector<DL> twin_layers;
+		twin_layers.push_back(DL::conv(Dims{ { 8, 8, 3 } }, 8));
+		twin_layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, twin_layers.back().get_output_dims()));
+		twin_layers.push_back(DL::pool(CATTLE_HIP_POOL_MAX, twin_layers.back().get_output_dims()));
+		twin_layers.push_back(DL::batch_norm(twin_layers.back().get_output_dims()));
+		twin_layers.push_back(DL::dense(twin_layers.back().get_output_dims(), 5));
+		DeviceFeedforwardNetwork<Scalar> twin(std::move(twin_layers));
+		twin.load_all_unique_params_values(g_dir, tag + "_params_");
+		const DT& out2 = twin.propagate(xd, false);
+		record(tag + ".convnet.reloaded_infer", sizeof(Scalar), { batch, 5 }, out2.to_host().data());
 	}
 }
 
@@ -196,10 +210,11 @@ static void run_lstm(const std::string& tag) {
 }
 
 int main(int argc, char** argv) {
-	if (argc != 2) {
-		std::fprintf(stderr, "usage: %s <records file>\n", argv[0]);
+	if (argc != 3) {
+		std::fprintf(stderr, "usage: %s <records file> <scratch directory>\n", argv[0]);
 		return 2;
 	}
+	g_dir = argv[2];
 	try {
 		check(cattle_hip_init(0));
 		g_out = std::fopen(argv[1], "wb");

@@ -30,9 +30,12 @@ def test_device_net_compiles_as_cpp11():
 def records(tmp_path_factory):
     if not os.path.exists(BINARY):
         pytest.fail("tests/compat/device_net_test is not built: run __graft_entry__.build()")
-    out = str(tmp_path_factory.mktemp("device_net") / "records.bin")
-    subprocess.check_call([BINARY, out], timeout=120)
-    return _read_records(out)
+    tmp = tmp_path_factory.mktemp("device_net")
+    out = str(tmp / "records.bin")
+    subprocess.check_call([BINARY, out, str(tmp)], timeout=120)
+    recs = _read_records(out)
+    recs["__dir__"] = str(tmp)
+    return recs
 
 
 def _replay(r, net, lr, adam, steps=3):
@@ -114,3 +117,32 @@ def test_convlstm_sequence(records, tag, tol):
         assert hp.rel_err(r["db%d" % k], layer.get_params()[1].get_grad()) < tol, k
     lr = float(np.float32(0.05)) if tag == "f32" else 0.05
     assert hp.rel_err(r["w3_updated"], r["w3"] - lr * orc.kernels()[3].get_params()[0].get_grad()) < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,dtype", [("f32", np.float32), ("f64", np.float64)])
+def test_parameter_files_have_the_reference_format(records, tag, dtype):
+    """save_all_unique_params_values writes what core/EigenProxy.hpp:147-159 writes (unsigned short scalar size,
+    unsigned rows, unsigned cols, column-major coefficients), one file per matrix of get_params() - the per-channel
+    batch norm as four 1x1 matrices per channel - and a fresh network that loads them infers bit for bit alike."""
+    import struct
+    r = {k[len(tag) + 9:]: v for k, v in records.items() if k.startswith(tag + ".convnet.")}
+    mats = []
+    i = 0
+    while True:
+        path = os.path.join(records["__dir__"], "%s_params_%d.prms" % (tag, i))
+        if not os.path.exists(path):
+            break
+        raw = open(path, "rb").read()
+        size, rows, cols = struct.unpack("<HII", raw[:10])
+        assert size == np.dtype(dtype).itemsize and len(raw) == 10 + size * rows * cols
+        mats.append(np.frombuffer(raw[10:], dtype=dtype).reshape((rows, cols), order="F"))
+        i += 1
+    # conv (weights, bias), 8 channels x (mean, inverse sd, gamma, beta), dense (weights, bias)
+    assert [m.shape for m in mats] == [(27, 8), (1, 8)] + [(1, 1)] * 32 + [(128, 5), (1, 5)]
+    assert np.array_equal(mats[0], r["final.0.0"]) and np.array_equal(mats[1], r["final.0.1"])
+    for c in range(8):
+        for k in range(4):
+            assert mats[2 + 4 * c + k][0, 0] == r["final.3.%d" % k][0, c]
+    assert np.array_equal(mats[34], r["final.4.0"]) and np.array_equal(mats[35], r["final.4.1"])
+    assert np.array_equal(r["reloaded_infer"], r["infer"])
