@@ -154,7 +154,22 @@ struct GatherLaunch {
 	int mtiles, tile_rows;
 	int main_count, main_blocks;
 	int split_count, ksplit, chunks_per_part;
+	int sample_blocks;      /* > 0: tile rows are blocks of 32 samples x BM / 32 positions, see tile_row_m */
 };
+
+/* Row `row` of M tile `tile` as an index m = n + N * (a + OA * b) of the GEMM. Plain order: the tile is BM
+ * consecutive m (BM consecutive samples of one output position when N >= BM). Blocked order (sample_blocks =
+ * N / 32 > 0, needs N % 32 == 0 and OA % (BM / 32) == 0): the tile is 32 samples of BM / 32 positions that
+ * follow one another along a, so that the receptor fields of its rows overlap and a tile touches about half
+ * as many distinct input bytes; tiles of one column b are numbered sample block fastest. Rows stay groups
+ * of 32 consecutive samples, so vector accesses along n are unaffected. */
+__device__ __forceinline__ int tile_row_m(const GatherLaunch& L, const GatherGeom& g, int tile, int BM, int row) {
+	if (L.sample_blocks == 0)
+		return tile * BM + row;
+	const int col = tile / L.tile_rows, r = tile - col * L.tile_rows;
+	const int ab = r / L.sample_blocks, nb = r - ab * L.sample_blocks;
+	return nb * 32 + (row & 31) + g.N * (ab * (BM / 32) + (row >> 5) + g.OA * col);
+}
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
@@ -196,7 +211,6 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	if (L.tile_rows > 0)
 		tile = swizzle_tile(tile, L.tile_rows, L.mtiles / L.tile_rows);
 	const int tid = threadIdx.x;
-	const int m0 = tile * BM;
 	const int f0 = blockIdx.y * BF;
 	/* this block's chunks of the reduction: all of them, or one part */
 	const int chunk0 = split ? part * L.chunks_per_part : 0;
@@ -231,7 +245,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 
 	/* --- per-thread gather state: a fixed group of VEC rows m --- */
 	const int acol = tid % ACOLS, arow0 = tid / ACOLS;
-	const int m = m0 + acol * VEC;
+	const int m = tile_row_m(L, g, tile, BM, acol * VEC);
 	const bool mvalid = m < g.M;
 	int n, ya0, yb0;
 	{
@@ -393,7 +407,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		return;
 	}
 	const bool vec_out = g.M % MB == 0 && (reinterpret_cast<uintptr_t>(out) & (VS * sizeof(T) - 1)) == 0;
-	const int mm = m0 + wm * WT_M + MB * lc;
+	const int mm = tile_row_m(L, g, tile, BM, wm * WT_M + MB * lc);
 	#pragma unroll
 	for (int i = 0; i < FB; ++i) {
 		#pragma unroll
@@ -768,8 +782,9 @@ void* split_workspace(size_t bytes) {
  * does not depend on how blocks were scheduled). One block per (walk position, f block) tile. */
 template<typename T>
 __global__ __launch_bounds__(256)
-void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ bias, T* __restrict__ out, int M, int F,
+void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ bias, T* __restrict__ out, const GatherGeom g,
 		const GatherLaunch L, int BM, int BF, int ftiles) {
+	const int M = g.M, F = g.F;
 	constexpr int V = 16 / (int) sizeof(T);             /* consecutive m per thread: one 16-byte load per part */
 	const int groups = BM * BF / (256 * V);             /* blocks per tile; tiles are multiples of 64 x 32 */
 	const int t = blockIdx.x / groups, grp = blockIdx.x % groups;
@@ -789,7 +804,7 @@ void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ b
 		for (int i = 0; i < V; ++i)
 			acc[i] += part[i];
 	}
-	const int m = tile * BM + e % BM, f = fb * BF + e / BM;
+	const int m = tile_row_m(L, g, tile, BM, e % BM), f = fb * BF + e / BM;
 	if (f >= F)
 		return;
 	const T bv = bias ? bias[f] : (T) 0;
@@ -943,6 +958,9 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	 * several columns; 0 switches the 2-D walk off */
 	const long column = (long) g.N * g.OA;
 	const int tile_rows = (column % v.bm == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE")) ? (int) (column / v.bm) : 0;
+	/* rows of a tile as 32 samples x several positions along a (see tile_row_m) where the shape allows it */
+	const int sample_blocks = (tile_rows > 0 && g.N % 32 == 0 && v.bm % 32 == 0 && g.OA % (v.bm / 32) == 0 &&
+			!std::getenv("CATTLE_HIP_NO_ROW_BLOCKS")) ? g.N / 32 : 0;
 	/* blocks the chip holds at once (registers, LDS, waves), as the runtime computes it for this kernel */
 	const int per_cu = std::max(1, v.blocks_per_cu(dyn, vec, divs));
 	const int slots = NUM_CUS * per_cu;
@@ -950,7 +968,7 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 
 	/* main_count whole tiles, the other mtiles - main_count with their reduction cut into about `ksplit` parts */
 	auto launch = [&](int main_count, int ksplit) {
-		GatherLaunch L = { mtiles, tile_rows, main_count, round_up(main_count, 8), mtiles - main_count, 1, nchunks };
+		GatherLaunch L = { mtiles, tile_rows, main_count, round_up(main_count, 8), mtiles - main_count, 1, nchunks, sample_blocks };
 		T* partials = nullptr;
 		if (L.split_count > 0) {
 			L.chunks_per_part = (nchunks + ksplit - 1) / ksplit;
@@ -962,7 +980,7 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if (L.split_count > 0) {
 			const int groups = v.bm * v.bf / (256 * (16 / (int) sizeof(T)));
 			split_reduce_kernel<T><<<dim3((unsigned) (L.split_count * ftiles * groups)), 256, 0, stream()>>>(partials, bias, out,
-					g.M, g.F, L, v.bm, v.bf, ftiles);
+					g, L, v.bm, v.bf, ftiles);
 			CATTLE_HIP_CHECK(hipGetLastError());
 		}
 	};
