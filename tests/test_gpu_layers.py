@@ -105,6 +105,44 @@ def test_conv_strided_dilated_larger():
     _check_conv((17, 19, 6, 40, 3, 2, 2, 1, 2, 3, 1, 0), 12, np.float32, seed=8)
 
 
+@pytest.mark.parametrize("dtype,N", [(np.float32, 256), (np.float64, 128)])
+def test_conv_config4_full_size(dtype, N):
+    """BASELINE config 4 at its real shape (56x56x64 -> 128 filters, 3x3 s1 p1; batch 256 in fp32): the tile
+    shapes, left-over-tile splits and weight-gradient slicing that only a problem of this size exercises.
+    Checked against the oracle run in the same precision (its own rounding is two orders below the tolerance)
+    and, independently of any oracle, through the adjoint identities <conv(x; W), g> = <x, dgrad(g; W)> =
+    <W, wgrad(x, g)> and bgrad = sum of g, evaluated in float64 on the GPU's outputs."""
+    case = (56, 56, 64, 128, 3, 3, 1, 1, 1, 1, 0, 0)
+    g = hp.rng(0xC0FFEE04)
+    x = hp.normal(g, (N, 56, 56, 64), dtype)
+    w = np.asfortranarray((g.standard_normal((576, 128)) * np.sqrt(2.0 / 576)).astype(dtype))      # He-normal
+    b = hp.uniform(g, (1, 128), -0.1, 0.1, dtype)
+    go = hp.normal(g, (N, 56, 56, 128), dtype)
+    layer = _conv_layer(dtype, case)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    out = layer.pass_forward(x, True)
+    dx = layer.pass_back(go)
+    dw, db = wp.get_grad(), bp.get_grad()
+    tol = _tol(dtype)
+    # adjoint identities (float64 accumulation of the products)
+    f64 = np.float64
+    lhs = np.vdot(np.asarray(out - b.reshape(1, 1, 1, -1), f64), np.asarray(go, f64))
+    scale = np.sqrt(float(np.vdot(np.asarray(out, f64), np.asarray(out, f64))) * float(np.vdot(np.asarray(go, f64), np.asarray(go, f64))))
+    assert abs(lhs - np.vdot(np.asarray(x, f64), np.asarray(dx, f64))) < tol * scale * 1e-2
+    assert abs(lhs - np.vdot(np.asarray(w, f64), np.asarray(dw, f64))) < tol * scale * 1e-2
+    assert hp.rel_err(db.reshape(-1), np.asarray(go, f64).reshape((-1, 128), order="F").sum(axis=0)) < tol
+    # the oracle on the same inputs
+    o_ref, cache = oracle.conv_forward(x, w, b, return_cache=True, **_geom(case))
+    assert hp.rel_err(out, o_ref) < tol
+    del out, o_ref
+    dx_ref, dw_ref, db_ref = oracle.conv_backward(x.shape, cache, w, go, **_geom(case))
+    assert hp.rel_err(dx, dx_ref) < tol
+    assert hp.rel_err(dw, dw_ref) < tol
+    assert hp.rel_err(db, db_ref) < tol
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_conv_accumulates_input_layer_and_clones(dtype):
     case = hp.REFERENCE_CONV_CASES[5]
@@ -307,6 +345,46 @@ def test_pools(H, W, C, RH, RW, sv, sh, dtype):
     assert hp.rel_err(mn.pass_back(go), oracle.meanpool_backward(x.shape, np.asarray(go, np.float64), RH, RW, sv, sh)) < tol
     mx.set_input_layer(True)
     assert mx.pass_back(go) is None
+
+
+def test_pointwise_layers_at_the_config4_activation_shape():
+    """Batch norm, ReLU and both pools on a 256 x 56 x 56 x 64 tensor (51 M elements, the shape the bandwidth
+    figures are quoted on): the multi-block reductions and grid-stride loops only a tensor this large exercises."""
+    dtype = np.float32
+    shape = (256, 56, 56, 64)
+    g = hp.rng(61)
+    x = hp.normal(g, shape, dtype, std=1.5) + dtype(0.3)
+    go = hp.normal(g, shape, dtype)
+    x64, go64 = np.asarray(x, np.float64), np.asarray(go, np.float64)
+    # batch norm, training pass and backward
+    bn = ch.BatchNormLayer(dtype, shape[1:])
+    gamma = (1 + 0.2 * g.standard_normal(64)).astype(dtype)
+    beta = (0.1 * g.standard_normal(64)).astype(dtype)
+    prm = bn.get_params()
+    prm[2].set_values(gamma.reshape(1, -1))
+    prm[3].set_values(beta.reshape(1, -1))
+    am, ais = np.zeros(64), np.zeros(64)
+    y_ref, std_ref, isd_ref = oracle.bn_forward(x64, np.asarray(gamma, np.float64), np.asarray(beta, np.float64), am, ais, False, True)
+    dx_ref, dg_ref, db_ref = oracle.bn_backward(go64, np.asarray(gamma, np.float64), std_ref, isd_ref)
+    assert hp.rel_err(bn.pass_forward(x, True), y_ref) < 1e-4
+    assert hp.rel_err(bn.pass_back(go), dx_ref) < 1e-3          # differences of O(L)-sized terms, L = 802,816
+    assert hp.rel_err(prm[2].get_grad().reshape(-1), dg_ref) < 1e-4 and hp.rel_err(prm[3].get_grad().reshape(-1), db_ref) < 1e-4
+    assert hp.rel_err(prm[0].get_values().reshape(-1), am) < 1e-4 and hp.rel_err(prm[1].get_values().reshape(-1), ais) < 1e-4
+    del y_ref, std_ref, dx_ref
+    # ReLU: selection, exact
+    relu = ch.ActivationLayer(dtype, "relu", shape[1:])
+    assert np.array_equal(relu.pass_forward(x, True), np.maximum(x, 0))
+    assert np.array_equal(relu.pass_back(go), np.where(x >= 0, go, dtype(0)))
+    # pools: max is a selection (exact, indices bit-exact); mean within tolerance
+    gp = hp.normal(g, (256, 28, 28, 64), dtype)
+    mx = ch.MaxPoolLayer(dtype, shape[1:])
+    o_ref, i_ref = oracle.maxpool_forward(x)
+    assert np.array_equal(mx.pass_forward(x, True), o_ref)
+    assert np.array_equal(mx.max_indices(256), i_ref)
+    assert np.array_equal(mx.pass_back(gp), oracle.maxpool_backward(shape, gp, i_ref))
+    mean = ch.MeanPoolLayer(dtype, shape[1:])
+    assert hp.rel_err(mean.pass_forward(x, True), oracle.meanpool_forward(x64)) < 1e-4
+    assert hp.rel_err(mean.pass_back(gp), oracle.meanpool_backward(shape, np.asarray(gp, np.float64))) < 1e-4
 
 
 def test_maxpool_nan_and_neg_inf_windows():
