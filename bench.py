@@ -156,7 +156,7 @@ def pointwise_run(args, dtype):
     add("meanpool 2x2 forward", timed(lambda: mn.forward_into(x, yp, True)), es + es / 4.0)
     add("meanpool 2x2 backward", timed(lambda: mn.backward_into(gp, dx)), es + es / 4.0)
     bn = ch.BatchNormLayer(dtype, (H, W, C))
-    add("batchnorm forward (training)", timed(lambda: bn.forward_into(x, y, True)), 5 * es)
+    add("batchnorm forward (training)", timed(lambda: bn.forward_into(x, y, True)), 4 * es)
     add("batchnorm backward", timed(lambda: bn.backward_into(g, dx)), 5 * es)
     return rows
 

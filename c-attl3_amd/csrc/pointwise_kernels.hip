@@ -280,22 +280,84 @@ void param_act_backward_kernel(int N, int V, const T* __restrict__ param, const 
 /* ----------------------------------------------------------------------------------------------
  * Batch norm (layer/BatchNormLayer.hpp:225-262 per channel, :411-456 per activation).
  * A statistics group is a contiguous slab of L elements. grid = (groups, splits); split s covers
- * [s*span, (s+1)*span) of the slab. Mean and variance are two separate passes (the variance is the
- * mean of squared *centred* values, as in the reference), each a shuffle + LDS block reduction
- * followed by an ascending sum of the per-split partials.
+ * [s*span, (s+1)*span) of the slab. Mean and variance (the mean of squared *centred* values, as in the
+ * reference) come from one pass that merges per-thread, per-block and per-split moments in fixed orders.
  * -------------------------------------------------------------------------------------------- */
+/* (count, mean, sum of squared deviations from the mean) of set b merged into those of set a (Chan, Golub,
+ * LeVeque): exact in real arithmetic and as well conditioned as the two-pass formula, so the variance is the
+ * mean of squared *centred* values, as in the reference, from a single read of the data. */
 template<typename T>
+__device__ __forceinline__ void moments_merge(T& n, T& mean, T& m2, T nb, T meanb, T m2b) {
+	const T nt = n + nb;
+	if (nt > (T) 0) {
+		const T d = meanb - mean, w = nb / nt;
+		mean += d * w;
+		m2 += m2b + (d * d) * (n * w);
+		n = nt;
+	}
+}
+
+template<typename T, int V> struct VecOf { typedef T type __attribute__((ext_vector_type(V))); };
+
+/* Per-split moments of a slab: every thread merges groups of eight values (group mean, then centred squares,
+ * both from registers), the 256 threads are merged pairwise in a fixed tree. V values per memory access;
+ * for V > 1 the slab length, the span and the pointers are multiples of V values. */
+template<typename T, int V>
 __global__ __launch_bounds__(256)
-void bn_sum_kernel(size_t L, size_t span, const T* __restrict__ x, T* __restrict__ ws_sum) {
-	__shared__ T lds[4];
+void bn_moments_kernel(size_t L, size_t span, const T* __restrict__ x, T* __restrict__ ws_mean, T* __restrict__ ws_m2) {
+	__shared__ T lds[3][256];
+	constexpr int G = 8, NV = G / V;
+	typedef typename VecOf<T, V>::type vt;
 	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
 	const T* xs = x + (size_t) blockIdx.x * L;
-	T s = (T) 0;
-	for (size_t i = begin + threadIdx.x; i < end; i += 256)
-		s += xs[i];
-	s = block_sum_256(s, lds);
-	if (threadIdx.x == 0)
-		ws_sum[(size_t) blockIdx.x * gridDim.y + blockIdx.y] = s;
+	T n = (T) 0, mean = (T) 0, m2 = (T) 0;
+	for (size_t i0 = begin + (size_t) threadIdx.x * V; i0 < end; i0 += (size_t) 256 * G) {
+		T v[G];
+		int cnt = 0;
+		#pragma unroll
+		for (int u = 0; u < NV; ++u) {
+			const size_t i = i0 + (size_t) u * 256 * V;
+			const bool in = i < end;
+			vt a = {0};
+			if (in)
+				a = *reinterpret_cast<const vt*>(xs + i);
+			#pragma unroll
+			for (int e = 0; e < V; ++e)
+				v[u * V + e] = a[e];
+			cnt += in ? V : 0;
+		}
+		T sum = (T) 0;
+		#pragma unroll
+		for (int u = 0; u < G; ++u)
+			sum += v[u];
+		const T gm = sum / (T) cnt;
+		T q = (T) 0;
+		#pragma unroll
+		for (int u = 0; u < G; ++u) {
+			const T d = u < cnt ? v[u] - gm : (T) 0;        /* values past the end are the trailing ones */
+			q += d * d;
+		}
+		moments_merge(n, mean, m2, (T) cnt, gm, q);
+	}
+	const int tid = threadIdx.x;
+	lds[0][tid] = n;
+	lds[1][tid] = mean;
+	lds[2][tid] = m2;
+	__syncthreads();
+	for (int off = 128; off > 0; off >>= 1) {
+		if (tid < off) {
+			T a_n = lds[0][tid], a_mean = lds[1][tid], a_m2 = lds[2][tid];
+			moments_merge(a_n, a_mean, a_m2, lds[0][tid + off], lds[1][tid + off], lds[2][tid + off]);
+			lds[0][tid] = a_n;
+			lds[1][tid] = a_mean;
+			lds[2][tid] = a_m2;
+		}
+		__syncthreads();
+	}
+	if (tid == 0) {
+		ws_mean[(size_t) blockIdx.x * gridDim.y + blockIdx.y] = lds[1][0];
+		ws_m2[(size_t) blockIdx.x * gridDim.y + blockIdx.y] = lds[2][0];
+	}
 }
 
 template<typename T>
@@ -306,25 +368,20 @@ __device__ __forceinline__ T sum_partials(const T* ws, int splits) {
 	return s;
 }
 
+/* Mean and biased variance of a slab from its per-split moments, merged in ascending order. */
 template<typename T>
-__global__ __launch_bounds__(256)
-void bn_sqdev_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __restrict__ ws_sum, T* __restrict__ ws_sq) {
-	__shared__ T lds[4];
-	const int splits = gridDim.y;
-	const T mean = sum_partials(ws_sum + (size_t) blockIdx.x * splits, splits) / (T) L;
-	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
-	const T* xs = x + (size_t) blockIdx.x * L;
-	T s = (T) 0;
-	for (size_t i = begin + threadIdx.x; i < end; i += 256) {
-		const T d = xs[i] - mean;
-		s += d * d;
+__device__ __forceinline__ void slab_moments(const T* ws_mean, const T* ws_m2, int splits, size_t L, size_t span, T& mean, T& var) {
+	T n = (T) 0, m2 = (T) 0;
+	mean = (T) 0;
+	for (int p = 0; p < splits; ++p) {
+		const size_t begin = (size_t) p * span;
+		const size_t cnt = begin >= L ? 0 : (begin + span < L ? span : L - begin);
+		moments_merge(n, mean, m2, (T) cnt, ws_mean[p], ws_m2[p]);
 	}
-	s = block_sum_256(s, lds);
-	if (threadIdx.x == 0)
-		ws_sq[(size_t) blockIdx.x * splits + blockIdx.y] = s;
+	var = m2 / (T) L;
 }
 
-template<typename T>
+template<typename T, int V>
 __global__ __launch_bounds__(256)
 void bn_train_apply_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __restrict__ gamma,
 		const T* __restrict__ beta, T* __restrict__ avg_mean, T* __restrict__ avg_inv_sd, bool stats_init, T decay, T eps,
@@ -332,17 +389,25 @@ void bn_train_apply_kernel(size_t L, size_t span, const T* __restrict__ x, const
 		T* __restrict__ inv_sd_cache) {
 	const int splits = gridDim.y;
 	const int grp = blockIdx.x;
-	const T mean = sum_partials(ws_sum + (size_t) grp * splits, splits) / (T) L;
-	const T inv_sd = (T) 1 / dev_sqrt(sum_partials(ws_sq + (size_t) grp * splits, splits) / (T) L + eps);
+	T mean, var;
+	slab_moments(ws_sum + (size_t) grp * splits, ws_sq + (size_t) grp * splits, splits, L, span, mean, var);
+	const T inv_sd = (T) 1 / dev_sqrt(var + eps);
 	const T ga = gamma[grp], be = beta[grp];
 	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
 	const T* xs = x + (size_t) grp * L;
 	T* ys = out + (size_t) grp * L;
 	T* sc = std_cache + (size_t) grp * L;
-	for (size_t i = begin + threadIdx.x; i < end; i += 256) {
-		const T sv = (xs[i] - mean) * inv_sd;
-		sc[i] = sv;
-		ys[i] = sv * ga + be;
+	typedef typename VecOf<T, V>::type vt;
+	for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
+		const vt xv = *reinterpret_cast<const vt*>(xs + i);
+		vt sv, yv;
+		#pragma unroll
+		for (int e = 0; e < V; ++e) {
+			sv[e] = (xv[e] - mean) * inv_sd;
+			yv[e] = sv[e] * ga + be;
+		}
+		*reinterpret_cast<vt*>(sc + i) = sv;
+		*reinterpret_cast<vt*>(ys + i) = yv;
 	}
 	if (blockIdx.y == 0 && threadIdx.x == 0) {
 		inv_sd_cache[grp] = inv_sd;
@@ -356,7 +421,7 @@ void bn_train_apply_kernel(size_t L, size_t span, const T* __restrict__ x, const
 	}
 }
 
-template<typename T>
+template<typename T, int V>
 __global__ __launch_bounds__(256)
 void bn_infer_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
 		const T* __restrict__ avg_mean, const T* __restrict__ avg_inv_sd, T* __restrict__ out) {
@@ -365,11 +430,18 @@ void bn_infer_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __
 	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
 	const T* xs = x + (size_t) grp * L;
 	T* ys = out + (size_t) grp * L;
-	for (size_t i = begin + threadIdx.x; i < end; i += 256)
-		ys[i] = ((xs[i] - mean) * inv_sd) * ga + be;
+	typedef typename VecOf<T, V>::type vt;
+	for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
+		const vt xv = *reinterpret_cast<const vt*>(xs + i);
+		vt yv;
+		#pragma unroll
+		for (int e = 0; e < V; ++e)
+			yv[e] = ((xv[e] - mean) * inv_sd) * ga + be;
+		*reinterpret_cast<vt*>(ys + i) = yv;
+	}
 }
 
-template<typename T>
+template<typename T, int V>
 __global__ __launch_bounds__(256)
 void bn_backward_sums_kernel(size_t L, size_t span, const T* __restrict__ g, const T* __restrict__ std_cache,
 		T* __restrict__ ws_g, T* __restrict__ ws_gs) {
@@ -377,11 +449,29 @@ void bn_backward_sums_kernel(size_t L, size_t span, const T* __restrict__ g, con
 	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
 	const T* gs = g + (size_t) blockIdx.x * L;
 	const T* sc = std_cache + (size_t) blockIdx.x * L;
+	typedef typename VecOf<T, V>::type vt;
+	constexpr int U = 4;        /* independent accesses in flight per thread and operand */
 	T s1 = (T) 0, s2 = (T) 0;
-	for (size_t i = begin + threadIdx.x; i < end; i += 256) {
-		const T gi = gs[i];
-		s1 += gi;
-		s2 += gi * sc[i];
+	for (size_t i0 = begin + (size_t) threadIdx.x * V; i0 < end; i0 += (size_t) 256 * V * U) {
+		vt gv[U], cv[U];
+		#pragma unroll
+		for (int u = 0; u < U; ++u) {
+			const size_t i = i0 + (size_t) u * 256 * V;
+			gv[u] = vt{0};
+			cv[u] = vt{0};
+			if (i < end) {
+				gv[u] = *reinterpret_cast<const vt*>(gs + i);
+				cv[u] = *reinterpret_cast<const vt*>(sc + i);
+			}
+		}
+		#pragma unroll
+		for (int u = 0; u < U; ++u) {
+			#pragma unroll
+			for (int e = 0; e < V; ++e) {
+				s1 += gv[u][e];
+				s2 += gv[u][e] * cv[u][e];
+			}
+		}
 	}
 	s1 = block_sum_256(s1, lds);
 	s2 = block_sum_256(s2, lds);
@@ -391,7 +481,7 @@ void bn_backward_sums_kernel(size_t L, size_t span, const T* __restrict__ g, con
 	}
 }
 
-template<typename T>
+template<typename T, int V>
 __global__ __launch_bounds__(256)
 void bn_backward_apply_kernel(size_t L, size_t span, const T* __restrict__ g, const T* __restrict__ gamma,
 		const T* __restrict__ std_cache, const T* __restrict__ inv_sd_cache, const T* __restrict__ ws_g,
@@ -413,8 +503,16 @@ void bn_backward_apply_kernel(size_t L, size_t span, const T* __restrict__ g, co
 	const T* gs = g + (size_t) grp * L;
 	const T* sc = std_cache + (size_t) grp * L;
 	T* dx = in_grad + (size_t) grp * L;
-	for (size_t i = begin + threadIdx.x; i < end; i += 256)
-		dx[i] = (((T) L * (gs[i] * ga) - sum_sg) - sc[i] * sum_ssg) * scale;
+	typedef typename VecOf<T, V>::type vt;
+	for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
+		const vt gv = *reinterpret_cast<const vt*>(gs + i);
+		const vt cv = *reinterpret_cast<const vt*>(sc + i);
+		vt o;
+		#pragma unroll
+		for (int e = 0; e < V; ++e)
+			o[e] = (((T) L * (gv[e] * ga) - sum_sg) - cv[e] * sum_ssg) * scale;
+		*reinterpret_cast<vt*>(dx + i) = o;
+	}
 }
 
 constexpr int BN_MAX_SPLITS = 64;
@@ -863,41 +961,67 @@ size_t bn_workspace(int groups, size_t L) {
 	return (size_t) 2 * groups * BN_MAX_SPLITS;
 }
 
-template<typename T>
-void bn_forward(int groups, size_t L, const T* x, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd,
+/* The span of a split is a multiple of four values, so that 16-byte accesses stay aligned within a slab. */
+size_t bn_span(size_t L, int splits) {
+	const size_t span = (L + splits - 1) / splits;
+	return (span + 3) / 4 * 4;
+}
+
+template<typename T, int V>
+void bn_forward_launch(int groups, size_t L, const T* x, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd,
 		bool stats_init, bool training, T decay, T eps, T* out, T* std_cache, T* inv_sd_cache, T* ws) {
 	const int splits = bn_splits(groups, L);
-	const size_t span = (L + splits - 1) / splits;
+	const size_t span = bn_span(L, splits);
 	dim3 grid((unsigned) groups, (unsigned) splits);
 	if (training) {
 		T* ws_sum = ws;
 		T* ws_sq = ws + (size_t) groups * BN_MAX_SPLITS;
-		bn_sum_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, ws_sum);
+		bn_moments_kernel<T, V><<<grid, 256, 0, stream()>>>(L, span, x, ws_sum, ws_sq);
 		check_launch();
-		bn_sqdev_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, ws_sum, ws_sq);
-		check_launch();
-		bn_train_apply_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, gamma, beta, avg_mean, avg_inv_sd, stats_init, decay,
+		bn_train_apply_kernel<T, V><<<grid, 256, 0, stream()>>>(L, span, x, gamma, beta, avg_mean, avg_inv_sd, stats_init, decay,
 				eps, ws_sum, ws_sq, out, std_cache, inv_sd_cache);
 		check_launch();
 	} else {
-		bn_infer_kernel<T><<<grid, 256, 0, stream()>>>(L, span, x, gamma, beta, avg_mean, avg_inv_sd, out);
+		bn_infer_kernel<T, V><<<grid, 256, 0, stream()>>>(L, span, x, gamma, beta, avg_mean, avg_inv_sd, out);
 		check_launch();
 	}
 }
 
 template<typename T>
-void bn_backward(int groups, size_t L, const T* out_grad, const T* gamma, const T* std_cache, const T* inv_sd_cache,
+void bn_forward(int groups, size_t L, const T* x, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd,
+		bool stats_init, bool training, T decay, T eps, T* out, T* std_cache, T* inv_sd_cache, T* ws) {
+	constexpr int V = Pack<T>::V;
+	if (L % V == 0 && aligned16(x) && aligned16(out) && (!training || aligned16(std_cache)))
+		bn_forward_launch<T, V>(groups, L, x, gamma, beta, avg_mean, avg_inv_sd, stats_init, training, decay, eps, out, std_cache,
+				inv_sd_cache, ws);
+	else
+		bn_forward_launch<T, 1>(groups, L, x, gamma, beta, avg_mean, avg_inv_sd, stats_init, training, decay, eps, out, std_cache,
+				inv_sd_cache, ws);
+}
+
+template<typename T, int V>
+void bn_backward_launch(int groups, size_t L, const T* out_grad, const T* gamma, const T* std_cache, const T* inv_sd_cache,
 		T* gamma_grad, T* beta_grad, T* in_grad, T* ws) {
 	const int splits = bn_splits(groups, L);
-	const size_t span = (L + splits - 1) / splits;
+	const size_t span = bn_span(L, splits);
 	dim3 grid((unsigned) groups, (unsigned) splits);
 	T* ws_g = ws;
 	T* ws_gs = ws + (size_t) groups * BN_MAX_SPLITS;
-	bn_backward_sums_kernel<T><<<grid, 256, 0, stream()>>>(L, span, out_grad, std_cache, ws_g, ws_gs);
+	bn_backward_sums_kernel<T, V><<<grid, 256, 0, stream()>>>(L, span, out_grad, std_cache, ws_g, ws_gs);
 	check_launch();
-	bn_backward_apply_kernel<T><<<grid, 256, 0, stream()>>>(L, span, out_grad, gamma, std_cache, inv_sd_cache, ws_g, ws_gs,
+	bn_backward_apply_kernel<T, V><<<grid, 256, 0, stream()>>>(L, span, out_grad, gamma, std_cache, inv_sd_cache, ws_g, ws_gs,
 			gamma_grad, beta_grad, in_grad);
 	check_launch();
+}
+
+template<typename T>
+void bn_backward(int groups, size_t L, const T* out_grad, const T* gamma, const T* std_cache, const T* inv_sd_cache,
+		T* gamma_grad, T* beta_grad, T* in_grad, T* ws) {
+	constexpr int V = Pack<T>::V;
+	if (L % V == 0 && aligned16(out_grad) && aligned16(std_cache) && (!in_grad || aligned16(in_grad)))
+		bn_backward_launch<T, V>(groups, L, out_grad, gamma, std_cache, inv_sd_cache, gamma_grad, beta_grad, in_grad, ws);
+	else
+		bn_backward_launch<T, 1>(groups, L, out_grad, gamma, std_cache, inv_sd_cache, gamma_grad, beta_grad, in_grad, ws);
 }
 
 /* float tensors use 4 samples per thread (16-byte accesses) when possible; doubles use 2 */
