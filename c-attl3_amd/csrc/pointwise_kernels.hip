@@ -90,11 +90,11 @@ void act_forward_kernel(size_t n, T p, const T* __restrict__ x, T* __restrict__ 
 	const size_t nv = n / V;
 	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
 		if constexpr (VECTOR) {
-			vt a = reinterpret_cast<const vt*>(x)[i], o;
+			vt a = __builtin_nontemporal_load(reinterpret_cast<const vt*>(x) + i), o;
 			#pragma unroll
 			for (int e = 0; e < V; ++e)
 				o[e] = act_f<T, KIND>(a[e], p);
-			reinterpret_cast<vt*>(y)[i] = o;
+			__builtin_nontemporal_store(o, reinterpret_cast<vt*>(y) + i);
 		} else {
 			y[i] = act_f<T, KIND>(x[i], p);
 		}
@@ -117,14 +117,14 @@ void act_backward_kernel(size_t n, T p, const T* __restrict__ x, const T* __rest
 		if constexpr (VECTOR) {
 			vt xv = {0}, yv = {0}, o;
 			if (act_needs_x(KIND))
-				xv = reinterpret_cast<const vt*>(x)[i];
+				xv = __builtin_nontemporal_load(reinterpret_cast<const vt*>(x) + i);
 			if (act_needs_y(KIND))
-				yv = reinterpret_cast<const vt*>(y)[i];
-			const vt gv = reinterpret_cast<const vt*>(g)[i];
+				yv = __builtin_nontemporal_load(reinterpret_cast<const vt*>(y) + i);
+			const vt gv = __builtin_nontemporal_load(reinterpret_cast<const vt*>(g) + i);
 			#pragma unroll
 			for (int e = 0; e < V; ++e)
 				o[e] = act_b<T, KIND>(xv[e], yv[e], gv[e], p);
-			reinterpret_cast<vt*>(dx)[i] = o;
+			__builtin_nontemporal_store(o, reinterpret_cast<vt*>(dx) + i);
 		} else {
 			dx[i] = act_b<T, KIND>(act_needs_x(KIND) ? x[i] : (T) 0, act_needs_y(KIND) ? y[i] : (T) 0, g[i], p);
 		}
@@ -297,7 +297,7 @@ __device__ __forceinline__ void moments_merge(T& n, T& mean, T& m2, T nb, T mean
 	}
 }
 
-template<typename T, int V> struct VecOf { typedef T type __attribute__((ext_vector_type(V))); };
+template<typename T, int V> struct SlabVec { typedef T type __attribute__((ext_vector_type(V))); };
 
 /* Per-split moments of a slab: every thread merges groups of eight values (group mean, then centred squares,
  * both from registers), the 256 threads are merged pairwise in a fixed tree. V values per memory access;
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(256)
 void bn_moments_kernel(size_t L, size_t span, const T* __restrict__ x, T* __restrict__ ws_mean, T* __restrict__ ws_m2) {
 	__shared__ T lds[3][256];
 	constexpr int G = 8, NV = G / V;
-	typedef typename VecOf<T, V>::type vt;
+	typedef typename SlabVec<T, V>::type vt;
 	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
 	const T* xs = x + (size_t) blockIdx.x * L;
 	T n = (T) 0, mean = (T) 0, m2 = (T) 0;
@@ -397,17 +397,17 @@ void bn_train_apply_kernel(size_t L, size_t span, const T* __restrict__ x, const
 	const T* xs = x + (size_t) grp * L;
 	T* ys = out + (size_t) grp * L;
 	T* sc = std_cache + (size_t) grp * L;
-	typedef typename VecOf<T, V>::type vt;
+	typedef typename SlabVec<T, V>::type vt;
 	for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
-		const vt xv = *reinterpret_cast<const vt*>(xs + i);
+		const vt xv = __builtin_nontemporal_load(reinterpret_cast<const vt*>(xs + i));
 		vt sv, yv;
 		#pragma unroll
 		for (int e = 0; e < V; ++e) {
 			sv[e] = (xv[e] - mean) * inv_sd;
 			yv[e] = sv[e] * ga + be;
 		}
-		*reinterpret_cast<vt*>(sc + i) = sv;
-		*reinterpret_cast<vt*>(ys + i) = yv;
+		__builtin_nontemporal_store(sv, reinterpret_cast<vt*>(sc + i));
+		__builtin_nontemporal_store(yv, reinterpret_cast<vt*>(ys + i));
 	}
 	if (blockIdx.y == 0 && threadIdx.x == 0) {
 		inv_sd_cache[grp] = inv_sd;
@@ -430,14 +430,14 @@ void bn_infer_kernel(size_t L, size_t span, const T* __restrict__ x, const T* __
 	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
 	const T* xs = x + (size_t) grp * L;
 	T* ys = out + (size_t) grp * L;
-	typedef typename VecOf<T, V>::type vt;
+	typedef typename SlabVec<T, V>::type vt;
 	for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
-		const vt xv = *reinterpret_cast<const vt*>(xs + i);
+		const vt xv = __builtin_nontemporal_load(reinterpret_cast<const vt*>(xs + i));
 		vt yv;
 		#pragma unroll
 		for (int e = 0; e < V; ++e)
 			yv[e] = ((xv[e] - mean) * inv_sd) * ga + be;
-		*reinterpret_cast<vt*>(ys + i) = yv;
+		__builtin_nontemporal_store(yv, reinterpret_cast<vt*>(ys + i));
 	}
 }
 
@@ -449,7 +449,7 @@ void bn_backward_sums_kernel(size_t L, size_t span, const T* __restrict__ g, con
 	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < L ? begin + span : L;
 	const T* gs = g + (size_t) blockIdx.x * L;
 	const T* sc = std_cache + (size_t) blockIdx.x * L;
-	typedef typename VecOf<T, V>::type vt;
+	typedef typename SlabVec<T, V>::type vt;
 	constexpr int U = 4;        /* independent accesses in flight per thread and operand */
 	T s1 = (T) 0, s2 = (T) 0;
 	for (size_t i0 = begin + (size_t) threadIdx.x * V; i0 < end; i0 += (size_t) 256 * V * U) {
@@ -503,15 +503,15 @@ void bn_backward_apply_kernel(size_t L, size_t span, const T* __restrict__ g, co
 	const T* gs = g + (size_t) grp * L;
 	const T* sc = std_cache + (size_t) grp * L;
 	T* dx = in_grad + (size_t) grp * L;
-	typedef typename VecOf<T, V>::type vt;
+	typedef typename SlabVec<T, V>::type vt;
 	for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
-		const vt gv = *reinterpret_cast<const vt*>(gs + i);
-		const vt cv = *reinterpret_cast<const vt*>(sc + i);
+		const vt gv = __builtin_nontemporal_load(reinterpret_cast<const vt*>(gs + i));
+		const vt cv = __builtin_nontemporal_load(reinterpret_cast<const vt*>(sc + i));
 		vt o;
 		#pragma unroll
 		for (int e = 0; e < V; ++e)
 			o[e] = (((T) L * (gv[e] * ga) - sum_sg) - cv[e] * sum_ssg) * scale;
-		*reinterpret_cast<vt*>(dx + i) = o;
+		__builtin_nontemporal_store(o, reinterpret_cast<vt*>(dx + i));
 	}
 }
 
@@ -562,7 +562,7 @@ __device__ __forceinline__ void pool_store(T* p, const T (&src)[VN]) {
 		#pragma unroll
 		for (int i = 0; i < VN; ++i)
 			v[i] = src[i];
-		*reinterpret_cast<vt*>(p) = v;
+		__builtin_nontemporal_store(v, reinterpret_cast<vt*>(p));
 	}
 }
 
