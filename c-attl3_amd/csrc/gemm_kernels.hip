@@ -709,23 +709,50 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	}
 }
 
-/* dst[i] += sum_s partials[s][i]. A block covers 64 outputs with four groups of threads; group j adds
- * the partials s = j, j+4, j+8, ... in ascending order and the four group sums are then added in
- * ascending order, so the summation order is fixed and results are reproducible. */
-template<typename T>
+/* dst[i] += sum_s partials[s][i] for the weight gradient (blocks below wblocks) and the bias gradient (the
+ * remaining blocks) in one launch. A block covers 64 outputs with GR groups of threads, V consecutive outputs
+ * per thread; group j adds the partials s = j, j+GR, j+2GR, ... in ascending order and the group sums are then
+ * added in ascending order, so the summation order is fixed and results are reproducible. For V > 1 both
+ * counts are multiples of V and the partials are 16-byte aligned. */
+template<typename T, int V>
 __global__ __launch_bounds__(256)
-void reduce_partials_kernel(const T* __restrict__ partials, T* __restrict__ dst, size_t count, int splits) {
-	__shared__ T lds[4][64];
-	const int ox = threadIdx.x % 64, grp = threadIdx.x / 64;
-	const size_t i = (size_t) blockIdx.x * 64 + ox;
-	T s = (T) 0;
+void reduce_partials_kernel(const T* __restrict__ partials, T* __restrict__ dst, size_t count,
+		const T* __restrict__ bias_partials, T* __restrict__ bias_dst, size_t bias_count, int wblocks, int splits) {
+	constexpr int OV = 64 / V, GR = 256 / OV;
+	__shared__ T lds[GR][64];
+	int blk = blockIdx.x;
+	if (blk >= wblocks) {
+		blk -= wblocks;
+		partials = bias_partials;
+		dst = bias_dst;
+		count = bias_count;
+	}
+	const int ox = (threadIdx.x % OV) * V, grp = threadIdx.x / OV;
+	const size_t i = (size_t) blk * 64 + ox;
+	T s[V];
+	#pragma unroll
+	for (int e = 0; e < V; ++e)
+		s[e] = (T) 0;
 	if (i < count)
-		for (int p = grp; p < splits; p += 4)
-			s += partials[(size_t) p * count + i];
-	lds[grp][ox] = s;
+		for (int p = grp; p < splits; p += GR) {
+			T v[V];
+			vec_load<T, V>(v, partials + (size_t) p * count + i);
+			#pragma unroll
+			for (int e = 0; e < V; ++e)
+				s[e] += v[e];
+		}
+	#pragma unroll
+	for (int e = 0; e < V; ++e)
+		lds[grp][ox + e] = s[e];
 	__syncthreads();
-	if (grp == 0 && i < count)
-		dst[i] += ((lds[0][ox] + lds[1][ox]) + lds[2][ox]) + lds[3][ox];
+	const size_t o = (size_t) blk * 64 + threadIdx.x;
+	if (threadIdx.x < 64 && o < count) {
+		T total = lds[0][threadIdx.x];
+		#pragma unroll
+		for (int j = 1; j < GR; ++j)
+			total += lds[j][threadIdx.x];
+		dst[o] += total;
+	}
 }
 
 /* Forward weights: wt[k][f] = w[k + K*f], zero-padded to Kp rows x ldw columns. */
@@ -1180,12 +1207,15 @@ void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_gr
 	const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
 			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
 	v.launch(x, out_grad, partials, bias_partials, g, split, vec);
-	reduce_partials_kernel<T><<<(unsigned) ((count + 63) / 64), 256, 0, stream()>>>(partials, wgrad, count, p.splits);
+	const int wblocks = (int) ((count + 63) / 64), bblocks = bgrad ? (g.F + 63) / 64 : 0;
+	constexpr int V = 16 / (int) sizeof(T);
+	if (count % V == 0 && g.F % V == 0 && (reinterpret_cast<uintptr_t>(partials) & 15) == 0)
+		reduce_partials_kernel<T, V><<<(unsigned) (wblocks + bblocks), 256, 0, stream()>>>(partials, wgrad, count, bias_partials,
+				bgrad, (size_t) g.F, wblocks, p.splits);
+	else
+		reduce_partials_kernel<T, 1><<<(unsigned) (wblocks + bblocks), 256, 0, stream()>>>(partials, wgrad, count, bias_partials,
+				bgrad, (size_t) g.F, wblocks, p.splits);
 	CATTLE_HIP_CHECK(hipGetLastError());
-	if (bgrad) {
-		reduce_partials_kernel<T><<<(unsigned) ((g.F + 63) / 64), 256, 0, stream()>>>(bias_partials, bgrad, (size_t) g.F, p.splits);
-		CATTLE_HIP_CHECK(hipGetLastError());
-	}
 }
 
 template<typename T>
