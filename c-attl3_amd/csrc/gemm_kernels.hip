@@ -785,7 +785,6 @@ constexpr int WT_ROW_PAD = 64;     /* a multiple of every KC: the last reduction
 constexpr int WT_COL_PAD = 128;    /* >= every BF */
 constexpr int NUM_CUS = 256;
 constexpr int LDS_PER_CU = 160 * 1024;
-constexpr int MAX_WAVES_PER_CU = 16;   /* four per SIMD: every kernel here stays within 128 registers per lane */
 
 
 /* Grow-only device scratch for split reductions. Calls into the library are serialised and issued on
@@ -1067,8 +1066,9 @@ constexpr int WGRAD_MC = 32;
 
 template<typename T>
 struct WgradVariant {
-	int bk, bf, waves, lds_bytes;
+	int bk, bf, waves;
 	void (*launch)(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom&, const WgradSplit&, bool vec);
+	int (*blocks_per_cu)();         /* what the runtime says fits on a CU (registers and LDS) */
 };
 
 template<typename T, int WK, int WF, int TK, int TF>
@@ -1084,13 +1084,25 @@ void launch_wgrad_variant(const T* x, const T* og, T* partials, T* bias_partials
 }
 
 template<typename T, int WK, int WF, int TK, int TF>
+int wgrad_variant_occupancy() {
+	static int cached = 0;
+	if (cached == 0) {
+		int n = 0;
+		CATTLE_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, GemmCfg<T>::VEC>,
+				64 * WK * WF, 0));
+		cached = std::max(1, n);
+	}
+	return cached;
+}
+
+template<typename T, int WK, int WF, int TK, int TF>
 WgradVariant<T> wgrad_variant() {
 	WgradVariant<T> v;
 	v.bk = WK * TK;
 	v.bf = WF * TF;
 	v.waves = WK * WF;
-	v.lds_bytes = (v.bk + v.bf) * (WGRAD_MC + 16 / (int) sizeof(T)) * (int) sizeof(T) + v.bk * 16;
 	v.launch = &launch_wgrad_variant<T, WK, WF, TK, TF>;
+	v.blocks_per_cu = &wgrad_variant_occupancy<T, WK, WF, TK, TF>;
 	return v;
 }
 
@@ -1108,9 +1120,10 @@ template<> struct WgradVariants<float> {
 	}
 };
 template<> struct WgradVariants<double> {
-	static constexpr int COUNT = 3;
+	static constexpr int COUNT = 4;
 	static const WgradVariant<double>* get() {
 		static const WgradVariant<double> v[COUNT] = {
+			wgrad_variant<double, 2, 4, 48, 32>(),      /* 96 x 128 */
 			wgrad_variant<double, 2, 4, 48, 16>(),      /* 96 x 64 */
 			wgrad_variant<double, 2, 2, 32, 32>(),      /* 64 x 64 */
 			wgrad_variant<double, 1, 4, 32, 16>(),      /* 32 x 64 */
@@ -1125,8 +1138,9 @@ struct WgradPlan {
 
 /* The tile shape with the least padding wins (larger tile on ties: it re-reads G less often); the
  * M range is then cut into as many slices as fill the chip once (blocks = tiles * splits <= slots),
- * so that no block runs in a second, mostly idle round. The plan depends on the shape only, which
- * keeps the summation order, and with it the result, reproducible. */
+ * so that no block runs in a second, mostly idle round; the slots are what the runtime's occupancy query
+ * reports for the variant. The plan depends on the shape and the build only, which keeps the summation
+ * order, and with it the result, reproducible. */
 template<typename T>
 WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	const WgradVariant<T>* vars = WgradVariants<T>::get();
@@ -1148,7 +1162,7 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	const WgradVariant<T>& v = vars[p.variant];
 	p.ktiles = (K + v.bk - 1) / v.bk;
 	p.ftiles = (F + v.bf - 1) / v.bf;
-	const int occ = std::max(1, std::min(std::min(LDS_PER_CU / v.lds_bytes, MAX_WAVES_PER_CU / v.waves), 3));
+	const int occ = std::max(1, std::min(v.blocks_per_cu(), 3));
 	const int slots = NUM_CUS * occ;
 	const int tiles = p.ktiles * p.ftiles;
 	const int chunks = (M + WGRAD_MC - 1) / WGRAD_MC;
