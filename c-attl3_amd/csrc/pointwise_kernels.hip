@@ -681,6 +681,47 @@ void pool_backward_kernel(PoolShape s, int N, int OH, int OW, PoolLaunch pl, con
 	}
 }
 
+/* Backward pass when the windows tile the input exactly (stride = receptor, no rows or columns left over): every
+ * input position belongs to one window, so a thread takes one window, reads its upstream gradient (and argmax)
+ * once and writes the window's RH x RW input gradients. Same values as the gather form. */
+template<typename T, bool MAX, int VN>
+__global__ __launch_bounds__(256)
+void pool_backward_tiled_kernel(PoolShape s, int N, int OH, int OW, PoolLaunch pl, const T* __restrict__ g,
+		const unsigned* __restrict__ inds, T* __restrict__ dx) {
+	unsigned b = blockIdx.x;
+	const int nb = (int) (b % (unsigned) pl.nblks);
+	b /= (unsigned) pl.nblks;
+	const int rb = (int) (b % (unsigned) pl.rblks);
+	b /= (unsigned) pl.rblks;
+	const int ow = (int) (b % (unsigned) OW);
+	const int c = (int) (b / (unsigned) OW);
+	const int n = (nb * pl.tx + (int) threadIdx.x % pl.tx) * VN;
+	if (n >= N)
+		return;
+	const T area = (T) (s.RH * s.RW);
+	const int row0 = rb * pl.ty * POOL_ROWS + (int) threadIdx.x / pl.tx;
+	#pragma unroll
+	for (int j = 0; j < POOL_ROWS; ++j) {
+		const int oh = row0 + j * pl.ty;
+		if (oh >= OH)
+			break;
+		T gv[VN];
+		unsigned ind[VN];
+		pool_load<T, VN>(gv, g + (n + (size_t) N * (oh + (size_t) OH * (ow + (size_t) OW * c))));
+		if (MAX)
+			pool_load<unsigned, VN>(ind, inds + (((size_t) ow * OH + oh) * ((size_t) s.C * N) + (size_t) c * N + n));
+		T* base = dx + n + (size_t) N * ((size_t) oh * s.RH + (size_t) s.H * ((size_t) ow * s.RW + (size_t) s.W * c));
+		for (int k = 0; k < s.RW; ++k)
+			for (int l = 0; l < s.RH; ++l) {
+				T o[VN];
+				#pragma unroll
+				for (int v = 0; v < VN; ++v)
+					o[v] = MAX ? (ind[v] == (unsigned) (k * s.RH + l) ? (T) 0 + gv[v] : (T) 0) : (T) 0 + gv[v] / area;
+				pool_store<T, VN>(base + (size_t) N * (l + (size_t) s.H * k), o);
+			}
+	}
+}
+
 /* vn = samples per thread */
 PoolLaunch pool_launch(int N, int rows, int vn) {
 	const int nthreads = (N + vn - 1) / vn;
@@ -1041,7 +1082,21 @@ void pool_forward_launch(const PoolShape& s, int N, const T* x, T* out, unsigned
 template<typename T, bool MAX>
 void pool_backward_launch(const PoolShape& s, int N, const T* out_grad, const unsigned* inds, T* in_grad) {
 	constexpr int VN = 16 / (int) sizeof(T);
-	if (N % 4 == 0 && aligned16(out_grad) && aligned16(in_grad) && (!inds || aligned16(inds))) {
+	const bool vec = N % 4 == 0 && aligned16(out_grad) && aligned16(in_grad) && (!inds || aligned16(inds));
+	if (s.sv == s.RH && s.sh == s.RW && s.OH() * s.RH == s.H && s.OW() * s.RW == s.W) {
+		if (vec) {
+			const PoolLaunch pl = pool_launch(N, s.OH(), VN);
+			pool_backward_tiled_kernel<T, MAX, VN><<<pool_grid(pl, s.OW(), s.C), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), pl,
+					out_grad, inds, in_grad);
+		} else {
+			const PoolLaunch pl = pool_launch(N, s.OH(), 1);
+			pool_backward_tiled_kernel<T, MAX, 1><<<pool_grid(pl, s.OW(), s.C), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), pl,
+					out_grad, inds, in_grad);
+		}
+		check_launch();
+		return;
+	}
+	if (vec) {
 		const PoolLaunch pl = pool_launch(N, s.H, VN);
 		pool_backward_kernel<T, MAX, VN><<<pool_grid(pl, s.W, s.C), 256, 0, stream()>>>(s, N, s.OH(), s.OW(), pl, out_grad, inds,
 				in_grad);

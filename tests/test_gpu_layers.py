@@ -320,15 +320,17 @@ def test_softmax_prelu_pswish(dtype):
         assert hp.rel_err(prm.get_grad().reshape(-1), pg_ref) < tol
 
 
+# the last two: windows that tile the input exactly with a receptor other than 2x2, and a 2x2 pool that leaves
+# a row and a column of the input outside every window (their gradient is zero)
 POOL_CASES = [(8, 8, 3, 2, 2, 2, 2), (16, 16, 2, 3, 2, 1, 2), (7, 9, 2, 3, 2, 2, 3), (32, 1, 2, 3, 1, 1, 1),
-              (32, 32, 32, 2, 2, 2, 2)]
+              (32, 32, 32, 2, 2, 2, 2), (9, 8, 2, 3, 2, 3, 2), (9, 9, 2, 2, 2, 2, 2)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N", [6, 8])                # scalar and 16-byte access paths
 @pytest.mark.parametrize("H,W,C,RH,RW,sv,sh", POOL_CASES)
-def test_pools(H, W, C, RH, RW, sv, sh, dtype):
+def test_pools(H, W, C, RH, RW, sv, sh, N, dtype):
     g = hp.rng(51)
-    N = 6
     x = hp.normal(g, (N, H, W, C), dtype)
     x[:, 0:2, 0, 0] = 3.5                            # ties inside the first window
     mx = ch.MaxPoolLayer(dtype, (H, W, C), RH, RW, sv, sh)
