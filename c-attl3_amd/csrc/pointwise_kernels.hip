@@ -141,7 +141,7 @@ bool aligned16(const void* p) {
 
 unsigned stream_grid(size_t work_items) {
 	const size_t blocks = (work_items + 255) / 256;
-	return (unsigned) std::max<size_t>(1, std::min<size_t>(blocks, 256 * 16));
+	return (unsigned) std::max<size_t>(1, std::min<size_t>(blocks, (size_t) 1 << 22));
 }
 
 template<typename T, int KIND>
