@@ -239,12 +239,11 @@ def train_steps_run(args, dtype):
             for l in reversed(layers):
                 g = l.pass_back(g)
             for p in params:
-                if p.are_optimizable():
+                if p.are_optimizable():          # update + reset_grad of SGDOptimizer::_train as one kernel
                     if adam:
-                        p.adam_update(t)
+                        p.optimizer_step("adam", [1e-3, 1e-1, 1e-3, 1e-5], timestep=t)
                     else:
-                        p.sgd_update(1e-3)
-                    p.reset_grad()
+                        p.optimizer_step("vanilla_sgd", [1e-3])
 
         for t in range(args.warmup):
             step(t)

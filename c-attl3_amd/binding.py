@@ -37,7 +37,7 @@ EXPORTS = [
     "cattle_hip_layer_num_params", "cattle_hip_layer_param_shape", "cattle_hip_layer_set_param_values",
     "cattle_hip_layer_get_param_values", "cattle_hip_layer_get_param_grad", "cattle_hip_layer_reset_param_grad",
     "cattle_hip_maxpool_indices", "cattle_hip_loss_function", "cattle_hip_loss_d_function",
-    "cattle_hip_layer_param_optimizer_update", "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
+    "cattle_hip_layer_param_optimizer_update", "cattle_hip_layer_param_optimizer_step", "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
     "cattle_hip_layer_param_reset_optimizer_state", "cattle_hip_convlstm_create", "cattle_hip_convlstm_propagate",
     "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
     "cattle_hip_convlstm_get_kernel_grad",
@@ -198,9 +198,15 @@ class Parameters(object):
     def optimizer_update(self, optimizer, hyper, epoch=0, timestep=0):
         """<Name>Optimizer::_update_params on the device; optimizer is a key of OPTIMIZERS, hyper the reference
         optimizer's constructor arguments in their order (see include/cattle_hip.h)."""
-        h = (ctypes.c_double * 4)(*(list(hyper) + [0.0] * (4 - len(hyper))))
+        h = _hyper_array(tuple(hyper))
         _check(lib().cattle_hip_layer_param_optimizer_update(self._layer._h, _sz(self._index), ctypes.c_int(OPTIMIZERS[optimizer]),
                                                              h, _sz(epoch), _sz(timestep)))
+
+    def optimizer_step(self, optimizer, hyper, epoch=0, timestep=0):
+        """optimizer_update followed by reset_grad (optimizer/SGDOptimizer.hpp:64, :68-70) as one kernel."""
+        h = _hyper_array(tuple(hyper))
+        _check(lib().cattle_hip_layer_param_optimizer_step(self._layer._h, _sz(self._index), ctypes.c_int(OPTIMIZERS[optimizer]),
+                                                           h, _sz(epoch), _sz(timestep)))
 
     def sgd_update(self, learning_rate=1e-3):
         """VanillaSGDOptimizer::_update_params on the device (optimizer/VanillaSGDOptimizer.hpp:38-43)."""
@@ -218,6 +224,15 @@ class Parameters(object):
 
 
 LOSS = {"squared": 0, "softmax_cross_entropy": 1}
+_HYPER_ARRAYS = {}
+
+
+def _hyper_array(hyper):
+    """The four-entry hyper-parameter array of an optimizer call (read-only on the C side, so one per value set)."""
+    h = _HYPER_ARRAYS.get(hyper)
+    if h is None:
+        h = _HYPER_ARRAYS[hyper] = (ctypes.c_double * 4)(*(list(hyper) + [0.0] * (4 - len(hyper))))
+    return h
 OPTIMIZERS = {"vanilla_sgd": 0, "momentum_sgd": 1, "nesterov_momentum_sgd": 2, "adagrad": 3, "rmsprop": 4, "adadelta": 5,
               "adam": 6, "adamax": 7, "nadam": 8, "amsgrad": 9}
 

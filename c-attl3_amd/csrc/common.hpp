@@ -148,8 +148,9 @@ enum { OPT_VANILLA_SGD = 0, OPT_MOMENTUM_SGD = 1, OPT_NESTEROV = 2, OPT_ADAGRAD 
 	OPT_ADAM = 6, OPT_ADAMAX = 7, OPT_NADAM = 8, OPT_AMSGRAD = 9 };
 template<typename T> struct OptCoef { T c[8]; };
 int optimizer_state_count(int rule);
+/* reset_grad: zero the gradient in the same kernel, after it has been used */
 template<typename T> void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n,
-		const T* grad, T* s0, T* s1, T* s2, T* values);
+		T* grad, T* s0, T* s1, T* s2, T* values, bool reset_grad);
 
 } /* namespace cattle_hip */
 

@@ -785,6 +785,29 @@ Param& optimizable_param(cattle_hip_layer_t layer, size_t index) {
 	return p;
 }
 
+/* One optimizer update of a parameter, optionally followed (in the same kernel) by the reset of its gradient. */
+void run_optimizer(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer, const double hyper[4], size_t epoch,
+		size_t timestep, bool reset_grad) {
+	Param& p = optimizable_param(layer, index);
+	CATTLE_HIP_REQUIRE(hyper != nullptr, "null hyper-parameter array");
+	const int states = optimizer_state_count((int) optimizer);
+	for (int i = p.moments_ready; i < states; ++i) {
+		fill_zero(p.moments[i].ensure(p.bytes()), p.bytes());
+		p.moments_ready = i + 1;
+	}
+	const size_t n = p.rows * p.cols;
+	if (p.esize == sizeof(float))
+		optimizer_update<float>((int) optimizer, hyper, epoch, timestep, n, static_cast<float*>(p.grad.p),
+				static_cast<float*>(p.moments[0].p), static_cast<float*>(p.moments[1].p), static_cast<float*>(p.moments[2].p),
+				static_cast<float*>(p.values.p), reset_grad);
+	else
+		optimizer_update<double>((int) optimizer, hyper, epoch, timestep, n, static_cast<double*>(p.grad.p),
+				static_cast<double*>(p.moments[0].p), static_cast<double*>(p.moments[1].p),
+				static_cast<double*>(p.moments[2].p), static_cast<double*>(p.values.p), reset_grad);
+	++p.version;
+}
+
+
 
 template<typename T>
 void convlstm_propagate(ConvLstm<T>* l, const void* input, int in_space, size_t batch, size_t in_len, size_t out_len,
@@ -1404,25 +1427,12 @@ int cattle_hip_loss_d_function(cattle_hip_dtype dtype, cattle_hip_loss kind, con
 
 int cattle_hip_layer_param_optimizer_update(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
 		const double hyper[4], size_t epoch, size_t timestep) {
-	return guarded([&] {
-		Param& p = optimizable_param(layer, index);
-		CATTLE_HIP_REQUIRE(hyper != nullptr, "null hyper-parameter array");
-		const int states = optimizer_state_count((int) optimizer);
-		for (int i = p.moments_ready; i < states; ++i) {
-			fill_zero(p.moments[i].ensure(p.bytes()), p.bytes());
-			p.moments_ready = i + 1;
-		}
-		const size_t n = p.rows * p.cols;
-		if (p.esize == sizeof(float))
-			optimizer_update<float>((int) optimizer, hyper, epoch, timestep, n, static_cast<const float*>(p.grad.p),
-					static_cast<float*>(p.moments[0].p), static_cast<float*>(p.moments[1].p), static_cast<float*>(p.moments[2].p),
-					static_cast<float*>(p.values.p));
-		else
-			optimizer_update<double>((int) optimizer, hyper, epoch, timestep, n, static_cast<const double*>(p.grad.p),
-					static_cast<double*>(p.moments[0].p), static_cast<double*>(p.moments[1].p),
-					static_cast<double*>(p.moments[2].p), static_cast<double*>(p.values.p));
-		++p.version;
-	});
+	return guarded([&] { run_optimizer(layer, index, optimizer, hyper, epoch, timestep, false); });
+}
+
+int cattle_hip_layer_param_optimizer_step(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
+		const double hyper[4], size_t epoch, size_t timestep) {
+	return guarded([&] { run_optimizer(layer, index, optimizer, hyper, epoch, timestep, true); });
 }
 
 int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate) {

@@ -139,8 +139,8 @@ void softmax_ce_kernel(int N, int T_steps, int V, T eps, T scale, const T* __res
  *   OPT_AMSGRAD       optimizer/AMSGradOptimizer.hpp:48-66           k: d1, d2, lr, -, eps */
 template<typename T, int RULE>
 __global__ __launch_bounds__(256)
-void optimizer_update_kernel(size_t total, OptCoef<T> k, const T* __restrict__ grad, T* __restrict__ s0, T* __restrict__ s1,
-		T* __restrict__ s2, T* __restrict__ values) {
+void optimizer_update_kernel(size_t total, OptCoef<T> k, T* __restrict__ grad, T* __restrict__ s0, T* __restrict__ s1,
+		T* __restrict__ s2, T* __restrict__ values, bool reset_grad) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
 	const T one = (T) 1;
 	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
@@ -190,6 +190,8 @@ void optimizer_update_kernel(size_t total, OptCoef<T> k, const T* __restrict__ g
 				}
 			}
 		}
+		if (reset_grad)                 /* Parameters::reset_grad after the update (optimizer/SGDOptimizer.hpp:68-70) */
+			grad[i] = (T) 0;
 	}
 }
 
@@ -253,8 +255,8 @@ int optimizer_state_count(int rule) {
 }
 
 template<typename T>
-void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n, const T* grad, T* s0, T* s1,
-		T* s2, T* values) {
+void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n, T* grad, T* s0, T* s1,
+		T* s2, T* values, bool reset_grad) {
 	if (n == 0)
 		return;
 	OptCoef<T> k;
@@ -303,16 +305,16 @@ void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t time
 	}
 	const unsigned grid = flat_grid(n);
 	switch (rule) {
-	case OPT_VANILLA_SGD: optimizer_update_kernel<T, OPT_VANILLA_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_MOMENTUM_SGD: optimizer_update_kernel<T, OPT_MOMENTUM_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_NESTEROV: optimizer_update_kernel<T, OPT_NESTEROV><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_ADAGRAD: optimizer_update_kernel<T, OPT_ADAGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_RMSPROP: optimizer_update_kernel<T, OPT_RMSPROP><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_ADADELTA: optimizer_update_kernel<T, OPT_ADADELTA><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_ADAM: optimizer_update_kernel<T, OPT_ADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_ADAMAX: optimizer_update_kernel<T, OPT_ADAMAX><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	case OPT_NADAM: optimizer_update_kernel<T, OPT_NADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
-	default: optimizer_update_kernel<T, OPT_AMSGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values); break;
+	case OPT_VANILLA_SGD: optimizer_update_kernel<T, OPT_VANILLA_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_MOMENTUM_SGD: optimizer_update_kernel<T, OPT_MOMENTUM_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_NESTEROV: optimizer_update_kernel<T, OPT_NESTEROV><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_ADAGRAD: optimizer_update_kernel<T, OPT_ADAGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_RMSPROP: optimizer_update_kernel<T, OPT_RMSPROP><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_ADADELTA: optimizer_update_kernel<T, OPT_ADADELTA><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_ADAM: optimizer_update_kernel<T, OPT_ADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_ADAMAX: optimizer_update_kernel<T, OPT_ADAMAX><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	case OPT_NADAM: optimizer_update_kernel<T, OPT_NADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	default: optimizer_update_kernel<T, OPT_AMSGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
 	}
 	check_launch();
 }
@@ -320,7 +322,7 @@ void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t time
 #define CATTLE_HIP_INSTANTIATE_TRAIN(T) \
 template void loss_function<T>(int, int, int, int, T, const T*, const T*, T*); \
 template void loss_d_function<T>(int, int, int, int, T, T, const T*, const T*, T*); \
-template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, const T*, T*, T*, T*, T*);
+template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, T*, T*, T*, T*, T*, bool);
 
 CATTLE_HIP_INSTANTIATE_TRAIN(float)
 CATTLE_HIP_INSTANTIATE_TRAIN(double)

@@ -269,6 +269,16 @@ public:
 					(double) epsilon, timestep));
 		});
 	}
+	/**
+	 * The update of every optimizable parameter followed by its reset_grad, as SGDOptimizer::_train applies them to
+	 * a batch (optimizer/SGDOptimizer.hpp:64, :68-70); the gradient is zeroed by the update kernel itself. Gradients
+	 * of non-optimizable parameters are never accumulated (parameters/StandardParameters.hpp:116-117) and stay zero.
+	 */
+	inline void optimizer_step(cattle_hip_optimizer optimizer, const double (&hyper)[4], std::size_t epoch, std::size_t timestep) {
+		for_each_optimizable([&](std::size_t i) {
+			check(cattle_hip_layer_param_optimizer_step(handle, i, optimizer, hyper, epoch, timestep));
+		});
+	}
 	/** AdamOptimizer::_fit. */
 	inline void reset_optimizer_state() {
 		const std::size_t n = num_params();
@@ -501,20 +511,18 @@ public:
 	inline Scalar train_batch_sgd(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,
 			const DeviceLoss<Scalar>& loss, Scalar learning_rate) {
 		const Scalar total = forward_backward(input, obj, loss);
-		for (std::size_t i = 0; i < layers.size(); ++i) {
-			layers[i].sgd_update(learning_rate);
-			layers[i].reset_grads();
-		}
+		const double hyper[4] = { (double) learning_rate, 0, 0, 0 };
+		for (std::size_t i = 0; i < layers.size(); ++i)
+			layers[i].optimizer_step(CATTLE_HIP_OPT_VANILLA_SGD, hyper, 0, 0);
 		return total;
 	}
 	inline Scalar train_batch_adam(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,
 			const DeviceLoss<Scalar>& loss, std::size_t timestep, Scalar learning_rate = 1e-3, Scalar l1_decay = 1e-1,
 			Scalar l2_decay = 1e-3, Scalar epsilon = 1e-5) {
 		const Scalar total = forward_backward(input, obj, loss);
-		for (std::size_t i = 0; i < layers.size(); ++i) {
-			layers[i].adam_update(timestep, learning_rate, l1_decay, l2_decay, epsilon);
-			layers[i].reset_grads();
-		}
+		const double hyper[4] = { (double) learning_rate, (double) l1_decay, (double) l2_decay, (double) epsilon };
+		for (std::size_t i = 0; i < layers.size(); ++i)
+			layers[i].optimizer_step(CATTLE_HIP_OPT_ADAM, hyper, 0, timestep);
 		return total;
 	}
 private:

@@ -238,6 +238,11 @@ typedef enum cattle_hip_optimizer {
 } cattle_hip_optimizer;
 int cattle_hip_layer_param_optimizer_update(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
 		const double hyper[4], size_t epoch, size_t timestep);
+/* The same update followed by Parameters::reset_grad of that parameter, the order in which SGDOptimizer::_train
+ * applies them to every batch (optimizer/SGDOptimizer.hpp:64, :68-70), as one kernel: the gradient is zeroed by
+ * the thread that has just used it. */
+int cattle_hip_layer_param_optimizer_step(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
+		const double hyper[4], size_t epoch, size_t timestep);
 
 /* VanillaSGDOptimizer::_update_params for one Parameters object (optimizer/VanillaSGDOptimizer.hpp:38-43):
  * values -= grad * learning_rate, in place on the device. Non-optimizable parameters are rejected. */

@@ -273,6 +273,25 @@ def test_every_optimizer_over_steps(rule, hyper, dtype):
     assert hp.rel_err(prm.get_values(), ref) < tol
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rule,hyper", [ALL_OPTIMIZERS[0], ALL_OPTIMIZERS[2], ALL_OPTIMIZERS[6], ALL_OPTIMIZERS[9]])
+def test_optimizer_step_is_update_then_reset(rule, hyper, dtype):
+    """optimizer_step (update and reset_grad in one kernel) leaves the same values, bit for bit, as optimizer_update
+    followed by reset_grad over three batches, and a zero gradient after each."""
+    a, ga, _, _ = _dense_with_grads(dtype, 1222)
+    c, gc, _, _ = _dense_with_grads(dtype, 1222)       # same seed: the same stream of inputs
+    pa, pc = a.get_params()[0], c.get_params()[0]
+    for t in range(3):
+        _accumulate(a, ga, dtype)
+        _accumulate(c, gc, dtype)
+        assert np.any(pa.get_grad()) and np.array_equal(pa.get_grad(), pc.get_grad())
+        pa.optimizer_update(rule, hyper, epoch=1, timestep=t)
+        pa.reset_grad()
+        pc.optimizer_step(rule, hyper, epoch=1, timestep=t)
+        assert np.array_equal(pa.get_values(), pc.get_values()), (rule, t)
+        assert not np.any(pc.get_grad())
+
+
 def test_optimizer_argument_checks():
     layer, g, w, b = _dense_with_grads(np.float32, 1221)
     prm = layer.get_params()[0]
