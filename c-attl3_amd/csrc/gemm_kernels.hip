@@ -908,12 +908,13 @@ GatherVariant<T> gather_variant() {
 
 template<typename T> struct GatherVariants;
 template<> struct GatherVariants<float> {
-	static constexpr int COUNT = 5, LARGE = 3;
+	static constexpr int COUNT = 6, LARGE = 4;
 	static const GatherVariant<float>* get() {
 		static const GatherVariant<float> v[COUNT] = {
 			gather_variant<float, 4, 2, 64, 64>(),      /* 256 x 128 */
 			gather_variant<float, 4, 2, 64, 32>(),      /* 256 x 64: eight waves of 64 x 32 beat four of 64 x 64 by 5 % */
 			gather_variant<float, 4, 1, 64, 32>(),      /* 256 x 32 */
+			gather_variant<float, 8, 1, 64, 64>(),      /* 512 x 64 for very tall problems: eight waves of 64 x 64, 1 % over 256 x 64 */
 			/* small problems (a few thousand rows): short tiles so that every CU gets a block, and long
 			 * reduction chunks because with one block per CU only the loads in flight hide memory latency */
 			gather_variant<float, 2, 2, 32, 32, 64>(),  /* 64 x 64 */

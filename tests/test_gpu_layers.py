@@ -105,6 +105,13 @@ def test_conv_strided_dilated_larger():
     _check_conv((17, 19, 6, 40, 3, 2, 2, 1, 2, 3, 1, 0), 12, np.float32, seed=8)
 
 
+@pytest.mark.parametrize("N", [33, 36])              # scalar and 16-byte loads
+def test_conv_tall_ragged_problem(N):
+    """More than half a million output rows and 40 filters: the 512-row forward tiles that only problems this tall
+    use, with partial tiles in M and F."""
+    _check_conv((127, 127, 3, 40, 3, 3, 1, 1, 1, 1, 0, 0), N, np.float32, seed=9)
+
+
 @pytest.mark.parametrize("dtype,N", [(np.float32, 256), (np.float64, 128)])
 def test_conv_config4_full_size(dtype, N):
     """BASELINE config 4 at its real shape (56x56x64 -> 128 filters, 3x3 s1 p1; batch 256 in fp32): the tile
