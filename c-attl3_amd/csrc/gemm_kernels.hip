@@ -155,20 +155,24 @@ struct GatherLaunch {
 	int main_count, main_blocks;
 	int split_count, ksplit, chunks_per_part;
 	int sample_blocks;      /* > 0: tile rows are blocks of 32 samples x BM / 32 positions, see tile_row_m */
+	int pos_b;              /* blocked order: positions of a tile along b (the other BM / 32 / pos_b lie along a) */
 };
 
 /* Row `row` of M tile `tile` as an index m = n + N * (a + OA * b) of the GEMM. Plain order: the tile is BM
  * consecutive m (BM consecutive samples of one output position when N >= BM). Blocked order (sample_blocks =
- * N / 32 > 0, needs N % 32 == 0 and OA % (BM / 32) == 0): the tile is 32 samples of BM / 32 positions that
- * follow one another along a, so that the receptor fields of its rows overlap and a tile touches about half
- * as many distinct input bytes; tiles of one column b are numbered sample block fastest. Rows stay groups
- * of 32 consecutive samples, so vector accesses along n are unaffected. */
+ * N / 32 > 0, needs N % 32 == 0): the tile is 32 samples of a pa x pos_b rectangle of output positions
+ * (pa = BM / 32 / pos_b along a, OA % pa == 0, OB % pos_b == 0), so that the receptor fields of its rows
+ * overlap and a tile touches about half as many distinct input bytes; tiles of one strip of pos_b columns are
+ * numbered sample block fastest, and tile_rows counts the tiles of a strip. Rows stay groups of 32 consecutive
+ * samples, so vector accesses along n are unaffected. */
 __device__ __forceinline__ int tile_row_m(const GatherLaunch& L, const GatherGeom& g, int tile, int BM, int row) {
 	if (L.sample_blocks == 0)
 		return tile * BM + row;
-	const int col = tile / L.tile_rows, r = tile - col * L.tile_rows;
+	const int strip = tile / L.tile_rows, r = tile - strip * L.tile_rows;
 	const int ab = r / L.sample_blocks, nb = r - ab * L.sample_blocks;
-	return nb * 32 + (row & 31) + g.N * (ab * (BM / 32) + (row >> 5) + g.OA * col);
+	const int pa = BM / 32 / L.pos_b, p = row >> 5;
+	const int pb_i = p / pa, pa_i = p - pb_i * pa;
+	return nb * 32 + (row & 31) + g.N * (ab * pa + pa_i + g.OA * (strip * L.pos_b + pb_i));
 }
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS>
@@ -984,10 +988,23 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	/* tiles per output column, if a column (N * OA rows of M) is a whole number of tiles and there are
 	 * several columns; 0 switches the 2-D walk off */
 	const long column = (long) g.N * g.OA;
-	const int tile_rows = (column % v.bm == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE")) ? (int) (column / v.bm) : 0;
-	/* rows of a tile as 32 samples x several positions along a (see tile_row_m) where the shape allows it */
-	const int sample_blocks = (tile_rows > 0 && g.N % 32 == 0 && v.bm % 32 == 0 && g.OA % (v.bm / 32) == 0 &&
-			!std::getenv("CATTLE_HIP_NO_ROW_BLOCKS")) ? g.N / 32 : 0;
+	int tile_rows = (column % v.bm == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE")) ? (int) (column / v.bm) : 0;
+	/* rows of a tile as 32 samples x a rectangle of positions (see tile_row_m) where the shape allows it: as many
+	 * positions along a as divide OA, the rest along b; the 2-D walk then runs over strips of pos_b columns */
+	int sample_blocks = 0, pos_b = 1;
+	if (g.N % 32 == 0 && v.bm % 32 == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE") &&
+			!std::getenv("CATTLE_HIP_NO_ROW_BLOCKS")) {
+		const int positions = v.bm / 32;
+		for (int pb = 1; pb <= positions; pb *= 2) {
+			const int pa = positions / pb;
+			if (positions % pb == 0 && g.OA % pa == 0 && g.OB % pb == 0 && g.OB / pb > 1) {
+				sample_blocks = g.N / 32;
+				pos_b = pb;
+				tile_rows = sample_blocks * (g.OA / pa);
+				break;
+			}
+		}
+	}
 	/* blocks the chip holds at once (registers, LDS, waves), as the runtime computes it for this kernel */
 	const int per_cu = std::max(1, v.blocks_per_cu(dyn, vec, divs));
 	const int slots = NUM_CUS * per_cu;
@@ -995,7 +1012,7 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 
 	/* main_count whole tiles, the other mtiles - main_count with their reduction cut into about `ksplit` parts */
 	auto launch = [&](int main_count, int ksplit) {
-		GatherLaunch L = { mtiles, tile_rows, main_count, round_up(main_count, 8), mtiles - main_count, 1, nchunks, sample_blocks };
+		GatherLaunch L = { mtiles, tile_rows, main_count, round_up(main_count, 8), mtiles - main_count, 1, nchunks, sample_blocks, pos_b };
 		T* partials = nullptr;
 		if (L.split_count > 0) {
 			L.chunks_per_part = (nchunks + ksplit - 1) / ksplit;
