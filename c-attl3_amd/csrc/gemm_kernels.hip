@@ -458,8 +458,8 @@ struct WgradSplit {
  * grid = tiles * splits blocks (1-D). Bias rows are dealt out over the k tiles (row f belongs to the
  * block with f % ktiles == k-tile index) so that every block does the same amount of extra work.
  * ---------------------------------------------------------------------------------------------- */
-template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC>
-__global__ __launch_bounds__(64 * WAVES_K * WAVES_F)
+template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, int MIN_WAVES>
+__global__ __launch_bounds__(64 * WAVES_K * WAVES_F, MIN_WAVES)      /* MIN_WAVES: wavefronts per SIMD the registers must allow */
 void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
 		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan) {
 	typedef Mfma<T> MF;
@@ -479,7 +479,6 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 
 	__shared__ __attribute__((aligned(16))) T Xs[BK][LDM];
 	__shared__ __attribute__((aligned(16))) T Gs[BF][LDM];
-	__shared__ int4 ktab[BK];      /* per k row: ya term, yb term, channel offset, valid */
 
 	const int tid = threadIdx.x;
 	/* blocks of one slice (its k and f tiles) get consecutive positions on one XCD: they read the same
@@ -509,14 +508,20 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		chunk_count = max(0, min(begin + plan.chunks_per_split, total_chunks) - begin);
 	}
 
-	for (int i = tid; i < BK; i += THREADS) {
-		const int k = k0 + i;
-		const int r = k % g.R, t = k / g.R;
-		const int s = t % g.S, ch = t / g.S;
-		ktab[i] = make_int4(r * g.RA, s * g.RB, g.N * g.LH * g.LW * ch, k < g.K ? 1 : 0);
-	}
-
 	const int col = tid % COLS, row0 = tid / COLS;
+	/* The k rows a thread loads are the same in every chunk, so what the gather needs of them stays in registers
+	 * instead of a table in LDS (whose reads sat in front of every global load): the receptor position packed
+	 * as r | s << 16 (-1 for a row outside K or outside the tile) and the channel. */
+	int krs[XSLOTS], kch[XSLOTS];
+	#pragma unroll
+	for (int s = 0; s < XSLOTS; ++s) {
+		const int row = row0 + s * RP, k = k0 + row;
+		const int r = k % g.R, t = k / g.R;
+		const int sb = t % g.S;
+		kch[s] = t / g.S;
+		krs[s] = (k < g.K && (BK % RP == 0 || row < BK)) ? (r | sb << 16) : -1;
+	}
+	const int slab = g.N * g.LH * g.LW;
 	/* (n, a, b) of this thread's vector for the next chunk to load */
 	int n, a, b, a0, b0, pleft = npix;
 	if (pixel_mode) {
@@ -540,15 +545,9 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		const int ya0 = a * g.SA + g.PA, yb0 = b * g.SB + g.PB;
 		#pragma unroll
 		for (int s = 0; s < XSLOTS; ++s) {
-			const int row = row0 + s * RP;
-			bool ok = false;
-			int off = 0;
-			if (BK % RP == 0 || row < BK) {
-				const int4 ke = ktab[row];
-				const int ya = ya0 + ke.x, yb = yb0 + ke.y;
-				ok = mvalid && ke.w && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
-				off = n + g.N * (ya + g.LH * yb) + ke.z;
-			}
+			const int ya = ya0 + (krs[s] & 0xffff) * g.RA, yb = yb0 + (krs[s] >> 16) * g.RB;
+			const bool ok = mvalid && krs[s] >= 0 && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
+			const int off = n + g.N * (ya + g.LH * yb) + kch[s] * slab;
 			if (ok) {
 				vec_load<T, VEC>(xreg[s], src + off);
 			} else {
@@ -623,7 +622,6 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	for (int it = 0; it < BIAS_IT; ++it)
 		bacc[it] = (T) 0;
 
-	__syncthreads();                  /* ktab visible */
 	if (chunk_count > 0)
 		load_tiles();
 	for (int c = 0; c < chunk_count; ++c) {
@@ -1077,6 +1075,7 @@ void check_sizes(const ConvShape& s, int N) {
 	const double padded = (double) N * (s.H + 2.0 * s.pv + s.RH * (s.dv + 1.0)) * (s.W + 2.0 * s.ph + s.RW * (s.dh + 1.0)) *
 			std::max(s.C, s.F);
 	CATTLE_HIP_REQUIRE(padded <= lim, "padded tensor exceeds 2^31-1 elements");
+	CATTLE_HIP_REQUIRE(s.RH < 32768 && s.RW < 32768, "receptor field too large");      /* packed as 16-bit fields in wgrad_kernel */
 }
 
 /* Weight-gradient tile shapes (K rows x F columns of the gradient per block) and the split of M. */
@@ -1089,38 +1088,38 @@ struct WgradVariant {
 	int (*blocks_per_cu)();         /* what the runtime says fits on a CU (registers and LDS) */
 };
 
-template<typename T, int WK, int WF, int TK, int TF>
+template<typename T, int WK, int WF, int TK, int TF, int MINW = 1>
 void launch_wgrad_variant(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom& g, const WgradSplit& plan,
 		bool vec) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	dim3 block(64 * WK * WF), grid((unsigned) round_up(plan.tiles * plan.splits, 8));
 	if (vec)
-		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, VEC><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
+		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, VEC, MINW><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
 	else
-		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
+		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, 1, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
-template<typename T, int WK, int WF, int TK, int TF>
+template<typename T, int WK, int WF, int TK, int TF, int MINW = 1>
 int wgrad_variant_occupancy() {
 	static int cached = 0;
 	if (cached == 0) {
 		int n = 0;
-		CATTLE_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, GemmCfg<T>::VEC>,
+		CATTLE_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, GemmCfg<T>::VEC, MINW>,
 				64 * WK * WF, 0));
 		cached = std::max(1, n);
 	}
 	return cached;
 }
 
-template<typename T, int WK, int WF, int TK, int TF>
+template<typename T, int WK, int WF, int TK, int TF, int MINW = 1>
 WgradVariant<T> wgrad_variant() {
 	WgradVariant<T> v;
 	v.bk = WK * TK;
 	v.bf = WF * TF;
 	v.waves = WK * WF;
-	v.launch = &launch_wgrad_variant<T, WK, WF, TK, TF>;
-	v.blocks_per_cu = &wgrad_variant_occupancy<T, WK, WF, TK, TF>;
+	v.launch = &launch_wgrad_variant<T, WK, WF, TK, TF, MINW>;
+	v.blocks_per_cu = &wgrad_variant_occupancy<T, WK, WF, TK, TF, MINW>;
 	return v;
 }
 
@@ -1129,7 +1128,7 @@ template<> struct WgradVariants<float> {
 	static constexpr int COUNT = 4;
 	static const WgradVariant<float>* get() {
 		static const WgradVariant<float> v[COUNT] = {
-			wgrad_variant<float, 2, 4, 96, 32>(),       /* 192 x 128 */
+			wgrad_variant<float, 2, 4, 96, 32, 4>(),    /* 192 x 128, registers held to four waves per SIMD = two blocks per CU */
 			wgrad_variant<float, 2, 2, 64, 64>(),       /* 128 x 128 */
 			wgrad_variant<float, 1, 4, 32, 32>(),       /*  32 x 128 */
 			wgrad_variant<float, 1, 4, 64, 32>(),       /*  64 x 128 */
