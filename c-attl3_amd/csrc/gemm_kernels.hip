@@ -510,18 +510,20 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 
 	const int col = tid % COLS, row0 = tid / COLS;
 	/* The k rows a thread loads are the same in every chunk, so what the gather needs of them stays in registers
-	 * instead of a table in LDS (whose reads sat in front of every global load): the receptor position packed
-	 * as r | s << 16 (-1 for a row outside K or outside the tile) and the channel. */
-	int krs[XSLOTS], kch[XSLOTS];
+	 * instead of a table in LDS (whose reads sat in front of every global load): the displacements of the
+	 * receptor position along both axes, packed as dya | dyb << 16 (both are below 32768, checked on the host;
+	 * -1 for a row outside K or outside the tile), and the element offset that the row adds to the offset of
+	 * the chunk's output position. */
+	int krs[XSLOTS], koff[XSLOTS];
 	#pragma unroll
 	for (int s = 0; s < XSLOTS; ++s) {
 		const int row = row0 + s * RP, k = k0 + row;
 		const int r = k % g.R, t = k / g.R;
-		const int sb = t % g.S;
-		kch[s] = t / g.S;
-		krs[s] = (k < g.K && (BK % RP == 0 || row < BK)) ? (r | sb << 16) : -1;
+		const int sb = t % g.S, ch = t / g.S;
+		const int dya = r * g.RA, dyb = sb * g.RB;
+		krs[s] = (k < g.K && (BK % RP == 0 || row < BK)) ? (dya | dyb << 16) : -1;
+		koff[s] = g.N * (dya + g.LH * dyb) + g.N * g.LH * g.LW * ch;
 	}
-	const int slab = g.N * g.LH * g.LW;
 	/* (n, a, b) of this thread's vector for the next chunk to load */
 	int n, a, b, a0, b0, pleft = npix;
 	if (pixel_mode) {
@@ -543,11 +545,12 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		const int m = n + g.N * (a + g.OA * b);
 		const bool mvalid = b < g.OB;
 		const int ya0 = a * g.SA + g.PA, yb0 = b * g.SB + g.PB;
+		const int base = n + g.N * (ya0 + g.LH * yb0);       /* may lie in the padding; only used when in range */
 		#pragma unroll
 		for (int s = 0; s < XSLOTS; ++s) {
-			const int ya = ya0 + (krs[s] & 0xffff) * g.RA, yb = yb0 + (krs[s] >> 16) * g.RB;
+			const int ya = ya0 + (krs[s] & 0xffff), yb = yb0 + (krs[s] >> 16);
 			const bool ok = mvalid && krs[s] >= 0 && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
-			const int off = n + g.N * (ya + g.LH * yb) + kch[s] * slab;
+			const int off = base + koff[s];
 			if (ok) {
 				vec_load<T, VEC>(xreg[s], src + off);
 			} else {
@@ -1075,7 +1078,8 @@ void check_sizes(const ConvShape& s, int N) {
 	const double padded = (double) N * (s.H + 2.0 * s.pv + s.RH * (s.dv + 1.0)) * (s.W + 2.0 * s.ph + s.RW * (s.dh + 1.0)) *
 			std::max(s.C, s.F);
 	CATTLE_HIP_REQUIRE(padded <= lim, "padded tensor exceeds 2^31-1 elements");
-	CATTLE_HIP_REQUIRE(s.RH < 32768 && s.RW < 32768, "receptor field too large");      /* packed as 16-bit fields in wgrad_kernel */
+	/* wgrad_kernel packs the displacements of a receptor position as two 16-bit fields */
+	CATTLE_HIP_REQUIRE((double) s.RH * (s.dv + 1) < 32768.0 && (double) s.RW * (s.dh + 1) < 32768.0, "dilated receptor field too large");
 }
 
 /* Weight-gradient tile shapes (K rows x F columns of the gradient per block) and the split of M. */
