@@ -363,6 +363,10 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		for (int st = 0; st < KC / KS; ++st) {
 			const int cur = st & 1, nxt = cur ^ 1;
 			if (st + 1 < KC / KS) {
+				/* lgkmcnt(0): this step's operands, read one step ago, have landed. Waiting here, before the
+				 * next step's reads go out, keeps the compiler from placing the same wait after them, where
+				 * it would hold this step's MFMAs back until the reads just issued have returned as well. */
+				__builtin_amdgcn_s_waitcnt(0xC07F);
 				vec_load<T, MB>(xa[nxt], &As[buf][(st + 1) * KS + lk][wm * WT_M + MB * lc]);
 				vec_load<T, FB>(wb[nxt], &Bs[buf][(st + 1) * KS + lk][wf * WT_F + FB * lc]);
 			}
