@@ -34,9 +34,9 @@ SHAPE = dict(H=56, W=56, C=64, F=128, RH=3, RW=3)
 MEASURED_TRAFFIC = {
     ("f32", 256): {
         # kernel read + written, then the reduce launches' read + written
-        "gather_gemm_kernel (forward)": 326.7e6 + 469.8e6 + 67.2e6 + 8.4e6,
-        "wgrad_kernel (+ reduce, bias column sums)": 954.3e6 + 50.3e6 + 50.5e6 + 0.3e6,
-        "gather_gemm_kernel (input gradient)": 574.0e6 + 264.2e6 + 63.0e6 + 4.2e6,
+        "gather_gemm_kernel (forward)": 325.8e6 + 469.8e6 + 67.2e6 + 8.4e6,
+        "wgrad_kernel (+ reduce, bias column sums)": 775.5e6 + 52.4e6 + 50.5e6 + 0.3e6,
+        "gather_gemm_kernel (input gradient)": 573.7e6 + 264.2e6 + 63.0e6 + 4.2e6,
     },
 }
 
