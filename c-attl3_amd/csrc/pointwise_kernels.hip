@@ -838,8 +838,10 @@ __device__ __forceinline__ T act_b_rt(int kind, T x, T y, T g, T p) {
 	}
 }
 
-__device__ __forceinline__ size_t seq_offset(size_t e, int N, int T_len, int t) {
-	const size_t n = e % (size_t) N, rest = e / (size_t) N;
+/* Offset of element (n, rest) of time step t in a sequence tensor (N, T_len, ...): element e = n + N * rest of a
+ * step's slab. A slab of P elements is a whole number of samples, so gate g of element e is (n, rest + g * P / N):
+ * one 32-bit division per element serves all of its accesses (the host checks that 4 P fits 32 bits). */
+__device__ __forceinline__ size_t seq_offset(unsigned n, unsigned rest, int N, int T_len, int t) {
 	return n + (size_t) N * ((size_t) t + (size_t) T_len * rest);
 }
 
@@ -850,14 +852,16 @@ void lstm_gates_forward_kernel(LstmActs<T> a, int N, size_t P, const T* __restri
 		T* __restrict__ state, T* __restrict__ act_state, T* __restrict__ hidden, T* __restrict__ hprev_all, int h_T, int h_t,
 		T* __restrict__ out, int out_T, int out_t) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	const unsigned slab_rows = (unsigned) (P / (size_t) N);
 	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < P; e += stride) {
+		const unsigned rest = (unsigned) e / (unsigned) N, n = (unsigned) e - rest * (unsigned) N;
 		T y[4];
 		#pragma unroll
 		for (int g = 0; g < 4; ++g) {
 			/* weighted input + weighted previous output (:312, :327, :342, :373) */
 			T v = (T) 0;
 			if (zx)
-				v = zx[seq_offset(e + g * P, N, zx_T, zx_t)];
+				v = zx[seq_offset(n, rest + g * slab_rows, N, zx_T, zx_t)];
 			if (zh)
 				v = zx ? v + zh[g * P + e] : zh[g * P + e];
 			z[g * P + e] = v;
@@ -874,9 +878,9 @@ void lstm_gates_forward_kernel(LstmActs<T> a, int N, size_t P, const T* __restri
 		const T h = y[3] * as;                                      /* read filter * activated state (:383) */
 		hidden[e] = h;
 		if (hprev_all)
-			hprev_all[seq_offset(e, N, h_T, h_t)] = h;
+			hprev_all[seq_offset(n, rest, N, h_T, h_t)] = h;
 		if (out)
-			out[seq_offset(e, N, out_T, out_t)] = h;
+			out[seq_offset(n, rest, N, out_T, out_t)] = h;
 	}
 }
 
@@ -887,10 +891,12 @@ void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restr
 		const T* __restrict__ state, const T* __restrict__ act_state, T* __restrict__ state_grad, T* __restrict__ dz,
 		T* __restrict__ dzx_all, int x_T, int x_t, T* __restrict__ dzh_all, int h_T, int h_t) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	const unsigned slab_rows = (unsigned) (P / (size_t) N);
 	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < P; e += stride) {
+		const unsigned rest = (unsigned) e / (unsigned) N, n = (unsigned) e - rest * (unsigned) N;
 		T hg = dh ? dh[e] : (T) 0;
 		if (out_grad)
-			hg += out_grad[seq_offset(e, N, og_T, og_t)];           /* :431-438 */
+			hg += out_grad[seq_offset(n, rest, N, og_T, og_t)];     /* :431-438 */
 		const T f = gates[e], w = gates[P + e], c = gates[2 * P + e], r = gates[3 * P + e];
 		const T as = act_state[e];
 		const T sg = state_grad[e] + act_b_rt<T>(a.kind[3], state[e], as, r * hg, a.param[3]);      /* :440 */
@@ -904,9 +910,9 @@ void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restr
 		for (int g = 0; g < 4; ++g) {
 			dz[g * P + e] = d[g];
 			if (dzx_all)
-				dzx_all[seq_offset(e + g * P, N, x_T, x_t)] = d[g];
+				dzx_all[seq_offset(n, rest + g * slab_rows, N, x_T, x_t)] = d[g];
 			if (dzh_all)
-				dzh_all[seq_offset(e + g * P, N, h_T, h_t)] = d[g];
+				dzh_all[seq_offset(n, rest + g * slab_rows, N, h_T, h_t)] = d[g];
 		}
 	}
 }
@@ -1172,6 +1178,7 @@ void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int 
 		int out_T, int out_t) {
 	if (P == 0)
 		return;
+	CATTLE_HIP_REQUIRE(P % (size_t) N == 0 && P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
 	lstm_gates_forward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, zx, zx_T, zx_t, zh, prev_state, z, gates, state,
 			act_state, hidden, hprev_all, h_T, h_t, out, out_T, out_t);
 	check_launch();
@@ -1183,6 +1190,7 @@ void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, con
 		int x_t, T* dzh_all, int h_T, int h_t) {
 	if (P == 0)
 		return;
+	CATTLE_HIP_REQUIRE(P % (size_t) N == 0 && P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
 	lstm_gates_backward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, dh, out_grad, og_T, og_t, z, gates, prev_state,
 			state, act_state, state_grad, dz, dzx_all, x_T, x_t, dzh_all, h_T, h_t);
 	check_launch();
