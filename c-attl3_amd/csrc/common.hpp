@@ -38,6 +38,12 @@ enum { ERR_INVALID = 1, ERR_STATE = 2, ERR_DEVICE = 3, ERR_OOM = 4 };
 /* The stream every kernel and copy of the library is issued on. */
 hipStream_t stream();
 
+/* Copies between pageable host memory and the device on that stream; both return when the host buffer may be
+ * reused (host_to_device) or holds the data (device_to_host). Large copies are staged through pinned buffers by
+ * several host threads (CATTLE_HIP_COPY_THREADS, default 4; 0 leaves the staging to the runtime). */
+void host_to_device(void* dst_dev, const void* src_host, size_t bytes);
+void device_to_host(void* dst_host, const void* src_dev, size_t bytes);
+
 /* Geometry of a gathered GEMM  out[M x F] = A[M x K] * Wt[K x F]  whose A matrix is never
  * materialised: A(m,k) is read from a column-major (N, LH, LW, LC) tensor.
  *   m = n + N*(a + OA*b)           k = r + R*(s + S*ch)

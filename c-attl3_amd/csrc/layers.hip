@@ -71,19 +71,19 @@ struct DevBuf {
 void copy_in(void* dst_dev, const void* src, int space, size_t bytes) {
 	if (bytes == 0)
 		return;
-	CATTLE_HIP_CHECK(hipMemcpyAsync(dst_dev, src, bytes, space == CATTLE_HIP_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice,
-			stream()));
 	if (space == CATTLE_HIP_HOST)
-		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));    /* the pageable source may be freed on return */
+		host_to_device(dst_dev, src, bytes);
+	else
+		CATTLE_HIP_CHECK(hipMemcpyAsync(dst_dev, src, bytes, hipMemcpyDeviceToDevice, stream()));
 }
 
 void copy_out(void* dst, int space, const void* src_dev, size_t bytes) {
 	if (bytes == 0)
 		return;
-	CATTLE_HIP_CHECK(hipMemcpyAsync(dst, src_dev, bytes, space == CATTLE_HIP_HOST ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice,
-			stream()));
 	if (space == CATTLE_HIP_HOST)
-		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+		device_to_host(dst, src_dev, bytes);
+	else
+		CATTLE_HIP_CHECK(hipMemcpyAsync(dst, src_dev, bytes, hipMemcpyDeviceToDevice, stream()));
 }
 
 void fill_zero(void* dst_dev, size_t bytes) {
