@@ -43,3 +43,37 @@ def test_upload_leaves_the_source_reusable_and_orders_with_kernels():
     y = ch.DeviceTensor(shape, dtype)
     relu.forward_into(d, y, True)
     assert np.array_equal(y.to_host(), np.maximum(keep, 0))
+
+
+def test_layers_driven_from_two_threads():
+    """Distinct layer objects may be driven from different threads at once (the reference's ParallelNeuralNetwork does,
+    neural_network/ParallelNeuralNetwork.hpp:158-171); ctypes releases the interpreter lock during a call, so the
+    calls of the two threads do overlap."""
+    import threading
+    ch.init(0)
+    dtype = np.float32
+    results = {}
+
+    def work(tag, seed):
+        g = np.random.default_rng(seed)
+        x = np.asfortranarray(g.standard_normal((48, 20, 20, 8)).astype(dtype))      # 6 MB of output: staged copies too
+        w = np.asfortranarray((0.2 * g.standard_normal((72, 40))).astype(dtype))
+        layer = ch.ConvKernelLayer(dtype, (20, 20, 8), 40)
+        layer.get_params()[0].set_values(w)
+        outs = [layer.pass_forward(x, True) for _ in range(6)]
+        results[tag] = (x, w, outs)
+
+    threads = [threading.Thread(target=work, args=(i, 50 + i)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    from oracle import oracle
+    for tag in range(2):
+        x, w, outs = results[tag]
+        ref, _ = oracle.conv_forward(np.asarray(x, np.float64), np.asarray(w, np.float64), np.zeros((1, 40)), return_cache=True,
+                                     RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0)
+        for o in outs:
+            assert np.array_equal(o, outs[0])
+        err = np.max(np.abs(outs[0] - ref)) / np.sqrt(np.mean(ref ** 2))
+        assert err < 1e-4
