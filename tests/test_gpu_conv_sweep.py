@@ -86,3 +86,90 @@ def test_random_geometry(case, N):
     assert hp.rel_err(dx, dx_ref) < tol, "input gradient"
     assert hp.rel_err(wp.get_grad(), dw_ref) < tol, "weight gradient"
     assert hp.rel_err(bp.get_grad(), db_ref) < tol, "bias gradient"
+
+
+def _transconv_cases(count, seed):
+    g = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        RH, RW = int(g.integers(1, 5)), int(g.integers(1, 5))
+        dv, dh = int(g.integers(0, 2)), int(g.integers(0, 2))
+        sv, sh = int(g.integers(1, 4)), int(g.integers(1, 4))
+        pv, ph = int(g.integers(0, RH)), int(g.integers(0, RW))
+        IH, IW = int(g.integers(1, 14)), int(g.integers(1, 14))
+        OH, OW = oracle.transconv_out_dims(IH, IW, RH, RW, pv, ph, sv, sh, dv, dh)
+        if OH < 1 or OW < 1:
+            continue
+        C = int(g.choice([1, 2, 3, 8, 16, 33]))
+        F = int(g.choice([1, 3, 16, 32, 40, 64]))
+        N = int(g.choice([1, 3, 4, 8, 32, 33]))
+        if N * OH * OW * RH * RW * C * F > 4e8:
+            continue
+        out.append(((IH, IW, C, F, RH, RW, pv, ph, sv, sh, dv, dh), N))
+    return out
+
+
+TRANS_CASES = _transconv_cases(64, 20240613)
+
+
+@pytest.mark.parametrize("case,N", TRANS_CASES,
+                         ids=["t%dx%dx%d-f%d-r%dx%d-p%d%d-s%d%d-d%d%d-n%d" % (c + (n,)) for c, n in TRANS_CASES])
+def test_random_transposed_geometry(case, N):
+    IH, IW, C, F, RH, RW, pv, ph, sv, sh, dv, dh = case
+    dtype = np.float32 if (IH + IW + C + F + N) % 3 else np.float64
+    tol = 1e-4 if dtype == np.float32 else 1e-10
+    geom = dict(RH=RH, RW=RW, pv=pv, ph=ph, sv=sv, sh=sh, dv=dv, dh=dh)
+    g = hp.rng(2000 + IH * 31 + IW * 7 + C + F + N)
+    OH, OW = oracle.transconv_out_dims(IH, IW, RH, RW, pv, ph, sv, sh, dv, dh)
+    x = hp.uniform(g, (N, IH, IW, C), -1, 1, dtype)
+    w = hp.uniform(g, (C, RH * RW * F), -1, 1, dtype)
+    b = hp.uniform(g, (1, OH * OW * F), -1, 1, dtype)
+    go = hp.uniform(g, (N, OH, OW, F), -1, 1, dtype)
+    layer = ch.TransConvKernelLayer(dtype, (IH, IW, C), F, RH, RW, pv, ph, sv, sh, dv, dh)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    out = layer.pass_forward(x, True)
+    dx = layer.pass_back(go)
+    x64, w64, b64, go64 = (np.asarray(a, np.float64) for a in (x, w, b, go))
+    o_ref = oracle.transconv_forward(x64, w64, b64, F, **geom)
+    dx_ref, dw_ref, db_ref = oracle.transconv_backward(x64, w64, go64, **geom)
+    assert out.shape == o_ref.shape
+    assert hp.rel_err(out, o_ref) < tol, "forward"
+    assert hp.rel_err(dx, dx_ref) < tol, "input gradient"
+    assert hp.rel_err(wp.get_grad(), dw_ref) < tol, "weight gradient"
+    assert hp.rel_err(bp.get_grad(), db_ref) < tol, "bias gradient"
+
+
+def _pool_cases(count, seed):
+    g = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        RH, RW = int(g.integers(1, 5)), int(g.integers(1, 5))
+        sv, sh = int(g.integers(1, 5)), int(g.integers(1, 5))
+        H, W = int(g.integers(RH, RH + 20)), int(g.integers(RW, RW + 20))
+        C = int(g.choice([1, 2, 3, 8, 17]))
+        N = int(g.choice([1, 3, 4, 8, 32, 36, 64]))
+        out.append((H, W, C, RH, RW, sv, sh, N))
+    return out
+
+
+POOL_SWEEP = _pool_cases(64, 20240614)
+
+
+@pytest.mark.parametrize("H,W,C,RH,RW,sv,sh,N", POOL_SWEEP)
+def test_random_pool_geometry(H, W, C, RH, RW, sv, sh, N):
+    dtype = np.float32 if (H + W + C + N) % 2 else np.float64
+    g = hp.rng(3000 + H * 31 + W * 7 + C + N)
+    x = np.round(hp.normal(g, (N, H, W, C), dtype), 1)          # rounded: ties inside windows are common
+    mx = ch.MaxPoolLayer(dtype, (H, W, C), RH, RW, sv, sh)
+    out = mx.pass_forward(x, True)
+    o_ref, i_ref = oracle.maxpool_forward(x, RH, RW, sv, sh)
+    assert np.array_equal(out, o_ref)
+    assert np.array_equal(mx.max_indices(N), i_ref)
+    go = hp.normal(g, out.shape, dtype)
+    assert np.array_equal(mx.pass_back(go), oracle.maxpool_backward(x.shape, go, i_ref, RH, RW, sv, sh))
+    mn = ch.MeanPoolLayer(dtype, (H, W, C), RH, RW, sv, sh)
+    tol = 1e-4 if dtype == np.float32 else 1e-10
+    assert hp.rel_err(mn.pass_forward(x, True), oracle.meanpool_forward(np.asarray(x, np.float64), RH, RW, sv, sh)) < tol
+    assert hp.rel_err(mn.pass_back(go), oracle.meanpool_backward(x.shape, np.asarray(go, np.float64), RH, RW, sv, sh)) < tol
