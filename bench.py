@@ -113,6 +113,61 @@ def gpu_run(args, dtype):
     return dict(wall_ms=wall_ms, M=M, K=K, F=F, gemm_flop=gemm_flop, kernels=kernels, bytes=nbytes)
 
 
+def small_convs_run(args, dtype):
+    """The convolution shapes of the other BASELINE configurations, one layer at a time on device-resident tensors:
+    forward, weight + bias gradient and input gradient timed with HIP events. These are small-K or few-row problems,
+    so each line carries both bounds: roofline time = max(FLOP / matrix peak, algorithmic bytes / 8 TB/s), and the
+    fraction of it that the measured time reaches."""
+    ch = importlib.import_module("c-attl3_amd")
+    ch.init(0)
+    es = np.dtype(dtype).itemsize
+    peak = PEAK_TFLOPS[args.dtype] * 1e12
+    shapes = [
+        ("configs[0] conv 64x32x32x3 -> 16", 64, 32, 32, 3, 16),
+        ("configs[2] conv1 128x32x32x3 -> 32", 128, 32, 32, 3, 32),
+        ("configs[2] conv2 128x16x16x32 -> 64", 128, 16, 16, 32, 64),
+        ("configs[4] input-side gates, all 10 steps, 320x16x16x8 -> 128", 320, 16, 16, 8, 128),
+        ("configs[4] recurrent gates, one step, 32x16x16x32 -> 128", 32, 16, 16, 32, 128),
+    ]
+    gen = np.random.default_rng(11)
+    timer = ch.Timer()
+    reps = max(20, args.steps)
+    rows = []
+    for name, N, H, W, C, F in shapes:
+        K, M = 9 * C, N * H * W
+        layer = ch.ConvKernelLayer(dtype, (H, W, C), F)
+        layer.get_params()[0].set_values(he_normal(gen, K, F, dtype))
+        x = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H, W, C)).astype(dtype)))
+        go = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H, W, F)).astype(dtype)))
+        out = ch.DeviceTensor((N, H, W, F), dtype)
+        dx = ch.DeviceTensor((N, H, W, C), dtype)
+
+        def timed(fn):
+            for _ in range(3):
+                fn()
+            timer.start()
+            for _ in range(reps):
+                fn()
+            return timer.stop() / reps
+
+        t_fwd = timed(lambda: layer.forward_into(x, out, True))
+        t_bwd = timed(lambda: layer.backward_into(go, dx))
+        in_b, out_b, w_b = M * C * es, M * F * es, K * F * es
+        flop = 2.0 * M * K * F
+        for pass_name, t_ms, launches, nbytes in (("forward", t_fwd, 1, in_b + w_b + out_b),
+                                                  ("backward (weight, bias and input gradients)", t_bwd, 2, 2 * (in_b + out_b + w_b))):
+            roof_s = max(launches * flop / peak, nbytes / 8e12)
+            rows.append({"layer": name, "pass": pass_name, "M": M, "K": K, "F": F, "ms": round(t_ms, 4),
+                         "gflops": round(launches * flop / (t_ms * 1e-3) / 1e9, 1), "GB/s": round(nbytes / (t_ms * 1e-3) / 1e9, 1),
+                         "bound": "mfma" if launches * flop / peak >= nbytes / 8e12 else "hbm",
+                         "roofline_us": round(roof_s * 1e6, 2), "frac_of_roofline": round(roof_s / (t_ms * 1e-3), 4)})
+        for t in (x, go, out, dx):
+            t.free()
+    return {"metric": "small_conv_layer_passes", "unit": "ms", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+            "config": {"workload": "convolution layers of BASELINE configs[0], [2] and [4], one pass per line, tensors resident in HBM"},
+            "rows": rows}
+
+
 def pointwise_run(args, dtype):
     """HBM-bound layers at the cfg4 activation shape (N x 56 x 56 x 64): achieved GB/s against the
     algorithmic bytes per element of each pass (read x, write y, ...)."""
@@ -297,10 +352,11 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel of x's size (for scaling rocprof byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm", "train_steps"], default="conv",
+    ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm", "train_steps", "small_convs"], default="conv",
                     help="conv: the headline benchmark; pointwise: HBM-bound layers, one line of per-kernel GB/s; "
                          "convlstm: the fused-gate ConvLSTM of BASELINE configs[4], sequences/s; "
-                         "train_steps: whole device-resident training steps of BASELINE configs[1] and [2]")
+                         "train_steps: whole device-resident training steps of BASELINE configs[1] and [2]; "
+                         "small_convs: the convolution layers of the other configurations against both rooflines")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
@@ -318,6 +374,9 @@ def main():
         return
     if args.workload == "convlstm":
         print(json.dumps(convlstm_run(args, dtype)))
+        return
+    if args.workload == "small_convs":
+        print(json.dumps(small_convs_run(args, dtype)))
         return
 
     r = gpu_run(args, dtype)
