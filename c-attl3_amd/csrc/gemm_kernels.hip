@@ -764,6 +764,33 @@ void reduce_partials_kernel(const T* __restrict__ partials, T* __restrict__ dst,
 	}
 }
 
+/* The same sums for a small gradient (a few thousand values) cut into many partials: a wavefront per output, lane l
+ * adds the partials s = l, l + 64, ... in ascending order and the 64 lane sums are combined by a fixed shuffle tree.
+ * With few outputs the kernel above is a handful of blocks walking hundreds of partials one after the other. */
+template<typename T>
+__global__ __launch_bounds__(256)
+void reduce_partials_wide_kernel(const T* __restrict__ partials, T* __restrict__ dst, size_t count,
+		const T* __restrict__ bias_partials, T* __restrict__ bias_dst, size_t bias_count, int splits) {
+	size_t i = (size_t) blockIdx.x * 4 + threadIdx.x / 64;
+	if (i >= count + bias_count)
+		return;
+	if (i >= count) {
+		i -= count;
+		partials = bias_partials;
+		dst = bias_dst;
+		count = bias_count;
+	}
+	const int lane = threadIdx.x % 64;
+	T s = (T) 0;
+	for (int p = lane; p < splits; p += 64)
+		s += partials[(size_t) p * count + i];
+	#pragma unroll
+	for (int off = 32; off > 0; off >>= 1)
+		s += __shfl_down(s, off, 64);
+	if (lane == 0)
+		dst[i] += s;
+}
+
 /* Forward weights: wt[k][f] = w[k + K*f], zero-padded to Kp rows x ldw columns. */
 template<typename T>
 __global__ void prep_fwd_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, int K, int F, int Kp, int ldw) {
@@ -1133,13 +1160,15 @@ WgradVariant<T> wgrad_variant() {
 
 template<typename T> struct WgradVariants;
 template<> struct WgradVariants<float> {
-	static constexpr int COUNT = 4;
+	static constexpr int COUNT = 6;
 	static const WgradVariant<float>* get() {
 		static const WgradVariant<float> v[COUNT] = {
 			wgrad_variant<float, 2, 4, 96, 32, 4>(),    /* 192 x 128, registers held to four waves per SIMD = two blocks per CU */
 			wgrad_variant<float, 2, 2, 64, 64>(),       /* 128 x 128 */
 			wgrad_variant<float, 1, 4, 32, 32>(),       /*  32 x 128 */
 			wgrad_variant<float, 1, 4, 64, 32>(),       /*  64 x 128 */
+			wgrad_variant<float, 2, 2, 32, 32>(),       /*  64 x 64: few filters */
+			wgrad_variant<float, 1, 1, 32, 32>(),       /*  32 x 32, one wave: the first layer of a network (K = 27, a few filters) */
 		};
 		return v;
 	}
@@ -1161,7 +1190,7 @@ struct WgradPlan {
 	int variant, ktiles, ftiles, splits, chunks_per_split, pixel_mode;
 };
 
-/* The tile shape with the least padding wins (larger tile on ties: it re-reads G less often); the
+/* The tile shape with the least padded area wins, weighted by how often it re-reads its operands; the
  * M range is then cut into as many slices as fill the chip once (blocks = tiles * splits <= slots),
  * so that no block runs in a second, mostly idle round; the slots are what the runtime's occupancy query
  * reports for the variant. The plan depends on the shape and the build only, which keeps the summation
@@ -1173,9 +1202,11 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	p.variant = 0;
 	long best = -1;
 	for (int i = 0; i < WgradVariants<T>::COUNT; ++i) {
+		/* MFMA work grows with the padded area, operand loads per unit of it with 1 / bk + 1 / bf */
 		const long padded = (long) round_up(K, vars[i].bk) * round_up(F, vars[i].bf);
-		if (best < 0 || padded < best) {
-			best = padded;
+		const long cost = padded + padded * 16 / vars[i].bk + padded * 16 / vars[i].bf;
+		if (best < 0 || cost < best) {
+			best = cost;
 			p.variant = i;
 		}
 	}
@@ -1187,7 +1218,8 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	const WgradVariant<T>& v = vars[p.variant];
 	p.ktiles = (K + v.bk - 1) / v.bk;
 	p.ftiles = (F + v.bf - 1) / v.bf;
-	const int occ = std::max(1, std::min(v.blocks_per_cu(), 3));
+	/* at most three blocks of eight waves per CU; small blocks up to sixteen waves' worth */
+	const int occ = std::max(1, std::min(v.blocks_per_cu(), std::max(3, 16 / v.waves)));
 	const int slots = NUM_CUS * occ;
 	const int tiles = p.ktiles * p.ftiles;
 	const int chunks = (M + WGRAD_MC - 1) / WGRAD_MC;
@@ -1248,6 +1280,13 @@ void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_gr
 	v.launch(x, out_grad, partials, bias_partials, g, split, vec);
 	const int wblocks = (int) ((count + 63) / 64), bblocks = bgrad ? (g.F + 63) / 64 : 0;
 	constexpr int V = 16 / (int) sizeof(T);
+	const size_t outputs = count + (bgrad ? (size_t) g.F : 0);
+	if (outputs <= 8192 && p.splits >= 32) {
+		reduce_partials_wide_kernel<T><<<(unsigned) ((outputs + 3) / 4), 256, 0, stream()>>>(partials, wgrad, count, bias_partials,
+				bgrad, bgrad ? (size_t) g.F : 0, p.splits);
+		CATTLE_HIP_CHECK(hipGetLastError());
+		return;
+	}
 	if (count % V == 0 && g.F % V == 0 && (reinterpret_cast<uintptr_t>(partials) & 15) == 0)
 		reduce_partials_kernel<T, V><<<(unsigned) (wblocks + bblocks), 256, 0, stream()>>>(partials, wgrad, count, bias_partials,
 				bgrad, (size_t) g.F, wblocks, p.splits);
