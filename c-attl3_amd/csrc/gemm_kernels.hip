@@ -944,7 +944,7 @@ GatherVariant<T> gather_variant() {
 
 template<typename T> struct GatherVariants;
 template<> struct GatherVariants<float> {
-	static constexpr int COUNT = 6, LARGE = 4;
+	static constexpr int COUNT = 8, LARGE = 4, SHORT = 2;
 	static const GatherVariant<float>* get() {
 		static const GatherVariant<float> v[COUNT] = {
 			gather_variant<float, 4, 2, 64, 64>(),      /* 256 x 128 */
@@ -955,12 +955,14 @@ template<> struct GatherVariants<float> {
 			 * reduction chunks because with one block per CU only the loads in flight hide memory latency */
 			gather_variant<float, 2, 2, 32, 32, 64>(),  /* 64 x 64 */
 			gather_variant<float, 2, 1, 32, 32, 64>(),  /* 64 x 32 */
+			gather_variant<float, 2, 2, 32, 32, 32>(),  /* 64 x 64, chunks of 32: several short tiles per CU */
+			gather_variant<float, 2, 1, 32, 32, 32>(),  /* 64 x 32, chunks of 32 */
 		};
 		return v;
 	}
 };
 template<> struct GatherVariants<double> {
-	static constexpr int COUNT = 5, LARGE = 3;
+	static constexpr int COUNT = 7, LARGE = 3, SHORT = 2;
 	static const GatherVariant<double>* get() {
 		static const GatherVariant<double> v[COUNT] = {
 			gather_variant<double, 8, 2, 32, 64>(),     /* 256 x 128, sixteen waves */
@@ -968,6 +970,8 @@ template<> struct GatherVariants<double> {
 			gather_variant<double, 4, 1, 64, 32>(),     /* 256 x 32 */
 			gather_variant<double, 2, 2, 32, 32, 32>(), /* 64 x 64, small problems */
 			gather_variant<double, 2, 1, 32, 32, 32>(), /* 64 x 32 */
+			gather_variant<double, 2, 2, 32, 32, 16>(), /* 64 x 64, chunks of 16: several short tiles per CU */
+			gather_variant<double, 2, 1, 32, 32, 16>(), /* 64 x 32, chunks of 16 */
 		};
 		return v;
 	}
@@ -992,10 +996,15 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	}
 	/* too few large tiles to give every CU one: take the short tiles (the narrowest that still covers F, else the widest) */
 	if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) < NUM_CUS) {
+		constexpr int SHORT = GatherVariants<T>::SHORT;       /* short shapes, each with long and with medium chunks */
 		best_v = GatherVariants<T>::LARGE;
-		for (int i = GatherVariants<T>::LARGE + 1; i < GatherVariants<T>::COUNT; ++i)
+		for (int i = GatherVariants<T>::LARGE + 1; i < GatherVariants<T>::LARGE + SHORT; ++i)
 			if (vars[i].bf >= g.F && vars[i].bf < vars[best_v].bf)
 				best_v = i;
+		/* enough short tiles for two or more per CU: the medium chunks, whose smaller LDS footprint lets four
+		 * blocks share a CU; fewer: the long chunks, with which one block keeps more loads in flight */
+		if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) >= 2 * NUM_CUS)
+			best_v += SHORT;
 	}
 	/* tuning overrides for experiments, keyed by the number of output columns F of the GEMM:
 	 * CATTLE_HIP_GATHER_VARIANT_F<F> = index into the variant table, CATTLE_HIP_GATHER_OCC_F<F> = blocks per CU
