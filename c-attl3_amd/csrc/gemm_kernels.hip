@@ -1199,7 +1199,7 @@ struct WgradPlan {
 	int variant, ktiles, ftiles, splits, chunks_per_split, pixel_mode;
 };
 
-/* The tile shape with the least padded area wins, weighted by how often it re-reads its operands; the
+/* The tile shape with the least padding wins (the earlier, larger one on ties: it re-reads G less often); the
  * M range is then cut into as many slices as fill the chip once (blocks = tiles * splits <= slots),
  * so that no block runs in a second, mostly idle round; the slots are what the runtime's occupancy query
  * reports for the variant. The plan depends on the shape and the build only, which keeps the summation
@@ -1211,11 +1211,9 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	p.variant = 0;
 	long best = -1;
 	for (int i = 0; i < WgradVariants<T>::COUNT; ++i) {
-		/* MFMA work grows with the padded area, operand loads per unit of it with 1 / bk + 1 / bf */
 		const long padded = (long) round_up(K, vars[i].bk) * round_up(F, vars[i].bf);
-		const long cost = padded + padded * 16 / vars[i].bk + padded * 16 / vars[i].bf;
-		if (best < 0 || cost < best) {
-			best = cost;
+		if (best < 0 || padded < best) {
+			best = padded;
 			p.variant = i;
 		}
 	}
