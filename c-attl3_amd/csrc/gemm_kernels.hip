@@ -1169,11 +1169,12 @@ WgradVariant<T> wgrad_variant() {
 
 template<typename T> struct WgradVariants;
 template<> struct WgradVariants<float> {
-	static constexpr int COUNT = 6;
+	static constexpr int COUNT = 7;
 	static const WgradVariant<float>* get() {
 		static const WgradVariant<float> v[COUNT] = {
 			wgrad_variant<float, 2, 4, 96, 32, 4>(),    /* 192 x 128, registers held to four waves per SIMD = two blocks per CU */
 			wgrad_variant<float, 2, 2, 64, 64>(),       /* 128 x 128 */
+			wgrad_variant<float, 1, 4, 96, 32>(),       /*  96 x 128: K = 288 (3 x 3 x 32 channels) without padding */
 			wgrad_variant<float, 1, 4, 32, 32>(),       /*  32 x 128 */
 			wgrad_variant<float, 1, 4, 64, 32>(),       /*  64 x 128 */
 			wgrad_variant<float, 2, 2, 32, 32>(),       /*  64 x 64: few filters */
