@@ -22,6 +22,7 @@
 #include <cstring>
 #include <mutex>
 #include <thread>
+#include <unistd.h>
 #include <vector>
 
 namespace cattle_hip {
@@ -42,8 +43,9 @@ struct CopyPool {
 	size_t bytes = 0, slice = 0;
 	unsigned long generation = 0;
 	int pending = 0;
+	pid_t owner;            /* threads do not survive fork(): a child process copies on its own thread */
 
-	explicit CopyPool(int threads) {
+	explicit CopyPool(int threads) : owner(getpid()) {
 		for (int i = 1; i < threads; ++i)
 			workers.emplace_back([this, i] { run(i); });
 		for (std::thread& t : workers)
@@ -73,7 +75,7 @@ struct CopyPool {
 	}
 	void copy(void* d, const void* s, size_t n) {
 		const int threads = (int) workers.size() + 1;
-		if (threads == 1 || n < ((size_t) 1 << 20)) {
+		if (threads == 1 || n < ((size_t) 1 << 20) || getpid() != owner) {
 			std::memcpy(d, s, n);
 			return;
 		}
