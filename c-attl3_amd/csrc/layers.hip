@@ -433,8 +433,9 @@ struct ConvLstm : LayerBase {
 		act_state.ensure(p * total * e);
 		hid.ensure(p * total * e);
 		zh.ensure(4 * p * e);
-		/* slab t of hprev_all is the hidden output of step t - 1 (slab 0 stays zero: no previous output) */
-		fill_zero(hprev_all.ensure(p * total * e), p * total * e);
+		/* slab t of hprev_all is the hidden output of step t - 1 (the first step's kernel zeroes slab 0: no previous
+		 * output); every slab is written once per pass */
+		hprev_all.ensure(p * total * e);
 		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
 		T* wth = (T*) wh.derived[0].ensure(wsh.wt_fwd * e);
 		for (size_t t = 0; t < total; ++t) {
@@ -448,7 +449,7 @@ struct ConvLstm : LayerBase {
 			lstm_gates_forward<T>(acts, n, p, has_in ? (const T*) zx_all.p : nullptr, (int) in_len, (int) t,
 					has_prev ? (const T*) zh.p : nullptr, has_prev ? step(state, t - 1, p) : nullptr, step(z, t, 4 * p),
 					step(gates, t, 4 * p), step(state, t, p), step(act_state, t, p), step(hid, t, p),
-					t + 1 < total ? (T*) hprev_all.p : nullptr, (int) total, (int) (t + 1), emits ? out : nullptr, (int) out_len,
+					(T*) hprev_all.p, (int) total, (int) (t + 1), emits ? out : nullptr, (int) out_len,
 					(int) (t - out_delay));
 		}
 		x_cache = input;
@@ -462,11 +463,11 @@ struct ConvLstm : LayerBase {
 		const int n = (int) N;
 		Param& wx = *params[0];
 		Param& wh = *params[2];
-		fill_zero(state_grad.ensure(p * e), p * e);                      /* :422-425 */
+		state_grad.ensure(p * e);                                        /* starts at zero (:422-425): the last step's kernel ignores it */
 		dz.ensure(4 * p * e);
 		dh.ensure(p * e);
 		dzx_all.ensure(4 * p * T_in * e);
-		fill_zero(dzh_all.ensure(4 * p * total * e), 4 * p * total * e);
+		dzh_all.ensure(4 * p * total * e);                               /* every slab is written; step 0 writes zeros */
 		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
 		T* wtd = (T*) wh.derived[1].ensure(wsh.wt_dgrad * e);
 		for (size_t t = total; t-- > 0;) {
@@ -475,7 +476,7 @@ struct ConvLstm : LayerBase {
 			lstm_gates_backward<T>(acts, n, p, t + 1 < total ? (const T*) dh.p : nullptr, emitted ? out_grad : nullptr,
 					(int) T_out, (int) (t - delay), step(z, t, 4 * p), step(gates, t, 4 * p),
 					has_prev ? step(state, t - 1, p) : nullptr, step(state, t, p), step(act_state, t, p), (T*) state_grad.p,
-					(T*) dz.p, has_in ? (T*) dzx_all.p : nullptr, (int) T_in, (int) t, has_prev ? (T*) dzh_all.p : nullptr,
+					(T*) dz.p, has_in ? (T*) dzx_all.p : nullptr, (int) T_in, (int) t, (T*) dzh_all.p,
 					(int) total, (int) t);
 			if (has_prev) {
 				/* the four output-side kernels' pass_back, summed (:470-473, :491-494): one input-gradient launch */

@@ -877,8 +877,12 @@ void lstm_gates_forward_kernel(LstmActs<T> a, int N, size_t P, const T* __restri
 		act_state[e] = as;
 		const T h = y[3] * as;                                      /* read filter * activated state (:383) */
 		hidden[e] = h;
-		if (hprev_all)
-			hprev_all[seq_offset(n, rest, N, h_T, h_t)] = h;
+		if (hprev_all) {
+			if (h_t < h_T)
+				hprev_all[seq_offset(n, rest, N, h_T, h_t)] = h;
+			if (!prev_state)                                        /* first step: no previous output, slab 0 is zero */
+				hprev_all[seq_offset(n, rest, N, h_T, 0)] = (T) 0;
+		}
 		if (out)
 			out[seq_offset(n, rest, N, out_T, out_t)] = h;
 	}
@@ -899,7 +903,8 @@ void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restr
 			hg += out_grad[seq_offset(n, rest, N, og_T, og_t)];     /* :431-438 */
 		const T f = gates[e], w = gates[P + e], c = gates[2 * P + e], r = gates[3 * P + e];
 		const T as = act_state[e];
-		const T sg = state_grad[e] + act_b_rt<T>(a.kind[3], state[e], as, r * hg, a.param[3]);      /* :440 */
+		/* the state gradient starts at zero (:422-425) at the last time step, the one without a dh */
+		const T sg = (dh ? state_grad[e] : (T) 0) + act_b_rt<T>(a.kind[3], state[e], as, r * hg, a.param[3]);      /* :440 */
 		T d[4];
 		d[3] = act_b_rt<T>(a.kind[4], z[3 * P + e], r, as * hg, a.param[4]);                       /* :441 */
 		d[2] = act_b_rt<T>(a.kind[2], z[2 * P + e], c, w * sg, a.param[2]);                        /* :442 */
@@ -911,8 +916,8 @@ void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restr
 			dz[g * P + e] = d[g];
 			if (dzx_all)
 				dzx_all[seq_offset(n, rest + g * slab_rows, N, x_T, x_t)] = d[g];
-			if (dzh_all)
-				dzh_all[seq_offset(n, rest + g * slab_rows, N, h_T, h_t)] = d[g];
+			if (dzh_all)        /* step 0 has no previous output to pair with: its slab is zero */
+				dzh_all[seq_offset(n, rest + g * slab_rows, N, h_T, h_t)] = prev_state ? d[g] : (T) 0;
 		}
 	}
 }

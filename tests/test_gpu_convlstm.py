@@ -123,3 +123,23 @@ def test_device_resident_sequences_and_errors():
     fresh = ch.ConvLSTMNetwork(np.float32, (6, 5, 3), 4)
     with pytest.raises(ch.CattleHipError):
         fresh.backpropagate(go)                                        # no propagate yet
+
+
+def test_a_network_reused_with_another_sequence_length():
+    """The step-shifted device buffers are written slab by slab in every pass, never cleared as a whole: a pass
+    after a longer one on the same network gives, bit for bit, what a fresh network gives."""
+    dtype, dims, hidden = np.float32, (6, 5, 3), 4
+    seq = lambda T: (T, 0)
+    used, _, g = _pair(dtype, dims, hidden, SMOOTH, False, seq, 21)
+    fresh, _, _ = _pair(dtype, dims, hidden, SMOOTH, False, seq, 21)
+    x_long = hp.normal(g, (6, 5) + dims, dtype)
+    used.propagate(x_long)
+    used.backpropagate(hp.normal(g, (6, 5, dims[0], dims[1], hidden), dtype))
+    for p in used.get_params():
+        p.reset_grad()
+    x = hp.normal(g, (4, 3) + dims, dtype)
+    go = hp.normal(g, (4, 3, dims[0], dims[1], hidden), dtype)
+    assert np.array_equal(used.propagate(x), fresh.propagate(x))
+    assert np.array_equal(used.backpropagate(go), fresh.backpropagate(go))
+    for a, b in zip(used.get_params(), fresh.get_params()):
+        assert np.array_equal(a.get_grad(), b.get_grad())
