@@ -37,7 +37,7 @@ EXPORTS = [
     "cattle_hip_layer_num_params", "cattle_hip_layer_param_shape", "cattle_hip_layer_set_param_values",
     "cattle_hip_layer_get_param_values", "cattle_hip_layer_get_param_grad", "cattle_hip_layer_reset_param_grad",
     "cattle_hip_maxpool_indices", "cattle_hip_loss_function", "cattle_hip_loss_d_function",
-    "cattle_hip_layer_param_optimizer_update", "cattle_hip_layer_param_optimizer_step", "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
+    "cattle_hip_layer_param_optimizer_update", "cattle_hip_layer_param_optimizer_step", "cattle_hip_optimizer_step_many", "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
     "cattle_hip_layer_param_reset_optimizer_state", "cattle_hip_convlstm_create", "cattle_hip_convlstm_propagate",
     "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
     "cattle_hip_convlstm_get_kernel_grad",
@@ -225,6 +225,25 @@ class Parameters(object):
 
 LOSS = {"squared": 0, "softmax_cross_entropy": 1}
 _HYPER_ARRAYS = {}
+
+
+class ParameterList(object):
+    """The optimizable parameters of a network, updated and reset together (optimizer_step of each, one launch per
+    sixteen): SGDOptimizer::_train's loops over get_all_unique_params (optimizer/SGDOptimizer.hpp:58-70)."""
+
+    def __init__(self, params):
+        self._params = [p for p in params if p.are_optimizable()]
+        n = len(self._params)
+        self._layers = (ctypes.c_void_p * n)(*[p._layer._h for p in self._params])
+        self._indices = (ctypes.c_size_t * n)(*[p._index for p in self._params])
+
+    def __len__(self):
+        return len(self._params)
+
+    def optimizer_step(self, optimizer, hyper, epoch=0, timestep=0):
+        _check(lib().cattle_hip_optimizer_step_many(self._layers, self._indices, _sz(len(self._params)),
+                                                    ctypes.c_int(OPTIMIZERS[optimizer]), _hyper_array(tuple(hyper)),
+                                                    _sz(epoch), _sz(timestep)))
 
 
 def _hyper_array(hyper):

@@ -77,6 +77,9 @@ struct ConvWorkspace {
 };
 
 template<typename T> ConvWorkspace conv_workspace(const ConvShape& s, int N);
+/* Row length of a prepared weight layout with `columns` used columns: wt_fwd is [rows][row length] over the F filters,
+ * wt_dgrad over the C channels (rows zero-padded to whole reduction chunks, columns to the row length). */
+int prepared_weight_row_length(int columns);
 
 /* Forward: out(N,OH,OW,F) = conv(x; w) + b. w is the reference's [K x F] column-major matrix.
  * wt is scratch of conv_workspace().wt_fwd elements; if wt_ready is false it is (re)built from w. */
@@ -154,6 +157,18 @@ enum { OPT_VANILLA_SGD = 0, OPT_MOMENTUM_SGD = 1, OPT_NESTEROV = 2, OPT_ADAGRAD 
 	OPT_ADAM = 6, OPT_ADAMAX = 7, OPT_NADAM = 8, OPT_AMSGRAD = 9 };
 template<typename T> struct OptCoef { T c[8]; };
 int optimizer_state_count(int rule);
+/* One parameter of a multi-parameter optimizer launch: its n elements, gradient, values and state matrices, and,
+ * for a K x F convolution or dense weight matrix whose prepared layouts are current, those layouts (wt_fwd with row
+ * length ldw_fwd; wt_dgrad for a receptor of RHW positions with row length ldw_dgrad), else null. */
+constexpr int OPT_BATCH = 16;
+template<typename T> struct OptParam {
+	T* grad; T* values; T* s0; T* s1; T* s2; T* wt_fwd; T* wt_dgrad;
+	size_t n;
+	int K, RHW, ldw_fwd, ldw_dgrad;
+};
+template<typename T> struct OptBatch { OptParam<T> p[OPT_BATCH]; int count; };
+/* update + gradient reset of every parameter of the batch, one launch */
+template<typename T> void optimizer_step_many(int rule, const double hyper[4], size_t epoch, size_t timestep, const OptBatch<T>& batch);
 /* reset_grad: zero the gradient in the same kernel, after it has been used */
 template<typename T> void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n,
 		T* grad, T* s0, T* s1, T* s2, T* values, bool reset_grad);

@@ -1248,6 +1248,10 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 
 } /* namespace */
 
+int prepared_weight_row_length(int columns) {
+	return round_up(columns, WT_COL_PAD);
+}
+
 template<typename T>
 ConvWorkspace conv_workspace(const ConvShape& s, int N) {
 	check_sizes(s, N);

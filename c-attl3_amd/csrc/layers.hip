@@ -808,6 +808,66 @@ void run_optimizer(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer 
 	++p.version;
 }
 
+/* The update + gradient reset of many parameters, OPT_BATCH per launch. A parameter shared by several of the listed
+ * layers is updated once. Weight matrices of convolution and dense layers whose prepared layouts are current have
+ * them rewritten by the same kernel and stay current. */
+template<typename T>
+void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices, size_t count, cattle_hip_optimizer optimizer,
+		const double hyper[4], size_t epoch, size_t timestep) {
+	const int states = optimizer_state_count((int) optimizer);
+	std::vector<Param*> seen;
+	OptBatch<T> batch;
+	batch.count = 0;
+	auto flush = [&] {
+		optimizer_step_many<T>((int) optimizer, hyper, epoch, timestep, batch);
+		batch.count = 0;
+	};
+	for (size_t i = 0; i < count; ++i) {
+		Param& p = optimizable_param(layers[i], indices[i]);
+		CATTLE_HIP_REQUIRE(p.esize == sizeof(T), "parameters of one optimizer step must share a scalar type");
+		if (std::find(seen.begin(), seen.end(), &p) != seen.end())
+			continue;
+		seen.push_back(&p);
+		for (int m = p.moments_ready; m < states; ++m) {
+			fill_zero(p.moments[m].ensure(p.bytes()), p.bytes());
+			p.moments_ready = m + 1;
+		}
+		OptParam<T>& q = batch.p[batch.count++];
+		q.grad = static_cast<T*>(p.grad.p);
+		q.values = static_cast<T*>(p.values.p);
+		q.s0 = static_cast<T*>(p.moments[0].p);
+		q.s1 = static_cast<T*>(p.moments[1].p);
+		q.s2 = static_cast<T*>(p.moments[2].p);
+		q.n = p.rows * p.cols;
+		q.wt_fwd = q.wt_dgrad = nullptr;
+		q.K = q.RHW = 1;
+		q.ldw_fwd = q.ldw_dgrad = 0;
+		const ConvLayer<T>* conv = dynamic_cast<const ConvLayer<T>*>(as_layer(layers[i]));
+		bool fwd_current = false, dgrad_current = false;
+		if (conv && indices[i] == 0) {
+			const ConvShape& cs = conv->shape;
+			fwd_current = p.derived[0].p && p.derived_version[0] == p.version;
+			dgrad_current = p.derived[1].p && p.derived_version[1] == p.version;
+			q.K = cs.K();
+			q.RHW = cs.RH * cs.RW;
+			q.ldw_fwd = prepared_weight_row_length(cs.F);
+			q.ldw_dgrad = prepared_weight_row_length(cs.C);
+			if (fwd_current)
+				q.wt_fwd = static_cast<T*>(p.derived[0].p);
+			if (dgrad_current)
+				q.wt_dgrad = static_cast<T*>(p.derived[1].p);
+		}
+		++p.version;
+		if (fwd_current)
+			p.derived_version[0] = p.version;
+		if (dgrad_current)
+			p.derived_version[1] = p.version;
+		if (batch.count == OPT_BATCH)
+			flush();
+	}
+	flush();
+}
+
 
 
 template<typename T>
@@ -1434,6 +1494,20 @@ int cattle_hip_layer_param_optimizer_update(cattle_hip_layer_t layer, size_t ind
 int cattle_hip_layer_param_optimizer_step(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
 		const double hyper[4], size_t epoch, size_t timestep) {
 	return guarded([&] { run_optimizer(layer, index, optimizer, hyper, epoch, timestep, true); });
+}
+
+int cattle_hip_optimizer_step_many(const cattle_hip_layer_t* layers, const size_t* indices, size_t count,
+		cattle_hip_optimizer optimizer, const double hyper[4], size_t epoch, size_t timestep) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(count == 0 || (layers != nullptr && indices != nullptr), "null parameter list");
+		CATTLE_HIP_REQUIRE(hyper != nullptr, "null hyper-parameter array");
+		if (count == 0)
+			return;
+		if (as_layer(layers[0])->dtype == CATTLE_HIP_F32)
+			run_optimizer_many<float>(layers, indices, count, optimizer, hyper, epoch, timestep);
+		else
+			run_optimizer_many<double>(layers, indices, count, optimizer, hyper, epoch, timestep);
+	});
 }
 
 int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate) {

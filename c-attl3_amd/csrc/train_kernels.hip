@@ -138,60 +138,117 @@ void softmax_ce_kernel(int N, int T_steps, int V, T eps, T scale, const T* __res
  *   OPT_NADAM         optimizer/NadamOptimizer.hpp:44-65             k: d1, d2, lr, l2_corr, eps, d1 * l1_corr, (1 - d1) * l1_next_corr
  *   OPT_AMSGRAD       optimizer/AMSGradOptimizer.hpp:48-66           k: d1, d2, lr, -, eps */
 template<typename T, int RULE>
+__device__ __forceinline__ T optimizer_element(const OptCoef<T>& k, T g, T v, T* __restrict__ s0, T* __restrict__ s1,
+		T* __restrict__ s2, size_t i) {
+	const T one = (T) 1;
+	if (RULE == OPT_VANILLA_SGD) {
+		return v - g * k.c[0];
+	} else if (RULE == OPT_MOMENTUM_SGD) {
+		const T s = s0[i] * k.c[1] + g * k.c[0];
+		s0[i] = s;
+		return v - s;
+	} else if (RULE == OPT_NESTEROV) {
+		const T old = s0[i];
+		const T s = old * k.c[1] - g * k.c[0];
+		s0[i] = s;
+		return v + old * -k.c[1] + s * (one + k.c[1]);
+	} else if (RULE == OPT_ADAGRAD || RULE == OPT_RMSPROP) {
+		const T a = RULE == OPT_ADAGRAD ? s0[i] + g * g : s0[i] * (one - k.c[2]) + g * g * k.c[2];
+		s0[i] = a;
+		return v - g * k.c[0] / (dev_sqrt(a) + k.c[1]);
+	} else if (RULE == OPT_ADADELTA) {
+		const T a = s0[i] * (one - k.c[0]) + g * g * k.c[0];
+		const T upd = -g * dev_sqrt(s1[i] + k.c[1]) / dev_sqrt(a + k.c[1]);
+		s0[i] = a;
+		s1[i] = s1[i] * (one - k.c[0]) + upd * upd * k.c[0];
+		return v + upd;
+	} else {
+		const T m = s0[i] * (one - k.c[0]) + g * k.c[0];
+		s0[i] = m;
+		if (RULE == OPT_ADAMAX) {
+			const T decayed = s1[i] * (one - k.c[1]), ag = g < (T) 0 ? -g : g;
+			const T u = decayed > ag ? decayed : ag;
+			s1[i] = u;
+			return v - (m * k.c[2]) / (u + k.c[4]);
+		}
+		const T sq = s1[i] * (one - k.c[1]) + g * g * k.c[1];
+		s1[i] = sq;
+		if (RULE == OPT_ADAM)
+			return v - (m * k.c[2]) / dev_sqrt(sq * k.c[3] + k.c[4]);
+		if (RULE == OPT_NADAM)
+			return v - ((g * k.c[5] + m * k.c[6]) * k.c[2]) / dev_sqrt(sq * k.c[3] + k.c[4]);
+		/* OPT_AMSGRAD */
+		const T prev = s2[i];
+		const T mx = sq > prev ? sq : prev;
+		s2[i] = mx;
+		return v - (m * k.c[2]) / dev_sqrt(mx + k.c[4]);
+	}
+}
+
+template<typename T, int RULE>
 __global__ __launch_bounds__(256)
 void optimizer_update_kernel(size_t total, OptCoef<T> k, T* __restrict__ grad, T* __restrict__ s0, T* __restrict__ s1,
 		T* __restrict__ s2, T* __restrict__ values, bool reset_grad) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
-	const T one = (T) 1;
 	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-		const T g = grad[i];
-		const T v = values[i];
-		if (RULE == OPT_VANILLA_SGD) {
-			values[i] = v - g * k.c[0];
-		} else if (RULE == OPT_MOMENTUM_SGD) {
-			const T s = s0[i] * k.c[1] + g * k.c[0];
-			s0[i] = s;
-			values[i] = v - s;
-		} else if (RULE == OPT_NESTEROV) {
-			const T old = s0[i];
-			const T s = old * k.c[1] - g * k.c[0];
-			s0[i] = s;
-			values[i] = v + old * -k.c[1] + s * (one + k.c[1]);
-		} else if (RULE == OPT_ADAGRAD || RULE == OPT_RMSPROP) {
-			const T a = RULE == OPT_ADAGRAD ? s0[i] + g * g : s0[i] * (one - k.c[2]) + g * g * k.c[2];
-			s0[i] = a;
-			values[i] = v - g * k.c[0] / (dev_sqrt(a) + k.c[1]);
-		} else if (RULE == OPT_ADADELTA) {
-			const T a = s0[i] * (one - k.c[0]) + g * g * k.c[0];
-			const T upd = -g * dev_sqrt(s1[i] + k.c[1]) / dev_sqrt(a + k.c[1]);
-			s0[i] = a;
-			values[i] = v + upd;
-			s1[i] = s1[i] * (one - k.c[0]) + upd * upd * k.c[0];
-		} else {
-			const T m = s0[i] * (one - k.c[0]) + g * k.c[0];
-			s0[i] = m;
-			if (RULE == OPT_ADAMAX) {
-				const T decayed = s1[i] * (one - k.c[1]), ag = g < (T) 0 ? -g : g;
-				const T u = decayed > ag ? decayed : ag;
-				s1[i] = u;
-				values[i] = v - (m * k.c[2]) / (u + k.c[4]);
-			} else {
-				const T sq = s1[i] * (one - k.c[1]) + g * g * k.c[1];
-				s1[i] = sq;
-				if (RULE == OPT_ADAM) {
-					values[i] = v - (m * k.c[2]) / dev_sqrt(sq * k.c[3] + k.c[4]);
-				} else if (RULE == OPT_NADAM) {
-					values[i] = v - ((g * k.c[5] + m * k.c[6]) * k.c[2]) / dev_sqrt(sq * k.c[3] + k.c[4]);
-				} else {        /* OPT_AMSGRAD */
-					const T prev = s2[i];
-					const T mx = sq > prev ? sq : prev;
-					s2[i] = mx;
-					values[i] = v - (m * k.c[2]) / dev_sqrt(mx + k.c[4]);
-				}
-			}
-		}
+		values[i] = optimizer_element<T, RULE>(k, grad[i], values[i], s0, s1, s2, i);
 		if (reset_grad)                 /* Parameters::reset_grad after the update (optimizer/SGDOptimizer.hpp:68-70) */
 			grad[i] = (T) 0;
+	}
+}
+
+/* The update and gradient reset of up to OPT_BATCH parameters in one launch (blockIdx.y picks the parameter,
+ * blockIdx.x a run of 1024 elements, or a 32 x 32 tile of the matrix). A convolution or dense weight matrix may
+ * bring its prepared layouts along (the forward layout wt[k][f] and the input-gradient layout wd[tap + RHW * f][c],
+ * both zero-padded when they were first built): the new values are written there as well, which saves the two
+ * re-layout launches of the next pass. The matrix is column-major (k fastest) and wt is f fastest, so a tile goes
+ * through LDS and both sides are accessed along their contiguous index. */
+template<typename T, int RULE>
+__global__ __launch_bounds__(256)
+void optimizer_step_many_kernel(OptBatch<T> batch, OptCoef<T> k) {
+	__shared__ T tile[32][33];
+	const OptParam<T>& q = batch.p[blockIdx.y];
+	const int tid = threadIdx.x;
+	if (!q.wt_fwd && !q.wt_dgrad) {
+		#pragma unroll
+		for (int j = 0; j < 4; ++j) {
+			const size_t i = (size_t) blockIdx.x * 1024 + tid + 256 * j;
+			if (i < q.n) {
+				q.values[i] = optimizer_element<T, RULE>(k, q.grad[i], q.values[i], q.s0, q.s1, q.s2, i);
+				q.grad[i] = (T) 0;
+			}
+		}
+		return;
+	}
+	const int F = (int) (q.n / (size_t) q.K);
+	const int tiles_k = (q.K + 31) / 32;
+	if ((int) blockIdx.x >= tiles_k * ((F + 31) / 32))
+		return;
+	const int k0 = ((int) blockIdx.x % tiles_k) * 32, f0 = ((int) blockIdx.x / tiles_k) * 32;
+	const int a = tid % 32, b = tid / 32;
+	#pragma unroll
+	for (int j = 0; j < 4; ++j) {
+		const int row = k0 + a, f = f0 + b + 8 * j;
+		if (row < q.K && f < F) {
+			const size_t i = (size_t) row + (size_t) q.K * f;
+			const T v = optimizer_element<T, RULE>(k, q.grad[i], q.values[i], q.s0, q.s1, q.s2, i);
+			q.values[i] = v;
+			q.grad[i] = (T) 0;
+			tile[b + 8 * j][a] = v;
+			if (q.wt_dgrad) {
+				const unsigned tap = (unsigned) row % (unsigned) q.RHW, c = (unsigned) row / (unsigned) q.RHW;
+				q.wt_dgrad[(size_t) (tap + (unsigned) q.RHW * f) * q.ldw_dgrad + c] = v;
+			}
+		}
+	}
+	if (!q.wt_fwd)
+		return;
+	__syncthreads();
+	#pragma unroll
+	for (int j = 0; j < 4; ++j) {
+		const int row = k0 + b + 8 * j, f = f0 + a;
+		if (row < q.K && f < F)
+			q.wt_fwd[(size_t) row * q.ldw_fwd + f] = tile[a][b + 8 * j];
 	}
 }
 
@@ -254,11 +311,9 @@ int optimizer_state_count(int rule) {
 	}
 }
 
+/* The scalars of one optimizer step. */
 template<typename T>
-void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n, T* grad, T* s0, T* s1,
-		T* s2, T* values, bool reset_grad) {
-	if (n == 0)
-		return;
+OptCoef<T> optimizer_coefficients(int rule, const double hyper[4], size_t epoch, size_t timestep) {
 	OptCoef<T> k;
 	for (int i = 0; i < 8; ++i)
 		k.c[i] = (T) 0;
@@ -303,26 +358,63 @@ void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t time
 	default:
 		throw Error(ERR_INVALID, "unknown optimizer");
 	}
-	const unsigned grid = flat_grid(n);
-	switch (rule) {
-	case OPT_VANILLA_SGD: optimizer_update_kernel<T, OPT_VANILLA_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_MOMENTUM_SGD: optimizer_update_kernel<T, OPT_MOMENTUM_SGD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_NESTEROV: optimizer_update_kernel<T, OPT_NESTEROV><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_ADAGRAD: optimizer_update_kernel<T, OPT_ADAGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_RMSPROP: optimizer_update_kernel<T, OPT_RMSPROP><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_ADADELTA: optimizer_update_kernel<T, OPT_ADADELTA><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_ADAM: optimizer_update_kernel<T, OPT_ADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_ADAMAX: optimizer_update_kernel<T, OPT_ADAMAX><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	case OPT_NADAM: optimizer_update_kernel<T, OPT_NADAM><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
-	default: optimizer_update_kernel<T, OPT_AMSGRAD><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad); break;
+	return k;
+}
+
+#define CATTLE_HIP_OPT_DISPATCH(rule, LAUNCH) \
+	switch (rule) { \
+	case OPT_VANILLA_SGD: LAUNCH(OPT_VANILLA_SGD); break; \
+	case OPT_MOMENTUM_SGD: LAUNCH(OPT_MOMENTUM_SGD); break; \
+	case OPT_NESTEROV: LAUNCH(OPT_NESTEROV); break; \
+	case OPT_ADAGRAD: LAUNCH(OPT_ADAGRAD); break; \
+	case OPT_RMSPROP: LAUNCH(OPT_RMSPROP); break; \
+	case OPT_ADADELTA: LAUNCH(OPT_ADADELTA); break; \
+	case OPT_ADAM: LAUNCH(OPT_ADAM); break; \
+	case OPT_ADAMAX: LAUNCH(OPT_ADAMAX); break; \
+	case OPT_NADAM: LAUNCH(OPT_NADAM); break; \
+	default: LAUNCH(OPT_AMSGRAD); break; \
 	}
+
+template<typename T>
+void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n, T* grad, T* s0, T* s1,
+		T* s2, T* values, bool reset_grad) {
+	if (n == 0)
+		return;
+	const OptCoef<T> k = optimizer_coefficients<T>(rule, hyper, epoch, timestep);
+	const unsigned grid = flat_grid(n);
+#define CATTLE_HIP_LAUNCH_ONE(R) optimizer_update_kernel<T, R><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad)
+	CATTLE_HIP_OPT_DISPATCH(rule, CATTLE_HIP_LAUNCH_ONE)
+#undef CATTLE_HIP_LAUNCH_ONE
+	check_launch();
+}
+
+template<typename T>
+void optimizer_step_many(int rule, const double hyper[4], size_t epoch, size_t timestep, const OptBatch<T>& batch) {
+	if (batch.count == 0)
+		return;
+	CATTLE_HIP_REQUIRE(batch.count <= OPT_BATCH, "too many parameters in one optimizer launch");
+	const OptCoef<T> k = optimizer_coefficients<T>(rule, hyper, epoch, timestep);
+	size_t blocks = 1;        /* of the parameter that needs the most: runs of 1024 elements or 32 x 32 tiles */
+	for (int i = 0; i < batch.count; ++i) {
+		const OptParam<T>& q = batch.p[i];
+		if (q.wt_fwd || q.wt_dgrad)
+			blocks = std::max(blocks, (size_t) ((q.K + 31) / 32) * ((q.n / (size_t) q.K + 31) / 32));
+		else
+			blocks = std::max(blocks, (q.n + 1023) / 1024);
+	}
+	CATTLE_HIP_REQUIRE(blocks <= 2147483647u, "parameter too large for one optimizer launch");
+	const dim3 grid((unsigned) blocks, (unsigned) batch.count);
+#define CATTLE_HIP_LAUNCH_MANY(R) optimizer_step_many_kernel<T, R><<<grid, 256, 0, stream()>>>(batch, k)
+	CATTLE_HIP_OPT_DISPATCH(rule, CATTLE_HIP_LAUNCH_MANY)
+#undef CATTLE_HIP_LAUNCH_MANY
 	check_launch();
 }
 
 #define CATTLE_HIP_INSTANTIATE_TRAIN(T) \
 template void loss_function<T>(int, int, int, int, T, const T*, const T*, T*); \
 template void loss_d_function<T>(int, int, int, int, T, T, const T*, const T*, T*); \
-template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, T*, T*, T*, T*, T*, bool);
+template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, T*, T*, T*, T*, T*, bool); \
+template void optimizer_step_many<T>(int, const double*, size_t, size_t, const OptBatch<T>&);
 
 CATTLE_HIP_INSTANTIATE_TRAIN(float)
 CATTLE_HIP_INSTANTIATE_TRAIN(double)

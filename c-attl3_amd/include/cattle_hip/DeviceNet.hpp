@@ -279,6 +279,13 @@ public:
 			check(cattle_hip_layer_param_optimizer_step(handle, i, optimizer, hyper, epoch, timestep));
 		});
 	}
+	/** Appends (handle, index) of every optimizable parameter of this layer. */
+	inline void append_optimizable(std::vector<cattle_hip_layer_t>& handles, std::vector<std::size_t>& indices) {
+		for_each_optimizable([&](std::size_t i) {
+			handles.push_back(handle);
+			indices.push_back(i);
+		});
+	}
 	/** AdamOptimizer::_fit. */
 	inline void reset_optimizer_state() {
 		const std::size_t n = num_params();
@@ -512,8 +519,7 @@ public:
 			const DeviceLoss<Scalar>& loss, Scalar learning_rate) {
 		const Scalar total = forward_backward(input, obj, loss);
 		const double hyper[4] = { (double) learning_rate, 0, 0, 0 };
-		for (std::size_t i = 0; i < layers.size(); ++i)
-			layers[i].optimizer_step(CATTLE_HIP_OPT_VANILLA_SGD, hyper, 0, 0);
+		optimizer_step(CATTLE_HIP_OPT_VANILLA_SGD, hyper, 0, 0);
 		return total;
 	}
 	inline Scalar train_batch_adam(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,
@@ -521,9 +527,20 @@ public:
 			Scalar l2_decay = 1e-3, Scalar epsilon = 1e-5) {
 		const Scalar total = forward_backward(input, obj, loss);
 		const double hyper[4] = { (double) learning_rate, (double) l1_decay, (double) l2_decay, (double) epsilon };
-		for (std::size_t i = 0; i < layers.size(); ++i)
-			layers[i].optimizer_step(CATTLE_HIP_OPT_ADAM, hyper, 0, timestep);
+		optimizer_step(CATTLE_HIP_OPT_ADAM, hyper, 0, timestep);
 		return total;
+	}
+	/**
+	 * The update of every optimizable parameter of the network followed by its reset_grad
+	 * (optimizer/SGDOptimizer.hpp:64, :68-70), sixteen parameters per launch.
+	 */
+	inline void optimizer_step(cattle_hip_optimizer optimizer, const double (&hyper)[4], std::size_t epoch, std::size_t timestep) {
+		std::vector<cattle_hip_layer_t> handles;
+		std::vector<std::size_t> indices;
+		for (std::size_t i = 0; i < layers.size(); ++i)
+			layers[i].append_optimizable(handles, indices);
+		if (!handles.empty())
+			check(cattle_hip_optimizer_step_many(handles.data(), indices.data(), handles.size(), optimizer, hyper, epoch, timestep));
 	}
 private:
 	inline Scalar forward_backward(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,

@@ -244,6 +244,13 @@ int cattle_hip_layer_param_optimizer_update(cattle_hip_layer_t layer, size_t ind
 int cattle_hip_layer_param_optimizer_step(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
 		const double hyper[4], size_t epoch, size_t timestep);
 
+/* The loop of SGDOptimizer::_train over the parameters of a network (optimizer/SGDOptimizer.hpp:64, :68-70) as one
+ * launch per sixteen parameters: entry i names parameter indices[i] of layers[i]; each is updated as by
+ * cattle_hip_layer_param_optimizer_step. A Parameters object shared by several listed layers is updated once (the
+ * reference's get_all_unique_params, core/NeuralNetwork.hpp). All listed layers must have one scalar type. */
+int cattle_hip_optimizer_step_many(const cattle_hip_layer_t* layers, const size_t* indices, size_t count,
+		cattle_hip_optimizer optimizer, const double hyper[4], size_t epoch, size_t timestep);
+
 /* VanillaSGDOptimizer::_update_params for one Parameters object (optimizer/VanillaSGDOptimizer.hpp:38-43):
  * values -= grad * learning_rate, in place on the device. Non-optimizable parameters are rejected. */
 int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, double learning_rate);

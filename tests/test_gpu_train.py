@@ -292,6 +292,61 @@ def test_optimizer_step_is_update_then_reset(rule, hyper, dtype):
         assert not np.any(pc.get_grad())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rule,hyper", [ALL_OPTIMIZERS[0], ALL_OPTIMIZERS[1], ALL_OPTIMIZERS[6]])
+def test_optimizer_step_of_a_whole_network(rule, hyper, dtype):
+    """ParameterList.optimizer_step (every parameter of a network in one launch per sixteen, prepared weight
+    layouts rewritten by the same kernel) against optimizer_step parameter by parameter on a twin network: the same
+    values bit for bit after each of three batches, zero gradients, and the next passes (which use the prepared
+    layouts) agree as well. conv - ReLU - conv (shared with a clone) - dense layers."""
+    def build():
+        c1 = ch.ConvKernelLayer(dtype, (8, 8, 3), 6)
+        c2 = ch.ConvKernelLayer(dtype, (8, 8, 6), 6, 3, 3, 2, 2, 1, 1, 1, 1)          # dilated, same size out
+        layers = [c1, ch.ReLUActivationLayer(dtype, (8, 8, 6)), c2, c2.clone_with_shared_params(),
+                  ch.DenseKernelLayer(dtype, (8, 8, 6), 5)]
+        layers += [ch.DenseKernelLayer(dtype, (5, 1, 1), 5) for _ in range(7)]        # more than sixteen parameters
+        g = hp.rng(1230)
+        for l in layers:
+            for p in l.get_params():
+                if p.get_rows() > 1:
+                    p.set_values(hp.normal(g, (p.get_rows(), p.get_cols()), dtype, 0.3))
+        return layers
+
+    def passes(layers, x, go):
+        a = x
+        for l in layers:
+            a = l.pass_forward(a, True)
+        g = go
+        for l in reversed(layers):
+            g = l.pass_back(g)
+        return a, g
+
+    one, many = build(), build()
+    plist = ch.ParameterList([p for l in many for p in l.get_params()])
+    assert len(plist) == 22                       # 20 distinct Parameters objects, two of them listed twice
+    g = hp.rng(1231)
+    for t in range(3):
+        x = hp.normal(g, (8, 8, 8, 3), dtype)
+        go = hp.normal(g, (8, 5, 1, 1), dtype)
+        out_a, dx_a = passes(one, x, go)
+        out_b, dx_b = passes(many, x, go)
+        assert np.array_equal(out_a, out_b) and np.array_equal(dx_a, dx_b), t
+        seen = set()
+        for l in one:
+            for p in l.get_params():
+                assert np.any(p.get_grad())
+        for i, l in enumerate(one):
+            if i == 3:
+                continue                      # the clone shares layer 2's parameters: update them once
+            for p in l.get_params():
+                p.optimizer_step(rule, hyper, epoch=1, timestep=t)
+        plist.optimizer_step(rule, hyper, epoch=1, timestep=t)
+        for la, lb in zip(one, many):
+            for pa, pb in zip(la.get_params(), lb.get_params()):
+                assert np.array_equal(pa.get_values(), pb.get_values()), (rule, t)
+                assert not np.any(pb.get_grad())
+
+
 def test_optimizer_argument_checks():
     layer, g, w, b = _dense_with_grads(np.float32, 1221)
     prm = layer.get_params()[0]
