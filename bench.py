@@ -310,8 +310,16 @@ def train_steps_run(args, dtype):
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
         rows.append({"workload": name, "ms_per_step": round(ms, 4), "samples_per_s": round(N / (ms * 1e-3), 1),
                      "gflops": round(flop / (ms * 1e-3) / 1e9, 1)})
-    return {"metric": "device_resident_training_step", "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "dtype": args.dtype, "data": "synthetic", "driver": "python (ctypes), one C-ABI call per layer pass, one for the optimizer step", "steps_timed": rows}
+    line = {"metric": "device_resident_training_step", "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "dtype": args.dtype, "data": "synthetic",
+            "driver": "python (ctypes), one C-ABI call per layer pass, one for the optimizer step", "steps_timed": rows}
+    # the same two steps driven from C++ through DeviceNet.hpp (fp32; each batch reads its loss back, as SGDOptimizer::_train does)
+    exe = os.path.join(ROOT, "c-attl3_amd", "examples", "train_steps")
+    if os.path.exists(exe) and args.dtype == "f32":
+        import subprocess
+        out = subprocess.run([exe, str(max(args.steps, 20)), str(args.warmup)], stdout=subprocess.PIPE, check=True).stdout
+        line["cpp_driver"] = json.loads(out.decode().strip().splitlines()[-1])
+    return line
 
 
 def cpu_baseline(args, dtype):

@@ -1,0 +1,130 @@
+/*
+ * train_steps.cpp — whole training steps on the device from C++, through cattle_hip/DeviceNet.hpp: the two
+ * feed-forward configurations of the benchmark definition, built layer by layer as a C-ATTL3 user would build
+ * them, trained with DeviceFeedforwardNetwork::train_batch_sgd / train_batch_adam (one batch of
+ * SGDOptimizer::_train, optimizer/SGDOptimizer.hpp:44-70: propagate, loss, gradient / batch size, backpropagate,
+ * update, reset), and timed. Prints one JSON line.
+ *
+ *   g++ -std=c++11 -O2 -I include -I c-attl3_amd/include c-attl3_amd/examples/train_steps.cpp \
+ *       -L c-attl3_amd -lcattle_hip -Wl,-rpath,'$ORIGIN/..' -o c-attl3_amd/examples/train_steps
+ *   c-attl3_amd/examples/train_steps [steps] [warmup]
+ */
+#include <chrono>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+#include <vector>
+
+#include "cattle_hip/DeviceNet.hpp"
+
+using namespace cattle::hip::device;
+
+typedef float Scalar;
+typedef DeviceTensor<Scalar> DT;
+typedef DeviceLayer<Scalar> DL;
+typedef DL::Dims Dims;
+
+struct Lcg {
+	std::uint64_t s;
+	explicit Lcg(std::uint64_t seed) : s(seed * 2862933555777941757ULL + 3037000493ULL) { }
+	double next() {                 /* uniform in [-1, 1) */
+		s = s * 6364136223846793005ULL + 1442695040888963407ULL;
+		return (double) (s >> 11) / 9007199254740992.0 * 2.0 - 1.0;
+	}
+};
+
+static std::vector<Scalar> random_values(std::size_t count, Lcg& g, double scale) {
+	std::vector<Scalar> v(count);
+	for (std::size_t i = 0; i < count; ++i)
+		v[i] = (Scalar) (g.next() * scale);
+	return v;
+}
+
+/* weight matrices uniform with the variance of He initialisation (2 / fan_in); biases, gamma, beta keep their initial values */
+static void init_weights(DeviceFeedforwardNetwork<Scalar>& net, Lcg& g) {
+	std::vector<DL>& layers = net.get_layers();
+	for (std::size_t l = 0; l < layers.size(); ++l)
+		for (std::size_t p = 0; p < layers[l].num_params(); ++p) {
+			std::size_t rows, cols;
+			bool optimizable;
+			layers[l].param_shape(p, rows, cols, optimizable);
+			if (optimizable && rows > 1) {
+				std::vector<Scalar> w = random_values(rows * cols, g, std::sqrt(6.0 / (double) rows));
+				layers[l].set_param_values(p, w.data());
+			}
+		}
+}
+
+static std::vector<Scalar> one_hot(std::size_t batch, std::size_t classes, Lcg& g) {
+	std::vector<Scalar> y(batch * classes, (Scalar) 0);
+	for (std::size_t n = 0; n < batch; ++n) {
+		std::size_t c = (std::size_t) ((g.next() + 1.0) / 2.0 * (double) classes);
+		y[n + batch * (c < classes ? c : classes - 1)] = 1;
+	}
+	return y;
+}
+
+template<typename Step>
+static double time_steps(std::size_t steps, std::size_t warmup, Step step) {
+	for (std::size_t t = 0; t < warmup; ++t)
+		step(t);
+	check(cattle_hip_synchronize());
+	const std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+	for (std::size_t t = 0; t < steps; ++t)
+		step(warmup + t);
+	check(cattle_hip_synchronize());
+	return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / (double) steps;
+}
+
+int main(int argc, char** argv) {
+	const std::size_t steps = argc > 1 ? (std::size_t) std::atol(argv[1]) : 50;
+	const std::size_t warmup = argc > 2 ? (std::size_t) std::atol(argv[2]) : 5;
+	try {
+		check(cattle_hip_init(0));
+		DeviceLoss<Scalar> loss(CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY);
+		Lcg g(2);
+		double mlp_ms, conv_ms;
+		{
+			/* MLP 784-512-256-10 with ReLU, batch 256, vanilla SGD */
+			const std::size_t batch = 256;
+			std::vector<DL> layers;
+			layers.push_back(DL::dense(Dims{ { 784, 1, 1 } }, 512));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+			layers.push_back(DL::dense(layers.back().get_output_dims(), 256));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+			layers.push_back(DL::dense(layers.back().get_output_dims(), 10));
+			DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
+			init_weights(net, g);
+			std::vector<Scalar> x = random_values(batch * 784, g, 1.0), y = one_hot(batch, 10, g);
+			DT xd(DT::Dims{ { batch, 784, 1, 1 } }, x.data()), yd(DT::Dims{ { batch, 10, 1, 1 } }, y.data());
+			mlp_ms = time_steps(steps, warmup, [&](std::size_t) { net.train_batch_sgd(xd, yd, loss, (Scalar) 1e-3); });
+		}
+		{
+			/* conv 3x3x32 - ReLU - max pool - conv 3x3x64 - batch norm - ReLU - max pool - dense 10, batch 128, Adam */
+			const std::size_t batch = 128;
+			std::vector<DL> layers;
+			layers.push_back(DL::conv(Dims{ { 32, 32, 3 } }, 32));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+			layers.push_back(DL::pool(CATTLE_HIP_POOL_MAX, layers.back().get_output_dims()));
+			layers.push_back(DL::conv(layers.back().get_output_dims(), 64));
+			layers.push_back(DL::batch_norm(layers.back().get_output_dims()));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+			layers.push_back(DL::pool(CATTLE_HIP_POOL_MAX, layers.back().get_output_dims()));
+			layers.push_back(DL::dense(layers.back().get_output_dims(), 10));
+			DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
+			init_weights(net, g);
+			std::vector<Scalar> x = random_values(batch * 32 * 32 * 3, g, 1.0), y = one_hot(batch, 10, g);
+			DT xd(DT::Dims{ { batch, 32, 32, 3 } }, x.data()), yd(DT::Dims{ { batch, 10, 1, 1 } }, y.data());
+			conv_ms = time_steps(steps, warmup, [&](std::size_t t) { net.train_batch_adam(xd, yd, loss, t); });
+		}
+		std::printf("{\"driver\": \"C++ (cattle_hip/DeviceNet.hpp), train_batch_sgd / train_batch_adam incl. the per-batch loss read-back\", "
+				"\"steps\": %zu, \"warmup\": %zu, \"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, \"convnet_32x32x3_batch128_adam_ms\": %.4f}\n",
+				steps, warmup, mlp_ms, conv_ms);
+	} catch (const std::exception& e) {
+		std::fprintf(stderr, "train_steps: %s\n", e.what());
+		return 1;
+	}
+	return 0;
+}
