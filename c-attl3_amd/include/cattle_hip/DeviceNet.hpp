@@ -615,6 +615,52 @@ public:
 		check(cattle_hip_layer_param_shape(handle, ((std::size_t) kernel % 2) * 2, &rows, &cols, &opt));
 		return bias ? hidden : rows * hidden;
 	}
+	/**
+	 * NeuralNetwork::save_all_unique_params_values / load_all_unique_params_values (core/NeuralNetwork.hpp:195-223) for
+	 * the LSTM: the parameter matrices in get_layers() order (:521-534), i.e. weights then bias of the eight kernels
+	 * (the five activations have none), each in the binary format of core/EigenProxy.hpp:147-159, :212-224.
+	 */
+	inline void save_all_unique_params_values(const std::string& dir_path,
+			const std::string& file_name_prefix = "c-attl3_neural_net_params_") const {
+		for (std::size_t i = 0; i < 16; ++i) {
+			const Kernel kernel = (Kernel) (i / 2);
+			const bool bias = i % 2 == 1;
+			const std::vector<Scalar> values = get_kernel_values(kernel, bias);
+			std::ofstream out(dir_path + "/" + file_name_prefix + std::to_string(i) + ".prms", std::ios::binary);
+			if (!out.is_open())
+				throw std::runtime_error("cannot write a parameter file under " + dir_path);
+			const unsigned short scalar_size = (unsigned short) sizeof(Scalar);
+			const unsigned rows = bias ? 1u : (unsigned) (values.size() / hidden), cols = (unsigned) hidden;
+			out.write(reinterpret_cast<const char*>(&scalar_size), sizeof(scalar_size));
+			out.write(reinterpret_cast<const char*>(&rows), sizeof(rows));
+			out.write(reinterpret_cast<const char*>(&cols), sizeof(cols));
+			out.write(reinterpret_cast<const char*>(values.data()), (std::streamsize) (values.size() * sizeof(Scalar)));
+		}
+	}
+	inline void load_all_unique_params_values(const std::string& dir_path,
+			const std::string& file_name_prefix = "c-attl3_neural_net_params_") {
+		for (std::size_t i = 0; i < 16; ++i) {
+			const Kernel kernel = (Kernel) (i / 2);
+			const bool bias = i % 2 == 1;
+			std::ifstream in(dir_path + "/" + file_name_prefix + std::to_string(i) + ".prms", std::ios::binary);
+			if (!in.is_open())
+				throw std::runtime_error("missing parameter file " + std::to_string(i) + " under " + dir_path);
+			unsigned short scalar_size = 0;
+			unsigned rows = 0, cols = 0;
+			in.read(reinterpret_cast<char*>(&scalar_size), sizeof(scalar_size));
+			in.read(reinterpret_cast<char*>(&rows), sizeof(rows));
+			in.read(reinterpret_cast<char*>(&cols), sizeof(cols));
+			if (!in || scalar_size != sizeof(Scalar))          /* assert(scalar_size == sizeof(Scalar)) */
+				throw std::runtime_error("parameter file of another scalar type or truncated");
+			if ((std::size_t) rows * cols != kernel_size(kernel, bias) || cols != hidden)
+				throw std::runtime_error("parameter file " + std::to_string(i) + " does not have the kernel's dimensions");
+			std::vector<Scalar> values((std::size_t) rows * cols);
+			in.read(reinterpret_cast<char*>(values.data()), (std::streamsize) (values.size() * sizeof(Scalar)));
+			if (!in)
+				throw std::runtime_error("truncated parameter file");
+			set_kernel_values(kernel, bias, values.data());
+		}
+	}
 	/** propagate (:236-403): `input` must stay alive and unmodified until backpropagate returns. */
 	inline Sequence propagate(const Sequence& input, bool training) {
 		const std::pair<std::size_t,std::size_t> out_seq = seq(input.dims[1]);

@@ -203,6 +203,14 @@ static void run_lstm(const std::string& tag) {
 		record(tag + ".lstm.dw" + std::to_string(k), sizeof(Scalar), { rows, hid }, net.get_kernel_grad(kernel, false).data());
 		record(tag + ".lstm.db" + std::to_string(k), sizeof(Scalar), { 1, hid }, net.get_kernel_grad(kernel, true).data());
 	}
+	/* the parameter files of the network as it stands, loaded by a fresh one, give the same output */
+	net.save_all_unique_params_values(g_dir, tag + "_lstm_params_");
+	{
+		Net fresh(typename Net::Dims{ { H, W, C } }, hid, &last_two_steps, false);
+		fresh.load_all_unique_params_values(g_dir, tag + "_lstm_params_");
+		typename Net::Sequence again = fresh.propagate(in, true);
+		record(tag + ".lstm.out_reloaded", sizeof(Scalar), { batch, 2, H, W, hid }, again.data.to_host().data());
+	}
 	net.sgd_update((Scalar) 0.05);
 	net.reset_grads();
 	record(tag + ".lstm.w3_updated", sizeof(Scalar), { net.kernel_size(Net::OUTPUT_WRITE, false) / hid, hid },

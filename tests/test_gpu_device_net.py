@@ -146,3 +146,24 @@ def test_parameter_files_have_the_reference_format(records, tag, dtype):
             assert mats[2 + 4 * c + k][0, 0] == r["final.3.%d" % k][0, c]
     assert np.array_equal(mats[34], r["final.4.0"]) and np.array_equal(mats[35], r["final.4.1"])
     assert np.array_equal(r["reloaded_infer"], r["infer"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,dtype", [("f32", np.float32), ("f64", np.float64)])
+def test_lstm_parameter_files_follow_the_layer_order(records, tag, dtype):
+    """DeviceConvLSTM::save_all_unique_params_values: sixteen files in the order of LSTMNeuralNetwork::get_layers()
+    (neural_network/LSTMNeuralNetwork.hpp:521-529: input and output kernel of the forget, write, candidate and read
+    gates, weights before bias), each in the binary format of core/EigenProxy.hpp:147-159; a fresh network that
+    loads them gives the same output bit for bit."""
+    import struct
+    r = {k[len(tag) + 6:]: v for k, v in records.items() if k.startswith(tag + ".lstm.")}
+    for i in range(16):
+        raw = open(os.path.join(records["__dir__"], "%s_lstm_params_%d.prms" % (tag, i)), "rb").read()
+        size, rows, cols = struct.unpack("<HII", raw[:10])
+        assert size == np.dtype(dtype).itemsize and len(raw) == 10 + size * rows * cols
+        m = np.frombuffer(raw[10:], dtype=dtype).reshape((rows, cols), order="F")
+        want = r["%s%d" % ("b" if i % 2 else "w", i // 2)]
+        assert m.shape == want.shape and np.array_equal(m, want), i
+    assert not os.path.exists(os.path.join(records["__dir__"], "%s_lstm_params_16.prms" % tag))
+    assert np.array_equal(r["out_reloaded"], r["out"])
+
