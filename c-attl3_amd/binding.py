@@ -223,7 +223,10 @@ class Parameters(object):
         _check(lib().cattle_hip_layer_param_reset_optimizer_state(self._layer._h, _sz(self._index)))
 
 
-LOSS = {"squared": 0, "softmax_cross_entropy": 1}
+LOSS = {"squared": 0, "softmax_cross_entropy": 1, "absolute": 2, "binary_cross_entropy": 3, "cross_entropy": 4,
+        "kullback_leibler": 5, "hinge": 6, "squared_hinge": 7, "multi_label_hinge": 8, "squared_multi_label_hinge": 9,
+        "multi_label_log": 10}
+LOSS_NEGATED = 0x100        # OR-ed into a kind: the loss wrapped in NegatedLoss (loss/NegatedLoss.hpp:41-46)
 _HYPER_ARRAYS = {}
 
 
@@ -272,18 +275,23 @@ def _loss_args(out, obj, sequential):
     return out, obj, batch, steps, size, (DEVICE if dev else HOST), ptr
 
 
-def loss_function(kind, out, obj, epsilon=1e-5, sequential=False):
+def _loss_kind(kind, negated):
+    return ctypes.c_int(LOSS[kind] | (LOSS_NEGATED if negated else 0))
+
+
+def loss_function(kind, out, obj, epsilon=1e-5, sequential=False, negated=False):
     """Loss::function: the per-sample losses of a batch as a numpy vector (loss/UniversalLoss.hpp:37-41, :99-110).
-    out/obj are numpy arrays or DeviceTensors of shape (N, ...) or, if sequential, (N, T, ...)."""
+    out/obj are numpy arrays or DeviceTensors of shape (N, ...) or, if sequential, (N, T, ...); `negated` is the
+    loss wrapped in NegatedLoss."""
     out, obj, batch, steps, size, space, ptr = _loss_args(out, obj, sequential)
     losses = np.empty((batch,), dtype=out.dtype)
-    _check(lib().cattle_hip_loss_function(_dtype_code(out.dtype), ctypes.c_int(LOSS[kind]), ptr(out), space, ptr(obj), space,
+    _check(lib().cattle_hip_loss_function(_dtype_code(out.dtype), _loss_kind(kind, negated), ptr(out), space, ptr(obj), space,
                                           _sz(batch), _sz(steps), _sz(size), ctypes.c_double(epsilon),
                                           ctypes.c_void_p(losses.ctypes.data), HOST))
     return losses
 
 
-def loss_d_function(kind, out, obj, epsilon=1e-5, scale=1.0, sequential=False):
+def loss_d_function(kind, out, obj, epsilon=1e-5, scale=1.0, sequential=False, negated=False):
     """Loss::d_function times scale (loss/UniversalLoss.hpp:42-46, :111-125); returns what it was given
     (numpy array or DeviceTensor) in the shape of out."""
     out, obj, batch, steps, size, space, ptr = _loss_args(out, obj, sequential)
@@ -291,7 +299,7 @@ def loss_d_function(kind, out, obj, epsilon=1e-5, scale=1.0, sequential=False):
         grad = DeviceTensor(out.shape, out.dtype)
     else:
         grad = np.empty(out.shape, dtype=out.dtype, order="F")
-    _check(lib().cattle_hip_loss_d_function(_dtype_code(out.dtype), ctypes.c_int(LOSS[kind]), ptr(out), space, ptr(obj), space,
+    _check(lib().cattle_hip_loss_d_function(_dtype_code(out.dtype), _loss_kind(kind, negated), ptr(out), space, ptr(obj), space,
                                             _sz(batch), _sz(steps), _sz(size), ctypes.c_double(epsilon),
                                             ctypes.c_double(scale), ptr(grad), space))
     return grad

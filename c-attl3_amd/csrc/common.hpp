@@ -147,7 +147,9 @@ template<typename T> void lstm_gates_backward(const LstmActs<T>& a, int N, size_
 
 /* Losses and optimizer updates (train_kernels.hip). A batch is N samples x T_steps x V elements,
  * column-major with the sample index fastest. */
-enum { LOSS_SQUARED = 0, LOSS_SOFTMAX_CROSS_ENTROPY = 1 };
+enum { LOSS_SQUARED = 0, LOSS_SOFTMAX_CROSS_ENTROPY = 1, LOSS_ABSOLUTE = 2, LOSS_BINARY_CROSS_ENTROPY = 3, LOSS_CROSS_ENTROPY = 4,
+	LOSS_KULLBACK_LEIBLER = 5, LOSS_HINGE = 6, LOSS_SQUARED_HINGE = 7, LOSS_MULTI_LABEL_HINGE = 8,
+	LOSS_SQUARED_MULTI_LABEL_HINGE = 9, LOSS_MULTI_LABEL_LOG = 10, LOSS_KINDS = 11, LOSS_NEGATED = 0x100 };
 template<typename T> void loss_function(int kind, int N, int T_steps, int V, T eps, const T* out, const T* obj, T* losses);
 template<typename T> void loss_d_function(int kind, int N, int T_steps, int V, T eps, T scale, const T* out, const T* obj,
 		T* grad);

@@ -769,7 +769,9 @@ void loss_entry(bool grad_pass, int dtype, int kind, const void* out, int out_sp
 	check_space(out_space);
 	check_space(obj_space);
 	check_space(dst_space);
-	CATTLE_HIP_REQUIRE(kind == CATTLE_HIP_LOSS_SQUARED || kind == CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY, "unknown loss kind");
+	CATTLE_HIP_REQUIRE((kind & ~CATTLE_HIP_LOSS_NEGATED) >= 0 && (kind & ~CATTLE_HIP_LOSS_NEGATED) < LOSS_KINDS, "unknown loss kind");
+	CATTLE_HIP_REQUIRE((kind & ~CATTLE_HIP_LOSS_NEGATED) != CATTLE_HIP_LOSS_BINARY_CROSS_ENTROPY || sample_size == 1,
+			"the binary cross entropy loss takes one value per sample and time step");
 	CATTLE_HIP_REQUIRE(out != nullptr && obj != nullptr && dst != nullptr, "null tensor buffer");
 	CATTLE_HIP_REQUIRE(batch > 0 && time_steps > 0 && sample_size > 0, "batch, time steps and sample size must be positive");
 	if (dtype == CATTLE_HIP_F32)

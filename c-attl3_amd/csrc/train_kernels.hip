@@ -42,10 +42,95 @@ __device__ __forceinline__ T row_combine(T v, T* lds) {
 	return acc;
 }
 
-/* Squared error (loss/SquaredLoss.hpp:25-34): L_n = sum_j (out - obj)^2. */
+template<typename T> struct MachineEps;
+template<> struct MachineEps<float> { static constexpr float value = 1.1920928955078125e-07f; };
+template<> struct MachineEps<double> { static constexpr double value = 2.220446049250313e-16; };
+
+__device__ __forceinline__ float dev_abs(float v) { return fabsf(v); }
+__device__ __forceinline__ double dev_abs(double v) { return fabs(v); }
+
+/* NumericUtils::almost_equal with its default epsilons (core/NumericUtils.hpp:42-49) */
 template<typename T>
+__device__ __forceinline__ bool almost_equal(T a, T b) {
+	const T e = MachineEps<T>::value;
+	const T diff = dev_abs(a - b);
+	if (diff <= e)
+		return true;
+	const T aa = dev_abs(a), ab = dev_abs(b);
+	return diff <= (aa > ab ? aa : ab) * e;
+}
+
+/* NumericUtils::decidedly_greater (core/NumericUtils.hpp:62-65) */
+template<typename T>
+__device__ __forceinline__ bool decidedly_greater(T a, T b) {
+	return a > b && !almost_equal(a, b);
+}
+
+/* The losses that are a plain sum over the elements of a sample: the summand of _function ...
+ *   LOSS_SQUARED                    loss/SquaredLoss.hpp:25-29             (o - y)^2
+ *   LOSS_ABSOLUTE                   loss/AbsoluteLoss.hpp:25-30            |o - y|
+ *   LOSS_BINARY_CROSS_ENTROPY       loss/BinaryCrossEntropyLoss.hpp:35-40  -(y ln(o + e) + (1 - y) ln((1 + e) - o))
+ *   LOSS_CROSS_ENTROPY              loss/CrossEntropyLoss.hpp:33-38        -ln(o + e) y
+ *   LOSS_KULLBACK_LEIBLER           loss/KullbackLeiblerLoss.hpp:32-39     -ln(o / (y + e) + e) y
+ *   LOSS_MULTI_LABEL_HINGE          loss/MultiLabelHingeLoss.hpp:31-49     max(0, 1 - y o), squared in the SQUARED kind
+ *   LOSS_MULTI_LABEL_LOG            loss/MultiLabelLogLoss.hpp:37-55       y ln(o + e) + (1 - y) ln(1 + e - o)
+ * (the cross entropies are negated after the sum in the reference; negating each summand gives the same value) */
+template<typename T, int KIND>
+__device__ __forceinline__ T loss_summand(T o, T y, T eps) {
+	const T one = (T) 1;
+	if (KIND == LOSS_SQUARED) {
+		const T d = o - y;
+		return d * d;
+	} else if (KIND == LOSS_ABSOLUTE) {
+		return dev_abs(o - y);
+	} else if (KIND == LOSS_BINARY_CROSS_ENTROPY) {
+		return -(y * dev_log(o + eps) + (one - y) * dev_log((one + eps) - o));
+	} else if (KIND == LOSS_CROSS_ENTROPY) {
+		return -(dev_log(o + eps) * y);
+	} else if (KIND == LOSS_KULLBACK_LEIBLER) {
+		return -(dev_log(o / (y + eps) + eps) * y);
+	} else if (KIND == LOSS_MULTI_LABEL_HINGE || KIND == LOSS_SQUARED_MULTI_LABEL_HINGE) {
+		const T m = one - y * o;
+		const T l = m > (T) 0 ? m : (T) 0;
+		return KIND == LOSS_SQUARED_MULTI_LABEL_HINGE ? l * l : l;
+	} else {
+		return y * dev_log(o + eps) + (one - y) * dev_log(one + eps - o);
+	}
+}
+
+/* ... and the element of _d_function:
+ *   squared 2 (o - y) (SquaredLoss.hpp:30-33); absolute +1 for o - y >= 0, else -1 (AbsoluteLoss.hpp:31-35);
+ *   binary cross entropy -(y / (o + e) - (1 - y) / ((1 + e) - o)) (BinaryCrossEntropyLoss.hpp:41-46);
+ *   cross entropy and Kullback-Leibler -y / (o + e) (CrossEntropyLoss.hpp:39-42, KullbackLeiblerLoss.hpp:40-43);
+ *   multi-label hinge -y, squared 2 o - 2 y, where 1 - y o is decidedly greater than 0, else 0
+ *   (MultiLabelHingeLoss.hpp:50-71); multi-label log (y - o') / (o (1 - o)) with o' = o, or e where o is exactly 0
+ *   (MultiLabelLogLoss.hpp:56-76). */
+template<typename T, int KIND>
+__device__ __forceinline__ T loss_derivative(T o, T y, T eps) {
+	const T one = (T) 1;
+	if (KIND == LOSS_SQUARED) {
+		return (T) 2 * (o - y);
+	} else if (KIND == LOSS_ABSOLUTE) {
+		return o - y >= (T) 0 ? one : -one;
+	} else if (KIND == LOSS_BINARY_CROSS_ENTROPY) {
+		return -(y / (o + eps) - (one - y) / ((one + eps) - o));
+	} else if (KIND == LOSS_CROSS_ENTROPY || KIND == LOSS_KULLBACK_LEIBLER) {
+		return -y / (o + eps);
+	} else if (KIND == LOSS_MULTI_LABEL_HINGE || KIND == LOSS_SQUARED_MULTI_LABEL_HINGE) {
+		if (!decidedly_greater(one - y * o, (T) 0))
+			return (T) 0;
+		return KIND == LOSS_SQUARED_MULTI_LABEL_HINGE ? (T) 2 * o - (T) 2 * y : -y;
+	} else {
+		const T denominator = o * (one - o);
+		const T numerator_o = o == (T) 0 ? o + eps : o;
+		return (y - numerator_o) / denominator;
+	}
+}
+
+/* L_n = sign * sum over the time steps and the elements of loss_summand. */
+template<typename T, int KIND>
 __global__ __launch_bounds__(ROWS * PARTS)
-void squared_loss_kernel(int N, int T_steps, int V, const T* __restrict__ out, const T* __restrict__ obj,
+void summed_loss_kernel(int N, int T_steps, int V, T eps, T sign, const T* __restrict__ out, const T* __restrict__ obj,
 		T* __restrict__ losses) {
 	__shared__ T lds[ROWS * PARTS];
 	const int n = blockIdx.x * ROWS + threadIdx.x;
@@ -56,30 +141,82 @@ void squared_loss_kernel(int N, int T_steps, int V, const T* __restrict__ out, c
 		T s = (T) 0;
 		if (live) {
 			const size_t base = (size_t) n + (size_t) N * t;
-			for (int j = threadIdx.y; j < V; j += PARTS) {
-				const T d = out[base + cs * j] - obj[base + cs * j];
-				s += d * d;
-			}
+			for (int j = threadIdx.y; j < V; j += PARTS)
+				s += loss_summand<T, KIND>(out[base + cs * j], obj[base + cs * j], eps);
 		}
 		total += row_combine<T, false>(s, lds);
 	}
 	if (live && threadIdx.y == 0)
-		losses[n] = total;
+		losses[n] = sign * total;
 }
 
-/* grad = scale * 2 (out - obj) */
-template<typename T>
+/* grad = scale * loss_derivative, element by element */
+template<typename T, int KIND>
 __global__ __launch_bounds__(256)
-void squared_loss_grad_kernel(size_t total, T two_scale, const T* __restrict__ out, const T* __restrict__ obj,
+void loss_derivative_kernel(size_t total, T eps, T scale, const T* __restrict__ out, const T* __restrict__ obj,
 		T* __restrict__ grad) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
 	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride)
-		grad[i] = two_scale * (out[i] - obj[i]);
+		grad[i] = scale * loss_derivative<T, KIND>(out[i], obj[i], eps);
+}
+
+/* Hinge loss over one-hot objectives (loss/HingeLoss.hpp:31-99). The class c of a row is its last element that
+ * almost equals 1; with s = out_c and m_j = out_j - s + 1 for j != c:
+ *   GRAD = false: L_n = sign * sum_j max(0, m_j)  (squared: max(0, m_j)^2), summed over the time steps
+ *   GRAD = true : grad_j = scale * g_j, g_j = 1 (squared: 2 m_j) where m_j is decidedly greater than 0, else 0,
+ *                 and grad_c = -scale * sum_j g_j.
+ * A row without a one (which the reference asserts against) gives NaN. */
+template<typename T, bool SQUARED, bool GRAD>
+__global__ __launch_bounds__(ROWS * PARTS)
+void hinge_loss_kernel(int N, int T_steps, int V, T scale, const T* __restrict__ out, const T* __restrict__ obj,
+		T* __restrict__ dst) {
+	__shared__ T lds[ROWS * PARTS];
+	const int n = blockIdx.x * ROWS + threadIdx.x;
+	const bool live = n < N;
+	const size_t cs = (size_t) N * T_steps;
+	T total = (T) 0;
+	for (int t = 0; t < T_steps; ++t) {
+		const size_t base = (size_t) (live ? n : 0) + (size_t) N * t;
+		T cls = (T) -1;
+		if (live)
+			for (int j = threadIdx.y; j < V; j += PARTS)
+				if (almost_equal(obj[base + cs * j], (T) 1))
+					cls = (T) j;
+		const int c = (int) row_combine<T, true>(cls, lds);
+		const T score = c >= 0 ? out[base + cs * c] : (T) NAN;
+		T s = (T) 0;
+		if (live)
+			for (int j = threadIdx.y; j < V; j += PARTS) {
+				if (j == c)
+					continue;
+				const T m = out[base + cs * j] - score + (T) 1;
+				if (GRAD) {
+					T g = (T) 0;
+					if (decidedly_greater(m, (T) 0))
+						g = SQUARED ? (T) 2 * m : (T) 1;
+					else if (c < 0)
+						g = (T) NAN;
+					s += g;
+					dst[base + cs * j] = scale * g;
+				} else {
+					const T l = m > (T) 0 ? m : (c < 0 ? (T) NAN : (T) 0);
+					s += SQUARED ? l * l : l;
+				}
+			}
+		s = row_combine<T, false>(s, lds);
+		if (GRAD) {
+			if (live && threadIdx.y == 0 && c >= 0)
+				dst[base + cs * c] = scale * -s;
+		} else
+			total += s;
+	}
+	if (!GRAD && live && threadIdx.y == 0)
+		dst[n] = scale * total;
 }
 
 /* Softmax cross entropy (loss/SoftmaxCrossEntropyLoss.hpp:33-50) with the reference's epsilon in
  * the softmax denominator: p_j = exp(o_j - max o) / (sum_i exp(o_i - max o) + eps).
- *   GRAD = false: L_n = - sum_j log(p_j) * obj_j   (summed over time steps)
+ *   GRAD = false: L_n = - scale * sum_j log(p_j) * obj_j   (summed over time steps; scale is +1 or -1)
  *   GRAD = true : grad_j = scale * (p_j - obj_j) */
 template<typename T, bool GRAD>
 __global__ __launch_bounds__(ROWS * PARTS)
@@ -121,7 +258,7 @@ void softmax_ce_kernel(int N, int T_steps, int V, T eps, T scale, const T* __res
 		}
 	}
 	if (!GRAD && live && threadIdx.y == 0)
-		dst[n] = total;
+		dst[n] = scale * total;
 }
 
 /* The _update_params bodies of the reference's optimizers, one element per thread, in place. The
@@ -263,22 +400,45 @@ void check_launch() {
 
 } /* namespace */
 
+/* kind | LOSS_NEGATED is the loss wrapped in NegatedLoss (loss/NegatedLoss.hpp:41-46): both results change sign. */
 template<typename T>
 void loss_function(int kind, int N, int T_steps, int V, T eps, const T* out, const T* obj, T* losses) {
 	if (N == 0)
 		return;
+	const T sign = (kind & LOSS_NEGATED) ? (T) -1 : (T) 1;
+	kind &= ~LOSS_NEGATED;
 	const dim3 block(ROWS, PARTS);
 	const unsigned grid = (unsigned) ((N + ROWS - 1) / ROWS);
+#define CATTLE_HIP_SUMMED_LOSS(KIND) \
+	case KIND: \
+		summed_loss_kernel<T, KIND><<<grid, block, 0, stream()>>>(N, T_steps, V, eps, sign, out, obj, losses); \
+		break;
 	switch (kind) {
-	case LOSS_SQUARED:
-		squared_loss_kernel<T><<<grid, block, 0, stream()>>>(N, T_steps, V, out, obj, losses);
+	CATTLE_HIP_SUMMED_LOSS(LOSS_SQUARED)
+	CATTLE_HIP_SUMMED_LOSS(LOSS_ABSOLUTE)
+	CATTLE_HIP_SUMMED_LOSS(LOSS_CROSS_ENTROPY)
+	CATTLE_HIP_SUMMED_LOSS(LOSS_KULLBACK_LEIBLER)
+	CATTLE_HIP_SUMMED_LOSS(LOSS_MULTI_LABEL_HINGE)
+	CATTLE_HIP_SUMMED_LOSS(LOSS_SQUARED_MULTI_LABEL_HINGE)
+	CATTLE_HIP_SUMMED_LOSS(LOSS_MULTI_LABEL_LOG)
+	case LOSS_BINARY_CROSS_ENTROPY:
+		if (V != 1)
+			throw Error(ERR_INVALID, "the binary cross entropy loss takes one value per sample and time step");
+		summed_loss_kernel<T, LOSS_BINARY_CROSS_ENTROPY><<<grid, block, 0, stream()>>>(N, T_steps, V, eps, sign, out, obj, losses);
 		break;
 	case LOSS_SOFTMAX_CROSS_ENTROPY:
-		softmax_ce_kernel<T, false><<<grid, block, 0, stream()>>>(N, T_steps, V, eps, (T) 1, out, obj, losses);
+		softmax_ce_kernel<T, false><<<grid, block, 0, stream()>>>(N, T_steps, V, eps, sign, out, obj, losses);
+		break;
+	case LOSS_HINGE:
+		hinge_loss_kernel<T, false, false><<<grid, block, 0, stream()>>>(N, T_steps, V, sign, out, obj, losses);
+		break;
+	case LOSS_SQUARED_HINGE:
+		hinge_loss_kernel<T, true, false><<<grid, block, 0, stream()>>>(N, T_steps, V, sign, out, obj, losses);
 		break;
 	default:
 		throw Error(ERR_INVALID, "unknown loss kind");
 	}
+#undef CATTLE_HIP_SUMMED_LOSS
 	check_launch();
 }
 
@@ -287,17 +447,41 @@ void loss_d_function(int kind, int N, int T_steps, int V, T eps, T scale, const 
 	const size_t total = (size_t) N * T_steps * V;
 	if (total == 0)
 		return;
+	if (kind & LOSS_NEGATED)
+		scale = -scale;
+	kind &= ~LOSS_NEGATED;
+	const dim3 block(ROWS, PARTS);
+	const unsigned rows_grid = (unsigned) ((N + ROWS - 1) / ROWS);
+#define CATTLE_HIP_LOSS_DERIVATIVE(KIND) \
+	case KIND: \
+		loss_derivative_kernel<T, KIND><<<flat_grid(total), 256, 0, stream()>>>(total, eps, scale, out, obj, grad); \
+		break;
 	switch (kind) {
-	case LOSS_SQUARED:
-		squared_loss_grad_kernel<T><<<flat_grid(total), 256, 0, stream()>>>(total, (T) 2 * scale, out, obj, grad);
+	CATTLE_HIP_LOSS_DERIVATIVE(LOSS_SQUARED)
+	CATTLE_HIP_LOSS_DERIVATIVE(LOSS_ABSOLUTE)
+	CATTLE_HIP_LOSS_DERIVATIVE(LOSS_CROSS_ENTROPY)
+	CATTLE_HIP_LOSS_DERIVATIVE(LOSS_KULLBACK_LEIBLER)
+	CATTLE_HIP_LOSS_DERIVATIVE(LOSS_MULTI_LABEL_HINGE)
+	CATTLE_HIP_LOSS_DERIVATIVE(LOSS_SQUARED_MULTI_LABEL_HINGE)
+	CATTLE_HIP_LOSS_DERIVATIVE(LOSS_MULTI_LABEL_LOG)
+	case LOSS_BINARY_CROSS_ENTROPY:
+		if (V != 1)
+			throw Error(ERR_INVALID, "the binary cross entropy loss takes one value per sample and time step");
+		loss_derivative_kernel<T, LOSS_BINARY_CROSS_ENTROPY><<<flat_grid(total), 256, 0, stream()>>>(total, eps, scale, out, obj, grad);
 		break;
 	case LOSS_SOFTMAX_CROSS_ENTROPY:
-		softmax_ce_kernel<T, true><<<(unsigned) ((N + ROWS - 1) / ROWS), dim3(ROWS, PARTS), 0, stream()>>>(
-				N, T_steps, V, eps, scale, out, obj, grad);
+		softmax_ce_kernel<T, true><<<rows_grid, block, 0, stream()>>>(N, T_steps, V, eps, scale, out, obj, grad);
+		break;
+	case LOSS_HINGE:
+		hinge_loss_kernel<T, false, true><<<rows_grid, block, 0, stream()>>>(N, T_steps, V, scale, out, obj, grad);
+		break;
+	case LOSS_SQUARED_HINGE:
+		hinge_loss_kernel<T, true, true><<<rows_grid, block, 0, stream()>>>(N, T_steps, V, scale, out, obj, grad);
 		break;
 	default:
 		throw Error(ERR_INVALID, "unknown loss kind");
 	}
+#undef CATTLE_HIP_LOSS_DERIVATIVE
 	check_launch();
 }
 

@@ -397,11 +397,15 @@ private:
 	bool params_per_column;
 };
 
-/** Loss::function / d_function on device tensors (loss/UniversalLoss.hpp:27-55, non-sequential data). */
+/**
+ * Loss::function / d_function on device tensors (loss/UniversalLoss.hpp:27-55, non-sequential data) for every
+ * loss of the loss/ directory; `negated` wraps it as NegatedLoss does (loss/NegatedLoss.hpp:41-46).
+ */
 template<typename Scalar>
 class DeviceLoss {
 public:
-	inline explicit DeviceLoss(cattle_hip_loss kind, Scalar epsilon = 1e-5) : kind(kind), epsilon(epsilon) { }
+	inline explicit DeviceLoss(cattle_hip_loss kind, Scalar epsilon = 1e-5, bool negated = false) :
+			kind((cattle_hip_loss) (negated ? kind | CATTLE_HIP_LOSS_NEGATED : kind)), epsilon(epsilon) { }
 	/** The per-sample losses, on the host (a column vector in the reference). */
 	inline std::vector<Scalar> function(const DeviceTensor<Scalar>& out, const DeviceTensor<Scalar>& obj) const {
 		assert(out.dimensions() == obj.dimensions());

@@ -197,14 +197,28 @@ int cattle_hip_maxpool_indices(cattle_hip_layer_t layer, unsigned* indices, catt
  * never leave HBM; only the per-sample losses come back if the caller asks for them. */
 
 typedef enum cattle_hip_loss {
-	CATTLE_HIP_LOSS_SQUARED = 0,                 /* loss/SquaredLoss.hpp:25-34 */
-	CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY = 1    /* loss/SoftmaxCrossEntropyLoss.hpp:33-50 */
+	CATTLE_HIP_LOSS_SQUARED = 0,                    /* loss/SquaredLoss.hpp:25-34 */
+	CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY = 1,      /* loss/SoftmaxCrossEntropyLoss.hpp:33-50 */
+	CATTLE_HIP_LOSS_ABSOLUTE = 2,                   /* loss/AbsoluteLoss.hpp:25-35 */
+	CATTLE_HIP_LOSS_BINARY_CROSS_ENTROPY = 3,       /* loss/BinaryCrossEntropyLoss.hpp:35-46; sample_size must be 1 */
+	CATTLE_HIP_LOSS_CROSS_ENTROPY = 4,              /* loss/CrossEntropyLoss.hpp:33-42 */
+	CATTLE_HIP_LOSS_KULLBACK_LEIBLER = 5,           /* loss/KullbackLeiblerLoss.hpp:32-43 */
+	CATTLE_HIP_LOSS_HINGE = 6,                      /* loss/HingeLoss.hpp:31-99, Squared = false */
+	CATTLE_HIP_LOSS_SQUARED_HINGE = 7,              /* loss/HingeLoss.hpp:31-99, Squared = true */
+	CATTLE_HIP_LOSS_MULTI_LABEL_HINGE = 8,          /* loss/MultiLabelHingeLoss.hpp:31-71, Squared = false */
+	CATTLE_HIP_LOSS_SQUARED_MULTI_LABEL_HINGE = 9,  /* loss/MultiLabelHingeLoss.hpp:31-71, Squared = true */
+	CATTLE_HIP_LOSS_MULTI_LABEL_LOG = 10,           /* loss/MultiLabelLogLoss.hpp:37-76 */
+	/* a flag to OR into one of the kinds above: the loss wrapped in NegatedLoss (loss/NegatedLoss.hpp:41-46),
+	 * whose function and d_function are the wrapped loss's with the opposite sign */
+	CATTLE_HIP_LOSS_NEGATED = 0x100
 } cattle_hip_loss;
 
 /* Loss::function (loss/UniversalLoss.hpp:37-41 non-sequential, :99-110 sequential): `losses`
  * receives one value per sample, summed over the time steps. `out` and `obj` are
  * (batch, time_steps, sample_size) column-major; pass time_steps = 1 for non-sequential data.
- * `epsilon` is SoftmaxCrossEntropyLoss's constructor argument (ignored by the squared loss). */
+ * `epsilon` is the constructor argument of the losses that have one (the cross entropies, Kullback-Leibler,
+ * multi-label log; ignored by the others). The hinge losses take one-hot objectives; a row without a one,
+ * which the reference asserts against, gets NaN as its loss and gradient. */
 int cattle_hip_loss_function(cattle_hip_dtype dtype, cattle_hip_loss kind, const void* out, cattle_hip_memspace out_space,
 		const void* obj, cattle_hip_memspace obj_space, size_t batch, size_t time_steps, size_t sample_size,
 		double epsilon, void* losses, cattle_hip_memspace losses_space);

@@ -20,8 +20,9 @@
  *   max/mean pool       pinned: brute force incl. crafted ties, NaN/-inf windows, overlaps.
  *   transposed conv     pinned: torch float64 conv_transpose2d with autograd, the adjoint identity with
  *                       the (pinned) convolution, output-size formula on the reference's test geometries.
- *   losses              pinned: torch float64 cross_entropy / mse (epsilon 0), numpy closed forms with
- *                       the epsilon, central differences of the loss against its gradient.
+ *   losses              pinned: torch float64 cross_entropy / mse / l1 / binary_cross_entropy / nll / kl_div /
+ *                       multi_margin_loss (epsilon 0) with autograd for the gradients, hand-worked rows at the
+ *                       hinge thresholds and with the epsilons, central differences of each loss against its gradient.
  *   other optimizers    pinned: torch's SGD (momentum, Nesterov), Adagrad, RMSprop, Adadelta and Adamax where the
  *                       recurrences coincide; first-step closed forms and the running-maximum property for
  *                       Nadam and AMSGrad, whose reference formulas differ from torch's.
@@ -699,13 +700,52 @@ int transconv_backward(TransGeom g, const T* x, const T* w, const T* out_grad, T
 }
 
 /* ---------------------------------------------------------------------------------------------
- * Losses (loss/SquaredLoss.hpp:25-34, loss/SoftmaxCrossEntropyLoss.hpp:33-50) under the
- * UniversalLoss drivers (loss/UniversalLoss.hpp:37-46 non-sequential; :99-125 sequential: every time
- * step is sliced out and treated as its own rows x cols matrix, losses add up over the steps).
- * A batch is (N, T, V) column-major; T = 1 is the non-sequential case.
+ * Losses under the UniversalLoss drivers (loss/UniversalLoss.hpp:37-46 non-sequential; :99-125
+ * sequential: every time step is sliced out and treated as its own rows x cols matrix, losses add up
+ * over the steps). A batch is (N, T, V) column-major; T = 1 is the non-sequential case.
+ *   0  loss/SquaredLoss.hpp:25-34               1  loss/SoftmaxCrossEntropyLoss.hpp:33-50
+ *   2  loss/AbsoluteLoss.hpp:25-35              3  loss/BinaryCrossEntropyLoss.hpp:35-46 (V must be 1)
+ *   4  loss/CrossEntropyLoss.hpp:33-42          5  loss/KullbackLeiblerLoss.hpp:32-43
+ *   6  loss/HingeLoss.hpp:31-99                 7  the same with Squared = true
+ *   8  loss/MultiLabelHingeLoss.hpp:31-71       9  the same with Squared = true
+ *   10 loss/MultiLabelLogLoss.hpp:37-76
+ * kind | 0x100 is the loss wrapped in NegatedLoss (loss/NegatedLoss.hpp:41-46): both results negated.
  * ------------------------------------------------------------------------------------------- */
+constexpr int LOSS_NEGATED = 0x100;
+
+/* core/NumericUtils.hpp:42-49 with the default epsilons (the scalar type's machine epsilon) */
+template<typename T>
+bool almost_equal(T a, T b) {
+	const T e = std::numeric_limits<T>::epsilon();
+	const T diff = std::abs(a - b);
+	if (diff <= e)
+		return true;
+	return diff <= std::max(std::abs(a), std::abs(b)) * e;
+}
+
+/* core/NumericUtils.hpp:62-65 */
+template<typename T>
+bool decidedly_greater(T a, T b) {
+	return a > b && !almost_equal(a, b);
+}
+
+/* the index of the one in a one-hot row (loss/HingeLoss.hpp:38-48: the last element that almost equals 1);
+ * -1 when there is none, which the reference asserts against */
+template<typename T>
+i64 one_hot_index(const T* y, i64 cs, i64 V) {
+	i64 ind = -1;
+	for (i64 j = 0; j < V; ++j)
+		if (almost_equal<T>(y[cs * j], (T) 1))
+			ind = j;
+	return ind;
+}
+
 template<typename T>
 int loss_function(int kind, i64 N, i64 Ts, i64 V, T eps, const T* out, const T* obj, T* losses) {
+	const bool negated = (kind & LOSS_NEGATED) != 0;
+	kind &= ~LOSS_NEGATED;
+	if (kind < 0 || kind > 10 || (kind == 3 && V != 1))
+		return 1;
 	std::vector<T> e((size_t) V);
 	for (i64 n = 0; n < N; ++n)
 		losses[n] = 0;
@@ -715,10 +755,12 @@ int loss_function(int kind, i64 N, i64 Ts, i64 V, T eps, const T* out, const T* 
 			const T* y = obj + n + N * t;
 			const i64 cs = N * Ts;
 			T l = 0;
-			if (kind == 0) {
+			switch (kind) {
+			case 0:
 				for (i64 j = 0; j < V; ++j)
 					l += (o[cs * j] - y[cs * j]) * (o[cs * j] - y[cs * j]);
-			} else {
+				break;
+			case 1: {
 				T mx = o[0];
 				for (i64 j = 1; j < V; ++j)
 					mx = std::max(mx, o[cs * j]);
@@ -730,8 +772,52 @@ int loss_function(int kind, i64 N, i64 Ts, i64 V, T eps, const T* out, const T* 
 				for (i64 j = 0; j < V; ++j)
 					l += std::log(e[j] / (sum + eps)) * y[cs * j];
 				l = -l;
+				break;
 			}
-			losses[n] += l;
+			case 2:
+				for (i64 j = 0; j < V; ++j)
+					l += std::abs(o[cs * j] - y[cs * j]);
+				break;
+			case 3:
+				l = -(y[0] * std::log(o[0] + eps) + ((T) 1 - y[0]) * std::log((T) (1 + eps) - o[0]));
+				break;
+			case 4:
+				for (i64 j = 0; j < V; ++j)
+					l += std::log(o[cs * j] + eps) * y[cs * j];
+				l = -l;
+				break;
+			case 5:
+				for (i64 j = 0; j < V; ++j)
+					l += std::log(o[cs * j] / (y[cs * j] + eps) + eps) * y[cs * j];
+				l = -l;
+				break;
+			case 6:
+			case 7: {
+				const i64 c = one_hot_index<T>(y, cs, V);
+				if (c < 0)
+					return 2;
+				const T score = o[cs * c];
+				for (i64 j = 0; j < V; ++j) {
+					if (j == c)
+						continue;
+					const T lj = std::max((T) 0, (T) (o[cs * j] - score + 1));
+					l += kind == 7 ? lj * lj : lj;
+				}
+				break;
+			}
+			case 8:
+			case 9:
+				for (i64 j = 0; j < V; ++j) {
+					const T lj = std::max((T) 0, (T) 1 - y[cs * j] * o[cs * j]);
+					l += kind == 9 ? lj * lj : lj;
+				}
+				break;
+			default:
+				for (i64 j = 0; j < V; ++j)
+					l += y[cs * j] * std::log(o[cs * j] + eps) + (1 - y[cs * j]) * std::log(1 + eps - o[cs * j]);
+				break;
+			}
+			losses[n] += negated ? -l : l;
 		}
 	return 0;
 }
@@ -740,25 +826,90 @@ int loss_function(int kind, i64 N, i64 Ts, i64 V, T eps, const T* out, const T* 
  * (optimizer/SGDOptimizer.hpp:54-55). */
 template<typename T>
 int loss_d_function(int kind, i64 N, i64 Ts, i64 V, T eps, T scale, const T* out, const T* obj, T* grad) {
+	if ((kind & LOSS_NEGATED) != 0) {
+		scale = -scale;
+		kind &= ~LOSS_NEGATED;
+	}
+	if (kind < 0 || kind > 10 || (kind == 3 && V != 1))
+		return 1;
 	std::vector<T> e((size_t) V);
 	const i64 cs = N * Ts;
 	for (i64 t = 0; t < Ts; ++t)
 		for (i64 n = 0; n < N; ++n) {
 			const i64 base = n + N * t;
-			if (kind == 0) {
+			const T* o = out + base;
+			const T* y = obj + base;
+			T* g = grad + base;
+			switch (kind) {
+			case 0:
 				for (i64 j = 0; j < V; ++j)
-					grad[base + cs * j] = scale * (2 * (out[base + cs * j] - obj[base + cs * j]));
-			} else {
-				T mx = out[base];
+					g[cs * j] = scale * (2 * (o[cs * j] - y[cs * j]));
+				break;
+			case 1: {
+				T mx = o[0];
 				for (i64 j = 1; j < V; ++j)
-					mx = std::max(mx, out[base + cs * j]);
+					mx = std::max(mx, o[cs * j]);
 				T sum = 0;
 				for (i64 j = 0; j < V; ++j) {
-					e[j] = std::exp(out[base + cs * j] - mx);
+					e[j] = std::exp(o[cs * j] - mx);
 					sum += e[j];
 				}
 				for (i64 j = 0; j < V; ++j)
-					grad[base + cs * j] = scale * (e[j] / (sum + eps) - obj[base + cs * j]);
+					g[cs * j] = scale * (e[j] / (sum + eps) - y[cs * j]);
+				break;
+			}
+			case 2:
+				for (i64 j = 0; j < V; ++j)
+					g[cs * j] = scale * (T) (o[cs * j] - y[cs * j] >= 0 ? 1 : -1);
+				break;
+			case 3:
+				g[0] = scale * -(y[0] / (o[0] + eps) - ((T) 1 - y[0]) / ((T) (1 + eps) - o[0]));
+				break;
+			case 4:
+			case 5:
+				for (i64 j = 0; j < V; ++j)
+					g[cs * j] = scale * (-y[cs * j] / (o[cs * j] + eps));
+				break;
+			case 6:
+			case 7: {
+				const i64 c = one_hot_index<T>(y, cs, V);
+				if (c < 0)
+					return 2;
+				const T score = o[cs * c];
+				T total = 0;
+				for (i64 j = 0; j < V; ++j) {
+					if (j == c)
+						continue;
+					const T margin = o[cs * j] - score + 1;
+					if (decidedly_greater<T>(margin, (T) 0)) {
+						const T gj = kind == 7 ? 2 * margin : 1;
+						total += gj;
+						g[cs * j] = scale * gj;
+					} else
+						g[cs * j] = scale * (T) 0;
+				}
+				g[cs * c] = scale * -total;
+				break;
+			}
+			case 8:
+			case 9:
+				for (i64 j = 0; j < V; ++j) {
+					const T margin = 1 - y[cs * j] * o[cs * j];
+					if (decidedly_greater<T>(margin, (T) 0))
+						g[cs * j] = scale * (kind == 9 ? 2 * o[cs * j] - 2 * y[cs * j] : -y[cs * j]);
+					else
+						g[cs * j] = scale * (T) 0;
+				}
+				break;
+			default:
+				for (i64 j = 0; j < V; ++j) {
+					T oj = o[cs * j];
+					const T denominator = oj * (1 - oj);
+					if (oj == 0)
+						oj += eps;
+					g[cs * j] = scale * ((y[cs * j] - oj) / denominator);
+				}
+				break;
 			}
 		}
 	return 0;

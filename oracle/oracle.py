@@ -326,7 +326,14 @@ def meanpool_backward(x_shape, out_grad, RH=2, RW=2, sv=2, sh=2):
     return dx
 
 
-LOSS_KINDS = {"squared": 0, "softmax_cross_entropy": 1}
+LOSS_KINDS = {"squared": 0, "softmax_cross_entropy": 1, "absolute": 2, "binary_cross_entropy": 3, "cross_entropy": 4,
+              "kullback_leibler": 5, "hinge": 6, "squared_hinge": 7, "multi_label_hinge": 8,
+              "squared_multi_label_hinge": 9, "multi_label_log": 10}
+LOSS_NEGATED = 0x100        # the loss wrapped in NegatedLoss (loss/NegatedLoss.hpp:41-46)
+
+
+def _loss_kind(kind, negated):
+    return ctypes.c_int(LOSS_KINDS[kind] | (LOSS_NEGATED if negated else 0))
 
 
 def _loss_dims(out, sequential):
@@ -335,23 +342,23 @@ def _loss_dims(out, sequential):
     return N, Ts, out.size // (N * Ts)
 
 
-def loss_function(kind, out, obj, eps=1e-5, sequential=False):
+def loss_function(kind, out, obj, eps=1e-5, sequential=False, negated=False):
     """Per-sample losses (summed over time steps when sequential: out is then (N, T, ...))."""
     dt = out.dtype
     out, obj = _f(out, dt), _f(obj, dt)
     N, Ts, V = _loss_dims(out, sequential)
     losses = np.empty((N,), dtype=dt)
-    _call("loss_function", dt, ctypes.c_int(LOSS_KINDS[kind]), *_ll(N, Ts, V), ctypes.c_double(eps), _p(out), _p(obj),
+    _call("loss_function", dt, _loss_kind(kind, negated), *_ll(N, Ts, V), ctypes.c_double(eps), _p(out), _p(obj),
           _p(losses))
     return losses
 
 
-def loss_d_function(kind, out, obj, eps=1e-5, scale=1.0, sequential=False):
+def loss_d_function(kind, out, obj, eps=1e-5, scale=1.0, sequential=False, negated=False):
     dt = out.dtype
     out, obj = _f(out, dt), _f(obj, dt)
     N, Ts, V = _loss_dims(out, sequential)
     grad = np.empty(out.shape, dtype=dt, order="F")
-    _call("loss_d_function", dt, ctypes.c_int(LOSS_KINDS[kind]), *_ll(N, Ts, V), ctypes.c_double(eps),
+    _call("loss_d_function", dt, _loss_kind(kind, negated), *_ll(N, Ts, V), ctypes.c_double(eps),
           ctypes.c_double(scale), _p(out), _p(obj), _p(grad))
     return grad
 

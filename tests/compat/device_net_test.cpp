@@ -126,6 +126,18 @@ static void run(const std::string& tag) {
 		record_final<Scalar>(tag + ".mlp", net);
 	}
 	{
+		/* another loss of the loss/ directory, wrapped as NegatedLoss wraps it */
+		Lcg g(13);
+		const std::size_t batch = 9, classes = 7;
+		std::vector<Scalar> o = random_values<Scalar>(batch * classes, g, 1.0), y = one_hot<Scalar>(batch, classes, g);
+		DT od(typename DT::Dims{ { batch, classes, 1, 1 } }, o.data()), yd(typename DT::Dims{ { batch, classes, 1, 1 } }, y.data());
+		DeviceLoss<Scalar> negated_hinge(CATTLE_HIP_LOSS_SQUARED_HINGE, (Scalar) 1e-5, true);
+		record(tag + ".loss.out", sizeof(Scalar), { batch, classes }, o.data());
+		record(tag + ".loss.obj", sizeof(Scalar), { batch, classes }, y.data());
+		record(tag + ".loss.values", sizeof(Scalar), { batch }, negated_hinge.function(od, yd).data());
+		record(tag + ".loss.grad", sizeof(Scalar), { batch, classes }, negated_hinge.d_function(od, yd, (Scalar) 0.5).to_host().data());
+	}
+	{
 		Lcg g(12);
 		const std::size_t batch = 16;
 		std::vector<DL> layers;

@@ -107,3 +107,40 @@ def brute_maxpool(x, RH, RW, sv, sh):
                     out[n, oh, ow, c] = best
                     inds[ow * OH + oh, c * N + n] = bi
     return out, inds
+
+
+ALL_LOSSES = ["squared", "softmax_cross_entropy", "absolute", "binary_cross_entropy", "cross_entropy", "kullback_leibler",
+              "hinge", "squared_hinge", "multi_label_hinge", "squared_multi_label_hinge", "multi_label_log"]
+
+
+def loss_inputs(gen, kind, N, dims, dtype, steps=None):
+    """Outputs and objectives a loss of this kind accepts (the ranges its class comment in loss/*.hpp names), as
+    (N, *dims) tensors or, with `steps`, (N, steps, *dims) sequences; element j of a sample's step is at Fortran
+    position j of its `dims`. binary_cross_entropy takes one value per sample and step (dims must multiply to 1)."""
+    Ts = 1 if steps is None else steps
+    V = int(np.prod(dims))
+    shape = (N, Ts, V)
+    if kind in ("squared", "absolute"):
+        out, obj = gen.standard_normal(shape), gen.standard_normal(shape)
+    elif kind == "softmax_cross_entropy":
+        out, obj = gen.standard_normal(shape) * 2, np.zeros(shape)
+        np.put_along_axis(obj, gen.integers(0, V, (N, Ts, 1)), 1.0, axis=2)
+    elif kind == "binary_cross_entropy":
+        assert V == 1
+        out, obj = gen.uniform(0.05, 0.95, shape), gen.uniform(0, 1, shape)
+    elif kind in ("cross_entropy", "kullback_leibler"):
+        out = gen.uniform(0.05, 1, shape)
+        out /= out.sum(axis=2, keepdims=True)
+        obj = gen.uniform(0.05, 1, shape)
+        obj /= obj.sum(axis=2, keepdims=True)
+    elif kind in ("hinge", "squared_hinge"):
+        out, obj = gen.standard_normal(shape), np.zeros(shape)
+        np.put_along_axis(obj, gen.integers(0, V, (N, Ts, 1)), 1.0, axis=2)
+    elif kind in ("multi_label_hinge", "squared_multi_label_hinge"):
+        out, obj = gen.standard_normal(shape), gen.integers(0, 2, shape) * 2.0 - 1.0
+    elif kind == "multi_label_log":
+        out, obj = gen.uniform(0.05, 0.95, shape), gen.integers(0, 2, shape) * 1.0
+    else:
+        raise KeyError(kind)
+    full = (N,) + (() if steps is None else (steps,)) + tuple(dims)
+    return tuple(np.asfortranarray(np.asfortranarray(a.astype(dtype)).reshape(full, order="F")) for a in (out, obj))

@@ -63,6 +63,14 @@ def out_shape(net):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-10)])
+def test_device_loss_of_another_kind_negated(records, tag, tol):
+    out, obj = np.asarray(records[tag + ".loss.out"], np.float64), np.asarray(records[tag + ".loss.obj"], np.float64)
+    assert hp.rel_err(records[tag + ".loss.values"], oracle.loss_function("squared_hinge", out, obj, negated=True)) < tol
+    assert hp.rel_err(records[tag + ".loss.grad"], oracle.loss_d_function("squared_hinge", out, obj, scale=0.5, negated=True)) < tol
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-9)])
 def test_mlp_sgd_batches(records, tag, tol):
     r = {k[len(tag) + 5:]: v for k, v in records.items() if k.startswith(tag + ".mlp.")}

@@ -70,16 +70,109 @@ def test_sequential_losses(kind, dtype):
                       oracle.loss_d_function(kind, o64, y64, eps=eps, scale=0.25, sequential=True)) < tol
 
 
+OTHER_LOSSES = hp.ALL_LOSSES[2:]
+# losses whose value or gradient switches at a threshold (a margin or difference of zero): their inputs are put
+# on a grid of 1/64 so that every margin is computed exactly, in float32 as in the float64 of the oracle, and
+# margins of exactly zero occur
+THRESHOLD_LOSSES = ("absolute", "hinge", "squared_hinge", "multi_label_hinge", "squared_multi_label_hinge")
+
+
+def _loss_case(gen, kind, N, dims, dtype, steps=None):
+    if kind == "binary_cross_entropy":
+        dims = (1,) * len(dims)
+    out, obj = hp.loss_inputs(gen, kind, N, dims, dtype, steps)
+    if kind in THRESHOLD_LOSSES:
+        out = np.asfortranarray(np.round(out * 64) / 64)
+        obj = np.asfortranarray(np.round(obj * 64) / 64)
+    return out, obj
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", OTHER_LOSSES)
+@pytest.mark.parametrize("N,dims", [(256, (10,)), (37, (3, 5, 2)), (1, (1,)), (70, (1000,)), (32, (16, 16, 32))])
+def test_the_other_losses(N, dims, kind, dtype):
+    g = hp.rng(1203)
+    out, obj = _loss_case(g, kind, N, dims, dtype)
+    o64, y64 = np.asarray(out, np.float64), np.asarray(obj, np.float64)
+    eps = float(dtype(1e-5))
+    tol = TOL[np.dtype(dtype)]
+    l_ref = oracle.loss_function(kind, o64, y64, eps=eps)
+    assert np.max(np.abs(ch.loss_function(kind, out, obj) - l_ref) / np.maximum(np.abs(l_ref), 1.0)) < tol
+    scale = float(dtype(1.0 / N))
+    g_ref = oracle.loss_d_function(kind, o64, y64, eps=eps, scale=scale)
+    got = ch.loss_d_function(kind, out, obj, scale=scale)
+    assert hp.rel_err(got, g_ref) < tol
+    if kind in THRESHOLD_LOSSES:            # which elements are inside the margin is decided identically
+        assert np.array_equal(got == 0, g_ref == 0)
+    # NegatedLoss: the same values with the opposite sign
+    assert np.array_equal(ch.loss_function(kind, out, obj, negated=True), -ch.loss_function(kind, out, obj))
+    assert np.array_equal(ch.loss_d_function(kind, out, obj, scale=scale, negated=True), -got)
+    # the same through device-resident buffers
+    od, yd = ch.DeviceTensor.from_host(out), ch.DeviceTensor.from_host(obj)
+    assert np.array_equal(ch.loss_function(kind, od, yd), ch.loss_function(kind, out, obj))
+    assert np.array_equal(ch.loss_d_function(kind, od, yd, scale=scale).to_host(), got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", OTHER_LOSSES)
+def test_the_other_losses_on_sequences(kind, dtype):
+    g = hp.rng(1204)
+    out, obj = _loss_case(g, kind, 33, (4, 3), dtype, steps=5)
+    o64, y64 = np.asarray(out, np.float64), np.asarray(obj, np.float64)
+    eps = float(dtype(1e-5))
+    tol = TOL[np.dtype(dtype)]
+    assert hp.rel_err(ch.loss_function(kind, out, obj, sequential=True),
+                      oracle.loss_function(kind, o64, y64, eps=eps, sequential=True)) < tol
+    assert hp.rel_err(ch.loss_d_function(kind, out, obj, scale=0.25, sequential=True),
+                      oracle.loss_d_function(kind, o64, y64, eps=eps, scale=0.25, sequential=True)) < tol
+    assert hp.rel_err(ch.loss_d_function(kind, out, obj, scale=0.25, sequential=True, negated=True),
+                      oracle.loss_d_function(kind, o64, y64, eps=eps, scale=0.25, sequential=True, negated=True)) < tol
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_loss_corner_values(dtype):
+    """The rows worked by hand for the oracle, on the device: margins at the machine epsilon, a zero difference,
+    an output of exactly zero under the multi-label log loss, the last one of a row as the hinge class."""
+    col = lambda *v: np.asfortranarray(np.array(v, dtype).reshape(1, -1))
+    tiny = np.finfo(dtype).eps
+    o, y = col(2.0, 1.0, 1.5, 1.0 + tiny), col(1, 0, 0, 0)
+    for kind in ("hinge", "squared_hinge"):
+        assert np.array_equal(ch.loss_function(kind, o, y), oracle.loss_function(kind, o, y))
+        assert np.array_equal(ch.loss_d_function(kind, o, y), [[-1.0, 0.0, 1.0, 0.0]])
+    assert np.array_equal(ch.loss_d_function("hinge", col(0.0, 0.0, 5.0), col(0, 1, 0)), [[1.0, -2.0, 1.0]])
+    assert np.array_equal(ch.loss_d_function("absolute", col(1.0, 2.0, 0.5), col(1.0, 3.0, 0.25)), [[1.0, -1.0, 1.0]])
+    o, y = col(0.5, -2.0, 1.0, -0.25, 1.0 - tiny), col(1, -1, 1, 1, 1)
+    assert np.array_equal(ch.loss_d_function("multi_label_hinge", o, y), [[-1.0, 0.0, 0.0, -1.0, 0.0]])
+    assert np.array_equal(ch.loss_d_function("squared_multi_label_hinge", o, y), [[-1.0, 0.0, 0.0, -2.5, 0.0]])
+    with np.errstate(all="ignore"):
+        inf = ch.loss_d_function("multi_label_log", col(0.0, 0.0, 0.25), col(1, 0, 1), epsilon=0.25)
+    assert inf[0, 0] == np.inf and inf[0, 1] == -np.inf and inf[0, 2] == 4.0
+    # a hinge row without a one (the reference asserts against it): NaN marks the row, other rows are unaffected
+    o = np.asfortranarray(np.array([[0.0, 1.0, 2.0], [2.0, 1.0, 1.5]], dtype))
+    y = np.asfortranarray(np.array([[0, 0, 0], [1, 0, 0]], dtype))
+    for kind in ("hinge", "squared_hinge"):
+        l, gr = ch.loss_function(kind, o, y), ch.loss_d_function(kind, o, y)
+        assert np.isnan(l[0]) and np.all(np.isnan(gr[0]))
+        assert l[1] == oracle.loss_function(kind, o[1:], y[1:])[0]
+        assert np.array_equal(gr[1:], oracle.loss_d_function(kind, o[1:], y[1:]))
+
+
 def test_loss_errors():
     a = np.zeros((4, 3), np.float32, order="F")
     with pytest.raises(ValueError):
         ch.loss_function("squared", a, np.zeros((4, 2), np.float32, order="F"))
     lib = ch.lib()
     import ctypes
-    rc = lib.cattle_hip_loss_function(0, 7, ctypes.c_void_p(a.ctypes.data), 0, ctypes.c_void_p(a.ctypes.data), 0,
-                                      ctypes.c_size_t(4), ctypes.c_size_t(1), ctypes.c_size_t(3), ctypes.c_double(1e-5),
-                                      ctypes.c_void_p(a.ctypes.data), 0)
-    assert rc != 0 and b"loss kind" in lib.cattle_hip_last_error()
+    for bad in (11, 0x100 | 11, -1, 0x200):
+        rc = lib.cattle_hip_loss_function(0, bad, ctypes.c_void_p(a.ctypes.data), 0, ctypes.c_void_p(a.ctypes.data), 0,
+                                          ctypes.c_size_t(4), ctypes.c_size_t(1), ctypes.c_size_t(3), ctypes.c_double(1e-5),
+                                          ctypes.c_void_p(a.ctypes.data), 0)
+        assert rc != 0 and b"loss kind" in lib.cattle_hip_last_error()
+    # the binary cross entropy takes one value per sample and time step (assert in BinaryCrossEntropyLoss.hpp:36,43)
+    with pytest.raises(ch.CattleHipError):
+        ch.loss_function("binary_cross_entropy", a, a)
+    with pytest.raises(ch.CattleHipError):
+        ch.loss_d_function("binary_cross_entropy", a, a)
 
 
 def _dense_with_grads(dtype, seed):

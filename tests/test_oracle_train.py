@@ -86,15 +86,126 @@ def test_loss_gradient_is_the_derivative(kind):
             assert abs(num - grad[n, j]) < 1e-7
 
 
-@pytest.mark.parametrize("kind", ["squared", "softmax_cross_entropy"])
+def _torch_loss(kind, o, y):
+    """Independent float64 implementations (torch's own loss routines where it has one) of the losses at
+    epsilon 0, as differentiable per-sample values; o, y are (N, V) torch tensors."""
+    F = torch.nn.functional
+    V = o.shape[1]
+    if kind == "absolute":
+        return F.l1_loss(o, y, reduction="none").sum(dim=1)
+    if kind == "binary_cross_entropy":
+        return F.binary_cross_entropy(o, y, reduction="none").sum(dim=1)
+    if kind == "cross_entropy":            # one-hot objectives: the negative log likelihood of the class
+        return F.nll_loss(torch.log(o), y.argmax(dim=1), reduction="none")
+    if kind == "kullback_leibler":         # -sum y ln(o / y) = KL(y || o)
+        return F.kl_div(torch.log(o), y, reduction="none").sum(dim=1)
+    if kind in ("hinge", "squared_hinge"):  # torch averages over the classes, the reference sums
+        return F.multi_margin_loss(o, y.argmax(dim=1), p=2 if kind == "squared_hinge" else 1, margin=1.0, reduction="none") * V
+    if kind in ("multi_label_hinge", "squared_multi_label_hinge"):
+        m = torch.clamp(1 - y * o, min=0)
+        return (m * m if kind == "squared_multi_label_hinge" else m).sum(dim=1)
+    if kind == "multi_label_log":          # the reference's value is the log likelihood itself, not its negative
+        return -F.binary_cross_entropy(o, y, reduction="none").sum(dim=1)
+    raise KeyError(kind)
+
+
+@pytest.mark.parametrize("kind", hp.ALL_LOSSES[2:])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_other_losses_against_torch(kind, dtype):
+    g = hp.rng(910)
+    N, V = 7, (1 if kind == "binary_cross_entropy" else 6)
+    src = "hinge" if kind == "cross_entropy" else kind          # one-hot objectives for the nll comparison
+    out, obj = hp.loss_inputs(g, src, N, (V,), dtype)
+    if kind == "cross_entropy":
+        out = hp.loss_inputs(g, kind, N, (V,), dtype)[0]
+    ot = torch.tensor(np.asarray(out, np.float64), requires_grad=True)
+    lt = _torch_loss(kind, ot, torch.tensor(np.asarray(obj, np.float64)))
+    lt.sum().backward()
+    tol = TOL[np.dtype(dtype)]
+    assert hp.rel_err(oracle.loss_function(kind, out, obj, eps=0.0), lt.detach().numpy()) < tol
+    assert hp.rel_err(oracle.loss_d_function(kind, out, obj, eps=0.0), ot.grad.numpy()) < tol
+    assert hp.rel_err(oracle.loss_d_function(kind, out, obj, eps=0.0, scale=0.25), ot.grad.numpy() / 4) < tol
+    # NegatedLoss (loss/NegatedLoss.hpp:41-46)
+    assert np.array_equal(oracle.loss_function(kind, out, obj, eps=0.0, negated=True), -oracle.loss_function(kind, out, obj, eps=0.0))
+    assert np.array_equal(oracle.loss_d_function(kind, out, obj, eps=0.0, scale=0.25, negated=True),
+                          -oracle.loss_d_function(kind, out, obj, eps=0.0, scale=0.25))
+
+
+def test_losses_hand_worked_rows():
+    """Rows small enough to work by hand, with epsilons large enough that a misplaced one shows, and the hinge
+    losses at their thresholds."""
+    f64 = np.float64
+    col = lambda *v: np.asfortranarray(np.array(v, f64).reshape(1, -1))
+    ln = np.log
+    # binary cross entropy, one value per sample: -(y ln(o + e) + (1 - y) ln((1 + e) - o)),  e = 0.25
+    o, y = np.asfortranarray(np.array([[0.25], [0.25]], f64)), np.asfortranarray(np.array([[1.0], [0.0]], f64))
+    assert np.allclose(oracle.loss_function("binary_cross_entropy", o, y, eps=0.25), [ln(2.0), 0.0], atol=1e-15)
+    assert np.allclose(oracle.loss_d_function("binary_cross_entropy", o, y, eps=0.25)[:, 0], [-2.0, 1.0], atol=1e-15)
+    with pytest.raises(RuntimeError):
+        oracle.loss_function("binary_cross_entropy", col(0.2, 0.3), col(1, 0))         # more than one value per sample
+    # cross entropy: -ln(o + e) y ; gradient -y / (o + e)
+    assert np.allclose(oracle.loss_function("cross_entropy", col(0.25, 0.5), col(1, 0), eps=0.25), [ln(2.0)], atol=1e-15)
+    assert np.allclose(oracle.loss_d_function("cross_entropy", col(0.25, 0.5), col(1, 0.5), eps=0.25), [[-2.0, -2.0 / 3]], atol=1e-15)
+    # Kullback-Leibler: -ln(o / (y + e) + e) y ; the reference's gradient is the cross entropy's, -y / (o + e)
+    assert np.allclose(oracle.loss_function("kullback_leibler", col(1.0, 3.0), col(0.5, 0.0), eps=0.5), [-0.5 * ln(1.5)], atol=1e-15)
+    assert np.allclose(oracle.loss_d_function("kullback_leibler", col(1.0, 3.0), col(0.5, 0.0), eps=0.5), [[-1.0 / 3, 0.0]], atol=1e-15)
+    # multi-label log: sum y ln(o + e) + (1 - y) ln(1 + e - o); gradient (y - o) / (o (1 - o)), where an output of
+    # exactly 0 becomes e in the numerator only, so the quotient is infinite
+    assert np.allclose(oracle.loss_function("multi_label_log", col(0.25, 0.75), col(1, 0), eps=0.25), [2 * ln(0.5)], atol=1e-15)
+    assert np.allclose(oracle.loss_d_function("multi_label_log", col(0.25, 0.5), col(1, 0), eps=0.25), [[4.0, -2.0]], atol=1e-15)
+    with np.errstate(all="ignore"):
+        inf = oracle.loss_d_function("multi_label_log", col(0.0, 0.0), col(1, 0), eps=0.25)
+    assert inf[0, 0] == np.inf and inf[0, 1] == -np.inf
+    # absolute: a zero difference has gradient +1 (loss/AbsoluteLoss.hpp:34)
+    assert np.array_equal(oracle.loss_d_function("absolute", col(1.0, 2.0, 0.5), col(1.0, 3.0, 0.25)), [[1.0, -1.0, 1.0]])
+    assert np.array_equal(oracle.loss_function("absolute", col(1.0, 2.0, 0.5), col(1.0, 3.0, 0.25)), [1.25])
+    # hinge, class 0 with score 2: margins of the others are 0 (no loss, no gradient), 0.5, and half a machine
+    # epsilon (counted by the loss, not "decidedly greater" than 0 for the gradient: core/NumericUtils.hpp:62-65)
+    tiny = np.finfo(f64).eps / 2
+    o, y = col(2.0, 1.0, 1.5, 1.0 + tiny * 2), col(1, 0, 0, 0)       # 1 + 2 tiny is the next double after 1
+    assert o[0, 3] - 2.0 + 1 == tiny * 2
+    assert np.allclose(oracle.loss_function("hinge", o, y), [0.5 + 2 * tiny], atol=1e-18)
+    assert np.array_equal(oracle.loss_d_function("hinge", o, y), [[-1.0, 0.0, 1.0, 0.0]])
+    assert np.allclose(oracle.loss_function("squared_hinge", o, y), [0.25], atol=1e-18)
+    assert np.array_equal(oracle.loss_d_function("squared_hinge", o, y), [[-1.0, 0.0, 1.0, 0.0]])
+    # the class is the LAST element that equals one (loss/HingeLoss.hpp:44-47); a row without a one is refused
+    assert np.array_equal(oracle.loss_d_function("hinge", col(0.0, 0.0, 5.0), col(0, 1, 0)), [[1.0, -2.0, 1.0]])
+    with pytest.raises(RuntimeError):
+        oracle.loss_function("hinge", col(0.0, 1.0), col(0, 0))
+    # multi-label hinge: max(0, 1 - y o); gradient -y, squared 2 o - 2 y, inside the margin only
+    o, y = col(0.5, -2.0, 1.0, -0.25), col(1, -1, 1, 1)
+    assert np.array_equal(oracle.loss_function("multi_label_hinge", o, y), [0.5 + 0 + 0 + 1.25])
+    assert np.array_equal(oracle.loss_d_function("multi_label_hinge", o, y), [[-1.0, 0.0, 0.0, -1.0]])
+    assert np.array_equal(oracle.loss_function("squared_multi_label_hinge", o, y), [0.25 + 1.5625])
+    assert np.array_equal(oracle.loss_d_function("squared_multi_label_hinge", o, y), [[-1.0, 0.0, 0.0, -2.5]])
+
+
+@pytest.mark.parametrize("kind", hp.ALL_LOSSES[2:])
+def test_the_other_losses_gradients_are_the_derivatives(kind):
+    """Central differences, as in the reference's own loss tests (test/gradient_test.cpp:819-1100), with an epsilon
+    small enough for the reference's simplified gradients to be the derivatives."""
+    g = hp.rng(911)
+    N, V = 3, (1 if kind == "binary_cross_entropy" else 5)
+    out, obj = hp.loss_inputs(g, kind, N, (V,), np.float64)
+    grad = oracle.loss_d_function(kind, out, obj, eps=1e-14)
+    h = 1e-6
+    for n in range(N):
+        for j in range(V):
+            up, dn = out.copy(order="F"), out.copy(order="F")
+            up[n, j] += h
+            dn[n, j] -= h
+            num = (oracle.loss_function(kind, up, obj, eps=1e-14).sum() - oracle.loss_function(kind, dn, obj, eps=1e-14).sum()) / (2 * h)
+            assert abs(num - grad[n, j]) < 1e-6 * max(1.0, abs(grad[n, j]))
+
+
+@pytest.mark.parametrize("kind", hp.ALL_LOSSES)
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_sequential_losses_are_per_time_step(kind, dtype):
     """loss/UniversalLoss.hpp:99-125: every time step is sliced out and handled as a non-sequential batch;
     losses add up over the steps, gradients are written back into the step's slice."""
     g = hp.rng(905)
-    N, Ts, dims = 5, 4, (3, 2)
-    out = hp.normal(g, (N, Ts) + dims, dtype)
-    obj = hp.uniform(g, (N, Ts) + dims, 0, 1, dtype)
+    N, Ts, dims = 5, 4, ((1, 1) if kind == "binary_cross_entropy" else (3, 2))
+    out, obj = hp.loss_inputs(g, kind, N, dims, dtype, steps=Ts)
     total = oracle.loss_function(kind, out, obj, sequential=True)
     grad = oracle.loss_d_function(kind, out, obj, scale=0.5, sequential=True)
     acc = np.zeros(N)
