@@ -20,8 +20,11 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
 #include <string>
 #include <type_traits>
+#include <unistd.h>
+#include <vector>
 
 namespace cattle_hip {
 
@@ -913,6 +916,11 @@ void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, con
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
 int gather_variant_occupancy(size_t dyn, bool vec, bool divs) {
 	constexpr int VEC = GemmCfg<T>::VEC;
+	/* the answer for the usual launch (no reserved dynamic LDS) is kept: one query per kernel instantiation */
+	static int cached[4] = { 0, 0, 0, 0 };
+	int& slot = cached[(vec ? 2 : 0) + (divs ? 1 : 0)];
+	if (dyn == 0 && slot > 0)
+		return slot;
 	int n = 0;
 	hipError_t e;
 	if (vec && !divs)
@@ -924,6 +932,8 @@ int gather_variant_occupancy(size_t dyn, bool vec, bool divs) {
 	else
 		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true>, 64 * WAVES_M * WAVES_F, dyn);
 	CATTLE_HIP_CHECK(e);
+	if (dyn == 0)
+		slot = n;
 	return n;
 }
 
@@ -977,6 +987,60 @@ template<> struct GatherVariants<double> {
 	}
 };
 
+/* Switches for experiments, read from the environment once, when the first GEMM is launched:
+ *   CATTLE_HIP_GATHER_VARIANT_F<F> = index into the gather variant table for GEMMs with F output columns,
+ *   CATTLE_HIP_GATHER_OCC_F<F>     = blocks per CU for them (enforced by reserving dynamic LDS),
+ *   CATTLE_HIP_NO_SWIZZLE, CATTLE_HIP_NO_ROW_BLOCKS, CATTLE_HIP_NO_SPLIT: tile walk, blocked tile rows, cut reductions off,
+ *   CATTLE_HIP_WGRAD_VARIANT, CATTLE_HIP_WGRAD_SPLITS, CATTLE_HIP_WGRAD_LINEAR: the weight-gradient plan. */
+struct Tuning {
+	struct PerF { int F, variant, occ; };
+	std::vector<PerF> per_f;
+	bool no_swizzle, no_row_blocks, no_split, wgrad_linear;
+	int wgrad_variant, wgrad_splits;
+
+	Tuning() {
+		no_swizzle = std::getenv("CATTLE_HIP_NO_SWIZZLE") != nullptr;
+		no_row_blocks = std::getenv("CATTLE_HIP_NO_ROW_BLOCKS") != nullptr;
+		no_split = std::getenv("CATTLE_HIP_NO_SPLIT") != nullptr;
+		wgrad_linear = std::getenv("CATTLE_HIP_WGRAD_LINEAR") != nullptr;
+		const char* e = std::getenv("CATTLE_HIP_WGRAD_VARIANT");
+		wgrad_variant = e ? std::atoi(e) : -1;
+		e = std::getenv("CATTLE_HIP_WGRAD_SPLITS");
+		wgrad_splits = e ? std::atoi(e) : 0;
+		for (char** v = environ; v && *v; ++v) {
+			static const char* const keys[2] = { "CATTLE_HIP_GATHER_VARIANT_F", "CATTLE_HIP_GATHER_OCC_F" };
+			for (int k = 0; k < 2; ++k) {
+				const size_t len = std::strlen(keys[k]);
+				if (std::strncmp(*v, keys[k], len) != 0)
+					continue;
+				const char* eq = std::strchr(*v + len, '=');
+				if (!eq)
+					continue;
+				PerF& slot = entry(std::atoi(*v + len));
+				(k == 0 ? slot.variant : slot.occ) = std::atoi(eq + 1);
+			}
+		}
+	}
+	PerF& entry(int F) {
+		for (PerF& p : per_f)
+			if (p.F == F)
+				return p;
+		per_f.push_back(PerF{ F, -1, 0 });
+		return per_f.back();
+	}
+	const PerF* find(int F) const {
+		for (const PerF& p : per_f)
+			if (p.F == F)
+				return &p;
+		return nullptr;
+	}
+};
+
+const Tuning& tuning() {
+	static const Tuning t;
+	return t;
+}
+
 /* Picks the tile shape: the narrowest F tile that covers all output columns in one block column (so
  * the gathered A operand, the expensive one, is read once), else the widest. Blocks run at the
  * occupancy their LDS and register use allows; measured on MI355X, more co-resident blocks beat
@@ -1006,18 +1070,13 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) >= 2 * NUM_CUS)
 			best_v += SHORT;
 	}
-	/* tuning overrides for experiments, keyed by the number of output columns F of the GEMM:
-	 * CATTLE_HIP_GATHER_VARIANT_F<F> = index into the variant table, CATTLE_HIP_GATHER_OCC_F<F> = blocks per CU
-	 * (enforced by reserving dynamic LDS) */
+	const Tuning& tune = tuning();
 	int occ = 0;
-	const std::string suffix = "_F" + std::to_string(g.F);
-	if (const char* e = std::getenv(("CATTLE_HIP_GATHER_VARIANT" + suffix).c_str())) {
-		const int i = std::atoi(e);
-		if (i >= 0 && i < GatherVariants<T>::COUNT)
-			best_v = i;
+	if (const Tuning::PerF* o = tune.find(g.F)) {
+		if (o->variant >= 0 && o->variant < GatherVariants<T>::COUNT)
+			best_v = o->variant;
+		occ = o->occ;
 	}
-	if (const char* e = std::getenv(("CATTLE_HIP_GATHER_OCC" + suffix).c_str()))
-		occ = std::atoi(e);
 	const GatherVariant<T>& v = vars[best_v];
 	size_t dyn = 0;
 	if (occ >= 1 && occ <= 8) {
@@ -1029,12 +1088,11 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	/* tiles per output column, if a column (N * OA rows of M) is a whole number of tiles and there are
 	 * several columns; 0 switches the 2-D walk off */
 	const long column = (long) g.N * g.OA;
-	int tile_rows = (column % v.bm == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE")) ? (int) (column / v.bm) : 0;
+	int tile_rows = (column % v.bm == 0 && g.OB > 1 && !tune.no_swizzle) ? (int) (column / v.bm) : 0;
 	/* rows of a tile as 32 samples x a rectangle of positions (see tile_row_m) where the shape allows it: as many
 	 * positions along a as divide OA, the rest along b; the 2-D walk then runs over strips of pos_b columns */
 	int sample_blocks = 0, pos_b = 1;
-	if (g.N % 32 == 0 && v.bm % 32 == 0 && g.OB > 1 && !std::getenv("CATTLE_HIP_NO_SWIZZLE") &&
-			!std::getenv("CATTLE_HIP_NO_ROW_BLOCKS")) {
+	if (g.N % 32 == 0 && v.bm % 32 == 0 && g.OB > 1 && !tune.no_swizzle && !tune.no_row_blocks) {
 		const int positions = v.bm / 32;
 		for (int pb = 1; pb <= positions; pb *= 2) {
 			const int pa = positions / pb;
@@ -1049,7 +1107,7 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	/* blocks the chip holds at once (registers, LDS, waves), as the runtime computes it for this kernel */
 	const int per_cu = std::max(1, v.blocks_per_cu(dyn, vec, divs));
 	const int slots = NUM_CUS * per_cu;
-	const bool no_split = std::getenv("CATTLE_HIP_NO_SPLIT") != nullptr;
+	const bool no_split = tune.no_split;
 
 	/* main_count whole tiles, the other mtiles - main_count with their reduction cut into about `ksplit` parts */
 	auto launch = [&](int main_count, int ksplit) {
@@ -1218,11 +1276,9 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 			p.variant = i;
 		}
 	}
-	if (const char* e = std::getenv("CATTLE_HIP_WGRAD_VARIANT")) {
-		const int i = std::atoi(e);
-		if (i >= 0 && i < WgradVariants<T>::COUNT)
-			p.variant = i;
-	}
+	const Tuning& tune = tuning();
+	if (tune.wgrad_variant >= 0 && tune.wgrad_variant < WgradVariants<T>::COUNT)
+		p.variant = tune.wgrad_variant;
 	const WgradVariant<T>& v = vars[p.variant];
 	p.ktiles = (K + v.bk - 1) / v.bk;
 	p.ftiles = (F + v.bf - 1) / v.bf;
@@ -1232,15 +1288,15 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	const int tiles = p.ktiles * p.ftiles;
 	const int chunks = (M + WGRAD_MC - 1) / WGRAD_MC;
 	int want = std::max(1, slots / tiles);
-	if (const char* e = std::getenv("CATTLE_HIP_WGRAD_SPLITS"))
-		want = std::max(1, std::atoi(e));
+	if (tune.wgrad_splits > 0)
+		want = tune.wgrad_splits;
 	want = std::min(want, std::max(1, chunks / 4));           /* at least four chunks per block */
 	p.chunks_per_split = (chunks + want - 1) / want;
 	p.splits = (chunks + p.chunks_per_split - 1) / p.chunks_per_split;
 	/* pixel mode: slices are ranges of output positions (each at least one), walked sample block by
 	 * sample block; needs chunks that do not straddle positions */
 	const int positions = M / N;
-	p.pixel_mode = N % WGRAD_MC == 0 && positions >= 2 && !std::getenv("CATTLE_HIP_WGRAD_LINEAR");
+	p.pixel_mode = N % WGRAD_MC == 0 && positions >= 2 && !tune.wgrad_linear;
 	if (p.pixel_mode)
 		p.splits = std::max(1, std::min(want, positions));
 	return p;

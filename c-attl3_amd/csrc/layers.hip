@@ -740,8 +740,10 @@ LossStage g_loss_stage;
 template<typename T>
 void run_loss(bool grad_pass, int kind, const void* out, int out_space, const void* obj, int obj_space, size_t batch,
 		size_t time_steps, size_t sample_size, double epsilon, double scale, void* dst, int dst_space) {
+	const size_t limit = 2147483647u;
+	CATTLE_HIP_REQUIRE(batch <= limit && time_steps <= limit / batch && sample_size <= limit / (batch * time_steps),
+			"tensor exceeds 2^31-1 elements");
 	const size_t count = batch * time_steps * sample_size;
-	CATTLE_HIP_REQUIRE(count <= 2147483647u, "tensor exceeds 2^31-1 elements");
 	const size_t bytes = count * sizeof(T), dst_bytes = grad_pass ? bytes : batch * sizeof(T);
 	const T* out_dev = static_cast<const T*>(out);
 	const T* obj_dev = static_cast<const T*>(obj);
