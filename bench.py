@@ -213,6 +213,12 @@ def pointwise_run(args, dtype):
     bn = ch.BatchNormLayer(dtype, (H, W, C))
     add("batchnorm forward (training)", timed(lambda: bn.forward_into(x, y, True)), 4 * es)
     add("batchnorm backward", timed(lambda: bn.backward_into(g, dx)), 5 * es)
+    dr = ch.DropoutLayer(dtype, (H, W, C), 0.25, seed=1)
+    add("dropout forward (training; the mask is regenerated, not stored)", timed(lambda: dr.forward_into(x, y, True)), 2 * es)
+    add("dropout backward", timed(lambda: dr.backward_into(g, dx)), 2 * es)
+    bc = ch.BroadcastLayer(dtype, (H // 2, W // 2, C), (2, 2, 1))
+    add("broadcast 2x2x1 forward (28x28x64 -> 56x56x64)", timed(lambda: bc.forward_into(yp, y, True)), es + es / 4.0)
+    add("broadcast 2x2x1 backward", timed(lambda: bc.backward_into(g, yp)), es + es / 4.0)
     return rows
 
 

@@ -31,6 +31,7 @@ EXPORTS = [
     "cattle_hip_timer_destroy", "cattle_hip_timer_start", "cattle_hip_timer_stop", "cattle_hip_conv_create",
     "cattle_hip_transconv_create", "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
     "cattle_hip_batchnorm_set_stats_initialized", "cattle_hip_activation_create", "cattle_hip_pool_create",
+    "cattle_hip_dropout_create", "cattle_hip_reshape_create", "cattle_hip_broadcast_create",
     "cattle_hip_layer_clone", "cattle_hip_layer_destroy", "cattle_hip_layer_input_dims",
     "cattle_hip_layer_output_dims", "cattle_hip_layer_is_input_layer", "cattle_hip_layer_set_input_layer",
     "cattle_hip_layer_empty_cache", "cattle_hip_layer_forward", "cattle_hip_layer_backward",
@@ -622,6 +623,41 @@ def SigmoidActivationLayer(dtype, dims):
 
 def TanhActivationLayer(dtype, dims):
     return ActivationLayer(dtype, "tanh", dims)
+
+
+def _dims3(dims):
+    return (ctypes.c_size_t * 3)(*_ext3(dims))
+
+
+class DropoutLayer(Layer):
+    """layer/DropoutLayer.hpp:33-96. `seed` keys the generator of the uniform numbers (the reference uses Eigen's global
+    one); the mask of training pass q is a function of (seed, q) and the element index."""
+
+    def __init__(self, dtype, dims, dropout_prob, epsilon=1e-5, seed=0):
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_dropout_create(_dtype_code(dtype), _sz(int(np.prod(dims))), ctypes.c_double(dropout_prob),
+                                               ctypes.c_double(epsilon), ctypes.c_ulonglong(seed), ctypes.byref(h)))
+        Layer.__init__(self, h, dtype, tuple(dims), tuple(dims))
+
+
+class ReshapeLayer(Layer):
+    """layer/ReshapeLayer.hpp:31-90"""
+
+    def __init__(self, dtype, input_dims, output_dims):
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_reshape_create(_dtype_code(dtype), _dims3(input_dims), _dims3(output_dims), ctypes.byref(h)))
+        Layer.__init__(self, h, dtype, tuple(input_dims), tuple(output_dims))
+
+
+class BroadcastLayer(Layer):
+    """layer/BroadcastLayer.hpp:31-101"""
+
+    def __init__(self, dtype, input_dims, broadcast):
+        if len(broadcast) != len(input_dims):
+            raise ValueError("one repetition count per rank")
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_broadcast_create(_dtype_code(dtype), _dims3(input_dims), _dims3(broadcast), ctypes.byref(h)))
+        Layer.__init__(self, h, dtype, tuple(input_dims), tuple(int(d) * int(b) for d, b in zip(input_dims, broadcast)))
 
 
 class _PoolLayer(Layer):

@@ -134,6 +134,14 @@ template<typename T> void add_row_vector(int N, size_t V, const T* row, T* x);
 /* row[e] += sum_n x[n + N*e]  (column sums of an N x V matrix, accumulated) */
 template<typename T> void accumulate_column_sums(int N, size_t V, const T* x, T* row);
 
+/* DropoutLayer: y = x * mask(u) with the uniform numbers u regenerated from `key` (the key of training pass `pass` of a
+ * layer seeded with `seed` is dropout_pass_key(seed, pass)); used for the forward and the backward pass. */
+unsigned long long dropout_pass_key(unsigned long long seed, unsigned long long pass);
+template<typename T> void dropout_apply(size_t n, unsigned long long key, T prob, T eps, const T* x, T* y);
+/* BroadcastLayer on (N, H, W, C) -> (N, H bh, W bw, C bc) and the sum of the replicas back. */
+template<typename T> void broadcast_forward(int H, int W, int C, int bh, int bw, int bc, int N, const T* x, T* out);
+template<typename T> void broadcast_backward(int H, int W, int C, int bh, int bw, int bc, int N, const T* out_grad, T* in_grad);
+
 /* The element-wise part of an LSTM cell step between the kernel layers. kind/param index: 0 forget,
  * 1 write, 2 candidate, 3 state, 4 read activation (element-wise kinds only). Per-step tensors hold
  * the four gates as consecutive blocks of P elements; `*_all` tensors are (N, T, ...) over all steps. */

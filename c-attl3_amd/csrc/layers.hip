@@ -690,6 +690,101 @@ struct PoolLayer : LayerBase {
 	}
 };
 
+/* DropoutLayer (layer/DropoutLayer.hpp:33-96). The mask of a training pass is not kept: the pass number is, and the
+ * backward pass regenerates the mask from it. An inference pass hands the input through. */
+template<typename T>
+struct DropoutLayer : LayerBase {
+	T prob, eps;
+	unsigned long long seed, passes = 0;      /* training passes so far; the last one's number is passes - 1 */
+	bool have_mask = false;
+
+	DropoutLayer(int dtype, size_t volume, T prob, T eps, unsigned long long seed) : LayerBase(dtype), prob(prob), eps(eps),
+			seed(seed) {
+		in_dims[0] = out_dims[0] = volume;
+		in_dims[1] = out_dims[1] = 1;
+		in_dims[2] = out_dims[2] = 1;
+	}
+	DropoutLayer(const DropoutLayer& o, bool share) : LayerBase(o.dtype), prob(o.prob), eps(o.eps), seed(o.seed),
+			passes(o.passes), have_mask(o.have_mask) {
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new DropoutLayer(*this, share);
+	}
+	void forward(const void* in, size_t N, bool training, void* out) override {
+		const size_t total = N * in_volume();
+		if (training) {
+			dropout_apply<T>(total, dropout_pass_key(seed, passes), prob, eps, (const T*) in, (T*) out);
+			++passes;
+			have_mask = true;
+		} else if (in != out)
+			CATTLE_HIP_CHECK(hipMemcpyAsync(out, in, total * sizeof(T), hipMemcpyDeviceToDevice, stream()));
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		/* assert(dropout_mask.dimension(0) == out_grad.dimension(0)), DropoutLayer.hpp:91 */
+		CATTLE_HIP_REQUIRE(have_mask, "pass_back without a training pass_forward");
+		if (in_grad)
+			dropout_apply<T>(N * in_volume(), dropout_pass_key(seed, passes - 1), prob, eps, (const T*) out_grad, (T*) in_grad);
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		have_mask = false;
+	}
+};
+
+/* ReshapeLayer (layer/ReshapeLayer.hpp:31-90): the same values under other dimensions; in column-major memory with
+ * the sample index first that is a copy. */
+struct ReshapeLayer : LayerBase {
+	ReshapeLayer(int dtype, const size_t in[3], const size_t out[3]) : LayerBase(dtype) {
+		std::memcpy(in_dims, in, sizeof(in_dims));
+		std::memcpy(out_dims, out, sizeof(out_dims));
+	}
+	ReshapeLayer(const ReshapeLayer& o, bool share) : LayerBase(o.dtype) {
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new ReshapeLayer(*this, share);
+	}
+	void forward(const void* in, size_t N, bool, void* out) override {
+		if (in != out)
+			CATTLE_HIP_CHECK(hipMemcpyAsync(out, in, N * in_volume() * esize(), hipMemcpyDeviceToDevice, stream()));
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		if (in_grad && in_grad != out_grad)
+			CATTLE_HIP_CHECK(hipMemcpyAsync(in_grad, out_grad, N * in_volume() * esize(), hipMemcpyDeviceToDevice, stream()));
+	}
+};
+
+/* BroadcastLayer (layer/BroadcastLayer.hpp:31-101) */
+template<typename T>
+struct BroadcastLayer : LayerBase {
+	int reps[3];
+
+	BroadcastLayer(int dtype, const size_t in[3], const size_t broadcast[3]) : LayerBase(dtype) {
+		for (int i = 0; i < 3; ++i) {
+			in_dims[i] = in[i];
+			out_dims[i] = in[i] * broadcast[i];
+			reps[i] = (int) broadcast[i];
+		}
+	}
+	BroadcastLayer(const BroadcastLayer& o, bool share) : LayerBase(o.dtype) {
+		std::memcpy(reps, o.reps, sizeof(reps));
+		copy_base(o, share);
+	}
+	LayerBase* clone(bool share) const override {
+		return new BroadcastLayer(*this, share);
+	}
+	void forward(const void* in, size_t N, bool, void* out) override {
+		broadcast_forward<T>((int) in_dims[0], (int) in_dims[1], (int) in_dims[2], reps[0], reps[1], reps[2],
+				checked_int(N, "batch size"), (const T*) in, (T*) out);
+	}
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		if (in_grad)
+			broadcast_backward<T>((int) in_dims[0], (int) in_dims[1], (int) in_dims[2], reps[0], reps[1], reps[2],
+					checked_int(N, "batch size"), (const T*) out_grad, (T*) in_grad);
+	}
+};
+
 struct Timer {
 	hipEvent_t start = nullptr, stop = nullptr;
 };
@@ -1313,6 +1408,60 @@ int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t 
 				(int) vertical_stride, (int) horizontal_stride };
 		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new PoolLayer<float>(dtype, kind, s) :
 				(LayerBase*) new PoolLayer<double>(dtype, kind, s);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_dropout_create(cattle_hip_dtype dtype, size_t volume, double dropout_prob, double epsilon, unsigned long long seed,
+		cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr, "null output pointer");
+		CATTLE_HIP_REQUIRE(volume > 0, "volume must be positive");
+		/* layer/DropoutLayer.hpp:39-41 */
+		CATTLE_HIP_REQUIRE(dropout_prob > 0 && dropout_prob <= 1, "dropout probability must be greater than 0 and no greater than 1");
+		CATTLE_HIP_REQUIRE(epsilon > 0, "epsilon must be greater than 0");
+		LayerBase* l = dtype == CATTLE_HIP_F32 ?
+				(LayerBase*) new DropoutLayer<float>(dtype, volume, (float) dropout_prob, (float) epsilon, seed) :
+				(LayerBase*) new DropoutLayer<double>(dtype, volume, dropout_prob, epsilon, seed);
+		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_reshape_create(cattle_hip_dtype dtype, const size_t input_dims[3], const size_t output_dims[3],
+		cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr && input_dims != nullptr && output_dims != nullptr, "null pointer");
+		const size_t lim = 2147483647u;
+		for (int i = 0; i < 3; ++i)
+			CATTLE_HIP_REQUIRE(input_dims[i] > 0 && output_dims[i] > 0 && input_dims[i] <= lim && output_dims[i] <= lim,
+					"dimensions must be positive and below 2^31");
+		CATTLE_HIP_REQUIRE(input_dims[0] * input_dims[1] <= lim / input_dims[2] &&
+				output_dims[0] * output_dims[1] <= lim / output_dims[2], "volume exceeds 2^31-1");
+		/* layer/ReshapeLayer.hpp:38 */
+		CATTLE_HIP_REQUIRE(input_dims[0] * input_dims[1] * input_dims[2] == output_dims[0] * output_dims[1] * output_dims[2],
+				"the input and output volumes differ");
+		*layer = reinterpret_cast<cattle_hip_layer_t>((LayerBase*) new ReshapeLayer(dtype, input_dims, output_dims));
+	});
+}
+
+int cattle_hip_broadcast_create(cattle_hip_dtype dtype, const size_t input_dims[3], const size_t broadcast[3],
+		cattle_hip_layer_t* layer) {
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(layer != nullptr && input_dims != nullptr && broadcast != nullptr, "null pointer");
+		const size_t lim = 2147483647u;
+		size_t volume = 1;
+		for (int i = 0; i < 3; ++i) {
+			/* layer/BroadcastLayer.hpp:38-39 */
+			CATTLE_HIP_REQUIRE(input_dims[i] > 0 && broadcast[i] > 0, "dimensions and repetitions must be positive");
+			CATTLE_HIP_REQUIRE(input_dims[i] <= lim && broadcast[i] <= lim / input_dims[i] &&
+					input_dims[i] * broadcast[i] <= lim / volume, "output volume exceeds 2^31-1");
+			volume *= input_dims[i] * broadcast[i];
+		}
+		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new BroadcastLayer<float>(dtype, input_dims, broadcast) :
+				(LayerBase*) new BroadcastLayer<double>(dtype, input_dims, broadcast);
 		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
 	});
 }

@@ -1201,6 +1201,185 @@ void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, con
 	check_launch();
 }
 
+/* ---- DropoutLayer (layer/DropoutLayer.hpp:74-96) ------------------------------------------------
+ * y = x * mask, mask = (u <= dropout_prob ? 0 : 1 / (1 - dropout_prob + epsilon)); the backward pass is the
+ * same product on the output gradient. The mask is never stored: both passes regenerate u from the pass key,
+ * which leaves 8 bytes of traffic per element and pass (fp32). The uniform numbers are outputs of splitmix64
+ * (Steele, Lea, Flood 2014) seeded with the key: a double takes the top 53 bits of output i, a float 24 bits of
+ * output i / 2 (bits 63..40 for even i, bits 31..8 for odd i), i being the linear index in the batch tensor. */
+typedef unsigned long long u64;
+
+__host__ __device__ __forceinline__ u64 splitmix64_output(u64 seed, u64 index) {
+	u64 z = seed + (index + 1) * 0x9E3779B97F4A7C15ull;
+	z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+	z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+	return z ^ (z >> 31);
+}
+
+__device__ __forceinline__ float dropout_uniform(u64 key, u64 i, float) {
+	const u64 bits = splitmix64_output(key, i >> 1);
+	return (float) (unsigned) ((i & 1) ? (bits >> 8) & 0xFFFFFFull : bits >> 40) * (1.0f / 16777216.0f);
+}
+__device__ __forceinline__ double dropout_uniform(u64 key, u64 i, double) {
+	return (double) (splitmix64_output(key, i) >> 11) * (1.0 / 9007199254740992.0);
+}
+
+template<typename T, bool VECTOR>
+__global__ __launch_bounds__(256)
+void dropout_kernel(size_t n, u64 key, T prob, T scaling_factor, const T* __restrict__ x, T* __restrict__ y) {
+	constexpr int V = VECTOR ? Pack<T>::V : 1;
+	typedef typename Pack<T>::type vt;
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	const size_t nv = n / V;
+	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+		if constexpr (VECTOR) {
+			const vt a = __builtin_nontemporal_load(reinterpret_cast<const vt*>(x) + i);
+			vt o;
+			#pragma unroll
+			for (int e = 0; e < V; ++e)
+				o[e] = a[e] * (dropout_uniform(key, (u64) i * V + e, T()) <= prob ? (T) 0 : scaling_factor);
+			__builtin_nontemporal_store(o, reinterpret_cast<vt*>(y) + i);
+		} else {
+			y[i] = x[i] * (dropout_uniform(key, (u64) i, T()) <= prob ? (T) 0 : scaling_factor);
+		}
+	}
+	if (VECTOR && blockIdx.x == 0 && threadIdx.x < n - nv * V) {
+		const size_t i = nv * V + threadIdx.x;
+		y[i] = x[i] * (dropout_uniform(key, (u64) i, T()) <= prob ? (T) 0 : scaling_factor);
+	}
+}
+
+u64 dropout_pass_key(u64 seed, u64 pass) {
+	return splitmix64_output(seed, pass);
+}
+
+template<typename T>
+void dropout_apply(size_t n, u64 key, T prob, T eps, const T* x, T* y) {
+	if (n == 0)
+		return;
+	const T scaling_factor = (T) 1 / ((T) 1 - prob + eps);
+	if (aligned16(x) && aligned16(y))
+		dropout_kernel<T, true><<<stream_grid(n / Pack<T>::V), 256, 0, stream()>>>(n, key, prob, scaling_factor, x, y);
+	else
+		dropout_kernel<T, false><<<stream_grid(n), 256, 0, stream()>>>(n, key, prob, scaling_factor, x, y);
+	check_launch();
+}
+
+/* ---- BroadcastLayer (layer/BroadcastLayer.hpp:69-101) --------------------------------------------
+ * forward: out(n, h, w, c) = in(n, h mod H, w mod W, c mod C) on an output of (H bh, W bw, C bc);
+ * backward: the replicas summed rank by rank as the reference does (first rank first, each sum from zero, slices in
+ * order). The sample index is the contiguous one in both tensors. */
+struct BroadcastShape {
+	int H, W, C, bh, bw, bc;
+};
+
+/* Both kernels use the pooling kernels' launch shape: a block covers a range of samples (VN per thread, 16-byte
+ * accesses) and of rows of one (column, channel) pair of the input, so that the divisions run once per block. */
+template<typename T, int VN>
+__global__ __launch_bounds__(256)
+void broadcast_forward_kernel(BroadcastShape s, int N, PoolLaunch pl, const T* __restrict__ x, T* __restrict__ out) {
+	const size_t OH = (size_t) s.H * s.bh, OW = (size_t) s.W * s.bw;
+	unsigned b = blockIdx.x;
+	const int nb = (int) (b % (unsigned) pl.nblks);
+	b /= (unsigned) pl.nblks;
+	const int rb = (int) (b % (unsigned) pl.rblks);
+	b /= (unsigned) pl.rblks;
+	const int w = (int) (b % (unsigned) s.W);
+	const int c = (int) (b / (unsigned) s.W);
+	const int n = (nb * pl.tx + (int) threadIdx.x % pl.tx) * VN;
+	if (n >= N)
+		return;
+	const int row0 = rb * pl.ty * POOL_ROWS + (int) threadIdx.x / pl.tx;
+	#pragma unroll
+	for (int j = 0; j < POOL_ROWS; ++j) {
+		const int h = row0 + j * pl.ty;
+		if (h >= s.H)
+			break;
+		/* an input element is read once and written to all its replicas */
+		T v[VN];
+		pool_load<T, VN>(v, x + n + (size_t) N * ((size_t) h + (size_t) s.H * ((size_t) w + (size_t) s.W * c)));
+		for (int jc = 0; jc < s.bc; ++jc)
+			for (int jw = 0; jw < s.bw; ++jw)
+				for (int jh = 0; jh < s.bh; ++jh)
+					pool_store<T, VN>(out + n + (size_t) N * (((size_t) h + (size_t) jh * s.H) +
+							OH * (((size_t) w + (size_t) jw * s.W) + OW * ((size_t) c + (size_t) jc * s.C))), v);
+	}
+}
+
+template<typename T, int VN>
+__global__ __launch_bounds__(256)
+void broadcast_backward_kernel(BroadcastShape s, int N, PoolLaunch pl, const T* __restrict__ g, T* __restrict__ dx) {
+	const size_t OH = (size_t) s.H * s.bh, OW = (size_t) s.W * s.bw;
+	unsigned b = blockIdx.x;
+	const int nb = (int) (b % (unsigned) pl.nblks);
+	b /= (unsigned) pl.nblks;
+	const int rb = (int) (b % (unsigned) pl.rblks);
+	b /= (unsigned) pl.rblks;
+	const int w = (int) (b % (unsigned) s.W);
+	const int c = (int) (b / (unsigned) s.W);
+	const int n = (nb * pl.tx + (int) threadIdx.x % pl.tx) * VN;
+	if (n >= N)
+		return;
+	const int row0 = rb * pl.ty * POOL_ROWS + (int) threadIdx.x / pl.tx;
+	#pragma unroll
+	for (int j = 0; j < POOL_ROWS; ++j) {
+		const int h = row0 + j * pl.ty;
+		if (h >= s.H)
+			break;
+		/* a rank that is not repeated is not summed over (no "0 +" for it): BroadcastLayer.hpp:86-87 */
+		T sum_c[VN];
+		for (int jc = 0; jc < s.bc; ++jc) {
+			T sum_w[VN];
+			for (int jw = 0; jw < s.bw; ++jw) {
+				T sum_h[VN];
+				for (int jh = 0; jh < s.bh; ++jh) {
+					T e[VN];
+					pool_load<T, VN>(e, g + n + (size_t) N * (((size_t) h + (size_t) jh * s.H) +
+							OH * (((size_t) w + (size_t) jw * s.W) + OW * ((size_t) c + (size_t) jc * s.C))));
+					#pragma unroll
+					for (int v = 0; v < VN; ++v)
+						sum_h[v] = jh == 0 ? (s.bh > 1 ? (T) 0 + e[v] : e[v]) : sum_h[v] + e[v];
+				}
+				#pragma unroll
+				for (int v = 0; v < VN; ++v)
+					sum_w[v] = jw == 0 ? (s.bw > 1 ? (T) 0 + sum_h[v] : sum_h[v]) : sum_w[v] + sum_h[v];
+			}
+			#pragma unroll
+			for (int v = 0; v < VN; ++v)
+				sum_c[v] = jc == 0 ? (s.bc > 1 ? (T) 0 + sum_w[v] : sum_w[v]) : sum_c[v] + sum_w[v];
+		}
+		pool_store<T, VN>(dx + n + (size_t) N * ((size_t) h + (size_t) s.H * ((size_t) w + (size_t) s.W * c)), sum_c);
+	}
+}
+
+template<typename T>
+void broadcast_forward(int H, int W, int C, int bh, int bw, int bc, int N, const T* x, T* out) {
+	const BroadcastShape s = { H, W, C, bh, bw, bc };
+	constexpr int VN = 16 / (int) sizeof(T);
+	if (N % VN == 0 && aligned16(x) && aligned16(out)) {
+		const PoolLaunch pl = pool_launch(N, H, VN);
+		broadcast_forward_kernel<T, VN><<<pool_grid(pl, W, C), 256, 0, stream()>>>(s, N, pl, x, out);
+	} else {
+		const PoolLaunch pl = pool_launch(N, H, 1);
+		broadcast_forward_kernel<T, 1><<<pool_grid(pl, W, C), 256, 0, stream()>>>(s, N, pl, x, out);
+	}
+	check_launch();
+}
+
+template<typename T>
+void broadcast_backward(int H, int W, int C, int bh, int bw, int bc, int N, const T* out_grad, T* in_grad) {
+	const BroadcastShape s = { H, W, C, bh, bw, bc };
+	constexpr int VN = 16 / (int) sizeof(T);
+	if (N % VN == 0 && aligned16(out_grad) && aligned16(in_grad)) {
+		const PoolLaunch pl = pool_launch(N, H, VN);
+		broadcast_backward_kernel<T, VN><<<pool_grid(pl, W, C), 256, 0, stream()>>>(s, N, pl, out_grad, in_grad);
+	} else {
+		const PoolLaunch pl = pool_launch(N, H, 1);
+		broadcast_backward_kernel<T, 1><<<pool_grid(pl, W, C), 256, 0, stream()>>>(s, N, pl, out_grad, in_grad);
+	}
+	check_launch();
+}
+
 #define CATTLE_HIP_INSTANTIATE(T) \
 template void act_forward<T>(int, size_t, T, const T*, T*); \
 template void act_backward<T>(int, size_t, T, const T*, const T*, const T*, T*); \
@@ -1220,6 +1399,9 @@ template void axpy_one<T>(size_t, const T*, T*); \
 template void transpose_matrix<T>(int, int, const T*, T*, bool); \
 template void add_row_vector<T>(int, size_t, const T*, T*); \
 template void accumulate_column_sums<T>(int, size_t, const T*, T*); \
+template void dropout_apply<T>(size_t, unsigned long long, T, T, const T*, T*); \
+template void broadcast_forward<T>(int, int, int, int, int, int, int, const T*, T*); \
+template void broadcast_backward<T>(int, int, int, int, int, int, int, const T*, T*); \
 template void lstm_gates_forward<T>(const LstmActs<T>&, int, size_t, const T*, int, int, const T*, const T*, T*, T*, T*, T*, T*, T*, int, int, \
 		T*, int, int); \
 template void lstm_gates_backward<T>(const LstmActs<T>&, int, size_t, const T*, const T*, int, int, const T*, const T*, const T*, const T*, \

@@ -158,6 +158,25 @@ public:
 				receptor_width, vertical_stride, horizontal_stride, &h));
 		return DeviceLayer(h);
 	}
+	/* layer/DropoutLayer.hpp:33-42; `seed` keys the generator of the masks (give every dropout layer its own) */
+	inline static DeviceLayer dropout(const Dims& dims, Scalar dropout_prob, unsigned long long seed = 0, Scalar epsilon = 1e-5) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_dropout_create(Code<Scalar>::value, dims[0] * dims[1] * dims[2], (double) dropout_prob, (double) epsilon,
+				seed, &h));
+		return DeviceLayer(h, dims, dims);
+	}
+	/* layer/ReshapeLayer.hpp:31-39 */
+	inline static DeviceLayer reshape(const Dims& input_dims, const Dims& output_dims) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_reshape_create(Code<Scalar>::value, input_dims.data(), output_dims.data(), &h));
+		return DeviceLayer(h);
+	}
+	/* layer/BroadcastLayer.hpp:31-40 */
+	inline static DeviceLayer broadcast(const Dims& input_dims, const Dims& broadcast) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_broadcast_create(Code<Scalar>::value, input_dims.data(), broadcast.data(), &h));
+		return DeviceLayer(h);
+	}
 	inline DeviceLayer(DeviceLayer&& other) : handle(other.handle), in_dims(other.in_dims), out_dims(other.out_dims),
 			cached_in(std::move(other.cached_in)), cached_out(std::move(other.cached_out)),
 			params_per_column(other.params_per_column) {

@@ -140,6 +140,25 @@ int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t 
 		size_t receptor_height, size_t receptor_width, size_t vertical_stride, size_t horizontal_stride,
 		cattle_hip_layer_t* layer);
 
+/* DropoutLayer<Scalar,Rank>(dims, dropout_prob, epsilon) - layer/DropoutLayer.hpp:33-42, passes :74-96: a training
+ * pass multiplies by the inverted-dropout mask (0 where u <= dropout_prob, else 1 / (1 - dropout_prob + epsilon)), an
+ * inference pass hands the input through, the backward pass multiplies the gradient by the mask of the last training
+ * pass. The reference draws u from Eigen's generator; here u comes from splitmix64 keyed by `seed` and the number of
+ * the training pass (bits per element as described in csrc/pointwise_kernels.hip), so runs are reproducible and the
+ * mask need not be stored. Layers that must drop independently need different seeds. volume = dims.get_volume(). */
+int cattle_hip_dropout_create(cattle_hip_dtype dtype, size_t volume, double dropout_prob, double epsilon, unsigned long long seed,
+		cattle_hip_layer_t* layer);
+
+/* ReshapeLayer<Scalar,Rank>(input_dims, output_dims) - layer/ReshapeLayer.hpp:31-39, passes :77-90. Dimensions as
+ * (height, width, channels); lower ranks pad with ones. */
+int cattle_hip_reshape_create(cattle_hip_dtype dtype, const size_t input_dims[3], const size_t output_dims[3],
+		cattle_hip_layer_t* layer);
+
+/* BroadcastLayer<Scalar,Rank>(input_dims, broadcast) - layer/BroadcastLayer.hpp:31-40, passes :69-101: the input
+ * repeated broadcast[i] times along rank i; the backward pass sums the replicas rank by rank. */
+int cattle_hip_broadcast_create(cattle_hip_dtype dtype, const size_t input_dims[3], const size_t broadcast[3],
+		cattle_hip_layer_t* layer);
+
 /* ---- the cattle::Layer contract (core/Layer.hpp:47-137) ------------------------------------- */
 
 /* Layer::clone() (:47) when share_params == 0: deep copy including parameter values and gradients;

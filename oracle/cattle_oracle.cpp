@@ -23,6 +23,10 @@
  *   losses              pinned: torch float64 cross_entropy / mse / l1 / binary_cross_entropy / nll / kl_div /
  *                       multi_margin_loss (epsilon 0) with autograd for the gradients, hand-worked rows at the
  *                       hinge thresholds and with the epsilons, central differences of each loss against its gradient.
+ *   dropout             pinned: the splitmix64 stream against its published outputs, the uniforms by their moments and
+ *                       bin counts, the mask rule on hand-worked values. The reference's own random stream (Eigen's)
+ *                       cannot be restated: which elements are dropped is "parity unpinned", by construction.
+ *   broadcast           pinned: numpy.tile forward, torch autograd of a tiled tensor and the adjoint identity backward.
  *   other optimizers    pinned: torch's SGD (momentum, Nesterov), Adagrad, RMSprop, Adadelta and Adamax where the
  *                       recurrences coincide; first-step closed forms and the running-maximum property for
  *                       Nadam and AMSGrad, whose reference formulas differ from torch's.
@@ -915,6 +919,95 @@ int loss_d_function(int kind, i64 N, i64 Ts, i64 V, T eps, T scale, const T* out
 	return 0;
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * DropoutLayer (layer/DropoutLayer.hpp:74-96). The reference draws its uniform numbers from Eigen's
+ * generator (in.random(), :79), whose stream cannot be restated; the mask is a function of those
+ * numbers, mask = (u <= dropout_prob ? 0 : 1 / (1 - dropout_prob + epsilon)), and both passes multiply
+ * by it. Here the numbers come from splitmix64 (Steele, Lea, Flood 2014; Vigna's public-domain
+ * splitmix64.c): pass number q of a layer seeded with s uses key = the q-th output of the stream seeded
+ * with s, and the elements of the batch tensor (linear index i, sample index fastest) take the outputs of the
+ * stream seeded with that key: a double the top 53 bits of output i, a float 24 bits of output i / 2 (bits 63..40
+ * for even i, bits 31..8 for odd i), scaled to [0, 1).
+ * ------------------------------------------------------------------------------------------- */
+typedef unsigned long long u64;
+
+u64 splitmix64_output(u64 seed, u64 index) {
+	u64 z = seed + (index + 1) * 0x9E3779B97F4A7C15ull;
+	z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+	z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+	return z ^ (z >> 31);
+}
+
+/* float: one output serves two elements, bits 63..40 the even one, bits 31..8 the odd one */
+float dropout_uniform(u64 key, u64 i, float) {
+	const u64 bits = splitmix64_output(key, i >> 1);
+	return (float) ((i & 1) ? (bits >> 8) & 0xFFFFFFull : bits >> 40) * (1.0f / 16777216.0f);
+}
+double dropout_uniform(u64 key, u64 i, double) {
+	return (double) (splitmix64_output(key, i) >> 11) * (1.0 / 9007199254740992.0);
+}
+
+template<typename T>
+int dropout_uniforms(u64 seed, u64 pass, i64 n, T* u) {
+	const u64 key = splitmix64_output(seed, pass);
+	for (i64 i = 0; i < n; ++i)
+		u[i] = dropout_uniform(key, (u64) i, T());
+	return 0;
+}
+
+/* y = x * mask(u): the forward pass on the input, the backward pass on the output gradient (:82, :95) */
+template<typename T>
+int dropout_apply(i64 n, T prob, T eps, const T* u, const T* x, T* y) {
+	const T scaling_factor = (T) 1 / (1 - prob + eps);
+	for (i64 i = 0; i < n; ++i)
+		y[i] = x[i] * (T) (u[i] <= prob ? 0 : scaling_factor);
+	return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * BroadcastLayer (layer/BroadcastLayer.hpp:69-101): the input repeated bh x bw x bc times along its three
+ * ranks (Eigen's broadcast: out(n, h, w, c) = in(n, h mod H, w mod W, c mod C)); backward sums the
+ * replicas rank by rank, first rank first, each sum starting from zero and taking the slices in order.
+ * ------------------------------------------------------------------------------------------- */
+template<typename T>
+int broadcast_forward(i64 N, i64 H, i64 W, i64 C, i64 bh, i64 bw, i64 bc, const T* x, T* out) {
+	const i64 OH = H * bh, OW = W * bw, OC = C * bc;
+	for (i64 c = 0; c < OC; ++c)
+		for (i64 w = 0; w < OW; ++w)
+			for (i64 h = 0; h < OH; ++h)
+				for (i64 n = 0; n < N; ++n)
+					out[n + N * (h + OH * (w + OW * c))] = x[n + N * ((h % H) + H * ((w % W) + W * (c % C)))];
+	return 0;
+}
+
+template<typename T>
+int broadcast_backward(i64 N, i64 H, i64 W, i64 C, i64 bh, i64 bw, i64 bc, const T* out_grad, T* in_grad) {
+	i64 dims[4] = { N, H * bh, W * bw, C * bc };           /* of the tensor being reduced */
+	const i64 in_dims[4] = { N, H, W, C }, reps[4] = { 1, bh, bw, bc };
+	std::vector<T> cur(out_grad, out_grad + dims[0] * dims[1] * dims[2] * dims[3]);
+	for (int r = 1; r < 4; ++r) {
+		if (reps[r] <= 1)
+			continue;
+		i64 nd[4] = { dims[0], dims[1], dims[2], dims[3] };
+		nd[r] = in_dims[r];
+		std::vector<T> work((size_t) (nd[0] * nd[1] * nd[2] * nd[3]), (T) 0);
+		for (i64 j = 0; j < reps[r]; ++j)
+			for (i64 c = 0; c < nd[3]; ++c)
+				for (i64 w = 0; w < nd[2]; ++w)
+					for (i64 h = 0; h < nd[1]; ++h)
+						for (i64 n = 0; n < nd[0]; ++n) {
+							i64 src[4] = { n, h, w, c };
+							src[r] += j * in_dims[r];
+							work[n + nd[0] * (h + nd[1] * (w + nd[2] * c))] +=
+									cur[src[0] + dims[0] * (src[1] + dims[1] * (src[2] + dims[2] * src[3]))];
+						}
+		cur.swap(work);
+		dims[r] = nd[r];
+	}
+	std::copy(cur.begin(), cur.end(), in_grad);
+	return 0;
+}
+
 /* optimizer/VanillaSGDOptimizer.hpp:38-43 */
 template<typename T>
 int sgd_update(i64 n, T lr, const T* grad, T* values) {
@@ -1061,6 +1154,14 @@ extern "C" int oracle_transconv_forward_##SFX(CONV_ARGS, const T* x, const T* w,
 extern "C" int oracle_transconv_backward_##SFX(CONV_ARGS, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad, \
 		T* in_grad) { TransGeom g = { N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh, 0, 0, 0, 0, 0, 0 }; \
 	return transconv_backward<T>(g, x, w, out_grad, wgrad, bgrad, in_grad); } \
+extern "C" int oracle_dropout_uniforms_##SFX(unsigned long long seed, unsigned long long pass, i64 n, T* u) { \
+	return dropout_uniforms<T>(seed, pass, n, u); } \
+extern "C" int oracle_dropout_apply_##SFX(i64 n, double prob, double eps, const T* u, const T* x, T* y) { \
+	return dropout_apply<T>(n, (T) prob, (T) eps, u, x, y); } \
+extern "C" int oracle_broadcast_forward_##SFX(i64 N, i64 H, i64 W, i64 C, i64 bh, i64 bw, i64 bc, const T* x, T* out) { \
+	return broadcast_forward<T>(N, H, W, C, bh, bw, bc, x, out); } \
+extern "C" int oracle_broadcast_backward_##SFX(i64 N, i64 H, i64 W, i64 C, i64 bh, i64 bw, i64 bc, const T* g, T* dx) { \
+	return broadcast_backward<T>(N, H, W, C, bh, bw, bc, g, dx); } \
 extern "C" int oracle_loss_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double eps, const T* out, const T* obj, T* losses) { \
 	return loss_function<T>(kind, N, Ts, V, (T) eps, out, obj, losses); } \
 extern "C" int oracle_loss_d_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double eps, double scale, const T* out, \
@@ -1074,6 +1175,10 @@ extern "C" int oracle_adam_update_##SFX(i64 n, double lr, double d1, double d2, 
 
 ORACLE_INSTANTIATE(float, f32)
 ORACLE_INSTANTIATE(double, f64)
+
+extern "C" unsigned long long oracle_splitmix64_output(unsigned long long seed, unsigned long long index) {
+	return splitmix64_output(seed, index);
+}
 
 extern "C" int oracle_num_threads(void) {
 #ifdef _OPENMP

@@ -326,6 +326,46 @@ def meanpool_backward(x_shape, out_grad, RH=2, RW=2, sv=2, sh=2):
     return dx
 
 
+def splitmix64_output(seed, index):
+    fn = lib().oracle_splitmix64_output
+    fn.restype = ctypes.c_ulonglong
+    return int(fn(ctypes.c_ulonglong(seed), ctypes.c_ulonglong(index)))
+
+
+def dropout_uniforms(seed, pass_index, shape, dtype):
+    """The uniform numbers of training pass `pass_index` of a dropout layer seeded with `seed`, in the shape of the batch."""
+    u = np.empty(shape, dtype=dtype, order="F")
+    _call("dropout_uniforms", np.dtype(dtype), ctypes.c_ulonglong(seed), ctypes.c_ulonglong(pass_index), *_ll(u.size), _p(u))
+    return u
+
+
+def dropout_apply(x, u, prob, eps=1e-5):
+    """x times the dropout mask of the uniforms u (layer/DropoutLayer.hpp:78-82, :95)."""
+    dt = x.dtype
+    x, u = _f(x, dt), _f(u, dt)
+    y = np.empty(x.shape, dtype=dt, order="F")
+    _call("dropout_apply", dt, *_ll(x.size), ctypes.c_double(prob), ctypes.c_double(eps), _p(u), _p(x), _p(y))
+    return y
+
+
+def broadcast_forward(x, bh, bw, bc):
+    dt = x.dtype
+    x = _f(x, dt)
+    N, H, W, C = x.shape
+    out = np.empty((N, H * bh, W * bw, C * bc), dtype=dt, order="F")
+    _call("broadcast_forward", dt, *_ll(N, H, W, C, bh, bw, bc), _p(x), _p(out))
+    return out
+
+
+def broadcast_backward(x_shape, out_grad, bh, bw, bc):
+    dt = out_grad.dtype
+    N, H, W, C = x_shape
+    g = _f(out_grad, dt)
+    dx = np.empty((N, H, W, C), dtype=dt, order="F")
+    _call("broadcast_backward", dt, *_ll(N, H, W, C, bh, bw, bc), _p(g), _p(dx))
+    return dx
+
+
 LOSS_KINDS = {"squared": 0, "softmax_cross_entropy": 1, "absolute": 2, "binary_cross_entropy": 3, "cross_entropy": 4,
               "kullback_leibler": 5, "hinge": 6, "squared_hinge": 7, "multi_label_hinge": 8,
               "squared_multi_label_hinge": 9, "multi_label_log": 10}

@@ -126,6 +126,23 @@ static void run(const std::string& tag) {
 		record_final<Scalar>(tag + ".mlp", net);
 	}
 	{
+		/* the data-movement layers of the reference's example networks: reshape -> broadcast -> dropout */
+		Lcg g(14);
+		const std::size_t batch = 5;
+		std::vector<DL> layers;
+		layers.push_back(DL::reshape(Dims{ { 12, 1, 1 } }, Dims{ { 3, 2, 2 } }));
+		layers.push_back(DL::broadcast(layers.back().get_output_dims(), Dims{ { 2, 1, 3 } }));
+		layers.push_back(DL::dropout(layers.back().get_output_dims(), (Scalar) 0.4, 321));
+		DeviceFeedforwardNetwork<Scalar> net(std::move(layers), false);
+		std::vector<Scalar> x = random_values<Scalar>(batch * 12, g, 1.0), go = random_values<Scalar>(batch * 72, g, 1.0);
+		DT xd(typename DT::Dims{ { batch, 12, 1, 1 } }, x.data()), gd(typename DT::Dims{ { batch, 6, 2, 6 } }, go.data());
+		record(tag + ".move.x", sizeof(Scalar), { batch, 12 }, x.data());
+		record(tag + ".move.go", sizeof(Scalar), { batch, 6, 2, 6 }, go.data());
+		record(tag + ".move.out", sizeof(Scalar), { batch, 6, 2, 6 }, net.propagate(xd, true).to_host().data());
+		record(tag + ".move.dx", sizeof(Scalar), { batch, 12 }, net.backpropagate(gd).to_host().data());
+		record(tag + ".move.infer", sizeof(Scalar), { batch, 6, 2, 6 }, net.propagate(xd, false).to_host().data());
+	}
+	{
 		/* another loss of the loss/ directory, wrapped as NegatedLoss wraps it */
 		Lcg g(13);
 		const std::size_t batch = 9, classes = 7;

@@ -63,6 +63,19 @@ def out_shape(net):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tag,dtype", [("f32", np.float32), ("f64", np.float64)])
+def test_reshape_broadcast_dropout_stack(records, tag, dtype):
+    x, go = records[tag + ".move.x"], records[tag + ".move.go"]
+    assert x.dtype == dtype
+    tiled = oracle.broadcast_forward(x.reshape((5, 3, 2, 2), order="F"), 2, 1, 3)
+    u = oracle.dropout_uniforms(321, 0, tiled.shape, dtype)
+    assert np.array_equal(records[tag + ".move.out"], oracle.dropout_apply(tiled, u, 0.4, 1e-5))
+    back = oracle.broadcast_backward((5, 3, 2, 2), oracle.dropout_apply(go, u, 0.4, 1e-5), 2, 1, 3)
+    assert np.array_equal(records[tag + ".move.dx"], back.reshape((5, 12), order="F"))
+    assert np.array_equal(records[tag + ".move.infer"], tiled)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-10)])
 def test_device_loss_of_another_kind_negated(records, tag, tol):
     out, obj = np.asarray(records[tag + ".loss.out"], np.float64), np.asarray(records[tag + ".loss.obj"], np.float64)
