@@ -1209,6 +1209,8 @@ void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, con
  * output i / 2 (bits 63..40 for even i, bits 31..8 for odd i), i being the linear index in the batch tensor. */
 typedef unsigned long long u64;
 
+namespace {
+
 __host__ __device__ __forceinline__ u64 splitmix64_output(u64 seed, u64 index) {
 	u64 z = seed + (index + 1) * 0x9E3779B97F4A7C15ull;
 	z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -1249,6 +1251,8 @@ void dropout_kernel(size_t n, u64 key, T prob, T scaling_factor, const T* __rest
 	}
 }
 
+} /* namespace */
+
 u64 dropout_pass_key(u64 seed, u64 pass) {
 	return splitmix64_output(seed, pass);
 }
@@ -1269,6 +1273,8 @@ void dropout_apply(size_t n, u64 key, T prob, T eps, const T* x, T* y) {
  * forward: out(n, h, w, c) = in(n, h mod H, w mod W, c mod C) on an output of (H bh, W bw, C bc);
  * backward: the replicas summed rank by rank as the reference does (first rank first, each sum from zero, slices in
  * order). The sample index is the contiguous one in both tensors. */
+namespace {
+
 struct BroadcastShape {
 	int H, W, C, bh, bw, bc;
 };
@@ -1351,6 +1357,8 @@ void broadcast_backward_kernel(BroadcastShape s, int N, PoolLaunch pl, const T* 
 		pool_store<T, VN>(dx + n + (size_t) N * ((size_t) h + (size_t) s.H * ((size_t) w + (size_t) s.W * c)), sum_c);
 	}
 }
+
+} /* namespace */
 
 template<typename T>
 void broadcast_forward(int H, int W, int C, int bh, int bw, int bc, int N, const T* x, T* out) {
