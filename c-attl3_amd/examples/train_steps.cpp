@@ -1,9 +1,10 @@
 /*
  * train_steps.cpp — whole training steps on the device from C++, through cattle_hip/DeviceNet.hpp: the two
- * feed-forward configurations of the benchmark definition, built layer by layer as a C-ATTL3 user would build
- * them, trained with DeviceFeedforwardNetwork::train_batch_sgd / train_batch_adam (one batch of
- * SGDOptimizer::_train, optimizer/SGDOptimizer.hpp:44-70: propagate, loss, gradient / batch size, backpropagate,
- * update, reset), and timed. Prints one JSON line.
+ * feed-forward configurations of the benchmark definition and the network of the reference's own example
+ * (examples/cifar_convnet.cpp:24-41), built layer by layer as a C-ATTL3 user would build them, trained with
+ * DeviceFeedforwardNetwork::train_batch* (one batch of SGDOptimizer::_train, optimizer/SGDOptimizer.hpp:44-70:
+ * propagate, loss, gradient / batch size, backpropagate, update, reset) on synthetic data, and timed. Prints one
+ * JSON line.
  *
  *   g++ -std=c++11 -O2 -I include -I c-attl3_amd/include c-attl3_amd/examples/train_steps.cpp \
  *       -L c-attl3_amd -lcattle_hip -Wl,-rpath,'$ORIGIN/..' -o c-attl3_amd/examples/train_steps
@@ -85,7 +86,7 @@ int main(int argc, char** argv) {
 		check(cattle_hip_init(0));
 		DeviceLoss<Scalar> loss(CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY);
 		Lcg g(2);
-		double mlp_ms, conv_ms;
+		double mlp_ms, conv_ms, cifar_ms;
 		{
 			/* MLP 784-512-256-10 with ReLU, batch 256, vanilla SGD */
 			const std::size_t batch = 256;
@@ -119,9 +120,38 @@ int main(int argc, char** argv) {
 			DT xd(DT::Dims{ { batch, 32, 32, 3 } }, x.data()), yd(DT::Dims{ { batch, 10, 1, 1 } }, y.data());
 			conv_ms = time_steps(steps, warmup, [&](std::size_t t) { net.train_batch_adam(xd, yd, loss, t); });
 		}
-		std::printf("{\"driver\": \"C++ (cattle_hip/DeviceNet.hpp), train_batch_sgd / train_batch_adam incl. the per-batch loss read-back\", "
-				"\"steps\": %zu, \"warmup\": %zu, \"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, \"convnet_32x32x3_batch128_adam_ms\": %.4f}\n",
-				steps, warmup, mlp_ms, conv_ms);
+		{
+			/* examples/cifar_convnet.cpp:24-41: conv 3x3x8 - ReLU - max pool - conv 3x3x8 - ReLU - max pool - dropout .25 -
+			 * dense 50 - ReLU - dropout .5 - dense 10 - softmax; CrossEntropyLoss; NadamOptimizer, batch 200 */
+			const std::size_t batch = 200;
+			std::vector<DL> layers;
+			layers.push_back(DL::conv(Dims{ { 32, 32, 3 } }, 8));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+			layers.push_back(DL::pool(CATTLE_HIP_POOL_MAX, layers.back().get_output_dims()));
+			layers.push_back(DL::conv(layers.back().get_output_dims(), 8));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+			layers.push_back(DL::pool(CATTLE_HIP_POOL_MAX, layers.back().get_output_dims()));
+			layers.push_back(DL::dropout(layers.back().get_output_dims(), (Scalar) .25, 1));
+			layers.push_back(DL::dense(layers.back().get_output_dims(), 50));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
+			layers.push_back(DL::dropout(layers.back().get_output_dims(), (Scalar) .5, 2));
+			layers.push_back(DL::dense(layers.back().get_output_dims(), 10));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_SOFTMAX, layers.back().get_output_dims(), (Scalar) 1e-5));
+			DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
+			init_weights(net, g);
+			std::vector<Scalar> x = random_values(batch * 32 * 32 * 3, g, 0.5), y = one_hot(batch, 10, g);
+			for (std::size_t i = 0; i < x.size(); ++i)
+				x[i] += (Scalar) 0.5;                                   /* pixel values in [0, 1) */
+			DT xd(DT::Dims{ { batch, 32, 32, 3 } }, x.data()), yd(DT::Dims{ { batch, 10, 1, 1 } }, y.data());
+			DeviceLoss<Scalar> cross_entropy(CATTLE_HIP_LOSS_CROSS_ENTROPY);
+			const double nadam[4] = { 1e-3, 1e-1, 1e-3, 1e-5 };        /* optimizer/NadamOptimizer.hpp:39-41 */
+			cifar_ms = time_steps(steps, warmup, [&](std::size_t t) {
+				net.train_batch(xd, yd, cross_entropy, CATTLE_HIP_OPT_NADAM, nadam, 0, t);
+			});
+		}
+		std::printf("{\"driver\": \"C++ (cattle_hip/DeviceNet.hpp), train_batch* incl. the per-batch loss read-back\", "
+				"\"steps\": %zu, \"warmup\": %zu, \"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, \"convnet_32x32x3_batch128_adam_ms\": %.4f, "
+				"\"reference_cifar_example_batch200_nadam_ms\": %.4f}\n", steps, warmup, mlp_ms, conv_ms, cifar_ms);
 	} catch (const std::exception& e) {
 		std::fprintf(stderr, "train_steps: %s\n", e.what());
 		return 1;

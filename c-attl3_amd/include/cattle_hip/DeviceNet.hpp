@@ -538,6 +538,13 @@ public:
 	 * Adam update: propagate, loss, gradient / batch size, backpropagate, update, reset. Returns the
 	 * sum of the per-sample losses of the batch.
 	 */
+	/** The same with any of the optimizers; `hyper` holds the optimizer's constructor arguments (include/cattle_hip.h). */
+	inline Scalar train_batch(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj, const DeviceLoss<Scalar>& loss,
+			cattle_hip_optimizer optimizer, const double (&hyper)[4], std::size_t epoch, std::size_t timestep) {
+		const Scalar total = forward_backward(input, obj, loss);
+		optimizer_step(optimizer, hyper, epoch, timestep);
+		return total;
+	}
 	inline Scalar train_batch_sgd(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj,
 			const DeviceLoss<Scalar>& loss, Scalar learning_rate) {
 		const Scalar total = forward_backward(input, obj, loss);

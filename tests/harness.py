@@ -131,12 +131,17 @@ class OracleActivation(OracleLayer):
 
     def pass_forward(self, x, training):
         self.x = np.asarray(x, self.dtype)
-        self.y = oracle.act_forward(self.kind, self.x, self.p)
+        if self.kind == "softmax":          # layer/activation/SoftmaxActivationLayer.hpp:49-78; the parameter is its epsilon
+            self.y = oracle.softmax_forward(self.x, self.p)
+        else:
+            self.y = oracle.act_forward(self.kind, self.x, self.p)
         return self.y
 
     def pass_back(self, g):
         if self.input_layer:
             return None
+        if self.kind == "softmax":
+            return oracle.softmax_backward(self.y, np.asarray(g, self.dtype))
         return oracle.act_backward(self.kind, self.x, self.y, np.asarray(g, self.dtype), self.p)
 
 
@@ -200,6 +205,34 @@ class OracleMaxPool(OracleLayer):
         return oracle.maxpool_backward(self.x_shape, np.asarray(g, self.dtype), self.inds, *self.g)
 
 
+class OracleDropout(OracleLayer):
+    """layer/DropoutLayer.hpp:74-96 with the uniform numbers of the device layer: they are drawn in `mask_dtype`, the
+    scalar type of the device layer this one is the twin of, whatever type the values are computed in."""
+
+    def __init__(self, dtype, dims, prob, seed=0, epsilon=1e-5, mask_dtype=None):
+        OracleLayer.__init__(self, dtype)
+        self.dims, self.seed, self.passes, self.mask = tuple(dims), seed, 0, None
+        mt = np.dtype(mask_dtype or dtype).type
+        self.mask_dtype, self.prob = np.dtype(mask_dtype or dtype), mt(prob)
+        self.scale = mt(1) / (mt(1) - mt(prob) + mt(epsilon))
+
+    def get_output_dims(self):
+        return self.dims
+
+    def pass_forward(self, x, training):
+        if not training:
+            return x
+        u = oracle.dropout_uniforms(self.seed, self.passes, x.shape, self.mask_dtype)
+        self.passes += 1
+        self.mask = np.where(u <= self.prob, self.mask_dtype.type(0), self.scale).astype(self.dtype)
+        return np.asfortranarray(x * self.mask)
+
+    def pass_back(self, g):
+        if self.input_layer:
+            return None
+        return np.asfortranarray(np.asarray(g, self.dtype) * self.mask)
+
+
 class OracleBackend(object):
     name = "oracle"
 
@@ -220,6 +253,9 @@ class OracleBackend(object):
 
     def maxpool(self, dims):
         return OracleMaxPool(self.dtype, dims)
+
+    def dropout(self, dims, prob, seed, mask_dtype=None):
+        return OracleDropout(self.dtype, dims, prob, seed, mask_dtype=mask_dtype)
 
 
 class HipBackend(object):
@@ -243,6 +279,9 @@ class HipBackend(object):
 
     def maxpool(self, dims):
         return self.ch.MaxPoolLayer(self.dtype, dims)
+
+    def dropout(self, dims, prob, seed, mask_dtype=None):
+        return self.ch.DropoutLayer(self.dtype, dims, prob, seed=seed)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -352,6 +391,17 @@ def build_convnet(backend):
     return FeedforwardNet([b.conv((32, 32, 3), 32), b.act("relu", (32, 32, 32)), b.maxpool((32, 32, 32)),
                            b.conv((16, 16, 32), 64), b.batchnorm((16, 16, 64)), b.act("relu", (16, 16, 64)),
                            b.maxpool((16, 16, 64)), b.dense((8, 8, 64), 10)])
+
+
+def build_cifar_example(backend, mask_dtype=None):
+    """The network of the reference's examples/cifar_convnet.cpp:24-36: conv 3x3x8 p1 -> ReLU -> maxpool -> conv 3x3x8 p1 ->
+    ReLU -> maxpool -> dropout .25 -> dense 50 -> ReLU -> dropout .5 -> dense 10 -> softmax."""
+    b = backend
+    return FeedforwardNet([b.conv((32, 32, 3), 8), b.act("relu", (32, 32, 8)), b.maxpool((32, 32, 8)),
+                           b.conv((16, 16, 8), 8), b.act("relu", (16, 16, 8)), b.maxpool((16, 16, 8)),
+                           b.dropout((8, 8, 8), 0.25, 101, mask_dtype), b.dense((8, 8, 8), 50), b.act("relu", (50, 1, 1)),
+                           b.dropout((50, 1, 1), 0.5, 102, mask_dtype), b.dense((50, 1, 1), 10),
+                           b.act("softmax", (10, 1, 1), 1e-5)])
 
 
 def init_kernel_weights(net, seed, dtype):

@@ -330,6 +330,50 @@ def test_whole_training_steps_stay_on_the_device(config):
         assert np.allclose(pd.get_values(), ps.get_values(), rtol=1e-4, atol=1e-5)
 
 
+def test_the_reference_cifar_example_network_trains_on_the_device():
+    """examples/cifar_convnet.cpp:24-41 (two conv / ReLU / max-pool stages, dropout, two dense layers, softmax,
+    CrossEntropyLoss, NadamOptimizer with its default hyper-parameters) on CIFAR-shaped synthetic data: four batches of
+    SGDOptimizer::_train with every tensor on the device, against the same network built from the oracle's layers in
+    float64 with the oracle's loss and optimizer. The dropout masks are those of the float32 device layers."""
+    import harness as hn
+    dt, N = np.float32, 200
+    gen = hp.rng(0xC0FFEE30)
+    x = np.asfortranarray(gen.uniform(0, 1, (N, 32, 32, 3)).astype(dt))
+    obj = _one_hot_labels(gen, N, (10, 1, 1), dt)
+    dev = hn.build_cifar_example(hn.HipBackend(dt))
+    ref = hn.build_cifar_example(hn.OracleBackend(np.float64), mask_dtype=dt)
+    hn.init_kernel_weights(dev, 30, dt)
+    for pd, pr in zip(dev.params(), ref.params()):
+        pr.set_values(np.asarray(pd.get_values(), np.float64))
+    hyper = [1e-3, 1e-1, 1e-3, 1e-5]                        # NadamOptimizer's defaults (optimizer/NadamOptimizer.hpp:39-41)
+    hyper32 = [float(np.float32(h)) for h in hyper]          # as the float network sees them
+    dev_params = ch.ParameterList([p for p in dev.params() if p.are_optimizable()])
+    states = [[np.zeros_like(p.get_values()) for _ in range(3)] for p in ref.params()]
+    xd, yd = ch.DeviceTensor.from_host(x), ch.DeviceTensor.from_host(obj)
+    x64, y64 = np.asarray(x, np.float64), np.asarray(obj, np.float64)
+    losses = []
+    for step in range(4):
+        out = dev.propagate(xd, True)
+        loss_dev = ch.loss_function("cross_entropy", out, yd)
+        dev.backpropagate(ch.loss_d_function("cross_entropy", out, yd, scale=1.0 / N))
+        dev_params.optimizer_step("nadam", hyper, 0, step)
+        out_r = ref.propagate(x64, True)
+        loss_ref = oracle.loss_function("cross_entropy", out_r, y64, eps=float(np.float32(1e-5)))
+        ref.backpropagate(oracle.loss_d_function("cross_entropy", out_r, y64, eps=float(np.float32(1e-5)), scale=float(np.float32(1.0 / N))))
+        for p, st in zip(ref.params(), states):
+            new, st[:] = oracle.optimizer_update("nadam", p.get_values(), p.get_grad(), st, hyper32, 0, step)
+            p.set_values(new)
+            p.reset_grad()
+        assert hp.rel_err(loss_dev, loss_ref) < 1e-3, step
+        losses.append(float(loss_ref.sum()))
+    for pd, pr in zip(dev.params(), ref.params()):
+        assert np.allclose(pd.get_values(), pr.get_values(), rtol=1e-3, atol=2e-5)
+    # inference: dropout hands its input through, the softmax outputs are probabilities
+    probs = dev.propagate(xd, False).to_host()
+    assert hp.rel_err(probs, ref.propagate(x64, False)) < 1e-3
+    assert np.allclose(probs.reshape((N, 10), order="F").sum(axis=1), 1.0, atol=1e-4)
+
+
 ALL_OPTIMIZERS = [("vanilla_sgd", [1e-2]), ("momentum_sgd", [1e-2, 1e-3, 0.9]), ("nesterov_momentum_sgd", [1e-2, 1e-3, 0.9]),
                   ("adagrad", [1e-2, 1e-5]), ("rmsprop", [1e-3, 1e-1, 1e-5]), ("adadelta", [5e-2, 1e-5]),
                   ("adam", [1e-3, 1e-1, 1e-3, 1e-5]), ("adamax", [1e-3, 1e-1, 1e-3, 1e-5]), ("nadam", [1e-3, 1e-1, 1e-3, 1e-5]),
