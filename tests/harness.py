@@ -233,6 +233,25 @@ class OracleDropout(OracleLayer):
         return np.asfortranarray(np.asarray(g, self.dtype) * self.mask)
 
 
+class OracleReshape(OracleLayer):
+    """layer/ReshapeLayer.hpp:77-90"""
+
+    def __init__(self, dtype, input_dims, output_dims):
+        OracleLayer.__init__(self, dtype)
+        self.in_dims, self.out_dims = tuple(input_dims), tuple(output_dims)
+
+    def get_output_dims(self):
+        return self.out_dims
+
+    def pass_forward(self, x, training):
+        return np.asfortranarray(x.reshape((x.shape[0],) + self.out_dims, order="F"))
+
+    def pass_back(self, g):
+        if self.input_layer:
+            return None
+        return np.asfortranarray(g.reshape((g.shape[0],) + self.in_dims, order="F"))
+
+
 class OracleBackend(object):
     name = "oracle"
 
@@ -256,6 +275,9 @@ class OracleBackend(object):
 
     def dropout(self, dims, prob, seed, mask_dtype=None):
         return OracleDropout(self.dtype, dims, prob, seed, mask_dtype=mask_dtype)
+
+    def reshape(self, input_dims, output_dims):
+        return OracleReshape(self.dtype, input_dims, output_dims)
 
 
 class HipBackend(object):
@@ -282,6 +304,9 @@ class HipBackend(object):
 
     def dropout(self, dims, prob, seed, mask_dtype=None):
         return self.ch.DropoutLayer(self.dtype, dims, prob, seed=seed)
+
+    def reshape(self, input_dims, output_dims):
+        return self.ch.ReshapeLayer(self.dtype, input_dims, output_dims)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -402,6 +427,21 @@ def build_cifar_example(backend, mask_dtype=None):
                            b.dropout((8, 8, 8), 0.25, 101, mask_dtype), b.dense((8, 8, 8), 50), b.act("relu", (50, 1, 1)),
                            b.dropout((50, 1, 1), 0.5, 102, mask_dtype), b.dense((50, 1, 1), 10),
                            b.act("softmax", (10, 1, 1), 1e-5)])
+
+
+def build_gan_example(backend, mask_dtype=None):
+    """The two networks of the reference's examples/mnist_gan.cpp:34-58: the generator (dense 100 -> 256 -> 512 -> 1024 ->
+    784 with leaky ReLUs, tanh, reshape to 28x28x1) and the discriminator (dense 784 -> 1024 -> 512 -> 256 -> 1 with leaky
+    ReLUs and dropout, sigmoid), which is not foremost: it sits on top of the generator in the StackedNeuralNetwork."""
+    b, a, d = backend, 0.2, 0.3
+    gen = FeedforwardNet([b.dense((1, 1, 100), 256), b.act("leaky_relu", (256, 1, 1), a), b.dense((256, 1, 1), 512),
+                          b.act("leaky_relu", (512, 1, 1), a), b.dense((512, 1, 1), 1024), b.act("leaky_relu", (1024, 1, 1), a),
+                          b.dense((1024, 1, 1), 784), b.act("tanh", (784, 1, 1)), b.reshape((784, 1, 1), (28, 28, 1))])
+    disc = FeedforwardNet([b.dense((28, 28, 1), 1024), b.act("leaky_relu", (1024, 1, 1), a), b.dropout((1024, 1, 1), d, 201, mask_dtype),
+                           b.dense((1024, 1, 1), 512), b.act("leaky_relu", (512, 1, 1), a), b.dropout((512, 1, 1), d, 202, mask_dtype),
+                           b.dense((512, 1, 1), 256), b.act("leaky_relu", (256, 1, 1), a), b.dropout((256, 1, 1), d, 203, mask_dtype),
+                           b.dense((256, 1, 1), 1), b.act("sigmoid", (1, 1, 1))], foremost=False)
+    return gen, disc
 
 
 def init_kernel_weights(net, seed, dtype):

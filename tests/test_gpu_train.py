@@ -374,6 +374,89 @@ def test_the_reference_cifar_example_network_trains_on_the_device():
     assert np.allclose(probs.reshape((N, 10), order="F").sum(axis=1), 1.0, atol=1e-4)
 
 
+def test_the_reference_gan_example_trains_on_the_device():
+    """examples/mnist_gan.cpp:34-107 on MNIST-shaped synthetic data: two rounds of its training loop - the discriminator
+    on a generated and on a real batch, then the generator through the frozen discriminator (whose gradients accumulate
+    and are reset, but whose values stay: optimizer/SGDOptimizer.hpp:58-70, optimizer/AdamOptimizer.hpp:71) - with
+    BinaryCrossEntropyLoss and two AdamOptimizers (learning rate 2e-4, first decay .5), every tensor on the device,
+    against the same two networks built from the oracle's layers in float64."""
+    import harness as hn
+    dt, m = np.float32, 100
+    gen = hp.rng(0xC0FFEE31)
+    f32 = lambda v: float(np.float32(v))
+    hyper = [f32(2e-4), f32(0.5), f32(1e-3), f32(1e-5)]
+    eps = f32(1e-5)
+
+    class Side(object):
+        """One implementation of the pair of networks with its losses and optimizers."""
+        def __init__(self, device):
+            self.device = device
+            self.G, self.D = hn.build_gan_example(hn.HipBackend(dt)) if device else \
+                hn.build_gan_example(hn.OracleBackend(np.float64), mask_dtype=dt)
+            self.steps = {"G": 0, "D": 0}
+            if device:
+                self.lists = {"G": ch.ParameterList(self.G.params()), "D": ch.ParameterList(self.D.params())}
+            else:
+                self.states = {k: [[np.zeros_like(p.get_values()) for _ in range(3)] for p in net.params()]
+                               for k, net in (("G", self.G), ("D", self.D))}
+
+        def tensor(self, a):
+            return ch.DeviceTensor.from_host(a) if self.device else np.asarray(a, np.float64)
+
+        def loss(self, out, obj):
+            if self.device:
+                return ch.loss_function("binary_cross_entropy", out, obj), \
+                    ch.loss_d_function("binary_cross_entropy", out, obj, scale=1.0 / m)
+            return oracle.loss_function("binary_cross_entropy", out, obj, eps=eps), \
+                oracle.loss_d_function("binary_cross_entropy", out, obj, eps=eps, scale=f32(1.0 / m))
+
+        def update(self, which):
+            net = self.G if which == "G" else self.D
+            if self.device:
+                self.lists[which].optimizer_step("adam", hyper, 0, self.steps[which])
+            else:
+                for p, st in zip(net.params(), self.states[which]):
+                    new, st[:] = oracle.optimizer_update("adam", p.get_values(), p.get_grad(), st, hyper, 0, self.steps[which])
+                    p.set_values(new)
+                    p.reset_grad()
+            self.steps[which] += 1
+
+        def round(self, z_fake, real, real_labels, z_gen):
+            losses = []
+            fake = self.G.propagate(self.tensor(z_fake), False)                       # infer
+            for data, labels in ((fake, np.zeros((m, 1, 1, 1), dt)), (self.tensor(real), real_labels)):
+                out = self.D.propagate(data, True)
+                l, g = self.loss(out, self.tensor(labels))
+                self.D.backpropagate(g)
+                self.update("D")
+                losses.append(np.asarray(l, np.float64))
+            out = self.D.propagate(self.G.propagate(self.tensor(z_gen), True), True)
+            l, g = self.loss(out, self.tensor(np.ones((m, 1, 1, 1), dt)))
+            self.G.backpropagate(self.D.backpropagate(g))
+            self.update("G")
+            for p in self.D.params():                                                 # frozen: reset, not updated
+                p.reset_grad()
+            losses.append(np.asarray(l, np.float64))
+            return losses
+
+    dev, ref = Side(True), Side(False)
+    for net_d, net_r, seed in ((dev.G, ref.G, 40), (dev.D, ref.D, 41)):
+        hn.init_kernel_weights(net_d, seed, dt)
+        for pd, pr in zip(net_d.params(), net_r.params()):
+            pr.set_values(np.asarray(pd.get_values(), np.float64))
+    for rnd in range(2):
+        z_fake = hp.normal(gen, (m, 1, 1, 100), dt)
+        real = hp.uniform(gen, (m, 28, 28, 1), -1, 1, dt)
+        real_labels = hp.uniform(gen, (m, 1, 1, 1), 0.9, 1.0, dt)                     # the example's smoothed labels
+        z_gen = hp.normal(gen, (m, 1, 1, 100), dt)
+        for k, (a, b) in enumerate(zip(dev.round(z_fake, real, real_labels, z_gen), ref.round(z_fake, real, real_labels, z_gen))):
+            assert hp.rel_err(a, b) < 1e-3, (rnd, k)
+    for net_d, net_r in ((dev.G, ref.G), (dev.D, ref.D)):
+        for pd, pr in zip(net_d.params(), net_r.params()):
+            assert np.allclose(pd.get_values(), pr.get_values(), rtol=1e-3, atol=2e-5)
+            assert np.all(pd.get_grad() == 0)
+
+
 ALL_OPTIMIZERS = [("vanilla_sgd", [1e-2]), ("momentum_sgd", [1e-2, 1e-3, 0.9]), ("nesterov_momentum_sgd", [1e-2, 1e-3, 0.9]),
                   ("adagrad", [1e-2, 1e-5]), ("rmsprop", [1e-3, 1e-1, 1e-5]), ("adadelta", [5e-2, 1e-5]),
                   ("adam", [1e-3, 1e-1, 1e-3, 1e-5]), ("adamax", [1e-3, 1e-1, 1e-3, 1e-5]), ("nadam", [1e-3, 1e-1, 1e-3, 1e-5]),
