@@ -94,6 +94,32 @@ class OracleConv(OracleLayer):
         return dx
 
 
+class OracleTransConv(OracleLayer):
+    """layer/kernel/TransConvKernelLayer.hpp:115-187: weights [C x RH*RW*F], a bias per output activation."""
+
+    def __init__(self, dtype, input_dims, filters, RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0):
+        OracleLayer.__init__(self, dtype)
+        H, W, C = input_dims
+        self.geom = dict(RH=RH, RW=RW, pv=pv, ph=ph, sv=sv, sh=sh, dv=dv, dh=dh)
+        OH, OW = oracle.transconv_out_dims(H, W, RH, RW, pv, ph, sv, sh, dv, dh)
+        self.out_dims, self.filters = (OH, OW, filters), filters
+        self.params = [HostParams(C, RH * RW * filters, dtype), HostParams(1, OH * OW * filters, dtype)]
+
+    def get_output_dims(self):
+        return self.out_dims
+
+    def pass_forward(self, x, training):
+        self.x = np.asarray(x, self.dtype)
+        return oracle.transconv_forward(self.x, self.params[0].values, self.params[1].values, self.filters, **self.geom)
+
+    def pass_back(self, g):
+        dx, dw, db = oracle.transconv_backward(self.x, self.params[0].values, np.asarray(g, self.dtype),
+                                               input_layer=self.input_layer, **self.geom)
+        self.params[0].accumulate_grad(dw)
+        self.params[1].accumulate_grad(db)
+        return dx
+
+
 class OracleDense(OracleLayer):
     """layer/kernel/DenseKernelLayer.hpp:92-115"""
 
@@ -264,6 +290,9 @@ class OracleBackend(object):
     def dense(self, dims, out):
         return OracleDense(self.dtype, dims, out)
 
+    def transconv(self, dims, filters, **kw):
+        return OracleTransConv(self.dtype, dims, filters, **kw)
+
     def act(self, kind, dims, param=0.0):
         return OracleActivation(self.dtype, kind, dims, param)
 
@@ -292,6 +321,9 @@ class HipBackend(object):
 
     def dense(self, dims, out):
         return self.ch.DenseKernelLayer(self.dtype, dims, out)
+
+    def transconv(self, dims, filters, RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0):
+        return self.ch.TransConvKernelLayer(self.dtype, dims, filters, RH, RW, pv, ph, sv, sh, dv, dh)
 
     def act(self, kind, dims, param=0.0):
         return self.ch.ActivationLayer(self.dtype, kind, dims, param)
@@ -427,6 +459,20 @@ def build_cifar_example(backend, mask_dtype=None):
                            b.dropout((8, 8, 8), 0.25, 101, mask_dtype), b.dense((8, 8, 8), 50), b.act("relu", (50, 1, 1)),
                            b.dropout((50, 1, 1), 0.5, 102, mask_dtype), b.dense((50, 1, 1), 10),
                            b.act("softmax", (10, 1, 1), 1e-5)])
+
+
+def build_autoencoder_example(backend):
+    """The stacked encoder and decoder of the reference's examples/mnist_autoencoder.cpp:25-48 as one layer stack
+    (StackedNeuralNetwork chains the modules: neural_network/StackedNeuralNetwork.hpp): conv 4x4 stride 2 -> softplus ->
+    conv 4x4 -> softplus -> dense 100 | dense 300 -> softplus -> reshape 10x10x3 -> transposed conv 4x4 -> softplus ->
+    transposed conv 4x4 stride 2; the receptors have no padding."""
+    b = backend
+    k = dict(RH=4, RW=4, pv=0, ph=0)
+    return FeedforwardNet([b.conv((28, 28, 1), 3, sv=2, sh=2, **k), b.act("softplus", (13, 13, 3)), b.conv((13, 13, 3), 3, **k),
+                           b.act("softplus", (10, 10, 3)), b.dense((10, 10, 3), 100),
+                           b.dense((100, 1, 1), 300), b.act("softplus", (300, 1, 1)), b.reshape((300, 1, 1), (10, 10, 3)),
+                           b.transconv((10, 10, 3), 3, **k), b.act("softplus", (13, 13, 3)),
+                           b.transconv((13, 13, 3), 1, sv=2, sh=2, **k)])
 
 
 def build_gan_example(backend, mask_dtype=None):

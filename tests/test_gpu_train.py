@@ -374,6 +374,41 @@ def test_the_reference_cifar_example_network_trains_on_the_device():
     assert np.allclose(probs.reshape((N, 10), order="F").sum(axis=1), 1.0, atol=1e-4)
 
 
+def test_the_reference_autoencoder_example_trains_on_the_device():
+    """examples/mnist_autoencoder.cpp:25-53 (strided convolutions without padding, softplus, dense bottleneck, reshape,
+    transposed convolutions, SquaredLoss against the input itself, NadamOptimizer) on MNIST-shaped synthetic data: three
+    batches on the device against the oracle's layers in float64."""
+    import harness as hn
+    dt, N = np.float32, 64
+    gen = hp.rng(0xC0FFEE32)
+    x = hp.uniform(gen, (N, 28, 28, 1), 0, 1, dt)
+    dev, ref = hn.build_autoencoder_example(hn.HipBackend(dt)), hn.build_autoencoder_example(hn.OracleBackend(np.float64))
+    assert dev.layers[-1].get_output_dims() == (28, 28, 1) and ref.layers[-1].get_output_dims() == (28, 28, 1)
+    hn.init_kernel_weights(dev, 50, dt)
+    for pd, pr in zip(dev.params(), ref.params()):
+        pr.set_values(np.asarray(pd.get_values(), np.float64))
+    hyper = [float(np.float32(h)) for h in (1e-3, 1e-1, 1e-3, 1e-5)]
+    plist = ch.ParameterList(dev.params())
+    states = [[np.zeros_like(p.get_values()) for _ in range(3)] for p in ref.params()]
+    xd, x64 = ch.DeviceTensor.from_host(x), np.asarray(x, np.float64)
+    for step in range(3):
+        out = dev.propagate(xd, True)
+        loss_dev = ch.loss_function("squared", out, xd)
+        dev.backpropagate(ch.loss_d_function("squared", out, xd, scale=1.0 / N))
+        plist.optimizer_step("nadam", hyper, 0, step)
+        out_r = ref.propagate(x64, True)
+        loss_ref = oracle.loss_function("squared", out_r, x64)
+        ref.backpropagate(oracle.loss_d_function("squared", out_r, x64, scale=float(np.float32(1.0 / N))))
+        for p, st in zip(ref.params(), states):
+            new, st[:] = oracle.optimizer_update("nadam", p.get_values(), p.get_grad(), st, hyper, 0, step)
+            p.set_values(new)
+            p.reset_grad()
+        assert hp.rel_err(loss_dev, loss_ref) < 1e-3, step
+    for pd, pr in zip(dev.params(), ref.params()):
+        assert np.allclose(pd.get_values(), pr.get_values(), rtol=1e-3, atol=2e-5)
+    assert hp.rel_err(dev.propagate(xd, False).to_host(), ref.propagate(x64, False)) < 1e-3
+
+
 def test_the_reference_gan_example_trains_on_the_device():
     """examples/mnist_gan.cpp:34-107 on MNIST-shaped synthetic data: two rounds of its training loop - the discriminator
     on a generated and on a real batch, then the generator through the frozen discriminator (whose gradients accumulate
