@@ -458,12 +458,45 @@ class DeviceFeedforwardNetwork {
 public:
 	inline explicit DeviceFeedforwardNetwork(std::vector<DeviceLayer<Scalar>> layers, bool foremost = true) :
 			layers(std::move(layers)),
-			foremost(foremost) {
+			foremost(foremost),
+			frozen(false) {
 		assert(!this->layers.empty());
 		this->layers[0].set_input_layer(foremost);
 	}
 	inline std::vector<DeviceLayer<Scalar>>& get_layers() {
 		return layers;
+	}
+	inline const typename DeviceLayer<Scalar>::Dims& get_input_dims() const {
+		return layers.front().get_input_dims();
+	}
+	inline const typename DeviceLayer<Scalar>::Dims& get_output_dims() const {
+		return layers.back().get_output_dims();
+	}
+	/** neural_network/FeedforwardNeuralNetwork.hpp:88-94 */
+	inline bool is_foremost() const {
+		return foremost;
+	}
+	inline void set_foremost(bool foremost) {
+		layers[0].set_input_layer(foremost);
+		this->foremost = foremost;
+	}
+	/**
+	 * NeuralNetwork::set_frozen (core/NeuralNetwork.hpp:166-169): the parameters of a frozen network still receive
+	 * gradients, optimizers leave their values alone and reset the gradients (optimizer/SGDOptimizer.hpp:58-70).
+	 */
+	inline bool is_frozen() const {
+		return frozen;
+	}
+	inline void set_frozen(bool frozen) {
+		this->frozen = frozen;
+	}
+	/** NeuralNetwork::infer (core/NeuralNetwork.hpp:225-228); the result lives until the next pass of the network. */
+	inline const DeviceTensor<Scalar>& infer(const DeviceTensor<Scalar>& input) {
+		return propagate(input, false);
+	}
+	inline void reset_grads() {
+		for (std::size_t i = 0; i < layers.size(); ++i)
+			layers[i].reset_grads();
 	}
 	/**
 	 * NeuralNetwork::save_all_unique_params_values / load_all_unique_params_values in the binary format
@@ -565,6 +598,10 @@ public:
 	 * (optimizer/SGDOptimizer.hpp:64, :68-70), sixteen parameters per launch.
 	 */
 	inline void optimizer_step(cattle_hip_optimizer optimizer, const double (&hyper)[4], std::size_t epoch, std::size_t timestep) {
+		if (frozen) {
+			reset_grads();
+			return;
+		}
 		std::vector<cattle_hip_layer_t> handles;
 		std::vector<std::size_t> indices;
 		for (std::size_t i = 0; i < layers.size(); ++i)
@@ -584,7 +621,76 @@ private:
 		return total;
 	}
 	std::vector<DeviceLayer<Scalar>> layers;
-	bool foremost;
+	bool foremost, frozen;
+};
+
+/**
+ * Feed-forward networks on top of one another (neural_network/StackedNeuralNetwork.hpp:33-120 on device tensors): only
+ * the first module can be foremost; propagate and backpropagate run through the modules in order and in reverse. Each
+ * module keeps its own frozen flag, so one optimizer step can update some modules and only reset the gradients of others,
+ * as the reference's generative-adversarial example does (examples/mnist_gan.cpp:107-109).
+ */
+template<typename Scalar>
+class DeviceStackedNetwork {
+public:
+	typedef DeviceFeedforwardNetwork<Scalar> Module;
+	inline explicit DeviceStackedNetwork(std::vector<Module> modules, bool foremost = true) : modules(std::move(modules)) {
+		if (this->modules.empty())
+			throw std::invalid_argument("modules must contain at least 1 element");
+		for (std::size_t i = 1; i < this->modules.size(); ++i) {
+			if (this->modules[i - 1].get_output_dims() != this->modules[i].get_input_dims())
+				throw std::invalid_argument("incompatible network dimensions");
+			this->modules[i].set_foremost(false);
+		}
+		this->modules[0].set_foremost(foremost);
+	}
+	inline std::vector<Module>& get_modules() {
+		return modules;
+	}
+	inline bool is_foremost() const {
+		return modules[0].is_foremost();
+	}
+	inline void set_foremost(bool foremost) {
+		modules[0].set_foremost(foremost);
+	}
+	inline void set_frozen(bool frozen) {
+		for (std::size_t i = 0; i < modules.size(); ++i)
+			modules[i].set_frozen(frozen);
+	}
+	/** `input` must stay alive and unmodified until backpropagate returns. */
+	inline const DeviceTensor<Scalar>& propagate(const DeviceTensor<Scalar>& input, bool training) {
+		const DeviceTensor<Scalar>* cur = &modules[0].propagate(input, training);
+		for (std::size_t i = 1; i < modules.size(); ++i)
+			cur = &modules[i].propagate(*cur, training);
+		return *cur;
+	}
+	inline const DeviceTensor<Scalar>& infer(const DeviceTensor<Scalar>& input) {
+		return propagate(input, false);
+	}
+	inline DeviceTensor<Scalar> backpropagate(const DeviceTensor<Scalar>& out_grad) {
+		DeviceTensor<Scalar> grad = modules.back().backpropagate(out_grad);
+		for (std::size_t i = modules.size() - 1; i-- > 0;)
+			grad = modules[i].backpropagate(grad);
+		return grad;
+	}
+	inline void optimizer_step(cattle_hip_optimizer optimizer, const double (&hyper)[4], std::size_t epoch, std::size_t timestep) {
+		for (std::size_t i = 0; i < modules.size(); ++i)
+			modules[i].optimizer_step(optimizer, hyper, epoch, timestep);
+	}
+	/** One batch of SGDOptimizer::_train (optimizer/SGDOptimizer.hpp:44-70); returns the sum of the per-sample losses. */
+	inline Scalar train_batch(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj, const DeviceLoss<Scalar>& loss,
+			cattle_hip_optimizer optimizer, const double (&hyper)[4], std::size_t epoch, std::size_t timestep) {
+		const DeviceTensor<Scalar>& out = propagate(input, true);
+		const std::vector<Scalar> losses = loss.function(out, obj);
+		Scalar total = 0;
+		for (std::size_t i = 0; i < losses.size(); ++i)
+			total += losses[i];
+		backpropagate(loss.d_function(out, obj, (Scalar) 1 / (Scalar) input.batch()));
+		optimizer_step(optimizer, hyper, epoch, timestep);
+		return total;
+	}
+private:
+	std::vector<Module> modules;
 };
 
 /**

@@ -143,6 +143,79 @@ static void run(const std::string& tag) {
 		record(tag + ".move.infer", sizeof(Scalar), { batch, 6, 2, 6 }, net.propagate(xd, false).to_host().data());
 	}
 	{
+		/* two stacked networks trained as the reference's generative-adversarial example trains them
+		 * (examples/mnist_gan.cpp:92-109), once through DeviceStackedNetwork and the frozen flag, once with the same calls
+		 * spelled out on two separate networks: the recorded parameters must be identical */
+		const std::size_t batch = 12;
+		const double adam[4] = { 2e-4, 0.5, 1e-3, 1e-5 };
+		DeviceLoss<Scalar> bce(CATTLE_HIP_LOSS_BINARY_CROSS_ENTROPY);
+		auto make_generator = [] {
+			std::vector<DL> layers;
+			layers.push_back(DL::dense(Dims{ { 1, 1, 10 } }, 24));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_LEAKY_RELU, layers.back().get_output_dims(), (Scalar) 0.2));
+			layers.push_back(DL::dense(layers.back().get_output_dims(), 18));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_TANH, layers.back().get_output_dims()));
+			layers.push_back(DL::reshape(layers.back().get_output_dims(), Dims{ { 3, 3, 2 } }));
+			return DeviceFeedforwardNetwork<Scalar>(std::move(layers));
+		};
+		auto make_discriminator = [] {
+			std::vector<DL> layers;
+			layers.push_back(DL::dense(Dims{ { 3, 3, 2 } }, 16));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_LEAKY_RELU, layers.back().get_output_dims(), (Scalar) 0.2));
+			layers.push_back(DL::dropout(layers.back().get_output_dims(), (Scalar) 0.3, 7));
+			layers.push_back(DL::dense(layers.back().get_output_dims(), 1));
+			layers.push_back(DL::activation(CATTLE_HIP_ACT_SIGMOID, layers.back().get_output_dims()));
+			return DeviceFeedforwardNetwork<Scalar>(std::move(layers), false);
+		};
+		Lcg g(15);
+		std::vector<Scalar> z = random_values<Scalar>(batch * 10, g, 1.0), real = random_values<Scalar>(batch * 18, g, 1.0);
+		std::vector<Scalar> ones(batch, (Scalar) 1), zeros(batch, (Scalar) 0);
+		DT zd(typename DT::Dims{ { batch, 1, 1, 10 } }, z.data()), reald(typename DT::Dims{ { batch, 3, 3, 2 } }, real.data());
+		DT oned(typename DT::Dims{ { batch, 1, 1, 1 } }, ones.data()), zerod(typename DT::Dims{ { batch, 1, 1, 1 } }, zeros.data());
+		for (int stacked = 0; stacked < 2; ++stacked) {
+			Lcg gw(16);
+			std::vector<DeviceFeedforwardNetwork<Scalar>> nets;
+			nets.push_back(make_generator());
+			nets.push_back(make_discriminator());
+			init_and_record<Scalar>(tag + ".gan" + std::to_string(stacked) + ".g", nets[0], gw);
+			init_and_record<Scalar>(tag + ".gan" + std::to_string(stacked) + ".d", nets[1], gw);
+			std::vector<Scalar> losses;
+			if (stacked) {
+				DeviceStackedNetwork<Scalar> gan(std::move(nets));
+				for (std::size_t t = 0; t < 2; ++t) {
+					const DT& fake = gan.get_modules()[0].infer(zd);      /* lives until the generator's next pass */
+					losses.push_back(gan.get_modules()[1].train_batch(fake, zerod, bce, CATTLE_HIP_OPT_ADAM, adam, 0, 2 * t));
+					losses.push_back(gan.get_modules()[1].train_batch(reald, oned, bce, CATTLE_HIP_OPT_ADAM, adam, 0, 2 * t + 1));
+					gan.get_modules()[1].set_frozen(true);
+					losses.push_back(gan.train_batch(zd, oned, bce, CATTLE_HIP_OPT_ADAM, adam, 0, t));
+					gan.get_modules()[1].set_frozen(false);
+				}
+				record_final<Scalar>(tag + ".gan1.g", gan.get_modules()[0]);
+				record_final<Scalar>(tag + ".gan1.d", gan.get_modules()[1]);
+			} else {
+				DeviceFeedforwardNetwork<Scalar>& gen = nets[0];
+				DeviceFeedforwardNetwork<Scalar>& disc = nets[1];
+				for (std::size_t t = 0; t < 2; ++t) {
+					const DT& fake = gen.propagate(zd, false);
+					losses.push_back(disc.train_batch(fake, zerod, bce, CATTLE_HIP_OPT_ADAM, adam, 0, 2 * t));
+					losses.push_back(disc.train_batch(reald, oned, bce, CATTLE_HIP_OPT_ADAM, adam, 0, 2 * t + 1));
+					const DT& out = disc.propagate(gen.propagate(zd, true), true);
+					Scalar total = 0;
+					const std::vector<Scalar> per_sample = bce.function(out, oned);
+					for (std::size_t i = 0; i < per_sample.size(); ++i)
+						total += per_sample[i];
+					losses.push_back(total);
+					gen.backpropagate(disc.backpropagate(bce.d_function(out, oned, (Scalar) 1 / (Scalar) batch)));
+					gen.optimizer_step(CATTLE_HIP_OPT_ADAM, adam, 0, t);
+					disc.reset_grads();
+				}
+				record_final<Scalar>(tag + ".gan0.g", gen);
+				record_final<Scalar>(tag + ".gan0.d", disc);
+			}
+			record(tag + ".gan" + std::to_string(stacked) + ".losses", sizeof(Scalar), { losses.size() }, losses.data());
+		}
+	}
+	{
 		/* another loss of the loss/ directory, wrapped as NegatedLoss wraps it */
 		Lcg g(13);
 		const std::size_t batch = 9, classes = 7;

@@ -63,6 +63,21 @@ def out_shape(net):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tag", ["f32", "f64"])
+def test_stacked_network_with_a_frozen_module(records, tag):
+    """DeviceStackedNetwork and set_frozen against the same training loop spelled out on two separate networks."""
+    spelled = {k[len(tag) + 6:]: v for k, v in records.items() if k.startswith(tag + ".gan0.")}
+    stacked = {k[len(tag) + 6:]: v for k, v in records.items() if k.startswith(tag + ".gan1.")}
+    assert set(spelled) == set(stacked) and len(spelled) == 2 * 4 * 2 + 1
+    for k in spelled:
+        assert np.array_equal(spelled[k], stacked[k]), k
+    assert np.all(np.isfinite(spelled["losses"])) and len(spelled["losses"]) == 6
+    # the generator moved in its own steps, the frozen discriminator only in the discriminator's
+    assert not np.array_equal(spelled["g.final.0.0"], spelled["g.init.0.0"])
+    assert not np.array_equal(spelled["d.final.0.0"], spelled["d.init.0.0"])
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("tag,dtype", [("f32", np.float32), ("f64", np.float64)])
 def test_reshape_broadcast_dropout_stack(records, tag, dtype):
     x, go = records[tag + ".move.x"], records[tag + ".move.go"]
