@@ -31,7 +31,7 @@ EXPORTS = [
     "cattle_hip_timer_destroy", "cattle_hip_timer_start", "cattle_hip_timer_stop", "cattle_hip_conv_create",
     "cattle_hip_transconv_create", "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
     "cattle_hip_batchnorm_set_stats_initialized", "cattle_hip_activation_create", "cattle_hip_pool_create",
-    "cattle_hip_dropout_create", "cattle_hip_reshape_create", "cattle_hip_broadcast_create",
+    "cattle_hip_convlstm_set_multiplicative_integration", "cattle_hip_dropout_create", "cattle_hip_reshape_create", "cattle_hip_broadcast_create",
     "cattle_hip_layer_clone", "cattle_hip_layer_destroy", "cattle_hip_layer_input_dims",
     "cattle_hip_layer_output_dims", "cattle_hip_layer_is_input_layer", "cattle_hip_layer_set_input_layer",
     "cattle_hip_layer_empty_cache", "cattle_hip_layer_forward", "cattle_hip_layer_backward",
@@ -507,7 +507,7 @@ class ConvLSTMNetwork(Layer):
     def __init__(self, dtype, input_dims, hidden_channels, receptor_height=3, receptor_width=3, vertical_padding=1,
                  horizontal_padding=1, vertical_dilation=0, horizontal_dilation=0,
                  activations=("sigmoid", "sigmoid", "tanh", "tanh", "sigmoid"), activation_params=(0, 0, 0, 0, 0),
-                 output_seq_size_func=lambda input_seq_length: (input_seq_length, 0), foremost=True):
+                 output_seq_size_func=lambda input_seq_length: (input_seq_length, 0), foremost=True, mul_int=False):
         H, W, C = (int(d) for d in input_dims)
         kinds = (ctypes.c_int * 5)(*[ACT[a] for a in activations])
         params = (ctypes.c_double * 5)(*[float(p) for p in activation_params])
@@ -522,6 +522,11 @@ class ConvLSTMNetwork(Layer):
         self._rv = (receptor_height * receptor_width * C, receptor_height * receptor_width * int(hidden_channels))
         self._hidden = int(hidden_channels)
         self._in_seq_shape = None
+        if mul_int:         # the MulInt template argument (neural_network/LSTMNeuralNetwork.hpp:44)
+            self.set_multiplicative_integration(True)
+
+    def set_multiplicative_integration(self, enabled):
+        _check(lib().cattle_hip_convlstm_set_multiplicative_integration(self._h, ctypes.c_int(int(bool(enabled)))))
 
     def is_foremost(self):
         return self._foremost

@@ -147,11 +147,13 @@ template<typename T> void broadcast_backward(int H, int W, int C, int bh, int bw
  * the four gates as consecutive blocks of P elements; `*_all` tensors are (N, T, ...) over all steps. */
 template<typename T> struct LstmActs { int kind[5]; T param[5]; };
 template<typename T> void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int zx_T, int zx_t,
-		const T* zh, const T* prev_state, T* z, T* gates, T* state, T* act_state, T* hidden, T* hprev_all, int h_T, int h_t,
-		T* out, int out_T, int out_t);
+		const T* zh, bool mul_int, const T* prev_state, T* z, T* gates, T* state, T* act_state, T* hidden, T* hprev_all, int h_T,
+		int h_t, T* out, int out_T, int out_t);
+/* zx_fwd / zh_fwd: the step's weighted input (in the all-steps tensor) and weighted previous output when the network
+ * integrates multiplicatively and the step had both; null otherwise. */
 template<typename T> void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, const T* out_grad, int og_T,
 		int og_t, const T* z, const T* gates, const T* prev_state, const T* state, const T* act_state, T* state_grad, T* dz,
-		T* dzx_all, int x_T, int x_t, T* dzh_all, int h_T, int h_t);
+		T* dzx_all, int x_T, int x_t, T* dzh_all, int h_T, int h_t, const T* zx_fwd, const T* zh_fwd);
 
 /* Losses and optimizer updates (train_kernels.hip). A batch is N samples x T_steps x V elements,
  * column-major with the sample index fastest. */

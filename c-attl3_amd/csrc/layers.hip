@@ -375,6 +375,7 @@ struct ConvLstm : LayerBase {
 	int hidden;
 	LstmActs<T> acts;
 	bool foremost;
+	bool mul_int = false;           /* LSTMNeuralNetwork<Scalar,Rank,MulInt = true> (:44, :303-311) */
 	/* alignment of the last propagate (:398-401) */
 	size_t T_in = 0, T_out = 0, delay = 0, steps = 0;
 	const T* x_cache = nullptr;
@@ -392,7 +393,7 @@ struct ConvLstm : LayerBase {
 		params.push_back(std::make_shared<Param>(1, (size_t) sh.F, true, sizeof(T)));
 	}
 	ConvLstm(const ConvLstm& o, bool share) : LayerBase(o.dtype), sx(o.sx), sh(o.sh), hidden(o.hidden), acts(o.acts),
-			foremost(o.foremost) {
+			foremost(o.foremost), mul_int(o.mul_int) {
 		copy_base(o, share);
 	}
 	LayerBase* clone(bool share) const override {
@@ -432,7 +433,8 @@ struct ConvLstm : LayerBase {
 		state.ensure(p * total * e);
 		act_state.ensure(p * total * e);
 		hid.ensure(p * total * e);
-		zh.ensure(4 * p * e);
+		/* with multiplicative integration the backward pass needs every step's weighted previous output */
+		zh.ensure(4 * p * (mul_int ? total : 1) * e);
 		/* slab t of hprev_all is the hidden output of step t - 1 (the first step's kernel zeroes slab 0: no previous
 		 * output); every slab is written once per pass */
 		hprev_all.ensure(p * total * e);
@@ -440,14 +442,15 @@ struct ConvLstm : LayerBase {
 		T* wth = (T*) wh.derived[0].ensure(wsh.wt_fwd * e);
 		for (size_t t = 0; t < total; ++t) {
 			const bool has_in = t < in_len, has_prev = t > 0;
+			T* zh_t = step(zh, mul_int ? t : 0, 4 * p);
 			if (has_prev) {
-				conv_forward<T>(sh, n, step(hid, t - 1, p), (const T*) wh.values.p, (const T*) params[3]->values.p, (T*) zh.p,
+				conv_forward<T>(sh, n, step(hid, t - 1, p), (const T*) wh.values.p, (const T*) params[3]->values.p, zh_t,
 						wth, wh.derived_version[0] == wh.version);
 				wh.derived_version[0] = wh.version;
 			}
 			const bool emits = t >= out_delay && t < out_delay + out_len;      /* :386-393 */
 			lstm_gates_forward<T>(acts, n, p, has_in ? (const T*) zx_all.p : nullptr, (int) in_len, (int) t,
-					has_prev ? (const T*) zh.p : nullptr, has_prev ? step(state, t - 1, p) : nullptr, step(z, t, 4 * p),
+					has_prev ? (const T*) zh_t : nullptr, mul_int, has_prev ? step(state, t - 1, p) : nullptr, step(z, t, 4 * p),
 					step(gates, t, 4 * p), step(state, t, p), step(act_state, t, p), step(hid, t, p),
 					(T*) hprev_all.p, (int) total, (int) (t + 1), emits ? out : nullptr, (int) out_len,
 					(int) (t - out_delay));
@@ -473,11 +476,12 @@ struct ConvLstm : LayerBase {
 		for (size_t t = total; t-- > 0;) {
 			const bool has_in = t < T_in, has_prev = t > 0;
 			const bool emitted = t >= delay && t < delay + T_out;
+			const bool both = mul_int && has_in && has_prev;
 			lstm_gates_backward<T>(acts, n, p, t + 1 < total ? (const T*) dh.p : nullptr, emitted ? out_grad : nullptr,
 					(int) T_out, (int) (t - delay), step(z, t, 4 * p), step(gates, t, 4 * p),
 					has_prev ? step(state, t - 1, p) : nullptr, step(state, t, p), step(act_state, t, p), (T*) state_grad.p,
 					(T*) dz.p, has_in ? (T*) dzx_all.p : nullptr, (int) T_in, (int) t, (T*) dzh_all.p,
-					(int) total, (int) t);
+					(int) total, (int) t, both ? (const T*) zx_all.p : nullptr, both ? (const T*) step(zh, t, 4 * p) : nullptr);
 			if (has_prev) {
 				/* the four output-side kernels' pass_back, summed (:470-473, :491-494): one input-gradient launch */
 				conv_input_gradient<T>(sh, n, (const T*) wh.values.p, (const T*) dz.p, (T*) dh.p, wtd,
@@ -1318,6 +1322,17 @@ int cattle_hip_convlstm_get_kernel_grad(cattle_hip_layer_t lstm, size_t kernel, 
 		size_t offset, bytes;
 		Param& p = lstm_kernel_param(lstm, kernel, bias, offset, bytes);
 		copy_out(grad, space, (const char*) p.grad.p + offset, bytes);
+	});
+}
+
+int cattle_hip_convlstm_set_multiplicative_integration(cattle_hip_layer_t lstm, int enabled) {
+	return guarded([&] {
+		LayerBase* l = as_layer(lstm);
+		ConvLstm<float>* f = dynamic_cast<ConvLstm<float>*>(l);
+		ConvLstm<double>* d = dynamic_cast<ConvLstm<double>*>(l);
+		CATTLE_HIP_REQUIRE(f || d, "not a ConvLSTM handle");
+		(f ? f->mul_int : d->mul_int) = enabled != 0;
+		l->empty_cache();           /* the caches of a pass made under the other rule do not fit this one */
 	});
 }
 

@@ -848,7 +848,7 @@ __device__ __forceinline__ size_t seq_offset(unsigned n, unsigned rest, int N, i
 template<typename T>
 __global__ __launch_bounds__(256)
 void lstm_gates_forward_kernel(LstmActs<T> a, int N, size_t P, const T* __restrict__ zx, int zx_T, int zx_t,
-		const T* __restrict__ zh, const T* __restrict__ prev_state, T* __restrict__ z, T* __restrict__ gates,
+		const T* __restrict__ zh, bool mul_int, const T* __restrict__ prev_state, T* __restrict__ z, T* __restrict__ gates,
 		T* __restrict__ state, T* __restrict__ act_state, T* __restrict__ hidden, T* __restrict__ hprev_all, int h_T, int h_t,
 		T* __restrict__ out, int out_T, int out_t) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
@@ -858,12 +858,13 @@ void lstm_gates_forward_kernel(LstmActs<T> a, int N, size_t P, const T* __restri
 		T y[4];
 		#pragma unroll
 		for (int g = 0; g < 4; ++g) {
-			/* weighted input + weighted previous output (:312, :327, :342, :373) */
+			/* weighted input + weighted previous output (:312, :327, :342, :373), their product with multiplicative
+			 * integration (:303-311); a step with only one of the two takes it as it is */
 			T v = (T) 0;
 			if (zx)
 				v = zx[seq_offset(n, rest + g * slab_rows, N, zx_T, zx_t)];
 			if (zh)
-				v = zx ? v + zh[g * P + e] : zh[g * P + e];
+				v = zx ? (mul_int ? v * zh[g * P + e] : v + zh[g * P + e]) : zh[g * P + e];
 			z[g * P + e] = v;
 			const int which = g < 3 ? g : 4;                        /* kinds: forget, write, candidate, state, read */
 			y[g] = act_f_rt<T>(a.kind[which], v, a.param[which]);
@@ -893,7 +894,8 @@ __global__ __launch_bounds__(256)
 void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restrict__ dh, const T* __restrict__ out_grad,
 		int og_T, int og_t, const T* __restrict__ z, const T* __restrict__ gates, const T* __restrict__ prev_state,
 		const T* __restrict__ state, const T* __restrict__ act_state, T* __restrict__ state_grad, T* __restrict__ dz,
-		T* __restrict__ dzx_all, int x_T, int x_t, T* __restrict__ dzh_all, int h_T, int h_t) {
+		T* __restrict__ dzx_all, int x_T, int x_t, T* __restrict__ dzh_all, int h_T, int h_t, const T* __restrict__ zx_fwd,
+		const T* __restrict__ zh_fwd) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
 	const unsigned slab_rows = (unsigned) (P / (size_t) N);
 	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < P; e += stride) {
@@ -913,11 +915,18 @@ void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restr
 		state_grad[e] = sg * f;                                                                    /* :445 */
 		#pragma unroll
 		for (int g = 0; g < 4; ++g) {
-			dz[g * P + e] = d[g];
+			/* multiplicative integration at a step with both an input and a previous output (zx_fwd and zh_fwd are that
+			 * step's weighted input and weighted output): each side's gradient carries the other side (:449-466) */
+			T to_input = d[g], to_output = d[g];
+			if (zx_fwd) {
+				to_input = zh_fwd[g * P + e] * d[g];
+				to_output = zx_fwd[seq_offset(n, rest + g * slab_rows, N, x_T, x_t)] * d[g];
+			}
+			dz[g * P + e] = to_output;                              /* what the output kernels' pass_back receives */
 			if (dzx_all)
-				dzx_all[seq_offset(n, rest + g * slab_rows, N, x_T, x_t)] = d[g];
+				dzx_all[seq_offset(n, rest + g * slab_rows, N, x_T, x_t)] = to_input;
 			if (dzh_all)        /* step 0 has no previous output to pair with: its slab is zero */
-				dzh_all[seq_offset(n, rest + g * slab_rows, N, h_T, h_t)] = prev_state ? d[g] : (T) 0;
+				dzh_all[seq_offset(n, rest + g * slab_rows, N, h_T, h_t)] = prev_state ? to_output : (T) 0;
 		}
 	}
 }
@@ -1178,26 +1187,27 @@ void accumulate_column_sums(int N, size_t V, const T* x, T* row) {
 }
 
 template<typename T>
-void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int zx_T, int zx_t, const T* zh,
+void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int zx_T, int zx_t, const T* zh, bool mul_int,
 		const T* prev_state, T* z, T* gates, T* state, T* act_state, T* hidden, T* hprev_all, int h_T, int h_t, T* out,
 		int out_T, int out_t) {
 	if (P == 0)
 		return;
 	CATTLE_HIP_REQUIRE(P % (size_t) N == 0 && P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
-	lstm_gates_forward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, zx, zx_T, zx_t, zh, prev_state, z, gates, state,
-			act_state, hidden, hprev_all, h_T, h_t, out, out_T, out_t);
+	lstm_gates_forward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, zx, zx_T, zx_t, zh, mul_int, prev_state, z, gates,
+			state, act_state, hidden, hprev_all, h_T, h_t, out, out_T, out_t);
 	check_launch();
 }
 
 template<typename T>
 void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, const T* out_grad, int og_T, int og_t, const T* z,
 		const T* gates, const T* prev_state, const T* state, const T* act_state, T* state_grad, T* dz, T* dzx_all, int x_T,
-		int x_t, T* dzh_all, int h_T, int h_t) {
+		int x_t, T* dzh_all, int h_T, int h_t, const T* zx_fwd, const T* zh_fwd) {
 	if (P == 0)
 		return;
 	CATTLE_HIP_REQUIRE(P % (size_t) N == 0 && P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
+	CATTLE_HIP_REQUIRE((zx_fwd == nullptr) == (zh_fwd == nullptr), "multiplicative integration needs both weighted tensors");
 	lstm_gates_backward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, dh, out_grad, og_T, og_t, z, gates, prev_state,
-			state, act_state, state_grad, dz, dzx_all, x_T, x_t, dzh_all, h_T, h_t);
+			state, act_state, state_grad, dz, dzx_all, x_T, x_t, dzh_all, h_T, h_t, zx_fwd, zh_fwd);
 	check_launch();
 }
 
@@ -1410,10 +1420,10 @@ template void accumulate_column_sums<T>(int, size_t, const T*, T*); \
 template void dropout_apply<T>(size_t, unsigned long long, T, T, const T*, T*); \
 template void broadcast_forward<T>(int, int, int, int, int, int, int, const T*, T*); \
 template void broadcast_backward<T>(int, int, int, int, int, int, int, const T*, T*); \
-template void lstm_gates_forward<T>(const LstmActs<T>&, int, size_t, const T*, int, int, const T*, const T*, T*, T*, T*, T*, T*, T*, int, int, \
-		T*, int, int); \
+template void lstm_gates_forward<T>(const LstmActs<T>&, int, size_t, const T*, int, int, const T*, bool, const T*, T*, T*, T*, T*, T*, T*, int, \
+		int, T*, int, int); \
 template void lstm_gates_backward<T>(const LstmActs<T>&, int, size_t, const T*, const T*, int, int, const T*, const T*, const T*, const T*, \
-		const T*, T*, T*, T*, int, int, T*, int, int);
+		const T*, T*, T*, T*, int, int, T*, int, int, const T*, const T*);
 
 CATTLE_HIP_INSTANTIATE(float)
 CATTLE_HIP_INSTANTIATE(double)

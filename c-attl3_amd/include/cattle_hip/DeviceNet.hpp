@@ -695,8 +695,9 @@ private:
 
 /**
  * LSTMNeuralNetwork<Scalar,3> over eight ConvKernelLayers with fused gates, on device tensors
- * (neural_network/LSTMNeuralNetwork.hpp:27-120, :236-503; no multiplicative integration, not stateful, not
- * reversed). Sequences are (batch, time, height, width, channels) column-major.
+ * (neural_network/LSTMNeuralNetwork.hpp:27-120, :236-503; multiplicative integration by
+ * set_multiplicative_integration; not stateful, not reversed). An LSTM over vectors, with DenseKernelLayers, is the case
+ * of 1 x 1 images and 1 x 1 receptors without padding. Sequences are (batch, time, height, width, channels) column-major.
  */
 template<typename Scalar>
 class DeviceConvLSTM {
@@ -730,6 +731,10 @@ public:
 	inline ~DeviceConvLSTM() {
 		if (handle)
 			cattle_hip_layer_destroy(handle);
+	}
+	/** The MulInt template argument of the reference network (neural_network/LSTMNeuralNetwork.hpp:44, :303-311). */
+	inline void set_multiplicative_integration(bool enabled) {
+		check(cattle_hip_convlstm_set_multiplicative_integration(handle, enabled ? 1 : 0));
 	}
 	inline void set_kernel_values(Kernel kernel, bool bias, const Scalar* host_values) {
 		check(cattle_hip_convlstm_set_kernel_values(handle, (std::size_t) kernel, bias ? 1 : 0, host_values, CATTLE_HIP_HOST));

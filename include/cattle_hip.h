@@ -297,9 +297,9 @@ int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, d
 int cattle_hip_layer_param_reset_optimizer_state(cattle_hip_layer_t layer, size_t index);
 
 /* ---- Convolutional LSTM with fused gates ------------------------------------------------------
- * LSTMNeuralNetwork<Scalar,3,false,false> (neural_network/LSTMNeuralNetwork.hpp:27-120 constructor,
- * :236-403 propagate, :404-503 backpropagate; no multiplicative integration, not stateful, not
- * reversed) whose eight kernels are ConvKernelLayers with `hidden_channels` filters and one receptor
+ * LSTMNeuralNetwork<Scalar,3,MulInt,false> (neural_network/LSTMNeuralNetwork.hpp:27-120 constructor,
+ * :236-403 propagate, :404-503 backpropagate; multiplicative integration by
+ * cattle_hip_convlstm_set_multiplicative_integration; not stateful, not reversed) whose eight kernels are ConvKernelLayers with `hidden_channels` filters and one receptor
  * geometry that keeps the spatial dimensions (stride 1), and whose five activations are element-wise
  * kinds (CATTLE_HIP_ACT_IDENTITY .. CATTLE_HIP_ACT_SWISH) given in the order forget, write, candidate,
  * state, read with their scalar arguments (NULL = all zero). `foremost` as in the constructor (:81):
@@ -335,6 +335,11 @@ int cattle_hip_convlstm_set_kernel_values(cattle_hip_layer_t lstm, size_t kernel
 int cattle_hip_convlstm_get_kernel_values(cattle_hip_layer_t lstm, size_t kernel, int bias, void* values,
 		cattle_hip_memspace space);
 int cattle_hip_convlstm_get_kernel_grad(cattle_hip_layer_t lstm, size_t kernel, int bias, void* grad, cattle_hip_memspace space);
+/* The MulInt template argument of LSTMNeuralNetwork (neural_network/LSTMNeuralNetwork.hpp:44): at a time step that has
+ * both an input and a previous output, each gate's weighted input and weighted output are multiplied instead of added
+ * (:303-311, :318-326, :334-342, :369-377; gradients :449-466). Off when the network is created. Changing it empties the
+ * caches: propagate again before backpropagate. */
+int cattle_hip_convlstm_set_multiplicative_integration(cattle_hip_layer_t lstm, int enabled);
 
 #ifdef __cplusplus
 }

@@ -589,8 +589,9 @@ class SeqConvLSTM(object):
     GATES = ("forget", "write", "candidate", "read")
 
     def __init__(self, backend, dims, hidden, activations=(("sigmoid", 0), ("sigmoid", 0), ("tanh", 0), ("tanh", 0), ("sigmoid", 0)),
-                 conv_kw=None, foremost=True):
+                 conv_kw=None, foremost=True, mul_int=False):
         self.b, self.dims, self.hdims, self.foremost = backend, tuple(dims), (dims[0], dims[1], hidden), foremost
+        self.mul_int = mul_int         # LSTMNeuralNetwork<Scalar,Rank,MulInt = true>: weighted input * weighted output (:303-311)
         kw = conv_kw or {}
         self.main = {}
         for gate in self.GATES:
@@ -628,7 +629,11 @@ class SeqConvLSTM(object):
                     w = c["in_" + gate].pass_forward(F(x[:, i]), True)
                 if i > 0:
                     wo = c["out_" + gate].pass_forward(hidden, True)
-                    w = wo if w is None else w + wo
+                    if w is not None and self.mul_int:
+                        c["wi_" + gate], c["wo_" + gate] = w, wo
+                        w = w * wo
+                    else:
+                        w = wo if w is None else w + wo
                 pre[gate] = F(w)
             c["forget_f"] = c["act_forget"].pass_forward(pre["forget"], True)
             c["prev_state"] = state
@@ -660,10 +665,11 @@ class SeqConvLSTM(object):
             g_forget = c["act_forget"].pass_back(F(c["prev_state"] * state_grad))
             state_grad = state_grad * c["forget_f"]
             grads = (("read", g_read), ("candidate", g_cand), ("write", g_write), ("forget", g_forget))
+            both = self.mul_int and i != 0 and i < self.T_in            # :449-466: each side's gradient carries the other side
             if i != 0:
-                hidden_grad = sum(c["out_" + gate].pass_back(g) for gate, g in grads)
+                hidden_grad = sum(c["out_" + gate].pass_back(F(c["wi_" + gate] * g) if both else g) for gate, g in grads)
             if i < self.T_in:
-                parts = [c["in_" + gate].pass_back(g) for gate, g in grads]
+                parts = [c["in_" + gate].pass_back(F(c["wo_" + gate] * g) if both else g) for gate, g in grads]
                 if not self.foremost:
                     in_grad[:, i] = sum(parts)
         return in_grad

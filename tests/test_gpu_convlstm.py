@@ -19,12 +19,13 @@ SMOOTH = (("sigmoid", 0), ("sigmoid", 0), ("tanh", 0), ("tanh", 0), ("sigmoid", 
 EXOTIC = (("softsign", 0), ("swish", 1.3), ("softplus", 0), ("elu", 0.7), ("scaled", 0.5))
 
 
-def _pair(dtype, dims, hidden, acts, foremost, seq, seed, conv_kw=None):
+def _pair(dtype, dims, hidden, acts, foremost, seq, seed, conv_kw=None, mul_int=False):
     kw = conv_kw or {}
     net = ch.ConvLSTMNetwork(dtype, dims, hidden, kw.get("RH", 3), kw.get("RW", 3), kw.get("pv", 1), kw.get("ph", 1),
                              kw.get("dv", 0), kw.get("dh", 0), activations=[a for a, _ in acts],
-                             activation_params=[p for _, p in acts], output_seq_size_func=seq, foremost=foremost)
-    orc = hn.SeqConvLSTM(hn.OracleBackend(np.float64), dims, hidden, acts, conv_kw, foremost)
+                             activation_params=[p for _, p in acts], output_seq_size_func=seq, foremost=foremost,
+                             mul_int=mul_int)
+    orc = hn.SeqConvLSTM(hn.OracleBackend(np.float64), dims, hidden, acts, conv_kw, foremost, mul_int)
     g = hp.rng(seed)
     for k, layer in enumerate(orc.kernels()):
         rows = layer.get_params()[0].get_values().shape[0]
@@ -37,8 +38,8 @@ def _pair(dtype, dims, hidden, acts, foremost, seq, seed, conv_kw=None):
     return net, orc, g
 
 
-def _check(dtype, N, T_in, dims, hidden, acts, foremost, seq, seed=7, conv_kw=None):
-    net, orc, g = _pair(dtype, dims, hidden, acts, foremost, seq, seed, conv_kw)
+def _check(dtype, N, T_in, dims, hidden, acts, foremost, seq, seed=7, conv_kw=None, mul_int=False):
+    net, orc, g = _pair(dtype, dims, hidden, acts, foremost, seq, seed, conv_kw, mul_int)
     out_len, delay = seq(T_in)
     x = hp.normal(g, (N, T_in) + tuple(dims), dtype)
     go = hp.normal(g, (N, out_len, dims[0], dims[1], hidden), dtype)
@@ -82,6 +83,36 @@ def test_sequence_alignments(dtype, foremost):
 def test_other_activations_and_receptors(dtype):
     _check(dtype, 4, 3, (7, 6, 2), 5, EXOTIC, False, lambda T: (T, 0), conv_kw=dict(RH=3, RW=1, pv=1, ph=0))
     _check(dtype, 4, 3, (8, 8, 2), 3, SMOOTH, False, lambda T: (T, 0), conv_kw=dict(RH=3, RW=3, pv=2, ph=2, dv=1, dh=1))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("mul_int", [False, True])
+def test_dense_lstm_is_the_one_by_one_case(dtype, mul_int):
+    """An LSTM over vectors (the DenseKernelLayer networks of test/gradient_test.cpp:656-699: 32 inputs, 5 hidden units,
+    an output at every step of three, and with multiplicative integration only the last of five) is the same network
+    on 1 x 1 images with 1 x 1 receptors: the input size is the channel count."""
+    one = dict(RH=1, RW=1, pv=0, ph=0)
+    _check(dtype, 6, 3, (1, 1, 32), 5, SMOOTH, False, lambda T: (T, 0), conv_kw=one, mul_int=mul_int)
+    _check(dtype, 6, 5, (1, 1, 32), 5, SMOOTH, False, lambda T: (1, T - 1), conv_kw=one, mul_int=mul_int)
+    _check(dtype, 33, 4, (1, 1, 7), 5, SMOOTH, True, lambda T: (3, 2), conv_kw=one, mul_int=mul_int)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("foremost", [True, False])
+def test_multiplicative_integration(dtype, foremost):
+    """LSTMNeuralNetwork<Scalar,3,true> (the rank-3 network of test/gradient_test.cpp:735-741 and the alignments above)."""
+    dims, hidden = (6, 5, 3), 4
+    _check(dtype, 5, 4, dims, hidden, SMOOTH, foremost, lambda T: (T, 0), mul_int=True)
+    _check(dtype, 4, 3, dims, hidden, SMOOTH, foremost, lambda T: (4, 1), mul_int=True)       # two steps on the output side only
+    _check(dtype, 4, 1, dims, hidden, SMOOTH, foremost, lambda T: (1, 0), mul_int=True)       # a single step: nothing to multiply
+    _check(dtype, 3, 5, dims, hidden, EXOTIC, foremost, lambda T: (2, 1), mul_int=True)
+    # switching the rule on an existing network empties its caches and takes effect at the next pass
+    net, orc, (x, go) = _check(dtype, 4, 3, dims, hidden, SMOOTH, foremost, lambda T: (T, 0), mul_int=False)
+    plain = net.propagate(x)
+    net.set_multiplicative_integration(True)
+    with pytest.raises(ch.CattleHipError):
+        net.backpropagate(go)
+    assert not np.allclose(net.propagate(x), plain)
 
 
 def test_gradients_accumulate_and_updates_apply():
