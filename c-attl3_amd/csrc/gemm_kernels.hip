@@ -1066,8 +1066,11 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 			if (vars[i].bf >= g.F && vars[i].bf < vars[best_v].bf)
 				best_v = i;
 		/* enough short tiles for two or more per CU: the medium chunks, whose smaller LDS footprint lets four
-		 * blocks share a CU; fewer: the long chunks, with which one block keeps more loads in flight */
-		if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) >= 2 * NUM_CUS)
+		 * blocks share a CU. Tiles for at most half of the CUs: the medium chunks too, because the reduction of every
+		 * tile is then cut into parts and shorter chunks give twice as many parts to fill the chip with. In between:
+		 * the long chunks, with which one block keeps more loads in flight */
+		const long short_tiles = (long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf);
+		if (short_tiles >= 2 * NUM_CUS || short_tiles * 2 <= NUM_CUS)
 			best_v += SHORT;
 	}
 	const Tuning& tune = tuning();
