@@ -31,7 +31,8 @@ EXPORTS = [
     "cattle_hip_timer_destroy", "cattle_hip_timer_start", "cattle_hip_timer_stop", "cattle_hip_conv_create",
     "cattle_hip_transconv_create", "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
     "cattle_hip_batchnorm_set_stats_initialized", "cattle_hip_activation_create", "cattle_hip_pool_create",
-    "cattle_hip_convlstm_set_multiplicative_integration", "cattle_hip_dropout_create", "cattle_hip_reshape_create", "cattle_hip_broadcast_create",
+    "cattle_hip_convlstm_set_multiplicative_integration", "cattle_hip_layer_param_set_regularization",
+    "cattle_hip_layer_param_regularization_penalty", "cattle_hip_dropout_create", "cattle_hip_reshape_create", "cattle_hip_broadcast_create",
     "cattle_hip_layer_clone", "cattle_hip_layer_destroy", "cattle_hip_layer_input_dims",
     "cattle_hip_layer_output_dims", "cattle_hip_layer_is_input_layer", "cattle_hip_layer_set_input_layer",
     "cattle_hip_layer_empty_cache", "cattle_hip_layer_forward", "cattle_hip_layer_backward",
@@ -208,6 +209,18 @@ class Parameters(object):
         h = _hyper_array(tuple(hyper))
         _check(lib().cattle_hip_layer_param_optimizer_step(self._layer._h, _sz(self._index), ctypes.c_int(OPTIMIZERS[optimizer]),
                                                            h, _sz(epoch), _sz(timestep)))
+
+    def set_regularization(self, l1_lambda=0.0, l2_lambda=0.0):
+        """The parameter's ParameterRegularization: L1 (l1, 0), L2 (0, l2), elastic net (l1, l2), none (0, 0)
+        (parameter_regularization/*.hpp); optimizer_step then regularizes before it updates."""
+        _check(lib().cattle_hip_layer_param_set_regularization(self._layer._h, _sz(self._index), ctypes.c_double(l1_lambda),
+                                                               ctypes.c_double(l2_lambda)))
+
+    def get_regularization_penalty(self):
+        """Parameters::get_regularization_penalty (parameters/StandardParameters.hpp:128-132)."""
+        v = ctypes.c_double()
+        _check(lib().cattle_hip_layer_param_regularization_penalty(self._layer._h, _sz(self._index), ctypes.byref(v)))
+        return float(v.value)
 
     def sgd_update(self, learning_rate=1e-3):
         """VanillaSGDOptimizer::_update_params on the device (optimizer/VanillaSGDOptimizer.hpp:38-43)."""

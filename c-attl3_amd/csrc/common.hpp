@@ -177,13 +177,17 @@ template<typename T> struct OptParam {
 	T* grad; T* values; T* s0; T* s1; T* s2; T* wt_fwd; T* wt_dgrad;
 	size_t n;
 	int K, RHW, ldw_fwd, ldw_dgrad;
+	T l1, l2;           /* the lambdas of the parameter's regularization (both 0: none) */
 };
 template<typename T> struct OptBatch { OptParam<T> p[OPT_BATCH]; int count; };
 /* update + gradient reset of every parameter of the batch, one launch */
 template<typename T> void optimizer_step_many(int rule, const double hyper[4], size_t epoch, size_t timestep, const OptBatch<T>& batch);
 /* reset_grad: zero the gradient in the same kernel, after it has been used */
+/* l1, l2: the lambdas of the parameter's regularization, whose gradient is added before the update (both 0: none) */
 template<typename T> void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n,
-		T* grad, T* s0, T* s1, T* s2, T* values, bool reset_grad);
+		T* grad, T* s0, T* s1, T* s2, T* values, bool reset_grad, T l1, T l2);
+/* sums[0] = sum |v|, sums[1] = sum v^2 over a parameter's n values (device pointers) */
+template<typename T> void regularization_sums(size_t n, const T* values, T* sums);
 
 } /* namespace cattle_hip */
 

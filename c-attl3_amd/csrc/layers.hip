@@ -158,6 +158,7 @@ struct Param {
 	uint64_t derived_version[3] = { 0, 0, 0 };
 	DevBuf moments[3];                 /* the optimizer's state matrices, allocated (zeroed) on first use */
 	int moments_ready = 0;             /* how many of them are */
+	double reg_l1 = 0, reg_l2 = 0;     /* ParameterRegularization of the parameter: L1 and L2 lambdas (both 0: none) */
 	Param(size_t rows, size_t cols, bool optimizable, size_t esize) : rows(rows), cols(cols), optimizable(optimizable), esize(esize) {
 		values.ensure(bytes());
 		grad.ensure(bytes());
@@ -171,6 +172,8 @@ struct Param {
 		std::shared_ptr<Param> c = std::make_shared<Param>(rows, cols, optimizable, esize);
 		copy_in(c->values.p, values.p, CATTLE_HIP_DEVICE, bytes());
 		copy_in(c->grad.p, grad.p, CATTLE_HIP_DEVICE, bytes());
+		c->reg_l1 = reg_l1;
+		c->reg_l2 = reg_l2;
 		return c;
 	}
 };
@@ -900,14 +903,16 @@ void run_optimizer(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer 
 		p.moments_ready = i + 1;
 	}
 	const size_t n = p.rows * p.cols;
+	/* the step form is SGDOptimizer::_train's regularize + update + reset; the plain update is _update_params alone */
+	const double l1 = reset_grad ? p.reg_l1 : 0, l2 = reset_grad ? p.reg_l2 : 0;
 	if (p.esize == sizeof(float))
 		optimizer_update<float>((int) optimizer, hyper, epoch, timestep, n, static_cast<float*>(p.grad.p),
 				static_cast<float*>(p.moments[0].p), static_cast<float*>(p.moments[1].p), static_cast<float*>(p.moments[2].p),
-				static_cast<float*>(p.values.p), reset_grad);
+				static_cast<float*>(p.values.p), reset_grad, (float) l1, (float) l2);
 	else
 		optimizer_update<double>((int) optimizer, hyper, epoch, timestep, n, static_cast<double*>(p.grad.p),
 				static_cast<double*>(p.moments[0].p), static_cast<double*>(p.moments[1].p),
-				static_cast<double*>(p.moments[2].p), static_cast<double*>(p.values.p), reset_grad);
+				static_cast<double*>(p.moments[2].p), static_cast<double*>(p.values.p), reset_grad, l1, l2);
 	++p.version;
 }
 
@@ -942,6 +947,8 @@ void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices,
 		q.s1 = static_cast<T*>(p.moments[1].p);
 		q.s2 = static_cast<T*>(p.moments[2].p);
 		q.n = p.rows * p.cols;
+		q.l1 = (T) p.reg_l1;
+		q.l2 = (T) p.reg_l2;
 		q.wt_fwd = q.wt_dgrad = nullptr;
 		q.K = q.RHW = 1;
 		q.ldw_fwd = q.ldw_dgrad = 0;
@@ -1662,6 +1669,40 @@ int cattle_hip_layer_param_optimizer_update(cattle_hip_layer_t layer, size_t ind
 int cattle_hip_layer_param_optimizer_step(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer optimizer,
 		const double hyper[4], size_t epoch, size_t timestep) {
 	return guarded([&] { run_optimizer(layer, index, optimizer, hyper, epoch, timestep, true); });
+}
+
+int cattle_hip_layer_param_set_regularization(cattle_hip_layer_t layer, size_t index, double l1_lambda, double l2_lambda) {
+	return guarded([&] {
+		Param& p = optimizable_param(layer, index);
+		CATTLE_HIP_REQUIRE(l1_lambda == l1_lambda && l2_lambda == l2_lambda, "lambda is not a number");
+		p.reg_l1 = l1_lambda;
+		p.reg_l2 = l2_lambda;
+	});
+}
+
+int cattle_hip_layer_param_regularization_penalty(cattle_hip_layer_t layer, size_t index, double* penalty) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(penalty != nullptr, "null output pointer");
+		Param& p = param_at(as_layer(layer), index);
+		*penalty = 0;
+		if (!p.optimizable || (p.reg_l1 == 0 && p.reg_l2 == 0))        /* StandardParameters.hpp:128-132 */
+			return;
+		static DevBuf sums;
+		sums.ensure(2 * sizeof(double));
+		if (p.esize == sizeof(float)) {
+			float h[2];
+			regularization_sums<float>(p.rows * p.cols, static_cast<const float*>(p.values.p), static_cast<float*>(sums.p));
+			copy_out(h, CATTLE_HIP_HOST, sums.p, sizeof(h));
+			/* in the parameter's scalar type, as the reference computes it */
+			const float l1 = (float) p.reg_l1, l2 = (float) p.reg_l2;
+			*penalty = (double) ((l1 != 0 ? h[0] * l1 : 0.0f) + (l2 != 0 ? h[1] * (0.5f * l2) : 0.0f));
+			return;
+		}
+		double h[2];
+		regularization_sums<double>(p.rows * p.cols, static_cast<const double*>(p.values.p), static_cast<double*>(sums.p));
+		copy_out(h, CATTLE_HIP_HOST, sums.p, sizeof(h));
+		*penalty = (p.reg_l1 != 0 ? h[0] * p.reg_l1 : 0.0) + (p.reg_l2 != 0 ? h[1] * (0.5 * p.reg_l2) : 0.0);
+	});
 }
 
 int cattle_hip_optimizer_step_many(const cattle_hip_layer_t* layers, const size_t* indices, size_t count,

@@ -322,15 +322,54 @@ __device__ __forceinline__ T optimizer_element(const OptCoef<T>& k, T g, T v, T*
 	}
 }
 
+/* Parameters::regularize before the update (optimizer/SGDOptimizer.hpp:59-63, parameters/StandardParameters.hpp:133-136):
+ * the gradient plus d_function of the parameter's regularization at its values - L1 (e >= 0 ? lambda : -lambda,
+ * parameter_regularization/L1ParameterRegularization.hpp:35-37), L2 (e * lambda, L2ParameterRegularization.hpp:35-37)
+ * or both (ElasticNetParameterRegularization.hpp:40-42). Both lambdas zero: no regularization, the gradient as it is. */
+template<typename T>
+__device__ __forceinline__ T regularized_gradient(T g, T v, T l1, T l2) {
+	if (l1 == (T) 0 && l2 == (T) 0)
+		return g;
+	const T sign_term = v >= (T) 0 ? l1 : -l1;
+	const T reg = l2 == (T) 0 ? sign_term : (l1 == (T) 0 ? v * l2 : sign_term + v * l2);
+	return g + reg;
+}
+
 template<typename T, int RULE>
 __global__ __launch_bounds__(256)
 void optimizer_update_kernel(size_t total, OptCoef<T> k, T* __restrict__ grad, T* __restrict__ s0, T* __restrict__ s1,
-		T* __restrict__ s2, T* __restrict__ values, bool reset_grad) {
+		T* __restrict__ s2, T* __restrict__ values, bool reset_grad, T l1, T l2) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
 	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-		values[i] = optimizer_element<T, RULE>(k, grad[i], values[i], s0, s1, s2, i);
+		values[i] = optimizer_element<T, RULE>(k, regularized_gradient(grad[i], values[i], l1, l2), values[i], s0, s1, s2, i);
 		if (reset_grad)                 /* Parameters::reset_grad after the update (optimizer/SGDOptimizer.hpp:68-70) */
 			grad[i] = (T) 0;
+	}
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void regularization_sums_kernel(size_t n, const T* __restrict__ values, T* __restrict__ sums) {
+	__shared__ T part[2][256];
+	T a = (T) 0, q = (T) 0;
+	for (size_t i = threadIdx.x; i < n; i += 256) {
+		const T v = values[i];
+		a += v < (T) 0 ? -v : v;
+		q += v * v;
+	}
+	part[0][threadIdx.x] = a;
+	part[1][threadIdx.x] = q;
+	__syncthreads();
+	for (int w = 128; w > 0; w >>= 1) {
+		if ((int) threadIdx.x < w) {
+			part[0][threadIdx.x] += part[0][threadIdx.x + w];
+			part[1][threadIdx.x] += part[1][threadIdx.x + w];
+		}
+		__syncthreads();
+	}
+	if (threadIdx.x == 0) {
+		sums[0] = part[0][0];
+		sums[1] = part[1][0];
 	}
 }
 
@@ -351,7 +390,8 @@ void optimizer_step_many_kernel(OptBatch<T> batch, OptCoef<T> k) {
 		for (int j = 0; j < 4; ++j) {
 			const size_t i = (size_t) blockIdx.x * 1024 + tid + 256 * j;
 			if (i < q.n) {
-				q.values[i] = optimizer_element<T, RULE>(k, q.grad[i], q.values[i], q.s0, q.s1, q.s2, i);
+				q.values[i] = optimizer_element<T, RULE>(k, regularized_gradient(q.grad[i], q.values[i], q.l1, q.l2), q.values[i], q.s0, q.s1,
+						q.s2, i);
 				q.grad[i] = (T) 0;
 			}
 		}
@@ -368,7 +408,8 @@ void optimizer_step_many_kernel(OptBatch<T> batch, OptCoef<T> k) {
 		const int row = k0 + a, f = f0 + b + 8 * j;
 		if (row < q.K && f < F) {
 			const size_t i = (size_t) row + (size_t) q.K * f;
-			const T v = optimizer_element<T, RULE>(k, q.grad[i], q.values[i], q.s0, q.s1, q.s2, i);
+			const T v = optimizer_element<T, RULE>(k, regularized_gradient(q.grad[i], q.values[i], q.l1, q.l2), q.values[i], q.s0, q.s1,
+					q.s2, i);
 			q.values[i] = v;
 			q.grad[i] = (T) 0;
 			tile[b + 8 * j][a] = v;
@@ -559,14 +600,23 @@ OptCoef<T> optimizer_coefficients(int rule, const double hyper[4], size_t epoch,
 	default: LAUNCH(OPT_AMSGRAD); break; \
 	}
 
+/* sums[0] = sum |v|, sums[1] = sum v^2: what the regularization penalties are made of (L1: lambda * sum |v|,
+ * L2: 0.5 * lambda * sum v^2; parameter_regularization/L1ParameterRegularization.hpp:32-34,
+ * L2ParameterRegularization.hpp:32-34). One block, fixed order: parameters are at most a few million values. */
+template<typename T>
+void regularization_sums(size_t n, const T* values, T* sums) {
+	regularization_sums_kernel<T><<<1, 256, 0, stream()>>>(n, values, sums);
+	check_launch();
+}
+
 template<typename T>
 void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n, T* grad, T* s0, T* s1,
-		T* s2, T* values, bool reset_grad) {
+		T* s2, T* values, bool reset_grad, T l1, T l2) {
 	if (n == 0)
 		return;
 	const OptCoef<T> k = optimizer_coefficients<T>(rule, hyper, epoch, timestep);
 	const unsigned grid = flat_grid(n);
-#define CATTLE_HIP_LAUNCH_ONE(R) optimizer_update_kernel<T, R><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad)
+#define CATTLE_HIP_LAUNCH_ONE(R) optimizer_update_kernel<T, R><<<grid, 256, 0, stream()>>>(n, k, grad, s0, s1, s2, values, reset_grad, l1, l2)
 	CATTLE_HIP_OPT_DISPATCH(rule, CATTLE_HIP_LAUNCH_ONE)
 #undef CATTLE_HIP_LAUNCH_ONE
 	check_launch();
@@ -597,7 +647,8 @@ void optimizer_step_many(int rule, const double hyper[4], size_t epoch, size_t t
 #define CATTLE_HIP_INSTANTIATE_TRAIN(T) \
 template void loss_function<T>(int, int, int, int, T, const T*, const T*, T*); \
 template void loss_d_function<T>(int, int, int, int, T, T, const T*, const T*, T*); \
-template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, T*, T*, T*, T*, T*, bool); \
+template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, T*, T*, T*, T*, T*, bool, T, T); \
+template void regularization_sums<T>(size_t, const T*, T*); \
 template void optimizer_step_many<T>(int, const double*, size_t, size_t, const OptBatch<T>&);
 
 CATTLE_HIP_INSTANTIATE_TRAIN(float)

@@ -268,6 +268,23 @@ public:
 	inline std::vector<Scalar> get_param_grad(std::size_t index) const {
 		return fetch(index, &cattle_hip_layer_get_param_grad);
 	}
+	/**
+	 * The ParameterRegularization of parameter `index` (the weight_reg / bias_reg arguments of the reference's kernel
+	 * layers): L1 = (lambda, 0), L2 = (0, lambda), elastic net = (l1, l2). optimizer_step regularizes before it updates.
+	 */
+	inline void set_regularization(std::size_t index, Scalar l1_lambda, Scalar l2_lambda) {
+		check(cattle_hip_layer_param_set_regularization(handle, index, (double) l1_lambda, (double) l2_lambda));
+	}
+	/** The sum of Parameters::get_regularization_penalty over the layer's parameters (optimizer/SGDOptimizer.hpp:62). */
+	inline Scalar get_regularization_penalty() const {
+		const std::size_t n = num_params();
+		double total = 0, one = 0;
+		for (std::size_t i = 0; i < n; ++i) {
+			check(cattle_hip_layer_param_regularization_penalty(handle, i, &one));
+			total += one;
+		}
+		return (Scalar) total;
+	}
 	/** reset_grad of every parameter (optimizer/SGDOptimizer.hpp:68-70). */
 	inline void reset_grads() {
 		const std::size_t n = num_params();
@@ -497,6 +514,13 @@ public:
 	inline void reset_grads() {
 		for (std::size_t i = 0; i < layers.size(); ++i)
 			layers[i].reset_grads();
+	}
+	/** The regularization loss SGDOptimizer::_train reports beside the objective (optimizer/SGDOptimizer.hpp:59-63). */
+	inline Scalar get_regularization_penalty() const {
+		Scalar total = 0;
+		for (std::size_t i = 0; i < layers.size(); ++i)
+			total += layers[i].get_regularization_penalty();
+		return total;
 	}
 	/**
 	 * NeuralNetwork::save_all_unique_params_values / load_all_unique_params_values in the binary format

@@ -293,6 +293,18 @@ int cattle_hip_layer_param_sgd_update(cattle_hip_layer_t layer, size_t index, do
  * layers that share the parameter) and start at zero. */
 int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, double learning_rate, double l1_decay,
 		double l2_decay, double epsilon, size_t timestep);
+/* The ParameterRegularization of a Parameters object (the `weight_reg` / `bias_reg` constructor arguments of the kernel
+ * layers, parameters/StandardParameters.hpp:60-76): L1ParameterRegularization(lambda) = (lambda, 0),
+ * L2ParameterRegularization(lambda) = (0, lambda), ElasticNetParameterRegularization(l1, l2) = (l1, l2), none = (0, 0)
+ * (parameter_regularization/*.hpp). cattle_hip_layer_param_optimizer_step and cattle_hip_optimizer_step_many then add
+ * the regularization's d_function at the current values to the gradient before the update, as SGDOptimizer::_train
+ * does through Parameters::regularize (optimizer/SGDOptimizer.hpp:59-63, StandardParameters.hpp:133-136);
+ * cattle_hip_layer_param_optimizer_update, which is _update_params alone, does not. */
+int cattle_hip_layer_param_set_regularization(cattle_hip_layer_t layer, size_t index, double l1_lambda, double l2_lambda);
+/* Parameters::get_regularization_penalty (StandardParameters.hpp:128-132): l1 * sum |v| + 0.5 * l2 * sum v^2, 0 for
+ * parameters without regularization or that are not optimizable. */
+int cattle_hip_layer_param_regularization_penalty(cattle_hip_layer_t layer, size_t index, double* penalty);
+
 /* The optimizer's _fit (e.g. optimizer/AdamOptimizer.hpp:55-65): zero the state matrices. */
 int cattle_hip_layer_param_reset_optimizer_state(cattle_hip_layer_t layer, size_t index);
 

@@ -30,6 +30,7 @@
  *   other optimizers    pinned: torch's SGD (momentum, Nesterov), Adagrad, RMSprop, Adadelta and Adamax where the
  *                       recurrences coincide; first-step closed forms and the running-maximum property for
  *                       Nadam and AMSGrad, whose reference formulas differ from torch's.
+ *   regularization      pinned: torch's weight decay (L2), hand-worked values, central differences of the penalty.
  *   SGD / Adam updates  pinned: numpy restatement in float64, first-step closed form, and torch's Adam
  *                       in the limit where the two formulas coincide.
  * What stays unpinned is only the bit pattern of Eigen's own summation order and of its
@@ -1008,6 +1009,23 @@ int broadcast_backward(i64 N, i64 H, i64 W, i64 C, i64 bh, i64 bw, i64 bc, const
 	return 0;
 }
 
+/* ParameterRegularization::function and d_function for L1 (l2 = 0; parameter_regularization/L1ParameterRegularization.hpp:32-37),
+ * L2 (l1 = 0; L2ParameterRegularization.hpp:32-37) and elastic net (ElasticNetParameterRegularization.hpp:36-42):
+ * penalty = l1 sum |v| + 0.5 l2 sum v^2; gradient = (v >= 0 ? l1 : -l1) + v l2, which Parameters::regularize adds to the
+ * gradient before the update (parameters/StandardParameters.hpp:133-136). */
+template<typename T>
+int regularization(i64 n, T l1, T l2, const T* values, T* penalty, T* grad) {
+	T abs_sum = 0, sq_sum = 0;
+	for (i64 i = 0; i < n; ++i) {
+		abs_sum += std::abs(values[i]);
+		sq_sum += values[i] * values[i];
+		const T sign_term = values[i] >= 0 ? l1 : -l1;
+		grad[i] = l2 == 0 ? sign_term : (l1 == 0 ? values[i] * l2 : sign_term + values[i] * l2);
+	}
+	*penalty = (l1 != 0 ? abs_sum * l1 : (T) 0) + (l2 != 0 ? sq_sum * ((T) .5 * l2) : (T) 0);
+	return 0;
+}
+
 /* optimizer/VanillaSGDOptimizer.hpp:38-43 */
 template<typename T>
 int sgd_update(i64 n, T lr, const T* grad, T* values) {
@@ -1166,6 +1184,8 @@ extern "C" int oracle_loss_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double
 	return loss_function<T>(kind, N, Ts, V, (T) eps, out, obj, losses); } \
 extern "C" int oracle_loss_d_function_##SFX(int kind, i64 N, i64 Ts, i64 V, double eps, double scale, const T* out, \
 		const T* obj, T* grad) { return loss_d_function<T>(kind, N, Ts, V, (T) eps, (T) scale, out, obj, grad); } \
+extern "C" int oracle_regularization_##SFX(i64 n, double l1, double l2, const T* values, T* penalty, T* grad) { \
+	return regularization<T>(n, (T) l1, (T) l2, values, penalty, grad); } \
 extern "C" int oracle_sgd_update_##SFX(i64 n, double lr, const T* grad, T* values) { \
 	return sgd_update<T>(n, (T) lr, grad, values); } \
 extern "C" int oracle_optimizer_update_##SFX(int rule, const double* h, i64 epoch, i64 timestep, i64 n, const T* grad, T* s0, \

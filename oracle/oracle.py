@@ -403,6 +403,16 @@ def loss_d_function(kind, out, obj, eps=1e-5, scale=1.0, sequential=False, negat
     return grad
 
 
+def regularization(values, l1=0.0, l2=0.0):
+    """(penalty, gradient) of a parameter's regularization at `values`: L1 (l1, 0), L2 (0, l2) or elastic net."""
+    dt = values.dtype
+    v = _f(values, dt)
+    grad = np.empty(v.shape, dtype=dt, order="F")
+    penalty = np.zeros((1,), dtype=dt)
+    _call("regularization", dt, *_ll(v.size), ctypes.c_double(l1), ctypes.c_double(l2), _p(v), _p(penalty), _p(grad))
+    return float(penalty[0]), grad
+
+
 def sgd_update(values, grad, lr=1e-3):
     """Returns the updated values (the inputs are left alone)."""
     dt = values.dtype

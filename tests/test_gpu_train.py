@@ -602,6 +602,56 @@ def test_optimizer_step_of_a_whole_network(rule, hyper, dtype):
                 assert not np.any(pb.get_grad())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("l1,l2", [(0.03, 0.0), (0.0, 0.2), (0.03, 0.2)])
+@pytest.mark.parametrize("rule,hyper", [ALL_OPTIMIZERS[0], ALL_OPTIMIZERS[6]])
+def test_regularized_optimizer_steps(rule, hyper, l1, l2, dtype):
+    """Parameters with an L1, L2 or elastic-net regularization: optimizer_step and the step of a whole network add its
+    gradient before the update (SGDOptimizer::_train: regularize, update, reset), the plain update does not, and the
+    penalty is Parameters::get_regularization_penalty."""
+    tol = TOL[np.dtype(dtype)]
+    layer, g, _, _ = _dense_with_grads(dtype, 1301)
+    _accumulate(layer, g, dtype)
+    conv = ch.ConvKernelLayer(dtype, (6, 5, 3), 4)
+    x = hp.normal(g, (8, 6, 5, 3), dtype)
+    conv.get_params()[0].set_values(hp.normal(g, (27, 4), dtype, 0.3))
+    conv.pass_forward(x, True)                                   # builds the prepared weight layout the step rewrites
+    conv.pass_back(hp.normal(g, (8, 6, 5, 4), dtype))
+    params = [layer.get_params()[0], conv.get_params()[0], conv.get_params()[1]]
+    for p in params:
+        p.set_regularization(l1, l2)
+    lam1, lam2 = float(dtype(l1)), float(dtype(l2))
+    hyper32 = [float(dtype(h)) for h in hyper]
+    want = []
+    for p in params:
+        v64, g64 = np.asarray(p.get_values(), np.float64), np.asarray(p.get_grad(), np.float64)
+        pen, reg = oracle.regularization(v64, lam1, lam2)
+        assert abs(p.get_regularization_penalty() - pen) <= tol * max(1.0, abs(pen))
+        new, _ = oracle.optimizer_update(rule, v64, g64 + reg, [np.zeros_like(v64)] * 3, hyper32, 0, 0)
+        want.append(new)
+    params[0].optimizer_step(rule, hyper, 0, 0)                  # one parameter
+    ch.ParameterList(params[1:]).optimizer_step(rule, hyper, 0, 0)         # several in one launch
+    for p, w in zip(params, want):
+        assert hp.rel_err(p.get_values(), w) < tol
+        assert np.all(p.get_grad() == 0)
+    # the convolution uses the regularized weights (its prepared layout was rewritten by the step)
+    ref, _ = oracle.conv_forward(np.asarray(x, np.float64), want[1], want[2], return_cache=True)
+    assert hp.rel_err(conv.pass_forward(x, True), ref) < tol
+    # the plain update is _update_params alone: no regularization
+    other, g2, _, _ = _dense_with_grads(dtype, 1302)
+    _accumulate(other, g2, dtype)
+    q = other.get_params()[0]
+    q.set_regularization(l1, l2)
+    v64, g64 = np.asarray(q.get_values(), np.float64), np.asarray(q.get_grad(), np.float64)
+    plain, _ = oracle.optimizer_update(rule, v64, g64, [np.zeros_like(v64)] * 3, hyper32, 0, 0)
+    q.optimizer_update(rule, hyper, 0, 0)
+    assert hp.rel_err(q.get_values(), plain) < tol
+    # none: penalty 0; a clone keeps the regularization
+    q.set_regularization(0.0, 0.0)
+    assert q.get_regularization_penalty() == 0.0
+    assert conv.clone().get_params()[0].get_regularization_penalty() == pytest.approx(conv.get_params()[0].get_regularization_penalty())
+
+
 def test_optimizer_argument_checks():
     layer, g, w, b = _dense_with_grads(np.float32, 1221)
     prm = layer.get_params()[0]

@@ -216,6 +216,48 @@ def test_sequential_losses_are_per_time_step(kind, dtype):
     assert hp.rel_err(total, acc) < TOL[np.dtype(dtype)]
 
 
+def test_regularization_by_hand_and_by_differences():
+    """parameter_regularization/*.hpp: L1 = lambda sum |v| with gradient +-lambda (+lambda at zero), L2 = lambda / 2 sum v^2
+    with gradient lambda v, the elastic net their sum."""
+    v = np.asfortranarray(np.array([[1.0, -2.0], [0.0, 0.5]]))
+    pen, grad = oracle.regularization(v, l1=0.1)
+    assert abs(pen - 0.35) < 1e-15 and np.array_equal(grad, [[0.1, -0.1], [0.1, 0.1]])
+    pen, grad = oracle.regularization(v, l2=0.2)
+    assert abs(pen - 0.1 * 5.25) < 1e-15 and np.allclose(grad, [[0.2, -0.4], [0.0, 0.1]], atol=1e-16)
+    pen, grad = oracle.regularization(v, l1=0.1, l2=0.2)
+    assert abs(pen - 0.875) < 1e-15 and np.allclose(grad, [[0.3, -0.5], [0.1, 0.2]], atol=1e-16)
+    pen, grad = oracle.regularization(v)
+    assert pen == 0 and np.all(grad == 0)
+    g = hp.rng(920)
+    w = hp.normal(g, (5, 4), np.float64)
+    _, grad = oracle.regularization(w, l1=0.03, l2=0.7)
+    h = 1e-6
+    for idx in [(0, 0), (2, 3), (4, 1)]:
+        up, dn = w.copy(order="F"), w.copy(order="F")
+        up[idx] += h
+        dn[idx] -= h
+        num = (oracle.regularization(up, l1=0.03, l2=0.7)[0] - oracle.regularization(dn, l1=0.03, l2=0.7)[0]) / (2 * h)
+        assert abs(num - grad[idx]) < 1e-8
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_l2_regularized_sgd_is_torch_weight_decay(dtype):
+    """SGDOptimizer::_train regularizes, then updates (optimizer/SGDOptimizer.hpp:59-64): with L2 regularization and
+    vanilla SGD that is torch's SGD with weight_decay = lambda."""
+    g = hp.rng(921)
+    w0, lam, lr = hp.normal(g, (6, 4), dtype), 0.05, 0.1
+    wt = torch.tensor(np.asarray(w0, np.float64), requires_grad=True)
+    opt = torch.optim.SGD([wt], lr=lr, weight_decay=lam)
+    w = w0
+    for _ in range(3):
+        grad = hp.normal(g, (6, 4), dtype)
+        wt.grad = torch.tensor(np.asarray(grad, np.float64))
+        opt.step()
+        _, reg = oracle.regularization(w, l2=lam)
+        w = oracle.sgd_update(w, grad + reg, lr)
+    assert hp.rel_err(w, wt.detach().numpy()) < TOL[np.dtype(dtype)]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_sgd_update(dtype):
     g = hp.rng(906)
