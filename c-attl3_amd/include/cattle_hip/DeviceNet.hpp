@@ -19,7 +19,9 @@
 #include <cassert>
 #include <cstddef>
 #include <fstream>
+#include <cmath>
 #include <memory>
+#include <random>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -39,6 +41,107 @@ inline void check(int status) {
 template<typename Scalar> struct Code;
 template<> struct Code<float> { static constexpr cattle_hip_dtype value = CATTLE_HIP_F32; };
 template<> struct Code<double> { static constexpr cattle_hip_dtype value = CATTLE_HIP_F64; };
+
+/**
+ * The parameter initializations of the parameter_initialization/ headers on a column-major host matrix (the values are
+ * uploaded by DeviceLayer::init_params). They use the standard library exactly as the reference does - a default-seeded
+ * std::default_random_engine per matrix and std::normal_distribution, filled column by column
+ * (GaussianParameterInitialization.hpp:34-44) - so a build against the same standard library starts from the reference's
+ * initial values.
+ */
+template<typename Scalar>
+class ParameterInitialization {
+public:
+	virtual ~ParameterInitialization() { }
+	virtual void apply(std::vector<Scalar>& values, std::size_t rows, std::size_t cols) const = 0;
+};
+
+/** parameter_initialization/GaussianParameterInitialization.hpp:28-52 */
+template<typename Scalar>
+class GaussianParameterInitialization : public ParameterInitialization<Scalar> {
+public:
+	inline GaussianParameterInitialization(Scalar mean = 0, Scalar sd_scaling_factor = 1) : mean(mean),
+			sd_scaling_factor(sd_scaling_factor) {
+		assert(sd_scaling_factor > 0);
+	}
+	inline void apply(std::vector<Scalar>& values, std::size_t rows, std::size_t cols) const {
+		std::default_random_engine gen;
+		std::normal_distribution<Scalar> dist(mean, sd_scaling_factor * _sd((unsigned) rows, (unsigned) cols));
+		values.resize(rows * cols);
+		for (std::size_t i = 0; i < cols; ++i)
+			for (std::size_t j = 0; j < rows; ++j)
+				values[j + rows * i] = dist(gen);
+	}
+protected:
+	inline virtual Scalar _sd(unsigned fan_ins, unsigned fan_outs) const {
+		return 1;
+	}
+private:
+	const Scalar mean, sd_scaling_factor;
+};
+
+/** parameter_initialization/HeParameterInitialization.hpp:27-36 */
+template<typename Scalar>
+class HeParameterInitialization : public GaussianParameterInitialization<Scalar> {
+public:
+	inline HeParameterInitialization(Scalar sd_scaling_factor = 1) : GaussianParameterInitialization<Scalar>(0, sd_scaling_factor) { }
+protected:
+	inline Scalar _sd(unsigned fan_ins, unsigned fan_outs) const {
+		return std::sqrt(2 / (Scalar) fan_ins);
+	}
+};
+
+/** parameter_initialization/GlorotParameterInitialization.hpp:27-36 */
+template<typename Scalar>
+class GlorotParameterInitialization : public GaussianParameterInitialization<Scalar> {
+public:
+	inline GlorotParameterInitialization(Scalar sd_scaling_factor = 1) : GaussianParameterInitialization<Scalar>(0, sd_scaling_factor) { }
+protected:
+	inline Scalar _sd(unsigned fan_ins, unsigned fan_outs) const {
+		return std::sqrt(2 / (Scalar) (fan_ins + fan_outs));
+	}
+};
+
+/** parameter_initialization/LeCunParameterInitialization.hpp:27-36 */
+template<typename Scalar>
+class LeCunParameterInitialization : public GaussianParameterInitialization<Scalar> {
+public:
+	inline LeCunParameterInitialization(Scalar sd_scaling_factor = 1) : GaussianParameterInitialization<Scalar>(0, sd_scaling_factor) { }
+protected:
+	inline Scalar _sd(unsigned fan_ins, unsigned fan_outs) const {
+		return std::sqrt(1 / (Scalar) fan_ins);
+	}
+};
+
+/** parameter_initialization/ConstantParameterInitialization.hpp:24-33 (Zero and One are its 0 and 1) */
+template<typename Scalar>
+class ConstantParameterInitialization : public ParameterInitialization<Scalar> {
+public:
+	inline ConstantParameterInitialization(Scalar constant) : constant(constant) { }
+	inline void apply(std::vector<Scalar>& values, std::size_t rows, std::size_t cols) const {
+		values.assign(rows * cols, constant);
+	}
+private:
+	const Scalar constant;
+};
+
+/** parameter_initialization/IncrementalParameterInitialization.hpp:24-42 */
+template<typename Scalar>
+class IncrementalParameterInitialization : public ParameterInitialization<Scalar> {
+public:
+	inline IncrementalParameterInitialization(Scalar start, Scalar inc) : start(start), inc(inc) { }
+	inline void apply(std::vector<Scalar>& values, std::size_t rows, std::size_t cols) const {
+		values.resize(rows * cols);
+		Scalar val = start;
+		for (std::size_t i = 0; i < cols; ++i)
+			for (std::size_t j = 0; j < rows; ++j) {
+				values[j + rows * i] = val;
+				val += inc;
+			}
+	}
+private:
+	const Scalar start, inc;
+};
 
 /** A tensor in device memory; move-only owner of its buffer (the role of CuDNNTensor in the reference). */
 template<typename Scalar>
@@ -126,13 +229,30 @@ public:
 		check(cattle_hip_conv_create(Code<Scalar>::value, input_dims[0], input_dims[1], input_dims[2], filters,
 				receptor_height, receptor_width, vertical_padding, horizontal_padding, vertical_stride, horizontal_stride,
 				vertical_dilation, horizontal_dilation, &h));
-		return DeviceLayer(h);
+		DeviceLayer layer(h);
+		layer.kernel_layer = true;
+		return layer;
+	}
+	/* layer/kernel/TransConvKernelLayer.hpp:290-304 */
+	inline static DeviceLayer trans_conv(const Dims& input_dims, std::size_t filters, std::size_t receptor_height = 3,
+			std::size_t receptor_width = 3, std::size_t vertical_padding = 1, std::size_t horizontal_padding = 1,
+			std::size_t vertical_stride = 1, std::size_t horizontal_stride = 1, std::size_t vertical_dilation = 0,
+			std::size_t horizontal_dilation = 0) {
+		cattle_hip_layer_t h = nullptr;
+		check(cattle_hip_transconv_create(Code<Scalar>::value, input_dims[0], input_dims[1], input_dims[2], filters,
+				receptor_height, receptor_width, vertical_padding, horizontal_padding, vertical_stride, horizontal_stride,
+				vertical_dilation, horizontal_dilation, &h));
+		DeviceLayer layer(h);
+		layer.kernel_layer = true;
+		return layer;
 	}
 	/* layer/kernel/DenseKernelLayer.hpp:61-77 */
 	inline static DeviceLayer dense(const Dims& input_dims, std::size_t output_size) {
 		cattle_hip_layer_t h = nullptr;
 		check(cattle_hip_dense_create(Code<Scalar>::value, input_dims[0] * input_dims[1] * input_dims[2], output_size, &h));
-		return DeviceLayer(h, input_dims);
+		DeviceLayer layer(h, input_dims);
+		layer.kernel_layer = true;
+		return layer;
 	}
 	/* layer/BatchNormLayer.hpp:66-101 (per channel) / :334-361 (per activation) */
 	inline static DeviceLayer batch_norm(const Dims& dims, bool per_last_rank = true, Scalar norm_avg_decay = .1,
@@ -179,7 +299,7 @@ public:
 	}
 	inline DeviceLayer(DeviceLayer&& other) : handle(other.handle), in_dims(other.in_dims), out_dims(other.out_dims),
 			cached_in(std::move(other.cached_in)), cached_out(std::move(other.cached_out)),
-			params_per_column(other.params_per_column) {
+			params_per_column(other.params_per_column), kernel_layer(other.kernel_layer) {
 		other.handle = nullptr;
 	}
 	DeviceLayer(const DeviceLayer&) = delete;
@@ -267,6 +387,22 @@ public:
 	}
 	inline std::vector<Scalar> get_param_grad(std::size_t index) const {
 		return fetch(index, &cattle_hip_layer_get_param_grad);
+	}
+	/** Whether the layer is a kernel layer: parameter 0 its weight matrix, parameter 1 its bias. */
+	inline bool is_kernel_layer() const {
+		return kernel_layer;
+	}
+	/**
+	 * Parameters::init_values (parameters/StandardParameters.hpp:91-95) for parameter `index`: the initialization applied
+	 * to a host matrix of the parameter's shape and uploaded.
+	 */
+	inline void init_params(std::size_t index, const ParameterInitialization<Scalar>& init) {
+		std::size_t rows, cols;
+		bool optimizable;
+		param_shape(index, rows, cols, optimizable);
+		std::vector<Scalar> values;
+		init.apply(values, rows, cols);
+		set_param_values(index, values.data());
 	}
 	/**
 	 * The ParameterRegularization of parameter `index` (the weight_reg / bias_reg arguments of the reference's kernel
@@ -395,7 +531,7 @@ public:
 		}
 	}
 private:
-	inline explicit DeviceLayer(cattle_hip_layer_t handle) : handle(handle), params_per_column(false) {
+	inline explicit DeviceLayer(cattle_hip_layer_t handle) : handle(handle), params_per_column(false), kernel_layer(false) {
 		std::size_t d[3];
 		check(cattle_hip_layer_input_dims(handle, d));
 		in_dims = Dims{ { d[0], d[1], d[2] } };
@@ -407,7 +543,7 @@ private:
 		in_dims = in;
 	}
 	inline DeviceLayer(cattle_hip_layer_t handle, const Dims& in, const Dims& out) : handle(handle), in_dims(in),
-			out_dims(out), params_per_column(false) { }
+			out_dims(out), params_per_column(false), kernel_layer(false) { }
 	template<typename Fn>
 	inline void for_each_optimizable(Fn fn) {
 		const std::size_t n = num_params();
@@ -431,6 +567,7 @@ private:
 	Dims in_dims, out_dims;
 	DeviceTensor<Scalar> cached_in, cached_out;
 	bool params_per_column;
+	bool kernel_layer;          /* a weight matrix (parameter 0) and a bias (parameter 1): conv, transposed conv, dense */
 };
 
 /**
@@ -514,6 +651,20 @@ public:
 	inline void reset_grads() {
 		for (std::size_t i = 0; i < layers.size(); ++i)
 			layers[i].reset_grads();
+	}
+	/**
+	 * NeuralNetwork::init (core/NeuralNetwork.hpp:173-176) with one weight initialization for all kernel layers: the
+	 * weight matrices (parameter 0 of the layers that have a weight matrix and a bias) take `weight_init`; biases,
+	 * batch-norm and activation parameters are back at the values their layers are created with (zero biases,
+	 * gamma 1 / beta 0, the constant of PReLU and PSwish), which is what the reference's layers initialize them to.
+	 */
+	inline void init(const ParameterInitialization<Scalar>& weight_init) {
+		for (std::size_t l = 0; l < layers.size(); ++l) {
+			if (!layers[l].is_kernel_layer())
+				continue;
+			layers[l].init_params(0, weight_init);
+			layers[l].init_params(1, ConstantParameterInitialization<Scalar>(0));
+		}
 	}
 	/** The regularization loss SGDOptimizer::_train reports beside the objective (optimizer/SGDOptimizer.hpp:59-63). */
 	inline Scalar get_regularization_penalty() const {

@@ -296,7 +296,7 @@ int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, d
 /* The ParameterRegularization of a Parameters object (the `weight_reg` / `bias_reg` constructor arguments of the kernel
  * layers, parameters/StandardParameters.hpp:60-76): L1ParameterRegularization(lambda) = (lambda, 0),
  * L2ParameterRegularization(lambda) = (0, lambda), ElasticNetParameterRegularization(l1, l2) = (l1, l2), none = (0, 0)
- * (parameter_regularization/*.hpp). cattle_hip_layer_param_optimizer_step and cattle_hip_optimizer_step_many then add
+ * (the headers of parameter_regularization/). cattle_hip_layer_param_optimizer_step and cattle_hip_optimizer_step_many then add
  * the regularization's d_function at the current values to the gradient before the update, as SGDOptimizer::_train
  * does through Parameters::regularize (optimizer/SGDOptimizer.hpp:59-63, StandardParameters.hpp:133-136);
  * cattle_hip_layer_param_optimizer_update, which is _update_params alone, does not. */

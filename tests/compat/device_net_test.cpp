@@ -13,6 +13,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <random>
 #include <string>
 
 using namespace cattle::hip::device;
@@ -214,6 +215,57 @@ static void run(const std::string& tag) {
 			}
 			record(tag + ".gan" + std::to_string(stacked) + ".losses", sizeof(Scalar), { losses.size() }, losses.data());
 		}
+	}
+	{
+		/* NeuralNetwork::init with He initialization (as examples/cifar_convnet.cpp:21 sets it up): the weights must be
+		 * what the reference's GaussianParameterInitialization::apply produces with the same standard library - a
+		 * default-seeded engine per matrix, filled column by column - and the biases zero */
+		std::vector<DL> layers;
+		layers.push_back(DL::conv(Dims{ { 6, 6, 3 } }, 4));
+		layers.push_back(DL::batch_norm(layers.back().get_output_dims()));
+		layers.push_back(DL::trans_conv(layers.back().get_output_dims(), 2, 4, 4, 1, 1, 2, 2));
+		layers.push_back(DL::dense(layers.back().get_output_dims(), 5));
+		DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
+		net.init(HeParameterInitialization<Scalar>((Scalar) 1e-1));
+		std::vector<Scalar> ok;
+		for (std::size_t l = 0; l < net.get_layers().size(); ++l) {
+			DL& layer = net.get_layers()[l];
+			if (!layer.is_kernel_layer())
+				continue;
+			std::size_t rows, cols;
+			bool optimizable;
+			layer.param_shape(0, rows, cols, optimizable);
+			std::default_random_engine gen;
+			std::normal_distribution<Scalar> dist(0, (Scalar) 1e-1 * std::sqrt(2 / (Scalar) rows));
+			std::vector<Scalar> want(rows * cols);
+			for (std::size_t i = 0; i < cols; ++i)
+				for (std::size_t j = 0; j < rows; ++j)
+					want[j + rows * i] = dist(gen);
+			ok.push_back(layer.get_param_values(0) == want ? (Scalar) 1 : (Scalar) 0);
+			const std::vector<Scalar> bias = layer.get_param_values(1);
+			Scalar nonzero = 0;
+			for (std::size_t i = 0; i < bias.size(); ++i)
+				nonzero += bias[i] != 0;
+			ok.push_back(nonzero == 0 ? (Scalar) 1 : (Scalar) 0);
+			record(tag + ".init_he.w" + std::to_string(l), sizeof(Scalar), { rows, cols }, want.data());
+		}
+		/* batch norm is no kernel layer: its first optimizable parameter, gamma, keeps its ones */
+		Scalar gamma_ok = 0;
+		for (std::size_t i = 0; i < net.get_layers()[1].num_params(); ++i) {
+			std::size_t rows, cols;
+			bool optimizable;
+			net.get_layers()[1].param_shape(i, rows, cols, optimizable);
+			if (optimizable) {
+				const std::vector<Scalar> gamma = net.get_layers()[1].get_param_values(i);
+				gamma_ok = gamma[0] == 1 && gamma[gamma.size() - 1] == 1 ? (Scalar) 1 : (Scalar) 0;
+				break;
+			}
+		}
+		ok.push_back(gamma_ok);
+		record(tag + ".init_he.ok", sizeof(Scalar), { ok.size() }, ok.data());
+		const Dims out_dims = net.get_layers()[2].get_output_dims();
+		const std::vector<Scalar> dims = { (Scalar) out_dims[0], (Scalar) out_dims[1], (Scalar) out_dims[2] };
+		record(tag + ".init_he.transconv_dims", sizeof(Scalar), { 3 }, dims.data());
 	}
 	{
 		/* another loss of the loss/ directory, wrapped as NegatedLoss wraps it */

@@ -64,6 +64,27 @@ def out_shape(net):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("tag", ["f32", "f64"])
+def test_network_init_is_the_reference_initialization(records, tag):
+    """DeviceFeedforwardNetwork::init(He): bit for bit what GaussianParameterInitialization::apply makes of the same standard
+    library (checked inside the C++ driver), zero biases, untouched batch-norm parameters; here the moments of the
+    recorded weights (standard deviation 0.1 sqrt(2 / fan_in)) and the transposed convolution's output dimensions."""
+    assert np.all(records[tag + ".init_he.ok"] == 1) and records[tag + ".init_he.ok"].size == 7
+    assert tuple(records[tag + ".init_he.transconv_dims"]) == oracle.transconv_out_dims(6, 6, 4, 4, 1, 1, 2, 2, 0, 0) + (2,)
+    for key, fan_in in ((".init_he.w0", 27), (".init_he.w2", 4), (".init_he.w3", 12 * 12 * 2)):
+        w = np.asarray(records[tag + key], np.float64)
+        assert w.shape[0] == fan_in
+        sd = 0.1 * np.sqrt(2.0 / fan_in)
+        assert abs(w.std() / sd - 1) < 4 / np.sqrt(2 * w.size) + 0.02 and abs(w.mean()) < 4 * sd / np.sqrt(w.size)
+    # every matrix starts a fresh default-seeded engine: matrices draw the same stream, scaled by their own deviation
+    a, b = records[tag + ".init_he.w0"], records[tag + ".init_he.w2"]
+    n = min(a.size, b.size)
+    ra = a.reshape(-1, order="F")[:n] / (0.1 * np.sqrt(2.0 / 27))
+    rb = b.reshape(-1, order="F")[:n] / (0.1 * np.sqrt(2.0 / 4))
+    assert np.allclose(ra, rb, rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", ["f32", "f64"])
 def test_stacked_network_with_a_frozen_module(records, tag):
     """DeviceStackedNetwork and set_frozen against the same training loop spelled out on two separate networks."""
     spelled = {k[len(tag) + 6:]: v for k, v in records.items() if k.startswith(tag + ".gan0.")}
