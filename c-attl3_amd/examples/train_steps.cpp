@@ -138,7 +138,14 @@ int main(int argc, char** argv) {
 			layers.push_back(DL::dense(layers.back().get_output_dims(), 10));
 			layers.push_back(DL::activation(CATTLE_HIP_ACT_SOFTMAX, layers.back().get_output_dims(), (Scalar) 1e-5));
 			DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
-			init_weights(net, g);
+			/* the example's initializations (examples/cifar_convnet.cpp:21-22): He for the convolutions, Glorot for the
+			 * dense layers, both scaled by 0.1 */
+			const HeParameterInitialization<Scalar> conv_init((Scalar) 1e-1);
+			const GlorotParameterInitialization<Scalar> dense_init((Scalar) 1e-1);
+			net.get_layers()[0].init_params(0, conv_init);
+			net.get_layers()[3].init_params(0, conv_init);
+			net.get_layers()[7].init_params(0, dense_init);
+			net.get_layers()[10].init_params(0, dense_init);
 			std::vector<Scalar> x = random_values(batch * 32 * 32 * 3, g, 0.5), y = one_hot(batch, 10, g);
 			for (std::size_t i = 0; i < x.size(); ++i)
 				x[i] += (Scalar) 0.5;                                   /* pixel values in [0, 1) */
