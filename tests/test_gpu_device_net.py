@@ -224,3 +224,17 @@ def test_lstm_parameter_files_follow_the_layer_order(records, tag, dtype):
     assert not os.path.exists(os.path.join(records["__dir__"], "%s_lstm_params_16.prms" % tag))
     assert np.array_equal(r["out_reloaded"], r["out"])
 
+
+@pytest.mark.gpu
+def test_the_cpp_example_runs():
+    """c-attl3_amd/examples/train_steps (built by __graft_entry__.build()): the two benchmark networks and the network of
+    the reference's cifar_convnet example train from C++ and report their time per step."""
+    import json
+    exe = os.path.join(HERE, "..", "c-attl3_amd", "examples", "train_steps")
+    if not os.path.exists(exe):
+        pytest.fail("c-attl3_amd/examples/train_steps is not built: run __graft_entry__.build()")
+    out = subprocess.run([exe, "3", "1"], stdout=subprocess.PIPE, check=True, timeout=120).stdout.decode()
+    line = json.loads(out.strip().splitlines()[-1])
+    for key in ("mlp_784_512_256_10_batch256_sgd_ms", "convnet_32x32x3_batch128_adam_ms", "reference_cifar_example_batch200_nadam_ms"):
+        assert 0 < line[key] < 100
+
