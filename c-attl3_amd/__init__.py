@@ -5,4 +5,4 @@ is the Python binding used by the tests and the benchmark; the directory name is
 identifier, so load it with importlib.import_module("c-attl3_amd").
 """
 from .binding import *  # noqa: F401,F403
-from .binding import build, lib, init, synchronize, trim, EXPORTS, LIB_PATH, CattleHipError  # noqa: F401
+from .binding import build, lib, init, synchronize, trim, memory_info, EXPORTS, LIB_PATH, CattleHipError  # noqa: F401

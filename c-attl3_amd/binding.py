@@ -26,7 +26,7 @@ ACT = {
 
 # every symbol include/cattle_hip.h declares
 EXPORTS = [
-    "cattle_hip_init", "cattle_hip_last_error", "cattle_hip_synchronize", "cattle_hip_alloc", "cattle_hip_free", "cattle_hip_trim",
+    "cattle_hip_init", "cattle_hip_last_error", "cattle_hip_synchronize", "cattle_hip_alloc", "cattle_hip_free", "cattle_hip_trim", "cattle_hip_memory_info",
     "cattle_hip_upload", "cattle_hip_download", "cattle_hip_fill_zero", "cattle_hip_timer_create",
     "cattle_hip_timer_destroy", "cattle_hip_timer_start", "cattle_hip_timer_stop", "cattle_hip_conv_create",
     "cattle_hip_transconv_create", "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
@@ -81,6 +81,13 @@ def _check(rc):
 
 def init(device=0):
     _check(lib().cattle_hip_init(ctypes.c_int(device)))
+
+
+def memory_info():
+    """(free, total) device memory in bytes; buffers idling in the library's pool count as used."""
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    _check(lib().cattle_hip_memory_info(ctypes.byref(free), ctypes.byref(total)))
+    return int(free.value), int(total.value)
 
 
 def trim():

@@ -1081,6 +1081,14 @@ int cattle_hip_trim(void) {
 	});
 }
 
+int cattle_hip_memory_info(size_t* free_bytes, size_t* total_bytes) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(free_bytes != nullptr && total_bytes != nullptr, "null output pointer");
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+		CATTLE_HIP_CHECK(hipMemGetInfo(free_bytes, total_bytes));
+	});
+}
+
 int cattle_hip_upload(void* dst_device, const void* src_host, size_t bytes) {
 	return guarded([&] {
 		CATTLE_HIP_REQUIRE(bytes == 0 || (dst_device && src_host), "null buffer");

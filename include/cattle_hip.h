@@ -74,6 +74,9 @@ int cattle_hip_alloc(void** device_ptr, size_t bytes);
  * layer of a step); cattle_hip_trim returns the idle ones to the driver. */
 int cattle_hip_free(void* device_ptr);
 int cattle_hip_trim(void);
+/* Free and total memory of the device as the driver reports them (pooled idle buffers count as used). No counterpart
+ * in the reference. */
+int cattle_hip_memory_info(size_t* free_bytes, size_t* total_bytes);
 int cattle_hip_upload(void* dst_device, const void* src_host, size_t bytes);
 int cattle_hip_download(void* dst_host, const void* src_device, size_t bytes);
 int cattle_hip_fill_zero(void* dst_device, size_t bytes);

@@ -665,3 +665,36 @@ def test_optimizer_argument_checks():
     h = (ctypes.c_double * 4)(1e-3, 0, 0, 0)
     assert ch.lib().cattle_hip_layer_param_optimizer_update(layer._h, ctypes.c_size_t(0), ctypes.c_int(17), h, ctypes.c_size_t(0),
                                                             ctypes.c_size_t(0)) != 0
+
+
+def test_device_memory_does_not_grow_over_steps_and_network_lifetimes():
+    """Activation buffers, staging areas and optimizer state come from the library's pooling allocator: after a first
+    network has trained, further networks of the same shape and any number of steps take no more device memory, and
+    cattle_hip_trim hands the pooled buffers back."""
+    import harness as hn
+    dt, N = np.float32, 64
+    gen = hp.rng(0xC0FFEE33)
+    xd = ch.DeviceTensor.from_host(hp.normal(gen, (N, 32, 32, 3), dt))
+    yd = ch.DeviceTensor.from_host(_one_hot_labels(gen, N, (10, 1, 1), dt))
+
+    def used_mib():
+        free, total = ch.memory_info()
+        return (total - free) / 2.0 ** 20
+
+    def lifetime(steps):
+        net = hn.build_convnet(hn.HipBackend(dt))
+        hn.init_kernel_weights(net, 60, dt)
+        plist = ch.ParameterList(net.params())
+        for t in range(steps):
+            out = net.propagate(xd, True)
+            net.backpropagate(ch.loss_d_function("softmax_cross_entropy", out, yd, scale=1.0 / N))
+            plist.optimizer_step("adam", [1e-3, 1e-1, 1e-3, 1e-5], 0, t)
+
+    lifetime(5)
+    base = used_mib()
+    for _ in range(3):
+        lifetime(40)
+        assert used_mib() - base <= 2.0            # MiB; the driver allocates in 2 MiB granules
+    ch.trim()
+    assert used_mib() <= base
+
