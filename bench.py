@@ -27,18 +27,36 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}      # MI355X dense matrix peaks (no sparsity)
 SHAPE = dict(H=56, W=56, C=64, F=128, RH=3, RW=3)
 
-# HBM bytes per launch (read + written) of the three GEMM kernels on the default workload (f32, batch 256):
-# rocprofv3 FETCH_SIZE and WRITE_SIZE readings of `bench.py --copy-calibration`, each scaled by what the same
-# counter reads for the calibration copy of known size (FETCH_SIZE x2.0, WRITE_SIZE x1.0). Counters cannot be
-# read while timing, so these are constants of the measured build; other shapes report null.
-MEASURED_TRAFFIC = {
-    ("f32", 256): {
-        # kernel read + written, then the reduce launches' read + written
-        "gather_gemm_kernel (forward)": 325.8e6 + 469.8e6 + 67.2e6 + 8.4e6,
-        "wgrad_kernel (+ reduce, bias column sums)": 775.5e6 + 52.4e6 + 50.5e6 + 0.3e6,
-        "gather_gemm_kernel (input gradient)": 573.7e6 + 264.2e6 + 63.0e6 + 4.2e6,
-    },
-}
+# HBM bytes per launch (read + written) of the three GEMM kernels come from rocprofv3 FETCH_SIZE and WRITE_SIZE readings
+# of `bench.py --copy-calibration`, each scaled by what the same counter reads for the calibration copy of known size.
+# Counters cannot be read while timing, so the figures live in a tracked file that `python -m c-attl3_amd.rocprof_summary`
+# rewrites from the counter runs, together with a hash of the kernel sources they were measured on; a build from other
+# sources reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "conv_cfg4_hbm_traffic.json")
+KERNEL_SOURCES = ("c-attl3_amd/csrc/gemm_kernels.hip", "c-attl3_amd/csrc/common.hpp")
+
+
+def kernel_sources_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(dtype_name, batch, kernel):
+    """(bytes or None, note) for one GEMM pass of the default workload from the tracked counter summary."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, "no tracked counter summary"
+    if rec.get("kernel_sources_sha256_16") != kernel_sources_hash():
+        return None, "the kernel sources changed since the counters were read (%s): re-run the counter passes" % rec.get("kernel_sources_sha256_16")
+    entry = rec.get("entries", {}).get("%s:%d" % (dtype_name, batch), {})
+    return entry.get(kernel), "rocprofv3 FETCH_SIZE x %.3f + WRITE_SIZE x %.3f, kernel and its reduce launch" % (
+        rec.get("fetch_factor", 0.0), rec.get("write_factor", 0.0))
 
 
 def he_normal(gen, rows, cols, dtype):
@@ -66,12 +84,16 @@ def gpu_run(args, dtype):
 
     for _ in range(args.warmup):
         step()
-    ch.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    ch.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    # the timed region, `repeats` times over: each is exactly `steps` steps between two synchronisations
+    walls = []
+    for _ in range(max(1, args.repeats)):
+        ch.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        ch.synchronize()
+        walls.append((time.perf_counter() - t0) * 1e3 / args.steps)
+    wall_ms = float(np.median(walls))
 
     # per-kernel durations with HIP events on the library's stream
     timer = ch.Timer()
@@ -110,7 +132,33 @@ def gpu_run(args, dtype):
         for _ in range(3):
             ident.forward_into(x, dx, True)
         ch.synchronize()
-    return dict(wall_ms=wall_ms, M=M, K=K, F=F, gemm_flop=gemm_flop, kernels=kernels, bytes=nbytes)
+    for t in (x, go, out, dx):
+        t.free()
+    return dict(wall_ms=wall_ms, walls=walls, M=M, K=K, F=F, gemm_flop=gemm_flop, kernels=kernels, bytes=nbytes)
+
+
+def host_tensor_run(args, dtype):
+    """The same step through the host-tensor Layer API (pageable numpy arrays in, numpy arrays out: what the drop-in
+    adapters do with Eigen tensors): PCIe-inclusive, never the headline value."""
+    ch = importlib.import_module("c-attl3_amd")
+    ch.init(0)
+    N, H, W, C, F = args.batch, SHAPE["H"], SHAPE["W"], SHAPE["C"], SHAPE["F"]
+    gen = np.random.default_rng(0xC0FFEE04)
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F)
+    layer.get_params()[0].set_values(he_normal(gen, 9 * C, F, dtype))
+    x = np.asfortranarray(gen.standard_normal((N, H, W, C)).astype(dtype))
+    go = np.asfortranarray(gen.standard_normal((N, H, W, F)).astype(dtype))
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        layer.pass_forward(x, True)
+        layer.pass_back(go)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    moved = 2.0 * (x.nbytes + go.nbytes)       # x in, out back, out_grad in, in_grad back
+    return {"ms_per_step": round(best * 1e3, 2), "GB/s": round(moved / best / 1e9, 1),
+            "tflops": round(6.0 * N * H * W * 9 * C * F / best / 1e12, 2), "bytes_moved": moved,
+            "note": "pass_forward + pass_back on pageable host arrays, outputs allocated per call, best of 3"}
 
 
 def small_convs_run(args, dtype):
@@ -366,6 +414,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel of x's size (for scaling rocprof byte counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--repeats", type=int, default=5, help="how often the timed loop of --steps steps is repeated (median reported)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the fp64 leg and the host-tensor leg of the default run")
     ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm", "train_steps", "small_convs"], default="conv",
                     help="conv: the headline benchmark; pointwise: HBM-bound layers, one line of per-kernel GB/s; "
                          "convlstm: the fused-gate ConvLSTM of BASELINE configs[4], sequences/s; "
@@ -410,11 +460,25 @@ def main():
         "frac_of_mfma_peak": round(gflops / 1e3 / peak, 4),
         "roofline": {"bound": "mfma", "kernel": name, "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4),
-                     "traffic": MEASURED_TRAFFIC.get((args.dtype, args.batch), {}).get(name),
+                     "traffic": None,
                      "algorithmic_bytes": r["bytes"][name],
                      "flop_per_launch": r["gemm_flop"], "ms_per_launch": round(t_ms, 4)},
         "kernel_ms": {k: round(v, 4) for k, v in r["kernels"].items()},
     }
+    line["roofline"]["traffic"], line["roofline"]["traffic_source"] = measured_traffic(args.dtype, args.batch, name)
+    line["repeats"] = {"n": len(r["walls"]), "ms_per_step_min": round(min(r["walls"]), 4),
+                       "ms_per_step_median": round(float(np.median(r["walls"])), 4), "ms_per_step_max": round(max(r["walls"]), 4)}
+    if not args.no_extra and args.dtype == "f32":
+        # BASELINE configs[3] asks for both MFMA paths: the same layer and step count in fp64
+        d = gpu_run(args, np.float64)
+        d_tflops = 3.0 * d["gemm_flop"] / (d["wall_ms"] * 1e-3) / 1e12
+        line["f64"] = {"ms_per_step": round(d["wall_ms"], 4), "tflops": round(d_tflops, 2),
+                       "frac_of_mfma_peak": round(d_tflops / PEAK_TFLOPS["f64"], 4), "peak": PEAK_TFLOPS["f64"],
+                       "samples_per_s": round(args.batch / (d["wall_ms"] * 1e-3), 1),
+                       "ms_per_step_min": round(min(d["walls"]), 4), "ms_per_step_max": round(max(d["walls"]), 4),
+                       "kernel_ms": {k: round(v, 4) for k, v in d["kernels"].items()}}
+    if not args.no_extra:
+        line["host_tensor_api"] = host_tensor_run(args, dtype)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args, dtype)
     print(json.dumps(line))

@@ -125,6 +125,8 @@ template<typename T> void maxpool_backward(const PoolShape& s, int N, const T* o
 template<typename T> void meanpool_forward(const PoolShape& s, int N, const T* x, T* out);
 template<typename T> void meanpool_backward(const PoolShape& s, int N, const T* out_grad, T* in_grad);
 
+/* Zeroes `bytes` bytes (a multiple of 4, at a 4-byte aligned address) with a kernel on the library's stream. */
+void device_zero_fill(void* dst, size_t bytes);
 /* dst[i] += src[i] */
 template<typename T> void axpy_one(size_t n, const T* src, T* dst);
 /* dst[c + cols*r] (+)= src[r + rows*c] for a column-major rows x cols matrix src */

@@ -87,7 +87,13 @@ void copy_out(void* dst, int space, const void* src_dev, size_t bytes) {
 }
 
 void fill_zero(void* dst_dev, size_t bytes) {
-	if (bytes)
+	if (bytes == 0)
+		return;
+	/* every buffer of the library is made of 4- or 8-byte scalars and is zeroed by a kernel, which a caller may record
+	 * into a graph; only an odd-sized caller buffer goes to the runtime's memset */
+	if ((reinterpret_cast<uintptr_t>(dst_dev) & 3) == 0 && bytes % 4 == 0)
+		device_zero_fill(dst_dev, bytes);
+	else
 		CATTLE_HIP_CHECK(hipMemsetAsync(dst_dev, 0, bytes, stream()));
 }
 
@@ -99,6 +105,7 @@ void fill_zero(void* dst_dev, size_t bytes) {
 struct DevicePool {
 	std::map<size_t, std::vector<void*>> idle;      /* size class -> blocks */
 	std::map<void*, size_t> live;                    /* block -> size class */
+	std::map<const char*, size_t> idle_index;        /* idle block -> size class, for released() */
 	size_t idle_bytes = 0;
 	static size_t size_class(size_t bytes) {
 		/* powers of two up to 1 MiB, then multiples of 1 MiB: at most 2x / ~0 % over-allocation */
@@ -114,6 +121,7 @@ struct DevicePool {
 		if (!bucket.empty()) {
 			p = bucket.back();
 			bucket.pop_back();
+			idle_index.erase(static_cast<const char*>(p));
 			idle_bytes -= c;
 		} else {
 			hipError_t e = hipMalloc(&p, c);
@@ -132,8 +140,19 @@ struct DevicePool {
 		std::map<void*, size_t>::iterator it = live.find(p);
 		CATTLE_HIP_REQUIRE(it != live.end(), "cattle_hip_free of a pointer that cattle_hip_alloc did not return");
 		idle[it->second].push_back(p);
+		idle_index[static_cast<const char*>(p)] = it->second;
 		idle_bytes += it->second;
 		live.erase(it);
+	}
+	/* whether p points into a block that was handed out and has been given back since */
+	bool released(const void* p) const {
+		if (!p || idle_index.empty())
+			return false;
+		std::map<const char*, size_t>::const_iterator it = idle_index.upper_bound(static_cast<const char*>(p));
+		if (it == idle_index.begin())
+			return false;
+		--it;
+		return static_cast<const char*>(p) < it->first + it->second;
 	}
 	void trim() {
 		for (std::map<size_t, std::vector<void*>>::iterator it = idle.begin(); it != idle.end(); ++it) {
@@ -141,6 +160,7 @@ struct DevicePool {
 				(void) hipFree(p);
 			it->second.clear();
 		}
+		idle_index.clear();
 		idle_bytes = 0;
 	}
 };
@@ -225,6 +245,13 @@ struct LayerBase {
 	virtual void empty_cache() {
 		have_forward = false;
 	}
+	/* A device tensor that the layer borrowed in its forward pass must still be the caller's in the backward pass: one
+	 * that went back to the pool through cattle_hip_free may hold another tensor by now. */
+	virtual void check_borrowed() const { }
+	static void require_not_released(const void* p) {
+		if (g_pool.released(p))
+			throw Error(ERR_STATE, "a device tensor that the layer borrowed in its forward pass was freed before the backward pass");
+	}
 };
 
 int checked_int(size_t v, const char* what) {
@@ -283,6 +310,9 @@ struct ConvLayer : LayerBase {
 	void empty_cache() override {
 		LayerBase::empty_cache();
 		x_cache = nullptr;
+	}
+	void check_borrowed() const override {
+		require_not_released(x_cache);
 	}
 };
 
@@ -354,6 +384,9 @@ struct TransConvLayer : LayerBase {
 	void empty_cache() override {
 		LayerBase::empty_cache();
 		x_cache = nullptr;
+	}
+	void check_borrowed() const override {
+		require_not_released(x_cache);
 	}
 };
 
@@ -514,6 +547,9 @@ struct ConvLstm : LayerBase {
 		LayerBase::empty_cache();
 		x_cache = nullptr;
 	}
+	void check_borrowed() const override {
+		require_not_released(x_cache);
+	}
 };
 
 template<typename T>
@@ -523,6 +559,7 @@ struct BatchNormLayer : LayerBase {
 	bool stats_init = false;
 	DevBuf std_cache, inv_sd_cache, ws;
 	bool cache_valid = false;
+	size_t cache_batch = 0;         /* batch size of the training pass that filled std_cache and inv_sd_cache */
 
 	BatchNormLayer(int dtype, size_t H, size_t W, size_t C, bool per_last_rank, T decay, T eps) :
 			LayerBase(dtype), per_last_rank(per_last_rank), decay(decay), eps(eps) {
@@ -562,12 +599,17 @@ struct BatchNormLayer : LayerBase {
 		if (training) {
 			stats_init = true;
 			cache_valid = true;
+			cache_batch = N;
 			++params[0]->version;
 			++params[1]->version;
 		}
 	}
 	void backward(const void* out_grad, size_t N, void* in_grad) override {
 		CATTLE_HIP_REQUIRE(cache_valid, "pass_back without a training-mode forward pass");
+		/* an inference pass in between leaves the caches of the last training pass in place; they only fit a gradient
+		 * of that pass's batch size (assert(std_in_mat_cache.rows() == out_grad rows), BatchNormLayer.hpp:194) */
+		if (N != cache_batch)
+			throw Error(ERR_STATE, "pass_back with a batch size other than that of the last training-mode forward pass");
 		const int g = checked_int(groups(), "statistics groups");
 		const size_t L = N * in_volume() / groups();
 		T* w = (T*) ws.ensure(bn_workspace(g, L) * sizeof(T));
@@ -648,6 +690,10 @@ struct ActivationLayer : LayerBase {
 	void empty_cache() override {
 		LayerBase::empty_cache();
 		x_cache = y_cache = nullptr;
+	}
+	void check_borrowed() const override {
+		require_not_released(x_cache);
+		require_not_released(y_cache);
 	}
 };
 
@@ -1000,6 +1046,7 @@ template<typename T>
 void convlstm_backpropagate(ConvLstm<T>* l, const void* out_grad, int og_space, void* in_grad, int ig_space) {
 	if (!l->have_forward)
 		throw Error(ERR_STATE, "backpropagate without a matching propagate");
+	l->check_borrowed();
 	const size_t og_bytes = l->batch * l->T_out * l->out_volume() * sizeof(T), ig_bytes = l->batch * l->T_in * l->in_volume() * sizeof(T);
 	const void* og_dev = out_grad;
 	if (og_space == CATTLE_HIP_HOST) {
@@ -1581,6 +1628,7 @@ int cattle_hip_layer_backward(cattle_hip_layer_t layer, const void* out_grad, ca
 			throw Error(ERR_STATE, "pass_back without a preceding pass_forward");
 		CATTLE_HIP_REQUIRE(batch > 0 && batch == l->batch, "batch size differs from the forward pass");   /* e.g. ConvKernelLayer.hpp:314 */
 		CATTLE_HIP_REQUIRE(in_grad != nullptr || l->input_layer, "in_grad may be NULL only for an input layer");
+		l->check_borrowed();
 		const size_t in_bytes = batch * l->in_volume() * l->esize(), out_bytes = batch * l->out_volume() * l->esize();
 		const void* og_dev = out_grad;
 		if (grad_space == CATTLE_HIP_HOST) {

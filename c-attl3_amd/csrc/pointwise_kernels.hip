@@ -741,6 +741,23 @@ unsigned pool_grid(const PoolLaunch& pl, int cols, int channels) {
 	return (unsigned) blocks;
 }
 
+/* Zero fill of `bytes` bytes at a 4-byte aligned address: 16-byte stores over the aligned middle, 4-byte stores over
+ * the ends. A kernel rather than a memset of the runtime, so that the call may be recorded into a graph. */
+__global__ __launch_bounds__(256)
+void zero_fill_kernel(unsigned* __restrict__ p, size_t words) {
+	const size_t head = std::min<size_t>(words, (size_t) ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4);
+	const size_t quads = (words - head) / 4;
+	uint4* q = reinterpret_cast<uint4*>(p + head);
+	const size_t stride = (size_t) gridDim.x * blockDim.x, t = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+	for (size_t i = t; i < quads; i += stride)
+		q[i] = make_uint4(0u, 0u, 0u, 0u);
+	if (t < head)
+		p[t] = 0u;
+	const size_t done = head + quads * 4;
+	if (t < words - done)
+		p[done + t] = 0u;
+}
+
 template<typename T>
 __global__ void axpy_one_kernel(size_t n, const T* __restrict__ src, T* __restrict__ dst) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
@@ -1146,6 +1163,16 @@ void meanpool_forward(const PoolShape& s, int N, const T* x, T* out) {
 template<typename T>
 void meanpool_backward(const PoolShape& s, int N, const T* out_grad, T* in_grad) {
 	pool_backward_launch<T, false>(s, N, out_grad, nullptr, in_grad);
+}
+
+void device_zero_fill(void* dst, size_t bytes) {
+	if (bytes == 0)
+		return;
+	CATTLE_HIP_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 3) == 0 && bytes % 4 == 0, "zero fill of a buffer that is not made of 4-byte words");
+	const size_t words = bytes / 4;
+	const size_t blocks = std::min<size_t>(std::max<size_t>(1, (words / 4 + 255) / 256), 2048);
+	zero_fill_kernel<<<(unsigned) blocks, 256, 0, stream()>>>(static_cast<unsigned*>(dst), words);
+	check_launch();
 }
 
 template<typename T>

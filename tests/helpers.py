@@ -42,11 +42,18 @@ def normal(gen, shape, dtype, std=1.0):
     return np.asfortranarray((gen.standard_normal(size=shape) * std).astype(dtype))
 
 
-def rel_err(a, b, floor_frac=0.1):
+# label -> (floored error, un-floored error over |ref| > floor, element count): what the labelled comparisons of a
+# test run achieved; tests/conftest.py prints the table at the end of the run
+ACHIEVED = {}
+
+
+def rel_err(a, b, floor_frac=0.1, label=None):
     """max_i |a_i - b_i| / max(|b_i|, floor), floor = floor_frac * RMS(b) (tiny if b is all zero).
 
     The absolute floor keeps the relative error meaningful for elements that are (near) zero by
-    cancellation: they are compared relative to a tenth of the tensor's RMS instead."""
+    cancellation: they are compared relative to a tenth of the tensor's RMS instead. With a label the
+    achieved error is recorded, beside the plain relative error max |a_i - b_i| / |b_i| over the
+    elements with |b_i| > floor (no floor in the denominator)."""
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
     assert a.shape == b.shape, (a.shape, b.shape)
@@ -54,7 +61,14 @@ def rel_err(a, b, floor_frac=0.1):
         return 0.0
     rms = float(np.sqrt(np.mean(b * b)))
     floor = max(floor_frac * rms, 1e-30)
-    return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), floor)))
+    diff = np.abs(a - b)
+    err = float(np.max(diff / np.maximum(np.abs(b), floor)))
+    if label is not None:
+        big = np.abs(b) > floor
+        plain = float(np.max(diff[big] / np.abs(b[big]))) if np.any(big) else 0.0
+        old = ACHIEVED.get(label, (0.0, 0.0, 0))
+        ACHIEVED[label] = (max(old[0], err), max(old[1], plain), old[2] + a.size)
+    return err
 
 
 def conv_dims(H, W, RH, RW, pv, ph, sv, sh, dv, dh):

@@ -89,7 +89,7 @@ def test_batchnorm_activations_pools(records, tag):
     am, ais = np.zeros(3), np.zeros(3)
     y1, std, isd = oracle.bn_forward(f("bn.x1"), gamma, beta, am, ais, False, True, decay=float(np.float32(0.2)) if tag == "f32" else 0.2)
     dx, dg, dbeta = oracle.bn_backward(f("bn.go"), gamma, std, isd)
-    assert hp.rel_err(r["bn.y1"], y1) < tol and hp.rel_err(r["bn.dx1"], dx) < 10 * tol
+    assert hp.rel_err(r["bn.y1"], y1) < tol and hp.rel_err(r["bn.dx1"], dx, label="adapter batchnorm dx " + tag) < tol
     assert hp.rel_err(f("bn.dgamma").reshape(-1), dg) < tol and hp.rel_err(f("bn.dbeta").reshape(-1), dbeta) < tol
     oracle.bn_forward(f("bn.x2"), gamma, beta, am, ais, True, True, decay=float(np.float32(0.2)) if tag == "f32" else 0.2)
     assert hp.rel_err(f("bn.avg_mean").reshape(-1), am) < tol and hp.rel_err(f("bn.avg_inv_sd").reshape(-1), ais) < tol
