@@ -42,7 +42,7 @@ EXPORTS = [
     "cattle_hip_layer_param_optimizer_update", "cattle_hip_layer_param_optimizer_step", "cattle_hip_optimizer_step_many", "cattle_hip_layer_param_sgd_update", "cattle_hip_layer_param_adam_update",
     "cattle_hip_layer_param_reset_optimizer_state", "cattle_hip_convlstm_create", "cattle_hip_convlstm_propagate",
     "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
-    "cattle_hip_convlstm_get_kernel_grad",
+    "cattle_hip_convlstm_get_kernel_grad", "cattle_hip_conv_forward_noalloc", "cattle_hip_static_scratch_bytes",
 ]
 
 
@@ -145,6 +145,25 @@ class DeviceTensor(object):
             self.free()
         except Exception:
             pass
+
+
+def static_scratch_bytes():
+    """Size of the fixed device array that conv_forward_noalloc takes its scratch memory from."""
+    v = ctypes.c_size_t()
+    _check(lib().cattle_hip_static_scratch_bytes(ctypes.byref(v)))
+    return int(v.value)
+
+
+def conv_forward_noalloc(x, weights, bias, out, receptor_height=3, receptor_width=3, vertical_padding=1, horizontal_padding=1,
+                         vertical_stride=1, horizontal_stride=1, vertical_dilation=0, horizontal_dilation=0):
+    """ConvKernelLayer::pass_forward on DeviceTensors the caller owns, through the entry point that allocates nothing:
+    x (N, H, W, C), weights (RH*RW*C, F), bias (1, F) or None, out (N, OH, OW, F)."""
+    N, H, W, C = x.shape
+    F = weights.shape[1]
+    _check(lib().cattle_hip_conv_forward_noalloc(
+        _dtype_code(x.dtype), _sz(N), _sz(H), _sz(W), _sz(C), _sz(F), _sz(receptor_height), _sz(receptor_width),
+        _sz(vertical_padding), _sz(horizontal_padding), _sz(vertical_stride), _sz(horizontal_stride), _sz(vertical_dilation),
+        _sz(horizontal_dilation), x.ptr, weights.ptr, None if bias is None else bias.ptr, out.ptr))
 
 
 class Timer(object):

@@ -86,6 +86,14 @@ int prepared_weight_row_length(int columns);
 template<typename T> void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out,
 		T* wt, bool wt_ready);
 
+/* The same forward pass for callers that cannot allocate device memory: the prepared weights and the partial sums of a
+ * split reduction live in a fixed device array of static_scratch_bytes() bytes per device, whose address
+ * static_scratch_setup() looks up for the current device (once; called when the library is initialised). Throws
+ * ERR_INVALID when the problem needs more scratch than that. Every call on a device uses the same array. */
+void static_scratch_setup();
+size_t static_scratch_bytes();
+template<typename T> void conv_forward_static(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out);
+
 /* Backward: wgrad[K x F] += A^T G, bgrad[F] += colsum(G), in_grad = dgrad (skipped if null). */
 template<typename T> void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad,
 		T* wgrad, T* bgrad, T* in_grad, T* wt_dgrad, bool wt_ready, T* partials);

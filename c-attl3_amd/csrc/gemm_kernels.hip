@@ -843,6 +843,29 @@ void* split_workspace(size_t bytes) {
 	return ptr;
 }
 
+/* Where a launch that must not allocate takes its scratch memory from: a caller-provided range of device memory that
+ * is handed out front to back. A null arena means the library's own grow-only buffers. */
+struct ScratchArena {
+	char* base;
+	size_t cap, used;
+	void* take(size_t bytes, const char* what) {
+		const size_t at = (used + 255) / 256 * 256;
+		if (at + bytes > cap)
+			throw Error(ERR_INVALID, std::string("the ") + what + " of this problem (" + std::to_string(bytes) +
+					" bytes) do not fit the static scratch buffer of " + std::to_string(cap) + " bytes");
+		used = at + bytes;
+		return base + at;
+	}
+};
+
+/* The scratch memory of the entry point that allocates nothing: a fixed array in the code object, so it exists once
+ * per device for the life of the process and no call ever allocates or frees it. Its name is only a stand-in on the
+ * host; the device address comes from hipGetSymbolAddress, once per device, and is what kernels and copies are given. */
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t) 72 << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+void* g_scratch_ptr[MAX_DEVICES] = { nullptr };
+
 /* out tile = bias + sum over the parts of a split reduction, parts taken in ascending order (so the result
  * does not depend on how blocks were scheduled). One block per (walk position, f block) tile. */
 template<typename T>
@@ -1046,7 +1069,7 @@ const Tuning& tuning() {
  * occupancy their LDS and register use allows; measured on MI355X, more co-resident blocks beat
  * fewer blocks even when the last round of blocks is mostly idle. */
 template<typename T>
-void launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g) {
+void launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, ScratchArena* arena = nullptr) {
 	const bool vec = g.N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
 	const bool divs = g.DA != 1 || g.DB != 1;
 	const GatherVariant<T>* vars = GatherVariants<T>::get();
@@ -1119,7 +1142,8 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if (L.split_count > 0) {
 			L.chunks_per_part = (nchunks + ksplit - 1) / ksplit;
 			L.ksplit = (nchunks + L.chunks_per_part - 1) / L.chunks_per_part;       /* no empty part */
-			partials = static_cast<T*>(split_workspace((size_t) L.split_count * ftiles * L.ksplit * v.bm * v.bf * sizeof(T)));
+			const size_t pbytes = (size_t) L.split_count * ftiles * L.ksplit * v.bm * v.bf * sizeof(T);
+			partials = static_cast<T*>(arena ? arena->take(pbytes, "partial sums of the split reduction") : split_workspace(pbytes));
 		}
 		dim3 grid((unsigned) (L.main_blocks + L.split_count * L.ksplit), (unsigned) ftiles);
 		v.launch(grid, dyn, src, wt, bias, out, g, L, partials, vec, divs);
@@ -1336,6 +1360,37 @@ void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b,
 	launch_gather<T>(x, wt, b, out, g);
 }
 
+void static_scratch_setup() {
+	int dev = -1;
+	CATTLE_HIP_CHECK(hipGetDevice(&dev));
+	CATTLE_HIP_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "device index beyond what the static scratch table holds");
+	if (g_scratch_ptr[dev])
+		return;
+	void* ptr = nullptr;
+	CATTLE_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+	g_scratch_ptr[dev] = ptr;
+}
+
+size_t static_scratch_bytes() {
+	return STATIC_SCRATCH_BYTES;
+}
+
+template<typename T>
+void conv_forward_static(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out) {
+	check_sizes(s, N);
+	int dev = -1;
+	CATTLE_HIP_CHECK(hipGetDevice(&dev));
+	CATTLE_HIP_REQUIRE(dev >= 0 && dev < MAX_DEVICES && g_scratch_ptr[dev] != nullptr, "the static scratch buffer of this device is not set up");
+	ScratchArena arena = { static_cast<char*>(g_scratch_ptr[dev]), STATIC_SCRATCH_BYTES, 0 };
+	const GatherGeom g = forward_geom(s, N);
+	const int Kp = round_up(g.K, WT_ROW_PAD);
+	const size_t count = (size_t) Kp * g.ldw;
+	T* wt = static_cast<T*>(arena.take(count * sizeof(T), "prepared weights"));
+	prep_fwd_weights_kernel<T><<<(unsigned) ((count + 255) / 256), 256, 0, stream()>>>(w, wt, g.K, g.F, Kp, g.ldw);
+	CATTLE_HIP_CHECK(hipGetLastError());
+	launch_gather<T>(x, wt, b, out, g, &arena);
+}
+
 template<typename T>
 void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials) {
 	check_sizes(s, N);
@@ -1393,6 +1448,8 @@ template ConvWorkspace conv_workspace<float>(const ConvShape&, int);
 template ConvWorkspace conv_workspace<double>(const ConvShape&, int);
 template void conv_forward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, bool);
 template void conv_forward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*, bool);
+template void conv_forward_static<float>(const ConvShape&, int, const float*, const float*, const float*, float*);
+template void conv_forward_static<double>(const ConvShape&, int, const double*, const double*, const double*, double*);
 template void conv_backward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, float*,
 		float*, bool, float*);
 template void conv_backward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*,

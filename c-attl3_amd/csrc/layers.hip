@@ -38,6 +38,7 @@ void ensure_init(int device) {
 	if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
 		throw Error(ERR_DEVICE, std::string("cattle_hip is built for gfx950 only, found ") + prop.gcnArchName);
 	CATTLE_HIP_CHECK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+	static_scratch_setup();
 	g_ready = true;
 }
 
@@ -1223,6 +1224,48 @@ int cattle_hip_conv_create(cattle_hip_dtype dtype, size_t height, size_t width, 
 		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new ConvLayer<float>(dtype, s, false) :
 				(LayerBase*) new ConvLayer<double>(dtype, s, false);
 		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_conv_forward_noalloc(cattle_hip_dtype dtype, size_t batch, size_t height, size_t width, size_t channels,
+		size_t filters, size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
+		const void* in_device, const void* weights_device, const void* bias_device, void* out_device) {
+	/* no allocation on this path: no layer object, no staging, no grow-only buffer; only kernel launches */
+	return guarded([&] {
+		check_dtype(dtype);
+		CATTLE_HIP_REQUIRE(in_device != nullptr && weights_device != nullptr && out_device != nullptr, "null tensor buffer");
+		CATTLE_HIP_REQUIRE(batch > 0 && batch <= 2147483647u, "batch size must be positive and below 2^31");
+		CATTLE_HIP_REQUIRE(height > 0 && width > 0 && channels > 0 && filters > 0, "dimensions must be positive");
+		CATTLE_HIP_REQUIRE(receptor_height > 0 && receptor_width > 0, "receptor dimensions must be positive");
+		CATTLE_HIP_REQUIRE(vertical_stride > 0 && horizontal_stride > 0, "strides must be positive");
+		const size_t lim = 1u << 20;
+		CATTLE_HIP_REQUIRE(height < lim && width < lim && channels < lim && filters < lim && receptor_height < lim &&
+				receptor_width < lim && vertical_padding < lim && horizontal_padding < lim && vertical_stride < lim &&
+				horizontal_stride < lim && vertical_dilation < lim && horizontal_dilation < lim, "dimension too large");
+		const size_t drh = receptor_height + (receptor_height - 1) * vertical_dilation;
+		const size_t drw = receptor_width + (receptor_width - 1) * horizontal_dilation;
+		CATTLE_HIP_REQUIRE(height + 2 * vertical_padding >= drh && width + 2 * horizontal_padding >= drw,
+				"dilated receptor larger than the padded input");
+		CATTLE_HIP_REQUIRE(receptor_height * receptor_width * channels <= 2147483647u / 2, "receptor volume too large");
+		const ConvShape s = { (int) height, (int) width, (int) channels, (int) filters, (int) receptor_height, (int) receptor_width,
+				(int) vertical_padding, (int) horizontal_padding, (int) vertical_stride, (int) horizontal_stride,
+				(int) vertical_dilation, (int) horizontal_dilation };
+		CATTLE_HIP_REQUIRE((double) batch * s.H * s.W * s.C <= 2147483647.0 && (double) batch * s.OH() * s.OW() * s.F <= 2147483647.0,
+				"tensor exceeds 2^31-1 elements");
+		if (dtype == CATTLE_HIP_F32)
+			conv_forward_static<float>(s, (int) batch, static_cast<const float*>(in_device), static_cast<const float*>(weights_device),
+					static_cast<const float*>(bias_device), static_cast<float*>(out_device));
+		else
+			conv_forward_static<double>(s, (int) batch, static_cast<const double*>(in_device),
+					static_cast<const double*>(weights_device), static_cast<const double*>(bias_device), static_cast<double*>(out_device));
+	});
+}
+
+int cattle_hip_static_scratch_bytes(size_t* bytes) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(bytes != nullptr, "null output pointer");
+		*bytes = static_scratch_bytes();
 	});
 }
 

@@ -100,6 +100,24 @@ int cattle_hip_conv_create(cattle_hip_dtype dtype, size_t height, size_t width, 
 		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
 		cattle_hip_layer_t* layer);
 
+/* ConvKernelLayer::pass_forward without any allocation. No counterpart in the reference: it is for callers that cannot
+ * allocate device memory while they call (code under HIP graph capture, tight serving loops, harnesses that forbid it).
+ * It computes what cattle_hip_layer_forward computes for a layer made by cattle_hip_conv_create with the same geometry,
+ * bit for bit, from buffers that the caller owns, all in device memory: `in_device` (batch, height, width, channels),
+ * `weights_device` [receptor_height*receptor_width*channels x filters] in the layout of parameter 0, `bias_device`
+ * [1 x filters] (NULL: no bias), `out_device` (batch, OH, OW, filters). Nothing is cached for a backward pass.
+ * Its scratch memory (the re-laid-out weights and, for launches that cut reductions into parts, their partial sums) is
+ * a fixed array inside the library, cattle_hip_static_scratch_bytes() bytes (72 MiB) per device, held from the moment the
+ * library is loaded on a device until the process ends; a problem that needs more is refused with CATTLE_HIP_ERR_INVALID
+ * and a message that names both sizes. Call cattle_hip_init() beforehand: the first call into the library creates its
+ * stream. Every call on a device uses the same array, so calls that overlap on one device race: issue them from one
+ * thread or serialise them (the library's own lock does; work that a caller issues outside the lock does not count). */
+int cattle_hip_conv_forward_noalloc(cattle_hip_dtype dtype, size_t batch, size_t height, size_t width, size_t channels,
+		size_t filters, size_t receptor_height, size_t receptor_width, size_t vertical_padding, size_t horizontal_padding,
+		size_t vertical_stride, size_t horizontal_stride, size_t vertical_dilation, size_t horizontal_dilation,
+		const void* in_device, const void* weights_device, const void* bias_device, void* out_device);
+int cattle_hip_static_scratch_bytes(size_t* bytes);
+
 /* TransConvKernelLayer<Scalar,Rank>(input_dims, filters, init, receptor_height, receptor_width,
  * vertical_padding, horizontal_padding, vertical_stride, horizontal_stride, vertical_dilation,
  * horizontal_dilation) — layer/kernel/TransConvKernelLayer.hpp:285-299 (rank 2 :345-360, rank 1
