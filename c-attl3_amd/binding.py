@@ -43,6 +43,7 @@ EXPORTS = [
     "cattle_hip_layer_param_reset_optimizer_state", "cattle_hip_convlstm_create", "cattle_hip_convlstm_propagate",
     "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
     "cattle_hip_convlstm_get_kernel_grad", "cattle_hip_conv_forward_noalloc", "cattle_hip_static_scratch_bytes",
+    "cattle_hip_fused_create", "cattle_hip_fused_last_mode",
 ]
 
 
@@ -740,3 +741,32 @@ class MeanPoolLayer(_PoolLayer):
     def __init__(self, dtype, input_dims, receptor_height=2, receptor_width=2, vertical_stride=2, horizontal_stride=2):
         _PoolLayer.__init__(self, POOL_MEAN, dtype, input_dims, receptor_height, receptor_width, vertical_stride,
                             horizontal_stride)
+
+
+class FusedKernelLayer(Layer):
+    """A kernel layer and the batch norm / activation / pool layers behind it as one layer (cattle_hip_fused_create): the
+    calls FeedforwardNeuralNetwork.hpp:112-141 makes one after another. The members keep their parameters and caches."""
+
+    MODES = {0: "none", 1: "unfused", 2: "act", 3: "pool", 4: "bn"}
+
+    def __init__(self, members):
+        members = list(members)
+        handles = (ctypes.c_void_p * len(members))(*[m._h for m in members])
+        h = ctypes.c_void_p()
+        _check(lib().cattle_hip_fused_create(handles, _sz(len(members)), ctypes.byref(h)))
+        Layer.__init__(self, h, members[0].dtype, members[0].get_input_dims(), members[-1].get_output_dims())
+        self.members = members          # borrowed by the handle: keep them alive
+
+    def last_mode(self):
+        v = ctypes.c_int()
+        _check(lib().cattle_hip_fused_last_mode(self._h, ctypes.byref(v)))
+        return self.MODES[int(v.value)]
+
+    def _clone(self, share):
+        c = Layer._clone(self, share)
+        c.members = []                  # the clone's handle owns clones of the members
+        return c
+
+    def __del__(self):
+        Layer.__del__(self)             # the fused handle goes before its members
+        self.members = None

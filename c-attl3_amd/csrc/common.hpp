@@ -135,6 +135,53 @@ template<typename T> void meanpool_backward(const PoolShape& s, int N, const T* 
 
 /* Zeroes `bytes` bytes (a multiple of 4, at a 4-byte aligned address) with a kernel on the library's stream. */
 void device_zero_fill(void* dst, size_t bytes);
+/* ---- fused kernel layer: convolution or dense -> [batch norm] -> [activation] -> [pool] --------------------------- */
+
+/* What the gather GEMM does with a finished output tile besides adding the bias:
+ *   EPI_NONE   out = acc + bias.
+ *   EPI_ACT    out = activation(acc + bias) in the coded form of act_math.hpp; the pre-activation values go to `pre`
+ *              when the activation's backward pass needs them.
+ *   EPI_POOL   activation, then max pooling with windows that tile the output (stride = receptor): `out` is the pooled
+ *              tensor, `inds` the arg-max cache in the layout of MaxPoolLayer (layer/pool/MaxPoolLayer.hpp:58-62), `pre`
+ *              the pre-activation value at each arg-max (or null). Needs the blocked tile order with whole windows per tile.
+ *   EPI_STATS  out = acc + bias, plus per tile and output column (count, mean, sum of squared deviations) of the tile's
+ *              rows in `stats` [mtiles][F][3]: the batch-norm moments of the convolution output without reading it again. */
+enum { EPI_NONE = 0, EPI_ACT = 1, EPI_POOL = 2, EPI_STATS = 3 };
+template<typename T>
+struct Epilogue {
+	int kind;               /* cattle_hip_activation, element-wise kinds */
+	T p;                    /* the activation's scalar argument */
+	T* pre;
+	unsigned* inds;
+	int prh, prw;           /* pooling receptor (= stride) along height and width */
+	int OHp, OWp;           /* pooled output extents */
+	T* stats;
+};
+/* conv_forward with a fused epilogue. Returns false, having launched nothing, when the problem does not allow the
+ * epilogue (no 16-byte accesses, windows that do not fit the tiles): the caller then runs the layers one by one; the
+ * prepared weights `wt` are valid afterwards either way.
+ * `mtiles` receives the row count of the EPI_STATS partials; conv_stats_rows() bounds it for any launch. */
+template<typename T> bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out, T* wt,
+		bool wt_ready, int epi, const Epilogue<T>& E, int* mtiles);
+size_t conv_stats_rows(const ConvShape& s, int N);
+/* The layers behind the kernel layer, on its output z (N, H, W, C): element-wise activation `kind` (argument p) and a
+ * pool (0 none, 1 max, 2 mean) whose prh x prw windows tile z exactly. */
+struct ChainShape {
+	int H, W, C, prh, prw, pool, kind;
+	double p;
+};
+/* dz from the gradient g of the (pooled) output, the arg-max cache, and the coded output y or the pre-activation
+ * values `pre` (both at the arg-max positions when pooled); max pooling or none */
+template<typename T> void chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* y, const T* pre, T* dz);
+/* With a per-channel batch norm between kernel layer and activation: out = pool(act(bn(z))), the channel moments merged
+ * from the GEMM epilogue's per-tile moments `stats` [mtiles][C][3] (training) or taken from the running statistics. */
+size_t bn_chain_workspace(int channels);
+template<typename T> void bn_chain_forward(const ChainShape& s, int N, int mtiles, bool training, bool stats_init, const T* z,
+		const T* stats, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd, T decay, T eps, T* mean_cache, T* inv_sd_cache,
+		T* out, unsigned* inds);
+template<typename T> void bn_chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* z, const T* gamma,
+		const T* beta, const T* mean_cache, const T* inv_sd_cache, T* gamma_grad, T* beta_grad, T* dz, T* ws);
+
 /* dst[i] += src[i] */
 template<typename T> void axpy_one(size_t n, const T* src, T* dst);
 /* dst[c + cols*r] (+)= src[r + rows*c] for a column-major rows x cols matrix src */

@@ -17,8 +17,10 @@
  * contiguous index of the output so that stores are coalesced.
  */
 #include "common.hpp"
+#include "act_math.hpp"
 
 #include <algorithm>
+#include <limits>
 #include <cstdlib>
 #include <cstring>
 #include <string>
@@ -157,31 +159,32 @@ struct GatherLaunch {
 	int mtiles, tile_rows;
 	int main_count, main_blocks;
 	int split_count, ksplit, chunks_per_part;
-	int sample_blocks;      /* > 0: tile rows are blocks of 32 samples x BM / 32 positions, see tile_row_m */
-	int pos_b;              /* blocked order: positions of a tile along b (the other BM / 32 / pos_b lie along a) */
+	int sample_blocks;      /* > 0: tile rows are blocks of SB samples x BM / SB positions, see tile_row_m */
+	int pos_b;              /* blocked order: positions of a tile along b (the other BM / SB / pos_b lie along a) */
+	int sb_shift;           /* log2 of SB, the samples per block of the blocked order: 5 except under a pooling epilogue */
 };
 
 /* Row `row` of M tile `tile` as an index m = n + N * (a + OA * b) of the GEMM. Plain order: the tile is BM
  * consecutive m (BM consecutive samples of one output position when N >= BM). Blocked order (sample_blocks =
- * N / 32 > 0, needs N % 32 == 0): the tile is 32 samples of a pa x pos_b rectangle of output positions
- * (pa = BM / 32 / pos_b along a, OA % pa == 0, OB % pos_b == 0), so that the receptor fields of its rows
- * overlap and a tile touches about half as many distinct input bytes; tiles of one strip of pos_b columns are
- * numbered sample block fastest, and tile_rows counts the tiles of a strip. Rows stay groups of 32 consecutive
- * samples, so vector accesses along n are unaffected. */
-__device__ __forceinline__ int tile_row_m(const GatherLaunch& L, const GatherGeom& g, int tile, int BM, int row) {
+ * N / SB > 0, needs N % SB == 0; SB = 32 unless a pooling epilogue picked fewer): the tile is SB samples of a pa x pos_b
+ * rectangle of output positions (pa = BM / SB / pos_b along a, OA % pa == 0, OB % pos_b == 0), so that the receptor
+ * fields of its rows overlap and a tile touches about half as many distinct input bytes; tiles of one strip of pos_b
+ * columns are numbered sample block fastest, and tile_rows counts the tiles of a strip. Rows stay groups of SB
+ * consecutive samples, so vector accesses along n are unaffected. */
+__device__ __forceinline__ int tile_row_m(const GatherLaunch& L, const GatherGeom& g, int tile, int BM, int row, int sb_shift = 5) {
 	if (L.sample_blocks == 0)
 		return tile * BM + row;
 	const int strip = tile / L.tile_rows, r = tile - strip * L.tile_rows;
 	const int ab = r / L.sample_blocks, nb = r - ab * L.sample_blocks;
-	const int pa = BM / 32 / L.pos_b, p = row >> 5;
+	const int pa = (BM >> sb_shift) / L.pos_b, p = row >> sb_shift;
 	const int pb_i = p / pa, pa_i = p - pb_i * pa;
-	return nb * 32 + (row & 31) + g.N * (ab * pa + pa_i + g.OA * (strip * L.pos_b + pb_i));
+	return (nb << sb_shift) + (row & ((1 << sb_shift) - 1)) + g.N * (ab * pa + pa_i + g.OA * (strip * L.pos_b + pb_i));
 }
 
-template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS>
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI = EPI_NONE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
 void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom g, const GatherLaunch L, T* __restrict__ partials) {
+		T* __restrict__ out, const GatherGeom g, const GatherLaunch L, T* __restrict__ partials, const Epilogue<T> E) {
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_M * WAVES_F;
 	constexpr int BM = WAVES_M * WT_M, BF = WAVES_F * WT_F;
@@ -252,7 +255,8 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 
 	/* --- per-thread gather state: a fixed group of VEC rows m --- */
 	const int acol = tid % ACOLS, arow0 = tid / ACOLS;
-	const int m = tile_row_m(L, g, tile, BM, acol * VEC);
+	const int sb_shift = EPI == EPI_POOL ? L.sb_shift : 5;
+	const int m = tile_row_m(L, g, tile, BM, acol * VEC, sb_shift);
 	const bool mvalid = m < g.M;
 	int n, ya0, yb0;
 	{
@@ -417,8 +421,180 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			}
 		return;
 	}
+	if constexpr (EPI == EPI_POOL) {
+		/* Pre-activation values of a group of output columns go through LDS (the operand buffers are free now), so
+		 * that the threads can be dealt out over (column, window, sample): a window's positions lie in different
+		 * lanes and waves. A pass stages, for one accumulator block i, the RG accumulator rows of group q of every
+		 * wave: FP = WAVES_F * RG columns x BM rows. */
+		constexpr int RG = std::is_same<T, float>::value ? 8 : 4, GROUPS = TL / RG, FP = WAVES_F * RG, LROW = BM + 4;
+		static_assert(FP * LROW <= 2 * KC * LDA, "the staging tile of the pooling epilogue reuses the A operand buffers");
+		T* const stage = &As[0][0][0];
+		const int SB = 1 << sb_shift, P = BM >> sb_shift, pa = P / L.pos_b;
+		const int W = P / (E.prh * E.prw), wa_n = pa / E.prh;
+		const int strip = tile / L.tile_rows, trow = tile - strip * L.tile_rows;
+		const int ab = trow / L.sample_blocks, nb = trow - ab * L.sample_blocks;
+		const int a_p0 = ab * wa_n, b_p0 = strip * (L.pos_b / E.prw);
+		act_dispatch(E.kind, [&](auto kc) {
+			constexpr int KIND = decltype(kc)::value;
+			#pragma unroll
+			for (int i = 0; i < FB; ++i) {
+				#pragma unroll
+				for (int q = 0; q < GROUPS; ++q) {
+					__syncthreads();
+					#pragma unroll
+					for (int r = 0; r < MF::NACC; ++r) {
+						if ((std::is_same<T, float>::value ? r / 4 : r) != q)
+							continue;
+						const int arow = acc_row<T>(r, lk);
+						const int f = f0 + wf * WT_F + FB * arow + i;
+						const T bv = (bias && f < g.F) ? bias[f] : (T) 0;
+						T v[MB];
+						#pragma unroll
+						for (int j = 0; j < MB; ++j)
+							v[j] = acc[i][j][r] + bv;
+						T* dst = stage + (wf * RG + arow - RG * q) * LROW + wm * WT_M + MB * lc;
+						#pragma unroll
+						for (int j0 = 0; j0 < MB; j0 += VS)
+							vec_store<T, VS>(dst + j0, *reinterpret_cast<T (*)[VS]>(&v[j0]));
+					}
+					__syncthreads();
+					for (int it = tid; it < FP * W * SB; it += THREADS) {
+						const int s_i = it & (SB - 1), t2 = it >> sb_shift;
+						const int fl = t2 / W, w = t2 - fl * W;
+						const int f = f0 + (fl / RG) * WT_F + FB * (RG * q + fl % RG) + i;
+						if (f >= g.F)
+							continue;
+						const int wb = w / wa_n, wa = w - wb * wa_n;
+						const T* col = stage + fl * LROW + s_i;
+						/* strict '>' from lowest(), width-major / height-minor scan (MaxPoolLayer.hpp:45-56) */
+						T best = std::numeric_limits<T>::lowest(), best_pre = col[((wa * E.prh) + pa * (wb * E.prw)) << sb_shift];
+						unsigned bi = 0;
+						for (int k = 0; k < E.prw; ++k)
+							for (int l = 0; l < E.prh; ++l) {
+								const T z = col[((wa * E.prh + l) + pa * (wb * E.prw + k)) << sb_shift];
+								const T y = act_f_coded<T, KIND>(z, E.p);
+								if (y > best) {
+									best = y;
+									best_pre = z;
+									bi = (unsigned) (k * E.prh + l);
+								}
+							}
+						const int n = (nb << sb_shift) + s_i, a_p = a_p0 + wa, b_p = b_p0 + wb;
+						out[(size_t) n + (size_t) g.N * (a_p + (size_t) E.OHp * (b_p + (size_t) E.OWp * f))] = best;
+						E.inds[((size_t) b_p * E.OHp + a_p) * ((size_t) g.F * g.N) + (size_t) f * g.N + n] = bi;
+						if (E.pre)
+							E.pre[(size_t) n + (size_t) g.N * (a_p + (size_t) E.OHp * (b_p + (size_t) E.OWp * f))] = best_pre;
+					}
+				}
+			}
+		});
+		return;
+	}
 	const bool vec_out = g.M % MB == 0 && (reinterpret_cast<uintptr_t>(out) & (VS * sizeof(T) - 1)) == 0;
 	const int mm = tile_row_m(L, g, tile, BM, wm * WT_M + MB * lc);
+	if constexpr (EPI == EPI_ACT) {
+		act_dispatch(E.kind, [&](auto kc) {
+			constexpr int KIND = decltype(kc)::value;
+			#pragma unroll
+			for (int i = 0; i < FB; ++i) {
+				#pragma unroll
+				for (int r = 0; r < MF::NACC; ++r) {
+					const int f = f0 + wf * WT_F + FB * acc_row<T>(r, lk) + i;
+					if (f >= g.F)
+						continue;
+					const T bv = bias ? bias[f] : (T) 0;
+					const size_t o = (size_t) mm + (size_t) g.M * f;
+					T z[MB], y[MB];
+					#pragma unroll
+					for (int j = 0; j < MB; ++j) {
+						z[j] = acc[i][j][r] + bv;
+						y[j] = act_f_coded<T, KIND>(z[j], E.p);
+					}
+					if (vec_out) {
+						if (mm < g.M) {
+							#pragma unroll
+							for (int j0 = 0; j0 < MB; j0 += VS) {
+								vec_store<T, VS>(out + o + j0, *reinterpret_cast<T (*)[VS]>(&y[j0]));
+								if (E.pre)
+									vec_store<T, VS>(E.pre + o + j0, *reinterpret_cast<T (*)[VS]>(&z[j0]));
+							}
+						}
+					} else {
+						#pragma unroll
+						for (int j = 0; j < MB; ++j)
+							if (mm + j < g.M) {
+								out[o + j] = y[j];
+								if (E.pre)
+									E.pre[o + j] = z[j];
+							}
+					}
+				}
+			}
+		});
+		return;
+	}
+	if constexpr (EPI == EPI_STATS) {
+		/* Moments of this tile's rows per output column, from the accumulators: per lane the sums of (z - c) and
+		 * (z - c)^2 about a value c of the same column (the first row of the wave's rows: a shift from within the
+		 * data, so the squares do not cancel), added over the lanes of a column by a butterfly, then the waves along
+		 * m merged in ascending order by the update of Chan et al. */
+		T* const red = &As[0][0][0];                    /* [WAVES_M][BF][4]: count, shift, sum, sum of squares */
+		static_assert(WAVES_M * (WAVES_F * WT_F) * 4 <= 2 * KC * LDA, "the moment partials reuse the A operand buffers");
+		#pragma unroll
+		for (int i = 0; i < FB; ++i) {
+			#pragma unroll
+			for (int r = 0; r < MF::NACC; ++r) {
+				const int fl = wf * WT_F + FB * acc_row<T>(r, lk) + i;
+				const T bv = (bias && f0 + fl < g.F) ? bias[f0 + fl] : (T) 0;
+				const T c = __shfl(acc[i][0][r] + bv, lane & ~(TL - 1), 64);
+				T cnt = (T) 0, s1 = (T) 0, s2 = (T) 0;
+				#pragma unroll
+				for (int j = 0; j < MB; ++j) {
+					const bool valid = mm + j < g.M;
+					const T d = valid ? (acc[i][j][r] + bv) - c : (T) 0;
+					cnt += valid ? (T) 1 : (T) 0;
+					s1 += d;
+					s2 += d * d;
+				}
+				#pragma unroll
+				for (int off = 1; off < TL; off <<= 1) {
+					cnt += __shfl_xor(cnt, off, 64);
+					s1 += __shfl_xor(s1, off, 64);
+					s2 += __shfl_xor(s2, off, 64);
+				}
+				if (lc == 0) {
+					T* dst = red + ((size_t) wm * BF + fl) * 4;
+					dst[0] = cnt;
+					dst[1] = c;
+					dst[2] = s1;
+					dst[3] = s2;
+				}
+			}
+		}
+		__syncthreads();
+		for (int fl = tid; fl < BF; fl += THREADS) {
+			if (f0 + fl >= g.F)
+				continue;
+			T n = (T) 0, mean = (T) 0, m2 = (T) 0;
+			#pragma unroll
+			for (int w = 0; w < WAVES_M; ++w) {
+				const T* src4 = red + ((size_t) w * BF + fl) * 4;
+				const T nb_ = src4[0];
+				if (nb_ > (T) 0) {
+					const T mb = src4[2] / nb_, meanb = src4[1] + mb, m2b = src4[3] - src4[2] * mb;
+					const T nt = n + nb_, d = meanb - mean, wgt = nb_ / nt;
+					mean += d * wgt;
+					m2 += m2b + (d * d) * (n * wgt);
+					n = nt;
+				}
+			}
+			T* dst = E.stats + ((size_t) tile * g.F + (f0 + fl)) * 3;
+			dst[0] = n;
+			dst[1] = mean;
+			dst[2] = m2;
+		}
+		/* the tile itself is stored below, like any other */
+	}
 	#pragma unroll
 	for (int i = 0; i < FB; ++i) {
 		#pragma unroll
@@ -868,10 +1044,10 @@ void* g_scratch_ptr[MAX_DEVICES] = { nullptr };
 
 /* out tile = bias + sum over the parts of a split reduction, parts taken in ascending order (so the result
  * does not depend on how blocks were scheduled). One block per (walk position, f block) tile. */
-template<typename T>
+template<typename T, bool ACT>
 __global__ __launch_bounds__(256)
 void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ bias, T* __restrict__ out, const GatherGeom g,
-		const GatherLaunch L, int BM, int BF, int ftiles) {
+		const GatherLaunch L, int BM, int BF, int ftiles, const Epilogue<T> E) {
 	const int M = g.M, F = g.F;
 	constexpr int V = 16 / (int) sizeof(T);             /* consecutive m per thread: one 16-byte load per part */
 	const int groups = BM * BF / (256 * V);             /* blocks per tile; tiles are multiples of 64 x 32 */
@@ -896,17 +1072,37 @@ void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ b
 	if (f >= F)
 		return;
 	const T bv = bias ? bias[f] : (T) 0;
-	T* dst = out + ((size_t) m + (size_t) M * f);
-	if (m + V <= M && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+	#pragma unroll
+	for (int i = 0; i < V; ++i)
+		acc[i] += bv;
+	T pre[V];
+	if constexpr (ACT) {
+		/* the activation epilogue of the whole tiles, applied to the summed parts (EPI_ACT) */
 		#pragma unroll
 		for (int i = 0; i < V; ++i)
-			acc[i] += bv;
+			pre[i] = acc[i];
+		act_dispatch(E.kind, [&](auto kc) {
+			#pragma unroll
+			for (int i = 0; i < V; ++i)
+				acc[i] = act_f_coded<T, decltype(kc)::value>(acc[i], E.p);
+		});
+	}
+	const size_t o = (size_t) m + (size_t) M * f;
+	T* dst = out + o;
+	if (m + V <= M && (reinterpret_cast<uintptr_t>(dst) & 15) == 0 && (!ACT || !E.pre || (reinterpret_cast<uintptr_t>(E.pre + o) & 15) == 0)) {
 		vec_store<T, V>(dst, acc);
+		if constexpr (ACT)
+			if (E.pre)
+				vec_store<T, V>(E.pre + o, pre);
 	} else {
 		#pragma unroll
 		for (int i = 0; i < V; ++i)
-			if (m + i < M)
-				dst[i] = acc[i] + bv;
+			if (m + i < M) {
+				dst[i] = acc[i];
+				if constexpr (ACT)
+					if (E.pre)
+						E.pre[o + i] = pre[i];
+			}
 	}
 }
 
@@ -916,44 +1112,60 @@ struct GatherVariant {
 	int bm, bf, waves, lds_bytes;
 	int kc;
 	void (*launch)(dim3 grid, size_t dyn_lds, const T*, const T*, const T*, T*, const GatherGeom&, const GatherLaunch&,
-			T* partials, bool vec, bool divs);
-	int (*blocks_per_cu)(size_t dyn_lds, bool vec, bool divs);       /* what the runtime says fits on a CU */
+			T* partials, bool vec, bool divs, int epi, const Epilogue<T>&);
+	int (*blocks_per_cu)(size_t dyn_lds, bool vec, bool divs, int epi);       /* what the runtime says fits on a CU */
 };
 
+/* The fused epilogues exist for the vectorised, divisor-free (forward) form of every tile shape. */
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
 void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g,
-		const GatherLaunch& L, T* partials, bool vec, bool divs) {
+		const GatherLaunch& L, T* partials, bool vec, bool divs, int epi, const Epilogue<T>& E) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	dim3 block(64 * WAVES_M * WAVES_F);
-	if (vec && !divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
+	if (epi != EPI_NONE) {
+		CATTLE_HIP_REQUIRE(vec && !divs, "a fused epilogue needs the vectorised forward form of the GEMM");
+		if (epi == EPI_ACT)
+			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+		else if (epi == EPI_POOL)
+			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+		else
+			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_STATS><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+	} else if (vec && !divs)
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else if (vec && divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else if (!divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
-int gather_variant_occupancy(size_t dyn, bool vec, bool divs) {
+int gather_variant_occupancy(size_t dyn, bool vec, bool divs, int epi) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	/* the answer for the usual launch (no reserved dynamic LDS) is kept: one query per kernel instantiation */
-	static int cached[4] = { 0, 0, 0, 0 };
-	int& slot = cached[(vec ? 2 : 0) + (divs ? 1 : 0)];
+	static int cached[7] = { 0, 0, 0, 0, 0, 0, 0 };
+	int& slot = cached[epi != EPI_NONE ? 3 + epi : (vec ? 2 : 0) + (divs ? 1 : 0)];
 	if (dyn == 0 && slot > 0)
 		return slot;
 	int n = 0;
 	hipError_t e;
-	if (vec && !divs)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false>, 64 * WAVES_M * WAVES_F, dyn);
+	constexpr int TH = 64 * WAVES_M * WAVES_F;
+	if (epi == EPI_ACT)
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT>, TH, dyn);
+	else if (epi == EPI_POOL)
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL>, TH, dyn);
+	else if (epi == EPI_STATS)
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_STATS>, TH, dyn);
+	else if (vec && !divs)
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false>, TH, dyn);
 	else if (vec && divs)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true>, 64 * WAVES_M * WAVES_F, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true>, TH, dyn);
 	else if (!divs)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false>, 64 * WAVES_M * WAVES_F, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false>, TH, dyn);
 	else
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true>, 64 * WAVES_M * WAVES_F, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true>, TH, dyn);
 	CATTLE_HIP_CHECK(e);
 	if (dyn == 0)
 		slot = n;
@@ -1068,10 +1280,53 @@ const Tuning& tuning() {
  * the gathered A operand, the expensive one, is read once), else the widest. Blocks run at the
  * occupancy their LDS and register use allows; measured on MI355X, more co-resident blocks beat
  * fewer blocks even when the last round of blocks is mostly idle. */
+/* The blocked tile order (tile_row_m) for tiles of bm rows: SB = 2^sb_shift samples x a pa x pos_b rectangle of
+ * output positions. With a pooling epilogue (prh x prw windows, stride = receptor) the rectangle must hold whole
+ * windows, and SB may shrink below 32 so that a tile holds at least one. */
+struct RowBlocks {
+	bool ok;
+	int sb_shift, sample_blocks, pos_b, tile_rows;
+};
+
 template<typename T>
-void launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, ScratchArena* arena = nullptr) {
+RowBlocks plan_row_blocks(const GatherGeom& g, int bm, int prh, int prw, bool pooled) {
+	RowBlocks rb = { false, 5, 0, 1, 0 };
+	const int min_shift = GemmCfg<T>::VEC == 4 ? 2 : 1;           /* a 16-byte access stays inside one sample block */
+	for (int shift = 5; shift >= (pooled ? min_shift : 5); --shift) {
+		const int sb = 1 << shift;
+		if (g.N % sb != 0 || bm % sb != 0)
+			continue;
+		const int positions = bm / sb;
+		for (int pb = prw; pb <= positions; pb *= 2) {
+			const int pa = positions / pb;
+			if (positions % pb == 0 && pa % prh == 0 && g.OA % pa == 0 && g.OB % pb == 0 && (pooled || g.OB / pb > 1)) {
+				rb.ok = true;
+				rb.sb_shift = shift;
+				rb.sample_blocks = g.N / sb;
+				rb.pos_b = pb;
+				rb.tile_rows = rb.sample_blocks * (g.OA / pa);
+				return rb;
+			}
+		}
+	}
+	return rb;
+}
+
+/* Picks the tile shape: the narrowest F tile that covers all output columns in one block column (so
+ * the gathered A operand, the expensive one, is read once), else the widest. Blocks run at the
+ * occupancy their LDS and register use allows; measured on MI355X, more co-resident blocks beat
+ * fewer blocks even when the last round of blocks is mostly idle.
+ * With a fused epilogue (epi != EPI_NONE; `E` its arguments) the launch needs 16-byte accesses; the pooling and the
+ * moments epilogue need whole tiles in one block (no cut reductions), the pooling epilogue the blocked tile order
+ * with whole windows per tile. Returns false, without launching, when the problem does not allow that; `mtiles_out`
+ * receives the number of M tiles (the row count of the moments epilogue's partials). */
+template<typename T>
+bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, ScratchArena* arena = nullptr,
+		int epi = EPI_NONE, const Epilogue<T>* E = nullptr, int* mtiles_out = nullptr) {
 	const bool vec = g.N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
 	const bool divs = g.DA != 1 || g.DB != 1;
+	if (epi != EPI_NONE && (!vec || divs || (reinterpret_cast<uintptr_t>(out) & 15) != 0))
+		return false;
 	const GatherVariant<T>* vars = GatherVariants<T>::get();
 	int best_v = 0;
 	for (int i = 1; i < GatherVariants<T>::LARGE; ++i) {
@@ -1103,6 +1358,20 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 			best_v = o->variant;
 		occ = o->occ;
 	}
+	const bool pooled = epi == EPI_POOL;
+	RowBlocks rb = { false, 5, 0, 1, 0 };
+	if (pooled) {
+		/* the chosen shape if whole windows fit its tiles, else the same width with the other height */
+		rb = plan_row_blocks<T>(g, vars[best_v].bm, E->prh, E->prw, true);
+		for (int i = 0; !rb.ok && i < GatherVariants<T>::COUNT; ++i)
+			if (vars[i].bf == vars[best_v].bf && vars[i].bm != vars[best_v].bm && vars[i].bm <= 256) {
+				rb = plan_row_blocks<T>(g, vars[i].bm, E->prh, E->prw, true);
+				if (rb.ok)
+					best_v = i;
+			}
+		if (!rb.ok)
+			return false;
+	}
 	const GatherVariant<T>& v = vars[best_v];
 	size_t dyn = 0;
 	if (occ >= 1 && occ <= 8) {
@@ -1114,30 +1383,35 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	/* tiles per output column, if a column (N * OA rows of M) is a whole number of tiles and there are
 	 * several columns; 0 switches the 2-D walk off */
 	const long column = (long) g.N * g.OA;
-	int tile_rows = (column % v.bm == 0 && g.OB > 1 && !tune.no_swizzle) ? (int) (column / v.bm) : 0;
+	int tile_rows = (column % v.bm == 0 && g.OB > 1 && !tune.no_swizzle && !pooled) ? (int) (column / v.bm) : 0;
 	/* rows of a tile as 32 samples x a rectangle of positions (see tile_row_m) where the shape allows it: as many
 	 * positions along a as divide OA, the rest along b; the 2-D walk then runs over strips of pos_b columns */
-	int sample_blocks = 0, pos_b = 1;
-	if (g.N % 32 == 0 && v.bm % 32 == 0 && g.OB > 1 && !tune.no_swizzle && !tune.no_row_blocks) {
-		const int positions = v.bm / 32;
-		for (int pb = 1; pb <= positions; pb *= 2) {
-			const int pa = positions / pb;
-			if (positions % pb == 0 && g.OA % pa == 0 && g.OB % pb == 0 && g.OB / pb > 1) {
-				sample_blocks = g.N / 32;
-				pos_b = pb;
-				tile_rows = sample_blocks * (g.OA / pa);
-				break;
-			}
+	int sample_blocks = 0, pos_b = 1, sb_shift = 5;
+	if (pooled) {
+		sample_blocks = rb.sample_blocks;
+		pos_b = rb.pos_b;
+		tile_rows = rb.tile_rows;
+		sb_shift = rb.sb_shift;
+	} else if (g.N % 32 == 0 && v.bm % 32 == 0 && g.OB > 1 && !tune.no_swizzle && !tune.no_row_blocks) {
+		rb = plan_row_blocks<T>(g, v.bm, 1, 1, false);
+		if (rb.ok) {
+			sample_blocks = rb.sample_blocks;
+			pos_b = rb.pos_b;
+			tile_rows = rb.tile_rows;
 		}
 	}
+	if (mtiles_out)
+		*mtiles_out = mtiles;
 	/* blocks the chip holds at once (registers, LDS, waves), as the runtime computes it for this kernel */
-	const int per_cu = std::max(1, v.blocks_per_cu(dyn, vec, divs));
+	const int per_cu = std::max(1, v.blocks_per_cu(dyn, vec, divs, epi));
 	const int slots = NUM_CUS * per_cu;
-	const bool no_split = tune.no_split;
+	const bool no_split = tune.no_split || epi == EPI_POOL || epi == EPI_STATS;
+	const Epilogue<T> none = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr };
+	const Epilogue<T>& epi_args = E ? *E : none;
 
 	/* main_count whole tiles, the other mtiles - main_count with their reduction cut into about `ksplit` parts */
 	auto launch = [&](int main_count, int ksplit) {
-		GatherLaunch L = { mtiles, tile_rows, main_count, round_up(main_count, 8), mtiles - main_count, 1, nchunks, sample_blocks, pos_b };
+		GatherLaunch L = { mtiles, tile_rows, main_count, round_up(main_count, 8), mtiles - main_count, 1, nchunks, sample_blocks, pos_b, sb_shift };
 		T* partials = nullptr;
 		if (L.split_count > 0) {
 			L.chunks_per_part = (nchunks + ksplit - 1) / ksplit;
@@ -1146,11 +1420,14 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 			partials = static_cast<T*>(arena ? arena->take(pbytes, "partial sums of the split reduction") : split_workspace(pbytes));
 		}
 		dim3 grid((unsigned) (L.main_blocks + L.split_count * L.ksplit), (unsigned) ftiles);
-		v.launch(grid, dyn, src, wt, bias, out, g, L, partials, vec, divs);
+		v.launch(grid, dyn, src, wt, bias, out, g, L, partials, vec, divs, epi, epi_args);
 		if (L.split_count > 0) {
 			const int groups = v.bm * v.bf / (256 * (16 / (int) sizeof(T)));
-			split_reduce_kernel<T><<<dim3((unsigned) (L.split_count * ftiles * groups)), 256, 0, stream()>>>(partials, bias, out,
-					g, L, v.bm, v.bf, ftiles);
+			const dim3 rgrid((unsigned) (L.split_count * ftiles * groups));
+			if (epi == EPI_ACT)
+				split_reduce_kernel<T, true><<<rgrid, 256, 0, stream()>>>(partials, bias, out, g, L, v.bm, v.bf, ftiles, epi_args);
+			else
+				split_reduce_kernel<T, false><<<rgrid, 256, 0, stream()>>>(partials, bias, out, g, L, v.bm, v.bf, ftiles, epi_args);
 			CATTLE_HIP_CHECK(hipGetLastError());
 		}
 	};
@@ -1159,7 +1436,7 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	if (!no_split && total * 2 <= slots && nchunks >= 4) {
 		/* far fewer tiles than the chip holds blocks: cut every tile's reduction so that it fills up */
 		launch(0, (int) std::min<long>(std::min<long>(slots / total, nchunks / 2), 16));
-		return;
+		return true;
 	}
 	const int rem = mtiles % slots;
 	if (!no_split && ftiles == 1 && mtiles > slots && rem > 0 && rem * 2 <= slots && nchunks >= 8) {
@@ -1167,9 +1444,10 @@ void launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		 * Their reduction is cut into parts instead; the part blocks come last in the grid and fill the
 		 * chip as the last round of whole tiles drains. */
 		launch(mtiles - rem, (int) std::min<long>(std::min(slots / rem, nchunks / 4), 16));
-		return;
+		return true;
 	}
 	launch(mtiles, 1);
+	return true;
 }
 
 GatherGeom forward_geom(const ConvShape& s, int N) {
@@ -1360,6 +1638,34 @@ void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b,
 	launch_gather<T>(x, wt, b, out, g);
 }
 
+template<typename T>
+bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out, T* wt, bool wt_ready, int epi,
+		const Epilogue<T>& E, int* mtiles) {
+	check_sizes(s, N);
+	const GatherGeom g = forward_geom(s, N);
+	if (epi == EPI_POOL) {
+		CATTLE_HIP_REQUIRE(E.prh > 0 && E.prw > 0 && g.OA % E.prh == 0 && g.OB % E.prw == 0 && E.OHp == g.OA / E.prh &&
+				E.OWp == g.OB / E.prw && E.inds != nullptr, "the pooling epilogue needs windows that tile the output");
+		/* the staging pass deals threads over windows of at most a tile's positions */
+		if (E.prh * E.prw > 64)
+			return false;
+	}
+	if (epi == EPI_STATS)
+		CATTLE_HIP_REQUIRE(E.stats != nullptr, "the moments epilogue needs a buffer for its partials");
+	if (!wt_ready) {
+		const int Kp = round_up(g.K, WT_ROW_PAD);
+		const size_t count = (size_t) Kp * g.ldw;
+		prep_fwd_weights_kernel<T><<<(unsigned) ((count + 255) / 256), 256, 0, stream()>>>(w, wt, g.K, g.F, Kp, g.ldw);
+		CATTLE_HIP_CHECK(hipGetLastError());
+	}
+	return launch_gather<T>(x, wt, b, out, g, nullptr, epi, &E, mtiles);
+}
+
+size_t conv_stats_rows(const ConvShape& s, int N) {
+	/* the shortest tile of either variant table has 64 rows */
+	return ((size_t) N * s.OH() * s.OW() + 63) / 64;
+}
+
 void static_scratch_setup() {
 	int dev = -1;
 	CATTLE_HIP_CHECK(hipGetDevice(&dev));
@@ -1448,6 +1754,10 @@ template ConvWorkspace conv_workspace<float>(const ConvShape&, int);
 template ConvWorkspace conv_workspace<double>(const ConvShape&, int);
 template void conv_forward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, bool);
 template void conv_forward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*, bool);
+template bool conv_forward_fused<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, bool, int,
+		const Epilogue<float>&, int*);
+template bool conv_forward_fused<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*, bool, int,
+		const Epilogue<double>&, int*);
 template void conv_forward_static<float>(const ConvShape&, int, const float*, const float*, const float*, float*);
 template void conv_forward_static<double>(const ConvShape&, int, const double*, const double*, const double*, double*);
 template void conv_backward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, float*,

@@ -7,6 +7,7 @@
  * and pointwise_kernels.hip. There is no host implementation of any operation here.
  */
 #include "common.hpp"
+#include "act_math.hpp"
 #include "../../include/cattle_hip.h"
 
 #include <cstring>
@@ -741,6 +742,297 @@ struct PoolLayer : LayerBase {
 		LayerBase::empty_cache();
 		inds_count = 0;
 		inds.release();
+	}
+};
+
+/* A kernel layer and the layers a feed-forward network calls right after it (FeedforwardNeuralNetwork.hpp:112-127:
+ * layers[i]->pass_forward one after another; backwards :129-141), run as one: convolution or dense -> [per-channel batch
+ * norm] -> [element-wise activation] -> [pool]. The member layers stay what they are (their own parameter objects, the
+ * running statistics and the arg-max cache of the batch norm and pool layer); this object only replaces the calls.
+ *   MODE_ACT   the activation is the GEMM's epilogue (the pool, if any, runs as its own pass);
+ *   MODE_POOL  activation and max pooling are the GEMM's epilogue: the full-size activation tensor is never written;
+ *   MODE_BN    the GEMM's epilogue also produces the per-tile moments of its output, and one more pass normalises,
+ *              activates and pools; the backward pass recomputes the normalised values from the GEMM output;
+ *   MODE_UNFUSED  the member layers' own passes, one after another, for everything else (batch sizes or alignments without
+ *              16-byte accesses, windows that overlap or do not fit the tiles, parametric activations, softmax).
+ * The mode is chosen per forward pass; results do not depend on it beyond rounding. */
+enum { MODE_NONE = 0, MODE_UNFUSED = 1, MODE_ACT = 2, MODE_POOL = 3, MODE_BN = 4 };
+
+template<typename T>
+struct FusedLayer : LayerBase {
+	ConvLayer<T>* conv = nullptr;
+	BatchNormLayer<T>* bn = nullptr;
+	ActivationLayer<T>* act = nullptr;
+	PoolLayer<T>* pool = nullptr;
+	std::vector<LayerBase*> members;        /* in call order */
+	bool owns_members = false;              /* a clone owns the clones of its members */
+	int mode = MODE_NONE;
+	bool pool_in_chain = false;             /* MODE_BN: the pool is part of the chain pass */
+	bool trained = false;                   /* the last forward pass was a training pass (MODE_BN keeps moments only then) */
+	const T* y_cache = nullptr;             /* (coded) output the backward pass derives act' from; may be the caller's buffer */
+	DevBuf z_buf, pre_buf, dz_buf, stats_buf, mean_buf, chain_ws;
+	std::vector<std::unique_ptr<DevBuf>> mid;       /* MODE_UNFUSED: outputs of all members but the last; gradients likewise */
+	DevBuf grad_a, grad_b;
+
+	FusedLayer(int dtype, const std::vector<LayerBase*>& layers, bool owns) : LayerBase(dtype), members(layers), owns_members(owns) {
+		CATTLE_HIP_REQUIRE(!layers.empty(), "a fused layer needs a kernel layer");
+		size_t at = 0;
+		conv = dynamic_cast<ConvLayer<T>*>(layers[at]);
+		CATTLE_HIP_REQUIRE(conv != nullptr, "the first member must be a convolutional or dense kernel layer of the same scalar type");
+		++at;
+		if (at < layers.size() && (bn = dynamic_cast<BatchNormLayer<T>*>(layers[at])))
+			++at;
+		if (at < layers.size() && (act = dynamic_cast<ActivationLayer<T>*>(layers[at])))
+			++at;
+		if (at < layers.size() && (pool = dynamic_cast<PoolLayer<T>*>(layers[at])))
+			++at;
+		CATTLE_HIP_REQUIRE(at == layers.size(), "members must be: kernel layer, then optionally batch norm, activation, pool, in this order");
+		for (size_t i = 0; i + 1 < layers.size(); ++i)
+			CATTLE_HIP_REQUIRE(layers[i]->out_volume() == layers[i + 1]->in_volume(), "member dimensions do not chain");
+		std::memcpy(in_dims, conv->in_dims, sizeof(in_dims));
+		std::memcpy(out_dims, layers.back()->out_dims, sizeof(out_dims));
+		input_layer = conv->input_layer;
+		for (LayerBase* l : layers)
+			for (const ParamPtr& q : l->params)
+				params.push_back(q);
+	}
+	~FusedLayer() override {
+		if (owns_members)
+			for (LayerBase* l : members)
+				delete l;
+	}
+	LayerBase* clone(bool share) const override {
+		std::vector<LayerBase*> copies;
+		for (LayerBase* l : members)
+			copies.push_back(l->clone(share));
+		FusedLayer* f = new FusedLayer(dtype, copies, true);
+		f->input_layer = input_layer;
+		return f;
+	}
+
+	int OH() const { return conv->shape.OH(); }
+	int OW() const { return conv->shape.OW(); }
+	int F() const { return conv->shape.F; }
+	bool act_fusable() const {
+		return !act || act->kind <= CATTLE_HIP_ACT_SWISH;
+	}
+	/* the pool's windows tile the kernel layer's output exactly */
+	bool pool_tiles() const {
+		if (!pool)
+			return false;
+		const PoolShape& ps = pool->shape;
+		return ps.H == OH() && ps.W == OW() && ps.C == F() && ps.sv == ps.RH && ps.sh == ps.RW && ps.H % ps.RH == 0 && ps.W % ps.RW == 0;
+	}
+	bool bn_fusable() const {
+		return bn && bn->groups() == (size_t) F();
+	}
+	ChainShape chain_shape(bool with_pool) const {
+		ChainShape cs;
+		cs.H = OH(); cs.W = OW(); cs.C = F();
+		cs.prh = with_pool ? pool->shape.RH : 1;
+		cs.prw = with_pool ? pool->shape.RW : 1;
+		cs.pool = with_pool ? (pool->kind == CATTLE_HIP_POOL_MAX ? 1 : 2) : 0;
+		cs.kind = act ? act->kind : CATTLE_HIP_ACT_IDENTITY;
+		cs.p = act ? (double) act->p : 0.0;
+		return cs;
+	}
+	T* prepared_weights(int n, bool& ready) {
+		const ConvWorkspace ws = conv_workspace<T>(conv->shape, n);
+		Param& w = *conv->params[0];
+		ready = w.derived_version[0] == w.version;
+		return (T*) w.derived[0].ensure(ws.wt_fwd * sizeof(T));
+	}
+	void weights_prepared() {
+		Param& w = *conv->params[0];
+		w.derived_version[0] = w.version;
+	}
+
+	void forward(const void* in, size_t N, bool training, void* out) override {
+		const int n = checked_int(N, "batch size");
+		const size_t zcount = N * conv->out_volume();
+		checked_int(zcount, "tensor size");
+		mode = MODE_NONE;
+		trained = training;
+		const T* x = (const T*) in;
+		const T* wv = (const T*) conv->params[0]->values.p;
+		const T* bv = (const T*) conv->params[1]->values.p;
+		const int kind = act ? act->kind : CATTLE_HIP_ACT_IDENTITY;
+		const T ap = act ? act->p : (T) 0;
+		Epilogue<T> E = { kind, ap, nullptr, nullptr, 1, 1, OH(), OW(), nullptr };
+		if (members.size() == 1 || !act_fusable() || (bn && !bn_fusable())) {
+			forward_unfused(in, N, training, out);
+			return;
+		}
+		bool ready;
+		T* wt = prepared_weights(n, ready);
+		if (bn) {
+			if (bn && !training)
+				CATTLE_HIP_REQUIRE(bn->stats_init, "inference before any training pass: running statistics unset");
+			T* z = (T*) z_buf.ensure(zcount * sizeof(T));
+			int mtiles = 0;
+			bool ok = true;
+			if (training) {
+				E.stats = (T*) stats_buf.ensure(conv_stats_rows(conv->shape, n) * F() * 3 * sizeof(T));
+				ok = conv_forward_fused<T>(conv->shape, n, x, wv, bv, z, wt, ready, EPI_STATS, E, &mtiles);
+				weights_prepared();
+			}
+			if (!ok) {
+				forward_unfused(in, N, training, out);
+				return;
+			}
+			if (!training) {
+				conv_forward<T>(conv->shape, n, x, wv, bv, z, wt, ready);
+				weights_prepared();
+			}
+			pool_in_chain = pool_tiles();
+			const ChainShape cs = chain_shape(pool_in_chain);
+			T* dst = (T*) out;
+			if (pool && !pool_in_chain)
+				dst = (T*) pre_buf.ensure(zcount * sizeof(T));      /* the pool's input */
+			unsigned* ip = nullptr;
+			if (pool_in_chain && pool->kind == CATTLE_HIP_POOL_MAX) {
+				pool->inds_count = N * pool->out_volume();
+				ip = (unsigned*) pool->inds.ensure(pool->inds_count * sizeof(unsigned));
+			}
+			T* mean_c = (T*) mean_buf.ensure((size_t) F() * sizeof(T));
+			T* isd_c = (T*) bn->inv_sd_cache.ensure((size_t) F() * sizeof(T));
+			bn_chain_forward<T>(cs, n, mtiles, training, bn->stats_init, z, E.stats, (const T*) bn->params[2]->values.p,
+					(const T*) bn->params[3]->values.p, (T*) bn->params[0]->values.p, (T*) bn->params[1]->values.p, bn->decay, bn->eps,
+					mean_c, isd_c, dst, ip);
+			if (training) {
+				bn->stats_init = true;
+				bn->cache_valid = false;        /* the member's own backward pass has nothing to work from */
+				++bn->params[0]->version;
+				++bn->params[1]->version;
+			}
+			if (pool && !pool_in_chain)
+				pool->forward(dst, N, training, out);
+			conv->x_cache = x;
+			mode = MODE_BN;
+			return;
+		}
+		const bool needs_pre = !act_backward_from_output(kind, (double) ap);
+		if (pool && pool->kind == CATTLE_HIP_POOL_MAX && pool_tiles()) {
+			const size_t pcount = N * pool->out_volume();
+			E.prh = pool->shape.RH;
+			E.prw = pool->shape.RW;
+			E.OHp = OH() / E.prh;
+			E.OWp = OW() / E.prw;
+			E.inds = (unsigned*) pool->inds.ensure(pcount * sizeof(unsigned));
+			E.pre = needs_pre ? (T*) pre_buf.ensure(pcount * sizeof(T)) : nullptr;
+			const bool ok = conv_forward_fused<T>(conv->shape, n, x, wv, bv, (T*) out, wt, ready, EPI_POOL, E, nullptr);
+			weights_prepared();
+			ready = true;
+			if (ok) {
+				pool->inds_count = pcount;
+				conv->x_cache = x;
+				y_cache = (const T*) out;
+				mode = MODE_POOL;
+				return;
+			}
+			E.inds = nullptr;
+			E.prh = E.prw = 1;
+			E.OHp = OH();
+			E.OWp = OW();
+		}
+		if (act) {
+			T* y = pool ? (T*) z_buf.ensure(zcount * sizeof(T)) : (T*) out;
+			E.pre = needs_pre ? (T*) pre_buf.ensure(zcount * sizeof(T)) : nullptr;
+			const bool ok = conv_forward_fused<T>(conv->shape, n, x, wv, bv, y, wt, ready, EPI_ACT, E, nullptr);
+			weights_prepared();
+			if (ok) {
+				if (pool)
+					pool->forward(y, N, training, out);
+				conv->x_cache = x;
+				y_cache = y;
+				mode = MODE_ACT;
+				return;
+			}
+		}
+		forward_unfused(in, N, training, out);
+	}
+
+	void forward_unfused(const void* in, size_t N, bool training, void* out) {
+		while (mid.size() + 1 < members.size())
+			mid.push_back(std::unique_ptr<DevBuf>(new DevBuf()));
+		const void* cur = in;
+		for (size_t i = 0; i < members.size(); ++i) {
+			LayerBase* l = members[i];
+			void* dst = i + 1 == members.size() ? out : mid[i]->ensure(N * l->out_volume() * esize());
+			l->forward(cur, N, training, dst);
+			cur = dst;
+		}
+		mode = MODE_UNFUSED;
+	}
+
+	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		CATTLE_HIP_REQUIRE(mode != MODE_NONE, "pass_back without a cached forward pass");
+		const int n = checked_int(N, "batch size");
+		const size_t zcount = N * conv->out_volume();
+		if (mode == MODE_UNFUSED) {
+			const void* g = out_grad;
+			for (size_t i = members.size(); i-- > 0;) {
+				LayerBase* l = members[i];
+				void* dst = in_grad;
+				if (i > 0)
+					dst = ((members.size() - i) % 2 ? grad_a : grad_b).ensure(N * l->in_volume() * esize());
+				l->backward(g, N, dst);
+				g = dst;
+			}
+			return;
+		}
+		const T* g = (const T*) out_grad;
+		T* dz = (T*) dz_buf.ensure(zcount * sizeof(T));
+		if (mode == MODE_BN) {
+			if (!trained)
+				throw Error(ERR_STATE, "pass_back without a training-mode forward pass");
+			if (pool && !pool_in_chain) {
+				T* gp = (T*) grad_a.ensure(zcount * sizeof(T));
+				pool->backward(g, N, gp);
+				g = gp;
+			}
+			const ChainShape cs = chain_shape(pool_in_chain);
+			T* ws = (T*) chain_ws.ensure(bn_chain_workspace(F()) * sizeof(T));
+			bn_chain_backward<T>(cs, n, g, pool_in_chain ? (const unsigned*) pool->inds.p : nullptr, (const T*) z_buf.p,
+					(const T*) bn->params[2]->values.p, (const T*) bn->params[3]->values.p, (const T*) mean_buf.p,
+					(const T*) bn->inv_sd_cache.p, (T*) bn->params[2]->grad.p, (T*) bn->params[3]->grad.p, dz, ws);
+		} else if (mode == MODE_POOL) {
+			CATTLE_HIP_REQUIRE(pool->inds_count == N * pool->out_volume(), "pass_back without cached max indices");
+			chain_backward<T>(chain_shape(true), n, g, (const unsigned*) pool->inds.p, y_cache, needs_pre() ? (const T*) pre_buf.p : nullptr, dz);
+		} else {
+			if (pool) {
+				T* gp = (T*) grad_a.ensure(zcount * sizeof(T));
+				pool->backward(g, N, gp);
+				g = gp;
+			}
+			chain_backward<T>(chain_shape(false), n, g, nullptr, y_cache, needs_pre() ? (const T*) pre_buf.p : nullptr, dz);
+		}
+		conv->backward(dz, N, in_grad);
+	}
+	bool needs_pre() const {
+		return act && !act_backward_from_output(act->kind, (double) act->p);
+	}
+	void empty_cache() override {
+		LayerBase::empty_cache();
+		for (LayerBase* l : members)
+			l->empty_cache();
+		mode = MODE_NONE;
+		y_cache = nullptr;
+		z_buf.release();
+		pre_buf.release();
+		dz_buf.release();
+		grad_a.release();
+		grad_b.release();
+		mid.clear();
+	}
+	void check_borrowed() const override {
+		if (mode == MODE_UNFUSED) {
+			for (LayerBase* l : members)
+				l->check_borrowed();
+			return;
+		}
+		require_not_released(conv->x_cache);
+		require_not_released(y_cache);
 	}
 };
 
@@ -1529,6 +1821,36 @@ int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t 
 		LayerBase* l = dtype == CATTLE_HIP_F32 ? (LayerBase*) new PoolLayer<float>(dtype, kind, s) :
 				(LayerBase*) new PoolLayer<double>(dtype, kind, s);
 		*layer = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_fused_create(const cattle_hip_layer_t* layers, size_t count, cattle_hip_layer_t* fused) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(layers != nullptr && fused != nullptr, "null pointer");
+		CATTLE_HIP_REQUIRE(count >= 1 && count <= 4, "a fused layer has one to four members");
+		std::vector<LayerBase*> members;
+		for (size_t i = 0; i < count; ++i) {
+			members.push_back(as_layer(layers[i]));
+			CATTLE_HIP_REQUIRE(members[i]->dtype == members[0]->dtype, "members differ in scalar type");
+			for (size_t j = 0; j < i; ++j)
+				CATTLE_HIP_REQUIRE(members[j] != members[i], "a layer is listed twice");
+		}
+		LayerBase* l = members[0]->dtype == CATTLE_HIP_F32 ? (LayerBase*) new FusedLayer<float>(CATTLE_HIP_F32, members, false) :
+				(LayerBase*) new FusedLayer<double>(CATTLE_HIP_F64, members, false);
+		*fused = reinterpret_cast<cattle_hip_layer_t>(l);
+	});
+}
+
+int cattle_hip_fused_last_mode(cattle_hip_layer_t fused, int* mode) {
+	return guarded([&] {
+		LayerBase* l = as_layer(fused);
+		CATTLE_HIP_REQUIRE(mode != nullptr, "null output pointer");
+		if (FusedLayer<float>* f = dynamic_cast<FusedLayer<float>*>(l))
+			*mode = f->mode;
+		else if (FusedLayer<double>* f = dynamic_cast<FusedLayer<double>*>(l))
+			*mode = f->mode;
+		else
+			throw Error(ERR_INVALID, "not a fused layer");
 	});
 }
 

@@ -7,6 +7,7 @@
  * order), so results are reproducible run to run; no atomics are used anywhere.
  */
 #include "common.hpp"
+#include "act_math.hpp"
 
 #include <algorithm>
 #include <limits>
@@ -15,69 +16,6 @@
 namespace cattle_hip {
 
 namespace {
-
-enum ActKind {
-	ACT_IDENTITY = 0, ACT_SCALED = 1, ACT_BINARY_STEP = 2, ACT_SIGMOID = 3, ACT_TANH = 4, ACT_SOFTSIGN = 5,
-	ACT_SOFTPLUS = 6, ACT_RELU = 7, ACT_LEAKY_RELU = 8, ACT_ELU = 9, ACT_SWISH = 10
-};
-
-__device__ __forceinline__ float dev_exp(float v) { return expf(v); }
-__device__ __forceinline__ double dev_exp(double v) { return exp(v); }
-__device__ __forceinline__ float dev_log(float v) { return logf(v); }
-__device__ __forceinline__ double dev_log(double v) { return log(v); }
-__device__ __forceinline__ float dev_tanh(float v) { return tanhf(v); }
-__device__ __forceinline__ double dev_tanh(double v) { return tanh(v); }
-__device__ __forceinline__ float dev_sqrt(float v) { return sqrtf(v); }
-__device__ __forceinline__ double dev_sqrt(double v) { return sqrt(v); }
-
-/* Forward functions; each cites the reference layer whose formula it evaluates. */
-template<typename T, int KIND>
-__device__ __forceinline__ T act_f(T x, T p) {
-	switch (KIND) {
-	case ACT_IDENTITY: return x;                                        /* IdentityActivationLayer.hpp:37-42 */
-	case ACT_SCALED: return x * p;                                      /* ScaledActivationLayer.hpp:38-43 */
-	case ACT_BINARY_STEP: return (T) (x >= (T) 0);                      /* BinaryStepActivationLayer.hpp:42-47 */
-	case ACT_SIGMOID: return (T) 1 / (dev_exp(-x) + (T) 1);             /* SigmoidActivationLayer.hpp:38-43 */
-	case ACT_TANH: return dev_tanh(x);                                  /* TanhActivationLayer.hpp:38-43 */
-	case ACT_SOFTSIGN: return x / ((T) 1 + (x < (T) 0 ? -x : x));       /* SoftsignActivationLayer.hpp:39-44 */
-	case ACT_SOFTPLUS: return dev_log(dev_exp(x) + (T) 1);              /* SoftplusActivationLayer.hpp:40-45 */
-	case ACT_RELU: return x > (T) 0 ? x : (x == x ? (T) 0 : x);         /* ReLUActivationLayer.hpp:45-50 */
-	case ACT_LEAKY_RELU: { const T ax = x * p; return x > ax ? x : (ax == ax ? ax : x); }   /* LeakyReLU :50-55 */
-	case ACT_ELU: return x >= (T) 0 ? x : p * (dev_exp(x) - (T) 1);     /* ELUActivationLayer.hpp:55-64 */
-	case ACT_SWISH: return x * ((T) 1 / (dev_exp(-p * x) + (T) 1));     /* SwishActivationLayer.hpp:45-51 */
-	}
-	return x;
-}
-
-/* Backward functions of (input x, output y, upstream gradient g). */
-template<typename T, int KIND>
-__device__ __forceinline__ T act_b(T x, T y, T g, T p) {
-	switch (KIND) {
-	case ACT_IDENTITY: return g;                                        /* IdentityActivationLayer.hpp:43-49 */
-	case ACT_SCALED: return g * p;                                      /* ScaledActivationLayer.hpp:44-50 */
-	case ACT_BINARY_STEP: return (T) 0;                                 /* BinaryStepActivationLayer.hpp:48-54 */
-	case ACT_SIGMOID: return (y * ((T) 1 - y)) * g;                     /* SigmoidActivationLayer.hpp:44-50 */
-	case ACT_TANH: return ((T) 1 - y * y) * g;                          /* TanhActivationLayer.hpp:44-50 */
-	case ACT_SOFTSIGN: { const T d = (T) 1 + (x < (T) 0 ? -x : x); return ((T) 1 / (d * d)) * g; }   /* :45-51 */
-	case ACT_SOFTPLUS: return ((T) 1 / (dev_exp(-x) + (T) 1)) * g;      /* SoftplusActivationLayer.hpp:46-52 */
-	case ACT_RELU: return (T) (x >= (T) 0) * g;                         /* ReLUActivationLayer.hpp:51-57 */
-	case ACT_LEAKY_RELU: return (x >= (T) 0 ? (T) 1 : p) * g;           /* LeakyReLUActivationLayer.hpp:56-62 */
-	case ACT_ELU: return (x >= (T) 0 ? (T) 1 : (y + p)) * g;            /* ELUActivationLayer.hpp:65-78 */
-	case ACT_SWISH: {                                                   /* SwishActivationLayer.hpp:52-59 */
-		const T s = (T) 1 / (dev_exp(-p * x) + (T) 1);
-		return s * ((((T) 1 - s) * p) * x + (T) 1) * g;
-	}
-	}
-	return g;
-}
-
-/* Which cached operands the backward of a kind actually reads (the others may be null). */
-__host__ __device__ constexpr bool act_needs_x(int k) {
-	return k == ACT_SOFTSIGN || k == ACT_SOFTPLUS || k == ACT_RELU || k == ACT_LEAKY_RELU || k == ACT_ELU || k == ACT_SWISH;
-}
-__host__ __device__ constexpr bool act_needs_y(int k) {
-	return k == ACT_SIGMOID || k == ACT_TANH || k == ACT_ELU;
-}
 
 template<typename T> struct Pack { static constexpr int V = 16 / (int) sizeof(T); typedef T type __attribute__((ext_vector_type(16 / sizeof(T)))); };
 
@@ -1425,8 +1363,448 @@ void broadcast_backward(int H, int W, int C, int bh, int bw, int bc, int N, cons
 	check_launch();
 }
 
+/* ----------------------------------------------------------------------------------------------
+ * The element-wise and pooling layers behind a kernel layer, run as one pass each way (a fused kernel layer:
+ * convolution or dense -> [batch norm] -> [activation] -> [pool]). `z` is the kernel layer's output (N, H, W, C);
+ * pooling windows tile it exactly (stride = receptor, H % prh == 0, W % prw == 0). A thread owns V consecutive
+ * samples of one window. Channel c is the slab [c * N*H*W, (c+1) * N*H*W) of z and [c * Lp, (c+1) * Lp) of the
+ * pooled tensor, Lp = N * (H/prh) * (W/prw).
+ * -------------------------------------------------------------------------------------------- */
+namespace {
+
+enum { CHAIN_POOL_NONE = 0, CHAIN_POOL_MAX = 1, CHAIN_POOL_MEAN = 2 };
+
+template<typename T, int V> struct ChainVec { typedef T type __attribute__((ext_vector_type(V))); typedef unsigned utype __attribute__((ext_vector_type(V))); };
+template<typename T> struct ChainVec<T, 1> { typedef T type; typedef unsigned utype; };
+
+template<typename T, int V>
+__device__ __forceinline__ void chain_load(T (&dst)[V], const T* p) {
+	if constexpr (V == 1) {
+		dst[0] = *p;
+	} else {
+		typedef T vt __attribute__((ext_vector_type(V)));
+		const vt v = *reinterpret_cast<const vt*>(p);
+		#pragma unroll
+		for (int i = 0; i < V; ++i)
+			dst[i] = v[i];
+	}
+}
+
+template<typename T, int V>
+__device__ __forceinline__ void chain_store(T* p, const T (&src)[V]) {
+	if constexpr (V == 1) {
+		*p = src[0];
+	} else {
+		typedef T vt __attribute__((ext_vector_type(V)));
+		vt v;
+		#pragma unroll
+		for (int i = 0; i < V; ++i)
+			v[i] = src[i];
+		*reinterpret_cast<vt*>(p) = v;
+	}
+}
+
+/* dz of a kernel layer followed by an activation and, with POOL, max pooling, from what the fused forward pass kept:
+ * the (coded) output `y` or, for activations whose derivative needs it, the pre-activation values `pre` (at the
+ * arg-max positions when pooled), and the arg-max cache. One thread per window and V samples:
+ * dz(position) = g * act'(.) at the arg-max position, 0 elsewhere (MaxPoolLayer.hpp:66-80 followed by the
+ * activation's pass_back). */
+template<typename T, int V, bool POOL>
+__global__ __launch_bounds__(256)
+void chain_backward_kernel(ChainShape s, int N, size_t total, const T* __restrict__ g, const unsigned* __restrict__ inds,
+		const T* __restrict__ y, const T* __restrict__ pre, T* __restrict__ dz) {
+	const size_t i = ((size_t) blockIdx.x * 256 + threadIdx.x) * V;
+	if (i >= total)
+		return;
+	const int OHp = s.H / s.prh, OWp = s.W / s.prw;
+	const int n = (int) (i % (size_t) N);
+	size_t t = i / (size_t) N;
+	const int a_p = (int) (t % (size_t) OHp);
+	t /= (size_t) OHp;
+	const int b_p = (int) (t % (size_t) OWp), c = (int) (t / (size_t) OWp);
+	T gv[V], yv[V], gb[V];
+	unsigned iv[V];
+	chain_load<T, V>(gv, g + i);
+	if (pre)
+		chain_load<T, V>(yv, pre + i);
+	else
+		chain_load<T, V>(yv, y + i);
+	act_dispatch(s.kind, [&](auto kc) {
+		constexpr int KIND = decltype(kc)::value;
+		#pragma unroll
+		for (int v = 0; v < V; ++v)
+			gb[v] = pre ? act_b<T, KIND>(yv[v], act_needs_y(KIND) ? act_f<T, KIND>(yv[v], (T) s.p) : (T) 0, gv[v], (T) s.p) :
+					act_b_coded<T, KIND>(yv[v], gv[v], (T) s.p);
+	});
+	if constexpr (!POOL) {
+		chain_store<T, V>(dz + i, gb);
+	} else {
+		chain_load<unsigned, V>(iv, inds + (((size_t) b_p * OHp + a_p) * ((size_t) s.C * N) + (size_t) c * N + n));
+		T* base = dz + n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw + (size_t) s.W * c));
+		for (int k = 0; k < s.prw; ++k)
+			for (int l = 0; l < s.prh; ++l) {
+				T o[V];
+				#pragma unroll
+				for (int v = 0; v < V; ++v)
+					o[v] = iv[v] == (unsigned) (k * s.prh + l) ? gb[v] : (T) 0;
+				chain_store<T, V>(base + (size_t) N * (l + (size_t) s.H * k), o);
+			}
+	}
+}
+
+/* Per-channel moments of z from the per-tile moments the GEMM epilogue wrote (stats [mtiles][C][3]: count, mean,
+ * sum of squared deviations): thread t merges tiles t, t + 256, ... in ascending order, then a fixed tree. */
+template<typename T>
+__device__ __forceinline__ void merge_tile_moments(const T* __restrict__ stats, int mtiles, int C, int c, T (*lds)[256], T& mean,
+		T& m2) {
+	const int tid = threadIdx.x;
+	T n = (T) 0;
+	mean = (T) 0;
+	m2 = (T) 0;
+	for (int tile = tid; tile < mtiles; tile += 256) {
+		const T* e = stats + ((size_t) tile * C + c) * 3;
+		moments_merge(n, mean, m2, e[0], e[1], e[2]);
+	}
+	lds[0][tid] = n;
+	lds[1][tid] = mean;
+	lds[2][tid] = m2;
+	__syncthreads();
+	for (int off = 128; off > 0; off >>= 1) {
+		if (tid < off) {
+			T a_n = lds[0][tid], a_mean = lds[1][tid], a_m2 = lds[2][tid];
+			moments_merge(a_n, a_mean, a_m2, lds[0][tid + off], lds[1][tid + off], lds[2][tid + off]);
+			lds[0][tid] = a_n;
+			lds[1][tid] = a_mean;
+			lds[2][tid] = a_m2;
+		}
+		__syncthreads();
+	}
+	mean = lds[1][0];
+	m2 = lds[2][0];
+}
+
+struct ChainBn {
+	int mtiles;             /* rows of the per-tile moments (training) */
+	int training, stats_init;
+};
+
+/* Forward pass behind the kernel layer with batch norm: channel moments (training: merged from the tiles' moments;
+ * inference: the running statistics), then y = act(gamma * (z - mean) * inv_sd + beta), pooled when POOL. The
+ * backward pass recomputes what it needs from z, so only mean and inverse standard deviation are kept per channel
+ * (BatchNormLayer.hpp:225-249 followed by the activation's and the pool's pass_forward). grid = (C, splits). */
+template<typename T, int V, int POOL>
+__global__ __launch_bounds__(256)
+void bn_chain_forward_kernel(ChainShape s, int N, size_t span, ChainBn bn, const T* __restrict__ z, const T* __restrict__ stats,
+		const T* __restrict__ gamma, const T* __restrict__ beta, T* __restrict__ avg_mean, T* __restrict__ avg_inv_sd, T decay, T eps,
+		T* __restrict__ mean_cache, T* __restrict__ inv_sd_cache, T* __restrict__ out, unsigned* __restrict__ inds) {
+	__shared__ T lds[3][256];
+	const int c = blockIdx.x;
+	const int OHp = s.H / s.prh, OWp = s.W / s.prw;
+	const size_t L = (size_t) N * s.H * s.W, Lp = (size_t) N * OHp * OWp;
+	T mean, inv_sd;
+	if (bn.training) {
+		T m2;
+		merge_tile_moments<T>(stats, bn.mtiles, s.C, c, lds, mean, m2);
+		inv_sd = (T) 1 / dev_sqrt(m2 / (T) L + eps);
+		if (blockIdx.y == 0 && threadIdx.x == 0) {
+			mean_cache[c] = mean;
+			inv_sd_cache[c] = inv_sd;
+			if (bn.stats_init) {       /* running average (BatchNormLayer.hpp:234-238) */
+				avg_mean[c] = ((T) 1 - decay) * avg_mean[c] + decay * mean;
+				avg_inv_sd[c] = ((T) 1 - decay) * avg_inv_sd[c] + decay * inv_sd;
+			} else {                   /* first call assigns (:239-243) */
+				avg_mean[c] = mean;
+				avg_inv_sd[c] = inv_sd;
+			}
+		}
+	} else {
+		mean = avg_mean[c];
+		inv_sd = avg_inv_sd[c];
+	}
+	const T ga = gamma[c], be = beta[c];
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < Lp ? begin + span : Lp;
+	const T* zc = z + (size_t) c * L;
+	T* oc = out + (size_t) c * Lp;
+	act_dispatch(s.kind, [&](auto kc) {
+		constexpr int KIND = decltype(kc)::value;
+		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
+			const int n = (int) (i % (size_t) N);
+			const size_t t = i / (size_t) N;
+			const int a_p = (int) (t % (size_t) OHp), b_p = (int) (t / (size_t) OHp);
+			const T* base = zc + n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw));
+			T res[V];
+			unsigned bi[V];
+			#pragma unroll
+			for (int v = 0; v < V; ++v) {
+				res[v] = POOL == CHAIN_POOL_MAX ? std::numeric_limits<T>::lowest() : (T) 0;
+				bi[v] = 0;
+			}
+			for (int k = 0; k < s.prw; ++k)
+				for (int l = 0; l < s.prh; ++l) {
+					T zv[V];
+					chain_load<T, V>(zv, base + (size_t) N * (l + (size_t) s.H * k));
+					#pragma unroll
+					for (int v = 0; v < V; ++v) {
+						const T yv = act_f<T, KIND>(((zv[v] - mean) * inv_sd) * ga + be, (T) s.p);
+						if (POOL == CHAIN_POOL_MAX) {
+							if (yv > res[v]) {
+								res[v] = yv;
+								bi[v] = (unsigned) (k * s.prh + l);
+							}
+						} else {
+							res[v] += yv;
+						}
+					}
+				}
+			if (POOL == CHAIN_POOL_MEAN) {
+				#pragma unroll
+				for (int v = 0; v < V; ++v)
+					res[v] = res[v] / (T) (s.prh * s.prw);
+			}
+			chain_store<T, V>(oc + i, res);
+			if (POOL == CHAIN_POOL_MAX)
+				chain_store<unsigned, V>(inds + (((size_t) b_p * OHp + a_p) * ((size_t) s.C * N) + (size_t) c * N + n), bi);
+		}
+	});
+}
+
+/* The gradient that reaches the batch norm's output at the window positions of one pooled element, and the
+ * normalised inputs there: g_bn = pool'(g) * act'(y_bn), recomputed from z. Calls fn(k, l, z, std, g_bn) per position
+ * (max pooling: the arg-max position only when ONLY_NONZERO). */
+template<typename T, int V, int POOL, int KIND, bool ONLY_NONZERO, typename Fn>
+__device__ __forceinline__ void chain_bn_window(const ChainShape& s, int N, const T* base, const T (&gv)[V], const unsigned (&iv)[V],
+		T mean, T inv_sd, T ga, T be, Fn fn) {
+	const T area = (T) (s.prh * s.prw);
+	if constexpr (POOL == CHAIN_POOL_MAX && ONLY_NONZERO) {
+		#pragma unroll
+		for (int v = 0; v < V; ++v) {
+			const int k = (int) iv[v] / s.prh, l = (int) iv[v] - k * s.prh;
+			const T zv = base[v + (size_t) N * (l + (size_t) s.H * k)];
+			const T sd = (zv - mean) * inv_sd, yb = sd * ga + be;
+			const T gb = act_b<T, KIND>(yb, act_needs_y(KIND) ? act_f<T, KIND>(yb, (T) s.p) : (T) 0, gv[v], (T) s.p);
+			fn(v, sd, gb);
+		}
+	} else
+	for (int k = 0; k < s.prw; ++k)
+		for (int l = 0; l < s.prh; ++l) {
+			T zv[V];
+			chain_load<T, V>(zv, base + (size_t) N * (l + (size_t) s.H * k));
+			#pragma unroll
+			for (int v = 0; v < V; ++v) {
+				const T sd = (zv[v] - mean) * inv_sd, yb = sd * ga + be;
+				T up = gv[v];
+				if (POOL == CHAIN_POOL_MEAN)
+					up = up / area;
+				T gb = act_b<T, KIND>(yb, act_needs_y(KIND) ? act_f<T, KIND>(yb, (T) s.p) : (T) 0, up, (T) s.p);
+				if (POOL == CHAIN_POOL_MAX && iv[v] != (unsigned) (k * s.prh + l))
+					gb = (T) 0;
+				fn(v, k, l, sd, gb);
+			}
+		}
+}
+
+/* Sums over a channel of g_bn and of g_bn * std (BatchNormLayer.hpp:252-254), per split. grid = (C, splits). */
+template<typename T, int V, int POOL>
+__global__ __launch_bounds__(256)
+void bn_chain_sums_kernel(ChainShape s, int N, size_t span, const T* __restrict__ g, const unsigned* __restrict__ inds,
+		const T* __restrict__ z, const T* __restrict__ gamma, const T* __restrict__ beta, const T* __restrict__ mean_cache,
+		const T* __restrict__ inv_sd_cache, T* __restrict__ ws_g, T* __restrict__ ws_gs) {
+	__shared__ T lds[4];
+	const int c = blockIdx.x;
+	const int OHp = s.H / s.prh, OWp = s.W / s.prw;
+	const size_t L = (size_t) N * s.H * s.W, Lp = (size_t) N * OHp * OWp;
+	const T mean = mean_cache[c], inv_sd = inv_sd_cache[c], ga = gamma[c], be = beta[c];
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < Lp ? begin + span : Lp;
+	const T* zc = z + (size_t) c * L;
+	const T* gc = g + (size_t) c * Lp;
+	T s1 = (T) 0, s2 = (T) 0;
+	act_dispatch(s.kind, [&](auto kc) {
+		constexpr int KIND = decltype(kc)::value;
+		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
+			const int n = (int) (i % (size_t) N);
+			const size_t t = i / (size_t) N;
+			const int a_p = (int) (t % (size_t) OHp), b_p = (int) (t / (size_t) OHp);
+			const T* base = zc + n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw));
+			T gv[V];
+			unsigned iv[V];
+			chain_load<T, V>(gv, gc + i);
+			if (POOL == CHAIN_POOL_MAX)
+				chain_load<unsigned, V>(iv, inds + (((size_t) b_p * OHp + a_p) * ((size_t) s.C * N) + (size_t) c * N + n));
+			if constexpr (POOL == CHAIN_POOL_MAX)
+				chain_bn_window<T, V, POOL, KIND, true>(s, N, base, gv, iv, mean, inv_sd, ga, be, [&](int, T sd, T gb) {
+					s1 += gb;
+					s2 += gb * sd;
+				});
+			else
+				chain_bn_window<T, V, POOL, KIND, false>(s, N, base, gv, iv, mean, inv_sd, ga, be, [&](int, int, int, T sd, T gb) {
+					s1 += gb;
+					s2 += gb * sd;
+				});
+		}
+	});
+	s1 = block_sum_256(s1, lds);
+	s2 = block_sum_256(s2, lds);
+	if (threadIdx.x == 0) {
+		ws_g[(size_t) c * gridDim.y + blockIdx.y] = s1;
+		ws_gs[(size_t) c * gridDim.y + blockIdx.y] = s2;
+	}
+}
+
+/* dz = (L * g_bn * gamma - sum(g_bn * gamma) - std * sum(std * g_bn * gamma)) * inv_sd / L at every position
+ * (BatchNormLayer.hpp:257-261), gamma and beta gradients accumulated by the first split's first thread. */
+template<typename T, int V, int POOL>
+__global__ __launch_bounds__(256)
+void bn_chain_apply_kernel(ChainShape s, int N, size_t span, const T* __restrict__ g, const unsigned* __restrict__ inds,
+		const T* __restrict__ z, const T* __restrict__ gamma, const T* __restrict__ beta, const T* __restrict__ mean_cache,
+		const T* __restrict__ inv_sd_cache, const T* __restrict__ ws_g, const T* __restrict__ ws_gs, T* __restrict__ gamma_grad,
+		T* __restrict__ beta_grad, T* __restrict__ dz) {
+	const int c = blockIdx.x, splits = gridDim.y;
+	const int OHp = s.H / s.prh, OWp = s.W / s.prw;
+	const size_t L = (size_t) N * s.H * s.W, Lp = (size_t) N * OHp * OWp;
+	const T sum_g = sum_partials(ws_g + (size_t) c * splits, splits);
+	const T sum_gs = sum_partials(ws_gs + (size_t) c * splits, splits);
+	if (blockIdx.y == 0 && threadIdx.x == 0) {
+		gamma_grad[c] += sum_gs;
+		beta_grad[c] += sum_g;
+	}
+	const T mean = mean_cache[c], inv_sd = inv_sd_cache[c], ga = gamma[c], be = beta[c];
+	const T sum_sg = sum_g * ga, sum_ssg = sum_gs * ga, scale = ((T) 1 / (T) L) * inv_sd;
+	const size_t begin = (size_t) blockIdx.y * span, end = begin + span < Lp ? begin + span : Lp;
+	const T* zc = z + (size_t) c * L;
+	const T* gc = g + (size_t) c * Lp;
+	T* dc = dz + (size_t) c * L;
+	act_dispatch(s.kind, [&](auto kc) {
+		constexpr int KIND = decltype(kc)::value;
+		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
+			const int n = (int) (i % (size_t) N);
+			const size_t t = i / (size_t) N;
+			const int a_p = (int) (t % (size_t) OHp), b_p = (int) (t / (size_t) OHp);
+			const size_t off = n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw));
+			T gv[V];
+			unsigned iv[V];
+			chain_load<T, V>(gv, gc + i);
+			if (POOL == CHAIN_POOL_MAX)
+				chain_load<unsigned, V>(iv, inds + (((size_t) b_p * OHp + a_p) * ((size_t) s.C * N) + (size_t) c * N + n));
+			T o[V];
+			chain_bn_window<T, V, POOL, KIND, false>(s, N, zc + off, gv, iv, mean, inv_sd, ga, be, [&](int v, int k, int l, T sd, T gb) {
+				o[v] = (((T) L * (gb * ga) - sum_sg) - sd * sum_ssg) * scale;
+				if (v == V - 1)
+					chain_store<T, V>(dc + off + (size_t) N * (l + (size_t) s.H * k), o);
+			});
+		}
+	});
+}
+
+unsigned chain_grid(size_t items) {
+	const size_t blocks = (items + 255) / 256;
+	CATTLE_HIP_REQUIRE(blocks < 2147483647u, "launch exceeds the grid limit");
+	return (unsigned) std::max<size_t>(1, blocks);
+}
+
+template<typename T>
+bool chain_vectors(int N, std::initializer_list<const void*> ptrs) {
+	if (N % Pack<T>::V != 0)
+		return false;
+	for (const void* p : ptrs)
+		if (p && !aligned16(p))
+			return false;
+	return true;
+}
+
+} /* namespace */
+
+template<typename T>
+void chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* y, const T* pre, T* dz) {
+	CATTLE_HIP_REQUIRE(s.pool != CHAIN_POOL_MEAN, "mean pooling needs the values at every position: not kept by the fused pass");
+	const size_t total = (size_t) N * (s.H / s.prh) * (s.W / s.prw) * s.C;
+	constexpr int V = Pack<T>::V;
+	const bool vec = chain_vectors<T>(N, { g, inds, y, pre, dz });
+	if (s.pool == CHAIN_POOL_MAX) {
+		if (vec)
+			chain_backward_kernel<T, V, true><<<chain_grid(total / V), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+		else
+			chain_backward_kernel<T, 1, true><<<chain_grid(total), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+	} else {
+		if (vec)
+			chain_backward_kernel<T, V, false><<<chain_grid(total / V), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+		else
+			chain_backward_kernel<T, 1, false><<<chain_grid(total), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+	}
+	check_launch();
+}
+
+size_t bn_chain_workspace(int channels) {
+	return (size_t) 2 * channels * BN_MAX_SPLITS;
+}
+
+template<typename T, int V, int POOL>
+void bn_chain_forward_launch(const ChainShape& s, int N, int mtiles, bool training, bool stats_init, const T* z, const T* stats,
+		const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd, T decay, T eps, T* mean_cache, T* inv_sd_cache, T* out,
+		unsigned* inds) {
+	const size_t Lp = (size_t) N * (s.H / s.prh) * (s.W / s.prw);
+	const int splits = bn_splits(s.C, Lp);
+	const ChainBn bn = { mtiles, training ? 1 : 0, stats_init ? 1 : 0 };
+	bn_chain_forward_kernel<T, V, POOL><<<dim3((unsigned) s.C, (unsigned) splits), 256, 0, stream()>>>(s, N, bn_span(Lp, splits), bn, z,
+			stats, gamma, beta, avg_mean, avg_inv_sd, decay, eps, mean_cache, inv_sd_cache, out, inds);
+	check_launch();
+}
+
+template<typename T>
+void bn_chain_forward(const ChainShape& s, int N, int mtiles, bool training, bool stats_init, const T* z, const T* stats,
+		const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd, T decay, T eps, T* mean_cache, T* inv_sd_cache, T* out,
+		unsigned* inds) {
+	constexpr int V = Pack<T>::V;
+	const bool vec = chain_vectors<T>(N, { z, out, inds });
+	#define CATTLE_HIP_CHAIN_FWD(VV, PP) bn_chain_forward_launch<T, VV, PP>(s, N, mtiles, training, stats_init, z, stats, gamma, beta, \
+			avg_mean, avg_inv_sd, decay, eps, mean_cache, inv_sd_cache, out, inds)
+	if (s.pool == CHAIN_POOL_MAX) {
+		if (vec) CATTLE_HIP_CHAIN_FWD(V, CHAIN_POOL_MAX); else CATTLE_HIP_CHAIN_FWD(1, CHAIN_POOL_MAX);
+	} else if (s.pool == CHAIN_POOL_MEAN) {
+		if (vec) CATTLE_HIP_CHAIN_FWD(V, CHAIN_POOL_MEAN); else CATTLE_HIP_CHAIN_FWD(1, CHAIN_POOL_MEAN);
+	} else {
+		if (vec) CATTLE_HIP_CHAIN_FWD(V, CHAIN_POOL_NONE); else CATTLE_HIP_CHAIN_FWD(1, CHAIN_POOL_NONE);
+	}
+	#undef CATTLE_HIP_CHAIN_FWD
+}
+
+template<typename T, int V, int POOL>
+void bn_chain_backward_launch(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* z, const T* gamma, const T* beta,
+		const T* mean_cache, const T* inv_sd_cache, T* gamma_grad, T* beta_grad, T* dz, T* ws) {
+	const size_t Lp = (size_t) N * (s.H / s.prh) * (s.W / s.prw);
+	const int splits = bn_splits(s.C, Lp);
+	const size_t span = bn_span(Lp, splits);
+	const dim3 grid((unsigned) s.C, (unsigned) splits);
+	T* ws_g = ws;
+	T* ws_gs = ws + (size_t) s.C * BN_MAX_SPLITS;
+	bn_chain_sums_kernel<T, V, POOL><<<grid, 256, 0, stream()>>>(s, N, span, g, inds, z, gamma, beta, mean_cache, inv_sd_cache, ws_g, ws_gs);
+	check_launch();
+	bn_chain_apply_kernel<T, V, POOL><<<grid, 256, 0, stream()>>>(s, N, span, g, inds, z, gamma, beta, mean_cache, inv_sd_cache, ws_g, ws_gs,
+			gamma_grad, beta_grad, dz);
+	check_launch();
+}
+
+template<typename T>
+void bn_chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* z, const T* gamma, const T* beta,
+		const T* mean_cache, const T* inv_sd_cache, T* gamma_grad, T* beta_grad, T* dz, T* ws) {
+	constexpr int V = Pack<T>::V;
+	const bool vec = chain_vectors<T>(N, { g, inds, z, dz });
+	#define CATTLE_HIP_CHAIN_BWD(VV, PP) bn_chain_backward_launch<T, VV, PP>(s, N, g, inds, z, gamma, beta, mean_cache, inv_sd_cache, \
+			gamma_grad, beta_grad, dz, ws)
+	if (s.pool == CHAIN_POOL_MAX) {
+		if (vec) CATTLE_HIP_CHAIN_BWD(V, CHAIN_POOL_MAX); else CATTLE_HIP_CHAIN_BWD(1, CHAIN_POOL_MAX);
+	} else if (s.pool == CHAIN_POOL_MEAN) {
+		if (vec) CATTLE_HIP_CHAIN_BWD(V, CHAIN_POOL_MEAN); else CATTLE_HIP_CHAIN_BWD(1, CHAIN_POOL_MEAN);
+	} else {
+		if (vec) CATTLE_HIP_CHAIN_BWD(V, CHAIN_POOL_NONE); else CATTLE_HIP_CHAIN_BWD(1, CHAIN_POOL_NONE);
+	}
+	#undef CATTLE_HIP_CHAIN_BWD
+}
+
 #define CATTLE_HIP_INSTANTIATE(T) \
 template void act_forward<T>(int, size_t, T, const T*, T*); \
+template void chain_backward<T>(const ChainShape&, int, const T*, const unsigned*, const T*, const T*, T*); \
+template void bn_chain_forward<T>(const ChainShape&, int, int, bool, bool, const T*, const T*, const T*, const T*, T*, T*, T, T, T*, T*, T*, unsigned*); \
+template void bn_chain_backward<T>(const ChainShape&, int, const T*, const unsigned*, const T*, const T*, const T*, const T*, const T*, T*, T*, T*, T*); \
 template void act_backward<T>(int, size_t, T, const T*, const T*, const T*, T*); \
 template void softmax_forward<T>(int, int, T, const T*, T*); \
 template void softmax_backward<T>(int, int, const T*, const T*, T*); \

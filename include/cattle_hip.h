@@ -161,6 +161,26 @@ int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t 
 		size_t receptor_height, size_t receptor_width, size_t vertical_stride, size_t horizontal_stride,
 		cattle_hip_layer_t* layer);
 
+/* A kernel layer and the layers that a feed-forward network calls right after it, run as one layer. The reference
+ * calls them one after another (neural_network/FeedforwardNeuralNetwork.hpp:112-127 forwards, :129-141 backwards: the
+ * shape of test/gradient_test.cpp:585-592 and examples/cifar_convnet.cpp:24-41 is conv -> ReLU -> max pool); here
+ * `layers` = { convolutional or dense layer [, batch norm] [, activation] [, pool] }, existing handles in call order, become
+ * one handle whose pass_forward / pass_back (cattle_hip_layer_forward / _backward) equal those calls in sequence:
+ * the activation (ActivationLayer.hpp:47-66 and the element-wise kinds above) is applied in the epilogue of the GEMM, max
+ * pooling over windows that tile the output (MaxPoolLayer.hpp:38-80; stride = receptor) too, so that the full-size
+ * activation tensor is never written, and the per-channel batch norm (BatchNormLayer.hpp:225-261) gets its moments from
+ * the GEMM's epilogue. The members keep their parameters (the fused handle lists them all, members' order, same objects),
+ * the batch norm its running statistics, the max pool its arg-max cache (cattle_hip_maxpool_indices on the member).
+ * Whatever cannot be fused (batch sizes without 16-byte rows, overlapping windows, softmax, PReLU, PSwish, per-activation
+ * batch norm behind a convolution) runs as the members' own passes, still on the device. Rectifier outputs (ReLU,
+ * LeakyReLU, ELU) carry the side of their input in the sign bit: -0 where a negative input was mapped to zero.
+ * The members are borrowed: they must outlive the fused handle, and must not be called on their own between a fused
+ * forward pass and its backward pass. A clone (cattle_hip_layer_clone) owns clones of the members. */
+int cattle_hip_fused_create(const cattle_hip_layer_t* layers, size_t count, cattle_hip_layer_t* fused);
+/* How the last forward pass of a fused handle ran: 0 none yet, 1 member by member, 2 activation in the GEMM epilogue,
+ * 3 activation and max pooling in the GEMM epilogue, 4 batch-norm moments from the GEMM epilogue + one chain pass. */
+int cattle_hip_fused_last_mode(cattle_hip_layer_t fused, int* mode);
+
 /* DropoutLayer<Scalar,Rank>(dims, dropout_prob, epsilon) - layer/DropoutLayer.hpp:33-42, passes :74-96: a training
  * pass multiplies by the inverted-dropout mask (0 where u <= dropout_prob, else 1 / (1 - dropout_prob + epsilon)), an
  * inference pass hands the input through, the backward pass multiplies the gradient by the mask of the last training
