@@ -770,3 +770,25 @@ class FusedKernelLayer(Layer):
     def __del__(self):
         Layer.__del__(self)             # the fused handle goes before its members
         self.members = None
+
+
+def fuse_layers(layers):
+    """The layer list of a feed-forward network with every convolutional or dense layer and the batch norm, activation
+    and pool layers right behind it (in this order, each optional) replaced by one FusedKernelLayer over them; the other
+    layers stay as they are. Calling the result in order equals calling `layers` in order."""
+    out, i = [], 0
+    while i < len(layers):
+        group = [layers[i]]
+        if isinstance(layers[i], (ConvKernelLayer, DenseKernelLayer)):
+            for cls in (BatchNormLayer, ActivationLayer, _PoolLayer):
+                j = i + len(group)
+                if j < len(layers) and isinstance(layers[j], cls) and layers[j].dtype == layers[i].dtype:
+                    group.append(layers[j])
+        if len(group) > 1:
+            fused = FusedKernelLayer(group)
+            fused.set_input_layer(group[0].is_input_layer())
+            out.append(fused)
+        else:
+            out.append(layers[i])
+        i += len(group)
+    return out

@@ -86,7 +86,7 @@ int main(int argc, char** argv) {
 		check(cattle_hip_init(0));
 		DeviceLoss<Scalar> loss(CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY);
 		Lcg g(2);
-		double mlp_ms, conv_ms, cifar_ms;
+		double mlp_ms, conv_ms, cifar_ms, mlp_fused_ms, conv_fused_ms, cifar_fused_ms;
 		{
 			/* MLP 784-512-256-10 with ReLU, batch 256, vanilla SGD */
 			const std::size_t batch = 256;
@@ -101,6 +101,9 @@ int main(int argc, char** argv) {
 			std::vector<Scalar> x = random_values(batch * 784, g, 1.0), y = one_hot(batch, 10, g);
 			DT xd(DT::Dims{ { batch, 784, 1, 1 } }, x.data()), yd(DT::Dims{ { batch, 10, 1, 1 } }, y.data());
 			mlp_ms = time_steps(steps, warmup, [&](std::size_t) { net.train_batch_sgd(xd, yd, loss, (Scalar) 1e-3); });
+			/* the same network with each dense layer and its ReLU run as one fused layer */
+			net.fuse();
+			mlp_fused_ms = time_steps(steps, warmup, [&](std::size_t) { net.train_batch_sgd(xd, yd, loss, (Scalar) 1e-3); });
 		}
 		{
 			/* conv 3x3x32 - ReLU - max pool - conv 3x3x64 - batch norm - ReLU - max pool - dense 10, batch 128, Adam */
@@ -119,6 +122,9 @@ int main(int argc, char** argv) {
 			std::vector<Scalar> x = random_values(batch * 32 * 32 * 3, g, 1.0), y = one_hot(batch, 10, g);
 			DT xd(DT::Dims{ { batch, 32, 32, 3 } }, x.data()), yd(DT::Dims{ { batch, 10, 1, 1 } }, y.data());
 			conv_ms = time_steps(steps, warmup, [&](std::size_t t) { net.train_batch_adam(xd, yd, loss, t); });
+			/* conv-ReLU-pool and conv-BN-ReLU-pool as fused layers */
+			net.fuse();
+			conv_fused_ms = time_steps(steps, warmup, [&](std::size_t t) { net.train_batch_adam(xd, yd, loss, steps + warmup + t); });
 		}
 		{
 			/* examples/cifar_convnet.cpp:24-41: conv 3x3x8 - ReLU - max pool - conv 3x3x8 - ReLU - max pool - dropout .25 -
@@ -155,10 +161,16 @@ int main(int argc, char** argv) {
 			cifar_ms = time_steps(steps, warmup, [&](std::size_t t) {
 				net.train_batch(xd, yd, cross_entropy, CATTLE_HIP_OPT_NADAM, nadam, 0, t);
 			});
+			net.fuse();
+			cifar_fused_ms = time_steps(steps, warmup, [&](std::size_t t) {
+				net.train_batch(xd, yd, cross_entropy, CATTLE_HIP_OPT_NADAM, nadam, 0, steps + warmup + t);
+			});
 		}
 		std::printf("{\"driver\": \"C++ (cattle_hip/DeviceNet.hpp), train_batch* incl. the per-batch loss read-back\", "
 				"\"steps\": %zu, \"warmup\": %zu, \"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, \"convnet_32x32x3_batch128_adam_ms\": %.4f, "
-				"\"reference_cifar_example_batch200_nadam_ms\": %.4f}\n", steps, warmup, mlp_ms, conv_ms, cifar_ms);
+				"\"reference_cifar_example_batch200_nadam_ms\": %.4f, \"fused\": {\"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, "
+				"\"convnet_32x32x3_batch128_adam_ms\": %.4f, \"reference_cifar_example_batch200_nadam_ms\": %.4f}}\n", steps, warmup, mlp_ms,
+				conv_ms, cifar_ms, mlp_fused_ms, conv_fused_ms, cifar_fused_ms);
 	} catch (const std::exception& e) {
 		std::fprintf(stderr, "train_steps: %s\n", e.what());
 		return 1;

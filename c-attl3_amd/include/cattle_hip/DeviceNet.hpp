@@ -297,6 +297,26 @@ public:
 		check(cattle_hip_broadcast_create(Code<Scalar>::value, input_dims.data(), broadcast.data(), &h));
 		return DeviceLayer(h);
 	}
+	/**
+	 * A kernel layer and the batch norm / activation / pool layers a network calls right after it as one layer
+	 * (cattle_hip_fused_create): `members` = { convolutional or dense layer [, batch norm] [, activation] [, pool] } in
+	 * call order. The members are borrowed (their parameters, running statistics and caches stay theirs) and must
+	 * outlive the result. Returns a layer without a handle (is_null()) if these layers cannot form a fused layer.
+	 */
+	inline static DeviceLayer fused(const DeviceLayer* const* members, std::size_t count) {
+		cattle_hip_layer_t handles[4] = { nullptr, nullptr, nullptr, nullptr };
+		cattle_hip_layer_t h = nullptr;
+		if (count < 2 || count > 4)
+			return DeviceLayer(nullptr, Dims(), Dims());
+		for (std::size_t i = 0; i < count; ++i)
+			handles[i] = members[i]->handle;
+		if (cattle_hip_fused_create(handles, count, &h) != CATTLE_HIP_OK)
+			return DeviceLayer(nullptr, Dims(), Dims());
+		return DeviceLayer(h, members[0]->in_dims, members[count - 1]->out_dims);
+	}
+	inline bool is_null() const {
+		return handle == nullptr;
+	}
 	inline DeviceLayer(DeviceLayer&& other) : handle(other.handle), in_dims(other.in_dims), out_dims(other.out_dims),
 			cached_in(std::move(other.cached_in)), cached_out(std::move(other.cached_out)),
 			params_per_column(other.params_per_column), kernel_layer(other.kernel_layer) {
@@ -616,9 +636,42 @@ public:
 			frozen(false) {
 		assert(!this->layers.empty());
 		this->layers[0].set_input_layer(foremost);
+		for (std::size_t i = 0; i < this->layers.size(); ++i)
+			units.push_back(Unit{ i, 1, NO_FUSED });
 	}
 	inline std::vector<DeviceLayer<Scalar>>& get_layers() {
 		return layers;
+	}
+	/**
+	 * From now on every kernel layer and the batch norm, element-wise activation and pool layers right behind it run as one
+	 * fused layer (DeviceLayer::fused): the same calls as FeedforwardNeuralNetwork.hpp:112-141 makes, with the activation,
+	 * the max pooling and the batch-norm moments computed in the epilogue of the layer's GEMM. get_layers(), the
+	 * parameters and everything that works on them are unaffected. Returns the number of fused groups.
+	 */
+	inline std::size_t fuse() {
+		units.clear();
+		fused_layers.clear();
+		std::size_t i = 0;
+		while (i < layers.size()) {
+			std::size_t len = 1;
+			if (layers[i].is_kernel_layer()) {
+				for (len = layers.size() - i < 4 ? layers.size() - i : 4; len > 1; --len) {
+					const DeviceLayer<Scalar>* members[4];
+					for (std::size_t k = 0; k < len; ++k)
+						members[k] = &layers[i + k];
+					DeviceLayer<Scalar> f = DeviceLayer<Scalar>::fused(members, len);
+					if (!f.is_null()) {
+						fused_layers.push_back(std::move(f));
+						break;
+					}
+				}
+			}
+			units.push_back(Unit{ i, len, len > 1 ? fused_layers.size() - 1 : NO_FUSED });
+			i += len;
+		}
+		if (units[0].fused != NO_FUSED)
+			fused_layers[units[0].fused].set_input_layer(foremost);
+		return fused_layers.size();
 	}
 	inline const typename DeviceLayer<Scalar>::Dims& get_input_dims() const {
 		return layers.front().get_input_dims();
@@ -632,6 +685,8 @@ public:
 	}
 	inline void set_foremost(bool foremost) {
 		layers[0].set_input_layer(foremost);
+		if (units[0].fused != NO_FUSED)
+			fused_layers[units[0].fused].set_input_layer(foremost);
 		this->foremost = foremost;
 	}
 	/**
@@ -728,16 +783,16 @@ public:
 	}
 	/** propagate: `input` must stay alive and unmodified until backpropagate returns. */
 	inline const DeviceTensor<Scalar>& propagate(const DeviceTensor<Scalar>& input, bool training) {
-		const DeviceTensor<Scalar>* cur = &layers[0].pass_forward_borrowed(input, training);
-		for (std::size_t i = 1; i < layers.size(); ++i)
-			cur = &layers[i].pass_forward_borrowed(*cur, training);      /* the producer keeps its output alive */
+		const DeviceTensor<Scalar>* cur = &unit(0).pass_forward_borrowed(input, training);
+		for (std::size_t i = 1; i < units.size(); ++i)
+			cur = &unit(i).pass_forward_borrowed(*cur, training);        /* the producer keeps its output alive */
 		return *cur;
 	}
 	inline DeviceTensor<Scalar> backpropagate(const DeviceTensor<Scalar>& out_grad) {
 		DeviceTensor<Scalar> grad;
-		for (std::size_t i = layers.size(); i-- > 0;) {
+		for (std::size_t i = units.size(); i-- > 0;) {
 			const bool needs = !(i == 0 && foremost);
-			grad = layers[i].pass_back(i + 1 == layers.size() ? out_grad : grad, needs);
+			grad = unit(i).pass_back(i + 1 == units.size() ? out_grad : grad, needs);
 		}
 		return grad;
 	}
@@ -795,9 +850,22 @@ private:
 		backpropagate(loss.d_function(out, obj, (Scalar) 1 / (Scalar) input.batch()));
 		return total;
 	}
+	/* what propagate calls: one layer, or `count` layers from `first` on through the fused layer over them */
+	struct Unit {
+		std::size_t first, count, fused;
+	};
+	static constexpr std::size_t NO_FUSED = (std::size_t) -1;
+	inline DeviceLayer<Scalar>& unit(std::size_t i) {
+		return units[i].fused == NO_FUSED ? layers[units[i].first] : fused_layers[units[i].fused];
+	}
 	std::vector<DeviceLayer<Scalar>> layers;
+	std::vector<DeviceLayer<Scalar>> fused_layers;      /* declared after `layers`: destroyed before the members they borrow */
+	std::vector<Unit> units;
 	bool foremost, frozen;
 };
+
+template<typename Scalar>
+constexpr std::size_t DeviceFeedforwardNetwork<Scalar>::NO_FUSED;
 
 /**
  * Feed-forward networks on top of one another (neural_network/StackedNeuralNetwork.hpp:33-120 on device tensors): only

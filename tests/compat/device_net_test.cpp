@@ -107,7 +107,9 @@ static void run(const std::string& tag) {
 	typedef typename DL::Dims Dims;
 	const std::size_t steps = 3;
 	DeviceLoss<Scalar> loss(CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY);
-	{
+	/* each of the two trained networks once layer by layer and once with DeviceFeedforwardNetwork::fuse() (records "...f") */
+	for (int fused = 0; fused < 2; ++fused) {
+		const std::string mlp = tag + (fused ? ".mlpf" : ".mlp");
 		Lcg g(11);
 		const std::size_t batch = 24;
 		std::vector<DL> layers;
@@ -115,16 +117,20 @@ static void run(const std::string& tag) {
 		layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, layers.back().get_output_dims()));
 		layers.push_back(DL::dense(layers.back().get_output_dims(), 6));
 		DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
-		init_and_record<Scalar>(tag + ".mlp", net, g);
+		if (fused) {
+			const Scalar groups = (Scalar) net.fuse();
+			record(mlp + ".groups", sizeof(Scalar), { 1 }, &groups);
+		}
+		init_and_record<Scalar>(mlp, net, g);
 		std::vector<Scalar> x = random_values<Scalar>(batch * 20, g, 1.0), y = one_hot<Scalar>(batch, 6, g);
-		record(tag + ".mlp.x", sizeof(Scalar), { batch, 20 }, x.data());
-		record(tag + ".mlp.y", sizeof(Scalar), { batch, 6 }, y.data());
+		record(mlp + ".x", sizeof(Scalar), { batch, 20 }, x.data());
+		record(mlp + ".y", sizeof(Scalar), { batch, 6 }, y.data());
 		DT xd(typename DT::Dims{ { batch, 20, 1, 1 } }, x.data()), yd(typename DT::Dims{ { batch, 6, 1, 1 } }, y.data());
 		std::vector<Scalar> totals;
 		for (std::size_t t = 0; t < steps; ++t)
 			totals.push_back(net.train_batch_sgd(xd, yd, loss, (Scalar) 0.05));
-		record(tag + ".mlp.losses", sizeof(Scalar), { steps }, totals.data());
-		record_final<Scalar>(tag + ".mlp", net);
+		record(mlp + ".losses", sizeof(Scalar), { steps }, totals.data());
+		record_final<Scalar>(mlp, net);
 	}
 	{
 		/* the data-movement layers of the reference's example networks: reshape -> broadcast -> dropout */
@@ -279,7 +285,8 @@ static void run(const std::string& tag) {
 		record(tag + ".loss.values", sizeof(Scalar), { batch }, negated_hinge.function(od, yd).data());
 		record(tag + ".loss.grad", sizeof(Scalar), { batch, classes }, negated_hinge.d_function(od, yd, (Scalar) 0.5).to_host().data());
 	}
-	{
+	for (int fused = 0; fused < 2; ++fused) {
+		const std::string convnet = tag + (fused ? ".convnetf" : ".convnet");
 		Lcg g(12);
 		const std::size_t batch = 16;
 		std::vector<DL> layers;
@@ -289,21 +296,25 @@ static void run(const std::string& tag) {
 		layers.push_back(DL::batch_norm(layers.back().get_output_dims()));
 		layers.push_back(DL::dense(layers.back().get_output_dims(), 5));
 		DeviceFeedforwardNetwork<Scalar> net(std::move(layers));
-		init_and_record<Scalar>(tag + ".convnet", net, g);
+		if (fused) {
+			const Scalar groups = (Scalar) net.fuse();
+			record(convnet + ".groups", sizeof(Scalar), { 1 }, &groups);
+		}
+		init_and_record<Scalar>(convnet, net, g);
 		std::vector<Scalar> x = random_values<Scalar>(batch * 8 * 8 * 3, g, 1.0), y = one_hot<Scalar>(batch, 5, g);
-		record(tag + ".convnet.x", sizeof(Scalar), { batch, 8, 8, 3 }, x.data());
-		record(tag + ".convnet.y", sizeof(Scalar), { batch, 5 }, y.data());
+		record(convnet + ".x", sizeof(Scalar), { batch, 8, 8, 3 }, x.data());
+		record(convnet + ".y", sizeof(Scalar), { batch, 5 }, y.data());
 		DT xd(typename DT::Dims{ { batch, 8, 8, 3 } }, x.data()), yd(typename DT::Dims{ { batch, 5, 1, 1 } }, y.data());
 		std::vector<Scalar> totals;
 		for (std::size_t t = 0; t < steps; ++t)
 			totals.push_back(net.train_batch_adam(xd, yd, loss, t, (Scalar) 0.01));
-		record(tag + ".convnet.losses", sizeof(Scalar), { steps }, totals.data());
-		record_final<Scalar>(tag + ".convnet", net);
+		record(convnet + ".losses", sizeof(Scalar), { steps }, totals.data());
+		record_final<Scalar>(convnet, net);
 		/* inference after training uses the running statistics */
 		const DT& out = net.propagate(xd, false);
-		record(tag + ".convnet.infer", sizeof(Scalar), { batch, 5 }, out.to_host().data());
+		record(convnet + ".infer", sizeof(Scalar), { batch, 5 }, out.to_host().data());
 		/* the reference's parameter files: written, then read back by a fresh network, which must infer alike */
-		net.save_all_unique_params_values(g_dir, tag + "_params_");
+		net.save_all_unique_params_values(g_dir, tag + (fused ? "_fparams_" : "_params_"));
 		std::vector<DL> twin_layers;
 		twin_layers.push_back(DL::conv(Dims{ { 8, 8, 3 } }, 8));
 		twin_layers.push_back(DL::activation(CATTLE_HIP_ACT_RELU, twin_layers.back().get_output_dims()));
@@ -311,9 +322,9 @@ static void run(const std::string& tag) {
 		twin_layers.push_back(DL::batch_norm(twin_layers.back().get_output_dims()));
 		twin_layers.push_back(DL::dense(twin_layers.back().get_output_dims(), 5));
 		DeviceFeedforwardNetwork<Scalar> twin(std::move(twin_layers));
-		twin.load_all_unique_params_values(g_dir, tag + "_params_");
+		twin.load_all_unique_params_values(g_dir, tag + (fused ? "_fparams_" : "_params_"));
 		const DT& out2 = twin.propagate(xd, false);
-		record(tag + ".convnet.reloaded_infer", sizeof(Scalar), { batch, 5 }, out2.to_host().data());
+		record(convnet + ".reloaded_infer", sizeof(Scalar), { batch, 5 }, out2.to_host().data());
 	}
 }
 

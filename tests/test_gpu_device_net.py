@@ -120,9 +120,12 @@ def test_device_loss_of_another_kind_negated(records, tag, tol):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["mlp", "mlpf"])       # layer by layer, and with DeviceFeedforwardNetwork::fuse()
 @pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-9)])
-def test_mlp_sgd_batches(records, tag, tol):
-    r = {k[len(tag) + 5:]: v for k, v in records.items() if k.startswith(tag + ".mlp.")}
+def test_mlp_sgd_batches(records, tag, tol, name):
+    r = {k[len(tag) + len(name) + 2:]: v for k, v in records.items() if k.startswith(tag + "." + name + ".")}
+    if name == "mlpf":
+        assert r["groups"][0] == 1                      # dense + ReLU
     be = hn.OracleBackend(np.float64)
     net = hn.FeedforwardNet([be.dense((20,), 16), be.act("relu", (16,)), be.dense((16,), 6)])
     lr = float(np.float32(0.05)) if tag == "f32" else 0.05
@@ -135,9 +138,12 @@ def test_mlp_sgd_batches(records, tag, tol):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["convnet", "convnetf"])
 @pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-9)])
-def test_convnet_adam_batches(records, tag, tol):
-    r = {k[len(tag) + 9:]: v for k, v in records.items() if k.startswith(tag + ".convnet.")}
+def test_convnet_adam_batches(records, tag, tol, name):
+    r = {k[len(tag) + len(name) + 2:]: v for k, v in records.items() if k.startswith(tag + "." + name + ".")}
+    if name == "convnetf":
+        assert r["groups"][0] == 1                      # conv + ReLU + max pool
     be = hn.OracleBackend(np.float64)
     net = hn.FeedforwardNet([be.conv((8, 8, 3), 8), be.act("relu", (8, 8, 8)), be.maxpool((8, 8, 8)),
                              be.batchnorm((4, 4, 8)), be.dense((4, 4, 8), 5)])
