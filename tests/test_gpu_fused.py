@@ -477,3 +477,78 @@ def test_fused_input_layer_skips_the_input_gradient():
     chain.forward(*(np.asarray(a, np.float64) for a in (x, w, b)))
     grads = chain.backward(np.asarray(x, np.float64), np.asarray(w, np.float64), np.asarray(g, np.float64))
     assert np.array_equal(members["conv"].get_params()[0].get_grad(), grads["dw"])
+
+
+# ---- a seeded sweep of fused groups over geometries nobody chose by hand ------------------------------------------------
+
+def _sweep_cases(count, seed):
+    g = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        RH, RW = int(g.integers(1, 4)), int(g.integers(1, 4))
+        dv, dh = int(g.integers(0, 2)), int(g.integers(0, 2))
+        sv, sh = int(g.integers(1, 3)), int(g.integers(1, 3))
+        pv, ph = int(g.integers(0, RH)), int(g.integers(0, RW))
+        H, W = int(g.integers(2, 34)), int(g.integers(2, 34))
+        eh, ew = (RH - 1) * (dv + 1) + 1, (RW - 1) * (dh + 1) + 1
+        if H + 2 * pv < eh or W + 2 * ph < ew:
+            continue
+        OH, OW = hp.conv_dims(H, W, RH, RW, pv, ph, sv, sh, dv, dh)
+        C = int(g.choice([1, 3, 8, 17]))
+        F = int(g.choice([1, 5, 16, 32, 33, 64, 96]))
+        N = int(g.choice([2, 4, 8, 12, 16, 32, 64, 128]))
+        if N * OH * OW * RH * RW * C * F > 4e8:
+            continue
+        act = [None, ("relu", 0.0), ("relu", 0.0), ("leaky_relu", 0.25), ("elu", 0.0), ("identity", 0.0)][int(g.integers(0, 6))]
+        pools = [None]
+        for prh in (1, 2, 3, 4):
+            for prw in (1, 2, 4):
+                if prh * prw > 1 and OH % prh == 0 and OW % prw == 0:
+                    pools.append(("max", prh, prw, prh, prw))
+        if OH >= 2 and OW >= 2:
+            pools += [("mean", 2, 2, 2, 2), ("max", 2, 2, 1, 1)]
+        pool = pools[int(g.integers(0, len(pools)))]
+        if act is None and pool is None:
+            continue
+        out.append((N, H, W, C, F, dict(RH=RH, RW=RW, pv=pv, ph=ph, sv=sv, sh=sh, dv=dv, dh=dh), act, pool))
+    return out
+
+
+SWEEP = _sweep_cases(120, 20250711)
+SWEEP_MODES = {}
+
+
+@pytest.mark.parametrize("index", range(len(SWEEP)))
+def test_fused_sweep_exact(index):
+    """Random fused groups on exactly representable data (see the module text): outputs, arg-max indices and every
+    gradient equal the oracle's chain bit for bit, in whichever mode the group ran."""
+    N, H, W, C, F, geom, act, pool = SWEEP[index]
+    dtype = np.float32 if index % 3 else np.float64
+    gen = hp.rng(4000 + index)
+    x = _dyadic(gen, (N, H, W, C), dtype)
+    w = _dyadic(gen, (geom["RH"] * geom["RW"] * C, F), dtype)
+    b = _dyadic(gen, (1, F), dtype)
+    if act is not None and act[0] == "elu":
+        act = ("elu", 0.0)      # alpha 0: 0 * (exp(x) - 1) = 0 below zero, exact; the derivative there is y + alpha = 0
+    fused, members, kdims = _build(dtype, N, H, W, C, F, conv=geom, act=act, pool=pool)
+    chain = Chain(geom, act=act, pool=pool)
+    x64, w64, b64 = (np.asarray(a, np.float64) for a in (x, w, b))
+    ref = chain.forward(x64, w64, b64)
+    g = _dyadic(gen, ref.shape, dtype)
+    out, dx, mode = _run_fused(fused, members, x, w, b, g)
+    SWEEP_MODES[mode] = SWEEP_MODES.get(mode, 0) + 1
+    grads = chain.backward(x64, w64, np.asarray(g, np.float64))
+    assert np.array_equal(out, ref), "output (%s)" % mode
+    if pool is not None and pool[0] == "max":
+        assert np.array_equal(members["pool"].max_indices(N), chain.inds), "arg-max indices (%s)" % mode
+    wp, bp = members["conv"].get_params()
+    assert np.array_equal(dx, grads["dx"]), "input gradient (%s)" % mode
+    assert np.array_equal(wp.get_grad(), grads["dw"]), "weight gradient (%s)" % mode
+    assert np.array_equal(bp.get_grad(), grads["db"].reshape(1, -1)), "bias gradient (%s)" % mode
+
+
+def test_fused_sweep_met_every_mode():
+    """Runs after the sweep: it must have exercised the epilogues, not only the member-by-member path."""
+    if sum(SWEEP_MODES.values()) < len(SWEEP):
+        pytest.skip("the sweep did not run in this session")
+    assert SWEEP_MODES.get("pool", 0) >= 15 and SWEEP_MODES.get("act", 0) >= 15, SWEEP_MODES
