@@ -92,6 +92,23 @@ __device__ __forceinline__ void vec_load(T (&dst)[V], const T* p) {
 	}
 }
 
+/* The same from a pointer that is known to point to global memory. A pointer the compiler cannot place (the select
+ * between the source tensor and the block of zeros, for one) makes it emit flat loads, and those count against the LDS
+ * counter as well as the memory counter: every wait for an LDS read in the MFMA loop then also waits for the global
+ * loads of the next chunk, which undoes the prefetch. */
+template<typename T, int V>
+__device__ __forceinline__ void vec_load_global(T (&dst)[V], const T* p) {
+	if constexpr (V == 1) {
+		dst[0] = *(const __attribute__((address_space(1))) T*) p;
+	} else {
+		typedef typename VecOf<T, V>::type vt;
+		const vt v = *(const __attribute__((address_space(1))) vt*) p;
+		#pragma unroll
+		for (int i = 0; i < V; ++i)
+			dst[i] = v[i];
+	}
+}
+
 template<typename T, int V>
 __device__ __forceinline__ void vec_store(T* p, const T (&src)[V]) {
 	if constexpr (V == 1) {
@@ -103,6 +120,16 @@ __device__ __forceinline__ void vec_store(T* p, const T (&src)[V]) {
 		for (int i = 0; i < V; ++i)
 			v[i] = src[i];
 		*reinterpret_cast<vt*>(p) = v;
+	}
+}
+
+/* fn(std::integral_constant<int, 0>()) ... fn(std::integral_constant<int, N - 1>()): a loop whose index is a
+ * compile-time constant in the body (register arrays indexed by it stay registers) */
+template<int N, typename Fn>
+__device__ __forceinline__ void static_for(Fn fn) {
+	if constexpr (N > 0) {
+		static_for<N - 1>(fn);
+		fn(std::integral_constant<int, N - 1>());
 	}
 }
 
@@ -181,7 +208,7 @@ __device__ __forceinline__ int tile_row_m(const GatherLaunch& L, const GatherGeo
 	return (nb << sb_shift) + (row & ((1 << sb_shift) - 1)) + g.N * (ab * pa + pa_i + g.OA * (strip * L.pos_b + pb_i));
 }
 
-template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI = EPI_NONE>
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI = EPI_NONE, int PF = 1>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
 void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom g, const GatherLaunch L, T* __restrict__ partials, const Epilogue<T> E) {
@@ -202,7 +229,11 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 
 	__shared__ __attribute__((aligned(32))) T As[2][KC][LDA];
 	__shared__ __attribute__((aligned(32))) T Bs[2][KC][LDB];
-	__shared__ int4 ktab[3][KC];     /* per reduction index: element offset, ya term, yb term, channel offset */
+	/* PF = how many chunks ahead of the MFMAs the global loads run (held in registers until their turn to be stored to
+	 * LDS): 1 for the large tiles, whose chunk of MFMA work covers the latency of a load; more for the short tiles of
+	 * small problems, where a chunk is a few hundred cycles of MFMAs and a load takes a thousand. */
+	constexpr int NSLOT = PF + 2;
+	__shared__ int4 ktab[NSLOT][KC];     /* per reduction index: element offset, ya term, yb term, channel offset */
 
 	int local, part = 0;
 	const bool split = (int) blockIdx.x >= L.main_blocks;
@@ -222,6 +253,13 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		tile = swizzle_tile(tile, L.tile_rows, L.mtiles / L.tile_rows);
 	const int tid = threadIdx.x;
 	const int f0 = blockIdx.y * BF;
+	/* The bias values of the tile's columns go through LDS: fetched now, read in the epilogue, many barriers later.
+	 * Read from global memory there, each of a lane's FB * NACC values was a load with a wait of its own in front
+	 * of its store: sixteen to thirty-two memory round trips in a row at the end of every block. */
+	static_assert(THREADS >= BF, "one thread per bias value");
+	__shared__ T bias_s[BF];
+	if (tid < BF)
+		bias_s[tid] = (bias != nullptr && f0 + tid < g.F) ? bias[f0 + tid] : (T) 0;
 	/* this block's chunks of the reduction: all of them, or one part */
 	const int chunk0 = split ? part * L.chunks_per_part : 0;
 	const int nchunks = split ? min(L.chunks_per_part, (g.K + KC - 1) / KC - chunk0) : (g.K + KC - 1) / KC;
@@ -280,13 +318,15 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	 * LDS (lane i of a wavefront lands at the wavefront's LDS base + 16 i, whatever address it reads), which
 	 * saves the registers, the LDS store instructions and the wait between load and store. Measured: 1-3 %
 	 * faster in fp32, slower in fp64, so fp32 only. */
-	constexpr bool DIRECT = sizeof(T) == 4 && VEC == 4 && ACOLS % 64 == 0;
+	constexpr bool DIRECT = sizeof(T) == 4 && VEC == 4 && ACOLS % 64 == 0 && PF == 1;
 	const int arow_u = __builtin_amdgcn_readfirstlane(arow0);
 	const int acol_u = __builtin_amdgcn_readfirstlane(acol / 64) * 64 * VEC;
-	T areg[DIRECT ? 1 : ASLOTS][VEC];
-	T breg[BITER][VB];
+	T areg[PF][DIRECT ? 1 : ASLOTS][VEC];
+	T breg[PF][BITER][VB];
 
-	auto load_tiles = [&](int slot, int abuf) {
+	/* `stage` (a std::integral_constant) names the register set of the chunk: chunk c uses set c % PF */
+	auto load_tiles = [&](int slot, int abuf, auto stage) {
+		constexpr int SG = decltype(stage)::value;
 		#pragma unroll
 		for (int s = 0; s < ASLOTS; ++s) {
 			const int4 e = ktab[slot][arow0 + s * ARP];
@@ -308,28 +348,29 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 				__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) p,
 						(__attribute__((address_space(3))) void*) &As[abuf][arow_u + s * ARP][acol_u], 16, 0, 0);
 			else
-				vec_load<T, VEC>(areg[s], p);
+				vec_load_global<T, VEC>(areg[SG][s], p);
 		}
 		#pragma unroll
 		for (int it = 0; it < BITER; ++it) {
 			if (BVECS % THREADS == 0 || tid + it * THREADS < BVECS) {
-				vec_load<T, VB>(breg[it], bptr[it]);
+				vec_load_global<T, VB>(breg[SG][it], bptr[it]);
 				bptr[it] += bstep;
 			}
 		}
 	};
-	auto store_tiles = [&](int buf) {
+	auto store_tiles = [&](int buf, auto stage) {
+		constexpr int SG = decltype(stage)::value;
 		if constexpr (!DIRECT) {
 			#pragma unroll
 			for (int s = 0; s < ASLOTS; ++s)
-				vec_store<T, VEC>(&As[buf][arow0 + s * ARP][acol * VEC], areg[s]);
+				vec_store<T, VEC>(&As[buf][arow0 + s * ARP][acol * VEC], areg[SG][s]);
 		}
 		#pragma unroll
 		for (int it = 0; it < BITER; ++it) {
 			const int idx = tid + it * THREADS;
 			if (BVECS % THREADS == 0 || idx < BVECS) {
 				const int brow = idx / BCOLS, bcol = idx % BCOLS;
-				vec_store<T, VB>(&Bs[buf][brow][bcol * VB], breg[it]);
+				vec_store<T, VB>(&Bs[buf][brow][bcol * VB], breg[SG][it]);
 			}
 		}
 	};
@@ -347,21 +388,33 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			for (int r = 0; r < MF::NACC; ++r)
 				acc[i][j][r] = (T) 0;
 
-	write_table(0);
-	write_table(1);
+	/* tables of chunks 0 .. PF, loads of chunks 0 .. PF - 1, chunk 0 into LDS */
+	#pragma unroll
+	for (int q = 0; q <= PF; ++q)
+		write_table(q);
 	__syncthreads();
-	load_tiles(0, 0);
-	store_tiles(0);
-	__builtin_amdgcn_s_waitcnt(0x0F70);      /* vmcnt(0): the direct loads have landed */
+	static_for<PF>([&](auto q) {
+		if (decltype(q)::value < nchunks)
+			load_tiles(decltype(q)::value, 0, q);
+	});
+	store_tiles(0, std::integral_constant<int, 0>());
+	if constexpr (DIRECT)
+		__builtin_amdgcn_s_waitcnt(0x0F70);  /* vmcnt(0): the direct loads have landed */
 	__syncthreads();
-	int slot_next = 1, slot_write = 2;       /* table slots of chunk c + 1 and c + 2 */
-	for (int c = 0; c < nchunks; ++c) {
+	int slot_load = PF % NSLOT, slot_write = (PF + 1) % NSLOT;      /* table slots of chunk c + PF and c + PF + 1 */
+	for (int c0 = 0; c0 < nchunks; c0 += PF)
+	static_for<PF>([&](auto stage) {
+		constexpr int SG = decltype(stage)::value;
+		const int c = c0 + SG;
+		if (c >= nchunks)
+			return;                          /* the same for every thread of the block: no barrier is skipped by some */
 		const int buf = c & 1;
 		write_table(slot_write);
-		if (c + 1 < nchunks)
-			load_tiles(slot_next, buf ^ 1);
-		slot_next = slot_next == 2 ? 0 : slot_next + 1;
-		slot_write = slot_write == 2 ? 0 : slot_write + 1;
+		if (c + PF < nchunks)
+			load_tiles(slot_load, buf ^ 1, stage);      /* this chunk's registers went to LDS one chunk ago */
+		slot_load = slot_load == NSLOT - 1 ? 0 : slot_load + 1;
+		slot_write = slot_write == NSLOT - 1 ? 0 : slot_write + 1;
+		constexpr std::integral_constant<int, (SG + 1) % PF> next_stage{};
 		/* operand fragments are fetched one reduction step ahead of the MFMAs that use them */
 		T xa[2][MB], wb[2][FB];
 		vec_load<T, MB>(xa[0], &As[buf][lk][wm * WT_M + MB * lc]);
@@ -381,7 +434,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			 * them: its stores (and the wait for its global loads) then overlap that MFMA work, and
 			 * only the barrier itself remains between the chunks */
 			if (KC / KS > 1 && st == KC / KS - 1 && c + 1 < nchunks)
-				store_tiles(buf ^ 1);
+				store_tiles(buf ^ 1, next_stage);
 			/* issue order matters (a wave issues in order and stalls on a busy MFMA pipe): the LDS reads
 			 * of the next step must go out before this step's MFMAs, so pin the schedule here */
 			__builtin_amdgcn_sched_barrier(0);
@@ -393,11 +446,11 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			__builtin_amdgcn_sched_barrier(0);
 		}
 		if (KC / KS <= 1 && c + 1 < nchunks)
-			store_tiles(buf ^ 1);
+			store_tiles(buf ^ 1, next_stage);
 		if constexpr (DIRECT)
 			__builtin_amdgcn_s_waitcnt(0x0F70);  /* vmcnt(0): this wave's direct loads of the next chunk have landed */
 		__syncthreads();
-	}
+	});
 
 	/* epilogue: D rows are filters (row rr of block i is filter FB*rr + i), D columns are m
 	 * (column lc of block j is row MB*lc + j of the tile), so a lane owns MB adjacent outputs */
@@ -446,8 +499,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 						if ((std::is_same<T, float>::value ? r / 4 : r) != q)
 							continue;
 						const int arow = acc_row<T>(r, lk);
-						const int f = f0 + wf * WT_F + FB * arow + i;
-						const T bv = (bias && f < g.F) ? bias[f] : (T) 0;
+						const T bv = bias_s[wf * WT_F + FB * arow + i];
 						T v[MB];
 						#pragma unroll
 						for (int j = 0; j < MB; ++j)
@@ -502,7 +554,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 					const int f = f0 + wf * WT_F + FB * acc_row<T>(r, lk) + i;
 					if (f >= g.F)
 						continue;
-					const T bv = bias ? bias[f] : (T) 0;
+					const T bv = bias_s[wf * WT_F + FB * acc_row<T>(r, lk) + i];
 					const size_t o = (size_t) mm + (size_t) g.M * f;
 					T z[MB], y[MB];
 					#pragma unroll
@@ -545,7 +597,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			#pragma unroll
 			for (int r = 0; r < MF::NACC; ++r) {
 				const int fl = wf * WT_F + FB * acc_row<T>(r, lk) + i;
-				const T bv = (bias && f0 + fl < g.F) ? bias[f0 + fl] : (T) 0;
+				const T bv = bias_s[fl];
 				const T c = __shfl(acc[i][0][r] + bv, lane & ~(TL - 1), 64);
 				T cnt = (T) 0, s1 = (T) 0, s2 = (T) 0;
 				#pragma unroll
@@ -601,7 +653,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		for (int r = 0; r < MF::NACC; ++r) {
 			const int f = f0 + wf * WT_F + FB * acc_row<T>(r, lk) + i;
 			if (f < g.F) {
-				const T bv = bias ? bias[f] : (T) 0;
+				const T bv = bias_s[wf * WT_F + FB * acc_row<T>(r, lk) + i];
 				T* dst = out + ((size_t) mm + (size_t) g.M * f);
 				if (vec_out) {
 					if (mm < g.M) {
@@ -628,6 +680,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 /* How the weight-gradient launch is cut: tiles = ktiles * ftiles blocks per slice, `splits` slices. */
 struct WgradSplit {
 	int ktiles, tiles, splits, chunks_per_split, pixel_mode;
+	int direct;     /* one slice only: the block adds its tile to the gradient itself, `partials` and `bias_partials` are the gradients */
 };
 
 /* ------------------------------------------------------------------------------------------------
@@ -860,7 +913,27 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		}
 	}
 
+	const bool direct = plan.direct != 0;
 	T* dst = partials + (size_t) split * ((size_t) g.K * g.F);
+	if (direct) {
+		/* gradients accumulate (StandardParameters.hpp:119): all of the tile's old values are fetched before the first
+		 * is needed, so that the block waits for memory once and not once per value */
+		#pragma unroll
+		for (int i = 0; i < FB; ++i)
+			#pragma unroll
+			for (int j = 0; j < KB; ++j) {
+				T old[MF::NACC];
+				const int k = min(k0 + wk * WT_K + j * TL + lc, g.K - 1);
+				#pragma unroll
+				for (int r = 0; r < MF::NACC; ++r) {
+					const int f = min(f0 + wf * WT_F + i * TL + acc_row<T>(r, lk), g.F - 1);
+					old[r] = dst[(size_t) k + (size_t) g.K * f];
+				}
+				#pragma unroll
+				for (int r = 0; r < MF::NACC; ++r)
+					acc[i][j][r] += old[r];
+			}
+	}
 	#pragma unroll
 	for (int i = 0; i < FB; ++i) {
 		#pragma unroll
@@ -888,12 +961,13 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 			bred[frow * Q + p % Q] = bacc[it];
 	}
 	__syncthreads();
-	if (tid < BF && tid % ktiles == kt && f0 + tid < g.F) {
+	if (tid < BF && tid % ktiles == kt && f0 + tid < g.F && bias_partials != nullptr) {
 		T s = (T) 0;
 		#pragma unroll
 		for (int q = 0; q < Q; ++q)
 			s += bred[tid * Q + q];
-		bias_partials[(size_t) split * g.F + f0 + tid] = s;
+		T* o = bias_partials + ((size_t) split * g.F + f0 + tid);
+		*o = direct ? *o + s : s;
 	}
 }
 
@@ -1117,7 +1191,7 @@ struct GatherVariant {
 };
 
 /* The fused epilogues exist for the vectorised, divisor-free (forward) form of every tile shape. */
-template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int PF>
 void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g,
 		const GatherLaunch& L, T* partials, bool vec, bool divs, int epi, const Epilogue<T>& E) {
 	constexpr int VEC = GemmCfg<T>::VEC;
@@ -1125,23 +1199,23 @@ void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, con
 	if (epi != EPI_NONE) {
 		CATTLE_HIP_REQUIRE(vec && !divs, "a fused epilogue needs the vectorised forward form of the GEMM");
 		if (epi == EPI_ACT)
-			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 		else if (epi == EPI_POOL)
-			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 		else
-			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_STATS><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_STATS, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	} else if (vec && !divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else if (vec && divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else if (!divs)
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else
-		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
-template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int PF>
 int gather_variant_occupancy(size_t dyn, bool vec, bool divs, int epi) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	/* the answer for the usual launch (no reserved dynamic LDS) is kept: one query per kernel instantiation */
@@ -1153,26 +1227,26 @@ int gather_variant_occupancy(size_t dyn, bool vec, bool divs, int epi) {
 	hipError_t e;
 	constexpr int TH = 64 * WAVES_M * WAVES_F;
 	if (epi == EPI_ACT)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT>, TH, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT, PF>, TH, dyn);
 	else if (epi == EPI_POOL)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL>, TH, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL, PF>, TH, dyn);
 	else if (epi == EPI_STATS)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_STATS>, TH, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_STATS, PF>, TH, dyn);
 	else if (vec && !divs)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false>, TH, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_NONE, PF>, TH, dyn);
 	else if (vec && divs)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true>, TH, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, true, EPI_NONE, PF>, TH, dyn);
 	else if (!divs)
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false>, TH, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false, EPI_NONE, PF>, TH, dyn);
 	else
-		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true>, TH, dyn);
+		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true, EPI_NONE, PF>, TH, dyn);
 	CATTLE_HIP_CHECK(e);
 	if (dyn == 0)
 		slot = n;
 	return n;
 }
 
-template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC = GemmCfg<T>::KC>
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC = GemmCfg<T>::KC, int PF = 1>
 GatherVariant<T> gather_variant() {
 	typedef GemmCfg<T> C;
 	static_assert(WT_ROW_PAD % KC == 0 && WAVES_F * WT_F <= WT_COL_PAD, "prepared weights are padded to whole tiles");
@@ -1180,16 +1254,16 @@ GatherVariant<T> gather_variant() {
 	v.bm = WAVES_M * WT_M;
 	v.bf = WAVES_F * WT_F;
 	v.waves = WAVES_M * WAVES_F;
-	v.lds_bytes = 2 * KC * (v.bm + v.bf + 2 * C::pad(v.bm)) * (int) sizeof(T) + 3 * KC * 16;
+	v.lds_bytes = 2 * KC * (v.bm + v.bf + 2 * C::pad(v.bm)) * (int) sizeof(T) + (PF + 2) * KC * 16;
 	v.kc = KC;
-	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC>;
-	v.blocks_per_cu = &gather_variant_occupancy<T, WAVES_M, WAVES_F, WT_M, WT_F, KC>;
+	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, PF>;
+	v.blocks_per_cu = &gather_variant_occupancy<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, PF>;
 	return v;
 }
 
 template<typename T> struct GatherVariants;
 template<> struct GatherVariants<float> {
-	static constexpr int COUNT = 8, LARGE = 4, SHORT = 2;
+	static constexpr int COUNT = 9, LARGE = 4, SHORT = 2, TALL32 = 8;
 	static const GatherVariant<float>* get() {
 		static const GatherVariant<float> v[COUNT] = {
 			gather_variant<float, 4, 2, 64, 64>(),      /* 256 x 128 */
@@ -1202,12 +1276,13 @@ template<> struct GatherVariants<float> {
 			gather_variant<float, 2, 1, 32, 32, 64>(),  /* 64 x 32 */
 			gather_variant<float, 2, 2, 32, 32, 32>(),  /* 64 x 64, chunks of 32: several short tiles per CU */
 			gather_variant<float, 2, 1, 32, 32, 32>(),  /* 64 x 32, chunks of 32 */
+			gather_variant<float, 4, 1, 32, 32, 32>(),  /* 128 x 32, four waves: few columns, a few hundred tiles */
 		};
 		return v;
 	}
 };
 template<> struct GatherVariants<double> {
-	static constexpr int COUNT = 7, LARGE = 3, SHORT = 2;
+	static constexpr int COUNT = 7, LARGE = 3, SHORT = 2, TALL32 = -1;
 	static const GatherVariant<double>* get() {
 		static const GatherVariant<double> v[COUNT] = {
 			gather_variant<double, 8, 2, 32, 64>(),     /* 256 x 128, sixteen waves */
@@ -1231,7 +1306,7 @@ struct Tuning {
 	struct PerF { int F, variant, occ; };
 	std::vector<PerF> per_f;
 	bool no_swizzle, no_row_blocks, no_split, wgrad_linear;
-	int wgrad_variant, wgrad_splits;
+	int wgrad_variant, wgrad_splits, wgrad_min_chunks;
 
 	Tuning() {
 		no_swizzle = std::getenv("CATTLE_HIP_NO_SWIZZLE") != nullptr;
@@ -1242,6 +1317,8 @@ struct Tuning {
 		wgrad_variant = e ? std::atoi(e) : -1;
 		e = std::getenv("CATTLE_HIP_WGRAD_SPLITS");
 		wgrad_splits = e ? std::atoi(e) : 0;
+		e = std::getenv("CATTLE_HIP_WGRAD_MIN_CHUNKS");
+		wgrad_min_chunks = e ? std::atoi(e) : 0;
 		for (char** v = environ; v && *v; ++v) {
 			static const char* const keys[2] = { "CATTLE_HIP_GATHER_VARIANT_F", "CATTLE_HIP_GATHER_OCC_F" };
 			for (int k = 0; k < 2; ++k) {
@@ -1336,6 +1413,14 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if (narrower || taller)
 			best_v = i;
 	}
+	/* The widest shape with at most one and a half blocks per CU: the next narrower one doubles the blocks, and with
+	 * them the blocks that overlap each other's memory waits on a CU (the input-side LSTM gates, 320 tiles of
+	 * 256 x 128 with K = 72: 37 -> 31 us). */
+	if (best_v == 0 && vars[0].bf > vars[1].bf && g.F > vars[1].bf) {
+		const long blocks = (long) ((g.M + vars[0].bm - 1) / vars[0].bm) * ((g.F + vars[0].bf - 1) / vars[0].bf);
+		if (blocks >= NUM_CUS && blocks * 2 <= 3 * NUM_CUS)
+			best_v = 1;
+	}
 	/* too few large tiles to give every CU one: take the short tiles (the narrowest that still covers F, else the widest) */
 	if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) < NUM_CUS) {
 		constexpr int SHORT = GatherVariants<T>::SHORT;       /* short shapes, each with long and with medium chunks */
@@ -1350,6 +1435,12 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		const long short_tiles = (long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf);
 		if (short_tiles >= 2 * NUM_CUS || short_tiles * 2 <= NUM_CUS)
 			best_v += SHORT;
+		/* 32 columns and enough rows for every CU to get a tile twice as tall: four waves share the table and the
+		 * barriers that two-wave blocks pay for alone (config 3's second input gradient, 512 tiles of 64 x 32 with
+		 * K = 576: 33 -> 25 us) */
+		if (GatherVariants<T>::TALL32 >= 0 && vars[best_v].bf == 32 &&
+				(long) ((g.M + 127) / 128) * ((g.F + 31) / 32) >= NUM_CUS)
+			best_v = GatherVariants<T>::TALL32;
 	}
 	const Tuning& tune = tuning();
 	int occ = 0;
@@ -1491,48 +1582,54 @@ constexpr int WGRAD_MC = 32;
 template<typename T>
 struct WgradVariant {
 	int bk, bf, waves;
+	int mc;                         /* rows of M per reduction chunk; above 32 only with 16-byte loads */
 	void (*launch)(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom&, const WgradSplit&, bool vec);
 	int (*blocks_per_cu)();         /* what the runtime says fits on a CU (registers and LDS) */
 };
 
-template<typename T, int WK, int WF, int TK, int TF, int MINW = 1>
+template<typename T, int WK, int WF, int TK, int TF, int MINW = 1, int MC = WGRAD_MC>
 void launch_wgrad_variant(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom& g, const WgradSplit& plan,
 		bool vec) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	dim3 block(64 * WK * WF), grid((unsigned) round_up(plan.tiles * plan.splits, 8));
-	if (vec)
-		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, VEC, MINW><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
-	else
-		wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, 1, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
+	if (vec) {
+		wgrad_kernel<T, WK, WF, TK, TF, MC, VEC, MINW><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
+	} else {
+		if constexpr (MC == WGRAD_MC)
+			wgrad_kernel<T, WK, WF, TK, TF, MC, 1, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
+		else
+			CATTLE_HIP_REQUIRE(false, "a weight-gradient variant with long chunks was planned for scalar loads");
+	}
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
-template<typename T, int WK, int WF, int TK, int TF, int MINW = 1>
+template<typename T, int WK, int WF, int TK, int TF, int MINW = 1, int MC = WGRAD_MC>
 int wgrad_variant_occupancy() {
 	static int cached = 0;
 	if (cached == 0) {
 		int n = 0;
-		CATTLE_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, wgrad_kernel<T, WK, WF, TK, TF, WGRAD_MC, GemmCfg<T>::VEC, MINW>,
+		CATTLE_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, wgrad_kernel<T, WK, WF, TK, TF, MC, GemmCfg<T>::VEC, MINW>,
 				64 * WK * WF, 0));
 		cached = std::max(1, n);
 	}
 	return cached;
 }
 
-template<typename T, int WK, int WF, int TK, int TF, int MINW = 1>
+template<typename T, int WK, int WF, int TK, int TF, int MINW = 1, int MC = WGRAD_MC>
 WgradVariant<T> wgrad_variant() {
 	WgradVariant<T> v;
 	v.bk = WK * TK;
 	v.bf = WF * TF;
 	v.waves = WK * WF;
-	v.launch = &launch_wgrad_variant<T, WK, WF, TK, TF, MINW>;
-	v.blocks_per_cu = &wgrad_variant_occupancy<T, WK, WF, TK, TF, MINW>;
+	v.mc = MC;
+	v.launch = &launch_wgrad_variant<T, WK, WF, TK, TF, MINW, MC>;
+	v.blocks_per_cu = &wgrad_variant_occupancy<T, WK, WF, TK, TF, MINW, MC>;
 	return v;
 }
 
 template<typename T> struct WgradVariants;
 template<> struct WgradVariants<float> {
-	static constexpr int COUNT = 7;
+	static constexpr int COUNT = 11, BASE = 7;      /* BASE: the variants with the standard chunk, which any problem may use */
 	static const WgradVariant<float>* get() {
 		static const WgradVariant<float> v[COUNT] = {
 			wgrad_variant<float, 2, 4, 96, 32, 4>(),    /* 192 x 128, registers held to four waves per SIMD = two blocks per CU */
@@ -1542,12 +1639,17 @@ template<> struct WgradVariants<float> {
 			wgrad_variant<float, 1, 4, 64, 32>(),       /*  64 x 128 */
 			wgrad_variant<float, 2, 2, 32, 32>(),       /*  64 x 64: few filters */
 			wgrad_variant<float, 1, 1, 32, 32>(),       /*  32 x 32, one wave: the first layer of a network (K = 27, a few filters) */
+			/* the same small tiles with longer chunks of M: fewer, larger rounds of loads for latency-bound problems */
+			wgrad_variant<float, 1, 1, 32, 32, 1, 128>(),
+			wgrad_variant<float, 1, 1, 32, 32, 1, 64>(),
+			wgrad_variant<float, 2, 2, 32, 32, 1, 64>(),
+			wgrad_variant<float, 2, 2, 32, 32, 1, 128>(),
 		};
 		return v;
 	}
 };
 template<> struct WgradVariants<double> {
-	static constexpr int COUNT = 4;
+	static constexpr int COUNT = 4, BASE = 4;
 	static const WgradVariant<double>* get() {
 		static const WgradVariant<double> v[COUNT] = {
 			wgrad_variant<double, 2, 4, 48, 32>(),      /* 96 x 128 */
@@ -1569,12 +1671,12 @@ struct WgradPlan {
  * reports for the variant. The plan depends on the shape and the build only, which keeps the summation
  * order, and with it the result, reproducible. */
 template<typename T>
-WgradPlan wgrad_plan(int M, int K, int F, int N) {
+WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 	const WgradVariant<T>* vars = WgradVariants<T>::get();
 	WgradPlan p;
 	p.variant = 0;
 	long best = -1;
-	for (int i = 0; i < WgradVariants<T>::COUNT; ++i) {
+	for (int i = 0; i < WgradVariants<T>::BASE; ++i) {
 		const long padded = (long) round_up(K, vars[i].bk) * round_up(F, vars[i].bf);
 		if (best < 0 || padded < best) {
 			best = padded;
@@ -1582,7 +1684,32 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 		}
 	}
 	const Tuning& tune = tuning();
-	if (tune.wgrad_variant >= 0 && tune.wgrad_variant < WgradVariants<T>::COUNT)
+	/* A short reduction (a dense layer: M is the batch size) cannot be cut into many slices, so the tiles must fill the
+	 * chip: among the shapes with the least padding, the largest whose tiles times the possible slices reach half of
+	 * the CUs, else the one with the most tiles. Two chunks per block then, not four: measured, a block's time is its
+	 * chain of chunks (about a microsecond each at these sizes), which the second launch that adds the slices costs less than. */
+	const bool short_m = (M + WGRAD_MC - 1) / WGRAD_MC <= 16;
+	if (short_m) {
+		const int max_splits = std::max(1, (M + WGRAD_MC - 1) / WGRAD_MC / 2);
+		int pick = -1;
+		long most = -1;
+		for (int i = 0; i < WgradVariants<T>::BASE; ++i) {
+			if ((long) round_up(K, vars[i].bk) * round_up(F, vars[i].bf) != best)
+				continue;
+			const long blocks = (long) ((K + vars[i].bk - 1) / vars[i].bk) * ((F + vars[i].bf - 1) / vars[i].bf) * max_splits;
+			if (blocks >= NUM_CUS / 2) {
+				pick = i;
+				break;
+			}
+			if (blocks > most) {
+				most = blocks;
+				pick = i;
+			}
+		}
+		if (pick >= 0)
+			p.variant = pick;
+	}
+	if (tune.wgrad_variant >= 0 && tune.wgrad_variant < WgradVariants<T>::COUNT && (vec || vars[tune.wgrad_variant].mc == WGRAD_MC))
 		p.variant = tune.wgrad_variant;
 	const WgradVariant<T>& v = vars[p.variant];
 	p.ktiles = (K + v.bk - 1) / v.bk;
@@ -1591,17 +1718,18 @@ WgradPlan wgrad_plan(int M, int K, int F, int N) {
 	const int occ = std::max(1, std::min(v.blocks_per_cu(), std::max(3, 16 / v.waves)));
 	const int slots = NUM_CUS * occ;
 	const int tiles = p.ktiles * p.ftiles;
-	const int chunks = (M + WGRAD_MC - 1) / WGRAD_MC;
+	const int chunks = (M + v.mc - 1) / v.mc;
 	int want = std::max(1, slots / tiles);
+	const int min_chunks = tune.wgrad_min_chunks > 0 ? tune.wgrad_min_chunks : (short_m ? 2 : 4);
+	want = std::min(want, std::max(1, chunks / min_chunks));  /* at least four chunks per block */
 	if (tune.wgrad_splits > 0)
-		want = tune.wgrad_splits;
-	want = std::min(want, std::max(1, chunks / 4));           /* at least four chunks per block */
+		want = std::min(tune.wgrad_splits, chunks);
 	p.chunks_per_split = (chunks + want - 1) / want;
 	p.splits = (chunks + p.chunks_per_split - 1) / p.chunks_per_split;
 	/* pixel mode: slices are ranges of output positions (each at least one), walked sample block by
 	 * sample block; needs chunks that do not straddle positions */
 	const int positions = M / N;
-	p.pixel_mode = N % WGRAD_MC == 0 && positions >= 2 && !tune.wgrad_linear;
+	p.pixel_mode = N % v.mc == 0 && positions >= 2 && !tune.wgrad_linear;
 	if (p.pixel_mode)
 		p.splits = std::max(1, std::min(want, positions));
 	return p;
@@ -1620,8 +1748,8 @@ ConvWorkspace conv_workspace(const ConvShape& s, int N) {
 	ws.wt_fwd = (size_t) round_up(s.K(), WT_ROW_PAD) * round_up(s.F, WT_COL_PAD);
 	ws.wt_dgrad = (size_t) round_up(s.RH * s.RW * s.F, WT_ROW_PAD) * round_up(s.C, WT_COL_PAD);
 	const int M = N * s.OH() * s.OW();
-	const WgradPlan p = wgrad_plan<T>(M, s.K(), s.F, N);
-	ws.partials = (size_t) p.splits * ((size_t) s.K() * s.F + (size_t) s.F);
+	const WgradPlan p = wgrad_plan<T>(M, s.K(), s.F, N, true), q = wgrad_plan<T>(M, s.K(), s.F, N, false);
+	ws.partials = (size_t) std::max(p.splits, q.splits) * ((size_t) s.K() * s.F + (size_t) s.F);
 	return ws;
 }
 
@@ -1702,13 +1830,19 @@ void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_gr
 	check_sizes(s, N);
 	const GatherGeom g = forward_geom(s, N);
 	/* split-M partials, then a fixed-order reduction that accumulates */
-	const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N);
+	const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
+	const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N, vec);
 	const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
 	const size_t count = (size_t) g.K * g.F;
 	T* bias_partials = partials + (size_t) p.splits * count;
-	const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode };
-	const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
+	if (p.splits == 1) {
+		/* one slice: every block owns its tile of the gradient and adds to it directly, no second launch */
+		const WgradSplit direct = { p.ktiles, p.ktiles * p.ftiles, 1, p.chunks_per_split, p.pixel_mode, 1 };
+		v.launch(x, out_grad, wgrad, bgrad, g, direct, vec);
+		return;
+	}
+	const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode, 0 };
 	v.launch(x, out_grad, partials, bias_partials, g, split, vec);
 	const int wblocks = (int) ((count + 63) / 64), bblocks = bgrad ? (g.F + 63) / 64 : 0;
 	constexpr int V = 16 / (int) sizeof(T);
