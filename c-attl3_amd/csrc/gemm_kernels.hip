@@ -592,36 +592,65 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		 * m merged in ascending order by the update of Chan et al. */
 		T* const red = &As[0][0][0];                    /* [WAVES_M][BF][4]: count, shift, sum, sum of squares */
 		static_assert(WAVES_M * (WAVES_F * WT_F) * 4 <= 2 * KC * LDA, "the moment partials reuse the A operand buffers");
+		/* The cross-lane steps are written level by level over all of a lane's FB * NACC columns: the shuffles of a
+		 * level do not depend on one another, so they go out together and are waited for once (a butterfly per column,
+		 * one after the other, is a chain of a few hundred LDS-crossbar round trips). */
+		T c[FB][MF::NACC], s1[FB][MF::NACC], s2[FB][MF::NACC];
 		#pragma unroll
-		for (int i = 0; i < FB; ++i) {
+		for (int i = 0; i < FB; ++i)
+			#pragma unroll
+			for (int r = 0; r < MF::NACC; ++r)
+				c[i][r] = acc[i][0][r] + bias_s[wf * WT_F + FB * acc_row<T>(r, lk) + i];
+		#pragma unroll
+		for (int i = 0; i < FB; ++i)
+			#pragma unroll
+			for (int r = 0; r < MF::NACC; ++r)
+				c[i][r] = __shfl(c[i][r], lane & ~(TL - 1), 64);
+		#pragma unroll
+		for (int i = 0; i < FB; ++i)
 			#pragma unroll
 			for (int r = 0; r < MF::NACC; ++r) {
-				const int fl = wf * WT_F + FB * acc_row<T>(r, lk) + i;
-				const T bv = bias_s[fl];
-				const T c = __shfl(acc[i][0][r] + bv, lane & ~(TL - 1), 64);
-				T cnt = (T) 0, s1 = (T) 0, s2 = (T) 0;
+				const T bv = bias_s[wf * WT_F + FB * acc_row<T>(r, lk) + i];
+				s1[i][r] = (T) 0;
+				s2[i][r] = (T) 0;
 				#pragma unroll
 				for (int j = 0; j < MB; ++j) {
-					const bool valid = mm + j < g.M;
-					const T d = valid ? (acc[i][j][r] + bv) - c : (T) 0;
-					cnt += valid ? (T) 1 : (T) 0;
-					s1 += d;
-					s2 += d * d;
-				}
-				#pragma unroll
-				for (int off = 1; off < TL; off <<= 1) {
-					cnt += __shfl_xor(cnt, off, 64);
-					s1 += __shfl_xor(s1, off, 64);
-					s2 += __shfl_xor(s2, off, 64);
-				}
-				if (lc == 0) {
-					T* dst = red + ((size_t) wm * BF + fl) * 4;
-					dst[0] = cnt;
-					dst[1] = c;
-					dst[2] = s1;
-					dst[3] = s2;
+					const T d = mm + j < g.M ? (acc[i][j][r] + bv) - c[i][r] : (T) 0;
+					s1[i][r] += d;
+					s2[i][r] += d * d;
 				}
 			}
+		#pragma unroll
+		for (int off = 1; off < TL; off <<= 1) {
+			T t1[FB][MF::NACC], t2[FB][MF::NACC];
+			#pragma unroll
+			for (int i = 0; i < FB; ++i)
+				#pragma unroll
+				for (int r = 0; r < MF::NACC; ++r) {
+					t1[i][r] = __shfl_xor(s1[i][r], off, 64);
+					t2[i][r] = __shfl_xor(s2[i][r], off, 64);
+				}
+			#pragma unroll
+			for (int i = 0; i < FB; ++i)
+				#pragma unroll
+				for (int r = 0; r < MF::NACC; ++r) {
+					s1[i][r] += t1[i][r];
+					s2[i][r] += t2[i][r];
+				}
+		}
+		/* rows of this wave that exist: all of them in the blocked order, else what is left of M */
+		const int wave_rows = L.sample_blocks > 0 ? WT_M : max(0, min(WT_M, g.M - (tile * BM + wm * WT_M)));
+		if (lc == 0) {
+			#pragma unroll
+			for (int i = 0; i < FB; ++i)
+				#pragma unroll
+				for (int r = 0; r < MF::NACC; ++r) {
+					T* dst = red + ((size_t) wm * BF + wf * WT_F + FB * acc_row<T>(r, lk) + i) * 4;
+					dst[0] = (T) wave_rows;
+					dst[1] = c[i][r];
+					dst[2] = s1[i][r];
+					dst[3] = s2[i][r];
+				}
 		}
 		__syncthreads();
 		for (int fl = tid; fl < BF; fl += THREADS) {
