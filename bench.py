@@ -303,12 +303,25 @@ def convlstm_run(args, dtype):
         step()
     ch.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    # the same propagate + backpropagate recorded once and launched as a HIP graph
+    with ch.Graph() as graph:
+        step()
+    for _ in range(args.warmup):
+        graph.launch()
+    ch.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.launch()
+    ch.synchronize()
+    graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    graph.destroy()
     M = N * H * W
     fwd = 2.0 * M * hid * 4 * (T * 9 * C + (T - 1) * 9 * hid)          # the 4+4 kernels of every step
     flop = 2 * fwd + 2.0 * M * 4 * hid * 9 * hid * (T - 1)              # + weight gradients + recurrent input gradients
     return {"metric": "convlstm_bptt_sequences_per_s", "value": round(N / (ms * 1e-3), 1), "unit": "sequences/s", "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
             "dtype": args.dtype, "data": "synthetic", "gflops": round(flop / (ms * 1e-3) / 1e9, 1),
+            "recorded_as_hip_graph": {"ms_per_step": round(graph_ms, 4), "sequences_per_s": round(N / (graph_ms * 1e-3), 1)},
             "config": {"workload": "ConvLSTM T=10 batch 32 16x16x8 -> 32 hidden, 3x3, propagate + BPTT (BASELINE configs[4])",
                        "flop_per_step": flop}}
 
@@ -376,6 +389,40 @@ def train_steps_run(args, dtype):
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
         rows.append({"workload": name, "ms_per_step": round(ms, 4), "samples_per_s": round(N / (ms * 1e-3), 1),
                      "gflops": round(flop / (ms * 1e-3) / 1e9, 1)})
+        if fuse:
+            # the same step recorded once and launched as a HIP graph (cattle_hip_graph_*); Adam's update depends on the
+            # time step, a scalar argument, so it stays outside the recording
+            def passes(t):
+                a = x
+                for l in layers:
+                    a = l.pass_forward(a, True)
+                g = ch.loss_d_function("softmax_cross_entropy", a, y, scale=1.0 / N)
+                for l in reversed(layers):
+                    g = l.pass_back(g)
+                if not adam:
+                    plist.optimizer_step("vanilla_sgd", [1e-3])
+
+            with ch.Graph() as graph:
+                passes(0)
+
+            def graph_step(t):
+                graph.launch()
+                if adam:
+                    plist.optimizer_step("adam", [1e-3, 1e-1, 1e-3, 1e-5], timestep=t)
+
+            for t in range(args.warmup):
+                graph_step(t)
+            ch.synchronize()
+            t0 = time.perf_counter()
+            for t in range(args.steps):
+                graph_step(t)
+            ch.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / args.steps
+            rows.append({"workload": name + ", recorded as a HIP graph" + (" (Adam step outside)" if adam else ""),
+                         "ms_per_step": round(ms, 4), "samples_per_s": round(N / (ms * 1e-3), 1),
+                         "gflops": round(flop / (ms * 1e-3) / 1e9, 1)})
+            ch.synchronize()
+            graph.destroy()
     line = {"metric": "device_resident_training_step", "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "dtype": args.dtype, "data": "synthetic",
             "driver": "python (ctypes), one C-ABI call per layer pass, one for the optimizer step", "steps_timed": rows}

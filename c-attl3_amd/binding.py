@@ -43,7 +43,8 @@ EXPORTS = [
     "cattle_hip_layer_param_reset_optimizer_state", "cattle_hip_convlstm_create", "cattle_hip_convlstm_propagate",
     "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
     "cattle_hip_convlstm_get_kernel_grad", "cattle_hip_conv_forward_noalloc", "cattle_hip_static_scratch_bytes",
-    "cattle_hip_fused_create", "cattle_hip_fused_last_mode",
+    "cattle_hip_fused_create", "cattle_hip_fused_last_mode", "cattle_hip_graph_begin_capture", "cattle_hip_graph_end_capture",
+    "cattle_hip_graph_launch", "cattle_hip_graph_destroy",
 ]
 
 
@@ -792,3 +793,38 @@ def fuse_layers(layers):
             out.append(layers[i])
         i += len(group)
     return out
+
+
+class Graph(object):
+    """A recorded sequence of device-side calls (cattle_hip_graph_*): `with Graph() as g: step()` records what step()
+    issues instead of running it, g.launch() runs it. step() must have run once before, use device tensors only and read
+    nothing back; the tensors it uses and creates belong to the graph until the graph is destroyed."""
+
+    def __init__(self):
+        self._h = None
+
+    def __enter__(self):
+        _check(lib().cattle_hip_graph_begin_capture())
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        h = ctypes.c_void_p()
+        rc = lib().cattle_hip_graph_end_capture(ctypes.byref(h))
+        if exc_type is None:
+            _check(rc)
+            self._h = h
+        return False
+
+    def launch(self):
+        _check(lib().cattle_hip_graph_launch(self._h))
+
+    def destroy(self):
+        if self._h is not None:
+            _check(lib().cattle_hip_graph_destroy(self._h))
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass

@@ -37,6 +37,10 @@ enum { ERR_INVALID = 1, ERR_STATE = 2, ERR_DEVICE = 3, ERR_OOM = 4 };
 
 /* The stream every kernel and copy of the library is issued on. */
 hipStream_t stream();
+/* Whether that stream is recording a graph (between cattle_hip_graph_begin_capture and _end_capture). Work that cannot
+ * be part of a graph - host copies, waits, allocations that replace a buffer - calls forbid_while_capturing. */
+bool capturing();
+void forbid_while_capturing(const char* what);
 
 /* Copies between pageable host memory and the device on that stream; both return when the host buffer may be
  * reused (host_to_device) or holds the data (device_to_host). Large copies are staged through pinned buffers by

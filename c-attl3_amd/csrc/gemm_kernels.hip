@@ -1111,6 +1111,7 @@ void* split_workspace(size_t bytes) {
 	static void* ptr = nullptr;
 	static size_t cap = 0;
 	if (bytes > cap) {
+		forbid_while_capturing("growing the scratch buffer of the split reductions (run the step once before recording it)");
 		if (ptr)
 			(void) hipFree(ptr);
 		ptr = nullptr;

@@ -125,6 +125,7 @@ Stager* stager() {
 } /* namespace */
 
 void host_to_device(void* dst_dev, const void* src_host, size_t bytes) {
+	forbid_while_capturing("a copy between host and device memory");
 	if (bytes == 0)
 		return;
 	Stager* st = bytes >= STAGE_MIN_BYTES ? stager() : nullptr;
@@ -151,6 +152,7 @@ void host_to_device(void* dst_dev, const void* src_host, size_t bytes) {
 }
 
 void device_to_host(void* dst_host, const void* src_dev, size_t bytes) {
+	forbid_while_capturing("a copy between host and device memory");
 	if (bytes == 0)
 		return;
 	Stager* st = bytes >= STAGE_MIN_BYTES ? stager() : nullptr;

@@ -10,6 +10,7 @@
 #include "act_math.hpp"
 #include "../../include/cattle_hip.h"
 
+#include <algorithm>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -24,6 +25,7 @@ std::recursive_mutex g_mutex;
 thread_local std::string g_last_error;
 bool g_ready = false;
 hipStream_t g_stream = nullptr;
+bool g_capturing = false;
 
 void ensure_init(int device) {
 	if (g_ready)
@@ -61,6 +63,8 @@ struct DevBuf {
 	}
 	void* ensure(size_t bytes) {
 		if (bytes > cap) {
+			/* recorded work may already point into the old buffer */
+			forbid_while_capturing("growing a buffer of a layer (run the step once, at this batch size, before recording it)");
 			release();
 			const size_t want = (bytes + 255) / 256 * 256;
 			CATTLE_HIP_CHECK(hipMalloc(&p, want));
@@ -93,10 +97,12 @@ void fill_zero(void* dst_dev, size_t bytes) {
 		return;
 	/* every buffer of the library is made of 4- or 8-byte scalars and is zeroed by a kernel, which a caller may record
 	 * into a graph; only an odd-sized caller buffer goes to the runtime's memset */
-	if ((reinterpret_cast<uintptr_t>(dst_dev) & 3) == 0 && bytes % 4 == 0)
+	if ((reinterpret_cast<uintptr_t>(dst_dev) & 3) == 0 && bytes % 4 == 0) {
 		device_zero_fill(dst_dev, bytes);
-	else
+	} else {
+		forbid_while_capturing("zeroing a buffer that is not made of 4-byte words");
 		CATTLE_HIP_CHECK(hipMemsetAsync(dst_dev, 0, bytes, stream()));
+	}
 }
 
 /* Device memory handed out through cattle_hip_alloc. Activations of a training step are allocated and
@@ -127,7 +133,7 @@ struct DevicePool {
 			idle_bytes -= c;
 		} else {
 			hipError_t e = hipMalloc(&p, c);
-			if (e == hipErrorOutOfMemory && idle_bytes > 0) {       /* give the idle blocks back and try again */
+			if (e == hipErrorOutOfMemory && idle_bytes > 0 && !g_capturing) {       /* give the idle blocks back and try again */
 				(void) hipGetLastError();
 				(void) hipStreamSynchronize(stream());
 				trim();
@@ -136,11 +142,42 @@ struct DevicePool {
 			CATTLE_HIP_CHECK(e);
 		}
 		live[p] = c;
+		if (g_capturing)
+			taken.push_back(p);
 		return p;
 	}
+	/* the end of a graph: its blocks become ordinary ones again, the freed ones idle */
+	void release_graph(std::vector<void*>* blocks) {
+		for (std::map<void*, std::vector<void*>*>::iterator it = owner.begin(); it != owner.end();) {
+			if (it->second == blocks)
+				it = owner.erase(it);
+			else
+				++it;
+		}
+		std::vector<void*> freed;
+		freed.swap(*blocks);
+		for (void* b : freed)
+			give_back(b);
+	}
+	/* Blocks that recorded kernels read and write at every launch of their graph must not be handed out again while
+	 * the graph exists: those freed during a recording wait in `held` for the graph object, and those taken during a
+	 * recording (`taken`, then `owner`) go to their graph, not to the idle lists, when they are freed later. */
+	std::vector<void*> held, taken;
+	std::map<void*, std::vector<void*>*> owner;
 	void give_back(void* p) {
 		std::map<void*, size_t>::iterator it = live.find(p);
 		CATTLE_HIP_REQUIRE(it != live.end(), "cattle_hip_free of a pointer that cattle_hip_alloc did not return");
+		if (g_capturing) {
+			if (std::find(held.begin(), held.end(), p) == held.end())
+				held.push_back(p);
+			return;
+		}
+		std::map<void*, std::vector<void*>*>::iterator own = owner.find(p);
+		if (own != owner.end()) {
+			if (std::find(own->second->begin(), own->second->end(), p) == own->second->end())
+				own->second->push_back(p);
+			return;
+		}
 		idle[it->second].push_back(p);
 		idle_index[static_cast<const char*>(p)] = it->second;
 		idle_bytes += it->second;
@@ -157,6 +194,7 @@ struct DevicePool {
 		return static_cast<const char*>(p) < it->first + it->second;
 	}
 	void trim() {
+		forbid_while_capturing("returning device memory to the driver");
 		for (std::map<size_t, std::vector<void*>>::iterator it = idle.begin(); it != idle.end(); ++it) {
 			for (void* p : it->second)
 				(void) hipFree(p);
@@ -1135,6 +1173,14 @@ struct Timer {
 	hipEvent_t start = nullptr, stop = nullptr;
 };
 
+/* A recorded sequence of library calls (kernels and device-to-device copies on the library's stream) that can be
+ * launched again as one unit. It keeps the blocks that were given back to the pool while it was recorded. */
+struct Graph {
+	hipGraph_t graph = nullptr;
+	hipGraphExec_t exec = nullptr;
+	std::vector<void*> blocks;
+};
+
 LayerBase* as_layer(cattle_hip_layer_t h) {
 	CATTLE_HIP_REQUIRE(h != nullptr, "null layer handle");
 	return reinterpret_cast<LayerBase*>(h);
@@ -1375,6 +1421,15 @@ hipStream_t stream() {
 	return g_stream;
 }
 
+bool capturing() {
+	return g_capturing;
+}
+
+void forbid_while_capturing(const char* what) {
+	if (g_capturing)
+		throw Error(ERR_STATE, std::string("not possible while a graph is being recorded: ") + what);
+}
+
 } /* namespace cattle_hip */
 
 using namespace cattle_hip;
@@ -1397,7 +1452,10 @@ const char* cattle_hip_last_error(void) {
 }
 
 int cattle_hip_synchronize(void) {
-	return guarded([&] { CATTLE_HIP_CHECK(hipStreamSynchronize(stream())); });
+	return guarded([&] {
+		forbid_while_capturing("waiting for the device");
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+	});
 }
 
 int cattle_hip_alloc(void** device_ptr, size_t bytes) {
@@ -1416,6 +1474,7 @@ int cattle_hip_free(void* device_ptr) {
 
 int cattle_hip_trim(void) {
 	return guarded([&] {
+		forbid_while_capturing("waiting for the device");
 		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
 		g_pool.trim();
 	});
@@ -1424,6 +1483,7 @@ int cattle_hip_trim(void) {
 int cattle_hip_memory_info(size_t* free_bytes, size_t* total_bytes) {
 	return guarded([&] {
 		CATTLE_HIP_REQUIRE(free_bytes != nullptr && total_bytes != nullptr, "null output pointer");
+		forbid_while_capturing("waiting for the device");
 		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
 		CATTLE_HIP_CHECK(hipMemGetInfo(free_bytes, total_bytes));
 	});
@@ -1474,6 +1534,7 @@ int cattle_hip_timer_destroy(cattle_hip_timer_t timer) {
 int cattle_hip_timer_start(cattle_hip_timer_t timer) {
 	return guarded([&] {
 		CATTLE_HIP_REQUIRE(timer != nullptr, "null timer");
+		forbid_while_capturing("timing");
 		CATTLE_HIP_CHECK(hipEventRecord(reinterpret_cast<Timer*>(timer)->start, stream()));
 	});
 }
@@ -1482,9 +1543,70 @@ int cattle_hip_timer_stop(cattle_hip_timer_t timer, float* elapsed_ms) {
 	return guarded([&] {
 		CATTLE_HIP_REQUIRE(timer != nullptr && elapsed_ms != nullptr, "null timer or output");
 		Timer* t = reinterpret_cast<Timer*>(timer);
+		forbid_while_capturing("timing");
 		CATTLE_HIP_CHECK(hipEventRecord(t->stop, stream()));
 		CATTLE_HIP_CHECK(hipEventSynchronize(t->stop));
 		CATTLE_HIP_CHECK(hipEventElapsedTime(elapsed_ms, t->start, t->stop));
+	});
+}
+
+int cattle_hip_graph_begin_capture(void) {
+	return guarded([&] {
+		if (g_capturing)
+			throw Error(ERR_STATE, "a graph is already being recorded");
+		CATTLE_HIP_CHECK(hipStreamBeginCapture(stream(), hipStreamCaptureModeRelaxed));
+		g_capturing = true;
+	});
+}
+
+int cattle_hip_graph_end_capture(cattle_hip_graph_t* graph) {
+	return guarded([&] {
+		if (!g_capturing)
+			throw Error(ERR_STATE, "no graph is being recorded");
+		g_capturing = false;
+		std::unique_ptr<Graph> gr(new Graph());
+		/* blocks freed during the recording stay out of circulation, whatever becomes of the graph */
+		gr->blocks.swap(g_pool.held);
+		for (void* b : g_pool.taken)
+			g_pool.owner[b] = &gr->blocks;
+		g_pool.taken.clear();
+		hipError_t e = hipStreamEndCapture(stream(), &gr->graph);
+		if (e == hipSuccess && gr->graph != nullptr)
+			e = hipGraphInstantiate(&gr->exec, gr->graph, nullptr, nullptr, 0);
+		if (e != hipSuccess || gr->graph == nullptr || graph == nullptr) {
+			if (gr->exec)
+				(void) hipGraphExecDestroy(gr->exec);
+			if (gr->graph)
+				(void) hipGraphDestroy(gr->graph);
+			(void) hipGetLastError();
+			g_pool.release_graph(&gr->blocks);
+			if (graph == nullptr)
+				throw Error(ERR_INVALID, "null output pointer");
+			throw Error(ERR_DEVICE, std::string("the recording could not be turned into a graph: ") + hipGetErrorString(e));
+		}
+		*graph = reinterpret_cast<cattle_hip_graph_t>(gr.release());
+	});
+}
+
+int cattle_hip_graph_launch(cattle_hip_graph_t graph) {
+	return guarded([&] {
+		CATTLE_HIP_REQUIRE(graph != nullptr, "null graph handle");
+		forbid_while_capturing("launching a graph");
+		CATTLE_HIP_CHECK(hipGraphLaunch(reinterpret_cast<Graph*>(graph)->exec, stream()));
+	});
+}
+
+int cattle_hip_graph_destroy(cattle_hip_graph_t graph) {
+	return guarded([&] {
+		if (!graph)
+			return;
+		forbid_while_capturing("destroying a graph");
+		Graph* gr = reinterpret_cast<Graph*>(graph);
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+		(void) hipGraphExecDestroy(gr->exec);
+		(void) hipGraphDestroy(gr->graph);
+		g_pool.release_graph(&gr->blocks);
+		delete gr;
 	});
 }
 
@@ -1918,7 +2040,8 @@ int cattle_hip_layer_clone(cattle_hip_layer_t layer, int share_params, cattle_hi
 int cattle_hip_layer_destroy(cattle_hip_layer_t layer) {
 	return guarded([&] {
 		if (layer) {
-			CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+			forbid_while_capturing("waiting for the device");
+		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
 			delete reinterpret_cast<LayerBase*>(layer);
 		}
 	});
@@ -1951,6 +2074,7 @@ int cattle_hip_layer_set_input_layer(cattle_hip_layer_t layer, int is_input_laye
 
 int cattle_hip_layer_empty_cache(cattle_hip_layer_t layer) {
 	return guarded([&] {
+		forbid_while_capturing("waiting for the device");
 		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
 		as_layer(layer)->empty_cache();
 	});

@@ -86,7 +86,7 @@ int main(int argc, char** argv) {
 		check(cattle_hip_init(0));
 		DeviceLoss<Scalar> loss(CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY);
 		Lcg g(2);
-		double mlp_ms, conv_ms, cifar_ms, mlp_fused_ms, conv_fused_ms, cifar_fused_ms;
+		double mlp_ms, conv_ms, cifar_ms, mlp_fused_ms, conv_fused_ms, cifar_fused_ms, mlp_rec_ms, conv_rec_ms;
 		{
 			/* MLP 784-512-256-10 with ReLU, batch 256, vanilla SGD */
 			const std::size_t batch = 256;
@@ -104,6 +104,10 @@ int main(int argc, char** argv) {
 			/* the same network with each dense layer and its ReLU run as one fused layer */
 			net.fuse();
 			mlp_fused_ms = time_steps(steps, warmup, [&](std::size_t) { net.train_batch_sgd(xd, yd, loss, (Scalar) 1e-3); });
+			/* the fused step recorded once and launched as a graph: one call instead of fourteen before the loss is read back */
+			DeviceFeedforwardNetwork<Scalar>::RecordedBatch rec = net.record_batch(xd, yd, loss);
+			const double sgd[4] = { 1e-3, 0, 0, 0 };
+			mlp_rec_ms = time_steps(steps, warmup, [&](std::size_t) { rec.run(CATTLE_HIP_OPT_VANILLA_SGD, sgd, 0, 0); });
 		}
 		{
 			/* conv 3x3x32 - ReLU - max pool - conv 3x3x64 - batch norm - ReLU - max pool - dense 10, batch 128, Adam */
@@ -125,6 +129,9 @@ int main(int argc, char** argv) {
 			/* conv-ReLU-pool and conv-BN-ReLU-pool as fused layers */
 			net.fuse();
 			conv_fused_ms = time_steps(steps, warmup, [&](std::size_t t) { net.train_batch_adam(xd, yd, loss, steps + warmup + t); });
+			DeviceFeedforwardNetwork<Scalar>::RecordedBatch rec = net.record_batch(xd, yd, loss);
+			const double adam[4] = { 1e-3, 1e-1, 1e-3, 1e-5 };
+			conv_rec_ms = time_steps(steps, warmup, [&](std::size_t t) { rec.run(CATTLE_HIP_OPT_ADAM, adam, 0, 2 * (steps + warmup) + t); });
 		}
 		{
 			/* examples/cifar_convnet.cpp:24-41: conv 3x3x8 - ReLU - max pool - conv 3x3x8 - ReLU - max pool - dropout .25 -
@@ -169,8 +176,9 @@ int main(int argc, char** argv) {
 		std::printf("{\"driver\": \"C++ (cattle_hip/DeviceNet.hpp), train_batch* incl. the per-batch loss read-back\", "
 				"\"steps\": %zu, \"warmup\": %zu, \"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, \"convnet_32x32x3_batch128_adam_ms\": %.4f, "
 				"\"reference_cifar_example_batch200_nadam_ms\": %.4f, \"fused\": {\"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, "
-				"\"convnet_32x32x3_batch128_adam_ms\": %.4f, \"reference_cifar_example_batch200_nadam_ms\": %.4f}}\n", steps, warmup, mlp_ms,
-				conv_ms, cifar_ms, mlp_fused_ms, conv_fused_ms, cifar_fused_ms);
+				"\"convnet_32x32x3_batch128_adam_ms\": %.4f, \"reference_cifar_example_batch200_nadam_ms\": %.4f}, "
+				"\"fused_and_recorded_as_hip_graph\": {\"mlp_784_512_256_10_batch256_sgd_ms\": %.4f, \"convnet_32x32x3_batch128_adam_ms\": %.4f}}\n",
+				steps, warmup, mlp_ms, conv_ms, cifar_ms, mlp_fused_ms, conv_fused_ms, cifar_fused_ms, mlp_rec_ms, conv_rec_ms);
 	} catch (const std::exception& e) {
 		std::fprintf(stderr, "train_steps: %s\n", e.what());
 		return 1;

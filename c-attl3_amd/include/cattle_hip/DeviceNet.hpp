@@ -609,6 +609,12 @@ public:
 		return losses;
 	}
 	/** scale * d_function; scale = 1 / batch_size is the optimizer's division (optimizer/SGDOptimizer.hpp:54-55). */
+	/** The same values left on the device: `losses` holds one scalar per sample (dims { batch, 1, 1, 1 }). */
+	inline void function_into(const DeviceTensor<Scalar>& out, const DeviceTensor<Scalar>& obj, DeviceTensor<Scalar>& losses) const {
+		assert(out.dimensions() == obj.dimensions() && losses.size() == out.batch());
+		check(cattle_hip_loss_function(Code<Scalar>::value, kind, out.data(), CATTLE_HIP_DEVICE, obj.data(), CATTLE_HIP_DEVICE,
+				out.batch(), 1, out.size() / out.batch(), (double) epsilon, losses.data(), CATTLE_HIP_DEVICE));
+	}
 	inline DeviceTensor<Scalar> d_function(const DeviceTensor<Scalar>& out, const DeviceTensor<Scalar>& obj,
 			Scalar scale = 1) const {
 		assert(out.dimensions() == obj.dimensions());
@@ -621,6 +627,39 @@ public:
 private:
 	cattle_hip_loss kind;
 	Scalar epsilon;
+};
+
+/**
+ * A recorded sequence of device-side calls (cattle_hip_graph_*): what is issued between begin() and end() is recorded
+ * instead of run, and launch() runs it as one HIP graph. The calls must have run once before, must use device tensors
+ * only and must read nothing back; tensors that were created during the recording stay allocated until the graph goes.
+ */
+class DeviceGraph {
+public:
+	inline DeviceGraph() : handle(nullptr) { }
+	DeviceGraph(const DeviceGraph&) = delete;
+	DeviceGraph& operator=(const DeviceGraph&) = delete;
+	inline DeviceGraph(DeviceGraph&& other) : handle(other.handle) {
+		other.handle = nullptr;
+	}
+	inline ~DeviceGraph() {
+		if (handle)
+			cattle_hip_graph_destroy(handle);
+	}
+	inline void begin() {
+		check(cattle_hip_graph_begin_capture());
+	}
+	inline void end() {
+		check(cattle_hip_graph_end_capture(&handle));
+	}
+	inline void launch() const {
+		check(cattle_hip_graph_launch(handle));
+	}
+	inline bool is_recorded() const {
+		return handle != nullptr;
+	}
+private:
+	cattle_hip_graph_t handle;
 };
 
 /**
@@ -822,6 +861,48 @@ public:
 		const double hyper[4] = { (double) learning_rate, (double) l1_decay, (double) l2_decay, (double) epsilon };
 		optimizer_step(CATTLE_HIP_OPT_ADAM, hyper, 0, timestep);
 		return total;
+	}
+	/**
+	 * One batch of SGDOptimizer::_train on fixed tensors, recorded once and repeated by every run(): propagate, the loss
+	 * of every sample, its gradient / batch size, backpropagate as one graph launch, then the optimizer step (outside the
+	 * graph: its scalars, the time step for one, change from batch to batch) and the read-back of the losses. The caller
+	 * refills `input` and `obj` in place between runs. Call train_batch once on the same tensors first, so that every
+	 * buffer of the layers exists when the recording starts.
+	 */
+	class RecordedBatch {
+	public:
+		inline Scalar run(cattle_hip_optimizer optimizer, const double (&hyper)[4], std::size_t epoch, std::size_t timestep) {
+			graph.launch();
+			net->optimizer_step(optimizer, hyper, epoch, timestep);
+			const std::vector<Scalar> host = losses.to_host();
+			Scalar total = 0;
+			for (std::size_t i = 0; i < host.size(); ++i)
+				total += host[i];
+			return total;
+		}
+	private:
+		friend class DeviceFeedforwardNetwork;
+		inline RecordedBatch(DeviceFeedforwardNetwork* net, std::size_t batch) : net(net),
+				losses(typename DeviceTensor<Scalar>::Dims{ { batch, 1, 1, 1 } }) { }
+		DeviceFeedforwardNetwork* net;
+		DeviceTensor<Scalar> losses;
+		DeviceGraph graph;
+	};
+	inline RecordedBatch record_batch(const DeviceTensor<Scalar>& input, const DeviceTensor<Scalar>& obj, const DeviceLoss<Scalar>& loss) {
+		RecordedBatch rec(this, input.batch());
+		rec.graph.begin();
+		try {
+			const DeviceTensor<Scalar>& out = propagate(input, true);
+			loss.function_into(out, obj, rec.losses);
+			backpropagate(loss.d_function(out, obj, (Scalar) 1 / (Scalar) input.batch()));
+		} catch (...) {
+			cattle_hip_graph_t dropped = nullptr;
+			if (cattle_hip_graph_end_capture(&dropped) == CATTLE_HIP_OK)
+				cattle_hip_graph_destroy(dropped);
+			throw;
+		}
+		rec.graph.end();
+		return rec;
 	}
 	/**
 	 * The update of every optimizable parameter of the network followed by its reset_grad

@@ -29,6 +29,7 @@ extern "C" {
 
 typedef struct cattle_hip_layer_s* cattle_hip_layer_t;
 typedef struct cattle_hip_timer_s* cattle_hip_timer_t;
+typedef struct cattle_hip_graph_s* cattle_hip_graph_t;
 
 enum {
 	CATTLE_HIP_OK = 0,
@@ -88,6 +89,25 @@ int cattle_hip_timer_start(cattle_hip_timer_t timer);
 int cattle_hip_timer_stop(cattle_hip_timer_t timer, float* elapsed_ms);   /* synchronises */
 
 /* ---- layer construction ------------------------------------------------------------------ */
+
+/* ---- recorded steps (no counterpart in the reference, whose training loop calls the layers anew for every batch:
+ * optimizer/SGDOptimizer.hpp:44-70) -----------------------------------------------------------------------------------
+ * Between cattle_hip_graph_begin_capture and cattle_hip_graph_end_capture the library's calls are recorded instead of
+ * run: layer passes, loss gradients, optimizer steps on device-resident parameters, on DEVICE buffers only. What was
+ * recorded runs, as one HIP graph, at every cattle_hip_graph_launch: a training step of twenty small kernels then costs
+ * the host one call, which matters to a loop that reads the loss back after every batch. Rules:
+ *  - run the same calls once, eagerly, first: buffers that a layer would have to allocate or grow, host copies, waits
+ *    (cattle_hip_synchronize, _download, _layer_empty_cache, timers) return CATTLE_HIP_ERR_STATE while recording;
+ *  - a launch repeats the recorded kernels with the recorded arguments: the same buffers (the caller's inputs, whatever
+ *    cattle_hip_alloc returned during the recording; cattle_hip_free on them takes effect when the graph is destroyed),
+ *    the same batch size, and the same scalars - an optimizer whose update depends on the time step or epoch (Adam,
+ *    Nadam, AMSGrad, ...) is therefore called outside the recording, as is anything whose result the host must see;
+ *  - layers that took part, and their caches, must be left alone while launches of the graph are in flight, and
+ *    destroyed only after the graph. */
+int cattle_hip_graph_begin_capture(void);
+int cattle_hip_graph_end_capture(cattle_hip_graph_t* graph);
+int cattle_hip_graph_launch(cattle_hip_graph_t graph);
+int cattle_hip_graph_destroy(cattle_hip_graph_t graph);
 
 /* ConvKernelLayer<Scalar,Rank>(input_dims, filters, init, receptor_height, receptor_width,
  * vertical_padding, horizontal_padding, vertical_stride, horizontal_stride, vertical_dilation,

@@ -108,8 +108,8 @@ static void run(const std::string& tag) {
 	const std::size_t steps = 3;
 	DeviceLoss<Scalar> loss(CATTLE_HIP_LOSS_SOFTMAX_CROSS_ENTROPY);
 	/* each of the two trained networks once layer by layer and once with DeviceFeedforwardNetwork::fuse() (records "...f") */
-	for (int fused = 0; fused < 2; ++fused) {
-		const std::string mlp = tag + (fused ? ".mlpf" : ".mlp");
+	for (int fused = 0; fused < 3; ++fused) {        /* 2: fused, and all batches after the first recorded once and launched as a graph ("...g") */
+		const std::string mlp = tag + (fused == 2 ? ".mlpg" : fused ? ".mlpf" : ".mlp");
 		Lcg g(11);
 		const std::size_t batch = 24;
 		std::vector<DL> layers;
@@ -127,8 +127,16 @@ static void run(const std::string& tag) {
 		record(mlp + ".y", sizeof(Scalar), { batch, 6 }, y.data());
 		DT xd(typename DT::Dims{ { batch, 20, 1, 1 } }, x.data()), yd(typename DT::Dims{ { batch, 6, 1, 1 } }, y.data());
 		std::vector<Scalar> totals;
-		for (std::size_t t = 0; t < steps; ++t)
+		if (fused == 2) {
 			totals.push_back(net.train_batch_sgd(xd, yd, loss, (Scalar) 0.05));
+			typename DeviceFeedforwardNetwork<Scalar>::RecordedBatch rec = net.record_batch(xd, yd, loss);
+			const double sgd[4] = { (double) (Scalar) 0.05, 0, 0, 0 };
+			for (std::size_t t = 1; t < steps; ++t)
+				totals.push_back(rec.run(CATTLE_HIP_OPT_VANILLA_SGD, sgd, 0, 0));
+		} else {
+			for (std::size_t t = 0; t < steps; ++t)
+				totals.push_back(net.train_batch_sgd(xd, yd, loss, (Scalar) 0.05));
+		}
 		record(mlp + ".losses", sizeof(Scalar), { steps }, totals.data());
 		record_final<Scalar>(mlp, net);
 	}

@@ -120,11 +120,11 @@ def test_device_loss_of_another_kind_negated(records, tag, tol):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["mlp", "mlpf"])       # layer by layer, and with DeviceFeedforwardNetwork::fuse()
+@pytest.mark.parametrize("name", ["mlp", "mlpf", "mlpg"])       # layer by layer, with DeviceFeedforwardNetwork::fuse(), and recorded as a graph
 @pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-9)])
 def test_mlp_sgd_batches(records, tag, tol, name):
     r = {k[len(tag) + len(name) + 2:]: v for k, v in records.items() if k.startswith(tag + "." + name + ".")}
-    if name == "mlpf":
+    if name != "mlp":
         assert r["groups"][0] == 1                      # dense + ReLU
     be = hn.OracleBackend(np.float64)
     net = hn.FeedforwardNet([be.dense((20,), 16), be.act("relu", (16,)), be.dense((16,), 6)])
