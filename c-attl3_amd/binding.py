@@ -44,7 +44,7 @@ EXPORTS = [
     "cattle_hip_convlstm_backpropagate", "cattle_hip_convlstm_set_kernel_values", "cattle_hip_convlstm_get_kernel_values",
     "cattle_hip_convlstm_get_kernel_grad", "cattle_hip_conv_forward_noalloc", "cattle_hip_static_scratch_bytes",
     "cattle_hip_fused_create", "cattle_hip_fused_last_mode", "cattle_hip_graph_begin_capture", "cattle_hip_graph_end_capture",
-    "cattle_hip_graph_launch", "cattle_hip_graph_destroy",
+    "cattle_hip_graph_launch", "cattle_hip_graph_destroy", "cattle_hip_layer_param_set_constraints",
 ]
 
 
@@ -243,6 +243,12 @@ class Parameters(object):
         (parameter_regularization/*.hpp); optimizer_step then regularizes before it updates."""
         _check(lib().cattle_hip_layer_param_set_regularization(self._layer._h, _sz(self._index), ctypes.c_double(l1_lambda),
                                                                ctypes.c_double(l2_lambda)))
+
+    def set_constraints(self, value_clip=0.0, value_max_l1_norm=0.0, value_max_l2_norm=0.0, grad_clip=0.0, grad_max_l1_norm=0.0,
+                        grad_max_l2_norm=0.0):
+        """The constraints of parameters/StandardParameters.hpp:61-76 on device-resident parameters; 0 = off."""
+        _check(lib().cattle_hip_layer_param_set_constraints(self._layer._h, _sz(self._index), *[ctypes.c_double(v) for v in (
+            value_clip, value_max_l1_norm, value_max_l2_norm, grad_clip, grad_max_l1_norm, grad_max_l2_norm)]))
 
     def get_regularization_penalty(self):
         """Parameters::get_regularization_penalty (parameters/StandardParameters.hpp:128-132)."""

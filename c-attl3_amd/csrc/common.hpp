@@ -249,6 +249,11 @@ template<typename T> void optimizer_update(int rule, const double hyper[4], size
 		T* grad, T* s0, T* s1, T* s2, T* values, bool reset_grad, T l1, T l2);
 /* sums[0] = sum |v|, sums[1] = sum v^2 over a parameter's n values (device pointers) */
 template<typename T> void regularization_sums(size_t n, const T* values, T* sums);
+/* The clip, "L1" and "L2" norm constraints of StandardParameters (:150-182) on a matrix of n values, in that order; a
+ * limit of zero is off. */
+template<typename T> void constrain_matrix(size_t n, T* m, double clip, double max_l1, double max_l2);
+/* grad += the regularization's d_function at the values (Parameters::regularize) */
+template<typename T> void add_regularization(size_t n, const T* values, T* grad, T l1, T l2);
 
 } /* namespace cattle_hip */
 

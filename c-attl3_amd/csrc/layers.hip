@@ -219,6 +219,14 @@ struct Param {
 	DevBuf moments[3];                 /* the optimizer's state matrices, allocated (zeroed) on first use */
 	int moments_ready = 0;             /* how many of them are */
 	double reg_l1 = 0, reg_l2 = 0;     /* ParameterRegularization of the parameter: L1 and L2 lambdas (both 0: none) */
+	/* the constraints of StandardParameters (:63-64): clip, max "L1" norm, max "L2" norm of the values and of the gradient; 0 = off */
+	double value_limits[3] = { 0, 0, 0 }, grad_limits[3] = { 0, 0, 0 };
+	bool constrains_values() const {
+		return value_limits[0] > 0 || value_limits[1] > 0 || value_limits[2] > 0;
+	}
+	bool constrains_grad() const {
+		return grad_limits[0] > 0 || grad_limits[1] > 0 || grad_limits[2] > 0;
+	}
 	Param(size_t rows, size_t cols, bool optimizable, size_t esize) : rows(rows), cols(cols), optimizable(optimizable), esize(esize) {
 		values.ensure(bytes());
 		grad.ensure(bytes());
@@ -234,6 +242,8 @@ struct Param {
 		copy_in(c->grad.p, grad.p, CATTLE_HIP_DEVICE, bytes());
 		c->reg_l1 = reg_l1;
 		c->reg_l2 = reg_l2;
+		std::memcpy(c->value_limits, value_limits, sizeof(value_limits));
+		std::memcpy(c->grad_limits, grad_limits, sizeof(grad_limits));
 		return c;
 	}
 };
@@ -245,6 +255,17 @@ void fill_constant(Param& p, T v) {
 	std::vector<T> host(p.rows * p.cols, v);
 	copy_in(p.values.p, host.data(), CATTLE_HIP_HOST, p.bytes());
 	++p.version;
+}
+
+/* enforce_clip_constraint, enforce_l1_norm_constraint, enforce_l2_norm_constraint on the values (set_values,
+ * StandardParameters.hpp:105-112) or on the gradient (accumulate_grad, :114-123) */
+void constrain(Param& p, bool values) {
+	const double* lim = values ? p.value_limits : p.grad_limits;
+	void* m = values ? p.values.p : p.grad.p;
+	if (p.esize == sizeof(float))
+		constrain_matrix<float>(p.rows * p.cols, static_cast<float*>(m), lim[0], lim[1], lim[2]);
+	else
+		constrain_matrix<double>(p.rows * p.cols, static_cast<double*>(m), lim[0], lim[1], lim[2]);
 }
 
 struct LayerBase {
@@ -1289,7 +1310,16 @@ void run_optimizer(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer 
 	}
 	const size_t n = p.rows * p.cols;
 	/* the step form is SGDOptimizer::_train's regularize + update + reset; the plain update is _update_params alone */
-	const double l1 = reset_grad ? p.reg_l1 : 0, l2 = reset_grad ? p.reg_l2 : 0;
+	double l1 = reset_grad ? p.reg_l1 : 0, l2 = reset_grad ? p.reg_l2 : 0;
+	if (p.constrains_grad() && (l1 != 0 || l2 != 0)) {
+		/* Parameters::regularize is an accumulate_grad: the constraints apply to gradient + regularization */
+		if (p.esize == sizeof(float))
+			add_regularization<float>(n, static_cast<const float*>(p.values.p), static_cast<float*>(p.grad.p), (float) l1, (float) l2);
+		else
+			add_regularization<double>(n, static_cast<const double*>(p.values.p), static_cast<double*>(p.grad.p), l1, l2);
+		constrain(p, false);
+		l1 = l2 = 0;
+	}
 	if (p.esize == sizeof(float))
 		optimizer_update<float>((int) optimizer, hyper, epoch, timestep, n, static_cast<float*>(p.grad.p),
 				static_cast<float*>(p.moments[0].p), static_cast<float*>(p.moments[1].p), static_cast<float*>(p.moments[2].p),
@@ -1298,6 +1328,8 @@ void run_optimizer(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer 
 		optimizer_update<double>((int) optimizer, hyper, epoch, timestep, n, static_cast<double*>(p.grad.p),
 				static_cast<double*>(p.moments[0].p), static_cast<double*>(p.moments[1].p),
 				static_cast<double*>(p.moments[2].p), static_cast<double*>(p.values.p), reset_grad, l1, l2);
+	if (p.constrains_values())
+		constrain(p, true);              /* the optimizers hand the new values to set_values */
 	++p.version;
 }
 
@@ -1308,7 +1340,7 @@ template<typename T>
 void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices, size_t count, cattle_hip_optimizer optimizer,
 		const double hyper[4], size_t epoch, size_t timestep) {
 	const int states = optimizer_state_count((int) optimizer);
-	std::vector<Param*> seen;
+	std::vector<Param*> seen, limited;
 	OptBatch<T> batch;
 	batch.count = 0;
 	auto flush = [&] {
@@ -1334,12 +1366,19 @@ void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices,
 		q.n = p.rows * p.cols;
 		q.l1 = (T) p.reg_l1;
 		q.l2 = (T) p.reg_l2;
+		if (p.constrains_grad() && (p.reg_l1 != 0 || p.reg_l2 != 0)) {
+			add_regularization<T>(p.rows * p.cols, static_cast<const T*>(p.values.p), static_cast<T*>(p.grad.p), q.l1, q.l2);
+			constrain(p, false);
+			q.l1 = q.l2 = (T) 0;
+		}
 		q.wt_fwd = q.wt_dgrad = nullptr;
 		q.K = q.RHW = 1;
 		q.ldw_fwd = q.ldw_dgrad = 0;
 		const ConvLayer<T>* conv = dynamic_cast<const ConvLayer<T>*>(as_layer(layers[i]));
 		bool fwd_current = false, dgrad_current = false;
-		if (conv && indices[i] == 0) {
+		if (p.constrains_values()) {
+			limited.push_back(&p);         /* constrained after the update; the prepared layouts are rebuilt from the result */
+		} else if (conv && indices[i] == 0) {
 			const ConvShape& cs = conv->shape;
 			fwd_current = p.derived[0].p && p.derived_version[0] == p.version;
 			dgrad_current = p.derived[1].p && p.derived_version[1] == p.version;
@@ -1361,6 +1400,8 @@ void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices,
 			flush();
 	}
 	flush();
+	for (Param* p : limited)
+		constrain(*p, true);
 }
 
 
@@ -2129,6 +2170,10 @@ int cattle_hip_layer_backward(cattle_hip_layer_t layer, const void* out_grad, ca
 		if (want_in_grad)
 			ig_dev = in_grad_space == CATTLE_HIP_HOST ? l->ig_stage.ensure(in_bytes) : in_grad;
 		l->backward(og_dev, batch, ig_dev);
+		/* accumulate_grad enforces the gradient's constraints after every accumulation (StandardParameters.hpp:119-122) */
+		for (const ParamPtr& q : l->params)
+			if (q->optimizable && q->constrains_grad())
+				constrain(*q, false);
 		if (want_in_grad && in_grad_space == CATTLE_HIP_HOST)
 			copy_out(in_grad, CATTLE_HIP_HOST, ig_dev, in_bytes);
 	});
@@ -2159,6 +2204,8 @@ int cattle_hip_layer_set_param_values(cattle_hip_layer_t layer, size_t index, co
 		CATTLE_HIP_REQUIRE(values != nullptr, "null buffer");
 		Param& p = param_at(as_layer(layer), index);
 		copy_in(p.values.p, values, space, p.bytes());
+		if (p.constrains_values())
+			constrain(p, true);
 		++p.version;
 	});
 }
@@ -2222,6 +2269,25 @@ int cattle_hip_layer_param_set_regularization(cattle_hip_layer_t layer, size_t i
 		CATTLE_HIP_REQUIRE(l1_lambda == l1_lambda && l2_lambda == l2_lambda, "lambda is not a number");
 		p.reg_l1 = l1_lambda;
 		p.reg_l2 = l2_lambda;
+	});
+}
+
+int cattle_hip_layer_param_set_constraints(cattle_hip_layer_t layer, size_t index, double value_clip, double value_max_l1_norm,
+		double value_max_l2_norm, double grad_clip, double grad_max_l1_norm, double grad_max_l2_norm) {
+	return guarded([&] {
+		LayerBase* l = as_layer(layer);
+		Param& p = param_at(l, index);
+		const double v[6] = { value_clip, value_max_l1_norm, value_max_l2_norm, grad_clip, grad_max_l1_norm, grad_max_l2_norm };
+		for (int i = 0; i < 6; ++i)
+			CATTLE_HIP_REQUIRE(v[i] == v[i], "a limit is not a number");
+		CATTLE_HIP_REQUIRE(dynamic_cast<ConvLstm<float>*>(l) == nullptr && dynamic_cast<ConvLstm<double>*>(l) == nullptr,
+				"the fused LSTM accumulates the gradients of all time steps at once: constraints per accumulation cannot be enforced");
+		std::memcpy(p.value_limits, v, sizeof(p.value_limits));
+		std::memcpy(p.grad_limits, v + 3, sizeof(p.grad_limits));
+		if (p.constrains_values()) {
+			constrain(p, true);
+			++p.version;
+		}
 	});
 }
 

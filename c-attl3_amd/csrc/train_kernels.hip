@@ -10,6 +10,8 @@
  */
 #include "common.hpp"
 
+#include <limits>
+
 namespace cattle_hip {
 
 namespace {
@@ -373,6 +375,69 @@ void regularization_sums_kernel(size_t n, const T* __restrict__ values, T* __res
 	}
 }
 
+/* The constraints of a Parameters object on its values or on its gradient (parameters/StandardParameters.hpp:150-182),
+ * in the order set_values and accumulate_grad enforce them (:109-111, :120-122): clip to [-clip, clip], then scale by
+ * max_l1 / norm() where the norm() - the Euclidean norm: that is what the "L1" constraint calls - exceeds max_l1, then
+ * scale by max_l2 / squaredNorm() where the squared norm (what the "L2" constraint compares with its limit) exceeds
+ * max_l2. A limit that is not decidedly greater than zero is off. One block: the sums are taken thread by thread in a
+ * fixed order, then by a fixed tree, so the result is reproducible. */
+template<typename T>
+__device__ __forceinline__ T block_sum_of_squares(size_t n, const T* m, T (&part)[256]) {
+	T q = (T) 0;
+	for (size_t i = threadIdx.x; i < n; i += 256)
+		q += m[i] * m[i];
+	part[threadIdx.x] = q;
+	__syncthreads();
+	for (int w = 128; w > 0; w >>= 1) {
+		if ((int) threadIdx.x < w)
+			part[threadIdx.x] += part[threadIdx.x + w];
+		__syncthreads();
+	}
+	const T total = part[0];
+	__syncthreads();
+	return total;
+}
+
+template<typename T>
+__global__ __launch_bounds__(256)
+void constrain_kernel(size_t n, T* __restrict__ m, T clip, T max_l1, T max_l2) {
+	__shared__ T part[256];
+	if (clip > (T) 0) {
+		for (size_t i = threadIdx.x; i < n; i += 256) {
+			const T v = m[i];
+			m[i] = v > clip ? clip : (v < -clip ? -clip : v);
+		}
+		__syncthreads();
+	}
+	if (max_l1 > (T) 0) {
+		const T norm = dev_sqrt(block_sum_of_squares<T>(n, m, part));
+		if (norm > max_l1) {
+			const T scale = max_l1 / norm;
+			for (size_t i = threadIdx.x; i < n; i += 256)
+				m[i] *= scale;
+		}
+		__syncthreads();
+	}
+	if (max_l2 > (T) 0) {
+		const T sq = block_sum_of_squares<T>(n, m, part);
+		if (sq > max_l2) {
+			const T scale = max_l2 / sq;
+			for (size_t i = threadIdx.x; i < n; i += 256)
+				m[i] *= scale;
+		}
+	}
+}
+
+/* grad += d_function of the regularization at the values: Parameters::regularize as a step of its own, for parameters
+ * whose gradient is constrained (the constraints apply to the sum, StandardParameters.hpp:133-136 through :114-123). */
+template<typename T>
+__global__ __launch_bounds__(256)
+void add_regularization_kernel(size_t n, const T* __restrict__ values, T* __restrict__ grad, T l1, T l2) {
+	const size_t stride = (size_t) gridDim.x * blockDim.x;
+	for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+		grad[i] = regularized_gradient(grad[i], values[i], l1, l2);
+}
+
 /* The update and gradient reset of up to OPT_BATCH parameters in one launch (blockIdx.y picks the parameter,
  * blockIdx.x a run of 1024 elements, or a 32 x 32 tile of the matrix). A convolution or dense weight matrix may
  * bring its prepared layouts along (the forward layout wt[k][f] and the input-gradient layout wd[tap + RHW * f][c],
@@ -609,6 +674,30 @@ void regularization_sums(size_t n, const T* values, T* sums) {
 	check_launch();
 }
 
+/* NumericUtils::decidedly_greater(limit, 0) with its default epsilons (core/NumericUtils.hpp:42-65) */
+template<typename T>
+T active_limit(double limit) {
+	const T l = (T) limit;
+	return l > std::numeric_limits<T>::epsilon() ? l : (T) 0;
+}
+
+template<typename T>
+void constrain_matrix(size_t n, T* m, double clip, double max_l1, double max_l2) {
+	const T c = active_limit<T>(clip), a = active_limit<T>(max_l1), b = active_limit<T>(max_l2);
+	if (n == 0 || (c == (T) 0 && a == (T) 0 && b == (T) 0))
+		return;
+	constrain_kernel<T><<<1, 256, 0, stream()>>>(n, m, c, a, b);
+	check_launch();
+}
+
+template<typename T>
+void add_regularization(size_t n, const T* values, T* grad, T l1, T l2) {
+	if (n == 0 || (l1 == (T) 0 && l2 == (T) 0))
+		return;
+	add_regularization_kernel<T><<<flat_grid(n), 256, 0, stream()>>>(n, values, grad, l1, l2);
+	check_launch();
+}
+
 template<typename T>
 void optimizer_update(int rule, const double hyper[4], size_t epoch, size_t timestep, size_t n, T* grad, T* s0, T* s1,
 		T* s2, T* values, bool reset_grad, T l1, T l2) {
@@ -649,6 +738,8 @@ template void loss_function<T>(int, int, int, int, T, const T*, const T*, T*); \
 template void loss_d_function<T>(int, int, int, int, T, T, const T*, const T*, T*); \
 template void optimizer_update<T>(int, const double*, size_t, size_t, size_t, T*, T*, T*, T*, T*, bool, T, T); \
 template void regularization_sums<T>(size_t, const T*, T*); \
+template void constrain_matrix<T>(size_t, T*, double, double, double); \
+template void add_regularization<T>(size_t, const T*, T*, T, T); \
 template void optimizer_step_many<T>(int, const double*, size_t, size_t, const OptBatch<T>&);
 
 CATTLE_HIP_INSTANTIATE_TRAIN(float)

@@ -362,6 +362,15 @@ int cattle_hip_layer_param_adam_update(cattle_hip_layer_t layer, size_t index, d
  * does through Parameters::regularize (optimizer/SGDOptimizer.hpp:59-63, StandardParameters.hpp:133-136);
  * cattle_hip_layer_param_optimizer_update, which is _update_params alone, does not. */
 int cattle_hip_layer_param_set_regularization(cattle_hip_layer_t layer, size_t index, double l1_lambda, double l2_lambda);
+/* The value and gradient constraints of a Parameters object (the weight_clip, weight_max_l1_norm, ... bias_grad_max_l2_norm
+ * constructor arguments of the kernel layers, parameters/StandardParameters.hpp:61-76), for parameters that stay on the
+ * device; 0 switches a limit off. As in the reference (:105-123, :150-182): the values are constrained whenever they are
+ * set (cattle_hip_layer_set_param_values, every optimizer update), the gradient after every accumulation (every
+ * cattle_hip_layer_backward of a layer that holds the parameter, and the regularization term of an optimizer step), each
+ * time in the order clip to [-clip, clip], scale by max_l1 / norm() if the Euclidean norm - which is what the reference's
+ * "L1" constraint measures - exceeds max_l1, scale by max_l2 / squaredNorm() if the squared norm exceeds max_l2. */
+int cattle_hip_layer_param_set_constraints(cattle_hip_layer_t layer, size_t index, double value_clip, double value_max_l1_norm,
+		double value_max_l2_norm, double grad_clip, double grad_max_l1_norm, double grad_max_l2_norm);
 /* Parameters::get_regularization_penalty (StandardParameters.hpp:128-132): l1 * sum |v| + 0.5 * l2 * sum v^2, 0 for
  * parameters without regularization or that are not optimizable. */
 int cattle_hip_layer_param_regularization_penalty(cattle_hip_layer_t layer, size_t index, double* penalty);

@@ -413,6 +413,35 @@ def regularization(values, l1=0.0, l2=0.0):
     return float(penalty[0]), grad
 
 
+def constrain(matrix, clip=0.0, max_l1_norm=0.0, max_l2_norm=0.0):
+    """The constraints StandardParameters enforces on its values in set_values and on its gradient in accumulate_grad
+    (parameters/StandardParameters.hpp:105-123), in the arithmetic of the matrix's type and in the reference's order:
+    enforce_clip_constraint (:150-156) clips to [-clip, clip]; enforce_l1_norm_constraint (:163-169) scales by
+    max_l1_norm / matrix.norm() - Eigen's norm() is the Euclidean one - if that norm exceeds the limit;
+    enforce_l2_norm_constraint (:176-182) scales by max_l2_norm / matrix.squaredNorm() if the squared norm exceeds the
+    limit. A limit takes effect if NumericUtils::decidedly_greater(limit, 0) (core/NumericUtils.hpp:42-65: greater than
+    zero and not within the type's epsilon of it). Returns a new matrix."""
+    dt = matrix.dtype
+    m = np.array(matrix, dtype=dt, order="F", copy=True)
+    eps = np.finfo(dt).eps
+
+    def on(limit):
+        return dt.type(limit) > eps
+
+    if on(clip):
+        c = dt.type(clip)
+        m = np.where(m > c, c, np.where(m < -c, -c, m)).astype(dt)
+    if on(max_l1_norm):
+        norm = np.sqrt(np.sum(m * m, dtype=dt), dtype=dt)
+        if norm > dt.type(max_l1_norm):
+            m = (m * (dt.type(max_l1_norm) / norm)).astype(dt)
+    if on(max_l2_norm):
+        sq = np.sum(m * m, dtype=dt)
+        if sq > dt.type(max_l2_norm):
+            m = (m * (dt.type(max_l2_norm) / sq)).astype(dt)
+    return np.asfortranarray(m)
+
+
 def sgd_update(values, grad, lr=1e-3):
     """Returns the updated values (the inputs are left alone)."""
     dt = values.dtype

@@ -240,6 +240,28 @@ def test_regularization_by_hand_and_by_differences():
         assert abs(num - grad[idx]) < 1e-8
 
 
+def test_parameter_constraints_by_hand():
+    """StandardParameters.hpp:150-182 on a 3-4-5 matrix: the clip, the "L1" constraint that measures the Euclidean norm, the
+    "L2" constraint that compares the squared norm with its limit and scales by their ratio (so that a matrix over the limit
+    ends up with the squared norm limit^2 / old squared norm, not with the limit), their order, and limits that are off."""
+    m = np.asfortranarray(np.array([[3.0, -4.0]]))
+    assert np.array_equal(oracle.constrain(m), m)
+    assert np.array_equal(oracle.constrain(m, clip=3.5), [[3.0, -3.5]])
+    assert np.array_equal(oracle.constrain(m, clip=1e-17), m)                        # not decidedly greater than zero: off
+    assert np.allclose(oracle.constrain(m, max_l1_norm=2.5), [[1.5, -2.0]], rtol=1e-15)   # norm() = 5: halved
+    assert np.array_equal(oracle.constrain(m, max_l1_norm=5.0), m)                   # not over the limit
+    assert np.array_equal(oracle.constrain(m, max_l1_norm=6.9), m)                   # an L1 norm of 7 would be over: not what is measured
+    out = oracle.constrain(m, max_l2_norm=5.0)                                       # squaredNorm() = 25 > 5: scaled by 5 / 25
+    assert np.allclose(out, [[0.6, -0.8]], rtol=1e-15) and abs(np.sum(out * out) - 1.0) < 1e-15
+    assert np.array_equal(oracle.constrain(m, max_l2_norm=25.0), m)
+    # order: clip to [-3.5, 3.5] -> (3, -3.5), norm sqrt(21.25) > 2 -> scaled to norm 2 (squared norm 4) -> 4 > 1 -> scaled by 1 / 4
+    out = oracle.constrain(m, clip=3.5, max_l1_norm=2.0, max_l2_norm=1.0)
+    want = np.array([[3.0, -3.5]]) * (2.0 / np.sqrt(21.25)) * 0.25
+    assert np.allclose(out, want, rtol=1e-14)
+    out32 = oracle.constrain(m.astype(np.float32), clip=3.5, max_l1_norm=2.0, max_l2_norm=1.0)
+    assert out32.dtype == np.float32 and np.allclose(out32, want, rtol=1e-6)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_l2_regularized_sgd_is_torch_weight_decay(dtype):
     """SGDOptimizer::_train regularizes, then updates (optimizer/SGDOptimizer.hpp:59-64): with L2 regularization and
