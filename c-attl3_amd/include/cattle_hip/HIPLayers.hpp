@@ -33,6 +33,7 @@
 #include <array>
 #include <cassert>
 #include <cstddef>
+#include <cstring>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -74,12 +75,34 @@ private:
 	cattle_hip_layer_t handle;
 };
 
-/* Parameters::get_values() -> device. */
+/* What the device holds of one parameter matrix: the values of the last upload. The host Parameters object stays the
+ * owner of the values (optimizers call its set_values), and most passes find it unchanged - every inference pass, the
+ * passes of frozen or shared layers, all passes between two optimizer steps - so a pass compares before it uploads: a
+ * comparison in host memory costs a fraction of the copy, the wait for it and the re-layout kernel that a new version
+ * of the weights triggers. */
 template<typename Scalar>
-inline void push_values(cattle_hip_layer_t layer, std::size_t index, const Parameters<Scalar>& params) {
+class UploadedValues {
+public:
+	inline bool differ(const Scalar* values, std::size_t count) const {
+		return last.size() != count || std::memcmp(last.data(), values, count * sizeof(Scalar)) != 0;
+	}
+	inline void remember(const Scalar* values, std::size_t count) {
+		last.assign(values, values + count);
+	}
+private:
+	std::vector<Scalar> last;
+};
+
+/* Parameters::get_values() -> device, if they are not there already. */
+template<typename Scalar>
+inline void push_values(cattle_hip_layer_t layer, std::size_t index, const Parameters<Scalar>& params, UploadedValues<Scalar>& uploaded) {
 	const Matrix<Scalar>& values = params.get_values();
 	assert((std::size_t) values.rows() == params.get_rows() && (std::size_t) values.cols() == params.get_cols());
+	const std::size_t count = params.get_rows() * params.get_cols();
+	if (!uploaded.differ(values.data(), count))
+		return;
 	check(cattle_hip_layer_set_param_values(layer, index, values.data(), CATTLE_HIP_HOST));
+	uploaded.remember(values.data(), count);
 }
 
 /* Device gradient of the last backward pass -> Parameters::accumulate_grad(); the device buffer is
@@ -156,8 +179,8 @@ public:
 		assert((detail::dims_match<typename Root::Data,typename Root::Dims,Rank>(in, Base::input_dims)));
 		assert(in.dimension(0) > 0);
 		batch_size = in.dimension(0);
-		detail::push_values<Scalar>(device.get(), 0, *Base::weights);
-		detail::push_values<Scalar>(device.get(), 1, *Base::bias);
+		detail::push_values<Scalar>(device.get(), 0, *Base::weights, uploaded_weights);
+		detail::push_values<Scalar>(device.get(), 1, *Base::bias, uploaded_bias);
 		typename Root::Data out(detail::batch_dims<typename Root::Dims,Rank>(batch_size, Base::output_dims));
 		detail::check(cattle_hip_layer_forward(device.get(), in.data(), CATTLE_HIP_HOST, batch_size, training ? 1 : 0,
 				out.data(), CATTLE_HIP_HOST));
@@ -224,6 +247,7 @@ private:
 	}
 	const Geometry geom;
 	detail::Handle device;
+	detail::UploadedValues<Scalar> uploaded_weights, uploaded_bias;
 	std::size_t batch_size;
 };
 
@@ -382,8 +406,8 @@ public:
 		assert((detail::dims_match<typename Root::Data,typename Root::Dims,Rank>(in, Base::input_dims)));
 		assert(in.dimension(0) > 0);
 		batch_size = in.dimension(0);
-		detail::push_values<Scalar>(device.get(), 0, *Base::weights);
-		detail::push_values<Scalar>(device.get(), 1, *Base::bias);
+		detail::push_values<Scalar>(device.get(), 0, *Base::weights, uploaded_weights);
+		detail::push_values<Scalar>(device.get(), 1, *Base::bias, uploaded_bias);
 		typename Root::Data out(detail::batch_dims<typename Root::Dims,Rank>(batch_size, Base::output_dims));
 		detail::check(cattle_hip_layer_forward(device.get(), in.data(), CATTLE_HIP_HOST, batch_size, training ? 1 : 0,
 				out.data(), CATTLE_HIP_HOST));
@@ -413,6 +437,7 @@ private:
 				Base::output_dims.get_volume(), device.out()));
 	}
 	detail::Handle device;
+	detail::UploadedValues<Scalar> uploaded_weights, uploaded_bias;
 	std::size_t batch_size;
 };
 
@@ -579,11 +604,15 @@ private:
 		for (std::size_t i = 0; i < set.size(); ++i)
 			for (std::size_t j = 0; j < param_cols; ++j)
 				row(0, i * param_cols + j) = set[i]->get_values()(0, j);
+		if (!uploaded[index].differ(row.data(), groups))
+			return;
 		detail::check(cattle_hip_layer_set_param_values(device.get(), index, row.data(), CATTLE_HIP_HOST));
+		uploaded[index].remember(row.data(), groups);
 	}
 	inline void pull_values(std::size_t index, ParamSet& set) {
 		Matrix<Scalar> row(1, groups);
 		detail::check(cattle_hip_layer_get_param_values(device.get(), index, row.data(), CATTLE_HIP_HOST));
+		uploaded[index].remember(row.data(), groups);          /* host and device agree from here on */
 		for (std::size_t i = 0; i < set.size(); ++i) {
 			Matrix<Scalar> part(1, param_cols);
 			for (std::size_t j = 0; j < param_cols; ++j)
@@ -609,6 +638,7 @@ private:
 	bool input_layer, avgs_init;
 	std::size_t batch_size;
 	ParamSet avg_means, avg_inv_sds, gammas, betas;
+	detail::UploadedValues<Scalar> uploaded[4];
 	detail::Handle device;
 };
 
@@ -649,7 +679,7 @@ public:
 		assert(in.dimension(0) > 0);
 		batch_size = in.dimension(0);
 		if (Base::params)
-			detail::push_values<Scalar>(device.get(), 0, *Base::params);
+			detail::push_values<Scalar>(device.get(), 0, *Base::params, uploaded_params);
 		typename Root::Data out(detail::batch_dims<typename Root::Dims,Rank>(batch_size, Base::dims));
 		detail::check(cattle_hip_layer_forward(device.get(), in.data(), CATTLE_HIP_HOST, batch_size, training ? 1 : 0,
 				out.data(), CATTLE_HIP_HOST));
@@ -676,6 +706,7 @@ private:
 				(double) param, device.out()));
 	}
 	const Scalar param;
+	detail::UploadedValues<Scalar> uploaded_params;
 	detail::Handle device;
 	std::size_t batch_size;
 };

@@ -164,6 +164,17 @@ static void run(const std::string& tag) {
 		record(tag + "dense.dx", dense.pass_back(go));
 		record(tag + "dense.dw", dense.get_params()[0]->get_grad());
 		record(tag + "dense.db", dense.get_params()[1]->get_grad());
+		/* the layer uploads a parameter only when its host values changed: unchanged values give the same output again,
+		 * values set through the Parameters object (what an optimizer does) show in the next pass */
+		auto again = dense.pass_forward(x, false);
+		for (std::size_t i = 0; i < out.size(); ++i)
+			if (again.data()[i] != out.data()[i])
+				throw std::runtime_error("a second pass with unchanged parameters differs");
+		randomize(*dense.get_params()[0], g, 0.3);
+		randomize(*dense.get_params()[1], g, 0.3);
+		record(tag + "dense.w2", dense.get_params()[0]->get_values());
+		record(tag + "dense.b2", dense.get_params()[1]->get_values());
+		record(tag + "dense.out2", dense.pass_forward(x, false));
 	}
 	/* 3. batch norm per channel: two training passes, then inference */
 	{

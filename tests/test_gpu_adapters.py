@@ -77,6 +77,8 @@ def test_kernel_layers(records, tag):
     dx, dw, db = oracle.dense_backward(X, r["dense.w"], r["dense.go"].reshape(out.shape, order="F"))
     assert hp.rel_err(r["dense.out"].reshape(out.shape, order="F"), out) < tol
     assert hp.rel_err(r["dense.dx"], dx) < tol and hp.rel_err(r["dense.dw"], dw) < tol and hp.rel_err(r["dense.db"], db) < tol
+    out2 = oracle.dense_forward(X, r["dense.w2"], r["dense.b2"])          # after the host values changed
+    assert hp.rel_err(r["dense.out2"].reshape(out2.shape, order="F"), out2) < tol
 
 
 @pytest.mark.gpu
