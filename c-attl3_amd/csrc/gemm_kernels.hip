@@ -1101,8 +1101,23 @@ int round_up(int v, int to) {
 
 constexpr int WT_ROW_PAD = 64;     /* a multiple of every KC: the last reduction chunk reads whole chunks of weight rows */
 constexpr int WT_COL_PAD = 128;    /* >= every BF */
-constexpr int NUM_CUS = 256;
-constexpr int LDS_PER_CU = 160 * 1024;
+/* Compute units and LDS bytes per compute unit of the current device, from the runtime (256 and 160 KB on an MI355X;
+ * a partitioned device reports its share), asked once. */
+struct DeviceShape {
+	int cus, lds_per_cu;
+	DeviceShape() {
+		int dev = 0;
+		hipDeviceProp_t prop;
+		CATTLE_HIP_CHECK(hipGetDevice(&dev));
+		CATTLE_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+		cus = std::max(1, prop.multiProcessorCount);
+		lds_per_cu = (int) std::max<size_t>(64 * 1024, prop.maxSharedMemoryPerMultiProcessor);
+	}
+};
+const DeviceShape& device_shape() {
+	static const DeviceShape shape;
+	return shape;
+}
 
 
 /* Grow-only device scratch for split reductions. Calls into the library are serialised and issued on
@@ -1439,7 +1454,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	for (int i = 1; i < GatherVariants<T>::LARGE; ++i) {
 		const bool narrower = vars[i].bf >= g.F && vars[i].bf < vars[best_v].bf;
 		/* same width, taller tile: half the A-operand loads per MFMA; worth it once it still fills the chip */
-		const bool taller = vars[i].bf == vars[best_v].bf && vars[i].bm > vars[best_v].bm && g.M >= vars[i].bm * NUM_CUS * 4;
+		const bool taller = vars[i].bf == vars[best_v].bf && vars[i].bm > vars[best_v].bm && g.M >= vars[i].bm * device_shape().cus * 4;
 		if (narrower || taller)
 			best_v = i;
 	}
@@ -1448,11 +1463,11 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	 * 256 x 128 with K = 72: 37 -> 31 us). */
 	if (best_v == 0 && vars[0].bf > vars[1].bf && g.F > vars[1].bf) {
 		const long blocks = (long) ((g.M + vars[0].bm - 1) / vars[0].bm) * ((g.F + vars[0].bf - 1) / vars[0].bf);
-		if (blocks >= NUM_CUS && blocks * 2 <= 3 * NUM_CUS)
+		if (blocks >= device_shape().cus && blocks * 2 <= 3 * device_shape().cus)
 			best_v = 1;
 	}
 	/* too few large tiles to give every CU one: take the short tiles (the narrowest that still covers F, else the widest) */
-	if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) < NUM_CUS) {
+	if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) < device_shape().cus) {
 		constexpr int SHORT = GatherVariants<T>::SHORT;       /* short shapes, each with long and with medium chunks */
 		best_v = GatherVariants<T>::LARGE;
 		for (int i = GatherVariants<T>::LARGE + 1; i < GatherVariants<T>::LARGE + SHORT; ++i)
@@ -1463,13 +1478,13 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		 * tile is then cut into parts and shorter chunks give twice as many parts to fill the chip with. In between:
 		 * the long chunks, with which one block keeps more loads in flight */
 		const long short_tiles = (long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf);
-		if (short_tiles >= 2 * NUM_CUS || short_tiles * 2 <= NUM_CUS)
+		if (short_tiles >= 2 * device_shape().cus || short_tiles * 2 <= device_shape().cus)
 			best_v += SHORT;
 		/* 32 columns and enough rows for every CU to get a tile twice as tall: four waves share the table and the
 		 * barriers that two-wave blocks pay for alone (config 3's second input gradient, 512 tiles of 64 x 32 with
 		 * K = 576: 33 -> 25 us) */
 		if (GatherVariants<T>::TALL32 >= 0 && vars[best_v].bf == 32 &&
-				(long) ((g.M + 127) / 128) * ((g.F + 31) / 32) >= NUM_CUS)
+				(long) ((g.M + 127) / 128) * ((g.F + 31) / 32) >= device_shape().cus)
 			best_v = GatherVariants<T>::TALL32;
 	}
 	const Tuning& tune = tuning();
@@ -1496,7 +1511,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	const GatherVariant<T>& v = vars[best_v];
 	size_t dyn = 0;
 	if (occ >= 1 && occ <= 8) {
-		const int want_bytes = LDS_PER_CU / (occ + 1) + 256;
+		const int want_bytes = device_shape().lds_per_cu / (occ + 1) + 256;
 		dyn = want_bytes > v.lds_bytes ? (size_t) (want_bytes - v.lds_bytes) : 0;
 	}
 	const int mtiles = (g.M + v.bm - 1) / v.bm, ftiles = (g.F + v.bf - 1) / v.bf;
@@ -1525,7 +1540,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		*mtiles_out = mtiles;
 	/* blocks the chip holds at once (registers, LDS, waves), as the runtime computes it for this kernel */
 	const int per_cu = std::max(1, v.blocks_per_cu(dyn, vec, divs, epi));
-	const int slots = NUM_CUS * per_cu;
+	const int slots = device_shape().cus * per_cu;
 	const bool no_split = tune.no_split || epi == EPI_POOL || epi == EPI_STATS;
 	const Epilogue<T> none = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr };
 	const Epilogue<T>& epi_args = E ? *E : none;
@@ -1660,6 +1675,7 @@ WgradVariant<T> wgrad_variant() {
 template<typename T> struct WgradVariants;
 template<> struct WgradVariants<float> {
 	static constexpr int COUNT = 11, BASE = 7;      /* BASE: the variants with the standard chunk, which any problem may use */
+	static constexpr int WIDE_CHUNKS = 10;          /* 64 x 64 with chunks of 128 rows */
 	static const WgradVariant<float>* get() {
 		static const WgradVariant<float> v[COUNT] = {
 			wgrad_variant<float, 2, 4, 96, 32, 4>(),    /* 192 x 128, registers held to four waves per SIMD = two blocks per CU */
@@ -1679,7 +1695,7 @@ template<> struct WgradVariants<float> {
 	}
 };
 template<> struct WgradVariants<double> {
-	static constexpr int COUNT = 4, BASE = 4;
+	static constexpr int COUNT = 4, BASE = 4, WIDE_CHUNKS = -1;
 	static const WgradVariant<double>* get() {
 		static const WgradVariant<double> v[COUNT] = {
 			wgrad_variant<double, 2, 4, 48, 32>(),      /* 96 x 128 */
@@ -1727,7 +1743,7 @@ WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 			if ((long) round_up(K, vars[i].bk) * round_up(F, vars[i].bf) != best)
 				continue;
 			const long blocks = (long) ((K + vars[i].bk - 1) / vars[i].bk) * ((F + vars[i].bf - 1) / vars[i].bf) * max_splits;
-			if (blocks >= NUM_CUS / 2) {
+			if (blocks >= device_shape().cus / 2) {
 				pick = i;
 				break;
 			}
@@ -1739,6 +1755,16 @@ WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 		if (pick >= 0)
 			p.variant = pick;
 	}
+	/* Many one-wave tiles over a long M (config 3's second convolution: 9 x 2 tiles of 32 x 32, 32768 rows): four-wave
+	 * 64 x 64 tiles with chunks of 128 rows load each operand row half as often and in longer runs; measured 35 -> 28 us
+	 * with the reduce launch. Needs 16-byte loads, and for the walk by positions a batch that is a multiple of the chunk. */
+	if (!short_m && vec && WgradVariants<T>::WIDE_CHUNKS >= 0 && vars[p.variant].waves == 1) {
+		const WgradVariant<T>& w = vars[WgradVariants<T>::WIDE_CHUNKS];
+		const long tiles = (long) ((K + vars[p.variant].bk - 1) / vars[p.variant].bk) * ((F + vars[p.variant].bf - 1) / vars[p.variant].bf);
+		const long padded = (long) round_up(K, w.bk) * round_up(F, w.bf);
+		if (tiles >= 16 && padded * 100 <= best * 115 && N % w.mc == 0)
+			p.variant = WgradVariants<T>::WIDE_CHUNKS;
+	}
 	if (tune.wgrad_variant >= 0 && tune.wgrad_variant < WgradVariants<T>::COUNT && (vec || vars[tune.wgrad_variant].mc == WGRAD_MC))
 		p.variant = tune.wgrad_variant;
 	const WgradVariant<T>& v = vars[p.variant];
@@ -1746,7 +1772,7 @@ WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 	p.ftiles = (F + v.bf - 1) / v.bf;
 	/* at most three blocks of eight waves per CU; small blocks up to sixteen waves' worth */
 	const int occ = std::max(1, std::min(v.blocks_per_cu(), std::max(3, 16 / v.waves)));
-	const int slots = NUM_CUS * occ;
+	const int slots = device_shape().cus * occ;
 	const int tiles = p.ktiles * p.ftiles;
 	const int chunks = (M + v.mc - 1) / v.mc;
 	int want = std::max(1, slots / tiles);
