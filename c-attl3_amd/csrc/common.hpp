@@ -63,6 +63,9 @@ struct GatherGeom {
 	int SA, SB, RA, RB, PA, PB, DA, DB;
 	int M, K, F;
 	int ldw;        /* row stride of the prepared weight matrix Wt (elements) */
+	int NS;         /* samples between two positions of the gathered tensor: N, or more when the N samples are the
+	                 * first of a larger batch (one time step of a sequence tensor (N, T, ...), whose step t starts
+	                 * N t elements into it and has N T samples between positions) */
 };
 
 /* Convolution hyper-parameters in the reference's terms (dilation 0 = dense receptor). */
@@ -86,9 +89,10 @@ template<typename T> ConvWorkspace conv_workspace(const ConvShape& s, int N);
 int prepared_weight_row_length(int columns);
 
 /* Forward: out(N,OH,OW,F) = conv(x; w) + b. w is the reference's [K x F] column-major matrix.
- * wt is scratch of conv_workspace().wt_fwd elements; if wt_ready is false it is (re)built from w. */
+ * wt is scratch of conv_workspace().wt_fwd elements; if wt_ready is false it is (re)built from w.
+ * x_batch > 0: x holds the first N of x_batch samples per position (GatherGeom::NS). */
 template<typename T> void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out,
-		T* wt, bool wt_ready);
+		T* wt, bool wt_ready, int x_batch = 0);
 
 /* The same forward pass for callers that cannot allocate device memory: the prepared weights and the partial sums of a
  * split reduction live in a fixed device array of static_scratch_bytes() bytes per device, whose address
@@ -106,8 +110,13 @@ template<typename T> void conv_backward(const ConvShape& s, int N, const T* x, c
  * of input and output exchanged). bgrad may be null. */
 template<typename T> void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad,
 		T* partials);
-template<typename T> void conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad,
-		T* wt_dgrad, bool wt_ready);
+template<typename T> struct LstmBackwardStep;
+/* og_batch > 0: out_grad holds the first N of og_batch samples per position (GatherGeom::NS). `then`, if given, is the LSTM backward step that consumes in_grad as the gradient of its hidden output: when the
+ * launch cuts every tile's reduction into parts, the kernel that sums the parts runs the element-wise part of that
+ * step on each sum instead of writing it. Returns whether it did; false: in_grad was written and the step is still to
+ * be run (lstm_gates_backward). */
+template<typename T> bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad,
+		T* wt_dgrad, bool wt_ready, const LstmBackwardStep<T>* then = nullptr, int og_batch = 0);
 
 /* Element-wise / reduction kernels (pointwise_kernels.hip). */
 template<typename T> void act_forward(int kind, size_t n, T p, const T* x, T* y);
@@ -207,14 +216,44 @@ template<typename T> void broadcast_backward(int H, int W, int C, int bh, int bw
  * 1 write, 2 candidate, 3 state, 4 read activation (element-wise kinds only). Per-step tensors hold
  * the four gates as consecutive blocks of P elements; `*_all` tensors are (N, T, ...) over all steps. */
 template<typename T> struct LstmActs { int kind[5]; T param[5]; };
-template<typename T> void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int zx_T, int zx_t,
-		const T* zh, bool mul_int, const T* prev_state, T* z, T* gates, T* state, T* act_state, T* hidden, T* hprev_all, int h_T,
-		int h_t, T* out, int out_T, int out_t);
-/* zx_fwd / zh_fwd: the step's weighted input (in the all-steps tensor) and weighted previous output when the network
- * integrates multiplicatively and the step had both; null otherwise. */
-template<typename T> void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, const T* out_grad, int og_T,
-		int og_t, const T* z, const T* gates, const T* prev_state, const T* state, const T* act_state, T* state_grad, T* dz,
-		T* dzx_all, int x_T, int x_t, T* dzh_all, int h_T, int h_t, const T* zx_fwd, const T* zh_fwd);
+/* The tensors of one forward step: zx the weighted inputs of all steps (null at a step without input), z / gates /
+ * state / act_state this step's slabs (z, the gates' pre-activation values, null when no gate activation's backward
+ * pass reads its input), hprev_all the hidden outputs of all steps shifted by one (slab h_t receives this step's: it
+ * is what the next step's output-side kernels read), out the network's output sequence (null at a step that emits
+ * nothing). */
+template<typename T> struct LstmForwardStep {
+	LstmActs<T> a;
+	int N;
+	size_t P;
+	const T* zx;
+	int zx_T, zx_t;
+	bool mul_int;
+	const T* prev_state;
+	T *z, *gates, *state, *act_state, *hprev_all;
+	int h_T, h_t;
+	T* out;
+	int out_T, out_t;
+};
+/* The tensors of one backward step. dzh_all, the gate gradients of all steps as the output-side kernels receive them,
+ * serves both their weight gradient at the end and, slab by slab, their input gradient. zx_fwd / zh_fwd: the step's weighted input (in the all-steps tensor) and weighted
+ * previous output when the network integrates multiplicatively and the step had both; null otherwise. */
+template<typename T> struct LstmBackwardStep {
+	LstmActs<T> a;
+	int N;
+	size_t P;
+	const T* out_grad;
+	int og_T, og_t;
+	const T *z, *gates, *prev_state, *state, *act_state;
+	T *state_grad, *dzx_all;
+	int x_T, x_t;
+	T* dzh_all;
+	int h_T, h_t;
+	const T *zx_fwd, *zh_fwd;
+};
+/* zh: the step's weighted previous output (four gate blocks of P elements), null at the first step */
+template<typename T> void lstm_gates_forward(const LstmForwardStep<T>& step, const T* zh);
+/* dh: the gradient of the hidden output that came back from the step after, null at the last step */
+template<typename T> void lstm_gates_backward(const LstmBackwardStep<T>& step, const T* dh);
 
 /* Losses and optimizer updates (train_kernels.hip). A batch is N samples x T_steps x V elements,
  * column-major with the sample index fastest. */

@@ -18,6 +18,7 @@
  */
 #include "common.hpp"
 #include "act_math.hpp"
+#include "lstm_math.hpp"
 
 #include <algorithm>
 #include <limits>
@@ -274,13 +275,13 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		tch = t / g.S;
 	}
 	const int eR = KC % g.R, eS = (KC / g.R) % g.S, eCh = (KC / g.R) / g.S;
-	const int plane = g.N * g.LH * g.LW;
+	const int plane = g.NS * g.LH * g.LW;
 	auto write_table = [&](int slot) {
 		if (tid < KC) {
 			const bool kv = tch < g.LC;
 			const int dya = tr * g.RA, dyb = ts * g.RB;
 			const int choff = kv ? plane * tch : 0;
-			ktab[slot][tid] = make_int4(kv ? g.N * (dya + g.LH * dyb) + choff : 0, kv ? dya : INVALID, dyb, choff);
+			ktab[slot][tid] = make_int4(kv ? g.NS * (dya + g.LH * dyb) + choff : 0, kv ? dya : INVALID, dyb, choff);
 			tr += eR;
 			const int c1 = tr >= g.R;
 			tr -= c1 ? g.R : 0;
@@ -304,7 +305,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		ya0 = a * g.SA + g.PA;
 		yb0 = b * g.SB + g.PB;
 	}
-	const int base_m = n + g.N * (ya0 + g.LH * yb0);      /* may be negative; only used when in range */
+	const int base_m = n + g.NS * (ya0 + g.LH * yb0);      /* may be negative; only used when in range */
 	const T* const zeros = reinterpret_cast<const T*>(g_zero_block);
 	const T* bptr[BITER];
 	#pragma unroll
@@ -338,7 +339,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 				ok &= (qa * g.DA == ya) & (qb * g.DB == yb);
 				ya = qa;
 				yb = qb;
-				off = n + g.N * (ya + g.LH * yb) + e.w;
+				off = n + g.NS * (ya + g.LH * yb) + e.w;
 			} else {
 				off = base_m + e.x;
 			}
@@ -1180,12 +1181,21 @@ void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ b
 	const T* base = partials + (size_t) t * L.ksplit * tile_elems + e;
 	T acc[V];
 	vec_load<T, V>(acc, base);
-	for (int z = 1; z < L.ksplit; ++z) {
-		T part[V];
-		vec_load<T, V>(part, base + (size_t) z * tile_elems);
+	/* eight parts' loads are issued before the first of their additions (a thread's loads are otherwise a chain of
+	 * memory round trips, one per part); past the last part the load repeats it and the addition is skipped */
+	constexpr int AHEAD = 8;
+	for (int z0 = 1; z0 < L.ksplit; z0 += AHEAD) {
+		T part[AHEAD][V];
 		#pragma unroll
-		for (int i = 0; i < V; ++i)
-			acc[i] += part[i];
+		for (int j = 0; j < AHEAD; ++j)
+			vec_load<T, V>(part[j], base + (size_t) min(z0 + j, L.ksplit - 1) * tile_elems);
+		#pragma unroll
+		for (int j = 0; j < AHEAD; ++j)
+			if (z0 + j < L.ksplit) {
+				#pragma unroll
+				for (int i = 0; i < V; ++i)
+					acc[i] += part[j][i];
+			}
 	}
 	const int m = tile_row_m(L, g, tile, BM, e % BM), f = fb * BF + e / BM;
 	if (f >= F)
@@ -1223,6 +1233,40 @@ void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ b
 						E.pre[o + i] = pre[i];
 			}
 	}
+}
+
+/* The same sums, taken as the gradient of an LSTM cell's hidden output (the input gradient of the output-side kernels
+ * of the step after) and handed, one element per thread, to the element-wise part of the step's backward pass: the
+ * gradient tensor itself is never written. */
+template<typename T>
+__global__ __launch_bounds__(256)
+void split_reduce_lstm_backward_kernel(const T* __restrict__ partials, const GatherGeom g, const GatherLaunch L, int BM, int BF,
+		int ftiles, const LstmBackwardStep<T> A) {
+	const int groups = BM * BF / 256;
+	const int t = blockIdx.x / groups, grp = blockIdx.x % groups;
+	const int local = t / ftiles, fb = t % ftiles;
+	int tile = L.main_count + local;
+	if (L.tile_rows > 0)
+		tile = swizzle_tile(tile, L.tile_rows, L.mtiles / L.tile_rows);
+	const size_t tile_elems = (size_t) BM * BF;
+	const int e = grp * 256 + threadIdx.x;
+	const T* base = partials + (size_t) t * L.ksplit * tile_elems + e;
+	T acc = base[0];
+	constexpr int AHEAD = 8;
+	for (int z0 = 1; z0 < L.ksplit; z0 += AHEAD) {
+		T part[AHEAD];
+		#pragma unroll
+		for (int j = 0; j < AHEAD; ++j)
+			part[j] = base[(size_t) min(z0 + j, L.ksplit - 1) * tile_elems];
+		#pragma unroll
+		for (int j = 0; j < AHEAD; ++j)
+			if (z0 + j < L.ksplit)
+				acc += part[j];
+	}
+	const int m = tile_row_m(L, g, tile, BM, e % BM), f = fb * BF + e / BM;
+	if (m >= g.M || f >= g.F)
+		return;
+	lstm_backward_element<T>(A, (unsigned) m + (unsigned) g.M * (unsigned) f, true, acc);
 }
 
 /* One instantiation of gather_gemm_kernel and what the tile chooser needs to know about it. */
@@ -1444,8 +1488,9 @@ RowBlocks plan_row_blocks(const GatherGeom& g, int bm, int prh, int prw, bool po
  * receives the number of M tiles (the row count of the moments epilogue's partials). */
 template<typename T>
 bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, ScratchArena* arena = nullptr,
-		int epi = EPI_NONE, const Epilogue<T>* E = nullptr, int* mtiles_out = nullptr) {
-	const bool vec = g.N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+		int epi = EPI_NONE, const Epilogue<T>* E = nullptr, int* mtiles_out = nullptr, const LstmBackwardStep<T>* then = nullptr,
+		bool* then_done = nullptr) {
+	const bool vec = g.N % GemmCfg<T>::VEC == 0 && g.NS % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
 	const bool divs = g.DA != 1 || g.DB != 1;
 	if (epi != EPI_NONE && (!vec || divs || (reinterpret_cast<uintptr_t>(out) & 15) != 0))
 		return false;
@@ -1560,7 +1605,11 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if (L.split_count > 0) {
 			const int groups = v.bm * v.bf / (256 * (16 / (int) sizeof(T)));
 			const dim3 rgrid((unsigned) (L.split_count * ftiles * groups));
-			if (epi == EPI_ACT)
+			if (then && main_count == 0 && bias == nullptr && epi == EPI_NONE && (size_t) g.M * g.F == then->P) {
+				const dim3 egrid((unsigned) (L.split_count * ftiles * (v.bm * v.bf / 256)));
+				split_reduce_lstm_backward_kernel<T><<<egrid, 256, 0, stream()>>>(partials, g, L, v.bm, v.bf, ftiles, *then);
+				*then_done = true;
+			} else if (epi == EPI_ACT)
 				split_reduce_kernel<T, true><<<rgrid, 256, 0, stream()>>>(partials, bias, out, g, L, v.bm, v.bf, ftiles, epi_args);
 			else
 				split_reduce_kernel<T, false><<<rgrid, 256, 0, stream()>>>(partials, bias, out, g, L, v.bm, v.bf, ftiles, epi_args);
@@ -1571,7 +1620,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	const long total = (long) mtiles * ftiles;
 	if (!no_split && total * 2 <= slots && nchunks >= 4) {
 		/* far fewer tiles than the chip holds blocks: cut every tile's reduction so that it fills up */
-		launch(0, (int) std::min<long>(std::min<long>(slots / total, nchunks / 2), 16));
+		launch(0, (int) std::min<long>(std::min<long>(slots / total, nchunks / 2), 32));
 		return true;
 	}
 	const int rem = mtiles % slots;
@@ -1588,7 +1637,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 
 GatherGeom forward_geom(const ConvShape& s, int N) {
 	GatherGeom g;
-	g.N = N; g.LH = s.H; g.LW = s.W; g.LC = s.C;
+	g.N = N; g.NS = N; g.LH = s.H; g.LW = s.W; g.LC = s.C;
 	g.OA = s.OH(); g.OB = s.OW();
 	g.R = s.RH; g.S = s.RW;
 	g.SA = s.sv; g.SB = s.sh; g.RA = s.dv + 1; g.RB = s.dh + 1; g.PA = -s.pv; g.PB = -s.ph; g.DA = 1; g.DB = 1;
@@ -1599,7 +1648,7 @@ GatherGeom forward_geom(const ConvShape& s, int N) {
 
 GatherGeom dgrad_geom(const ConvShape& s, int N) {
 	GatherGeom g;
-	g.N = N; g.LH = s.OH(); g.LW = s.OW(); g.LC = s.F;
+	g.N = N; g.NS = N; g.LH = s.OH(); g.LW = s.OW(); g.LC = s.F;
 	g.OA = s.H; g.OB = s.W;
 	g.R = s.RH; g.S = s.RW;
 	g.SA = 1; g.SB = 1; g.RA = -(s.dv + 1); g.RB = -(s.dh + 1); g.PA = s.pv; g.PB = s.ph; g.DA = s.sv; g.DB = s.sh;
@@ -1810,9 +1859,11 @@ ConvWorkspace conv_workspace(const ConvShape& s, int N) {
 }
 
 template<typename T>
-void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out, T* wt, bool wt_ready) {
-	check_sizes(s, N);
-	const GatherGeom g = forward_geom(s, N);
+void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out, T* wt, bool wt_ready, int x_batch) {
+	check_sizes(s, std::max(N, x_batch));
+	GatherGeom g = forward_geom(s, N);
+	if (x_batch > 0)
+		g.NS = x_batch;
 	if (!wt_ready) {
 		const int Kp = round_up(g.K, WT_ROW_PAD);
 		const size_t count = (size_t) Kp * g.ldw;
@@ -1919,9 +1970,12 @@ void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_gr
 }
 
 template<typename T>
-void conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad, T* wt_dgrad, bool wt_ready) {
-	check_sizes(s, N);
-	const GatherGeom d = dgrad_geom(s, N);
+bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad, T* wt_dgrad, bool wt_ready,
+		const LstmBackwardStep<T>* then, int og_batch) {
+	check_sizes(s, std::max(N, og_batch));
+	GatherGeom d = dgrad_geom(s, N);
+	if (og_batch > 0)
+		d.NS = og_batch;
 	if (!wt_ready) {
 		const int Kp = round_up(d.K, WT_ROW_PAD);
 		const size_t count = (size_t) Kp * d.ldw;
@@ -1929,7 +1983,9 @@ void conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_gra
 				Kp, d.ldw);
 		CATTLE_HIP_CHECK(hipGetLastError());
 	}
-	launch_gather<T>(out_grad, wt_dgrad, (const T*) nullptr, in_grad, d);
+	bool then_done = false;
+	launch_gather<T>(out_grad, wt_dgrad, (const T*) nullptr, in_grad, d, nullptr, EPI_NONE, nullptr, nullptr, then, &then_done);
+	return then_done;
 }
 
 template<typename T>
@@ -1937,13 +1993,13 @@ void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* o
 		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials) {
 	conv_weight_gradient<T>(s, N, x, out_grad, wgrad, bgrad, partials);
 	if (in_grad)
-		conv_input_gradient<T>(s, N, w, out_grad, in_grad, wt_dgrad, wt_ready);
+		conv_input_gradient<T>(s, N, w, out_grad, in_grad, wt_dgrad, wt_ready, nullptr, 0);
 }
 
 template ConvWorkspace conv_workspace<float>(const ConvShape&, int);
 template ConvWorkspace conv_workspace<double>(const ConvShape&, int);
-template void conv_forward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, bool);
-template void conv_forward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*, bool);
+template void conv_forward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, bool, int);
+template void conv_forward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*, bool, int);
 template bool conv_forward_fused<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, bool, int,
 		const Epilogue<float>&, int*);
 template bool conv_forward_fused<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*, bool, int,
@@ -1956,7 +2012,9 @@ template void conv_backward<double>(const ConvShape&, int, const double*, const 
 		double*, double*, bool, double*);
 template void conv_weight_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, float*);
 template void conv_weight_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, double*);
-template void conv_input_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, bool);
-template void conv_input_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, bool);
+template bool conv_input_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, bool,
+		const LstmBackwardStep<float>*, int);
+template bool conv_input_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, bool,
+		const LstmBackwardStep<double>*, int);
 
 } /* namespace cattle_hip */

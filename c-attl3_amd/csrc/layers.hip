@@ -476,7 +476,7 @@ struct ConvLstm : LayerBase {
 	/* alignment of the last propagate (:398-401) */
 	size_t T_in = 0, T_out = 0, delay = 0, steps = 0;
 	const T* x_cache = nullptr;
-	DevBuf zx_all, zh, z, gates, state, act_state, hid, hprev_all, dzx_all, dzh_all, dz, dh, state_grad, partials;
+	DevBuf zx_all, zh, z, gates, state, act_state, hprev_all, dzx_all, dzh_all, dh, state_grad, partials;
 	DevBuf seq_in_stage, seq_out_stage, seq_og_stage, seq_ig_stage;
 
 	ConvLstm(int dtype, const ConvShape& x_shape, const ConvShape& h_shape, const LstmActs<T>& acts, bool foremost) :
@@ -502,6 +502,13 @@ struct ConvLstm : LayerBase {
 	void backward(const void*, size_t, void*) override {
 		throw Error(ERR_STATE, "a recurrent network takes sequences: use cattle_hip_convlstm_backpropagate");
 	}
+	/* the gates' pre-activation values are kept for the backward pass only if an activation's derivative reads them */
+	bool keeps_z() const {
+		for (int i = 0; i < 5; ++i)
+			if (act_needs_x(acts.kind[i]))
+				return true;
+		return false;
+	}
 	size_t P(size_t N) const {            /* state elements of one step */
 		return N * out_volume();
 	}
@@ -525,15 +532,16 @@ struct ConvLstm : LayerBase {
 					(T*) zx_all.ensure(4 * p * in_len * e), wt, wx.derived_version[0] == wx.version);
 			wx.derived_version[0] = wx.version;
 		}
-		z.ensure(4 * p * total * e);
+		CATTLE_HIP_REQUIRE((double) (4 * p) * (double) std::max(total, in_len) <= 2147483647.0, "sequence tensor exceeds 2^31-1 elements");
+		if (keeps_z())
+			z.ensure(4 * p * total * e);
 		gates.ensure(4 * p * total * e);
 		state.ensure(p * total * e);
 		act_state.ensure(p * total * e);
-		hid.ensure(p * total * e);
 		/* with multiplicative integration the backward pass needs every step's weighted previous output */
 		zh.ensure(4 * p * (mul_int ? total : 1) * e);
 		/* slab t of hprev_all is the hidden output of step t - 1 (the first step's kernel zeroes slab 0: no previous
-		 * output); every slab is written once per pass */
+		 * output); every slab is written once per pass. The last step's hidden output goes to `out` only. */
 		hprev_all.ensure(p * total * e);
 		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
 		T* wth = (T*) wh.derived[0].ensure(wsh.wt_fwd * e);
@@ -541,16 +549,17 @@ struct ConvLstm : LayerBase {
 			const bool has_in = t < in_len, has_prev = t > 0;
 			T* zh_t = step(zh, mul_int ? t : 0, 4 * p);
 			if (has_prev) {
-				conv_forward<T>(sh, n, step(hid, t - 1, p), (const T*) wh.values.p, (const T*) params[3]->values.p, zh_t,
-						wth, wh.derived_version[0] == wh.version);
+				/* the previous hidden output where the previous step left it: slab t of (N, total, H, W, hidden) */
+				conv_forward<T>(sh, n, (const T*) hprev_all.p + N * t, (const T*) wh.values.p, (const T*) params[3]->values.p, zh_t,
+						wth, wh.derived_version[0] == wh.version, (int) (N * total));
 				wh.derived_version[0] = wh.version;
 			}
 			const bool emits = t >= out_delay && t < out_delay + out_len;      /* :386-393 */
-			lstm_gates_forward<T>(acts, n, p, has_in ? (const T*) zx_all.p : nullptr, (int) in_len, (int) t,
-					has_prev ? (const T*) zh_t : nullptr, mul_int, has_prev ? step(state, t - 1, p) : nullptr, step(z, t, 4 * p),
-					step(gates, t, 4 * p), step(state, t, p), step(act_state, t, p), step(hid, t, p),
-					(T*) hprev_all.p, (int) total, (int) (t + 1), emits ? out : nullptr, (int) out_len,
-					(int) (t - out_delay));
+			const LstmForwardStep<T> fs = { acts, n, p, has_in ? (const T*) zx_all.p : nullptr, (int) in_len, (int) t, mul_int,
+					has_prev ? step(state, t - 1, p) : nullptr, keeps_z() ? step(z, t, 4 * p) : nullptr, step(gates, t, 4 * p),
+					step(state, t, p), step(act_state, t, p), (T*) hprev_all.p, (int) total, (int) (t + 1), emits ? out : nullptr,
+					(int) out_len, (int) (t - out_delay) };
+			lstm_gates_forward<T>(fs, has_prev ? (const T*) zh_t : nullptr);
 		}
 		x_cache = input;
 		batch = N;
@@ -564,27 +573,34 @@ struct ConvLstm : LayerBase {
 		Param& wx = *params[0];
 		Param& wh = *params[2];
 		state_grad.ensure(p * e);                                        /* starts at zero (:422-425): the last step's kernel ignores it */
-		dz.ensure(4 * p * e);
 		dh.ensure(p * e);
 		dzx_all.ensure(4 * p * T_in * e);
 		dzh_all.ensure(4 * p * total * e);                               /* every slab is written; step 0 writes zeros */
 		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
 		T* wtd = (T*) wh.derived[1].ensure(wsh.wt_dgrad * e);
-		for (size_t t = total; t-- > 0;) {
+		auto backward_step = [&](size_t t) {
 			const bool has_in = t < T_in, has_prev = t > 0;
 			const bool emitted = t >= delay && t < delay + T_out;
 			const bool both = mul_int && has_in && has_prev;
-			lstm_gates_backward<T>(acts, n, p, t + 1 < total ? (const T*) dh.p : nullptr, emitted ? out_grad : nullptr,
-					(int) T_out, (int) (t - delay), step(z, t, 4 * p), step(gates, t, 4 * p),
-					has_prev ? step(state, t - 1, p) : nullptr, step(state, t, p), step(act_state, t, p), (T*) state_grad.p,
-					(T*) dz.p, has_in ? (T*) dzx_all.p : nullptr, (int) T_in, (int) t, (T*) dzh_all.p,
-					(int) total, (int) t, both ? (const T*) zx_all.p : nullptr, both ? (const T*) step(zh, t, 4 * p) : nullptr);
-			if (has_prev) {
-				/* the four output-side kernels' pass_back, summed (:470-473, :491-494): one input-gradient launch */
-				conv_input_gradient<T>(sh, n, (const T*) wh.values.p, (const T*) dz.p, (T*) dh.p, wtd,
-						wh.derived_version[1] == wh.version);
-				wh.derived_version[1] = wh.version;
-			}
+			const LstmBackwardStep<T> bs = { acts, n, p, emitted ? out_grad : nullptr, (int) T_out, (int) (t - delay),
+					keeps_z() ? step(z, t, 4 * p) : nullptr, step(gates, t, 4 * p), has_prev ? step(state, t - 1, p) : nullptr,
+					step(state, t, p), step(act_state, t, p), (T*) state_grad.p, has_in ? (T*) dzx_all.p : nullptr, (int) T_in, (int) t,
+					(T*) dzh_all.p, (int) total, (int) t, both ? (const T*) zx_all.p : nullptr,
+					both ? (const T*) step(zh, t, 4 * p) : nullptr };
+			return bs;
+		};
+		if (total > 0)
+			lstm_gates_backward<T>(backward_step(total - 1), (const T*) nullptr);
+		for (size_t t = total; t-- > 1;) {
+			/* the four output-side kernels' pass_back, summed (:470-473, :491-494), is one input-gradient launch, and
+			 * the element-wise part of step t - 1, which is all that reads its result, runs in the kernel that sums the
+			 * parts of that launch's reductions when the launch has such a kernel */
+			const LstmBackwardStep<T> before = backward_step(t - 1);
+			const bool done = conv_input_gradient<T>(sh, n, (const T*) wh.values.p, (const T*) dzh_all.p + N * t, (T*) dh.p, wtd,
+					wh.derived_version[1] == wh.version, &before, (int) (N * total));
+			wh.derived_version[1] = wh.version;
+			if (!done)
+				lstm_gates_backward<T>(before, (const T*) dh.p);
 		}
 		/* parameter gradients of all steps at once: slab 0 of dzh_all and of hprev_all is zero */
 		if (total > 1) {

@@ -8,6 +8,7 @@
  */
 #include "common.hpp"
 #include "act_math.hpp"
+#include "lstm_math.hpp"
 
 #include <algorithm>
 #include <limits>
@@ -753,137 +754,29 @@ void column_sums_kernel(int N, size_t V, const T* __restrict__ x, T* __restrict_
 }
 
 /* ----------------------------------------------------------------------------------------------
- * LSTM cell arithmetic between the kernel layers (neural_network/LSTMNeuralNetwork.hpp:283-394
- * forward, :436-441 backward), one thread per state element. The four gates (forget, write,
- * candidate, read) are the channel blocks of one tensor, so gate g of element e sits at g*P + e in a
- * per-step tensor. Tensors that span all time steps are (N, T, ...) column-major: element e of step t
- * is at n + N*(t + T*rest) with n = e % N, rest = e / N.
+ * LSTM cell arithmetic between the kernel layers (lstm_math.hpp), one thread per state element.
  * -------------------------------------------------------------------------------------------- */
 template<typename T>
-__device__ __forceinline__ T act_f_rt(int kind, T x, T p) {
-	switch (kind) {
-	case ACT_IDENTITY: return act_f<T, ACT_IDENTITY>(x, p);
-	case ACT_SCALED: return act_f<T, ACT_SCALED>(x, p);
-	case ACT_BINARY_STEP: return act_f<T, ACT_BINARY_STEP>(x, p);
-	case ACT_SIGMOID: return act_f<T, ACT_SIGMOID>(x, p);
-	case ACT_TANH: return act_f<T, ACT_TANH>(x, p);
-	case ACT_SOFTSIGN: return act_f<T, ACT_SOFTSIGN>(x, p);
-	case ACT_SOFTPLUS: return act_f<T, ACT_SOFTPLUS>(x, p);
-	case ACT_RELU: return act_f<T, ACT_RELU>(x, p);
-	case ACT_LEAKY_RELU: return act_f<T, ACT_LEAKY_RELU>(x, p);
-	case ACT_ELU: return act_f<T, ACT_ELU>(x, p);
-	default: return act_f<T, ACT_SWISH>(x, p);
-	}
-}
-
-template<typename T>
-__device__ __forceinline__ T act_b_rt(int kind, T x, T y, T g, T p) {
-	switch (kind) {
-	case ACT_IDENTITY: return act_b<T, ACT_IDENTITY>(x, y, g, p);
-	case ACT_SCALED: return act_b<T, ACT_SCALED>(x, y, g, p);
-	case ACT_BINARY_STEP: return act_b<T, ACT_BINARY_STEP>(x, y, g, p);
-	case ACT_SIGMOID: return act_b<T, ACT_SIGMOID>(x, y, g, p);
-	case ACT_TANH: return act_b<T, ACT_TANH>(x, y, g, p);
-	case ACT_SOFTSIGN: return act_b<T, ACT_SOFTSIGN>(x, y, g, p);
-	case ACT_SOFTPLUS: return act_b<T, ACT_SOFTPLUS>(x, y, g, p);
-	case ACT_RELU: return act_b<T, ACT_RELU>(x, y, g, p);
-	case ACT_LEAKY_RELU: return act_b<T, ACT_LEAKY_RELU>(x, y, g, p);
-	case ACT_ELU: return act_b<T, ACT_ELU>(x, y, g, p);
-	default: return act_b<T, ACT_SWISH>(x, y, g, p);
-	}
-}
-
-/* Offset of element (n, rest) of time step t in a sequence tensor (N, T_len, ...): element e = n + N * rest of a
- * step's slab. A slab of P elements is a whole number of samples, so gate g of element e is (n, rest + g * P / N):
- * one 32-bit division per element serves all of its accesses (the host checks that 4 P fits 32 bits). */
-__device__ __forceinline__ size_t seq_offset(unsigned n, unsigned rest, int N, int T_len, int t) {
-	return n + (size_t) N * ((size_t) t + (size_t) T_len * rest);
-}
-
-template<typename T>
 __global__ __launch_bounds__(256)
-void lstm_gates_forward_kernel(LstmActs<T> a, int N, size_t P, const T* __restrict__ zx, int zx_T, int zx_t,
-		const T* __restrict__ zh, bool mul_int, const T* __restrict__ prev_state, T* __restrict__ z, T* __restrict__ gates,
-		T* __restrict__ state, T* __restrict__ act_state, T* __restrict__ hidden, T* __restrict__ hprev_all, int h_T, int h_t,
-		T* __restrict__ out, int out_T, int out_t) {
+void lstm_gates_forward_kernel(const LstmForwardStep<T> A, const T* __restrict__ zh) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
-	const unsigned slab_rows = (unsigned) (P / (size_t) N);
-	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < P; e += stride) {
-		const unsigned rest = (unsigned) e / (unsigned) N, n = (unsigned) e - rest * (unsigned) N;
-		T y[4];
-		#pragma unroll
-		for (int g = 0; g < 4; ++g) {
-			/* weighted input + weighted previous output (:312, :327, :342, :373), their product with multiplicative
-			 * integration (:303-311); a step with only one of the two takes it as it is */
-			T v = (T) 0;
-			if (zx)
-				v = zx[seq_offset(n, rest + g * slab_rows, N, zx_T, zx_t)];
-			if (zh)
-				v = zx ? (mul_int ? v * zh[g * P + e] : v + zh[g * P + e]) : zh[g * P + e];
-			z[g * P + e] = v;
-			const int which = g < 3 ? g : 4;                        /* kinds: forget, write, candidate, state, read */
-			y[g] = act_f_rt<T>(a.kind[which], v, a.param[which]);
-			gates[g * P + e] = y[g];
+	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < A.P; e += stride) {
+		T zh4[4];
+		if (zh) {
+			#pragma unroll
+			for (int g = 0; g < 4; ++g)
+				zh4[g] = zh[g * A.P + e];
 		}
-		const T prev = prev_state ? prev_state[e] : (T) 0;
-		T s = y[0] * prev;                                          /* selective remembrance (:314) */
-		s += y[1] * y[2];                                           /* write filter * candidates (:345) */
-		state[e] = s;
-		const T as = act_f_rt<T>(a.kind[3], s, a.param[3]);
-		act_state[e] = as;
-		const T h = y[3] * as;                                      /* read filter * activated state (:383) */
-		hidden[e] = h;
-		if (hprev_all) {
-			if (h_t < h_T)
-				hprev_all[seq_offset(n, rest, N, h_T, h_t)] = h;
-			if (!prev_state)                                        /* first step: no previous output, slab 0 is zero */
-				hprev_all[seq_offset(n, rest, N, h_T, 0)] = (T) 0;
-		}
-		if (out)
-			out[seq_offset(n, rest, N, out_T, out_t)] = h;
+		lstm_forward_element<T>(A, (unsigned) e, zh ? zh4 : nullptr);
 	}
 }
 
 template<typename T>
 __global__ __launch_bounds__(256)
-void lstm_gates_backward_kernel(LstmActs<T> a, int N, size_t P, const T* __restrict__ dh, const T* __restrict__ out_grad,
-		int og_T, int og_t, const T* __restrict__ z, const T* __restrict__ gates, const T* __restrict__ prev_state,
-		const T* __restrict__ state, const T* __restrict__ act_state, T* __restrict__ state_grad, T* __restrict__ dz,
-		T* __restrict__ dzx_all, int x_T, int x_t, T* __restrict__ dzh_all, int h_T, int h_t, const T* __restrict__ zx_fwd,
-		const T* __restrict__ zh_fwd) {
+void lstm_gates_backward_kernel(const LstmBackwardStep<T> A, const T* __restrict__ dh) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
-	const unsigned slab_rows = (unsigned) (P / (size_t) N);
-	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < P; e += stride) {
-		const unsigned rest = (unsigned) e / (unsigned) N, n = (unsigned) e - rest * (unsigned) N;
-		T hg = dh ? dh[e] : (T) 0;
-		if (out_grad)
-			hg += out_grad[seq_offset(n, rest, N, og_T, og_t)];     /* :431-438 */
-		const T f = gates[e], w = gates[P + e], c = gates[2 * P + e], r = gates[3 * P + e];
-		const T as = act_state[e];
-		/* the state gradient starts at zero (:422-425) at the last time step, the one without a dh */
-		const T sg = (dh ? state_grad[e] : (T) 0) + act_b_rt<T>(a.kind[3], state[e], as, r * hg, a.param[3]);      /* :440 */
-		T d[4];
-		d[3] = act_b_rt<T>(a.kind[4], z[3 * P + e], r, as * hg, a.param[4]);                       /* :441 */
-		d[2] = act_b_rt<T>(a.kind[2], z[2 * P + e], c, w * sg, a.param[2]);                        /* :442 */
-		d[1] = act_b_rt<T>(a.kind[1], z[P + e], w, c * sg, a.param[1]);                            /* :443 */
-		d[0] = act_b_rt<T>(a.kind[0], z[e], f, (prev_state ? prev_state[e] : (T) 0) * sg, a.param[0]);   /* :444 */
-		state_grad[e] = sg * f;                                                                    /* :445 */
-		#pragma unroll
-		for (int g = 0; g < 4; ++g) {
-			/* multiplicative integration at a step with both an input and a previous output (zx_fwd and zh_fwd are that
-			 * step's weighted input and weighted output): each side's gradient carries the other side (:449-466) */
-			T to_input = d[g], to_output = d[g];
-			if (zx_fwd) {
-				to_input = zh_fwd[g * P + e] * d[g];
-				to_output = zx_fwd[seq_offset(n, rest + g * slab_rows, N, x_T, x_t)] * d[g];
-			}
-			dz[g * P + e] = to_output;                              /* what the output kernels' pass_back receives */
-			if (dzx_all)
-				dzx_all[seq_offset(n, rest + g * slab_rows, N, x_T, x_t)] = to_input;
-			if (dzh_all)        /* step 0 has no previous output to pair with: its slab is zero */
-				dzh_all[seq_offset(n, rest + g * slab_rows, N, h_T, h_t)] = prev_state ? to_output : (T) 0;
-		}
-	}
+	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < A.P; e += stride)
+		lstm_backward_element<T>(A, (unsigned) e, dh != nullptr, dh ? dh[e] : (T) 0);
 }
 
 void check_launch() {
@@ -1152,27 +1045,21 @@ void accumulate_column_sums(int N, size_t V, const T* x, T* row) {
 }
 
 template<typename T>
-void lstm_gates_forward(const LstmActs<T>& a, int N, size_t P, const T* zx, int zx_T, int zx_t, const T* zh, bool mul_int,
-		const T* prev_state, T* z, T* gates, T* state, T* act_state, T* hidden, T* hprev_all, int h_T, int h_t, T* out,
-		int out_T, int out_t) {
-	if (P == 0)
+void lstm_gates_forward(const LstmForwardStep<T>& A, const T* zh) {
+	if (A.P == 0)
 		return;
-	CATTLE_HIP_REQUIRE(P % (size_t) N == 0 && P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
-	lstm_gates_forward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, zx, zx_T, zx_t, zh, mul_int, prev_state, z, gates,
-			state, act_state, hidden, hprev_all, h_T, h_t, out, out_T, out_t);
+	CATTLE_HIP_REQUIRE(A.P % (size_t) A.N == 0 && A.P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
+	lstm_gates_forward_kernel<T><<<stream_grid(A.P), 256, 0, stream()>>>(A, zh);
 	check_launch();
 }
 
 template<typename T>
-void lstm_gates_backward(const LstmActs<T>& a, int N, size_t P, const T* dh, const T* out_grad, int og_T, int og_t, const T* z,
-		const T* gates, const T* prev_state, const T* state, const T* act_state, T* state_grad, T* dz, T* dzx_all, int x_T,
-		int x_t, T* dzh_all, int h_T, int h_t, const T* zx_fwd, const T* zh_fwd) {
-	if (P == 0)
+void lstm_gates_backward(const LstmBackwardStep<T>& A, const T* dh) {
+	if (A.P == 0)
 		return;
-	CATTLE_HIP_REQUIRE(P % (size_t) N == 0 && P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
-	CATTLE_HIP_REQUIRE((zx_fwd == nullptr) == (zh_fwd == nullptr), "multiplicative integration needs both weighted tensors");
-	lstm_gates_backward_kernel<T><<<stream_grid(P), 256, 0, stream()>>>(a, N, P, dh, out_grad, og_T, og_t, z, gates, prev_state,
-			state, act_state, state_grad, dz, dzx_all, x_T, x_t, dzh_all, h_T, h_t, zx_fwd, zh_fwd);
+	CATTLE_HIP_REQUIRE(A.P % (size_t) A.N == 0 && A.P <= 0x3fffffffu, "LSTM slab: whole samples, at most 2^30 elements");
+	CATTLE_HIP_REQUIRE((A.zx_fwd == nullptr) == (A.zh_fwd == nullptr), "multiplicative integration needs both weighted tensors");
+	lstm_gates_backward_kernel<T><<<stream_grid(A.P), 256, 0, stream()>>>(A, dh);
 	check_launch();
 }
 
@@ -1825,10 +1712,8 @@ template void accumulate_column_sums<T>(int, size_t, const T*, T*); \
 template void dropout_apply<T>(size_t, unsigned long long, T, T, const T*, T*); \
 template void broadcast_forward<T>(int, int, int, int, int, int, int, const T*, T*); \
 template void broadcast_backward<T>(int, int, int, int, int, int, int, const T*, T*); \
-template void lstm_gates_forward<T>(const LstmActs<T>&, int, size_t, const T*, int, int, const T*, bool, const T*, T*, T*, T*, T*, T*, T*, int, \
-		int, T*, int, int); \
-template void lstm_gates_backward<T>(const LstmActs<T>&, int, size_t, const T*, const T*, int, int, const T*, const T*, const T*, const T*, \
-		const T*, T*, T*, T*, int, int, T*, int, int, const T*, const T*);
+template void lstm_gates_forward<T>(const LstmForwardStep<T>&, const T*); \
+template void lstm_gates_backward<T>(const LstmBackwardStep<T>&, const T*);
 
 CATTLE_HIP_INSTANTIATE(float)
 CATTLE_HIP_INSTANTIATE(double)

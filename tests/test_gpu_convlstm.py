@@ -69,6 +69,14 @@ def test_config5_convlstm_fused():
     _check(np.float32, 32, 10, (16, 16, 8), 32, SMOOTH, True, lambda T: (1, T - 1))
 
 
+@pytest.mark.parametrize("mul_int", [False, True])
+def test_a_batch_whose_recurrent_input_gradient_runs_as_whole_tiles(mul_int):
+    """At config 5's size the input gradient of the output-side kernels is a launch whose reductions are cut into
+    parts, and the kernel that sums the parts runs the cell's backward step on the sums. With 131072 rows the same launch
+    works on whole tiles and writes the gradient tensor; the backward step is then a kernel of its own."""
+    _check(np.float32, 64, 3, (64, 32, 4), 8, SMOOTH, False, lambda T: (T, 0), mul_int=mul_int)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("foremost", [True, False])
 def test_sequence_alignments(dtype, foremost):
