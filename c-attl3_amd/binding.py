@@ -31,7 +31,7 @@ EXPORTS = [
     "cattle_hip_timer_destroy", "cattle_hip_timer_start", "cattle_hip_timer_stop", "cattle_hip_conv_create",
     "cattle_hip_transconv_create", "cattle_hip_dense_create", "cattle_hip_batchnorm_create", "cattle_hip_batchnorm_get_stats_initialized",
     "cattle_hip_batchnorm_set_stats_initialized", "cattle_hip_activation_create", "cattle_hip_pool_create",
-    "cattle_hip_convlstm_set_multiplicative_integration", "cattle_hip_layer_param_set_regularization",
+    "cattle_hip_convlstm_set_multiplicative_integration", "cattle_hip_convlstm_fused_steps", "cattle_hip_layer_param_set_regularization",
     "cattle_hip_layer_param_regularization_penalty", "cattle_hip_dropout_create", "cattle_hip_reshape_create", "cattle_hip_broadcast_create",
     "cattle_hip_layer_clone", "cattle_hip_layer_destroy", "cattle_hip_layer_input_dims",
     "cattle_hip_layer_output_dims", "cattle_hip_layer_is_input_layer", "cattle_hip_layer_set_input_layer",
@@ -574,6 +574,13 @@ class ConvLSTMNetwork(Layer):
 
     def set_multiplicative_integration(self, enabled):
         _check(lib().cattle_hip_convlstm_set_multiplicative_integration(self._h, ctypes.c_int(int(bool(enabled)))))
+
+    def fused_steps(self):
+        """(forward, backward): the time steps of the last propagate / backpropagate whose element-wise part ran inside a
+        kernel of the output-side convolutions."""
+        f, b = ctypes.c_int(), ctypes.c_int()
+        _check(lib().cattle_hip_convlstm_fused_steps(self._h, ctypes.byref(f), ctypes.byref(b)))
+        return int(f.value), int(b.value)
 
     def is_foremost(self):
         return self._foremost

@@ -150,68 +150,6 @@ template<typename T> void meanpool_backward(const PoolShape& s, int N, const T* 
 void device_zero_fill(void* dst, size_t bytes);
 /* ---- fused kernel layer: convolution or dense -> [batch norm] -> [activation] -> [pool] --------------------------- */
 
-/* What the gather GEMM does with a finished output tile besides adding the bias:
- *   EPI_NONE   out = acc + bias.
- *   EPI_ACT    out = activation(acc + bias) in the coded form of act_math.hpp; the pre-activation values go to `pre`
- *              when the activation's backward pass needs them.
- *   EPI_POOL   activation, then max pooling with windows that tile the output (stride = receptor): `out` is the pooled
- *              tensor, `inds` the arg-max cache in the layout of MaxPoolLayer (layer/pool/MaxPoolLayer.hpp:58-62), `pre`
- *              the pre-activation value at each arg-max (or null). Needs the blocked tile order with whole windows per tile.
- *   EPI_STATS  out = acc + bias, plus per tile and output column (count, mean, sum of squared deviations) of the tile's
- *              rows in `stats` [mtiles][F][3]: the batch-norm moments of the convolution output without reading it again. */
-enum { EPI_NONE = 0, EPI_ACT = 1, EPI_POOL = 2, EPI_STATS = 3 };
-template<typename T>
-struct Epilogue {
-	int kind;               /* cattle_hip_activation, element-wise kinds */
-	T p;                    /* the activation's scalar argument */
-	T* pre;
-	unsigned* inds;
-	int prh, prw;           /* pooling receptor (= stride) along height and width */
-	int OHp, OWp;           /* pooled output extents */
-	T* stats;
-};
-/* conv_forward with a fused epilogue. Returns false, having launched nothing, when the problem does not allow the
- * epilogue (no 16-byte accesses, windows that do not fit the tiles): the caller then runs the layers one by one; the
- * prepared weights `wt` are valid afterwards either way.
- * `mtiles` receives the row count of the EPI_STATS partials; conv_stats_rows() bounds it for any launch. */
-template<typename T> bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out, T* wt,
-		bool wt_ready, int epi, const Epilogue<T>& E, int* mtiles);
-size_t conv_stats_rows(const ConvShape& s, int N);
-/* The layers behind the kernel layer, on its output z (N, H, W, C): element-wise activation `kind` (argument p) and a
- * pool (0 none, 1 max, 2 mean) whose prh x prw windows tile z exactly. */
-struct ChainShape {
-	int H, W, C, prh, prw, pool, kind;
-	double p;
-};
-/* dz from the gradient g of the (pooled) output, the arg-max cache, and the coded output y or the pre-activation
- * values `pre` (both at the arg-max positions when pooled); max pooling or none */
-template<typename T> void chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* y, const T* pre, T* dz);
-/* With a per-channel batch norm between kernel layer and activation: out = pool(act(bn(z))), the channel moments merged
- * from the GEMM epilogue's per-tile moments `stats` [mtiles][C][3] (training) or taken from the running statistics. */
-size_t bn_chain_workspace(int channels);
-template<typename T> void bn_chain_forward(const ChainShape& s, int N, int mtiles, bool training, bool stats_init, const T* z,
-		const T* stats, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd, T decay, T eps, T* mean_cache, T* inv_sd_cache,
-		T* out, unsigned* inds);
-template<typename T> void bn_chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* z, const T* gamma,
-		const T* beta, const T* mean_cache, const T* inv_sd_cache, T* gamma_grad, T* beta_grad, T* dz, T* ws);
-
-/* dst[i] += src[i] */
-template<typename T> void axpy_one(size_t n, const T* src, T* dst);
-/* dst[c + cols*r] (+)= src[r + rows*c] for a column-major rows x cols matrix src */
-template<typename T> void transpose_matrix(int rows, int cols, const T* src, T* dst, bool accumulate);
-/* x[n + N*e] += row[e]  (a 1 x V row vector added to every row of an N x V matrix) */
-template<typename T> void add_row_vector(int N, size_t V, const T* row, T* x);
-/* row[e] += sum_n x[n + N*e]  (column sums of an N x V matrix, accumulated) */
-template<typename T> void accumulate_column_sums(int N, size_t V, const T* x, T* row);
-
-/* DropoutLayer: y = x * mask(u) with the uniform numbers u regenerated from `key` (the key of training pass `pass` of a
- * layer seeded with `seed` is dropout_pass_key(seed, pass)); used for the forward and the backward pass. */
-unsigned long long dropout_pass_key(unsigned long long seed, unsigned long long pass);
-template<typename T> void dropout_apply(size_t n, unsigned long long key, T prob, T eps, const T* x, T* y);
-/* BroadcastLayer on (N, H, W, C) -> (N, H bh, W bw, C bc) and the sum of the replicas back. */
-template<typename T> void broadcast_forward(int H, int W, int C, int bh, int bw, int bc, int N, const T* x, T* out);
-template<typename T> void broadcast_backward(int H, int W, int C, int bh, int bw, int bc, int N, const T* out_grad, T* in_grad);
-
 /* The element-wise part of an LSTM cell step between the kernel layers. kind/param index: 0 forget,
  * 1 write, 2 candidate, 3 state, 4 read activation (element-wise kinds only). Per-step tensors hold
  * the four gates as consecutive blocks of P elements; `*_all` tensors are (N, T, ...) over all steps. */
@@ -250,6 +188,80 @@ template<typename T> struct LstmBackwardStep {
 	int h_T, h_t;
 	const T *zx_fwd, *zh_fwd;
 };
+/* What the gather GEMM does with a finished output tile besides adding the bias:
+ *   EPI_NONE   out = acc + bias.
+ *   EPI_ACT    out = activation(acc + bias) in the coded form of act_math.hpp; the pre-activation values go to `pre`
+ *              when the activation's backward pass needs them.
+ *   EPI_POOL   activation, then max pooling with windows that tile the output (stride = receptor): `out` is the pooled
+ *              tensor, `inds` the arg-max cache in the layout of MaxPoolLayer (layer/pool/MaxPoolLayer.hpp:58-62), `pre`
+ *              the pre-activation value at each arg-max (or null). Needs the blocked tile order with whole windows per tile.
+ *   EPI_STATS  out = acc + bias, plus per tile and output column (count, mean, sum of squared deviations) of the tile's
+ *              rows in `stats` [mtiles][F][3]: the batch-norm moments of the convolution output without reading it again.
+ *   EPI_LSTM   the output columns are the four gates' weighted previous outputs of an LSTM cell; the element-wise part of
+ *              the cell's forward step (`lstm`) runs on them and `out` is not written. The prepared weights' columns are
+ *              then ordered so that a tile holds all four gates of its hidden channels (conv_forward_lstm). */
+enum { EPI_NONE = 0, EPI_ACT = 1, EPI_POOL = 2, EPI_STATS = 3, EPI_LSTM = 4 };
+template<typename T>
+struct Epilogue {
+	int kind;               /* cattle_hip_activation, element-wise kinds */
+	T p;                    /* the activation's scalar argument */
+	T* pre;
+	unsigned* inds;
+	int prh, prw;           /* pooling receptor (= stride) along height and width */
+	int OHp, OWp;           /* pooled output extents */
+	T* stats;
+	LstmForwardStep<T> lstm;
+};
+/* conv_forward with a fused epilogue. Returns false, having launched nothing, when the problem does not allow the
+ * epilogue (no 16-byte accesses, windows that do not fit the tiles): the caller then runs the layers one by one; the
+ * prepared weights `wt` are valid afterwards either way.
+ * `mtiles` receives the row count of the EPI_STATS partials; conv_stats_rows() bounds it for any launch. */
+template<typename T> bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out, T* wt,
+		bool wt_ready, int epi, const Epilogue<T>& E, int* mtiles);
+size_t conv_stats_rows(const ConvShape& s, int N);
+/* The output-side kernels of an LSTM cell step (s.F = 4 * hidden filters: forget | write | candidate | read) on the
+ * previous hidden output x (the first N of x_batch samples per position if x_batch > 0), followed in the same kernel
+ * by the element-wise part of the step: the weighted previous outputs never reach memory. `wt` (conv_workspace().wt_fwd
+ * elements) is a prepared layout of its own, not the one conv_forward builds. Returns false, having launched nothing
+ * and leaving wt alone, when the problem does not allow it (no 16-byte accesses, too many rows for the short tiles
+ * that can stage a whole tile, a hidden size that does not fill tiles with whole gate groups). */
+template<typename T> bool conv_forward_lstm(const ConvShape& s, int N, const T* x, int x_batch, const T* w, const T* b, T* wt,
+		bool wt_ready, const LstmForwardStep<T>& step);
+/* The layers behind the kernel layer, on its output z (N, H, W, C): element-wise activation `kind` (argument p) and a
+ * pool (0 none, 1 max, 2 mean) whose prh x prw windows tile z exactly. */
+struct ChainShape {
+	int H, W, C, prh, prw, pool, kind;
+	double p;
+};
+/* dz from the gradient g of the (pooled) output, the arg-max cache, and the coded output y or the pre-activation
+ * values `pre` (both at the arg-max positions when pooled); max pooling or none */
+template<typename T> void chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* y, const T* pre, T* dz);
+/* With a per-channel batch norm between kernel layer and activation: out = pool(act(bn(z))), the channel moments merged
+ * from the GEMM epilogue's per-tile moments `stats` [mtiles][C][3] (training) or taken from the running statistics. */
+size_t bn_chain_workspace(int channels);
+template<typename T> void bn_chain_forward(const ChainShape& s, int N, int mtiles, bool training, bool stats_init, const T* z,
+		const T* stats, const T* gamma, const T* beta, T* avg_mean, T* avg_inv_sd, T decay, T eps, T* mean_cache, T* inv_sd_cache,
+		T* out, unsigned* inds);
+template<typename T> void bn_chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* z, const T* gamma,
+		const T* beta, const T* mean_cache, const T* inv_sd_cache, T* gamma_grad, T* beta_grad, T* dz, T* ws);
+
+/* dst[i] += src[i] */
+template<typename T> void axpy_one(size_t n, const T* src, T* dst);
+/* dst[c + cols*r] (+)= src[r + rows*c] for a column-major rows x cols matrix src */
+template<typename T> void transpose_matrix(int rows, int cols, const T* src, T* dst, bool accumulate);
+/* x[n + N*e] += row[e]  (a 1 x V row vector added to every row of an N x V matrix) */
+template<typename T> void add_row_vector(int N, size_t V, const T* row, T* x);
+/* row[e] += sum_n x[n + N*e]  (column sums of an N x V matrix, accumulated) */
+template<typename T> void accumulate_column_sums(int N, size_t V, const T* x, T* row);
+
+/* DropoutLayer: y = x * mask(u) with the uniform numbers u regenerated from `key` (the key of training pass `pass` of a
+ * layer seeded with `seed` is dropout_pass_key(seed, pass)); used for the forward and the backward pass. */
+unsigned long long dropout_pass_key(unsigned long long seed, unsigned long long pass);
+template<typename T> void dropout_apply(size_t n, unsigned long long key, T prob, T eps, const T* x, T* y);
+/* BroadcastLayer on (N, H, W, C) -> (N, H bh, W bw, C bc) and the sum of the replicas back. */
+template<typename T> void broadcast_forward(int H, int W, int C, int bh, int bw, int bc, int N, const T* x, T* out);
+template<typename T> void broadcast_backward(int H, int W, int C, int bh, int bw, int bc, int N, const T* out_grad, T* in_grad);
+
 /* zh: the step's weighted previous output (four gate blocks of P elements), null at the first step */
 template<typename T> void lstm_gates_forward(const LstmForwardStep<T>& step, const T* zh);
 /* dh: the gradient of the hidden output that came back from the step after, null at the last step */

@@ -21,6 +21,7 @@
 #include "lstm_math.hpp"
 
 #include <algorithm>
+#include <functional>
 #include <limits>
 #include <cstdlib>
 #include <cstring>
@@ -259,11 +260,30 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 	 * of its store: sixteen to thirty-two memory round trips in a row at the end of every block. */
 	static_assert(THREADS >= BF, "one thread per bias value");
 	__shared__ T bias_s[BF];
-	if (tid < BF)
-		bias_s[tid] = (bias != nullptr && f0 + tid < g.F) ? bias[f0 + tid] : (T) 0;
+	if (tid < BF) {
+		const int fsrc = EPI == EPI_LSTM && f0 + tid < g.F ? lstm_gate_column(f0 + tid, BF / 4, g.F / 4) : f0 + tid;
+		bias_s[tid] = (bias != nullptr && f0 + tid < g.F) ? bias[fsrc] : (T) 0;
+	}
 	/* this block's chunks of the reduction: all of them, or one part */
 	const int chunk0 = split ? part * L.chunks_per_part : 0;
 	const int nchunks = split ? min(L.chunks_per_part, (g.K + KC - 1) / KC - chunk0) : (g.K + KC - 1) / KC;
+
+	/* EPI_LSTM: this thread's state elements (row idx % BM of the tile, hidden channel idx / BM of the tile's CB) and
+	 * what their forward step reads besides this kernel's own sums, fetched now and used in the epilogue */
+	constexpr int CB = BF / 4, LSTM_ELEMS = EPI == EPI_LSTM ? BM * CB / THREADS : 1;
+	unsigned lstm_e[LSTM_ELEMS];
+	LstmForwardInputs<T> lstm_in[LSTM_ELEMS];
+	if constexpr (EPI == EPI_LSTM) {
+		static_assert(BM * CB % THREADS == 0, "whole rounds of threads over a tile's state elements");
+		#pragma unroll
+		for (int it = 0; it < LSTM_ELEMS; ++it) {
+			const int idx = tid + it * THREADS, row = idx % BM, cl = idx / BM;
+			const int mrow = tile_row_m(L, g, tile, BM, row);
+			lstm_e[it] = mrow < g.M ? (unsigned) mrow + (unsigned) g.M * (unsigned) (blockIdx.y * CB + cl) : 0xffffffffu;
+			if (lstm_e[it] != 0xffffffffu)
+				lstm_in[it] = lstm_forward_load<T>(E.lstm, lstm_e[it]);
+		}
+	}
 
 	/* --- table writer state: thread t < KC walks k = k0 + t, k0 + t + KC, ... from the first chunk's k0 --- */
 	int tr, ts, tch;
@@ -473,6 +493,54 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 					vec_store<T, VS>(dst + j0, v);
 				}
 			}
+		return;
+	}
+	if constexpr (EPI == EPI_LSTM) {
+		/* The tile (bias added) goes through LDS so that the four gates of a state element, which lie in four column
+		 * groups and so in different lanes and waves, meet in one thread; the tile's own buffer, not the operand
+		 * buffers: only the short tiles have this epilogue, and theirs are too small for a whole tile. */
+		constexpr int LROW = BM + 4;
+		__shared__ __attribute__((aligned(16))) T lstm_stage[BF * LROW];
+		#pragma unroll
+		for (int i = 0; i < FB; ++i)
+			#pragma unroll
+			for (int r = 0; r < MF::NACC; ++r) {
+				const int col = wf * WT_F + FB * acc_row<T>(r, lk) + i;
+				const T bv = bias_s[col];
+				T v[MB];
+				#pragma unroll
+				for (int j = 0; j < MB; ++j)
+					v[j] = acc[i][j][r] + bv;
+				T* dst = lstm_stage + col * LROW + wm * WT_M + MB * lc;
+				#pragma unroll
+				for (int j0 = 0; j0 < MB; j0 += VS)
+					vec_store<T, VS>(dst + j0, *reinterpret_cast<T (*)[VS]>(&v[j0]));
+			}
+		__syncthreads();
+		/* the arithmetic of all of a thread's elements before the first store: independent chains that the compiler
+		 * may interleave (stores in between would keep them apart), which matters with a wavefront per SIMD */
+		LstmForwardOutputs<T> res[LSTM_ELEMS];
+		T zh4[LSTM_ELEMS][4];
+		#pragma unroll
+		for (int it = 0; it < LSTM_ELEMS; ++it) {
+			const int idx = tid + it * THREADS, row = idx % BM, cl = idx / BM;
+			#pragma unroll
+			for (int gt = 0; gt < 4; ++gt)
+				zh4[it][gt] = lstm_stage[(gt * CB + cl) * LROW + row];
+		}
+		if (lstm_standard_acts(E.lstm.a)) {
+			#pragma unroll
+			for (int it = 0; it < LSTM_ELEMS; ++it)
+				res[it] = lstm_forward_compute<T, true>(E.lstm, lstm_in[it], zh4[it]);
+		} else {
+			#pragma unroll
+			for (int it = 0; it < LSTM_ELEMS; ++it)
+				res[it] = lstm_forward_compute<T, false>(E.lstm, lstm_in[it], zh4[it]);
+		}
+		#pragma unroll
+		for (int it = 0; it < LSTM_ELEMS; ++it)
+			if (lstm_e[it] != 0xffffffffu)
+				lstm_forward_store<T>(E.lstm, lstm_e[it], res[it]);
 		return;
 	}
 	if constexpr (EPI == EPI_POOL) {
@@ -1074,14 +1142,17 @@ void reduce_partials_wide_kernel(const T* __restrict__ partials, T* __restrict__
 		dst[i] += s;
 }
 
-/* Forward weights: wt[k][f] = w[k + K*f], zero-padded to Kp rows x ldw columns. */
+/* Forward weights: wt[k][f] = w[k + K*f], zero-padded to Kp rows x ldw columns. gate_block > 0: the columns in the
+ * order of lstm_gate_column (F = 4 * hidden). */
 template<typename T>
-__global__ void prep_fwd_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, int K, int F, int Kp, int ldw) {
+__global__ void prep_fwd_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, int K, int F, int Kp, int ldw,
+		int gate_block = 0) {
 	const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
 	if (i >= (size_t) Kp * ldw)
 		return;
 	const int f = (int) (i % ldw), k = (int) (i / ldw);
-	wt[i] = (k < K && f < F) ? w[(size_t) k + (size_t) K * f] : (T) 0;
+	const int fs = gate_block > 0 && f < F ? lstm_gate_column(f, gate_block, F / 4) : f;
+	wt[i] = (k < K && f < F) ? w[(size_t) k + (size_t) K * fs] : (T) 0;
 }
 
 /* Input-gradient weights: wt[k' = rh + RH*(rw + RW*f)][c] = w[rh + RH*(rw + RW*c) + K*f]. */
@@ -1266,7 +1337,10 @@ void split_reduce_lstm_backward_kernel(const T* __restrict__ partials, const Gat
 	const int m = tile_row_m(L, g, tile, BM, e % BM), f = fb * BF + e / BM;
 	if (m >= g.M || f >= g.F)
 		return;
-	lstm_backward_element<T>(A, (unsigned) m + (unsigned) g.M * (unsigned) f, true, acc);
+	if (lstm_standard_acts(A.a))
+		lstm_backward_element<T, true>(A, (unsigned) m + (unsigned) g.M * (unsigned) f, true, acc);
+	else
+		lstm_backward_element<T, false>(A, (unsigned) m + (unsigned) g.M * (unsigned) f, true, acc);
 }
 
 /* One instantiation of gather_gemm_kernel and what the tile chooser needs to know about it. */
@@ -1287,7 +1361,12 @@ void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, con
 	dim3 block(64 * WAVES_M * WAVES_F);
 	if (epi != EPI_NONE) {
 		CATTLE_HIP_REQUIRE(vec && !divs, "a fused epilogue needs the vectorised forward form of the GEMM");
-		if (epi == EPI_ACT)
+		if (epi == EPI_LSTM) {
+			if constexpr (WAVES_M * WT_M <= 128)
+				gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_LSTM, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+			else
+				throw Error(ERR_INVALID, "the LSTM epilogue exists for the short tiles only");
+		} else if (epi == EPI_ACT)
 			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 		else if (epi == EPI_POOL)
 			gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
@@ -1308,14 +1387,19 @@ template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int P
 int gather_variant_occupancy(size_t dyn, bool vec, bool divs, int epi) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	/* the answer for the usual launch (no reserved dynamic LDS) is kept: one query per kernel instantiation */
-	static int cached[7] = { 0, 0, 0, 0, 0, 0, 0 };
+	static int cached[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
 	int& slot = cached[epi != EPI_NONE ? 3 + epi : (vec ? 2 : 0) + (divs ? 1 : 0)];
 	if (dyn == 0 && slot > 0)
 		return slot;
 	int n = 0;
 	hipError_t e;
 	constexpr int TH = 64 * WAVES_M * WAVES_F;
-	if (epi == EPI_ACT)
+	if (epi == EPI_LSTM) {
+		if constexpr (WAVES_M * WT_M <= 128)
+			e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_LSTM, PF>, TH, dyn);
+		else
+			return 0;
+	} else if (epi == EPI_ACT)
 		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_ACT, PF>, TH, dyn);
 	else if (epi == EPI_POOL)
 		e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_POOL, PF>, TH, dyn);
@@ -1489,7 +1573,7 @@ RowBlocks plan_row_blocks(const GatherGeom& g, int bm, int prh, int prw, bool po
 template<typename T>
 bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, ScratchArena* arena = nullptr,
 		int epi = EPI_NONE, const Epilogue<T>* E = nullptr, int* mtiles_out = nullptr, const LstmBackwardStep<T>* then = nullptr,
-		bool* then_done = nullptr) {
+		bool* then_done = nullptr, const std::function<void(int bf)>* before_launch = nullptr) {
 	const bool vec = g.N % GemmCfg<T>::VEC == 0 && g.NS % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
 	const bool divs = g.DA != 1 || g.DB != 1;
 	if (epi != EPI_NONE && (!vec || divs || (reinterpret_cast<uintptr_t>(out) & 15) != 0))
@@ -1554,6 +1638,14 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 			return false;
 	}
 	const GatherVariant<T>& v = vars[best_v];
+	if (epi == EPI_LSTM) {
+		/* a short tile (it stages itself whole) whose column groups are whole gate groups of the hidden channels */
+		const int hidden = g.F / 4;
+		if (v.bm > 128 || g.F % 4 != 0 || hidden % (v.bf / 4) != 0 || (size_t) g.M * hidden != E->lstm.P)
+			return false;
+	}
+	if (before_launch)
+		(*before_launch)(v.bf);
 	size_t dyn = 0;
 	if (occ >= 1 && occ <= 8) {
 		const int want_bytes = device_shape().lds_per_cu / (occ + 1) + 256;
@@ -1586,8 +1678,8 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	/* blocks the chip holds at once (registers, LDS, waves), as the runtime computes it for this kernel */
 	const int per_cu = std::max(1, v.blocks_per_cu(dyn, vec, divs, epi));
 	const int slots = device_shape().cus * per_cu;
-	const bool no_split = tune.no_split || epi == EPI_POOL || epi == EPI_STATS;
-	const Epilogue<T> none = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr };
+	const bool no_split = tune.no_split || epi == EPI_POOL || epi == EPI_STATS || epi == EPI_LSTM;
+	const Epilogue<T> none = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr, {} };
 	const Epilogue<T>& epi_args = E ? *E : none;
 
 	/* main_count whole tiles, the other mtiles - main_count with their reduction cut into about `ksplit` parts */
@@ -1874,6 +1966,26 @@ void conv_forward(const ConvShape& s, int N, const T* x, const T* w, const T* b,
 }
 
 template<typename T>
+bool conv_forward_lstm(const ConvShape& s, int N, const T* x, int x_batch, const T* w, const T* b, T* wt, bool wt_ready,
+		const LstmForwardStep<T>& step) {
+	check_sizes(s, std::max(N, x_batch));
+	GatherGeom g = forward_geom(s, N);
+	if (x_batch > 0)
+		g.NS = x_batch;
+	Epilogue<T> E = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr, step };
+	/* the prepared columns depend on the tile width, which the launcher chooses */
+	const std::function<void(int)> prepare = [&](int bf) {
+		if (wt_ready)
+			return;
+		const int Kp = round_up(g.K, WT_ROW_PAD);
+		const size_t count = (size_t) Kp * g.ldw;
+		prep_fwd_weights_kernel<T><<<(unsigned) ((count + 255) / 256), 256, 0, stream()>>>(w, wt, g.K, g.F, Kp, g.ldw, bf / 4);
+		CATTLE_HIP_CHECK(hipGetLastError());
+	};
+	return launch_gather<T>(x, wt, b, (T*) nullptr, g, nullptr, EPI_LSTM, &E, nullptr, nullptr, nullptr, &prepare);
+}
+
+template<typename T>
 bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out, T* wt, bool wt_ready, int epi,
 		const Epilogue<T>& E, int* mtiles) {
 	check_sizes(s, N);
@@ -2004,6 +2116,10 @@ template bool conv_forward_fused<float>(const ConvShape&, int, const float*, con
 		const Epilogue<float>&, int*);
 template bool conv_forward_fused<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*, bool, int,
 		const Epilogue<double>&, int*);
+template bool conv_forward_lstm<float>(const ConvShape&, int, const float*, int, const float*, const float*, float*, bool,
+		const LstmForwardStep<float>&);
+template bool conv_forward_lstm<double>(const ConvShape&, int, const double*, int, const double*, const double*, double*, bool,
+		const LstmForwardStep<double>&);
 template void conv_forward_static<float>(const ConvShape&, int, const float*, const float*, const float*, float*);
 template void conv_forward_static<double>(const ConvShape&, int, const double*, const double*, const double*, double*);
 template void conv_backward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, float*,

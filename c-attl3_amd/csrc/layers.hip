@@ -11,6 +11,7 @@
 #include "../../include/cattle_hip.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -473,6 +474,7 @@ struct ConvLstm : LayerBase {
 	LstmActs<T> acts;
 	bool foremost;
 	bool mul_int = false;           /* LSTMNeuralNetwork<Scalar,Rank,MulInt = true> (:44, :303-311) */
+	int fused_forward_steps = 0, fused_backward_steps = 0;      /* of the last propagate / backpropagate */
 	/* alignment of the last propagate (:398-401) */
 	size_t T_in = 0, T_out = 0, delay = 0, steps = 0;
 	const T* x_cache = nullptr;
@@ -545,20 +547,40 @@ struct ConvLstm : LayerBase {
 		hprev_all.ensure(p * total * e);
 		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
 		T* wth = (T*) wh.derived[0].ensure(wsh.wt_fwd * e);
+		/* CATTLE_HIP_NO_LSTM_FUSION (experiments; read once): every step's element-wise part as a kernel of its own */
+		static const bool no_fusion = std::getenv("CATTLE_HIP_NO_LSTM_FUSION") != nullptr;
+		bool fused_steps = !no_fusion;
+		fused_forward_steps = 0;
+		T* wth_gates = nullptr;             /* the prepared layout of the kernel that runs the step itself */
 		for (size_t t = 0; t < total; ++t) {
 			const bool has_in = t < in_len, has_prev = t > 0;
-			T* zh_t = step(zh, mul_int ? t : 0, 4 * p);
-			if (has_prev) {
-				/* the previous hidden output where the previous step left it: slab t of (N, total, H, W, hidden) */
-				conv_forward<T>(sh, n, (const T*) hprev_all.p + N * t, (const T*) wh.values.p, (const T*) params[3]->values.p, zh_t,
-						wth, wh.derived_version[0] == wh.version, (int) (N * total));
-				wh.derived_version[0] = wh.version;
-			}
 			const bool emits = t >= out_delay && t < out_delay + out_len;      /* :386-393 */
 			const LstmForwardStep<T> fs = { acts, n, p, has_in ? (const T*) zx_all.p : nullptr, (int) in_len, (int) t, mul_int,
 					has_prev ? step(state, t - 1, p) : nullptr, keeps_z() ? step(z, t, 4 * p) : nullptr, step(gates, t, 4 * p),
 					step(state, t, p), step(act_state, t, p), (T*) hprev_all.p, (int) total, (int) (t + 1), emits ? out : nullptr,
 					(int) out_len, (int) (t - out_delay) };
+			/* the previous hidden output where the previous step left it: slab t of (N, total, H, W, hidden) */
+			const T* hprev = (const T*) hprev_all.p + N * t;
+			if (has_prev && !mul_int && fused_steps) {
+				/* the output-side kernels and the element-wise part of the step in one launch where the problem allows:
+				 * the weighted previous output then exists only inside that kernel (with multiplicative integration
+				 * the backward pass reads it, so it has to be stored) */
+				if (!wth_gates)
+					wth_gates = (T*) wh.derived[2].ensure(wsh.wt_fwd * e);
+				if (conv_forward_lstm<T>(sh, n, hprev, (int) (N * total), (const T*) wh.values.p, (const T*) params[3]->values.p,
+						wth_gates, wh.derived_version[2] == wh.version, fs)) {
+					wh.derived_version[2] = wh.version;
+					++fused_forward_steps;
+					continue;
+				}
+				fused_steps = false;            /* the answer depends on the shapes only: do not ask again */
+			}
+			T* zh_t = step(zh, mul_int ? t : 0, 4 * p);
+			if (has_prev) {
+				conv_forward<T>(sh, n, hprev, (const T*) wh.values.p, (const T*) params[3]->values.p, zh_t,
+						wth, wh.derived_version[0] == wh.version, (int) (N * total));
+				wh.derived_version[0] = wh.version;
+			}
 			lstm_gates_forward<T>(fs, has_prev ? (const T*) zh_t : nullptr);
 		}
 		x_cache = input;
@@ -589,17 +611,21 @@ struct ConvLstm : LayerBase {
 					both ? (const T*) step(zh, t, 4 * p) : nullptr };
 			return bs;
 		};
+		fused_backward_steps = 0;
 		if (total > 0)
 			lstm_gates_backward<T>(backward_step(total - 1), (const T*) nullptr);
 		for (size_t t = total; t-- > 1;) {
 			/* the four output-side kernels' pass_back, summed (:470-473, :491-494), is one input-gradient launch, and
 			 * the element-wise part of step t - 1, which is all that reads its result, runs in the kernel that sums the
 			 * parts of that launch's reductions when the launch has such a kernel */
+			static const bool no_fusion = std::getenv("CATTLE_HIP_NO_LSTM_FUSION") != nullptr;
 			const LstmBackwardStep<T> before = backward_step(t - 1);
 			const bool done = conv_input_gradient<T>(sh, n, (const T*) wh.values.p, (const T*) dzh_all.p + N * t, (T*) dh.p, wtd,
-					wh.derived_version[1] == wh.version, &before, (int) (N * total));
+					wh.derived_version[1] == wh.version, no_fusion ? nullptr : &before, (int) (N * total));
 			wh.derived_version[1] = wh.version;
-			if (!done)
+			if (done)
+				++fused_backward_steps;
+			else
 				lstm_gates_backward<T>(before, (const T*) dh.p);
 		}
 		/* parameter gradients of all steps at once: slab 0 of dzh_all and of hprev_all is zero */
@@ -1909,6 +1935,18 @@ int cattle_hip_convlstm_set_multiplicative_integration(cattle_hip_layer_t lstm, 
 		CATTLE_HIP_REQUIRE(f || d, "not a ConvLSTM handle");
 		(f ? f->mul_int : d->mul_int) = enabled != 0;
 		l->empty_cache();           /* the caches of a pass made under the other rule do not fit this one */
+	});
+}
+
+int cattle_hip_convlstm_fused_steps(cattle_hip_layer_t lstm, int* forward_steps, int* backward_steps) {
+	return guarded([&] {
+		LayerBase* l = as_layer(lstm);
+		ConvLstm<float>* f = dynamic_cast<ConvLstm<float>*>(l);
+		ConvLstm<double>* d = dynamic_cast<ConvLstm<double>*>(l);
+		CATTLE_HIP_REQUIRE(f || d, "not a ConvLSTM handle");
+		CATTLE_HIP_REQUIRE(forward_steps != nullptr && backward_steps != nullptr, "null output pointer");
+		*forward_steps = f ? f->fused_forward_steps : d->fused_forward_steps;
+		*backward_steps = f ? f->fused_backward_steps : d->fused_backward_steps;
 	});
 }
 

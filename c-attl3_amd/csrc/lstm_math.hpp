@@ -49,6 +49,30 @@ __device__ __forceinline__ T act_b_rt(int kind, T x, T y, T g, T p) {
 	}
 }
 
+/* The usual cell: sigmoid gates, tanh on the candidates and on the state. Kernels test for it once and run the
+ * arithmetic with the kinds known at compile time (STD): straight-line code whose independent elements the compiler can
+ * interleave, where the run-time switch is a chain of branches per activation. */
+template<typename T>
+__device__ __forceinline__ bool lstm_standard_acts(const LstmActs<T>& a) {
+	return a.kind[0] == ACT_SIGMOID && a.kind[1] == ACT_SIGMOID && a.kind[2] == ACT_TANH && a.kind[3] == ACT_TANH &&
+			a.kind[4] == ACT_SIGMOID;
+}
+/* activation WHICH of the cell (0 forget, 1 write, 2 candidate, 3 state, 4 read) */
+template<typename T, bool STD, int WHICH>
+__device__ __forceinline__ T lstm_act_f(const LstmActs<T>& a, T x) {
+	if constexpr (STD)
+		return act_f<T, (WHICH == 2 || WHICH == 3) ? ACT_TANH : ACT_SIGMOID>(x, (T) 0);
+	else
+		return act_f_rt<T>(a.kind[WHICH], x, a.param[WHICH]);
+}
+template<typename T, bool STD, int WHICH>
+__device__ __forceinline__ T lstm_act_b(const LstmActs<T>& a, T x, T y, T g) {
+	if constexpr (STD)
+		return act_b<T, (WHICH == 2 || WHICH == 3) ? ACT_TANH : ACT_SIGMOID>(x, y, g, (T) 0);
+	else
+		return act_b_rt<T>(a.kind[WHICH], x, y, g, a.param[WHICH]);
+}
+
 /* Offset of element (n, rest) of time step t in a sequence tensor (N, T_len, ...): element e = n + N * rest of a
  * step's slab. A slab of P elements is a whole number of samples, so gate g of element e is (n, rest + g * P / N):
  * one 32-bit division per element serves all of its accesses (the host checks that 4 P fits 32 bits). */
@@ -56,55 +80,92 @@ __device__ __forceinline__ size_t seq_offset(unsigned n, unsigned rest, int N, i
 	return n + (size_t) N * ((size_t) t + (size_t) T_len * rest);
 }
 
-/* Forward step of element e. zh4: the weighted previous output of the element's four gates (bias included), or null
- * at the first step. */
+/* Column of the weight matrix [forget | write | candidate | read] (hidden columns each) that sits at column f of the
+ * layout whose groups of 4 cb columns hold the four gates of cb hidden channels: gate (f / cb) % 4 of channel
+ * (f / (4 cb)) cb + f % cb. */
+__host__ __device__ __forceinline__ int lstm_gate_column(int f, int cb, int hidden) {
+	return ((f / cb) & 3) * hidden + (f / (4 * cb)) * cb + f % cb;
+}
+
+/* What the forward step of an element reads besides the weighted previous output. */
+template<typename T> struct LstmForwardInputs { T zx[4]; T prev; };
+
 template<typename T>
-__device__ __forceinline__ void lstm_forward_element(const LstmForwardStep<T>& A, unsigned e, const T* zh4) {
-	const unsigned N = (unsigned) A.N, P = (unsigned) A.P;
-	const unsigned slab_rows = P / N;
+__device__ __forceinline__ LstmForwardInputs<T> lstm_forward_load(const LstmForwardStep<T>& A, unsigned e) {
+	const unsigned N = (unsigned) A.N, slab_rows = (unsigned) A.P / N;
 	const unsigned rest = e / N, n = e - rest * N;
-	/* every load of the element before its first store: the tensors are not declared free of aliases, and a store
-	 * between two loads would make the second wait for the first */
-	T v[4], y[4];
+	LstmForwardInputs<T> in;
+	#pragma unroll
+	for (int g = 0; g < 4; ++g)
+		in.zx[g] = A.zx ? A.zx[seq_offset(n, rest + g * slab_rows, A.N, A.zx_T, A.zx_t)] : (T) 0;
+	in.prev = A.prev_state ? A.prev_state[e] : (T) 0;
+	return in;
+}
+
+/* What the forward step of an element writes: the gates' pre-activation values and values, the state, the activated
+ * state and the hidden output. */
+template<typename T> struct LstmForwardOutputs { T v[4], y[4], s, as, h; };
+
+/* The arithmetic of the forward step, registers only. zh4: the weighted previous output of the element's four gates
+ * (bias included), or null at the first step. */
+template<typename T, bool STD = false>
+__device__ __forceinline__ LstmForwardOutputs<T> lstm_forward_compute(const LstmForwardStep<T>& A, const LstmForwardInputs<T>& in,
+		const T* zh4) {
+	LstmForwardOutputs<T> o;
 	#pragma unroll
 	for (int g = 0; g < 4; ++g) {
 		/* weighted input + weighted previous output (:312, :327, :342, :373), their product with multiplicative
 		 * integration (:303-311); a step with only one of the two takes it as it is */
-		v[g] = (T) 0;
-		if (A.zx)
-			v[g] = A.zx[seq_offset(n, rest + g * slab_rows, A.N, A.zx_T, A.zx_t)];
+		T v = in.zx[g];
 		if (zh4)
-			v[g] = A.zx ? (A.mul_int ? v[g] * zh4[g] : v[g] + zh4[g]) : zh4[g];
+			v = A.zx ? (A.mul_int ? v * zh4[g] : v + zh4[g]) : zh4[g];
+		o.v[g] = v;
 	}
-	const T prev = A.prev_state ? A.prev_state[e] : (T) 0;
+	o.y[0] = lstm_act_f<T, STD, 0>(A.a, o.v[0]);
+	o.y[1] = lstm_act_f<T, STD, 1>(A.a, o.v[1]);
+	o.y[2] = lstm_act_f<T, STD, 2>(A.a, o.v[2]);
+	o.y[3] = lstm_act_f<T, STD, 4>(A.a, o.v[3]);                /* the fourth gate is the read filter */
+	o.s = o.y[0] * in.prev;                                     /* selective remembrance (:314) */
+	o.s += o.y[1] * o.y[2];                                     /* write filter * candidates (:345) */
+	o.as = lstm_act_f<T, STD, 3>(A.a, o.s);
+	o.h = o.y[3] * o.as;                                        /* read filter * activated state (:383) */
+	return o;
+}
+
+template<typename T>
+__device__ __forceinline__ void lstm_forward_store(const LstmForwardStep<T>& A, unsigned e, const LstmForwardOutputs<T>& o) {
+	const unsigned N = (unsigned) A.N, P = (unsigned) A.P;
+	const unsigned rest = e / N, n = e - rest * N;
 	#pragma unroll
 	for (int g = 0; g < 4; ++g) {
 		if (A.z)
-			A.z[(size_t) g * P + e] = v[g];
-		const int which = g < 3 ? g : 4;                        /* kinds: forget, write, candidate, state, read */
-		y[g] = act_f_rt<T>(A.a.kind[which], v[g], A.a.param[which]);
-		A.gates[(size_t) g * P + e] = y[g];
+			A.z[(size_t) g * P + e] = o.v[g];
+		A.gates[(size_t) g * P + e] = o.y[g];
 	}
-	T s = y[0] * prev;                                          /* selective remembrance (:314) */
-	s += y[1] * y[2];                                           /* write filter * candidates (:345) */
-	A.state[e] = s;
-	const T as = act_f_rt<T>(A.a.kind[3], s, A.a.param[3]);
-	A.act_state[e] = as;
-	const T h = y[3] * as;                                      /* read filter * activated state (:383) */
+	A.state[e] = o.s;
+	A.act_state[e] = o.as;
 	if (A.hprev_all) {
 		if (A.h_t < A.h_T)
-			A.hprev_all[seq_offset(n, rest, A.N, A.h_T, A.h_t)] = h;
+			A.hprev_all[seq_offset(n, rest, A.N, A.h_T, A.h_t)] = o.h;
 		if (!A.prev_state)                                      /* first step: no previous output, slab 0 is zero */
 			A.hprev_all[seq_offset(n, rest, A.N, A.h_T, 0)] = (T) 0;
 	}
 	if (A.out)
-		A.out[seq_offset(n, rest, A.N, A.out_T, A.out_t)] = h;
+		A.out[seq_offset(n, rest, A.N, A.out_T, A.out_t)] = o.h;
+}
+
+/* Every load of the element comes before its first store: the tensors are not declared free of aliases, and a store
+ * between two loads would make the second wait for the first. */
+template<typename T, bool STD = false>
+__device__ __forceinline__ void lstm_forward_element(const LstmForwardStep<T>& A, unsigned e, const T* zh4) {
+	const LstmForwardInputs<T> in = lstm_forward_load<T>(A, e);
+	lstm_forward_store<T>(A, e, lstm_forward_compute<T, STD>(A, in, zh4));
 }
 
 /* Backward step of element e. dh: the gradient of the element's hidden output that came back through the next
  * step's output-side kernels; has_dh is false at the last time step, where there is none and the state gradient
  * starts at zero (:422-425). */
-template<typename T>
+template<typename T, bool STD = false>
 __device__ __forceinline__ void lstm_backward_element(const LstmBackwardStep<T>& A, unsigned e, bool has_dh, T dh) {
 	const unsigned N = (unsigned) A.N, P = (unsigned) A.P;
 	const unsigned slab_rows = P / N;
@@ -114,7 +175,7 @@ __device__ __forceinline__ void lstm_backward_element(const LstmBackwardStep<T>&
 		hg += A.out_grad[seq_offset(n, rest, A.N, A.og_T, A.og_t)];       /* :431-438 */
 	const T f = A.gates[e], w = A.gates[(size_t) P + e], c = A.gates[(size_t) 2 * P + e], r = A.gates[(size_t) 3 * P + e];
 	const T as = A.act_state[e];
-	const T sg = (has_dh ? A.state_grad[e] : (T) 0) + act_b_rt<T>(A.a.kind[3], A.state[e], as, r * hg, A.a.param[3]);      /* :440 */
+	const T sg = (has_dh ? A.state_grad[e] : (T) 0) + lstm_act_b<T, STD, 3>(A.a, A.state[e], as, r * hg);      /* :440 */
 	T zin[4] = { (T) 0, (T) 0, (T) 0, (T) 0 };
 	if (A.z) {
 		#pragma unroll
@@ -122,10 +183,10 @@ __device__ __forceinline__ void lstm_backward_element(const LstmBackwardStep<T>&
 			zin[g] = A.z[(size_t) g * P + e];
 	}
 	T d[4];
-	d[3] = act_b_rt<T>(A.a.kind[4], zin[3], r, as * hg, A.a.param[4]);                       /* :441 */
-	d[2] = act_b_rt<T>(A.a.kind[2], zin[2], c, w * sg, A.a.param[2]);                        /* :442 */
-	d[1] = act_b_rt<T>(A.a.kind[1], zin[1], w, c * sg, A.a.param[1]);                            /* :443 */
-	d[0] = act_b_rt<T>(A.a.kind[0], zin[0], f, (A.prev_state ? A.prev_state[e] : (T) 0) * sg, A.a.param[0]);  /* :444 */
+	d[3] = lstm_act_b<T, STD, 4>(A.a, zin[3], r, as * hg);                       /* :441 */
+	d[2] = lstm_act_b<T, STD, 2>(A.a, zin[2], c, w * sg);                        /* :442 */
+	d[1] = lstm_act_b<T, STD, 1>(A.a, zin[1], w, c * sg);                            /* :443 */
+	d[0] = lstm_act_b<T, STD, 0>(A.a, zin[0], f, (A.prev_state ? A.prev_state[e] : (T) 0) * sg);  /* :444 */
 	/* multiplicative integration at a step with both an input and a previous output (zx_fwd and zh_fwd are that
 	 * step's weighted input and weighted output): each side's gradient carries the other side (:449-466) */
 	T to_input[4], to_output[4];

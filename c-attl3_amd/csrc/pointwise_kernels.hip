@@ -767,7 +767,10 @@ void lstm_gates_forward_kernel(const LstmForwardStep<T> A, const T* __restrict__
 			for (int g = 0; g < 4; ++g)
 				zh4[g] = zh[g * A.P + e];
 		}
-		lstm_forward_element<T>(A, (unsigned) e, zh ? zh4 : nullptr);
+		if (lstm_standard_acts(A.a))
+			lstm_forward_element<T, true>(A, (unsigned) e, zh ? zh4 : nullptr);
+		else
+			lstm_forward_element<T, false>(A, (unsigned) e, zh ? zh4 : nullptr);
 	}
 }
 
@@ -775,8 +778,12 @@ template<typename T>
 __global__ __launch_bounds__(256)
 void lstm_gates_backward_kernel(const LstmBackwardStep<T> A, const T* __restrict__ dh) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
-	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < A.P; e += stride)
-		lstm_backward_element<T>(A, (unsigned) e, dh != nullptr, dh ? dh[e] : (T) 0);
+	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < A.P; e += stride) {
+		if (lstm_standard_acts(A.a))
+			lstm_backward_element<T, true>(A, (unsigned) e, dh != nullptr, dh ? dh[e] : (T) 0);
+		else
+			lstm_backward_element<T, false>(A, (unsigned) e, dh != nullptr, dh ? dh[e] : (T) 0);
+	}
 }
 
 void check_launch() {

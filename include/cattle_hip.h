@@ -422,6 +422,14 @@ int cattle_hip_convlstm_get_kernel_grad(cattle_hip_layer_t lstm, size_t kernel, 
  * (:303-311, :318-326, :334-342, :369-377; gradients :449-466). Off when the network is created. Changing it empties the
  * caches: propagate again before backpropagate. */
 int cattle_hip_convlstm_set_multiplicative_integration(cattle_hip_layer_t lstm, int enabled);
+/* How the last propagate and the last backpropagate ran (no counterpart in the reference; for tests and profiles): the
+ * number of time steps whose element-wise part (gate activations and state update, :283-394; their backward, :436-466)
+ * ran inside a kernel of the output-side convolutions instead of a kernel of its own - forward in the epilogue of the
+ * convolution, backward in the kernel that sums the parts of the input gradient's reductions. Which steps can depends
+ * on the shapes only (batch sizes with 16-byte rows, problems small enough for the short tiles, hidden sizes that are
+ * multiples of 8 or 16, no multiplicative integration for the forward step); results are the same either way to
+ * rounding. */
+int cattle_hip_convlstm_fused_steps(cattle_hip_layer_t lstm, int* forward_steps, int* backward_steps);
 
 #ifdef __cplusplus
 }

@@ -65,8 +65,40 @@ def _check(dtype, N, T_in, dims, hidden, acts, foremost, seq, seed=7, conv_kw=No
 
 
 def test_config5_convlstm_fused():
-    """BASELINE config 5: T=10, batch 32, 16x16x8 input, 32 hidden channels, output = last hidden state."""
-    _check(np.float32, 32, 10, (16, 16, 8), 32, SMOOTH, True, lambda T: (1, T - 1))
+    """BASELINE config 5: T=10, batch 32, 16x16x8 input, 32 hidden channels, output = last hidden state. At this size
+    every step after the first runs its element-wise part inside the output-side convolution (forward) and inside the
+    kernel that sums the parts of that convolution's input gradient (backward)."""
+    net, _, _ = _check(np.float32, 32, 10, (16, 16, 8), 32, SMOOTH, True, lambda T: (1, T - 1))
+    assert net.fused_steps() == (9, 9)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("acts", [SMOOTH, EXOTIC], ids=["smooth", "exotic"])
+def test_steps_inside_the_recurrent_kernels(dtype, acts):
+    """Hidden sizes that fill the tiles' column groups with whole gate groups (multiples of 8 with 32 output columns,
+    of 16 with more) and batch sizes with 16-byte rows: the forward step runs in the convolution's epilogue. Both
+    precisions, the usual activations (compile-time kinds) and others (run-time kinds, pre-activation values kept)."""
+    # (the unbounded activations of EXOTIC grow from step to step, faster with more hidden channels: fewer steps for them)
+    smooth = acts is SMOOTH
+    T_in = 4 if smooth else 3
+    net, _, _ = _check(dtype, 8, T_in, (6, 5, 3), 8, acts, False, lambda T: (T, 0))
+    assert net.fused_steps() == (T_in - 1, T_in - 1)
+    if smooth:
+        net, _, _ = _check(dtype, 8, 3, (6, 5, 3), 16, acts, False, lambda T: (2, 2))      # runs one step past the input
+        assert net.fused_steps() == (3, 3)
+        net, _, _ = _check(dtype, 4, 3, (4, 4, 2), 48, acts, True, lambda T: (1, T - 1))   # three column tiles
+        assert net.fused_steps() == (2, 2)
+    else:
+        net, _, _ = _check(dtype, 8, 2, (6, 5, 3), 16, acts, False, lambda T: (T, 0))
+        assert net.fused_steps() == (1, 1)
+    # a hidden size that does not fill the column groups, a batch size without 16-byte rows: kernels of their own
+    net, _, _ = _check(dtype, 8, 2, (6, 5, 3), 12, acts, False, lambda T: (T, 0))
+    assert net.fused_steps()[0] == 0
+    net, _, _ = _check(dtype, 5, 2, (6, 5, 3), 8, acts, False, lambda T: (T, 0))
+    assert net.fused_steps()[0] == 0
+    # multiplicative integration keeps the weighted previous outputs for the backward pass: no fused forward step
+    net, _, _ = _check(dtype, 8, 2, (6, 5, 3), 8, acts, False, lambda T: (T, 0), mul_int=True)
+    assert net.fused_steps()[0] == 0
 
 
 @pytest.mark.parametrize("mul_int", [False, True])
@@ -74,7 +106,8 @@ def test_a_batch_whose_recurrent_input_gradient_runs_as_whole_tiles(mul_int):
     """At config 5's size the input gradient of the output-side kernels is a launch whose reductions are cut into
     parts, and the kernel that sums the parts runs the cell's backward step on the sums. With 131072 rows the same launch
     works on whole tiles and writes the gradient tensor; the backward step is then a kernel of its own."""
-    _check(np.float32, 64, 3, (64, 32, 4), 8, SMOOTH, False, lambda T: (T, 0), mul_int=mul_int)
+    net, _, _ = _check(np.float32, 64, 3, (64, 32, 4), 8, SMOOTH, False, lambda T: (T, 0), mul_int=mul_int)
+    assert net.fused_steps() == (0, 0)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
