@@ -431,6 +431,16 @@ public:
 	inline void set_regularization(std::size_t index, Scalar l1_lambda, Scalar l2_lambda) {
 		check(cattle_hip_layer_param_set_regularization(handle, index, (double) l1_lambda, (double) l2_lambda));
 	}
+	/**
+	 * The value and gradient constraints of parameter `index` (the weight_clip, weight_max_l1_norm, weight_max_l2_norm,
+	 * weight_grad_clip, ... arguments of the reference's kernel layers, parameters/StandardParameters.hpp:61-76; 0 = none),
+	 * enforced where StandardParameters enforces them (:105-123, :150-182).
+	 */
+	inline void set_constraints(std::size_t index, Scalar value_clip, Scalar value_max_l1_norm, Scalar value_max_l2_norm,
+			Scalar grad_clip, Scalar grad_max_l1_norm, Scalar grad_max_l2_norm) {
+		check(cattle_hip_layer_param_set_constraints(handle, index, (double) value_clip, (double) value_max_l1_norm,
+				(double) value_max_l2_norm, (double) grad_clip, (double) grad_max_l1_norm, (double) grad_max_l2_norm));
+	}
 	/** The sum of Parameters::get_regularization_penalty over the layer's parameters (optimizer/SGDOptimizer.hpp:62). */
 	inline Scalar get_regularization_penalty() const {
 		const std::size_t n = num_params();

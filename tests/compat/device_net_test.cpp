@@ -141,6 +141,25 @@ static void run(const std::string& tag) {
 		record_final<Scalar>(mlp, net);
 	}
 	{
+		/* value and gradient constraints of a device-resident parameter (parameters/StandardParameters.hpp:105-123):
+		 * values constrained when they are set, the gradient after the backward pass */
+		Lcg g(15);
+		const std::size_t batch = 6;
+		DL dense = DL::dense(Dims{ { 7, 1, 1 } }, 4);
+		dense.set_constraints(0, (Scalar) 0.3, (Scalar) 0.9, (Scalar) 0.5, (Scalar) 0.2, (Scalar) 0.6, (Scalar) 0.25);
+		std::vector<Scalar> w = random_values<Scalar>(7 * 4, g, 1.0);
+		dense.set_param_values(0, w.data());
+		std::vector<Scalar> x = random_values<Scalar>(batch * 7, g, 1.0), go = random_values<Scalar>(batch * 4, g, 1.0);
+		DT xd(typename DT::Dims{ { batch, 7, 1, 1 } }, x.data()), gd(typename DT::Dims{ { batch, 4, 1, 1 } }, go.data());
+		dense.pass_forward_borrowed(xd, true);
+		dense.pass_back(gd);
+		record(tag + ".cons.w", sizeof(Scalar), { 7, 4 }, w.data());
+		record(tag + ".cons.x", sizeof(Scalar), { batch, 7 }, x.data());
+		record(tag + ".cons.go", sizeof(Scalar), { batch, 4 }, go.data());
+		record(tag + ".cons.values", sizeof(Scalar), { 7, 4 }, dense.get_param_values(0).data());
+		record(tag + ".cons.grad", sizeof(Scalar), { 7, 4 }, dense.get_param_grad(0).data());
+	}
+	{
 		/* the data-movement layers of the reference's example networks: reshape -> broadcast -> dropout */
 		Lcg g(14);
 		const std::size_t batch = 5;

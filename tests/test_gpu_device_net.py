@@ -112,6 +112,20 @@ def test_reshape_broadcast_dropout_stack(records, tag, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tag,tol", [("f32", 1e-5), ("f64", 1e-12)])
+def test_parameter_constraints_through_the_front_end(records, tag, tol):
+    """DeviceLayer::set_constraints: the values as StandardParameters::set_values leaves them, the gradient as
+    accumulate_grad leaves it (clip, then the two norm limits)."""
+    r = {k[len(tag) + 6:]: v for k, v in records.items() if k.startswith(tag + ".cons.")}
+    values = oracle.constrain(r["w"], 0.3, 0.9, 0.5)
+    assert not np.array_equal(values, r["w"])                     # the limits do bite on these values
+    assert hp.rel_err(r["values"], values) < tol
+    raw = np.asarray(r["x"], np.float64).T @ np.asarray(r["go"], np.float64)      # dense weight gradient: x^T g
+    grad = oracle.constrain(np.asfortranarray(raw.astype(r["w"].dtype)), 0.2, 0.6, 0.25)
+    assert hp.rel_err(r["grad"], grad) < 10 * tol
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("tag,tol", [("f32", 1e-4), ("f64", 1e-10)])
 def test_device_loss_of_another_kind_negated(records, tag, tol):
     out, obj = np.asarray(records[tag + ".loss.out"], np.float64), np.asarray(records[tag + ".loss.obj"], np.float64)
