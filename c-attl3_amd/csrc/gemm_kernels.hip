@@ -800,7 +800,10 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	constexpr int THREADS = 64 * WAVES_K * WAVES_F;
 	constexpr int BK = WAVES_K * WT_K, BF = WAVES_F * WT_F;
 	constexpr int VR = 16 / (int) sizeof(T);
-	constexpr int LDM = MC + VR;
+	/* row stride of the staged tiles: the chunk plus 16 bytes in fp32, plus 48 bytes in fp64 (measured at config 4:
+	 * 2.08 -> 1.98 ms for the fp64 kernel, whose LDS bank conflicts were 13 % of its busy cycles with 16 bytes; fp32,
+	 * which has next to none, gets 0.5-2 % slower with more) */
+	constexpr int LDM = MC + (sizeof(T) == 8 ? 3 : 1) * VR;
 	constexpr int TL = MF::TL, KS = MF::KS;
 	constexpr int KB = WT_K / TL, FB = WT_F / TL;
 	constexpr int COLS = MC / VEC, RP = THREADS / COLS;
@@ -1852,7 +1855,8 @@ struct WgradPlan {
 	int variant, ktiles, ftiles, splits, chunks_per_split, pixel_mode;
 };
 
-/* The tile shape with the least padding wins (the earlier, larger one on ties: it re-reads G less often); the
+/* The tile shape with the least padding wins (on ties the earlier, larger one, which re-reads G less often, unless only
+ * a later one fits a CU twice); the
  * M range is then cut into as many slices as fill the chip once (blocks = tiles * splits <= slots),
  * so that no block runs in a second, mostly idle round; the slots are what the runtime's occupancy query
  * reports for the variant. The plan depends on the shape and the build only, which keeps the summation
@@ -1870,6 +1874,15 @@ WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 			p.variant = i;
 		}
 	}
+	/* Among the shapes with that padding, the first of which a CU holds two blocks: alone on its CU a block has nothing
+	 * to cover its barriers and load waits with (fp64 at config 4: the 96 x 128 tile, one block per CU at 160 registers,
+	 * 2.17 ms; the 96 x 64 tile, two blocks, 1.98 ms although it reads the input twice as often). */
+	if (vars[p.variant].blocks_per_cu() < 2)
+		for (int i = 0; i < WgradVariants<T>::BASE; ++i)
+			if ((long) round_up(K, vars[i].bk) * round_up(F, vars[i].bf) == best && vars[i].blocks_per_cu() >= 2) {
+				p.variant = i;
+				break;
+			}
 	const Tuning& tune = tuning();
 	/* A short reduction (a dense layer: M is the batch size) cannot be cut into many slices, so the tiles must fill the
 	 * chip: among the shapes with the least padding, the largest whose tiles times the possible slices reach half of
