@@ -800,10 +800,7 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	constexpr int THREADS = 64 * WAVES_K * WAVES_F;
 	constexpr int BK = WAVES_K * WT_K, BF = WAVES_F * WT_F;
 	constexpr int VR = 16 / (int) sizeof(T);
-	/* row stride of the staged tiles: the chunk plus 16 bytes in fp32, plus 48 bytes in fp64 (measured at config 4:
-	 * 2.08 -> 1.98 ms for the fp64 kernel, whose LDS bank conflicts were 13 % of its busy cycles with 16 bytes; fp32,
-	 * which has next to none, gets 0.5-2 % slower with more) */
-	constexpr int LDM = MC + (sizeof(T) == 8 ? 3 : 1) * VR;
+	constexpr int LDM = MC + VR;
 	constexpr int TL = MF::TL, KS = MF::KS;
 	constexpr int KB = WT_K / TL, FB = WT_F / TL;
 	constexpr int COLS = MC / VEC, RP = THREADS / COLS;
