@@ -75,9 +75,10 @@ __device__ __forceinline__ T lstm_act_b(const LstmActs<T>& a, T x, T y, T g) {
 
 /* Offset of element (n, rest) of time step t in a sequence tensor (N, T_len, ...): element e = n + N * rest of a
  * step's slab. A slab of P elements is a whole number of samples, so gate g of element e is (n, rest + g * P / N):
- * one 32-bit division per element serves all of its accesses (the host checks that 4 P fits 32 bits). */
-__device__ __forceinline__ size_t seq_offset(unsigned n, unsigned rest, int N, int T_len, int t) {
-	return n + (size_t) N * ((size_t) t + (size_t) T_len * rest);
+ * one 32-bit division per element serves all of its accesses. All offsets are formed in 32 bits: the host checks that
+ * four slabs, and every sequence tensor, stay below 2^31 elements. */
+__device__ __forceinline__ unsigned seq_offset(unsigned n, unsigned rest, int N, int T_len, int t) {
+	return n + (unsigned) N * ((unsigned) t + (unsigned) T_len * rest);
 }
 
 /* Column of the weight matrix [forget | write | candidate | read] (hidden columns each) that sits at column f of the
@@ -139,8 +140,8 @@ __device__ __forceinline__ void lstm_forward_store(const LstmForwardStep<T>& A, 
 	#pragma unroll
 	for (int g = 0; g < 4; ++g) {
 		if (A.z)
-			A.z[(size_t) g * P + e] = o.v[g];
-		A.gates[(size_t) g * P + e] = o.y[g];
+			A.z[(unsigned) g * P + e] = o.v[g];
+		A.gates[(unsigned) g * P + e] = o.y[g];
 	}
 	A.state[e] = o.s;
 	A.act_state[e] = o.as;
@@ -173,14 +174,14 @@ __device__ __forceinline__ void lstm_backward_element(const LstmBackwardStep<T>&
 	T hg = has_dh ? dh : (T) 0;
 	if (A.out_grad)
 		hg += A.out_grad[seq_offset(n, rest, A.N, A.og_T, A.og_t)];       /* :431-438 */
-	const T f = A.gates[e], w = A.gates[(size_t) P + e], c = A.gates[(size_t) 2 * P + e], r = A.gates[(size_t) 3 * P + e];
+	const T f = A.gates[e], w = A.gates[P + e], c = A.gates[2u * P + e], r = A.gates[3u * P + e];
 	const T as = A.act_state[e];
 	const T sg = (has_dh ? A.state_grad[e] : (T) 0) + lstm_act_b<T, STD, 3>(A.a, A.state[e], as, r * hg);      /* :440 */
 	T zin[4] = { (T) 0, (T) 0, (T) 0, (T) 0 };
 	if (A.z) {
 		#pragma unroll
 		for (int g = 0; g < 4; ++g)
-			zin[g] = A.z[(size_t) g * P + e];
+			zin[g] = A.z[(unsigned) g * P + e];
 	}
 	T d[4];
 	d[3] = lstm_act_b<T, STD, 4>(A.a, zin[3], r, as * hg);                       /* :441 */
@@ -194,7 +195,7 @@ __device__ __forceinline__ void lstm_backward_element(const LstmBackwardStep<T>&
 	for (int g = 0; g < 4; ++g) {
 		to_input[g] = to_output[g] = d[g];
 		if (A.zx_fwd) {
-			to_input[g] = A.zh_fwd[(size_t) g * P + e] * d[g];
+			to_input[g] = A.zh_fwd[(unsigned) g * P + e] * d[g];
 			to_output[g] = A.zx_fwd[seq_offset(n, rest + g * slab_rows, A.N, A.x_T, A.x_t)] * d[g];
 		}
 	}
