@@ -102,14 +102,26 @@ void static_scratch_setup();
 size_t static_scratch_bytes();
 template<typename T> void conv_forward_static(const ConvShape& s, int N, const T* x, const T* w, const T* b, T* out);
 
-/* Backward: wgrad[K x F] += A^T G, bgrad[F] += colsum(G), in_grad = dgrad (skipped if null). */
+/* An element-wise activation behind the kernel layer, undone while the weight gradient loads its G operand: out_grad is
+ * then the gradient of the activation's output y (the coded output of a fused forward pass, act_math.hpp), the operand
+ * is dz = act'(y) * out_grad, formed in registers on the way into LDS. dz, if not null, also receives it (written once,
+ * by the blocks of the first k tile), for the input-gradient launch that follows. The rectifier family only (ReLU, LeakyReLU and ELU
+ * with non-negative arguments), whose derivative is a function of the coded output's sign bit. */
+template<typename T> struct WgradAct {
+	const T* y;
+	T* dz;
+	int kind;
+	T p;
+};
+/* Backward: wgrad[K x F] += A^T G, bgrad[F] += colsum(G), in_grad = dgrad (skipped if null). With `act`, G is
+ * act'(y) * out_grad (see WgradAct; act->dz must be given when in_grad is). */
 template<typename T> void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad,
-		T* wgrad, T* bgrad, T* in_grad, T* wt_dgrad, bool wt_ready, T* partials);
+		T* wgrad, T* bgrad, T* in_grad, T* wt_dgrad, bool wt_ready, T* partials, const WgradAct<T>* act = nullptr);
 
 /* The two halves of conv_backward on their own (the transposed convolution uses them with the roles
  * of input and output exchanged). bgrad may be null. */
 template<typename T> void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad,
-		T* partials);
+		T* partials, const WgradAct<T>* act = nullptr);
 template<typename T> struct LstmBackwardStep;
 /* og_batch > 0: out_grad holds the first N of og_batch samples per position (GatherGeom::NS). `then`, if given, is the LSTM backward step that consumes in_grad as the gradient of its hidden output: when the
  * launch cuts every tile's reduction into parts, the kernel that sums the parts runs the element-wise part of that

@@ -792,10 +792,13 @@ struct WgradSplit {
  * grid = tiles * splits blocks (1-D). Bias rows are dealt out over the k tiles (row f belongs to the
  * block with f % ktiles == k-tile index) so that every block does the same amount of extra work.
  * ---------------------------------------------------------------------------------------------- */
-template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, int MIN_WAVES>
+template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, int MIN_WAVES, bool ACTG = false>
 __global__ __launch_bounds__(64 * WAVES_K * WAVES_F, MIN_WAVES)      /* MIN_WAVES: wavefronts per SIMD the registers must allow */
 void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
-		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan) {
+		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan, const T* __restrict__ act_y,
+		T* __restrict__ act_dz, T act_p0, T act_p1) {
+	/* (the activation's tensors as parameters of their own: pointers inside a structure are not known to point to global
+	 * memory, and flat loads count against the LDS counter as well, see vec_load_global) */
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_K * WAVES_F;
 	constexpr int BK = WAVES_K * WT_K, BF = WAVES_F * WT_F;
@@ -874,6 +877,11 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	const int eN = MC % g.N, eA = (MC / g.N) % g.OA, eB = (MC / g.N) / g.OA;
 
 	T xreg[XSLOTS][VEC], greg[GSLOTS][VEC];
+	/* ACTG: the activation outputs beside the gradient values, and where both came from; the derivative is applied
+	 * when the chunk is stored to LDS, a chunk after its loads were issued, so that nothing waits for them here */
+	T yreg[ACTG ? GSLOTS : 1][VEC];
+	int gm_loaded = 0;
+	bool gvalid_loaded = false;
 
 	auto load_tiles = [&]() {
 		const int m = n + g.N * (a + g.OA * b);
@@ -899,12 +907,19 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 			const int f = f0 + row;
 			if (mvalid && f < g.F && (BF % RP == 0 || row < BF)) {
 				vec_load<T, VEC>(greg[s], og + ((size_t) m + (size_t) g.M * f));
+				if constexpr (ACTG)
+					vec_load<T, VEC>(yreg[s], act_y + ((size_t) m + (size_t) g.M * f));
 			} else {
 				#pragma unroll
-				for (int v = 0; v < VEC; ++v)
+				for (int v = 0; v < VEC; ++v) {
 					greg[s][v] = (T) 0;
+					if constexpr (ACTG)
+						yreg[s][v] = (T) 0;
+				}
 			}
 		}
+		gm_loaded = m;
+		gvalid_loaded = mvalid;
 		if (pixel_mode) {
 			/* next position of the slice; after the last one, back to the first with the next samples */
 			a += 1;
@@ -933,10 +948,33 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 		for (int s = 0; s < XSLOTS; ++s)
 			if (BK % RP == 0 || row0 + s * RP < BK)
 				vec_store<T, VEC>(&Xs[row0 + s * RP][col * VEC], xreg[s]);
-		#pragma unroll
-		for (int s = 0; s < GSLOTS; ++s)
-			if (BF % RP == 0 || row0 + s * RP < BF)
-				vec_store<T, VEC>(&Gs[row0 + s * RP][col * VEC], greg[s]);
+		if constexpr (ACTG) {
+			/* The rectifier family, without a branch on the kind (a switch here, even outside the loops, turned the
+			 * register arrays into scratch memory): the derivative is 1 on the non-negative side and act_p0 + act_p1 * y
+			 * on the negative side, which the coded output's sign bit names - 0 for ReLU, alpha for LeakyReLU,
+			 * y + alpha for ELU, the expressions of act_b_coded. Rows outside the tile or the matrix were loaded as zeros. */
+			#pragma unroll
+			for (int s = 0; s < GSLOTS; ++s) {
+				if (BF % RP == 0 || row0 + s * RP < BF) {
+					const bool live = gvalid_loaded && f0 + row0 + s * RP < g.F;
+					T dzv[VEC];
+					#pragma unroll
+					for (int v = 0; v < VEC; ++v) {
+						const T slope = sign_bit(yreg[s][v]) ? act_p1 * yreg[s][v] + act_p0 : (T) 1;
+						dzv[v] = live ? slope * greg[s][v] : (T) 0;
+					}
+					vec_store<T, VEC>(&Gs[row0 + s * RP][col * VEC], dzv);
+					/* each element of G belongs to one (slice, f tile): the blocks of the first k tile write it */
+					if (act_dz != nullptr && kt == 0 && live)
+						vec_store<T, VEC>(act_dz + ((size_t) gm_loaded + (size_t) g.M * (f0 + row0 + s * RP)), dzv);
+				}
+			}
+		} else {
+			#pragma unroll
+			for (int s = 0; s < GSLOTS; ++s)
+				if (BF % RP == 0 || row0 + s * RP < BF)
+					vec_store<T, VEC>(&Gs[row0 + s * RP][col * VEC], greg[s]);
+		}
 	};
 
 	const int lane = tid % 64, wave = tid / 64;
@@ -1769,21 +1807,35 @@ template<typename T>
 struct WgradVariant {
 	int bk, bf, waves;
 	int mc;                         /* rows of M per reduction chunk; above 32 only with 16-byte loads */
-	void (*launch)(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom&, const WgradSplit&, bool vec);
+	void (*launch)(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom&, const WgradSplit&, bool vec,
+			const WgradAct<T>* act);
 	int (*blocks_per_cu)();         /* what the runtime says fits on a CU (registers and LDS) */
 };
 
 template<typename T, int WK, int WF, int TK, int TF, int MINW = 1, int MC = WGRAD_MC>
 void launch_wgrad_variant(const T* x, const T* og, T* partials, T* bias_partials, const GatherGeom& g, const WgradSplit& plan,
-		bool vec) {
+		bool vec, const WgradAct<T>* act) {
 	constexpr int VEC = GemmCfg<T>::VEC;
 	dim3 block(64 * WK * WF), grid((unsigned) round_up(plan.tiles * plan.splits, 8));
+	/* derivative on the negative side: p0 + p1 * y */
+	T p0 = (T) 0, p1 = (T) 0;
+	if (act) {
+		CATTLE_HIP_REQUIRE(act_sign_coded(act->kind) && act->p >= (T) 0, "only a rectifier can be undone while the gradient is loaded");
+		p0 = act->kind == ACT_RELU ? (T) 0 : act->p;
+		p1 = act->kind == ACT_ELU ? (T) 1 : (T) 0;
+	}
 	if (vec) {
-		wgrad_kernel<T, WK, WF, TK, TF, MC, VEC, MINW><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
-	} else {
-		if constexpr (MC == WGRAD_MC)
-			wgrad_kernel<T, WK, WF, TK, TF, MC, 1, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan);
+		if (act)        /* the extra operand registers do not fit a register cap: MIN_WAVES 1 */
+			wgrad_kernel<T, WK, WF, TK, TF, MC, VEC, 1, true><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan, act->y, act->dz, p0, p1);
 		else
+			wgrad_kernel<T, WK, WF, TK, TF, MC, VEC, MINW><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan, (const T*) nullptr, (T*) nullptr, (T) 0, (T) 0);
+	} else {
+		if constexpr (MC == WGRAD_MC) {
+			if (act)
+				wgrad_kernel<T, WK, WF, TK, TF, MC, 1, 1, true><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan, act->y, act->dz, p0, p1);
+			else
+				wgrad_kernel<T, WK, WF, TK, TF, MC, 1, 1><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan, (const T*) nullptr, (T*) nullptr, (T) 0, (T) 0);
+		} else
 			CATTLE_HIP_REQUIRE(false, "a weight-gradient variant with long chunks was planned for scalar loads");
 	}
 	CATTLE_HIP_CHECK(hipGetLastError());
@@ -2055,12 +2107,14 @@ void conv_forward_static(const ConvShape& s, int N, const T* x, const T* w, cons
 }
 
 template<typename T>
-void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials) {
+void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials,
+		const WgradAct<T>* act) {
 	check_sizes(s, N);
 	const GatherGeom g = forward_geom(s, N);
 	/* split-M partials, then a fixed-order reduction that accumulates */
 	const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
+			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0 &&
+			(!act || ((reinterpret_cast<uintptr_t>(act->y) & 15) == 0 && (reinterpret_cast<uintptr_t>(act->dz) & 15) == 0));
 	const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N, vec);
 	const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
 	const size_t count = (size_t) g.K * g.F;
@@ -2068,11 +2122,11 @@ void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_gr
 	if (p.splits == 1) {
 		/* one slice: every block owns its tile of the gradient and adds to it directly, no second launch */
 		const WgradSplit direct = { p.ktiles, p.ktiles * p.ftiles, 1, p.chunks_per_split, p.pixel_mode, 1 };
-		v.launch(x, out_grad, wgrad, bgrad, g, direct, vec);
+		v.launch(x, out_grad, wgrad, bgrad, g, direct, vec, act);
 		return;
 	}
 	const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode, 0 };
-	v.launch(x, out_grad, partials, bias_partials, g, split, vec);
+	v.launch(x, out_grad, partials, bias_partials, g, split, vec, act);
 	const int wblocks = (int) ((count + 63) / 64), bblocks = bgrad ? (g.F + 63) / 64 : 0;
 	constexpr int V = 16 / (int) sizeof(T);
 	const size_t outputs = count + (bgrad ? (size_t) g.F : 0);
@@ -2112,10 +2166,11 @@ bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_gra
 
 template<typename T>
 void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad,
-		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials) {
-	conv_weight_gradient<T>(s, N, x, out_grad, wgrad, bgrad, partials);
+		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials, const WgradAct<T>* act) {
+	CATTLE_HIP_REQUIRE(!act || !in_grad || act->dz != nullptr, "the input gradient needs the gradient before the activation");
+	conv_weight_gradient<T>(s, N, x, out_grad, wgrad, bgrad, partials, act);
 	if (in_grad)
-		conv_input_gradient<T>(s, N, w, out_grad, in_grad, wt_dgrad, wt_ready, nullptr, 0);
+		conv_input_gradient<T>(s, N, w, act ? (const T*) act->dz : out_grad, in_grad, wt_dgrad, wt_ready, nullptr, 0);
 }
 
 template ConvWorkspace conv_workspace<float>(const ConvShape&, int);
@@ -2133,11 +2188,13 @@ template bool conv_forward_lstm<double>(const ConvShape&, int, const double*, in
 template void conv_forward_static<float>(const ConvShape&, int, const float*, const float*, const float*, float*);
 template void conv_forward_static<double>(const ConvShape&, int, const double*, const double*, const double*, double*);
 template void conv_backward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, float*,
-		float*, bool, float*);
+		float*, bool, float*, const WgradAct<float>*);
 template void conv_backward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*,
-		double*, double*, bool, double*);
-template void conv_weight_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, float*);
-template void conv_weight_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, double*);
+		double*, double*, bool, double*, const WgradAct<double>*);
+template void conv_weight_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, float*,
+		const WgradAct<float>*);
+template void conv_weight_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, double*,
+		const WgradAct<double>*);
 template bool conv_input_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, bool,
 		const LstmBackwardStep<float>*, int);
 template bool conv_input_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, bool,

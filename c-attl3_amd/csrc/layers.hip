@@ -357,6 +357,11 @@ struct ConvLayer : LayerBase {
 		x_cache = (const T*) in;       /* the reference caches the patch matrix (ConvKernelLayer.hpp:127); the input suffices */
 	}
 	void backward(const void* out_grad, size_t N, void* in_grad) override {
+		backward_through(out_grad, N, in_grad, nullptr);
+	}
+	/* `act`: out_grad is the gradient behind an element-wise activation whose derivative the weight-gradient launch
+	 * applies on its way (WgradAct) */
+	void backward_through(const void* out_grad, size_t N, void* in_grad, const WgradAct<T>* act) {
 		CATTLE_HIP_REQUIRE(x_cache != nullptr, "pass_back without a cached forward input");
 		const int n = checked_int(N, "batch size");
 		const ConvWorkspace ws = conv_workspace<T>(shape, n);
@@ -365,7 +370,7 @@ struct ConvLayer : LayerBase {
 		const bool ready = w.derived_version[1] == w.version;
 		T* part = (T*) partials.ensure(ws.partials * sizeof(T));
 		conv_backward<T>(shape, n, x_cache, (const T*) w.values.p, (const T*) out_grad, (T*) w.grad.p, (T*) params[1]->grad.p,
-				(T*) in_grad, wt, ready, part);
+				(T*) in_grad, wt, ready, part, act);
 		if (in_grad)
 			w.derived_version[1] = w.version;
 	}
@@ -1105,6 +1110,14 @@ struct FusedLayer : LayerBase {
 				T* gp = (T*) grad_a.ensure(zcount * sizeof(T));
 				pool->backward(g, N, gp);
 				g = gp;
+			}
+			if (act && act_sign_coded(act->kind) && act->p >= 0) {
+				/* a rectifier, whose derivative the sign bit of the coded output names: applied by the weight-gradient
+				 * launch while it loads the gradient, which also leaves dz behind for the input-gradient launch - no
+				 * pass of its own */
+				const WgradAct<T> through = { y_cache, in_grad ? dz : nullptr, act->kind, (T) act->p };
+				conv->backward_through(g, N, in_grad, &through);
+				return;
 			}
 			chain_backward<T>(chain_shape(false), n, g, nullptr, y_cache, needs_pre() ? (const T*) pre_buf.p : nullptr, dz);
 		}
