@@ -280,8 +280,8 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			const int idx = tid + it * THREADS, row = idx % BM, cl = idx / BM;
 			const int mrow = tile_row_m(L, g, tile, BM, row);
 			lstm_e[it] = mrow < g.M ? (unsigned) mrow + (unsigned) g.M * (unsigned) (blockIdx.y * CB + cl) : 0xffffffffu;
-			if (lstm_e[it] != 0xffffffffu)
-				lstm_in[it] = lstm_forward_load<T>(E.lstm, lstm_e[it]);
+			/* (every element of the array assigned: a partly initialised register array ends up in scratch memory) */
+			lstm_in[it] = lstm_forward_load<T>(E.lstm, lstm_e[it] != 0xffffffffu ? lstm_e[it] : 0u);
 		}
 	}
 

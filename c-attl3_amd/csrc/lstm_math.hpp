@@ -49,6 +49,18 @@ __device__ __forceinline__ T act_b_rt(int kind, T x, T y, T g, T p) {
 	}
 }
 
+/* Accesses through the pointers of the step structures, told to be global memory: a pointer that sits in a structure is
+ * not known to be one, the compiler then emits flat accesses, and those count against the LDS counter as well as the
+ * memory counter - inside a GEMM kernel every wait for an LDS read would wait for them too. */
+template<typename T>
+__device__ __forceinline__ T lstm_ld(const T* p, unsigned i) {
+	return ((const __attribute__((address_space(1))) T*) p)[i];
+}
+template<typename T>
+__device__ __forceinline__ void lstm_st(T* p, unsigned i, T v) {
+	((__attribute__((address_space(1))) T*) p)[i] = v;
+}
+
 /* The usual cell: sigmoid gates, tanh on the candidates and on the state. Kernels test for it once and run the
  * arithmetic with the kinds known at compile time (STD): straight-line code whose independent elements the compiler can
  * interleave, where the run-time switch is a chain of branches per activation. */
@@ -98,8 +110,8 @@ __device__ __forceinline__ LstmForwardInputs<T> lstm_forward_load(const LstmForw
 	LstmForwardInputs<T> in;
 	#pragma unroll
 	for (int g = 0; g < 4; ++g)
-		in.zx[g] = A.zx ? A.zx[seq_offset(n, rest + g * slab_rows, A.N, A.zx_T, A.zx_t)] : (T) 0;
-	in.prev = A.prev_state ? A.prev_state[e] : (T) 0;
+		in.zx[g] = A.zx ? lstm_ld<T>(A.zx, seq_offset(n, rest + g * slab_rows, A.N, A.zx_T, A.zx_t)) : (T) 0;
+	in.prev = A.prev_state ? lstm_ld<T>(A.prev_state, e) : (T) 0;
 	return in;
 }
 
@@ -140,19 +152,19 @@ __device__ __forceinline__ void lstm_forward_store(const LstmForwardStep<T>& A, 
 	#pragma unroll
 	for (int g = 0; g < 4; ++g) {
 		if (A.z)
-			A.z[(unsigned) g * P + e] = o.v[g];
-		A.gates[(unsigned) g * P + e] = o.y[g];
+			lstm_st<T>(A.z, (unsigned) g * P + e, o.v[g]);
+		lstm_st<T>(A.gates, (unsigned) g * P + e, o.y[g]);
 	}
-	A.state[e] = o.s;
-	A.act_state[e] = o.as;
+	lstm_st<T>(A.state, e, o.s);
+	lstm_st<T>(A.act_state, e, o.as);
 	if (A.hprev_all) {
 		if (A.h_t < A.h_T)
-			A.hprev_all[seq_offset(n, rest, A.N, A.h_T, A.h_t)] = o.h;
+			lstm_st<T>(A.hprev_all, seq_offset(n, rest, A.N, A.h_T, A.h_t), o.h);
 		if (!A.prev_state)                                      /* first step: no previous output, slab 0 is zero */
-			A.hprev_all[seq_offset(n, rest, A.N, A.h_T, 0)] = (T) 0;
+			lstm_st<T>(A.hprev_all, seq_offset(n, rest, A.N, A.h_T, 0), (T) 0);
 	}
 	if (A.out)
-		A.out[seq_offset(n, rest, A.N, A.out_T, A.out_t)] = o.h;
+		lstm_st<T>(A.out, seq_offset(n, rest, A.N, A.out_T, A.out_t), o.h);
 }
 
 /* Every load of the element comes before its first store: the tensors are not declared free of aliases, and a store
@@ -173,21 +185,21 @@ __device__ __forceinline__ void lstm_backward_element(const LstmBackwardStep<T>&
 	const unsigned rest = e / N, n = e - rest * N;
 	T hg = has_dh ? dh : (T) 0;
 	if (A.out_grad)
-		hg += A.out_grad[seq_offset(n, rest, A.N, A.og_T, A.og_t)];       /* :431-438 */
-	const T f = A.gates[e], w = A.gates[P + e], c = A.gates[2u * P + e], r = A.gates[3u * P + e];
-	const T as = A.act_state[e];
-	const T sg = (has_dh ? A.state_grad[e] : (T) 0) + lstm_act_b<T, STD, 3>(A.a, A.state[e], as, r * hg);      /* :440 */
+		hg += lstm_ld<T>(A.out_grad, seq_offset(n, rest, A.N, A.og_T, A.og_t));       /* :431-438 */
+	const T f = lstm_ld<T>(A.gates, e), w = lstm_ld<T>(A.gates, P + e), c = lstm_ld<T>(A.gates, 2u * P + e), r = lstm_ld<T>(A.gates, 3u * P + e);
+	const T as = lstm_ld<T>(A.act_state, e);
+	const T sg = (has_dh ? lstm_ld<T>(A.state_grad, e) : (T) 0) + lstm_act_b<T, STD, 3>(A.a, lstm_ld<T>(A.state, e), as, r * hg);      /* :440 */
 	T zin[4] = { (T) 0, (T) 0, (T) 0, (T) 0 };
 	if (A.z) {
 		#pragma unroll
 		for (int g = 0; g < 4; ++g)
-			zin[g] = A.z[(unsigned) g * P + e];
+			zin[g] = lstm_ld<T>(A.z, (unsigned) g * P + e);
 	}
 	T d[4];
 	d[3] = lstm_act_b<T, STD, 4>(A.a, zin[3], r, as * hg);                       /* :441 */
 	d[2] = lstm_act_b<T, STD, 2>(A.a, zin[2], c, w * sg);                        /* :442 */
 	d[1] = lstm_act_b<T, STD, 1>(A.a, zin[1], w, c * sg);                            /* :443 */
-	d[0] = lstm_act_b<T, STD, 0>(A.a, zin[0], f, (A.prev_state ? A.prev_state[e] : (T) 0) * sg);  /* :444 */
+	d[0] = lstm_act_b<T, STD, 0>(A.a, zin[0], f, (A.prev_state ? lstm_ld<T>(A.prev_state, e) : (T) 0) * sg);  /* :444 */
 	/* multiplicative integration at a step with both an input and a previous output (zx_fwd and zh_fwd are that
 	 * step's weighted input and weighted output): each side's gradient carries the other side (:449-466) */
 	T to_input[4], to_output[4];
@@ -195,18 +207,18 @@ __device__ __forceinline__ void lstm_backward_element(const LstmBackwardStep<T>&
 	for (int g = 0; g < 4; ++g) {
 		to_input[g] = to_output[g] = d[g];
 		if (A.zx_fwd) {
-			to_input[g] = A.zh_fwd[(unsigned) g * P + e] * d[g];
-			to_output[g] = A.zx_fwd[seq_offset(n, rest + g * slab_rows, A.N, A.x_T, A.x_t)] * d[g];
+			to_input[g] = lstm_ld<T>(A.zh_fwd, (unsigned) g * P + e) * d[g];
+			to_output[g] = lstm_ld<T>(A.zx_fwd, seq_offset(n, rest + g * slab_rows, A.N, A.x_T, A.x_t)) * d[g];
 		}
 	}
-	A.state_grad[e] = sg * f;                                                                                  /* :445 */
+	lstm_st<T>(A.state_grad, e, sg * f);                                                                                  /* :445 */
 	#pragma unroll
 	for (int g = 0; g < 4; ++g) {
 		if (A.dzx_all)
-			A.dzx_all[seq_offset(n, rest + g * slab_rows, A.N, A.x_T, A.x_t)] = to_input[g];
+			lstm_st<T>(A.dzx_all, seq_offset(n, rest + g * slab_rows, A.N, A.x_T, A.x_t), to_input[g]);
 		/* what the output-side kernels' pass_back receives; step 0 has no previous output to pair with: its slab is zero */
 		if (A.dzh_all)
-			A.dzh_all[seq_offset(n, rest + g * slab_rows, A.N, A.h_T, A.h_t)] = A.prev_state ? to_output[g] : (T) 0;
+			lstm_st<T>(A.dzh_all, seq_offset(n, rest + g * slab_rows, A.N, A.h_T, A.h_t), A.prev_state ? to_output[g] : (T) 0);
 	}
 }
 
