@@ -531,11 +531,11 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		if (lstm_standard_acts(E.lstm.a)) {
 			#pragma unroll
 			for (int it = 0; it < LSTM_ELEMS; ++it)
-				res[it] = lstm_forward_compute<T, true>(E.lstm, lstm_in[it], zh4[it]);
+				res[it] = lstm_forward_compute<T, true>(E.lstm, lstm_in[it], true, zh4[it]);
 		} else {
 			#pragma unroll
 			for (int it = 0; it < LSTM_ELEMS; ++it)
-				res[it] = lstm_forward_compute<T, false>(E.lstm, lstm_in[it], zh4[it]);
+				res[it] = lstm_forward_compute<T, false>(E.lstm, lstm_in[it], true, zh4[it]);
 		}
 		#pragma unroll
 		for (int it = 0; it < LSTM_ELEMS; ++it)

@@ -120,17 +120,18 @@ __device__ __forceinline__ LstmForwardInputs<T> lstm_forward_load(const LstmForw
 template<typename T> struct LstmForwardOutputs { T v[4], y[4], s, as, h; };
 
 /* The arithmetic of the forward step, registers only. zh4: the weighted previous output of the element's four gates
- * (bias included), or null at the first step. */
+ * (bias included) if has_zh; there is none at the first step. (An array and a flag, not a pointer that may be null: the
+ * array behind such a pointer cannot stay in registers.) */
 template<typename T, bool STD = false>
 __device__ __forceinline__ LstmForwardOutputs<T> lstm_forward_compute(const LstmForwardStep<T>& A, const LstmForwardInputs<T>& in,
-		const T* zh4) {
+		bool has_zh, const T (&zh4)[4]) {
 	LstmForwardOutputs<T> o;
 	#pragma unroll
 	for (int g = 0; g < 4; ++g) {
 		/* weighted input + weighted previous output (:312, :327, :342, :373), their product with multiplicative
 		 * integration (:303-311); a step with only one of the two takes it as it is */
 		T v = in.zx[g];
-		if (zh4)
+		if (has_zh)
 			v = A.zx ? (A.mul_int ? v * zh4[g] : v + zh4[g]) : zh4[g];
 		o.v[g] = v;
 	}
@@ -170,9 +171,9 @@ __device__ __forceinline__ void lstm_forward_store(const LstmForwardStep<T>& A, 
 /* Every load of the element comes before its first store: the tensors are not declared free of aliases, and a store
  * between two loads would make the second wait for the first. */
 template<typename T, bool STD = false>
-__device__ __forceinline__ void lstm_forward_element(const LstmForwardStep<T>& A, unsigned e, const T* zh4) {
+__device__ __forceinline__ void lstm_forward_element(const LstmForwardStep<T>& A, unsigned e, bool has_zh, const T (&zh4)[4]) {
 	const LstmForwardInputs<T> in = lstm_forward_load<T>(A, e);
-	lstm_forward_store<T>(A, e, lstm_forward_compute<T, STD>(A, in, zh4));
+	lstm_forward_store<T>(A, e, lstm_forward_compute<T, STD>(A, in, has_zh, zh4));
 }
 
 /* Backward step of element e. dh: the gradient of the element's hidden output that came back through the next

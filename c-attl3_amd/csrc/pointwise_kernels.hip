@@ -761,16 +761,14 @@ __global__ __launch_bounds__(256)
 void lstm_gates_forward_kernel(const LstmForwardStep<T> A, const T* __restrict__ zh) {
 	const size_t stride = (size_t) gridDim.x * blockDim.x;
 	for (size_t e = (size_t) blockIdx.x * blockDim.x + threadIdx.x; e < A.P; e += stride) {
-		T zh4[4];
-		if (zh) {
-			#pragma unroll
-			for (int g = 0; g < 4; ++g)
-				zh4[g] = zh[g * A.P + e];
-		}
+		T zh4[4];       /* (assigned on every path: a partly initialised register array ends up in scratch memory) */
+		#pragma unroll
+		for (int g = 0; g < 4; ++g)
+			zh4[g] = zh ? zh[g * A.P + e] : (T) 0;
 		if (lstm_standard_acts(A.a))
-			lstm_forward_element<T, true>(A, (unsigned) e, zh ? zh4 : nullptr);
+			lstm_forward_element<T, true>(A, (unsigned) e, zh != nullptr, zh4);
 		else
-			lstm_forward_element<T, false>(A, (unsigned) e, zh ? zh4 : nullptr);
+			lstm_forward_element<T, false>(A, (unsigned) e, zh != nullptr, zh4);
 	}
 }
 
