@@ -160,8 +160,30 @@ def conv_forward_noalloc(x, weights, bias, out, receptor_height=3, receptor_widt
                          vertical_stride=1, horizontal_stride=1, vertical_dilation=0, horizontal_dilation=0):
     """ConvKernelLayer::pass_forward on DeviceTensors the caller owns, through the entry point that allocates nothing:
     x (N, H, W, C), weights (RH*RW*C, F), bias (1, F) or None, out (N, OH, OW, F)."""
+    if len(x.shape) != 4 or len(weights.shape) != 2 or len(out.shape) != 4:
+        raise ValueError("x and out must be (N, H, W, C) tensors, weights a matrix")
     N, H, W, C = x.shape
     F = weights.shape[1]
+    # the entry point takes raw addresses and cannot know the buffers' sizes: every extent is checked here
+    drh = receptor_height + (receptor_height - 1) * vertical_dilation
+    drw = receptor_width + (receptor_width - 1) * horizontal_dilation
+    if min(receptor_height, receptor_width, vertical_stride, horizontal_stride) < 1 or min(
+            vertical_padding, horizontal_padding, vertical_dilation, horizontal_dilation) < 0:
+        raise ValueError("receptor and strides must be positive, paddings and dilations non-negative")
+    if H + 2 * vertical_padding < drh or W + 2 * horizontal_padding < drw:
+        raise ValueError("dilated receptor larger than the padded input")
+    OH = (H + 2 * vertical_padding - drh) // vertical_stride + 1          # ConvKernelLayer.hpp:194-197
+    OW = (W + 2 * horizontal_padding - drw) // horizontal_stride + 1
+    if weights.shape[0] != receptor_height * receptor_width * C:
+        raise ValueError("weights must have receptor_height * receptor_width * channels = %d rows, not %d"
+                         % (receptor_height * receptor_width * C, weights.shape[0]))
+    if bias is not None and tuple(bias.shape) != (1, F):
+        raise ValueError("bias must be a (1, %d) matrix, not %s" % (F, tuple(bias.shape)))
+    if tuple(out.shape) != (N, OH, OW, F):
+        raise ValueError("out must be %s, not %s" % ((N, OH, OW, F), tuple(out.shape)))
+    for name, t in (("weights", weights), ("bias", bias), ("out", out)):
+        if t is not None and np.dtype(t.dtype) != np.dtype(x.dtype):
+            raise ValueError("%s is %s, x is %s" % (name, np.dtype(t.dtype), np.dtype(x.dtype)))
     _check(lib().cattle_hip_conv_forward_noalloc(
         _dtype_code(x.dtype), _sz(N), _sz(H), _sz(W), _sz(C), _sz(F), _sz(receptor_height), _sz(receptor_width),
         _sz(vertical_padding), _sz(horizontal_padding), _sz(vertical_stride), _sz(horizontal_stride), _sz(vertical_dilation),
@@ -826,6 +848,10 @@ class Graph(object):
         if exc_type is None:
             _check(rc)
             self._h = h
+        elif rc == 0:
+            # the body failed: the graph is of no use, and dropping its handle would keep the graph and every pool
+            # block of the recording out of circulation for good
+            lib().cattle_hip_graph_destroy(h)
         return False
 
     def launch(self):

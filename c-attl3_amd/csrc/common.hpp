@@ -42,6 +42,13 @@ hipStream_t stream();
 bool capturing();
 void forbid_while_capturing(const char* what);
 
+/* Allocations and recorded graphs share a clock: a device allocation made at alloc_clock_tick() is pinned while a graph
+ * recorded later is alive (it may hold the address), and then must not be freed: its owner refuses to grow or release
+ * it, or hands it to park_allocation, which frees it when the last such graph is destroyed. */
+uint64_t alloc_clock_tick();
+bool pinned_by_graph(uint64_t born);
+void park_allocation(void* p, uint64_t born);
+
 /* Copies between pageable host memory and the device on that stream; both return when the host buffer may be
  * reused (host_to_device) or holds the data (device_to_host). Large copies are staged through pinned buffers by
  * several host threads (CATTLE_HIP_COPY_THREADS, default 4; 0 leaves the staging to the runtime). */

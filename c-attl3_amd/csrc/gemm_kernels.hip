@@ -1235,8 +1235,13 @@ const DeviceShape& device_shape() {
 void* split_workspace(size_t bytes) {
 	static void* ptr = nullptr;
 	static size_t cap = 0;
+	static uint64_t born = 0;
 	if (bytes > cap) {
 		forbid_while_capturing("growing the scratch buffer of the split reductions (run the step once before recording it)");
+		/* every layer shares this buffer: a living graph recorded since it was allocated may point into it */
+		if (ptr && pinned_by_graph(born))
+			throw Error(ERR_STATE, "a recorded graph may point into the scratch buffer of the split reductions, which this call "
+					"has to grow: destroy the graph (cattle_hip_graph_destroy) first, or run this problem once before recording");
 		if (ptr)
 			(void) hipFree(ptr);
 		ptr = nullptr;
@@ -1244,6 +1249,7 @@ void* split_workspace(size_t bytes) {
 		const size_t want = (bytes + 4095) / 4096 * 4096;
 		CATTLE_HIP_CHECK(hipMalloc(&ptr, want));
 		cap = want;
+		born = alloc_clock_tick();
 	}
 	return ptr;
 }
@@ -1508,18 +1514,20 @@ template<> struct GatherVariants<double> {
 	}
 };
 
-/* Switches for experiments, read from the environment once, when the first GEMM is launched:
+/* Switches for experiments. A build with -DCATTLE_HIP_EXPERIMENTS reads them from the environment once, when the first
+ * GEMM is launched; the library as shipped has none of them and always takes the launch plan its rules give:
  *   CATTLE_HIP_GATHER_VARIANT_F<F> = index into the gather variant table for GEMMs with F output columns,
  *   CATTLE_HIP_GATHER_OCC_F<F>     = blocks per CU for them (enforced by reserving dynamic LDS),
  *   CATTLE_HIP_NO_SWIZZLE, CATTLE_HIP_NO_ROW_BLOCKS, CATTLE_HIP_NO_SPLIT: tile walk, blocked tile rows, cut reductions off,
- *   CATTLE_HIP_WGRAD_VARIANT, CATTLE_HIP_WGRAD_SPLITS, CATTLE_HIP_WGRAD_LINEAR: the weight-gradient plan. */
+ *   CATTLE_HIP_WGRAD_VARIANT, CATTLE_HIP_WGRAD_SPLITS, CATTLE_HIP_WGRAD_LINEAR, CATTLE_HIP_WGRAD_MIN_CHUNKS: the weight-gradient plan. */
 struct Tuning {
 	struct PerF { int F, variant, occ; };
 	std::vector<PerF> per_f;
-	bool no_swizzle, no_row_blocks, no_split, wgrad_linear;
-	int wgrad_variant, wgrad_splits, wgrad_min_chunks;
+	bool no_swizzle = false, no_row_blocks = false, no_split = false, wgrad_linear = false;
+	int wgrad_variant = -1, wgrad_splits = 0, wgrad_min_chunks = 0;
 
 	Tuning() {
+#ifdef CATTLE_HIP_EXPERIMENTS
 		no_swizzle = std::getenv("CATTLE_HIP_NO_SWIZZLE") != nullptr;
 		no_row_blocks = std::getenv("CATTLE_HIP_NO_ROW_BLOCKS") != nullptr;
 		no_split = std::getenv("CATTLE_HIP_NO_SPLIT") != nullptr;
@@ -1543,6 +1551,7 @@ struct Tuning {
 				(k == 0 ? slot.variant : slot.occ) = std::atoi(eq + 1);
 			}
 		}
+#endif
 	}
 	PerF& entry(int F) {
 		for (PerF& p : per_f)
@@ -2055,18 +2064,19 @@ bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const
 	if (epi == EPI_POOL) {
 		CATTLE_HIP_REQUIRE(E.prh > 0 && E.prw > 0 && g.OA % E.prh == 0 && g.OB % E.prw == 0 && E.OHp == g.OA / E.prh &&
 				E.OWp == g.OB / E.prw && E.inds != nullptr, "the pooling epilogue needs windows that tile the output");
-		/* the staging pass deals threads over windows of at most a tile's positions */
-		if (E.prh * E.prw > 64)
-			return false;
 	}
 	if (epi == EPI_STATS)
 		CATTLE_HIP_REQUIRE(E.stats != nullptr, "the moments epilogue needs a buffer for its partials");
+	/* the prepared weights come first: they are valid afterwards whatever the answer is */
 	if (!wt_ready) {
 		const int Kp = round_up(g.K, WT_ROW_PAD);
 		const size_t count = (size_t) Kp * g.ldw;
 		prep_fwd_weights_kernel<T><<<(unsigned) ((count + 255) / 256), 256, 0, stream()>>>(w, wt, g.K, g.F, Kp, g.ldw);
 		CATTLE_HIP_CHECK(hipGetLastError());
 	}
+	/* the staging pass deals threads over windows of at most a tile's positions */
+	if (epi == EPI_POOL && E.prh * E.prw > 64)
+		return false;
 	return launch_gather<T>(x, wt, b, out, g, nullptr, epi, &E, mtiles);
 }
 

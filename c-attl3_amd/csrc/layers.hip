@@ -46,17 +46,56 @@ void ensure_init(int device) {
 	g_ready = true;
 }
 
+/* Recorded graphs keep the device addresses of the buffers their kernels were given. A clock that ticks at every
+ * allocation and at the end of every recording orders the two: an allocation made before the newest recording that
+ * is still alive may be what that graph points into, so it must neither move nor go back to the driver until the
+ * graph is destroyed. Growing or releasing such a buffer is refused (ERR_STATE); one whose owner is destroyed is
+ * parked and freed when no living graph is older than it. */
+uint64_t g_alloc_clock = 0;
+std::vector<uint64_t> g_live_graphs;           /* clock values at which the living graphs were recorded */
+struct Parked { void* p; uint64_t born; };
+std::vector<Parked> g_parked;
+
+uint64_t newest_live_graph() {
+	uint64_t newest = 0;
+	for (uint64_t at : g_live_graphs)
+		newest = std::max(newest, at);
+	return newest;
+}
+
+void free_unpinned_parked() {
+	const uint64_t newest = newest_live_graph();
+	size_t kept = 0;
+	for (size_t i = 0; i < g_parked.size(); ++i) {
+		if (g_parked[i].born < newest)
+			g_parked[kept++] = g_parked[i];
+		else
+			(void) hipFree(g_parked[i].p);
+	}
+	g_parked.resize(kept);
+}
+
 /* Grow-only device buffer. */
 struct DevBuf {
 	void* p = nullptr;
 	size_t cap = 0;
+	uint64_t born = 0;
 	DevBuf() { }
 	DevBuf(const DevBuf&) = delete;
 	DevBuf& operator=(const DevBuf&) = delete;
 	~DevBuf() {
-		release();
+		/* the owner goes away: what a living graph may still point into waits for that graph's end */
+		if (p && pinned_by_graph(born))
+			park_allocation(p, born);
+		else if (p)
+			(void) hipFree(p);
+	}
+	bool pinned() const {
+		return p != nullptr && pinned_by_graph(born);
 	}
 	void release() {
+		if (pinned())
+			throw Error(ERR_STATE, "a recorded graph may point into this buffer: destroy the graph (cattle_hip_graph_destroy) before releasing it");
 		if (p)
 			(void) hipFree(p);
 		p = nullptr;
@@ -66,10 +105,14 @@ struct DevBuf {
 		if (bytes > cap) {
 			/* recorded work may already point into the old buffer */
 			forbid_while_capturing("growing a buffer of a layer (run the step once, at this batch size, before recording it)");
+			if (pinned())
+				throw Error(ERR_STATE, "a recorded graph may point into a buffer that this call has to grow: destroy the graph "
+						"(cattle_hip_graph_destroy) first, or run at the largest size before recording");
 			release();
 			const size_t want = (bytes + 255) / 256 * 256;
 			CATTLE_HIP_CHECK(hipMalloc(&p, want));
 			cap = want;
+			born = alloc_clock_tick();
 		}
 		return p;
 	}
@@ -278,8 +321,9 @@ struct LayerBase {
 	DevBuf in_stage, out_stage, og_stage, ig_stage;
 	size_t batch = 0;
 	bool have_forward = false;
+	uint64_t created;                  /* on the allocation clock: all buffers of the layer are younger */
 
-	LayerBase(int dtype) : dtype(dtype) { }
+	LayerBase(int dtype) : dtype(dtype), created(alloc_clock_tick()) { }
 	virtual ~LayerBase() { }
 	size_t esize() const {
 		return dtype == CATTLE_HIP_F32 ? 4 : 8;
@@ -479,6 +523,7 @@ struct ConvLstm : LayerBase {
 	LstmActs<T> acts;
 	bool foremost;
 	bool mul_int = false;           /* LSTMNeuralNetwork<Scalar,Rank,MulInt = true> (:44, :303-311) */
+	bool fuse_steps = true;         /* run the element-wise part of a step inside the recurrent kernels where the shapes allow */
 	int fused_forward_steps = 0, fused_backward_steps = 0;      /* of the last propagate / backpropagate */
 	/* alignment of the last propagate (:398-401) */
 	size_t T_in = 0, T_out = 0, delay = 0, steps = 0;
@@ -552,9 +597,7 @@ struct ConvLstm : LayerBase {
 		hprev_all.ensure(p * total * e);
 		const ConvWorkspace wsh = conv_workspace<T>(sh, n);
 		T* wth = (T*) wh.derived[0].ensure(wsh.wt_fwd * e);
-		/* CATTLE_HIP_NO_LSTM_FUSION (experiments; read once): every step's element-wise part as a kernel of its own */
-		static const bool no_fusion = std::getenv("CATTLE_HIP_NO_LSTM_FUSION") != nullptr;
-		bool fused_steps = !no_fusion;
+		bool fused_steps = fuse_steps;
 		fused_forward_steps = 0;
 		T* wth_gates = nullptr;             /* the prepared layout of the kernel that runs the step itself */
 		for (size_t t = 0; t < total; ++t) {
@@ -623,7 +666,7 @@ struct ConvLstm : LayerBase {
 			/* the four output-side kernels' pass_back, summed (:470-473, :491-494), is one input-gradient launch, and
 			 * the element-wise part of step t - 1, which is all that reads its result, runs in the kernel that sums the
 			 * parts of that launch's reductions when the launch has such a kernel */
-			static const bool no_fusion = std::getenv("CATTLE_HIP_NO_LSTM_FUSION") != nullptr;
+			const bool no_fusion = !fuse_steps;
 			const LstmBackwardStep<T> before = backward_step(t - 1);
 			const bool done = conv_input_gradient<T>(sh, n, (const T*) wh.values.p, (const T*) dzh_all.p + N * t, (T*) dh.p, wtd,
 					wh.derived_version[1] == wh.version, no_fusion ? nullptr : &before, (int) (N * total));
@@ -1174,6 +1217,9 @@ struct DropoutLayer : LayerBase {
 	void forward(const void* in, size_t N, bool training, void* out) override {
 		const size_t total = N * in_volume();
 		if (training) {
+			/* the mask's key, a function of the number of the pass, is an argument of the kernel: a recorded launch
+			 * would draw the same mask at every replay */
+			forbid_while_capturing("a training pass of a dropout layer (its mask changes from pass to pass; record the layers around it)");
 			dropout_apply<T>(total, dropout_pass_key(seed, passes), prob, eps, (const T*) in, (T*) out);
 			++passes;
 			have_mask = true;
@@ -1255,6 +1301,7 @@ struct Graph {
 	hipGraph_t graph = nullptr;
 	hipGraphExec_t exec = nullptr;
 	std::vector<void*> blocks;
+	uint64_t recorded_at = 0;          /* on the allocation clock: older allocations are pinned while the graph lives */
 };
 
 LayerBase* as_layer(cattle_hip_layer_t h) {
@@ -1517,6 +1564,18 @@ hipStream_t stream() {
 	return g_stream;
 }
 
+uint64_t alloc_clock_tick() {
+	return ++g_alloc_clock;
+}
+
+bool pinned_by_graph(uint64_t born) {
+	return born < newest_live_graph();
+}
+
+void park_allocation(void* p, uint64_t born) {
+	g_parked.push_back(Parked{ p, born });
+}
+
 bool capturing() {
 	return g_capturing;
 }
@@ -1680,6 +1739,8 @@ int cattle_hip_graph_end_capture(cattle_hip_graph_t* graph) {
 				throw Error(ERR_INVALID, "null output pointer");
 			throw Error(ERR_DEVICE, std::string("the recording could not be turned into a graph: ") + hipGetErrorString(e));
 		}
+		gr->recorded_at = alloc_clock_tick();
+		g_live_graphs.push_back(gr->recorded_at);
 		*graph = reinterpret_cast<cattle_hip_graph_t>(gr.release());
 	});
 }
@@ -1702,6 +1763,10 @@ int cattle_hip_graph_destroy(cattle_hip_graph_t graph) {
 		(void) hipGraphExecDestroy(gr->exec);
 		(void) hipGraphDestroy(gr->graph);
 		g_pool.release_graph(&gr->blocks);
+		std::vector<uint64_t>::iterator at = std::find(g_live_graphs.begin(), g_live_graphs.end(), gr->recorded_at);
+		if (at != g_live_graphs.end())
+			g_live_graphs.erase(at);
+		free_unpinned_parked();
 		delete gr;
 	});
 }
@@ -2149,7 +2214,7 @@ int cattle_hip_layer_destroy(cattle_hip_layer_t layer) {
 	return guarded([&] {
 		if (layer) {
 			forbid_while_capturing("waiting for the device");
-		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
+			CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
 			delete reinterpret_cast<LayerBase*>(layer);
 		}
 	});
@@ -2183,6 +2248,10 @@ int cattle_hip_layer_set_input_layer(cattle_hip_layer_t layer, int is_input_laye
 int cattle_hip_layer_empty_cache(cattle_hip_layer_t layer) {
 	return guarded([&] {
 		forbid_while_capturing("waiting for the device");
+		/* the caches it frees may be what a living graph, recorded after the layer was created, points into */
+		if (pinned_by_graph(as_layer(layer)->created))
+			throw Error(ERR_STATE, "a recorded graph may point into the layer's caches: destroy the graph (cattle_hip_graph_destroy) "
+					"before emptying them");
 		CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
 		as_layer(layer)->empty_cache();
 	});

@@ -102,8 +102,16 @@ int cattle_hip_timer_stop(cattle_hip_timer_t timer, float* elapsed_ms);   /* syn
  *    cattle_hip_alloc returned during the recording; cattle_hip_free on them takes effect when the graph is destroyed),
  *    the same batch size, and the same scalars - an optimizer whose update depends on the time step or epoch (Adam,
  *    Nadam, AMSGrad, ...) is therefore called outside the recording, as is anything whose result the host must see;
- *  - layers that took part, and their caches, must be left alone while launches of the graph are in flight, and
- *    destroyed only after the graph. */
+ *  - a training pass of a dropout layer cannot be recorded (CATTLE_HIP_ERR_STATE): its mask is a function of the number
+ *    of the pass, which a replay would not advance; record the layers on either side of it;
+ *  - a graph holds the device addresses it was recorded with. As long as it exists, a buffer of the library that was
+ *    allocated before the recording ended stays where it is: a call that would have to grow one (a layer that took
+ *    part run at a larger batch size; any layer whose split reduction needs more of the shared scratch buffer than
+ *    every call before the recording did) and cattle_hip_layer_empty_cache on a layer created before the recording
+ *    return CATTLE_HIP_ERR_STATE until cattle_hip_graph_destroy; the buffers of a layer that is destroyed while the
+ *    graph exists are kept until then, so that a later launch still finds memory of its own (its results are then
+ *    meaningless, never a fault). Layers and buffers created after the recording are free to change;
+ *  - layers that took part, and their caches, must be left alone while launches of the graph are in flight. */
 int cattle_hip_graph_begin_capture(void);
 int cattle_hip_graph_end_capture(cattle_hip_graph_t* graph);
 int cattle_hip_graph_launch(cattle_hip_graph_t graph);

@@ -35,3 +35,39 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(binding, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(pkg.CattleHipError):
         binding.lib()
+
+
+class _FakeTensor(object):
+    """Stands in for a DeviceTensor: the wrapper's checks read shape and dtype only and must fire before any call."""
+
+    def __init__(self, shape, dtype="float32"):
+        import numpy as np
+        self.shape, self.dtype, self.ptr = tuple(shape), np.dtype(dtype), None
+
+
+@pytest.mark.parametrize("what, kw", [
+    ("weights rows", dict(weights=_FakeTensor((26, 8)))),
+    ("bias shape", dict(bias=_FakeTensor((8, 1)))),
+    ("out extent", dict(out=_FakeTensor((4, 6, 5, 8)))),
+    ("out filters", dict(out=_FakeTensor((4, 6, 6, 7)))),
+    ("out dtype", dict(out=_FakeTensor((4, 6, 6, 8), "float64"))),
+    ("weights dtype", dict(weights=_FakeTensor((27, 8), "float64"))),
+    ("rank", dict(x=_FakeTensor((4, 6, 6)))),
+    ("receptor larger than input", dict(receptor_height=9)),
+])
+def test_noalloc_wrapper_refuses_mismatched_buffers(monkeypatch, what, kw):
+    """The C entry point takes raw addresses: the Python wrapper is where extents can be checked. Every mismatch must be
+    refused before the library is called (the library is replaced by an object that fails on any use)."""
+    binding = importlib.import_module("c-attl3_amd.binding")
+
+    class Untouchable(object):
+        def __getattr__(self, name):
+            raise AssertionError("the library was called: " + name)
+
+    monkeypatch.setattr(binding, "_lib", Untouchable())
+    args = dict(x=_FakeTensor((4, 6, 6, 3)), weights=_FakeTensor((27, 8)), bias=_FakeTensor((1, 8)), out=_FakeTensor((4, 6, 6, 8)))
+    geom = {}
+    for k, v in kw.items():
+        (args if k in args else geom)[k] = v
+    with pytest.raises(ValueError):
+        binding.conv_forward_noalloc(args["x"], args["weights"], args["bias"], args["out"], **geom)

@@ -150,6 +150,10 @@ EXACT_CASES = [
     (16, 9, 9, 3, 6, ("relu", 0.0), ("max", 3, 3, 2, 2), "act"),            # overlapping windows: the pool runs on its own
     (6, 8, 8, 3, 6, ("relu", 0.0), ("max", 2, 2, 2, 2), None),               # rows of 6: 16-byte accesses in fp64 only
     (7, 8, 8, 3, 6, ("relu", 0.0), ("max", 2, 2, 2, 2), "unfused"),          # rows of 7: member by member
+    # tiling windows of more than 64 elements: the pooling epilogue declines, the activation epilogue takes over
+    (16, 16, 16, 3, 8, ("relu", 0.0), ("max", 16, 16, 16, 16), "act"),
+    (16, 18, 18, 3, 8, ("relu", 0.0), ("max", 9, 9, 9, 9), "act"),
+    (16, 16, 16, 3, 8, None, ("max", 8, 16, 8, 16), "unfused"),
 ]
 
 
@@ -178,6 +182,41 @@ def test_fused_selections_exact(case, dtype):
     assert np.array_equal(dx, grads["dx"]), "input gradient"
     assert np.array_equal(wp.get_grad(), grads["dw"]), "weight gradient"
     assert np.array_equal(bp.get_grad(), grads["db"].reshape(1, -1)), "bias gradient"
+
+
+@pytest.mark.parametrize("pool", [("max", 16, 16, 16, 16), ("max", 9, 9, 9, 9), ("max", 2, 2, 2, 2)], ids=lambda p: "%dx%d" % p[1:3])
+def test_fused_forward_after_weight_change(pool):
+    """The prepared weight layout must follow the weights whichever epilogue a forward pass ends up with: a first pass,
+    then an optimizer step on the device, then a second pass, each against the oracle chain on the current weights."""
+    dtype, N, C, F = np.float32, 16, 3, 8
+    H = W = 18 if pool[1] == 9 else 16
+    gen = hp.rng(91)
+    x = _dyadic(gen, (N, H, W, C), dtype)
+    w = _dyadic(gen, (9 * C, F), dtype)
+    b = _dyadic(gen, (1, F), dtype)
+    fused, members, kdims = _build(dtype, N, H, W, C, F, conv=GEOM_3X3, act=("relu", 0.0), pool=pool)
+    chain = Chain(GEOM_3X3, act=("relu", 0.0), pool=pool)
+    wp, bp = members["conv"].get_params()
+    for round_ in range(2):
+        ref = chain.forward(*(np.asarray(a, np.float64) for a in (x, w, b)))
+        g = _dyadic(gen, ref.shape, dtype)
+        out, dx, mode = _run_fused(fused, members, x, w, b, g)
+        assert mode == ("pool" if pool[1] == 2 else "act")
+        grads = chain.backward(np.asarray(x, np.float64), np.asarray(w, np.float64), np.asarray(g, np.float64))
+        if round_ == 0:
+            assert np.array_equal(out, ref), "output"
+            assert np.array_equal(members["pool"].max_indices(N), chain.inds)
+            assert np.array_equal(dx, grads["dx"])
+            assert np.array_equal(wp.get_grad(), grads["dw"])
+        else:       # the updated weights are finer-grained: sums may round
+            assert hp.rel_err(out, ref, label="fused forward, updated weights") < 1e-5
+            assert hp.rel_err(wp.get_grad(), grads["dw"], label="fused dw, updated weights") < 1e-5
+        # a step of -1/4 times the (dyadic) gradient keeps the weights dyadic, then one more forward pass on them
+        wp.optimizer_update("vanilla_sgd", [0.25])
+        w = wp.get_values()
+        out2 = fused.pass_forward(x, True)
+        ref2 = chain.forward(np.asarray(x, np.float64), np.asarray(w, np.float64), np.asarray(b, np.float64))
+        assert hp.rel_err(out2, ref2, label="fused forward after update") < 1e-5, "pass after the update %d" % round_
 
 
 def test_fused_rectifier_side_of_zero():

@@ -190,3 +190,98 @@ def test_what_cannot_be_recorded_is_refused():
     graph.destroy()
     h = ctypes.c_void_p()
     assert ch.lib().cattle_hip_graph_end_capture(ctypes.byref(h)) == 2       # no recording in progress
+
+
+def test_a_living_graph_pins_the_buffers_it_may_point_into():
+    """A graph keeps device addresses. While it exists, nothing that was allocated before its recording ended may move
+    or be freed: growth and empty_cache are refused with the state error (no kernel ever runs on freed memory), and
+    everything is allowed again once the graph is destroyed."""
+    dtype, N = np.float32, 16
+    gen = hp.rng(5)
+    net, params, _ = _mlp(dtype, True)
+    _init(params, 5, dtype)
+    plist = ch.ParameterList(params)
+    x = ch.DeviceTensor.from_host(hp.uniform(gen, (N, 20), -1, 1, dtype))
+    y_host = np.zeros((N, 6), dtype, order="F")
+    y_host[np.arange(N), gen.integers(0, 6, N)] = 1
+    y = ch.DeviceTensor.from_host(y_host)
+    # an unrelated convolution whose cut reduction will want more of the shared scratch buffer than anything so far
+    conv = ch.ConvKernelLayer(dtype, (16, 16, 64), 32)
+    xc_small = ch.DeviceTensor.from_host(hp.normal(gen, (4, 16, 16, 64), dtype))
+    conv.pass_forward(xc_small, True)
+    conv.pass_back(ch.DeviceTensor.from_host(hp.normal(gen, (4, 16, 16, 32), dtype)))      # its partial-sum buffer exists now
+    ch.trim()                                               # nothing idle that the tests before left behind
+    _step(net, plist, x, y, N)
+    with ch.Graph() as graph:
+        _step(net, plist, x, y, N)
+    big = 4 * N
+    xb = ch.DeviceTensor.from_host(hp.uniform(gen, (big, 20), -1, 1, dtype))
+    # (a) the recorded layers at a larger batch: their buffers would have to grow
+    with pytest.raises(ch.CattleHipError) as e:
+        a = xb
+        for l in net:
+            a = l.pass_forward(a, True)
+        for l in reversed(net):
+            a = l.pass_back(a)
+    assert e.value.code == 2 and "graph" in str(e.value)
+    # (b) empty_cache of a recorded layer
+    with pytest.raises(ch.CattleHipError) as e:
+        net[0].empty_cache()
+    assert e.value.code == 2 and "graph" in str(e.value)
+    # (c) an unrelated, older layer that needs a larger shared scratch buffer (8 tiles cut into many parts)
+    xc_big = ch.DeviceTensor.from_host(hp.normal(gen, (64, 16, 16, 64), dtype))
+    grew = True
+    try:
+        conv.pass_forward(xc_big, True)
+        conv.pass_back(ch.DeviceTensor.from_host(hp.normal(gen, (64, 16, 16, 32), dtype)))
+        grew = False
+    except ch.CattleHipError as err:
+        assert err.code == 2 and "graph" in str(err)
+    assert grew, "the larger problem was expected to need a larger scratch or partials buffer"
+    # the graph still launches, on memory of its own
+    graph.launch()
+    ch.synchronize()
+    # a layer created after the recording is free to grow and to empty its caches
+    young = ch.DenseKernelLayer(dtype, (20,), 7)
+    young.pass_forward(x, True)
+    young.pass_forward(xb, True)
+    young.empty_cache()
+    graph.destroy()
+    # and so is everything else once the graph is gone
+    a = xb
+    for l in net:
+        a = l.pass_forward(a, True)
+    net[0].empty_cache()
+    conv.pass_forward(xc_big, True)
+    ch.synchronize()
+
+
+def test_destroying_a_recorded_layer_keeps_its_buffers_until_the_graph_goes():
+    dtype, N = np.float32, 8
+    layer = ch.DenseKernelLayer(dtype, (12,), 5)
+    x = ch.DeviceTensor.from_host(hp.uniform(hp.rng(1), (N, 12), -1, 1, dtype))
+    out = layer.pass_forward(x, True)
+    with ch.Graph() as graph:
+        layer.forward_into(x, out, True)
+    del layer                                   # its parameter buffers are what the recorded kernels read
+    graph.launch()                              # must not touch freed memory: the buffers are parked
+    ch.synchronize()
+    graph.destroy()
+    ch.synchronize()
+
+
+def test_dropout_training_pass_is_not_recorded():
+    dtype, N = np.float32, 8
+    drop = ch.DropoutLayer(dtype, (12,), 0.5, seed=3)
+    x = ch.DeviceTensor.from_host(hp.uniform(hp.rng(1), (N, 12), -1, 1, dtype))
+    y = ch.DeviceTensor((N, 12), dtype)
+    drop.forward_into(x, y, True)
+    with ch.Graph() as graph:
+        with pytest.raises(ch.CattleHipError) as e:
+            drop.forward_into(x, y, True)
+        assert e.value.code == 2 and "dropout" in str(e.value)
+        drop.forward_into(x, y, False)          # inference hands the input through: a copy, recordable
+    graph.launch()
+    ch.synchronize()
+    assert np.array_equal(y.to_host(), x.to_host())
+    graph.destroy()
