@@ -120,15 +120,33 @@ template<typename T> struct WgradAct {
 	int kind;
 	T p;
 };
+/* Partial sums that wait to be added to their gradients: entry e is `splits` matrices of `count` values each, one
+ * after the other at `partials`, to be added to dst in the fixed order of reduce_partials_many (first_block is filled in
+ * by it; wide / vec pick the form of the sum, set by whoever wrote the partials). */
+constexpr int REDUCE_BATCH = 32;
+template<typename T> struct ReduceEntry {
+	const T* partials;
+	T* dst;
+	size_t count;
+	int splits, first_block;
+	bool wide, vec;
+};
+template<typename T> struct ReduceBatch { ReduceEntry<T> e[REDUCE_BATCH]; int count; };
+/* dst += sum of the partials, for every entry, in one launch */
+template<typename T> void reduce_partials_many(ReduceBatch<T> batch);
+
 /* Backward: wgrad[K x F] += A^T G, bgrad[F] += colsum(G), in_grad = dgrad (skipped if null). With `act`, G is
- * act'(y) * out_grad (see WgradAct; act->dz must be given when in_grad is). */
+ * act'(y) * out_grad (see WgradAct; act->dz must be given when in_grad is). With `deferred`, a weight gradient cut into
+ * slices of M leaves the sum of its slices to the caller: the entries (none if the launch added to the gradients
+ * itself) go to reduce_partials_many whenever the gradients are first needed, which spares a launch per layer. */
 template<typename T> void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad,
-		T* wgrad, T* bgrad, T* in_grad, T* wt_dgrad, bool wt_ready, T* partials, const WgradAct<T>* act = nullptr);
+		T* wgrad, T* bgrad, T* in_grad, T* wt_dgrad, bool wt_ready, T* partials, const WgradAct<T>* act = nullptr,
+		ReduceBatch<T>* deferred = nullptr);
 
 /* The two halves of conv_backward on their own (the transposed convolution uses them with the roles
  * of input and output exchanged). bgrad may be null. */
 template<typename T> void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad,
-		T* partials, const WgradAct<T>* act = nullptr);
+		T* partials, const WgradAct<T>* act = nullptr, ReduceBatch<T>* deferred = nullptr);
 template<typename T> struct LstmBackwardStep;
 /* og_batch > 0: out_grad holds the first N of og_batch samples per position (GatherGeom::NS). `then`, if given, is the LSTM backward step that consumes in_grad as the gradient of its hidden output: when the
  * launch cuts every tile's reduction into parts, the kernel that sums the parts runs the element-wise part of that
@@ -309,7 +327,13 @@ template<typename T> struct OptParam {
 	size_t n;
 	int K, RHW, ldw_fwd, ldw_dgrad;
 	T l1, l2;           /* the lambdas of the parameter's regularization (both 0: none) */
+	/* `splits` partial sums of the gradient, n values each, that still wait to be added to it (a weight gradient cut
+	 * into a few slices): the kernel adds them in ascending order, as reduce_partials_many would have; null: none */
+	const T* parts;
+	int splits;
 };
+/* how many partial sums an optimizer launch takes along per parameter (more go through reduce_partials_many first) */
+constexpr int OPT_MAX_PARTS = 8;
 template<typename T> struct OptBatch { OptParam<T> p[OPT_BATCH]; int count; };
 /* update + gradient reset of every parameter of the batch, one launch */
 template<typename T> void optimizer_step_many(int rule, const double hyper[4], size_t epoch, size_t timestep, const OptBatch<T>& batch);

@@ -1107,24 +1107,15 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	}
 }
 
-/* dst[i] += sum_s partials[s][i] for the weight gradient (blocks below wblocks) and the bias gradient (the
- * remaining blocks) in one launch. A block covers 64 outputs with GR groups of threads, V consecutive outputs
- * per thread; group j adds the partials s = j, j+GR, j+2GR, ... in ascending order and the group sums are then
- * added in ascending order, so the summation order is fixed and results are reproducible. For V > 1 both
- * counts are multiples of V and the partials are 16-byte aligned. */
+/* dst[i] += sum_s partials[s][i] for 64 outputs of one matrix: block `blk` of it covers outputs [64 blk, 64 blk + 64)
+ * with GR groups of threads, V consecutive outputs per thread; group j adds the partials s = j, j+GR, j+2GR, ... in
+ * ascending order and the group sums are then added in ascending order, so the summation order is fixed and results
+ * are reproducible. For V > 1 the count is a multiple of V and the partials are 16-byte aligned. */
 template<typename T, int V>
-__global__ __launch_bounds__(256)
-void reduce_partials_kernel(const T* __restrict__ partials, T* __restrict__ dst, size_t count,
-		const T* __restrict__ bias_partials, T* __restrict__ bias_dst, size_t bias_count, int wblocks, int splits) {
+__device__ __forceinline__ void reduce_partials_block(const T* __restrict__ partials, T* __restrict__ dst, size_t count, int blk,
+		int splits, T (&lds)[16][64]) {
 	constexpr int OV = 64 / V, GR = 256 / OV;
-	__shared__ T lds[GR][64];
-	int blk = blockIdx.x;
-	if (blk >= wblocks) {
-		blk -= wblocks;
-		partials = bias_partials;
-		dst = bias_dst;
-		count = bias_count;
-	}
+	static_assert(GR <= 16, "group sums fit the staging array");
 	const int ox = (threadIdx.x % OV) * V, grp = threadIdx.x / OV;
 	const size_t i = (size_t) blk * 64 + ox;
 	T s[V];
@@ -1153,22 +1144,15 @@ void reduce_partials_kernel(const T* __restrict__ partials, T* __restrict__ dst,
 	}
 }
 
-/* The same sums for a small gradient (a few thousand values) cut into many partials: a wavefront per output, lane l
- * adds the partials s = l, l + 64, ... in ascending order and the 64 lane sums are combined by a fixed shuffle tree.
- * With few outputs the kernel above is a handful of blocks walking hundreds of partials one after the other. */
+/* The same sums for a small gradient (a few thousand values) cut into many partials: a wavefront per output (four per
+ * block), lane l adds the partials s = l, l + 64, ... in ascending order and the 64 lane sums are combined by a fixed
+ * shuffle tree. With few outputs the form above is a handful of blocks walking hundreds of partials one after the other. */
 template<typename T>
-__global__ __launch_bounds__(256)
-void reduce_partials_wide_kernel(const T* __restrict__ partials, T* __restrict__ dst, size_t count,
-		const T* __restrict__ bias_partials, T* __restrict__ bias_dst, size_t bias_count, int splits) {
-	size_t i = (size_t) blockIdx.x * 4 + threadIdx.x / 64;
-	if (i >= count + bias_count)
+__device__ __forceinline__ void reduce_partials_wide_block(const T* __restrict__ partials, T* __restrict__ dst, size_t count, int blk,
+		int splits) {
+	const size_t i = (size_t) blk * 4 + threadIdx.x / 64;
+	if (i >= count)
 		return;
-	if (i >= count) {
-		i -= count;
-		partials = bias_partials;
-		dst = bias_dst;
-		count = bias_count;
-	}
 	const int lane = threadIdx.x % 64;
 	T s = (T) 0;
 	for (int p = lane; p < splits; p += 64)
@@ -1178,6 +1162,26 @@ void reduce_partials_wide_kernel(const T* __restrict__ partials, T* __restrict__
 		s += __shfl_down(s, off, 64);
 	if (lane == 0)
 		dst[i] += s;
+}
+
+/* The partial sums of up to REDUCE_BATCH matrices (the weight and the bias gradients of several layers) added to their
+ * gradients in one launch: block b belongs to the entry whose range of blocks holds it. Every entry is summed in the
+ * order the forms above fix, whatever else shares the launch. */
+template<typename T>
+__global__ __launch_bounds__(256)
+void reduce_partials_many_kernel(const ReduceBatch<T> batch) {
+	__shared__ T lds[16][64];
+	int e = 0;
+	while (e + 1 < batch.count && (int) blockIdx.x >= batch.e[e + 1].first_block)
+		++e;
+	const ReduceEntry<T>& q = batch.e[e];
+	const int blk = (int) blockIdx.x - q.first_block;
+	if (q.wide)
+		reduce_partials_wide_block<T>(q.partials, q.dst, q.count, blk, q.splits);
+	else if (q.vec)
+		reduce_partials_block<T, 16 / (int) sizeof(T)>(q.partials, q.dst, q.count, blk, q.splits, lds);
+	else
+		reduce_partials_block<T, 1>(q.partials, q.dst, q.count, blk, q.splits, lds);
 }
 
 /* Forward weights: wt[k][f] = w[k + K*f], zero-padded to Kp rows x ldw columns. gate_block > 0: the columns in the
@@ -2118,8 +2122,10 @@ void conv_forward_static(const ConvShape& s, int N, const T* x, const T* w, cons
 
 template<typename T>
 void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials,
-		const WgradAct<T>* act) {
+		const WgradAct<T>* act, ReduceBatch<T>* deferred) {
 	check_sizes(s, N);
+	if (deferred)
+		deferred->count = 0;
 	const GatherGeom g = forward_geom(s, N);
 	/* split-M partials, then a fixed-order reduction that accumulates */
 	const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
@@ -2137,21 +2143,42 @@ void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_gr
 	}
 	const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode, 0 };
 	v.launch(x, out_grad, partials, bias_partials, g, split, vec, act);
-	const int wblocks = (int) ((count + 63) / 64), bblocks = bgrad ? (g.F + 63) / 64 : 0;
+	/* a few thousand outputs cut into many partials: a wavefront per output; else 64 outputs per block, 16-byte loads
+	 * where counts and alignment allow */
 	constexpr int V = 16 / (int) sizeof(T);
 	const size_t outputs = count + (bgrad ? (size_t) g.F : 0);
-	if (outputs <= 8192 && p.splits >= 32) {
-		reduce_partials_wide_kernel<T><<<(unsigned) ((outputs + 3) / 4), 256, 0, stream()>>>(partials, wgrad, count, bias_partials,
-				bgrad, bgrad ? (size_t) g.F : 0, p.splits);
-		CATTLE_HIP_CHECK(hipGetLastError());
+	const bool wide = outputs <= 8192 && p.splits >= 32;
+	const bool vec_sum = count % V == 0 && g.F % V == 0 && (reinterpret_cast<uintptr_t>(partials) & 15) == 0;
+	ReduceBatch<T> both;
+	both.count = 0;
+	both.e[both.count++] = ReduceEntry<T>{ partials, wgrad, count, p.splits, 0, wide, vec_sum };
+	if (bgrad)
+		both.e[both.count++] = ReduceEntry<T>{ bias_partials, bgrad, (size_t) g.F, p.splits, 0, wide, vec_sum };
+	if (deferred) {
+		/* the caller adds the partial sums to the gradients later, together with those of other layers */
+		*deferred = both;
 		return;
 	}
-	if (count % V == 0 && g.F % V == 0 && (reinterpret_cast<uintptr_t>(partials) & 15) == 0)
-		reduce_partials_kernel<T, V><<<(unsigned) (wblocks + bblocks), 256, 0, stream()>>>(partials, wgrad, count, bias_partials,
-				bgrad, (size_t) g.F, wblocks, p.splits);
-	else
-		reduce_partials_kernel<T, 1><<<(unsigned) (wblocks + bblocks), 256, 0, stream()>>>(partials, wgrad, count, bias_partials,
-				bgrad, (size_t) g.F, wblocks, p.splits);
+	reduce_partials_many<T>(both);
+}
+
+template<typename T>
+void reduce_partials_many(ReduceBatch<T> batch) {
+	if (batch.count == 0)
+		return;
+	CATTLE_HIP_REQUIRE(batch.count <= REDUCE_BATCH, "too many matrices in one reduce launch");
+	int blocks = 0;
+	for (int i = 0; i < batch.count; ++i) {
+		ReduceEntry<T>& q = batch.e[i];
+		q.first_block = blocks;
+		const size_t per = q.wide ? 4 : 64;
+		const size_t need = (q.count + per - 1) / per;
+		CATTLE_HIP_REQUIRE(need + (size_t) blocks <= 2147483647u, "gradients too large for one reduce launch");
+		blocks += (int) need;
+	}
+	if (blocks == 0)
+		return;
+	reduce_partials_many_kernel<T><<<(unsigned) blocks, 256, 0, stream()>>>(batch);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
@@ -2176,9 +2203,9 @@ bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_gra
 
 template<typename T>
 void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad,
-		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials, const WgradAct<T>* act) {
+		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials, const WgradAct<T>* act, ReduceBatch<T>* deferred) {
 	CATTLE_HIP_REQUIRE(!act || !in_grad || act->dz != nullptr, "the input gradient needs the gradient before the activation");
-	conv_weight_gradient<T>(s, N, x, out_grad, wgrad, bgrad, partials, act);
+	conv_weight_gradient<T>(s, N, x, out_grad, wgrad, bgrad, partials, act, deferred);
 	if (in_grad)
 		conv_input_gradient<T>(s, N, w, act ? (const T*) act->dz : out_grad, in_grad, wt_dgrad, wt_ready, nullptr, 0);
 }
@@ -2198,13 +2225,15 @@ template bool conv_forward_lstm<double>(const ConvShape&, int, const double*, in
 template void conv_forward_static<float>(const ConvShape&, int, const float*, const float*, const float*, float*);
 template void conv_forward_static<double>(const ConvShape&, int, const double*, const double*, const double*, double*);
 template void conv_backward<float>(const ConvShape&, int, const float*, const float*, const float*, float*, float*, float*,
-		float*, bool, float*, const WgradAct<float>*);
+		float*, bool, float*, const WgradAct<float>*, ReduceBatch<float>*);
 template void conv_backward<double>(const ConvShape&, int, const double*, const double*, const double*, double*, double*,
-		double*, double*, bool, double*, const WgradAct<double>*);
+		double*, double*, bool, double*, const WgradAct<double>*, ReduceBatch<double>*);
 template void conv_weight_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, float*,
-		const WgradAct<float>*);
+		const WgradAct<float>*, ReduceBatch<float>*);
 template void conv_weight_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, double*,
-		const WgradAct<double>*);
+		const WgradAct<double>*, ReduceBatch<double>*);
+template void reduce_partials_many<float>(ReduceBatch<float>);
+template void reduce_partials_many<double>(ReduceBatch<double>);
 template bool conv_input_gradient<float>(const ConvShape&, int, const float*, const float*, float*, float*, bool,
 		const LstmBackwardStep<float>*, int);
 template bool conv_input_gradient<double>(const ConvShape&, int, const double*, const double*, double*, double*, bool,

@@ -260,6 +260,11 @@ struct Param {
 	uint64_t version = 1;
 	DevBuf derived[3];
 	uint64_t derived_version[3] = { 0, 0, 0 };
+	/* A weight matrix: the partial sums of the last weight-gradient launch that was cut into slices (its own and, behind
+	 * them, those of the bias gradient). They are added to the gradients when a gradient is first needed - by the
+	 * optimizer step as a rule, in one launch for all layers - and until then `pending` lists them (see Deferred). */
+	DevBuf partials;
+	bool pending = false;
 	DevBuf moments[3];                 /* the optimizer's state matrices, allocated (zeroed) on first use */
 	int moments_ready = 0;             /* how many of them are */
 	double reg_l1 = 0, reg_l2 = 0;     /* ParameterRegularization of the parameter: L1 and L2 lambdas (both 0: none) */
@@ -271,6 +276,7 @@ struct Param {
 	bool constrains_grad() const {
 		return grad_limits[0] > 0 || grad_limits[1] > 0 || grad_limits[2] > 0;
 	}
+	~Param();
 	Param(size_t rows, size_t cols, bool optimizable, size_t esize) : rows(rows), cols(cols), optimizable(optimizable), esize(esize) {
 		values.ensure(bytes());
 		grad.ensure(bytes());
@@ -293,6 +299,96 @@ struct Param {
 };
 
 typedef std::shared_ptr<Param> ParamPtr;
+
+/* Sums of weight-gradient slices that have not been added to their gradients yet. Nothing reads a gradient between the
+ * backward pass of its layer and the optimizer step (FeedforwardNeuralNetwork.hpp:129-141 runs the layers back to front,
+ * SGDOptimizer.hpp:64 is the first reader), so the sums of all layers are taken there in one launch instead of one
+ * launch per layer inside the chain of backward launches. Whatever else touches a gradient (reading it, resetting it,
+ * its constraints, a deep copy, the next backward pass that would overwrite the partial sums, the start and the end
+ * of a recording) settles the sums first. The order of each sum is fixed by reduce_partials_many, so results do not
+ * depend on when it is taken. */
+struct Deferred {
+	struct Entry { Param* owner; ReduceEntry<float> f; ReduceEntry<double> d; };
+	std::vector<Entry> entries;
+	template<typename T> void add(Param* owner, const ReduceBatch<T>& batch) {
+		for (int i = 0; i < batch.count; ++i) {
+			Entry e = { owner, {}, {} };
+			pick<T>(e) = batch.e[i];
+			entries.push_back(e);
+		}
+		if (batch.count > 0)
+			owner->pending = true;
+	}
+	template<typename T> static ReduceEntry<T>& pick(Entry& e);
+	void settle() {
+		if (entries.empty())
+			return;
+		ReduceBatch<float> bf;
+		ReduceBatch<double> bd;
+		bf.count = bd.count = 0;
+		for (Entry& e : entries) {
+			e.owner->pending = false;
+			if (e.owner->esize == sizeof(float)) {
+				bf.e[bf.count++] = e.f;
+				if (bf.count == REDUCE_BATCH) {
+					reduce_partials_many<float>(bf);
+					bf.count = 0;
+				}
+			} else {
+				bd.e[bd.count++] = e.d;
+				if (bd.count == REDUCE_BATCH) {
+					reduce_partials_many<double>(bd);
+					bd.count = 0;
+				}
+			}
+		}
+		entries.clear();
+		reduce_partials_many<float>(bf);
+		reduce_partials_many<double>(bd);
+	}
+	/* The one entry that waits to be added to `grad`, if it is few enough slices for the optimizer launch to add them on
+	 * its way (in the order reduce_partials_many would: for up to as many slices as it has groups of threads that is
+	 * plain ascending order); the entry is then taken off the list. Null: none, several, or too many slices. */
+	template<typename T> bool take_for_optimizer(const T* grad, ReduceEntry<T>& out) {
+		int found = -1;
+		for (size_t i = 0; i < entries.size(); ++i)
+			if (pick<T>(entries[i]).dst == grad && entries[i].owner->esize == sizeof(T)) {
+				if (found >= 0)
+					return false;
+				found = (int) i;
+			}
+		if (found < 0)
+			return false;
+		const ReduceEntry<T>& e = pick<T>(entries[found]);
+		const int groups = e.vec ? 16 : 4;          /* reduce_partials_block's GR for 16-byte and for scalar loads */
+		if (e.wide || e.splits > std::min(OPT_MAX_PARTS, groups))
+			return false;
+		out = e;
+		Param* owner = entries[found].owner;
+		entries.erase(entries.begin() + found);
+		bool more = false;
+		for (const Entry& o : entries)
+			more = more || o.owner == owner;
+		owner->pending = more;
+		return true;
+	}
+	/* the owner goes away, and its gradient and partial sums with it */
+	void forget(Param* owner) {
+		size_t kept = 0;
+		for (size_t i = 0; i < entries.size(); ++i)
+			if (entries[i].owner != owner)
+				entries[kept++] = entries[i];
+		entries.resize(kept);
+	}
+};
+template<> ReduceEntry<float>& Deferred::pick<float>(Entry& e) { return e.f; }
+template<> ReduceEntry<double>& Deferred::pick<double>(Entry& e) { return e.d; }
+Deferred g_deferred;
+
+Param::~Param() {
+	if (pending)
+		g_deferred.forget(this);
+}
 
 template<typename T>
 void fill_constant(Param& p, T v) {
@@ -371,7 +467,6 @@ template<typename T>
 struct ConvLayer : LayerBase {
 	ConvShape shape;
 	const T* x_cache = nullptr;
-	DevBuf partials;
 
 	ConvLayer(int dtype, const ConvShape& s, bool dense) : LayerBase(dtype), shape(s) {
 		if (dense) {
@@ -412,9 +507,14 @@ struct ConvLayer : LayerBase {
 		Param& w = *params[0];
 		T* wt = (T*) w.derived[1].ensure(ws.wt_dgrad * sizeof(T));
 		const bool ready = w.derived_version[1] == w.version;
-		T* part = (T*) partials.ensure(ws.partials * sizeof(T));
+		/* the partial sums of the launch before, if they still wait, would be overwritten */
+		if (w.pending)
+			g_deferred.settle();
+		T* part = (T*) w.partials.ensure(ws.partials * sizeof(T));
+		ReduceBatch<T> later;
 		conv_backward<T>(shape, n, x_cache, (const T*) w.values.p, (const T*) out_grad, (T*) w.grad.p, (T*) params[1]->grad.p,
-				(T*) in_grad, wt, ready, part, act);
+				(T*) in_grad, wt, ready, part, act, &later);
+		g_deferred.add<T>(&w, later);
 		if (in_grad)
 			w.derived_version[1] = w.version;
 	}
@@ -528,7 +628,7 @@ struct ConvLstm : LayerBase {
 	/* alignment of the last propagate (:398-401) */
 	size_t T_in = 0, T_out = 0, delay = 0, steps = 0;
 	const T* x_cache = nullptr;
-	DevBuf zx_all, zh, z, gates, state, act_state, hprev_all, dzx_all, dzh_all, dh, state_grad, partials;
+	DevBuf zx_all, zh, z, gates, state, act_state, hprev_all, dzx_all, dzh_all, dh, state_grad;
 	DevBuf seq_in_stage, seq_out_stage, seq_og_stage, seq_ig_stage;
 
 	ConvLstm(int dtype, const ConvShape& x_shape, const ConvShape& h_shape, const LstmActs<T>& acts, bool foremost) :
@@ -676,16 +776,22 @@ struct ConvLstm : LayerBase {
 			else
 				lstm_gates_backward<T>(before, (const T*) dh.p);
 		}
-		/* parameter gradients of all steps at once: slab 0 of dzh_all and of hprev_all is zero */
+		/* parameter gradients of all steps at once: slab 0 of dzh_all and of hprev_all is zero. Each launch leaves the
+		 * sum of its slices to whoever reads the gradients first (Deferred). */
+		if (wh.pending || wx.pending)
+			g_deferred.settle();
+		ReduceBatch<T> later;
 		if (total > 1) {
 			const ConvWorkspace ws = conv_workspace<T>(sh, (int) (N * total));
 			conv_weight_gradient<T>(sh, (int) (N * total), (const T*) hprev_all.p, (const T*) dzh_all.p, (T*) wh.grad.p,
-					(T*) params[3]->grad.p, (T*) partials.ensure(ws.partials * e));
+					(T*) params[3]->grad.p, (T*) wh.partials.ensure(ws.partials * e), nullptr, &later);
+			g_deferred.add<T>(&wh, later);
 		}
 		{
 			const ConvWorkspace ws = conv_workspace<T>(sx, (int) (N * T_in));
 			conv_weight_gradient<T>(sx, (int) (N * T_in), x_cache, (const T*) dzx_all.p, (T*) wx.grad.p, (T*) params[1]->grad.p,
-					(T*) partials.ensure(ws.partials * e));
+					(T*) wx.partials.ensure(ws.partials * e), nullptr, &later);
+			g_deferred.add<T>(&wx, later);
 			if (in_grad) {
 				T* wt = (T*) wx.derived[1].ensure(ws.wt_dgrad * e);
 				conv_input_gradient<T>(sx, (int) (N * T_in), (const T*) wx.values.p, (const T*) dzx_all.p, in_grad, wt,
@@ -1405,6 +1511,7 @@ void run_optimizer(cattle_hip_layer_t layer, size_t index, cattle_hip_optimizer 
 		size_t timestep, bool reset_grad) {
 	Param& p = optimizable_param(layer, index);
 	CATTLE_HIP_REQUIRE(hyper != nullptr, "null hyper-parameter array");
+	g_deferred.settle();
 	const int states = optimizer_state_count((int) optimizer);
 	for (int i = p.moments_ready; i < states; ++i) {
 		fill_zero(p.moments[i].ensure(p.bytes()), p.bytes());
@@ -1442,7 +1549,17 @@ template<typename T>
 void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices, size_t count, cattle_hip_optimizer optimizer,
 		const double hyper[4], size_t epoch, size_t timestep) {
 	const int states = optimizer_state_count((int) optimizer);
+	/* The gradients become whole here. Partial sums of few slices ride along with the update of their parameter; the
+	 * others are added to their gradients first, in one launch for all layers. */
 	std::vector<Param*> seen, limited;
+	std::vector<std::pair<Param*, ReduceEntry<T>>> riding;
+	for (size_t i = 0; i < count; ++i) {
+		Param& p = optimizable_param(layers[i], indices[i]);
+		ReduceEntry<T> e;
+		if (p.esize == sizeof(T) && !p.constrains_grad() && g_deferred.take_for_optimizer<T>(static_cast<const T*>(p.grad.p), e))
+			riding.push_back(std::make_pair(&p, e));
+	}
+	g_deferred.settle();
 	OptBatch<T> batch;
 	batch.count = 0;
 	auto flush = [&] {
@@ -1468,6 +1585,13 @@ void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices,
 		q.n = p.rows * p.cols;
 		q.l1 = (T) p.reg_l1;
 		q.l2 = (T) p.reg_l2;
+		q.parts = nullptr;
+		q.splits = 0;
+		for (const std::pair<Param*, ReduceEntry<T>>& r : riding)
+			if (r.first == &p) {
+				q.parts = r.second.partials;
+				q.splits = r.second.splits;
+			}
 		if (p.constrains_grad() && (p.reg_l1 != 0 || p.reg_l2 != 0)) {
 			add_regularization<T>(p.rows * p.cols, static_cast<const T*>(p.values.p), static_cast<T*>(p.grad.p), q.l1, q.l2);
 			constrain(p, false);
@@ -1709,6 +1833,7 @@ int cattle_hip_graph_begin_capture(void) {
 	return guarded([&] {
 		if (g_capturing)
 			throw Error(ERR_STATE, "a graph is already being recorded");
+		g_deferred.settle();            /* nothing pending crosses into the recording ... */
 		CATTLE_HIP_CHECK(hipStreamBeginCapture(stream(), hipStreamCaptureModeRelaxed));
 		g_capturing = true;
 	});
@@ -1718,6 +1843,14 @@ int cattle_hip_graph_end_capture(cattle_hip_graph_t* graph) {
 	return guarded([&] {
 		if (!g_capturing)
 			throw Error(ERR_STATE, "no graph is being recorded");
+		/* ... or out of it: what the recorded passes left pending is summed by the recording itself, so that a launch
+		 * of the graph leaves whole gradients whatever the host does next */
+		bool settled = true;
+		try {
+			g_deferred.settle();
+		} catch (const Error&) {
+			settled = false;
+		}
 		g_capturing = false;
 		std::unique_ptr<Graph> gr(new Graph());
 		/* blocks freed during the recording stay out of circulation, whatever becomes of the graph */
@@ -1726,6 +1859,8 @@ int cattle_hip_graph_end_capture(cattle_hip_graph_t* graph) {
 			g_pool.owner[b] = &gr->blocks;
 		g_pool.taken.clear();
 		hipError_t e = hipStreamEndCapture(stream(), &gr->graph);
+		if (e == hipSuccess && !settled)
+			e = hipErrorUnknown;
 		if (e == hipSuccess && gr->graph != nullptr)
 			e = hipGraphInstantiate(&gr->exec, gr->graph, nullptr, nullptr, 0);
 		if (e != hipSuccess || gr->graph == nullptr || graph == nullptr) {
@@ -1749,6 +1884,7 @@ int cattle_hip_graph_launch(cattle_hip_graph_t graph) {
 	return guarded([&] {
 		CATTLE_HIP_REQUIRE(graph != nullptr, "null graph handle");
 		forbid_while_capturing("launching a graph");
+		g_deferred.settle();            /* the recorded calls did not know of sums that eager passes have left pending since */
 		CATTLE_HIP_CHECK(hipGraphLaunch(reinterpret_cast<Graph*>(graph)->exec, stream()));
 	});
 }
@@ -2001,6 +2137,7 @@ int cattle_hip_convlstm_get_kernel_grad(cattle_hip_layer_t lstm, size_t kernel, 
 		CATTLE_HIP_REQUIRE(grad != nullptr, "null buffer");
 		size_t offset, bytes;
 		Param& p = lstm_kernel_param(lstm, kernel, bias, offset, bytes);
+		g_deferred.settle();
 		copy_out(grad, space, (const char*) p.grad.p + offset, bytes);
 	});
 }
@@ -2206,6 +2343,7 @@ int cattle_hip_broadcast_create(cattle_hip_dtype dtype, const size_t input_dims[
 int cattle_hip_layer_clone(cattle_hip_layer_t layer, int share_params, cattle_hip_layer_t* clone) {
 	return guarded([&] {
 		CATTLE_HIP_REQUIRE(clone != nullptr, "null output pointer");
+		g_deferred.settle();            /* a deep copy copies the gradients */
 		*clone = reinterpret_cast<cattle_hip_layer_t>(as_layer(layer)->clone(share_params != 0));
 	});
 }
@@ -2214,6 +2352,7 @@ int cattle_hip_layer_destroy(cattle_hip_layer_t layer) {
 	return guarded([&] {
 		if (layer) {
 			forbid_while_capturing("waiting for the device");
+			g_deferred.settle();        /* partial sums of a bias gradient lie in the buffer of the weights' parameter object */
 			CATTLE_HIP_CHECK(hipStreamSynchronize(stream()));
 			delete reinterpret_cast<LayerBase*>(layer);
 		}
@@ -2308,8 +2447,10 @@ int cattle_hip_layer_backward(cattle_hip_layer_t layer, const void* out_grad, ca
 		l->backward(og_dev, batch, ig_dev);
 		/* accumulate_grad enforces the gradient's constraints after every accumulation (StandardParameters.hpp:119-122) */
 		for (const ParamPtr& q : l->params)
-			if (q->optimizable && q->constrains_grad())
+			if (q->optimizable && q->constrains_grad()) {
+				g_deferred.settle();
 				constrain(*q, false);
+			}
 		if (want_in_grad && in_grad_space == CATTLE_HIP_HOST)
 			copy_out(in_grad, CATTLE_HIP_HOST, ig_dev, in_bytes);
 	});
@@ -2360,6 +2501,7 @@ int cattle_hip_layer_get_param_grad(cattle_hip_layer_t layer, size_t index, void
 		check_space(space);
 		CATTLE_HIP_REQUIRE(grad != nullptr, "null buffer");
 		Param& p = param_at(as_layer(layer), index);
+		g_deferred.settle();
 		copy_out(grad, space, p.grad.p, p.bytes());
 	});
 }
@@ -2367,6 +2509,7 @@ int cattle_hip_layer_get_param_grad(cattle_hip_layer_t layer, size_t index, void
 int cattle_hip_layer_reset_param_grad(cattle_hip_layer_t layer, size_t index) {
 	return guarded([&] {
 		Param& p = param_at(as_layer(layer), index);
+		g_deferred.settle();
 		fill_zero(p.grad.p, p.bytes());
 	});
 }

@@ -444,6 +444,20 @@ void add_regularization_kernel(size_t n, const T* __restrict__ values, T* __rest
  * both zero-padded when they were first built): the new values are written there as well, which saves the two
  * re-layout launches of the next pass. The matrix is column-major (k fastest) and wt is f fastest, so a tile goes
  * through LDS and both sides are accessed along their contiguous index. */
+/* the gradient of element i: what has been accumulated plus the partial sums that still wait, these added up first, in
+ * ascending order from zero (the order and grouping of reduce_partials_many for so few of them) */
+template<typename T>
+__device__ __forceinline__ T whole_gradient(const OptParam<T>& q, size_t i) {
+	T g = q.grad[i];
+	if (q.parts != nullptr) {
+		T t = (T) 0;
+		for (int s = 0; s < q.splits; ++s)
+			t += q.parts[(size_t) s * q.n + i];
+		g += t;
+	}
+	return g;
+}
+
 template<typename T, int RULE>
 __global__ __launch_bounds__(256)
 void optimizer_step_many_kernel(OptBatch<T> batch, OptCoef<T> k) {
@@ -455,7 +469,7 @@ void optimizer_step_many_kernel(OptBatch<T> batch, OptCoef<T> k) {
 		for (int j = 0; j < 4; ++j) {
 			const size_t i = (size_t) blockIdx.x * 1024 + tid + 256 * j;
 			if (i < q.n) {
-				q.values[i] = optimizer_element<T, RULE>(k, regularized_gradient(q.grad[i], q.values[i], q.l1, q.l2), q.values[i], q.s0, q.s1,
+				q.values[i] = optimizer_element<T, RULE>(k, regularized_gradient(whole_gradient(q, i), q.values[i], q.l1, q.l2), q.values[i], q.s0, q.s1,
 						q.s2, i);
 				q.grad[i] = (T) 0;
 			}
@@ -473,7 +487,7 @@ void optimizer_step_many_kernel(OptBatch<T> batch, OptCoef<T> k) {
 		const int row = k0 + a, f = f0 + b + 8 * j;
 		if (row < q.K && f < F) {
 			const size_t i = (size_t) row + (size_t) q.K * f;
-			const T v = optimizer_element<T, RULE>(k, regularized_gradient(q.grad[i], q.values[i], q.l1, q.l2), q.values[i], q.s0, q.s1,
+			const T v = optimizer_element<T, RULE>(k, regularized_gradient(whole_gradient(q, i), q.values[i], q.l1, q.l2), q.values[i], q.s0, q.s1,
 					q.s2, i);
 			q.values[i] = v;
 			q.grad[i] = (T) 0;

@@ -18,7 +18,20 @@ def pytest_terminal_summary(terminalreporter):
     import helpers
     if not helpers.ACHIEVED:
         return
-    terminalreporter.write_line("achieved max relative errors (label: floored | plain over |ref| > floor | elements)")
-    for label in sorted(helpers.ACHIEVED):
+    # the rows of the sweeps over fused-layer variants first, the BASELINE configurations and the batch-norm input gradients
+    # last: a reader who only keeps the end of the output keeps those
+    labels = sorted(helpers.ACHIEVED, key=lambda l: (not l.startswith("fused "), l))
+    lines = ["achieved max relative errors (label: floored | plain over |ref| > floor | elements)"]
+    for label in labels:
         e, plain, n = helpers.ACHIEVED[label]
-        terminalreporter.write_line("  %-60s %.3e | %.3e | %d" % (label, e, plain, n))
+        lines.append("  %-60s %.3e | %.3e | %d" % (label, e, plain, n))
+    for line in lines:
+        terminalreporter.write_line(line)
+    # the whole table as a file beside the run's other output
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, "parity_achieved.txt"), "w") as f:
+            f.write("\n".join(lines) + "\n")
+    except OSError:
+        pass
