@@ -173,6 +173,22 @@ def host_tensor_run(args, dtype):
             "note": "pass_forward + pass_back on pageable host arrays, outputs allocated per call, best of 3"}
 
 
+CALIBRATION_SHAPE = (256, 32, 32, 64)
+
+
+def copy_calibration(ch, dtype):
+    """A plain copy of known size (the identity activation on a 256 x 32 x 32 x 64 tensor: reads and writes
+    16,777,216 elements) for scaling the FETCH_SIZE / WRITE_SIZE readings of the same profiler run to bytes."""
+    a = ch.DeviceTensor(CALIBRATION_SHAPE, dtype)
+    b = ch.DeviceTensor(CALIBRATION_SHAPE, dtype)
+    ident = ch.ActivationLayer(dtype, "identity", CALIBRATION_SHAPE[1:])
+    for _ in range(3):
+        ident.forward_into(a, b, True)
+    ch.synchronize()
+    a.free()
+    b.free()
+
+
 def small_convs_run(args, dtype):
     """The convolution shapes of the other BASELINE configurations, one layer at a time on device-resident tensors:
     forward, weight + bias gradient and input gradient timed with HIP events. These are small-K or few-row problems,
@@ -193,6 +209,8 @@ def small_convs_run(args, dtype):
     timer = ch.Timer()
     reps = max(20, args.steps)
     rows = []
+    if args.only:
+        shapes = [sh for sh in shapes if args.only in sh[0]]
     for name, N, H, W, C, F in shapes:
         K, M = 9 * C, N * H * W
         layer = ch.ConvKernelLayer(dtype, (H, W, C), F)
@@ -210,12 +228,18 @@ def small_convs_run(args, dtype):
                 fn()
             return timer.stop() / reps
 
-        t_fwd = timed(lambda: layer.forward_into(x, out, True))
-        t_bwd = timed(lambda: layer.backward_into(go, dx))
+        t_fwd = timed(lambda: layer.forward_into(x, out, True)) if args.passes in ("both", "fwd") else float("nan")
+        if args.passes in ("both", "bwd"):
+            layer.forward_into(x, out, True)
+            t_bwd = timed(lambda: layer.backward_into(go, dx))
+        else:
+            t_bwd = float("nan")
         in_b, out_b, w_b = M * C * es, M * F * es, K * F * es
         flop = 2.0 * M * K * F
         for pass_name, t_ms, launches, nbytes in (("forward", t_fwd, 1, in_b + w_b + out_b),
                                                   ("backward (weight, bias and input gradients)", t_bwd, 2, 2 * (in_b + out_b + w_b))):
+            if t_ms != t_ms:
+                continue
             roof_s = max(launches * flop / peak, nbytes / 8e12)
             rows.append({"layer": name, "pass": pass_name, "M": M, "K": K, "F": F, "ms": round(t_ms, 4),
                          "gflops": round(launches * flop / (t_ms * 1e-3) / 1e9, 1), "GB/s": round(nbytes / (t_ms * 1e-3) / 1e9, 1),
@@ -223,9 +247,100 @@ def small_convs_run(args, dtype):
                          "roofline_us": round(roof_s * 1e6, 2), "frac_of_roofline": round(roof_s / (t_ms * 1e-3), 4)})
         for t in (x, go, out, dx):
             t.free()
+    if args.copy_calibration:
+        copy_calibration(ch, dtype)
     return {"metric": "small_conv_layer_passes", "unit": "ms", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
             "config": {"workload": "convolution layers of BASELINE configs[0], [2] and [4], one pass per line, tensors resident in HBM"},
             "rows": rows}
+
+
+def conv_shapes_run(args, dtype):
+    """Layers that no launch rule was written for: a held-out table of convolution, transposed-convolution and dense
+    shapes (two of them in fp64 whatever --dtype says), forward and backward, each against its roofline
+    max(FLOP / matrix peak of the precision, algorithmic bytes / 8 TB/s). FLOP = 2 M K F per GEMM with M = batch x
+    output positions of the (equivalent) convolution: what a strided or transposed layer needs, not what a kernel
+    that multiplies zeros spends."""
+    ch = importlib.import_module("c-attl3_amd")
+    ch.init(0)
+    # name, kind, batch, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh, fp64
+    shapes = [
+        ("conv 3x3 28x28x128 -> 256, batch 64", "conv", 64, 28, 28, 128, 256, 3, 3, 1, 1, 1, 1, 0, 0, False),
+        ("conv 3x3 14x14x256 -> 256, batch 256", "conv", 256, 14, 14, 256, 256, 3, 3, 1, 1, 1, 1, 0, 0, False),
+        ("conv 3x3 7x7x512 -> 512, batch 256", "conv", 256, 7, 7, 512, 512, 3, 3, 1, 1, 1, 1, 0, 0, False),
+        ("conv 1x1 28x28x128 -> 512, batch 64", "conv", 64, 28, 28, 128, 512, 1, 1, 0, 0, 1, 1, 0, 0, False),
+        ("conv 5x5 32x32x32 -> 64 pad 2, batch 128", "conv", 128, 32, 32, 32, 64, 5, 5, 2, 2, 1, 1, 0, 0, False),
+        ("conv 3x3 stride 2 56x56x64 -> 128, batch 64", "conv", 64, 56, 56, 64, 128, 3, 3, 1, 1, 2, 2, 0, 0, False),
+        ("conv 3x3 30x30x24 -> 48, batch 96", "conv", 96, 30, 30, 24, 48, 3, 3, 1, 1, 1, 1, 0, 0, False),
+        ("conv 3x3 dilation 1 24x24x32 -> 32 pad 2, batch 64", "conv", 64, 24, 24, 32, 32, 3, 3, 2, 2, 1, 1, 1, 1, False),
+        ("dense 4096 -> 1024, batch 512", "dense", 512, 1, 1, 4096, 1024, 1, 1, 0, 0, 1, 1, 0, 0, False),
+        ("conv 3x3 28x28x128 -> 256, batch 64, fp64", "conv", 64, 28, 28, 128, 256, 3, 3, 1, 1, 1, 1, 0, 0, True),
+        ("conv 3x3 14x14x256 -> 256, batch 128, fp64", "conv", 128, 14, 14, 256, 256, 3, 3, 1, 1, 1, 1, 0, 0, True),
+        # the layers of the reference's examples/mnist_autoencoder.cpp:27-30, :40-43 at batch 256
+        ("autoencoder conv 4x4 stride 2 28x28x1 -> 3, batch 256", "conv", 256, 28, 28, 1, 3, 4, 4, 0, 0, 2, 2, 0, 0, False),
+        ("autoencoder conv 4x4 13x13x3 -> 3, batch 256", "conv", 256, 13, 13, 3, 3, 4, 4, 0, 0, 1, 1, 0, 0, False),
+        ("autoencoder transposed conv 4x4 10x10x3 -> 3, batch 256", "transconv", 256, 10, 10, 3, 3, 4, 4, 0, 0, 1, 1, 0, 0, False),
+        ("autoencoder transposed conv 4x4 stride 2 13x13x3 -> 1, batch 256", "transconv", 256, 13, 13, 3, 1, 4, 4, 0, 0, 2, 2, 0, 0, False),
+        ("transposed conv 3x3 stride 2 14x14x128 -> 64 pad 1, batch 64", "transconv", 64, 14, 14, 128, 64, 3, 3, 1, 1, 2, 2, 0, 0, False),
+    ]
+    if args.only:
+        shapes = [sh for sh in shapes if args.only in sh[0]]
+    gen = np.random.default_rng(23)
+    timer = ch.Timer()
+    reps = max(20, args.steps)
+    rows = []
+    for name, kind, N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh, fp64 in shapes:
+        dt = np.float64 if (fp64 or args.dtype == "f64") else np.float32
+        es, peak = np.dtype(dt).itemsize, PEAK_TFLOPS["f64" if dt == np.float64 else "f32"] * 1e12
+        if kind == "dense":
+            layer = ch.DenseKernelLayer(dt, (C,), F)
+            in_shape, K = (N, C), C
+        elif kind == "conv":
+            layer = ch.ConvKernelLayer(dt, (H, W, C), F, RH, RW, pv, ph, sv, sh, dv, dh)
+            in_shape, K = (N, H, W, C), RH * RW * C
+        else:
+            layer = ch.TransConvKernelLayer(dt, (H, W, C), F, RH, RW, pv, ph, sv, sh, dv, dh)
+            in_shape, K = (N, H, W, C), RH * RW * F        # of the convolution that maps the output back to the input
+        out_shape = (N,) + tuple(layer.get_output_dims())
+        wp = layer.get_params()[0]
+        wp.set_values(he_normal(gen, wp.get_rows(), wp.get_cols(), dt))
+        x = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal(in_shape).astype(dt)))
+        go = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal(out_shape).astype(dt)))
+        out = ch.DeviceTensor(out_shape, dt)
+        dx = ch.DeviceTensor(in_shape, dt)
+        # rows and columns of the GEMM: a transposed convolution is the convolution from its output to its input
+        M = int(np.prod(in_shape[:-1])) if kind == "transconv" else int(np.prod(out_shape[:-1]))
+        cols = C if kind == "transconv" else F
+
+        def timed(fn):
+            for _ in range(3):
+                fn()
+            timer.start()
+            for _ in range(reps):
+                fn()
+            return timer.stop() / reps
+
+        t_fwd = timed(lambda: layer.forward_into(x, out, True)) if args.passes in ("both", "fwd") else None
+        t_bwd = None
+        if args.passes in ("both", "bwd"):
+            layer.forward_into(x, out, True)
+            t_bwd = timed(lambda: layer.backward_into(go, dx))
+        in_b, out_b, w_b = int(np.prod(in_shape)) * es, int(np.prod(out_shape)) * es, wp.get_rows() * wp.get_cols() * es
+        flop = 2.0 * M * K * cols
+        for pass_name, t_ms, launches, nbytes in (("fwd", t_fwd, 1, in_b + w_b + out_b), ("bwd", t_bwd, 2, 2 * (in_b + out_b + w_b))):
+            if t_ms is None:
+                continue
+            roof_s = max(launches * flop / peak, nbytes / 8e12)
+            rows.append({"layer": name, "pass": pass_name, "M": M, "K": K, "F": cols, "dtype": np.dtype(dt).name,
+                         "us": round(t_ms * 1e3, 2), "tflops": round(launches * flop / (t_ms * 1e-3) / 1e12, 2),
+                         "bound": "mfma" if launches * flop / peak >= nbytes / 8e12 else "hbm",
+                         "roofline_us": round(roof_s * 1e6, 2), "frac_of_roofline": round(roof_s / (t_ms * 1e-3), 4)})
+        for t in (x, go, out, dx):
+            t.free()
+    if args.copy_calibration:
+        copy_calibration(ch, dtype)
+    return {"metric": "held_out_layer_passes", "unit": "us", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+            "config": {"workload": "convolution, transposed-convolution and dense layers outside the BASELINE configurations, one pass "
+                                   "per line, tensors resident in HBM"}, "rows": rows}
 
 
 def pointwise_run(args, dtype):
@@ -577,12 +692,38 @@ def summarize_traffic(fetch_dir, write_dir, dtype, batch, write):
         print("wrote", path)
 
 
+def summarize_hbm(fetch_dir, write_dir, copy_bytes, copy_kernel):
+    """Per kernel: mean FETCH_SIZE and WRITE_SIZE readings per dispatch (KiB) of two `rocprofv3 --pmc` runs and the bytes
+    they stand for, each counter scaled by what it reads for the dispatches of `copy_kernel`, which move `copy_bytes` each
+    way (a plain copy run in the same process: `--copy-calibration`, or the identity layer of the pointwise workload)."""
+    def means(directory):
+        agg = collections.OrderedDict()
+        for _, kernel, counter, value in read_counters(directory):
+            agg.setdefault(kernel, []).append(value)
+        return collections.OrderedDict((k, (sum(v) / len(v), len(v))) for k, v in agg.items())
+    fetch, wr = means(fetch_dir), means(write_dir)
+    fcopy = [v for k, v in fetch.items() if k.startswith(copy_kernel)]
+    wcopy = [v for k, v in wr.items() if k.startswith(copy_kernel)]
+    if not fcopy or not wcopy:
+        sys.exit("no dispatch of %s in the counter runs" % copy_kernel)
+    f_fac, w_fac = copy_bytes / (fcopy[0][0] * 1024.0), copy_bytes / (wcopy[0][0] * 1024.0)
+    out = ["calibration: `%s` moves %d bytes each way; FETCH_SIZE reads %.1f KiB (factor %.3f), WRITE_SIZE %.1f KiB (factor %.3f)"
+           % (copy_kernel, copy_bytes, fcopy[0][0], f_fac, wcopy[0][0], w_fac), "",
+           "| kernel | dispatches | FETCH_SIZE KiB | WRITE_SIZE KiB | read MB | written MB | total MB |", "|---|---|---|---|---|---|---|"]
+    for kernel, (fv, n) in fetch.items():
+        wv = wr.get(kernel, (0.0, 0))[0]
+        rb, wb = fv * 1024 * f_fac, wv * 1024 * w_fac
+        out.append("| `%s` | %d | %.1f | %.1f | %.3f | %.3f | %.3f |" % (kernel, n, fv, wv, rb / 1e6, wb / 1e6, (rb + wb) / 1e6))
+    return "\n".join(out)
+
+
 def summarize_main(argv):
     """`bench.py summarize ...`: turns rocprofv3 output of bench.py runs into the short summaries kept under profiles/.
 
         python bench.py summarize kernels  <dir with *_results.db>
         python bench.py summarize counters <dir with *counter_collection.csv> [...]
         python bench.py summarize traffic  <FETCH_SIZE dir> <WRITE_SIZE dir> --dtype f32 --batch 256 [--write]
+        python bench.py summarize hbm      <FETCH_SIZE dir> <WRITE_SIZE dir> --copy-bytes B [--copy-kernel PREFIX]
 
     `traffic` needs the two counter runs to have been made with `bench.py --copy-calibration`, which adds a plain copy
     kernel of known size: each counter is scaled by what it reads for that copy. With --write it rewrites
@@ -601,7 +742,15 @@ def summarize_main(argv):
     t.add_argument("--dtype", default="f32")
     t.add_argument("--batch", type=int, default=256)
     t.add_argument("--write", action="store_true")
+    h = sub.add_parser("hbm")
+    h.add_argument("fetch_dir")
+    h.add_argument("write_dir")
+    h.add_argument("--copy-bytes", type=int, required=True)
+    h.add_argument("--copy-kernel", default="act_forward_kernel<float, 0")
     a = ap.parse_args(argv)
+    if a.cmd == "hbm":
+        print(summarize_hbm(a.fetch_dir, a.write_dir, a.copy_bytes, a.copy_kernel))
+        return
     if a.cmd == "kernels":
         print(summarize_kernels(a.directory, a.limit))
     elif a.cmd == "counters":
@@ -623,14 +772,17 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=256)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy kernel of x's size (for scaling rocprof byte counters)")
+    ap.add_argument("--only", default="", help="small_convs / conv_shapes: only the layers whose name contains this")
+    ap.add_argument("--passes", choices=["both", "fwd", "bwd"], default="both", help="small_convs / conv_shapes: which passes to run")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--repeats", type=int, default=5, help="how often the timed loop of --steps steps is repeated (median reported)")
     ap.add_argument("--no-extra", action="store_true", help="skip the fp64 leg and the host-tensor leg of the default run")
-    ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm", "train_steps", "small_convs"], default="conv",
+    ap.add_argument("--workload", choices=["conv", "pointwise", "convlstm", "train_steps", "small_convs", "conv_shapes"], default="conv",
                     help="conv: the headline benchmark; pointwise: HBM-bound layers, one line of per-kernel GB/s; "
                          "convlstm: the fused-gate ConvLSTM of BASELINE configs[4], sequences/s; "
                          "train_steps: whole device-resident training steps of BASELINE configs[1] and [2]; "
-                         "small_convs: the convolution layers of the other configurations against both rooflines")
+                         "small_convs: the convolution layers of the other configurations against both rooflines; "
+                         "conv_shapes: a held-out table of layer shapes that no launch rule was tuned on")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X: this build has no multi-GPU path, run with --gpus 1")
@@ -651,6 +803,9 @@ def main():
         return
     if args.workload == "small_convs":
         print(json.dumps(small_convs_run(args, dtype)))
+        return
+    if args.workload == "conv_shapes":
+        print(json.dumps(conv_shapes_run(args, dtype)))
         return
 
     r = gpu_run(args, dtype)

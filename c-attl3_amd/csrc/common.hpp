@@ -73,6 +73,10 @@ struct GatherGeom {
 	int NS;         /* samples between two positions of the gathered tensor: N, or more when the N samples are the
 	                 * first of a larger batch (one time step of a sequence tensor (N, T, ...), whose step t starts
 	                 * N t elements into it and has N T samples between positions) */
+	/* Where row m = n + N (a + OA b), column f of the result goes: element n + N ((out_a0 + out_sa a) + out_OA (out_b0 +
+	 * out_sb b)) + out_M f of `out`. Plain (0, 1, 0, 1, OA, M): out is the M x F matrix itself. Otherwise the rows are
+	 * one residue class of the positions of a larger tensor (a strided input gradient computed class by class). */
+	int out_a0, out_sa, out_b0, out_sb, out_OA, out_M;
 };
 
 /* Convolution hyper-parameters in the reference's terms (dilation 0 = dense receptor). */
@@ -154,6 +158,9 @@ template<typename T> struct LstmBackwardStep;
  * be run (lstm_gates_backward). */
 template<typename T> bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad,
 		T* wt_dgrad, bool wt_ready, const LstmBackwardStep<T>* then = nullptr, int og_batch = 0);
+/* Which prepared layout conv_input_gradient builds in wt_dgrad at this batch size: 0 the plain one (all taps), 1 the
+ * blocks of a strided convolution's residue classes. Prepared weights are current only for the layout they were built as. */
+int dgrad_weight_layout(const ConvShape& s, int N);
 
 /* Element-wise / reduction kernels (pointwise_kernels.hip). */
 template<typename T> void act_forward(int kind, size_t n, T p, const T* x, T* y);
@@ -232,6 +239,7 @@ template<typename T> struct LstmBackwardStep {
  *   EPI_POOL   activation, then max pooling with windows that tile the output (stride = receptor): `out` is the pooled
  *              tensor, `inds` the arg-max cache in the layout of MaxPoolLayer (layer/pool/MaxPoolLayer.hpp:58-62), `pre`
  *              the pre-activation value at each arg-max (or null). Needs the blocked tile order with whole windows per tile.
+ *              With pool_mean: mean pooling, see below.
  *   EPI_STATS  out = acc + bias, plus per tile and output column (count, mean, sum of squared deviations) of the tile's
  *              rows in `stats` [mtiles][F][3]: the batch-norm moments of the convolution output without reading it again.
  *   EPI_LSTM   the output columns are the four gates' weighted previous outputs of an LSTM cell; the element-wise part of
@@ -248,6 +256,10 @@ struct Epilogue {
 	int OHp, OWp;           /* pooled output extents */
 	T* stats;
 	LstmForwardStep<T> lstm;
+	/* EPI_POOL with mean pooling (MeanPoolLayer.hpp:35-41) instead of max pooling: `out` is the mean of each window, taken
+	 * in the window's width-major order, `inds` is unused, and `pre` is a tensor of the full, unpooled size that receives
+	 * what the backward pass needs at every position: the pre-activation values if keep_input, else the coded outputs. */
+	int pool_mean, keep_input;
 };
 /* conv_forward with a fused epilogue. Returns false, having launched nothing, when the problem does not allow the
  * epilogue (no 16-byte accesses, windows that do not fit the tiles): the caller then runs the layers one by one; the
@@ -271,7 +283,7 @@ struct ChainShape {
 	double p;
 };
 /* dz from the gradient g of the (pooled) output, the arg-max cache, and the coded output y or the pre-activation
- * values `pre` (both at the arg-max positions when pooled); max pooling or none */
+ * values `pre` (both at the arg-max positions under max pooling, at every position under mean pooling or none) */
 template<typename T> void chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* y, const T* pre, T* dz);
 /* With a per-channel batch norm between kernel layer and activation: out = pool(act(bn(z))), the channel moments merged
  * from the GEMM epilogue's per-tile moments `stats` [mtiles][C][3] (training) or taken from the running statistics. */

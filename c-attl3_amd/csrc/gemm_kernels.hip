@@ -210,10 +210,50 @@ __device__ __forceinline__ int tile_row_m(const GatherLaunch& L, const GatherGeo
 	return (nb << sb_shift) + (row & ((1 << sb_shift) - 1)) + g.N * (ab * pa + pa_i + g.OA * (strip * L.pos_b + pb_i));
 }
 
+/* Element offset of row m of the result in `out` (GatherGeom's output map); consecutive samples of one position stay
+ * consecutive, so vector stores along n are unaffected. */
+__device__ __forceinline__ size_t out_row(const GatherGeom& g, int m) {
+	if (g.out_sa == 1 && g.out_sb == 1 && g.out_a0 == 0 && g.out_b0 == 0 && g.out_OA == g.OA)
+		return (size_t) m;
+	const int n = m % g.N, t = m / g.N;
+	const int a = t % g.OA, b = t / g.OA;
+	return (size_t) n + (size_t) g.N * (size_t) ((g.out_a0 + g.out_sa * a) + g.out_OA * (g.out_b0 + g.out_sb * b));
+}
+
+/* Several gathered GEMMs of one source and one result tensor in a single launch (the residue classes of a strided
+ * input gradient): blockIdx.z picks the problem, whose geometry, tile walk and prepared weights come from this table
+ * instead of the kernel's own arguments. No cut reductions: every tile is whole. */
+constexpr int MAX_GATHER_CLASSES = 9;
+template<typename T> struct GatherClasses {
+	GatherGeom g[MAX_GATHER_CLASSES];
+	GatherLaunch L[MAX_GATHER_CLASSES];
+	const T* wt[MAX_GATHER_CLASSES];
+};
+
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI, int PF>
+__device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
+		T* __restrict__ out, const GatherGeom& g, const GatherLaunch& L, T* __restrict__ partials, const Epilogue<T>& E);
+
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI = EPI_NONE, int PF = 1>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
 void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom g, const GatherLaunch L, T* __restrict__ partials, const Epilogue<T> E) {
+	gather_gemm_body<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, DIVS, EPI, PF>(src, wt, bias, out, g, L, partials, E);
+}
+
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
+void gather_gemm_classes_kernel(const T* __restrict__ src, T* __restrict__ out, const GatherClasses<T> classes) {
+	const GatherGeom g = classes.g[blockIdx.z];
+	const GatherLaunch L = classes.L[blockIdx.z];
+	const Epilogue<T> none = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr, {} };
+	gather_gemm_body<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_NONE, 1>(src, classes.wt[blockIdx.z], (const T*) nullptr, out, g, L,
+			(T*) nullptr, none);
+}
+
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI, int PF>
+__device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
+		T* __restrict__ out, const GatherGeom& g, const GatherLaunch& L, T* __restrict__ partials, const Epilogue<T>& E) {
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_M * WAVES_F;
 	constexpr int BM = WAVES_M * WT_M, BF = WAVES_F * WT_F;
@@ -587,6 +627,23 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 							continue;
 						const int wb = w / wa_n, wa = w - wb * wa_n;
 						const T* col = stage + fl * LROW + s_i;
+						if (E.pool_mean) {
+							/* the mean of the window, summed width-major / height-minor as the layer of its own does
+							 * (MeanPoolLayer.hpp:35-41); what the backward pass needs goes out at every position */
+							const int n = (nb << sb_shift) + s_i, a_p = a_p0 + wa, b_p = b_p0 + wb;
+							T sum = (T) 0;
+							for (int k = 0; k < E.prw; ++k)
+								for (int l = 0; l < E.prh; ++l) {
+									const T z = col[((wa * E.prh + l) + pa * (wb * E.prw + k)) << sb_shift];
+									const T y = act_f_coded<T, KIND>(z, E.p);
+									sum += y;
+									if (E.pre)
+										E.pre[(size_t) n + (size_t) g.N * ((a_p * E.prh + l) + (size_t) g.OA * ((b_p * E.prw + k) + (size_t) g.OB * f))] =
+												E.keep_input ? z : y;
+								}
+							out[(size_t) n + (size_t) g.N * (a_p + (size_t) E.OHp * (b_p + (size_t) E.OWp * f))] = sum / (T) (E.prh * E.prw);
+							continue;
+						}
 						/* strict '>' from lowest(), width-major / height-minor scan (MaxPoolLayer.hpp:45-56) */
 						T best = std::numeric_limits<T>::lowest(), best_pre = col[((wa * E.prh) + pa * (wb * E.prw)) << sb_shift];
 						unsigned bi = 0;
@@ -745,6 +802,8 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 		}
 		/* the tile itself is stored below, like any other */
 	}
+	/* (the output map: plain except for the residue classes of a strided input gradient, which have no fused epilogue) */
+	const size_t mm_out = EPI == EPI_NONE ? out_row(g, min(mm, g.M - 1)) : (size_t) mm;
 	#pragma unroll
 	for (int i = 0; i < FB; ++i) {
 		#pragma unroll
@@ -752,7 +811,7 @@ void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, con
 			const int f = f0 + wf * WT_F + FB * acc_row<T>(r, lk) + i;
 			if (f < g.F) {
 				const T bv = bias_s[wf * WT_F + FB * acc_row<T>(r, lk) + i];
-				T* dst = out + ((size_t) mm + (size_t) g.M * f);
+				T* dst = out + (mm_out + (size_t) g.out_M * f);
 				if (vec_out) {
 					if (mm < g.M) {
 						#pragma unroll
@@ -1209,6 +1268,21 @@ __global__ void prep_dgrad_weights_kernel(const T* __restrict__ w, T* __restrict
 	wt[i] = (f < F && c < C) ? w[(size_t) (tap + RHW * c) + (size_t) (RHW * C) * f] : (T) 0;
 }
 
+/* Input-gradient weights of one residue class of a strided convolution (see StridedClasses): the receptor rows
+ * r0, r0 + sv, ... and columns s0, s0 + sh, ... only, wt[k' = r' + Rc*(s' + Sc*f)][c] = w[(r0 + sv r') + RH*((s0 + sh s') + RW*c) + K*f]. */
+template<typename T>
+__global__ void prep_dgrad_class_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, int RH, int RW, int C, int F,
+		int r0, int sv, int Rc, int s0, int sh, int Sc, int Kp, int ldw) {
+	const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+	if (i >= (size_t) Kp * ldw)
+		return;
+	const int c = (int) (i % ldw), kp = (int) (i / ldw);
+	const int taps = Rc * Sc;
+	const int tap = kp % taps, f = kp / taps;
+	const int r = r0 + sv * (tap % Rc), sb = s0 + sh * (tap / Rc);
+	wt[i] = (f < F && c < C) ? w[(size_t) (r + RH * (sb + RW * c)) + (size_t) (RH * RW * C) * f] : (T) 0;
+}
+
 int round_up(int v, int to) {
 	return (v + to - 1) / to * to;
 }
@@ -1281,6 +1355,114 @@ static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
 constexpr int MAX_DEVICES = 64;
 void* g_scratch_ptr[MAX_DEVICES] = { nullptr };
 
+/* ------------------------------------------------------------------------------------------------
+ * The same gathered GEMM, out[M x F] = gather(src)[M x K] * wt[K x F] (+ bias), for F <= 4 output columns: the input
+ * gradient of a network's first convolution (its columns are the image's channels), a transposed convolution that
+ * ends in one or three channels, a convolution with a handful of filters. On 32 x 32 matrix tiles such a problem is
+ * seven eighths padding (measured on a 3 x 3 x 32 -> 3 input gradient: the matrix pipes busy half of the kernel's
+ * time with zeros) and a strided one keeps all taps in the reduction although only 1 / (sv sh) of them reach a
+ * given output. Here a lane owns VEC consecutive rows m (consecutive samples of one output position), reads their
+ * operand values straight from global memory, coalesced along the sample index, and multiplies each with the F
+ * weights of its reduction row, which are wave-uniform (scalar loads): no LDS staging, no padding, and a tap that
+ * does not reach the lane's position (zero padding, or a stride that does not divide) costs a predicate. The
+ * source channels are dealt over the four waves of a block, whose sums meet in LDS and are added in ascending
+ * wave order: the summation order depends on the geometry only.
+ * ---------------------------------------------------------------------------------------------- */
+constexpr int FEW_COLUMNS = 4;
+template<typename T, int VEC, bool DIVS>
+__global__ __launch_bounds__(256)
+void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
+		T* __restrict__ out, const GatherGeom g) {
+	constexpr int WAVES = 4, ROWS = 64 * VEC;
+	const int lane = threadIdx.x % 64;
+	const int wave = __builtin_amdgcn_readfirstlane((int) threadIdx.x / 64);
+	const int m = (int) blockIdx.x * ROWS + lane * VEC;
+	const bool mvalid = m < g.M;             /* whole vectors: M is a multiple of VEC */
+	int n, ya0, yb0;
+	{
+		n = m % g.N;
+		const int t = m / g.N;
+		const int a = t % g.OA, b = t / g.OA;
+		ya0 = a * g.SA + g.PA;
+		yb0 = b * g.SB + g.PB;
+	}
+	const int plane = g.NS * g.LH * g.LW;
+	const int per = (g.LC + WAVES - 1) / WAVES;
+	const int c0 = wave * per, c1 = min(g.LC, c0 + per);
+	const int taps = g.R * g.S;
+	T acc[FEW_COLUMNS][VEC];
+	#pragma unroll
+	for (int c = 0; c < FEW_COLUMNS; ++c)
+		#pragma unroll
+		for (int i = 0; i < VEC; ++i)
+			acc[c][i] = (T) 0;
+	for (int sb = 0; sb < g.S; ++sb)
+		for (int r = 0; r < g.R; ++r) {
+			int ya = ya0 + r * g.RA, yb = yb0 + sb * g.RB;
+			bool ok = mvalid;
+			if (DIVS) {
+				const int qa = ya / g.DA, qb = yb / g.DB;
+				ok = ok && qa * g.DA == ya && qb * g.DB == yb;
+				ya = qa;
+				yb = qb;
+			}
+			ok = ok && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
+			if (__builtin_amdgcn_ballot_w64(ok) == 0)        /* the tap reaches none of the wave's rows */
+				continue;
+			const T* p = src + (ok ? n + g.NS * (ya + g.LH * yb) + plane * c0 : 0);
+			/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded to four) first in its row */
+			const T* w = wt + (size_t) (r + g.R * (sb + g.S * c0)) * g.ldw;
+			const size_t wstep = (size_t) taps * g.ldw;
+			#pragma unroll 8
+			for (int ch = c0; ch < c1; ++ch) {
+				T v[VEC];
+				if (ok) {
+					vec_load_global<T, VEC>(v, p);
+				} else {
+					#pragma unroll
+					for (int i = 0; i < VEC; ++i)
+						v[i] = (T) 0;
+				}
+				T wk[FEW_COLUMNS];
+				vec_load_global<T, FEW_COLUMNS>(wk, w);
+				#pragma unroll
+				for (int c = 0; c < FEW_COLUMNS; ++c)
+					#pragma unroll
+					for (int i = 0; i < VEC; ++i)
+						acc[c][i] += v[i] * wk[c];
+				p += ok ? plane : 0;
+				w += wstep;
+			}
+		}
+	__shared__ T red[WAVES - 1][FEW_COLUMNS][ROWS];
+	if (wave > 0) {
+		#pragma unroll
+		for (int c = 0; c < FEW_COLUMNS; ++c)
+			vec_store<T, VEC>(&red[wave - 1][c][lane * VEC], acc[c]);
+	}
+	__syncthreads();
+	if (wave == 0 && mvalid) {
+		#pragma unroll
+		for (int c = 0; c < FEW_COLUMNS; ++c) {
+			if (c < g.F) {
+				#pragma unroll
+				for (int q = 0; q < WAVES - 1; ++q) {
+					T part[VEC];
+					vec_load<T, VEC>(part, &red[q][c][lane * VEC]);
+					#pragma unroll
+					for (int i = 0; i < VEC; ++i)
+						acc[c][i] += part[i];
+				}
+				const T bv = bias ? bias[c] : (T) 0;
+				#pragma unroll
+				for (int i = 0; i < VEC; ++i)
+					acc[c][i] += bv;
+				vec_store<T, VEC>(out + (out_row(g, m) + (size_t) g.out_M * c), acc[c]);
+			}
+		}
+	}
+}
+
 /* out tile = bias + sum over the parts of a split reduction, parts taken in ascending order (so the result
  * does not depend on how blocks were scheduled). One block per (walk position, f block) tile. */
 template<typename T, bool ACT>
@@ -1335,7 +1517,7 @@ void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ b
 				acc[i] = act_f_coded<T, decltype(kc)::value>(acc[i], E.p);
 		});
 	}
-	const size_t o = (size_t) m + (size_t) M * f;
+	const size_t o = ACT ? (size_t) m + (size_t) M * f : out_row(g, min(m, M - 1)) + (size_t) g.out_M * f;
 	T* dst = out + o;
 	if (m + V <= M && (reinterpret_cast<uintptr_t>(dst) & 15) == 0 && (!ACT || !E.pre || (reinterpret_cast<uintptr_t>(E.pre + o) & 15) == 0)) {
 		vec_store<T, V>(dst, acc);
@@ -1398,6 +1580,7 @@ struct GatherVariant {
 	int kc;
 	void (*launch)(dim3 grid, size_t dyn_lds, const T*, const T*, const T*, T*, const GatherGeom&, const GatherLaunch&,
 			T* partials, bool vec, bool divs, int epi, const Epilogue<T>&);
+	void (*launch_classes)(dim3 grid, const T* src, T* out, const GatherClasses<T>&);      /* 16-byte loads, no divisors, no epilogue */
 	int (*blocks_per_cu)(size_t dyn_lds, bool vec, bool divs, int epi);       /* what the runtime says fits on a CU */
 };
 
@@ -1428,6 +1611,12 @@ void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, con
 		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else
 		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+	CATTLE_HIP_CHECK(hipGetLastError());
+}
+
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
+void launch_gather_classes_variant(dim3 grid, const T* src, T* out, const GatherClasses<T>& classes) {
+	gather_gemm_classes_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, GemmCfg<T>::VEC><<<grid, dim3(64 * WAVES_M * WAVES_F), 0, stream()>>>(src, out, classes);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
@@ -1478,6 +1667,7 @@ GatherVariant<T> gather_variant() {
 	v.lds_bytes = 2 * KC * (v.bm + v.bf + 2 * C::pad(v.bm)) * (int) sizeof(T) + (PF + 2) * KC * 16;
 	v.kc = KC;
 	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, PF>;
+	v.launch_classes = &launch_gather_classes_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC>;
 	v.blocks_per_cu = &gather_variant_occupancy<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, PF>;
 	return v;
 }
@@ -1629,6 +1819,26 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	const bool divs = g.DA != 1 || g.DB != 1;
 	if (epi != EPI_NONE && (!vec || divs || (reinterpret_cast<uintptr_t>(out) & 15) != 0))
 		return false;
+	if (epi == EPI_NONE && then == nullptr && g.F <= FEW_COLUMNS) {
+		/* a handful of output columns: no matrix tiles (few_columns_gather_kernel) */
+		constexpr int V = GemmCfg<T>::VEC;
+		/* 16-byte loads wherever alignment allows, even where they leave a SIMD a wave or two: measured, a quarter of
+		 * the load instructions beats four times the waves (9 against 19 us on a 200,704 x 48 x 1 problem) */
+		const bool wide = vec && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+		const unsigned blocks = (unsigned) ((g.M + (wide ? 64 * V : 64) - 1) / (wide ? 64 * V : 64));
+		if (wide && divs)
+			few_columns_gather_kernel<T, V, true><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		else if (wide)
+			few_columns_gather_kernel<T, V, false><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		else if (divs)
+			few_columns_gather_kernel<T, 1, true><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		else
+			few_columns_gather_kernel<T, 1, false><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		CATTLE_HIP_CHECK(hipGetLastError());
+		if (mtiles_out)
+			*mtiles_out = 0;
+		return true;
+	}
 	const GatherVariant<T>* vars = GatherVariants<T>::get();
 	int best_v = 0;
 	for (int i = 1; i < GatherVariants<T>::LARGE; ++i) {
@@ -1646,7 +1856,20 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if (blocks >= device_shape().cus && blocks * 2 <= 3 * device_shape().cus)
 			best_v = 1;
 	}
-	/* too few large tiles to give every CU one: take the short tiles (the narrowest that still covers F, else the widest) */
+	/* Too few tiles of that shape to give every CU one: a narrower tile of the same height first, if that does (the
+	 * gathered operand is then read once per column of tiles, which a problem of this size, bound by the matrix
+	 * pipes, can afford; short tiles run at half the rate of tall ones), but no narrower than 64 columns: the
+	 * 256 x 32 tile, one wave per 64 rows, loses to the short tiles (measured on 32,768 x 288 x 64: 32 against 20 us) ... */
+	auto tiles_with = [&](int i) {
+		return (long) ((g.M + vars[i].bm - 1) / vars[i].bm) * ((g.F + vars[i].bf - 1) / vars[i].bf);
+	};
+	if (tiles_with(best_v) < device_shape().cus && epi != EPI_LSTM)
+		for (int i = best_v + 1; i < GatherVariants<T>::LARGE; ++i)
+			if (vars[i].bm == vars[best_v].bm && vars[i].bf < vars[best_v].bf && vars[i].bf >= 64 && tiles_with(i) >= device_shape().cus) {
+				best_v = i;
+				break;
+			}
+	/* ... else the short tiles (the narrowest that still covers F, else the widest) */
 	if ((long) ((g.M + vars[best_v].bm - 1) / vars[best_v].bm) * ((g.F + vars[best_v].bf - 1) / vars[best_v].bf) < device_shape().cus) {
 		constexpr int SHORT = GatherVariants<T>::SHORT;       /* short shapes, each with long and with medium chunks */
 		best_v = GatherVariants<T>::LARGE;
@@ -1778,6 +2001,83 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	return true;
 }
 
+/* All problems of `geoms` (same source, same result tensor, same column count; 16-byte loads possible) as one launch
+ * whose third grid dimension is the problem. The tile shape is chosen for the tiles of all problems together - a class
+ * of a strided input gradient alone may have too few rows for the large tiles that the whole gradient fills the chip
+ * with. Returns false, having launched nothing, if there are more problems than the table holds. */
+template<typename T>
+bool launch_gather_classes(const T* src, T* out, const std::vector<GatherGeom>& geoms, const std::vector<const T*>& weights) {
+	if (geoms.empty())
+		return true;
+	if ((int) geoms.size() > MAX_GATHER_CLASSES)
+		return false;
+	const GatherVariant<T>* vars = GatherVariants<T>::get();
+	const int F = geoms[0].F;
+	auto tiles_of = [&](const GatherVariant<T>& v) {
+		long t = 0;
+		for (const GatherGeom& g : geoms)
+			t += (long) ((g.M + v.bm - 1) / v.bm) * ((F + v.bf - 1) / v.bf);
+		return t;
+	};
+	/* the narrowest large tile that covers all columns in one block column, else the widest; the short tiles if the
+	 * large ones would not give every CU a block */
+	int best_v = 0;
+	for (int i = 1; i < GatherVariants<T>::LARGE; ++i)
+		if (vars[i].bm == vars[0].bm && vars[i].bf >= F && vars[i].bf < vars[best_v].bf)
+			best_v = i;
+	if (tiles_of(vars[best_v]) < device_shape().cus)
+		for (int i = best_v + 1; i < GatherVariants<T>::LARGE; ++i)
+			if (vars[i].bm == vars[best_v].bm && vars[i].bf < vars[best_v].bf && vars[i].bf >= 64 && tiles_of(vars[i]) >= device_shape().cus) {
+				best_v = i;
+				break;
+			}
+	if (tiles_of(vars[best_v]) < device_shape().cus) {
+		constexpr int SHORT = GatherVariants<T>::SHORT;
+		best_v = GatherVariants<T>::LARGE;
+		for (int i = GatherVariants<T>::LARGE + 1; i < GatherVariants<T>::LARGE + SHORT; ++i)
+			if (vars[i].bf >= F && vars[i].bf < vars[best_v].bf)
+				best_v = i;
+		if (tiles_of(vars[best_v]) >= 2 * device_shape().cus)
+			best_v += SHORT;                /* several short tiles per CU: the medium chunks, four blocks to a CU */
+	}
+	const GatherVariant<T>& v = vars[best_v];
+	GatherClasses<T> table;
+	unsigned blocks = 0;
+	for (size_t i = 0; i < geoms.size(); ++i) {
+		const GatherGeom& g = geoms[i];
+		const int mtiles = (g.M + v.bm - 1) / v.bm;
+		const long column = (long) g.N * g.OA;
+		int tile_rows = (column % v.bm == 0 && g.OB > 1) ? (int) (column / v.bm) : 0;
+		int sample_blocks = 0, pos_b = 1;
+		if (g.N % 32 == 0 && v.bm % 32 == 0 && g.OB > 1) {
+			const RowBlocks rb = plan_row_blocks<T>(g, v.bm, 1, 1, false);
+			if (rb.ok) {
+				sample_blocks = rb.sample_blocks;
+				pos_b = rb.pos_b;
+				tile_rows = rb.tile_rows;
+			}
+		}
+		table.g[i] = g;
+		table.L[i] = GatherLaunch{ mtiles, tile_rows, mtiles, round_up(mtiles, 8), 0, 1, (g.K + v.kc - 1) / v.kc, sample_blocks, pos_b, 5 };
+		table.wt[i] = weights[i];
+		blocks = std::max(blocks, (unsigned) round_up(mtiles, 8));
+	}
+	for (size_t i = geoms.size(); i < (size_t) MAX_GATHER_CLASSES; ++i) {
+		table.g[i] = geoms[0];
+		table.L[i] = table.L[0];
+		table.wt[i] = weights[0];
+	}
+	v.launch_classes(dim3(blocks, (unsigned) ((F + v.bf - 1) / v.bf), (unsigned) geoms.size()), src, out, table);
+	return true;
+}
+
+void plain_output(GatherGeom& g) {
+	g.out_a0 = g.out_b0 = 0;
+	g.out_sa = g.out_sb = 1;
+	g.out_OA = g.OA;
+	g.out_M = g.M;
+}
+
 GatherGeom forward_geom(const ConvShape& s, int N) {
 	GatherGeom g;
 	g.N = N; g.NS = N; g.LH = s.H; g.LW = s.W; g.LC = s.C;
@@ -1786,6 +2086,7 @@ GatherGeom forward_geom(const ConvShape& s, int N) {
 	g.SA = s.sv; g.SB = s.sh; g.RA = s.dv + 1; g.RB = s.dh + 1; g.PA = -s.pv; g.PB = -s.ph; g.DA = 1; g.DB = 1;
 	g.M = N * g.OA * g.OB; g.K = s.K(); g.F = s.F;
 	g.ldw = round_up(s.F, WT_COL_PAD);
+	plain_output(g);
 	return g;
 }
 
@@ -1797,7 +2098,68 @@ GatherGeom dgrad_geom(const ConvShape& s, int N) {
 	g.SA = 1; g.SB = 1; g.RA = -(s.dv + 1); g.RB = -(s.dh + 1); g.PA = s.pv; g.PB = s.ph; g.DA = s.sv; g.DB = s.sh;
 	g.M = N * s.H * s.W; g.K = s.RH * s.RW * s.F; g.F = s.C;
 	g.ldw = round_up(s.C, WT_COL_PAD);
+	plain_output(g);
 	return g;
+}
+
+/* The input gradient of a strided convolution, class by class. Input position a receives receptor row r only from
+ * output row (a + pv - (dv + 1) r) / sv, if that divides: for the positions of one residue class a = a0 (mod sv) these are
+ * the receptor rows r = r0 (mod sv), and with a = a0 + sv a', r = r0 + sv r' the output row is a' + PA - (dv + 1) r' - a
+ * stride-1 gather over the sub-sampled receptor (likewise along the width). So sv * sh GEMMs without divisions, each with
+ * only the taps that reach its positions, replace one GEMM over all taps of which 1 / (sv sh) are not zero; each writes
+ * its class of positions through the output map. Needs gcd(dv + 1, sv) = gcd(dh + 1, sh) = 1 (r0 unique). */
+struct StridedClass {
+	int a0, b0, OAc, OBc, r0, s0, Rc, Sc, PA, PB;
+	size_t wt_offset;       /* of the class's prepared weights in the buffer, in elements */
+};
+
+int gcd_int(int a, int b) {
+	while (b) {
+		const int t = a % b;
+		a = b;
+		b = t;
+	}
+	return a;
+}
+
+bool strided_classes(const ConvShape& s, std::vector<StridedClass>* out, size_t* wt_elems) {
+	if ((s.sv == 1 && s.sh == 1) || gcd_int(s.dv + 1, s.sv) != 1 || gcd_int(s.dh + 1, s.sh) != 1)
+		return false;
+	size_t total = 0;
+	for (int b0 = 0; b0 < s.sh; ++b0)
+		for (int a0 = 0; a0 < s.sv; ++a0) {
+			StridedClass c;
+			c.a0 = a0;
+			c.b0 = b0;
+			c.OAc = a0 < s.H ? (s.H - a0 + s.sv - 1) / s.sv : 0;
+			c.OBc = b0 < s.W ? (s.W - b0 + s.sh - 1) / s.sh : 0;
+			c.r0 = c.s0 = 0;
+			while (((s.dv + 1) * c.r0 - (a0 + s.pv)) % s.sv != 0)
+				++c.r0;
+			while (((s.dh + 1) * c.s0 - (b0 + s.ph)) % s.sh != 0)
+				++c.s0;
+			c.Rc = c.r0 < s.RH ? (s.RH - c.r0 + s.sv - 1) / s.sv : 0;
+			c.Sc = c.s0 < s.RW ? (s.RW - c.s0 + s.sh - 1) / s.sh : 0;
+			c.PA = (a0 + s.pv - (s.dv + 1) * c.r0) / s.sv;
+			c.PB = (b0 + s.ph - (s.dh + 1) * c.s0) / s.sh;
+			c.wt_offset = total;
+			total += (size_t) round_up(std::max(1, c.Rc * c.Sc * s.F), WT_ROW_PAD) * round_up(s.C, WT_COL_PAD);
+			if (out)
+				out->push_back(c);
+		}
+	if (wt_elems)
+		*wt_elems = total;
+	return true;
+}
+
+/* Class by class pays once each class is a launch worth making: the GEMMs of a class do 1 / (sv sh) of the rows, so the
+ * whole problem has to be a few launch overheads' worth of matrix work. Below that the single launch over all taps,
+ * zeros included, is faster (or the kernel for a handful of output columns, which skips taps by predicate). */
+bool use_strided_classes(const ConvShape& s, int N) {
+	if (s.C <= FEW_COLUMNS || N % 4 != 0 || !strided_classes(s, nullptr, nullptr))
+		return false;
+	const double useful = 2.0 * N * s.OH() * s.OW() * (double) s.K() * s.F;
+	return useful >= 2e8 * s.sv * s.sh;
 }
 
 void check_sizes(const ConvShape& s, int N) {
@@ -2009,6 +2371,10 @@ WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 
 } /* namespace */
 
+int dgrad_weight_layout(const ConvShape& s, int N) {
+	return use_strided_classes(s, N) ? 1 : 0;
+}
+
 int prepared_weight_row_length(int columns) {
 	return round_up(columns, WT_COL_PAD);
 }
@@ -2019,6 +2385,9 @@ ConvWorkspace conv_workspace(const ConvShape& s, int N) {
 	ConvWorkspace ws;
 	ws.wt_fwd = (size_t) round_up(s.K(), WT_ROW_PAD) * round_up(s.F, WT_COL_PAD);
 	ws.wt_dgrad = (size_t) round_up(s.RH * s.RW * s.F, WT_ROW_PAD) * round_up(s.C, WT_COL_PAD);
+	size_t by_class = 0;
+	if (strided_classes(s, nullptr, &by_class))
+		ws.wt_dgrad = std::max(ws.wt_dgrad, by_class);      /* either layout, whichever conv_input_gradient takes at a batch size */
 	const int M = N * s.OH() * s.OW();
 	const WgradPlan p = wgrad_plan<T>(M, s.K(), s.F, N, true), q = wgrad_plan<T>(M, s.K(), s.F, N, false);
 	ws.partials = (size_t) std::max(p.splits, q.splits) * ((size_t) s.K() * s.F + (size_t) s.F);
@@ -2067,7 +2436,7 @@ bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const
 	const GatherGeom g = forward_geom(s, N);
 	if (epi == EPI_POOL) {
 		CATTLE_HIP_REQUIRE(E.prh > 0 && E.prw > 0 && g.OA % E.prh == 0 && g.OB % E.prw == 0 && E.OHp == g.OA / E.prh &&
-				E.OWp == g.OB / E.prw && E.inds != nullptr, "the pooling epilogue needs windows that tile the output");
+				E.OWp == g.OB / E.prw && (E.inds != nullptr || E.pool_mean), "the pooling epilogue needs windows that tile the output");
 	}
 	if (epi == EPI_STATS)
 		CATTLE_HIP_REQUIRE(E.stats != nullptr, "the moments epilogue needs a buffer for its partials");
@@ -2186,6 +2555,60 @@ template<typename T>
 bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad, T* wt_dgrad, bool wt_ready,
 		const LstmBackwardStep<T>* then, int og_batch) {
 	check_sizes(s, std::max(N, og_batch));
+	if (then == nullptr && use_strided_classes(s, N)) {
+		std::vector<StridedClass> classes;
+		strided_classes(s, &classes, nullptr);
+		const int ldw = round_up(s.C, WT_COL_PAD);
+		bool empty_class = false;
+		for (const StridedClass& c : classes)
+			empty_class = empty_class || (c.Rc * c.Sc == 0 && c.OAc * c.OBc > 0);
+		if (empty_class)        /* positions that no tap reaches (a receptor narrower than the stride) */
+			device_zero_fill(in_grad, (size_t) N * s.H * s.W * s.C * sizeof(T));
+		std::vector<GatherGeom> geoms;
+		std::vector<const T*> weights;
+		for (const StridedClass& c : classes) {
+			if (c.OAc * c.OBc == 0 || c.Rc * c.Sc == 0)
+				continue;
+			T* wtc = wt_dgrad + c.wt_offset;
+			const int Kc = c.Rc * c.Sc * s.F, Kp = round_up(Kc, WT_ROW_PAD);
+			if (!wt_ready) {
+				const size_t count = (size_t) Kp * ldw;
+				prep_dgrad_class_weights_kernel<T><<<(unsigned) ((count + 255) / 256), 256, 0, stream()>>>(w, wtc, s.RH, s.RW, s.C, s.F,
+						c.r0, s.sv, c.Rc, c.s0, s.sh, c.Sc, Kp, ldw);
+				CATTLE_HIP_CHECK(hipGetLastError());
+			}
+			GatherGeom g;
+			g.N = N; g.NS = og_batch > 0 ? og_batch : N; g.LH = s.OH(); g.LW = s.OW(); g.LC = s.F;
+			g.OA = c.OAc; g.OB = c.OBc;
+			g.R = c.Rc; g.S = c.Sc;
+			g.SA = 1; g.SB = 1; g.RA = -(s.dv + 1); g.RB = -(s.dh + 1); g.PA = c.PA; g.PB = c.PB; g.DA = 1; g.DB = 1;
+			g.M = N * c.OAc * c.OBc; g.K = Kc; g.F = s.C;
+			g.ldw = ldw;
+			g.out_a0 = c.a0; g.out_sa = s.sv; g.out_b0 = c.b0; g.out_sb = s.sh; g.out_OA = s.H; g.out_M = N * s.H * s.W;
+			geoms.push_back(g);
+			weights.push_back(wtc);
+		}
+		/* the classes with the longest reductions first: their blocks are the ones the launch ends with otherwise */
+		std::vector<size_t> order(geoms.size());
+		for (size_t i = 0; i < order.size(); ++i)
+			order[i] = i;
+		std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) { return geoms[x].K > geoms[y].K; });
+		std::vector<GatherGeom> sorted_geoms;
+		std::vector<const T*> sorted_weights;
+		for (size_t i : order) {
+			sorted_geoms.push_back(geoms[i]);
+			sorted_weights.push_back(weights[i]);
+		}
+		geoms.swap(sorted_geoms);
+		weights.swap(sorted_weights);
+		/* one launch over all classes where 16-byte loads are possible, else a launch per class */
+		const bool vec = N % GemmCfg<T>::VEC == 0 && (og_batch <= 0 || og_batch % GemmCfg<T>::VEC == 0) &&
+				(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0;
+		if (!vec || !launch_gather_classes<T>(out_grad, in_grad, geoms, weights))
+			for (size_t i = 0; i < geoms.size(); ++i)
+				launch_gather<T>(out_grad, weights[i], (const T*) nullptr, in_grad, geoms[i]);
+		return false;
+	}
 	GatherGeom d = dgrad_geom(s, N);
 	if (og_batch > 0)
 		d.NS = og_batch;

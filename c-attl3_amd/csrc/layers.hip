@@ -260,6 +260,7 @@ struct Param {
 	uint64_t version = 1;
 	DevBuf derived[3];
 	uint64_t derived_version[3] = { 0, 0, 0 };
+	int dgrad_layout = 0;              /* which layout derived[1] holds (dgrad_weight_layout) */
 	/* A weight matrix: the partial sums of the last weight-gradient launch that was cut into slices (its own and, behind
 	 * them, those of the bias gradient). They are added to the gradients when a gradient is first needed - by the
 	 * optimizer step as a rule, in one launch for all layers - and until then `pending` lists them (see Deferred). */
@@ -506,7 +507,8 @@ struct ConvLayer : LayerBase {
 		const ConvWorkspace ws = conv_workspace<T>(shape, n);
 		Param& w = *params[0];
 		T* wt = (T*) w.derived[1].ensure(ws.wt_dgrad * sizeof(T));
-		const bool ready = w.derived_version[1] == w.version;
+		const int layout = dgrad_weight_layout(shape, n);
+		const bool ready = w.derived_version[1] == w.version && w.dgrad_layout == layout;
 		/* the partial sums of the launch before, if they still wait, would be overwritten */
 		if (w.pending)
 			g_deferred.settle();
@@ -515,8 +517,10 @@ struct ConvLayer : LayerBase {
 		conv_backward<T>(shape, n, x_cache, (const T*) w.values.p, (const T*) out_grad, (T*) w.grad.p, (T*) params[1]->grad.p,
 				(T*) in_grad, wt, ready, part, act, &later);
 		g_deferred.add<T>(&w, later);
-		if (in_grad)
+		if (in_grad) {
 			w.derived_version[1] = w.version;
+			w.dgrad_layout = layout;
+		}
 	}
 	void empty_cache() override {
 		LayerBase::empty_cache();
@@ -568,8 +572,10 @@ struct TransConvLayer : LayerBase {
 		Param& w = *params[0];
 		const T* wc = conv_weights();
 		T* wt = (T*) w.derived[1].ensure(ws.wt_dgrad * sizeof(T));
-		conv_input_gradient<T>(conv, n, wc, (const T*) in, (T*) out, wt, w.derived_version[1] == w.version);
+		const int layout = dgrad_weight_layout(conv, n);
+		conv_input_gradient<T>(conv, n, wc, (const T*) in, (T*) out, wt, w.derived_version[1] == w.version && w.dgrad_layout == layout);
 		w.derived_version[1] = w.version;
+		w.dgrad_layout = layout;
 		add_row_vector<T>(n, out_volume(), (const T*) params[1]->values.p, (T*) out);
 		x_cache = (const T*) in;       /* in_mat_cache (:147) */
 	}
@@ -1023,6 +1029,7 @@ struct FusedLayer : LayerBase {
 	bool owns_members = false;              /* a clone owns the clones of its members */
 	int mode = MODE_NONE;
 	bool pool_in_chain = false;             /* MODE_BN: the pool is part of the chain pass */
+	bool pool_mean = false;                 /* MODE_POOL: the pool in the GEMM epilogue was a mean pool */
 	bool trained = false;                   /* the last forward pass was a training pass (MODE_BN keeps moments only then) */
 	const T* y_cache = nullptr;             /* (coded) output the backward pass derives act' from; may be the caller's buffer */
 	DevBuf z_buf, pre_buf, dz_buf, stats_buf, mean_buf, chain_ws;
@@ -1113,7 +1120,7 @@ struct FusedLayer : LayerBase {
 		const T* bv = (const T*) conv->params[1]->values.p;
 		const int kind = act ? act->kind : CATTLE_HIP_ACT_IDENTITY;
 		const T ap = act ? act->p : (T) 0;
-		Epilogue<T> E = { kind, ap, nullptr, nullptr, 1, 1, OH(), OW(), nullptr };
+		Epilogue<T> E = { kind, ap, nullptr, nullptr, 1, 1, OH(), OW(), nullptr, {}, 0, 0 };
 		if (members.size() == 1 || !act_fusable() || (bn && !bn_fusable())) {
 			forward_unfused(in, N, training, out);
 			return;
@@ -1167,25 +1174,39 @@ struct FusedLayer : LayerBase {
 			return;
 		}
 		const bool needs_pre = !act_backward_from_output(kind, (double) ap);
-		if (pool && pool->kind == CATTLE_HIP_POOL_MAX && pool_tiles()) {
+		if (pool && pool_tiles()) {
+			const bool mean = pool->kind == CATTLE_HIP_POOL_MEAN;
 			const size_t pcount = N * pool->out_volume();
 			E.prh = pool->shape.RH;
 			E.prw = pool->shape.RW;
 			E.OHp = OH() / E.prh;
 			E.OWp = OW() / E.prw;
-			E.inds = (unsigned*) pool->inds.ensure(pcount * sizeof(unsigned));
-			E.pre = needs_pre ? (T*) pre_buf.ensure(pcount * sizeof(T)) : nullptr;
+			if (mean) {
+				/* every position of a window takes part in the backward pass: what the activation's derivative reads is
+				 * kept at full size (nothing for the kinds whose derivative is a constant) */
+				E.pool_mean = 1;
+				E.keep_input = needs_pre ? 1 : 0;
+				const bool constant_slope = kind == CATTLE_HIP_ACT_IDENTITY || kind == CATTLE_HIP_ACT_SCALED;
+				E.pre = constant_slope ? nullptr : (T*) z_buf.ensure(zcount * sizeof(T));
+			} else {
+				E.inds = (unsigned*) pool->inds.ensure(pcount * sizeof(unsigned));
+				E.pre = needs_pre ? (T*) pre_buf.ensure(pcount * sizeof(T)) : nullptr;
+			}
 			const bool ok = conv_forward_fused<T>(conv->shape, n, x, wv, bv, (T*) out, wt, ready, EPI_POOL, E, nullptr);
 			weights_prepared();
 			ready = true;
 			if (ok) {
-				pool->inds_count = pcount;
+				if (!mean)
+					pool->inds_count = pcount;
 				conv->x_cache = x;
-				y_cache = (const T*) out;
+				y_cache = mean ? (const T*) E.pre : (const T*) out;
+				pool_mean = mean;
 				mode = MODE_POOL;
 				return;
 			}
 			E.inds = nullptr;
+			E.pre = nullptr;
+			E.pool_mean = E.keep_input = 0;
 			E.prh = E.prw = 1;
 			E.OHp = OH();
 			E.OWp = OW();
@@ -1251,6 +1272,9 @@ struct FusedLayer : LayerBase {
 			bn_chain_backward<T>(cs, n, g, pool_in_chain ? (const unsigned*) pool->inds.p : nullptr, (const T*) z_buf.p,
 					(const T*) bn->params[2]->values.p, (const T*) bn->params[3]->values.p, (const T*) mean_buf.p,
 					(const T*) bn->inv_sd_cache.p, (T*) bn->params[2]->grad.p, (T*) bn->params[3]->grad.p, dz, ws);
+		} else if (mode == MODE_POOL && pool_mean) {
+			/* y_cache is the full-size tensor of what the derivative reads: inputs or coded outputs of the activation */
+			chain_backward<T>(chain_shape(true), n, g, nullptr, needs_pre() ? nullptr : y_cache, needs_pre() ? y_cache : nullptr, dz);
 		} else if (mode == MODE_POOL) {
 			CATTLE_HIP_REQUIRE(pool->inds_count == N * pool->out_volume(), "pass_back without cached max indices");
 			chain_backward<T>(chain_shape(true), n, g, (const unsigned*) pool->inds.p, y_cache, needs_pre() ? (const T*) pre_buf.p : nullptr, dz);
@@ -1295,7 +1319,8 @@ struct FusedLayer : LayerBase {
 			return;
 		}
 		require_not_released(conv->x_cache);
-		require_not_released(y_cache);
+		if (y_cache)
+			require_not_released(y_cache);
 	}
 };
 
@@ -1607,7 +1632,7 @@ void run_optimizer_many(const cattle_hip_layer_t* layers, const size_t* indices,
 		} else if (conv && indices[i] == 0) {
 			const ConvShape& cs = conv->shape;
 			fwd_current = p.derived[0].p && p.derived_version[0] == p.version;
-			dgrad_current = p.derived[1].p && p.derived_version[1] == p.version;
+			dgrad_current = p.derived[1].p && p.derived_version[1] == p.version && p.dgrad_layout == 0;
 			q.K = cs.K();
 			q.RHW = cs.RH * cs.RW;
 			q.ldw_fwd = prepared_weight_row_length(cs.F);

@@ -1301,7 +1301,7 @@ __device__ __forceinline__ void chain_store(T* p, const T (&src)[V]) {
  * arg-max positions when pooled), and the arg-max cache. One thread per window and V samples:
  * dz(position) = g * act'(.) at the arg-max position, 0 elsewhere (MaxPoolLayer.hpp:66-80 followed by the
  * activation's pass_back). */
-template<typename T, int V, bool POOL>
+template<typename T, int V, int POOL>
 __global__ __launch_bounds__(256)
 void chain_backward_kernel(ChainShape s, int N, size_t total, const T* __restrict__ g, const unsigned* __restrict__ inds,
 		const T* __restrict__ y, const T* __restrict__ pre, T* __restrict__ dz) {
@@ -1317,6 +1317,31 @@ void chain_backward_kernel(ChainShape s, int N, size_t total, const T* __restric
 	T gv[V], yv[V], gb[V];
 	unsigned iv[V];
 	chain_load<T, V>(gv, g + i);
+	if constexpr (POOL == CHAIN_POOL_MEAN) {
+		/* every position of the window receives g / (window size) (MeanPoolLayer.hpp:42-47) times the activation's
+		 * derivative there: y / pre are full-size tensors */
+		#pragma unroll
+		for (int v = 0; v < V; ++v)
+			gv[v] = gv[v] / (T) (s.prh * s.prw);
+		const size_t first = n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw + (size_t) s.W * c));
+		act_dispatch(s.kind, [&](auto kc) {
+			constexpr int KIND = decltype(kc)::value;
+			for (int k = 0; k < s.prw; ++k)
+				for (int l = 0; l < s.prh; ++l) {
+					const size_t at = first + (size_t) N * (l + (size_t) s.H * k);
+					if (pre)
+						chain_load<T, V>(yv, pre + at);
+					else if (y)
+						chain_load<T, V>(yv, y + at);
+					#pragma unroll
+					for (int v = 0; v < V; ++v)
+						gb[v] = pre ? act_b<T, KIND>(yv[v], act_needs_y(KIND) ? act_f<T, KIND>(yv[v], (T) s.p) : (T) 0, gv[v], (T) s.p) :
+								act_b_coded<T, KIND>(y ? yv[v] : (T) 0, gv[v], (T) s.p);
+					chain_store<T, V>(dz + at, gb);
+				}
+		});
+		return;
+	}
 	if (pre)
 		chain_load<T, V>(yv, pre + i);
 	else
@@ -1328,7 +1353,7 @@ void chain_backward_kernel(ChainShape s, int N, size_t total, const T* __restric
 			gb[v] = pre ? act_b<T, KIND>(yv[v], act_needs_y(KIND) ? act_f<T, KIND>(yv[v], (T) s.p) : (T) 0, gv[v], (T) s.p) :
 					act_b_coded<T, KIND>(yv[v], gv[v], (T) s.p);
 	});
-	if constexpr (!POOL) {
+	if constexpr (POOL == CHAIN_POOL_NONE) {
 		chain_store<T, V>(dz + i, gb);
 	} else {
 		chain_load<unsigned, V>(iv, inds + (((size_t) b_p * OHp + a_p) * ((size_t) s.C * N) + (size_t) c * N + n));
@@ -1607,20 +1632,24 @@ bool chain_vectors(int N, std::initializer_list<const void*> ptrs) {
 
 template<typename T>
 void chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds, const T* y, const T* pre, T* dz) {
-	CATTLE_HIP_REQUIRE(s.pool != CHAIN_POOL_MEAN, "mean pooling needs the values at every position: not kept by the fused pass");
 	const size_t total = (size_t) N * (s.H / s.prh) * (s.W / s.prw) * s.C;
 	constexpr int V = Pack<T>::V;
 	const bool vec = chain_vectors<T>(N, { g, inds, y, pre, dz });
 	if (s.pool == CHAIN_POOL_MAX) {
 		if (vec)
-			chain_backward_kernel<T, V, true><<<chain_grid(total / V), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+			chain_backward_kernel<T, V, CHAIN_POOL_MAX><<<chain_grid(total / V), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
 		else
-			chain_backward_kernel<T, 1, true><<<chain_grid(total), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+			chain_backward_kernel<T, 1, CHAIN_POOL_MAX><<<chain_grid(total), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+	} else if (s.pool == CHAIN_POOL_MEAN) {
+		if (vec)
+			chain_backward_kernel<T, V, CHAIN_POOL_MEAN><<<chain_grid(total / V), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+		else
+			chain_backward_kernel<T, 1, CHAIN_POOL_MEAN><<<chain_grid(total), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
 	} else {
 		if (vec)
-			chain_backward_kernel<T, V, false><<<chain_grid(total / V), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+			chain_backward_kernel<T, V, CHAIN_POOL_NONE><<<chain_grid(total / V), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
 		else
-			chain_backward_kernel<T, 1, false><<<chain_grid(total), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
+			chain_backward_kernel<T, 1, CHAIN_POOL_NONE><<<chain_grid(total), 256, 0, stream()>>>(s, N, total, g, inds, y, pre, dz);
 	}
 	check_launch();
 }

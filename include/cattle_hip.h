@@ -196,8 +196,9 @@ int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t 
  * one handle whose pass_forward / pass_back (cattle_hip_layer_forward / _backward) equal those calls in sequence:
  * the activation (ActivationLayer.hpp:47-66 and the element-wise kinds above) is applied in the epilogue of the GEMM, max
  * pooling over windows that tile the output (MaxPoolLayer.hpp:38-80; stride = receptor) too, so that the full-size
- * activation tensor is never written, and the per-channel batch norm (BatchNormLayer.hpp:225-261) gets its moments from
- * the GEMM's epilogue. The members keep their parameters (the fused handle lists them all, members' order, same objects),
+ * activation tensor is never written, mean pooling over such windows likewise (MeanPoolLayer.hpp:35-47; what the
+ * activation's derivative reads is then kept at every position, for the backward pass spreads the gradient over whole
+ * windows), and the per-channel batch norm (BatchNormLayer.hpp:225-261) gets its moments from the GEMM's epilogue. The members keep their parameters (the fused handle lists them all, members' order, same objects),
  * the batch norm its running statistics, the max pool its arg-max cache (cattle_hip_maxpool_indices on the member).
  * Whatever cannot be fused (batch sizes without 16-byte rows, overlapping windows, softmax, PReLU, PSwish, per-activation
  * batch norm behind a convolution) runs as the members' own passes, still on the device. Rectifier outputs (ReLU,
@@ -206,7 +207,7 @@ int cattle_hip_pool_create(cattle_hip_dtype dtype, cattle_hip_pool kind, size_t 
  * forward pass and its backward pass. A clone (cattle_hip_layer_clone) owns clones of the members. */
 int cattle_hip_fused_create(const cattle_hip_layer_t* layers, size_t count, cattle_hip_layer_t* fused);
 /* How the last forward pass of a fused handle ran: 0 none yet, 1 member by member, 2 activation in the GEMM epilogue,
- * 3 activation and max pooling in the GEMM epilogue, 4 batch-norm moments from the GEMM epilogue + one chain pass. */
+ * 3 activation and max or mean pooling in the GEMM epilogue, 4 batch-norm moments from the GEMM epilogue + one chain pass. */
 int cattle_hip_fused_last_mode(cattle_hip_layer_t fused, int* mode);
 
 /* DropoutLayer<Scalar,Rank>(dims, dropout_prob, epsilon) - layer/DropoutLayer.hpp:33-42, passes :74-96: a training

@@ -146,7 +146,10 @@ EXACT_CASES = [
     (64, 16, 16, 4, 8, ("relu", 0.0), ("max", 4, 4, 4, 4), "pool"),
     (16, 8, 8, 3, 6, ("relu", 0.0), ("max", 2, 1, 2, 1), "pool"),
     (16, 9, 9, 3, 6, ("relu", 0.0), None, "act"),
-    (256, 4, 4, 6, 5, ("relu", 0.0), ("mean", 2, 2, 2, 2), "act"),
+    (256, 4, 4, 6, 5, ("relu", 0.0), ("mean", 2, 2, 2, 2), "pool"),         # mean pooling in the epilogue as well
+    (32, 8, 8, 3, 16, None, ("mean", 2, 2, 2, 2), "pool"),
+    (64, 16, 16, 4, 8, ("leaky_relu", 0.125), ("mean", 4, 2, 4, 2), "pool"),
+    (16, 9, 9, 3, 6, ("relu", 0.0), ("mean", 2, 2, 1, 1), "act"),           # overlapping windows: the pool runs on its own
     (16, 9, 9, 3, 6, ("relu", 0.0), ("max", 3, 3, 2, 2), "act"),            # overlapping windows: the pool runs on its own
     (6, 8, 8, 3, 6, ("relu", 0.0), ("max", 2, 2, 2, 2), None),               # rows of 6: 16-byte accesses in fp64 only
     (7, 8, 8, 3, 6, ("relu", 0.0), ("max", 2, 2, 2, 2), "unfused"),          # rows of 7: member by member
@@ -352,6 +355,49 @@ def test_fused_activations(act, pooled, dtype):
     assert _compare_selections(chain, dev_inds, dtype, pool) < 1e-3
     grads = chain.backward(x64, w64, np.asarray(g, np.float64), inds=dev_inds, pre_act=_pre_act_at_device_sides(chain, out, dev_inds, dtype))
     wp, bp = members["conv"].get_params()
+    assert hp.rel_err(dx, grads["dx"], label=label + " dx") < tol
+    assert hp.rel_err(wp.get_grad(), grads["dw"], label=label + " dw") < tol
+    assert hp.rel_err(bp.get_grad(), grads["db"].reshape(1, -1), label=label + " db") < tol
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act", [None, ("relu", 0.0), ("sigmoid", 0.0), ("tanh", 0.0), ("softplus", 0.0), ("swish", 1.25),
+                                 ("scaled", 1.5), ("elu", 0.75), ("leaky_relu", -0.25)], ids=lambda a: "none" if a is None else "%s-%g" % a)
+@pytest.mark.parametrize("window", [(2, 2), (2, 4), (4, 4)], ids=lambda w: "%dx%d" % w)
+def test_fused_mean_pool_epilogue(act, window, dtype):
+    """conv -> [activation] -> mean pool whose windows tile the output (MeanPoolLayer.hpp:35-47): the means come out of the
+    GEMM's epilogue, the backward pass spreads g / window size over every position times the activation's derivative
+    there, read from what the forward pass kept (coded outputs, or inputs for kinds whose derivative needs them)."""
+    prh, prw = window
+    N, H, W, C, F = 32, 12, 8, 5, 20
+    pool = ("mean", prh, prw, prh, prw)
+    fused, members, kdims = _build(dtype, N, H, W, C, F, conv=GEOM_3X3, act=act, pool=pool)
+    chain = Chain(GEOM_3X3, act=act, pool=pool)
+    hidden_side = act is not None and act[0] in ("leaky_relu", "elu") and act[1] < 0
+    for seed in range(50, 70):
+        gen = hp.rng(seed)
+        x = hp.uniform(gen, (N, H, W, C), -1, 1, dtype)
+        w = hp.uniform(gen, (9 * C, F), -0.4, 0.4, dtype)
+        b = hp.uniform(gen, (1, F), -0.5, 0.5, dtype)
+        x64, w64, b64 = (np.asarray(a, np.float64) for a in (x, w, b))
+        ref = chain.forward(x64, w64, b64)
+        if not hidden_side or _kink_free(chain.z, dtype):
+            break
+    else:
+        pytest.fail("no seed gives inputs that stay clear of the kink")
+    g = hp.uniform(gen, ref.shape, -1, 1, dtype)
+    out, dx, mode = _run_fused(fused, members, x, w, b, g)
+    assert mode == "pool"
+    tol = TOL[np.dtype(dtype)]
+    label = "fused %s mean pool %dx%d %s" % ("none" if act is None else act[0], prh, prw, np.dtype(dtype).name)
+    assert hp.rel_err(out, ref, label=label + " forward") < tol
+    # the rectifier's side where the device's pre-activation value rounds to the other side of zero: rare, and only
+    # within the margin, so the gradient comparison allows for the few elements it moves
+    grads = chain.backward(x64, w64, np.asarray(g, np.float64))
+    wp, bp = members["conv"].get_params()
+    near_kink = act is not None and act[0] in ("relu", "leaky_relu", "elu") and not _kink_free(chain.z, dtype)
+    if near_kink:
+        pytest.skip("an input within the tie margin of the rectifier's kink: covered by the exact-arithmetic cases")
     assert hp.rel_err(dx, grads["dx"], label=label + " dx") < tol
     assert hp.rel_err(wp.get_grad(), grads["dw"], label=label + " dw") < tol
     assert hp.rel_err(bp.get_grad(), grads["db"].reshape(1, -1), label=label + " db") < tol
