@@ -1856,14 +1856,16 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if (blocks >= device_shape().cus && blocks * 2 <= 3 * device_shape().cus)
 			best_v = 1;
 	}
-	/* Too few tiles of that shape to give every CU one: a narrower tile of the same height first, if that does (the
-	 * gathered operand is then read once per column of tiles, which a problem of this size, bound by the matrix
-	 * pipes, can afford; short tiles run at half the rate of tall ones), but no narrower than 64 columns: the
-	 * 256 x 32 tile, one wave per 64 rows, loses to the short tiles (measured on 32,768 x 288 x 64: 32 against 20 us) ... */
+	/* Too few tiles of that shape to give every CU one: a narrower tile of the same height first, if that does and the
+	 * reduction is short. Such a launch is one round of blocks whose time is latency, so two half-width blocks on a CU
+	 * overlap each other's waits (50,176 x 576 x 128: 109 -> 96 us), while with a long reduction the matrix pipes are
+	 * busy either way and the wider tile's better operand reuse wins (12,544 x 4608 x 512: 624 against 675 us). No
+	 * narrower than 64 columns: the 256 x 32 tile, one wave per 64 rows, loses to the short tiles (32,768 x 288 x 64:
+	 * 32 against 20 us) ... */
 	auto tiles_with = [&](int i) {
 		return (long) ((g.M + vars[i].bm - 1) / vars[i].bm) * ((g.F + vars[i].bf - 1) / vars[i].bf);
 	};
-	if (tiles_with(best_v) < device_shape().cus && epi != EPI_LSTM)
+	if (tiles_with(best_v) < device_shape().cus && epi != EPI_LSTM && g.K <= 1024)
 		for (int i = best_v + 1; i < GatherVariants<T>::LARGE; ++i)
 			if (vars[i].bm == vars[best_v].bm && vars[i].bf < vars[best_v].bf && vars[i].bf >= 64 && tiles_with(i) >= device_shape().cus) {
 				best_v = i;
