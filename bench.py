@@ -394,6 +394,24 @@ def pointwise_run(args, dtype):
     bc = ch.BroadcastLayer(dtype, (H // 2, W // 2, C), (2, 2, 1))
     add("broadcast 2x2x1 forward (28x28x64 -> 56x56x64)", timed(lambda: bc.forward_into(yp, y, True)), es + es / 4.0)
     add("broadcast 2x2x1 backward", timed(lambda: bc.backward_into(g, yp)), es + es / 4.0)
+    # The passes of a fused layer that stream the activation tensor (they run between GEMM launches, so HIP events around a
+    # layer call cannot isolate them: their durations and HBM bytes are read from a kernel trace / counter run of this
+    # workload): a 1x1 convolution 8 -> 64 channels, so that the tensor behind it has the shape above, followed by
+    # batch norm + ReLU + 2x2 max pool (bn_chain_forward / bn_chain_sums / bn_chain_apply kernels), by ReLU + max pool
+    # and by sigmoid + mean pool (chain_backward kernels).
+    x8 = ch.DeviceTensor.from_host(np.asfortranarray(gen.standard_normal((N, H, W, 8)).astype(dtype)))
+    dx8 = ch.DeviceTensor((N, H, W, 8), dtype)
+    for members in ((ch.BatchNormLayer(dtype, (H, W, C)), ch.ActivationLayer(dtype, "relu", (H, W, C)), ch.MaxPoolLayer(dtype, (H, W, C))),
+                    (ch.ActivationLayer(dtype, "relu", (H, W, C)), ch.MaxPoolLayer(dtype, (H, W, C))),
+                    (ch.ActivationLayer(dtype, "sigmoid", (H, W, C)), ch.MeanPoolLayer(dtype, (H, W, C)))):
+        conv = ch.ConvKernelLayer(dtype, (H, W, 8), C, 1, 1, 0, 0)
+        conv.get_params()[0].set_values(he_normal(gen, 8, C, dtype))
+        fused = ch.FusedKernelLayer((conv,) + members)
+        for _ in range(reps + 1):
+            fused.forward_into(x8, yp, True)
+            fused.backward_into(gp, dx8)
+        ch.synchronize()
+        del fused
     return rows
 
 
@@ -646,7 +664,10 @@ def per_pass(rows, copy_kernel_prefix="act_forward_kernel"):
             current = PASSES[1]
             last = "wgrad"
             sums[current + " | kernel"].append(value)
-        elif kernel.startswith("split_reduce_kernel") or kernel.startswith("reduce_partials"):
+        elif kernel.startswith("reduce_partials"):
+            # the weight gradient's slices are summed when the gradient is next needed: by the backward pass after
+            sums[PASSES[1] + " | reduce"].append(value)
+        elif kernel.startswith("split_reduce_kernel"):
             if current is not None:
                 sums[current + " | reduce"].append(value)
         elif kernel.startswith(copy_kernel_prefix):
