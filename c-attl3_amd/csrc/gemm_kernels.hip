@@ -1463,6 +1463,161 @@ void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ 
 	}
 }
 
+/* ------------------------------------------------------------------------------------------------
+ * The same product for problems with far fewer output tiles than the chip has wavefront slots, as one launch without
+ * partial sums in memory: a block owns one TL x TL tile of the result (one matrix-instruction tile) and its WAVES
+ * wavefronts each take a contiguous share of the reduction; their partial tiles meet in LDS and are added in ascending
+ * wavefront order, then bias, activation (or the LSTM backward step that consumes the sums) and the store, one output
+ * element per thread. Operands go from global memory straight into the operand registers of the matrix instruction (a
+ * lane loads the one element per operand that the instruction wants from it: TL consecutive m, or TL consecutive
+ * columns of a prepared weight row, per reduction slot - whole 128-byte lines).
+ * The reduction runs tap by tap (receptor position), channels innermost, the KS reduction slots of an instruction being
+ * KS consecutive channels of one tap: a sum may be taken in any order, and in this one a lane's padding test and
+ * position are fixed for a whole tap and a step costs two offset additions, two selects, two loads and the matrix
+ * instruction - a wavefront issues one vector instruction per four cycles, and the address arithmetic of a gather by
+ * reduction index would outweigh the matrix instruction it feeds. Needs LC % KS == 0.
+ * grid = (M tiles rounded up to 8, F tiles).
+ * ---------------------------------------------------------------------------------------------- */
+enum { WS_PLAIN = 0, WS_ACT = 1, WS_LSTM_BACKWARD = 2 };
+
+template<typename T, int WAVES, bool DIVS, int TAIL>
+__global__ __launch_bounds__(64 * WAVES)
+void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias, T* __restrict__ out,
+		const GatherGeom g, int mtiles, const Epilogue<T> E, const LstmBackwardStep<T> then) {
+	typedef Mfma<T> MF;
+	constexpr int THREADS = 64 * WAVES;
+	constexpr int TL = MF::TL, KS = MF::KS;
+	constexpr int B = 16;                   /* reduction steps per batch of loads */
+	__shared__ T red[WAVES * TL * TL];
+
+	const int mtile = xcd_tile(blockIdx.x, mtiles);
+	if (mtile >= mtiles)
+		return;
+	const int tid = threadIdx.x;
+	const int lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+	const int lc = lane % TL, lk = lane / TL;
+	const int m0 = mtile * TL, f0 = (int) blockIdx.y * TL;
+	const int plane = g.NS * g.LH * g.LW;
+	const int m = m0 + lc;
+	const bool mvalid = m < g.M;
+	int n, ya0, yb0;
+	{
+		n = m % g.N;
+		const int t = m / g.N;
+		const int a = t % g.OA, b = t / g.OA;
+		ya0 = a * g.SA + g.PA;
+		yb0 = b * g.SB + g.PB;
+	}
+	/* this wavefront's steps of the reduction, numbered tap-major: step = tap * spt + channel group */
+	const int taps = g.R * g.S, spt = g.LC / KS;
+	const int total = taps * spt;
+	const int per = (total + WAVES - 1) / WAVES;
+	const int s_begin = wave * per, s_end = min(total, s_begin + per);
+	const unsigned astep = (unsigned) (plane * KS) * (unsigned) sizeof(T), bstep = (unsigned) (taps * KS * g.ldw) * (unsigned) sizeof(T);   /* bytes */
+
+	typename MF::acc_t acc[2];
+	#pragma unroll
+	for (int i = 0; i < 2; ++i)
+		#pragma unroll
+		for (int r = 0; r < MF::NACC; ++r)
+			acc[i][r] = (T) 0;
+
+	for (int s0 = s_begin; s0 < s_end;) {
+		const int tap = s0 / spt, cg0 = s0 - tap * spt;
+		const int count = min(spt - cg0, s_end - s0);        /* this wavefront's steps inside the tap */
+		const int r = tap % g.R, sb = tap / g.R;
+		int ya = ya0 + r * g.RA, yb = yb0 + sb * g.RB;
+		bool ok = mvalid;
+		if (DIVS) {
+			const int qa = ya / g.DA, qb = yb / g.DB;
+			ok = ok && qa * g.DA == ya && qb * g.DB == yb;
+			ya = qa;
+			yb = qb;
+		}
+		ok = ok && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
+		const int c_first = cg0 * KS + lk;
+		/* 32-bit byte offsets from the kernel's own pointers: a load then needs one address register, not two, and
+		 * sixteen steps' worth of loads fit beside the accumulators. Lanes in the padding read element 0 and drop it. */
+		unsigned aoff = ok ? (unsigned) (n + g.NS * (ya + g.LH * yb) + plane * c_first) * (unsigned) sizeof(T) : 0u;
+		const unsigned ainc = ok ? astep : 0u;
+		unsigned boff = (unsigned) ((tap + taps * c_first) * g.ldw + f0 + lc) * (unsigned) sizeof(T);
+		auto load_a = [&](unsigned off) {
+			return *(const __attribute__((address_space(1))) T*) (reinterpret_cast<const char*>(src) + (size_t) off);
+		};
+		auto load_b = [&](unsigned off) {
+			return *(const __attribute__((address_space(1))) T*) (reinterpret_cast<const char*>(wt) + (size_t) off);
+		};
+		/* Batches of B steps: all of a batch's loads are issued, then its matrix instructions run as the values arrive;
+		 * the other wavefronts of the SIMD cover the wait. (Loads of the next batch issued ahead of this one's matrix
+		 * instructions were tried: the values carried around the loop cost register copies that wait for every load.) */
+		int i = 0;
+		for (; i + B <= count; i += B) {
+			T xa[B], wb[B];
+			#pragma unroll
+			for (int u = 0; u < B; ++u) {
+				xa[u] = load_a(aoff + (unsigned) u * ainc);
+				wb[u] = load_b(boff + (unsigned) u * bstep);
+			}
+			aoff += B * ainc;
+			boff += B * bstep;
+			__builtin_amdgcn_sched_barrier(0);
+			#pragma unroll
+			for (int u = 0; u < B; ++u)
+				acc[u & 1] = MF::mma(wb[u], ok ? xa[u] : (T) 0, acc[u & 1]);
+			__builtin_amdgcn_sched_barrier(0);
+		}
+		if (i < count) {
+			/* the last, short batch: steps past the end read the last step's addresses again and drop the gathered value */
+			const int rem = count - i;
+			T xa[B], wb[B];
+			#pragma unroll
+			for (int u = 0; u < B; ++u) {
+				const unsigned uu = (unsigned) min(u, rem - 1);
+				xa[u] = load_a(aoff + uu * ainc);
+				wb[u] = load_b(boff + uu * bstep);
+			}
+			__builtin_amdgcn_sched_barrier(0);
+			#pragma unroll
+			for (int u = 0; u < B; ++u)
+				acc[u & 1] = MF::mma(wb[u], (ok && u < rem) ? xa[u] : (T) 0, acc[u & 1]);
+			__builtin_amdgcn_sched_barrier(0);
+		}
+		s0 += count;
+	}
+	#pragma unroll
+	for (int r = 0; r < MF::NACC; ++r)
+		red[(wave * TL + acc_row<T>(r, lk)) * TL + lc] = acc[0][r] + acc[1][r];
+	__syncthreads();
+	for (int o = tid; o < TL * TL; o += THREADS) {
+		T v = red[o];
+		#pragma unroll
+		for (int w = 1; w < WAVES; ++w)
+			v += red[w * TL * TL + o];
+		const int mo = m0 + o % TL, f = f0 + o / TL;
+		if (mo >= g.M || f >= g.F)
+			continue;
+		if constexpr (TAIL == WS_LSTM_BACKWARD) {
+			if (lstm_standard_acts(then.a))
+				lstm_backward_element<T, true>(then, (unsigned) mo + (unsigned) g.M * (unsigned) f, true, v);
+			else
+				lstm_backward_element<T, false>(then, (unsigned) mo + (unsigned) g.M * (unsigned) f, true, v);
+		} else {
+			v += bias ? bias[f] : (T) 0;
+			if constexpr (TAIL == WS_ACT) {
+				const size_t at = (size_t) mo + (size_t) g.M * f;
+				if (E.pre)
+					E.pre[at] = v;
+				act_dispatch(E.kind, [&](auto kc) {
+					v = act_f_coded<T, decltype(kc)::value>(v, E.p);
+				});
+				out[at] = v;
+			} else {
+				out[out_row(g, mo) + (size_t) g.out_M * f] = v;
+			}
+		}
+	}
+}
+
 /* out tile = bias + sum over the parts of a split reduction, parts taken in ascending order (so the result
  * does not depend on how blocks were scheduled). One block per (walk position, f block) tile. */
 template<typename T, bool ACT>
@@ -1717,7 +1872,7 @@ template<> struct GatherVariants<double> {
 struct Tuning {
 	struct PerF { int F, variant, occ; };
 	std::vector<PerF> per_f;
-	bool no_swizzle = false, no_row_blocks = false, no_split = false, wgrad_linear = false;
+	bool no_swizzle = false, no_row_blocks = false, no_split = false, wgrad_linear = false, no_wave_split = false;
 	int wgrad_variant = -1, wgrad_splits = 0, wgrad_min_chunks = 0;
 
 	Tuning() {
@@ -1725,6 +1880,7 @@ struct Tuning {
 		no_swizzle = std::getenv("CATTLE_HIP_NO_SWIZZLE") != nullptr;
 		no_row_blocks = std::getenv("CATTLE_HIP_NO_ROW_BLOCKS") != nullptr;
 		no_split = std::getenv("CATTLE_HIP_NO_SPLIT") != nullptr;
+		no_wave_split = std::getenv("CATTLE_HIP_NO_WAVE_SPLIT") != nullptr;
 		wgrad_linear = std::getenv("CATTLE_HIP_WGRAD_LINEAR") != nullptr;
 		const char* e = std::getenv("CATTLE_HIP_WGRAD_VARIANT");
 		wgrad_variant = e ? std::atoi(e) : -1;
@@ -1811,6 +1967,55 @@ RowBlocks plan_row_blocks(const GatherGeom& g, int bm, int prh, int prw, bool po
  * moments epilogue need whole tiles in one block (no cut reductions), the pooling epilogue the blocked tile order
  * with whole windows per tile. Returns false, without launching, when the problem does not allow that; `mtiles_out`
  * receives the number of M tiles (the row count of the moments epilogue's partials). */
+/* Whether, and with how many wavefronts per block, a problem runs as wave_split_gemm_kernel: few enough tiles of one
+ * matrix instruction that they and their wavefronts fit the chip at once (sixteen wavefronts per CU), a reduction long
+ * enough to deal out, and operand traffic (every tile reads its TL rows of both operands whole) that the L2 caches carry in
+ * a few microseconds. 0 = no. */
+template<typename T>
+int wave_split_waves(const GatherGeom& g) {
+	constexpr int TL = Mfma<T>::TL, KS = Mfma<T>::KS;
+	const long tiles = (long) ((g.M + TL - 1) / TL) * ((g.F + TL - 1) / TL);
+	const long slots = (long) device_shape().cus * 16;
+	if (g.LC % KS != 0 || g.LC < 4 * KS || tiles * 4 > slots)
+		return 0;
+	const int steps = g.K / KS;
+	if (steps < 32)
+		return 0;
+	if (((double) g.R * g.S * g.LC + 64) * g.ldw * sizeof(T) >= 4294967296.0 || (double) g.NS * g.LH * g.LW * g.LC * sizeof(T) >= 4294967296.0)
+		return 0;               /* 32-bit byte offsets */
+	int waves = 16;
+	while (waves > 4 && (tiles * waves > slots || steps < 8 * waves))
+		waves /= 2;
+	/* A wavefront's share of the reduction is a chain of batches of sixteen steps, each a round trip to memory of two
+	 * microseconds or more: three batches where the wavefronts are few (their round trips coincide), five where the chip
+	 * is full of them (blocks at different points of their chains overlap). Longer reductions are cut across blocks
+	 * (measured: a dense layer 4096 -> 10 at batch 128, four tiles, 23 us this way, 12 us cut across blocks). */
+	const int per_wave = (steps + waves - 1) / waves;
+	if (per_wave > (tiles * waves * 2 <= slots ? 48 : 80))
+		return 0;
+	return waves;
+}
+
+template<typename T, int WAVES>
+void launch_wave_split_variant(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, bool divs, int tail,
+		const Epilogue<T>& E, const LstmBackwardStep<T>* then) {
+	constexpr int TL = Mfma<T>::TL;
+	const int mtiles = (g.M + TL - 1) / TL, ftiles = (g.F + TL - 1) / TL;
+	const dim3 grid((unsigned) round_up(mtiles, 8), (unsigned) ftiles), block(64 * WAVES);
+	const size_t lds = 0;
+	LstmBackwardStep<T> none;
+	std::memset(&none, 0, sizeof none);
+	if (tail == WS_LSTM_BACKWARD)
+		wave_split_gemm_kernel<T, WAVES, false, WS_LSTM_BACKWARD><<<grid, block, lds, stream()>>>(src, wt, bias, out, g, mtiles, E, *then);
+	else if (tail == WS_ACT)
+		wave_split_gemm_kernel<T, WAVES, false, WS_ACT><<<grid, block, lds, stream()>>>(src, wt, bias, out, g, mtiles, E, none);
+	else if (divs)
+		wave_split_gemm_kernel<T, WAVES, true, WS_PLAIN><<<grid, block, lds, stream()>>>(src, wt, bias, out, g, mtiles, E, none);
+	else
+		wave_split_gemm_kernel<T, WAVES, false, WS_PLAIN><<<grid, block, lds, stream()>>>(src, wt, bias, out, g, mtiles, E, none);
+	CATTLE_HIP_CHECK(hipGetLastError());
+}
+
 template<typename T>
 bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, ScratchArena* arena = nullptr,
 		int epi = EPI_NONE, const Epilogue<T>* E = nullptr, int* mtiles_out = nullptr, const LstmBackwardStep<T>* then = nullptr,
@@ -1987,7 +2192,23 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 
 	const long total = (long) mtiles * ftiles;
 	if (!no_split && total * 2 <= slots && nchunks >= 4) {
-		/* far fewer tiles than the chip holds blocks: cut every tile's reduction so that it fills up */
+		/* far fewer tiles than the chip holds blocks: the reduction of every tile is dealt to the wavefronts of one block
+		 * where it is short enough for that (wave_split_gemm_kernel: one launch, no partial sums in memory), else cut into
+		 * parts, one block each, which a second launch adds up */
+		const bool lstm_tail = then != nullptr && epi == EPI_NONE && bias == nullptr && (size_t) g.M * g.F == then->P;
+		const int tail = lstm_tail ? WS_LSTM_BACKWARD : epi == EPI_ACT ? WS_ACT : WS_PLAIN;
+		const int waves = ((divs && tail != WS_PLAIN) || tune.no_wave_split) ? 0 : wave_split_waves<T>(g);
+		if (waves > 0) {
+			if (waves == 16)
+				launch_wave_split_variant<T, 16>(src, wt, bias, out, g, divs, tail, epi_args, then);
+			else if (waves == 8)
+				launch_wave_split_variant<T, 8>(src, wt, bias, out, g, divs, tail, epi_args, then);
+			else
+				launch_wave_split_variant<T, 4>(src, wt, bias, out, g, divs, tail, epi_args, then);
+			if (lstm_tail)
+				*then_done = true;
+			return true;
+		}
 		launch(0, (int) std::min<long>(std::min<long>(slots / total, nchunks / 2), 32));
 		return true;
 	}
