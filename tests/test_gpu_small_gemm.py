@@ -1,0 +1,141 @@
+"""Small products whose reduction is dealt to the wavefronts of one block (a block per 32 x 32 tile in fp32, 16 x 16 in
+fp64; taken when a problem has far fewer tiles than the chip holds blocks and at most a few dozen reduction steps per
+wavefront): dense layers forward and backward with and without a fused activation, convolutions with padding whose input
+gradient has few output tiles, a strided input gradient of that size, row and column counts that leave partial tiles,
+channel counts around the batch of sixteen steps, against the oracle (fp32 1e-4, fp64 1e-10; DenseKernelLayer.hpp:78-115,
+ConvKernelLayer.hpp:125-181)."""
+import importlib
+
+import numpy as np
+import pytest
+
+import helpers as hp
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+ch = importlib.import_module("c-attl3_amd")
+
+TOL = {np.dtype(np.float32): 1e-4, np.dtype(np.float64): 1e-10}
+
+# batch, inputs, outputs: reductions of one short batch, exactly one batch, several batches with a remainder; outputs that
+# leave a partial tile; batches that are not multiples of a tile or of a vector
+DENSE = [(256, 784, 512), (256, 512, 256), (256, 256, 10), (128, 1024, 10), (96, 1536, 40), (50, 200, 33), (37, 130, 7),
+         (64, 64, 64), (300, 96, 17)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("act", [None, "relu", "tanh", "softplus"])
+@pytest.mark.parametrize("case", DENSE, ids=lambda c: "x".join(str(v) for v in c))
+def test_dense_layers(case, act, dtype):
+    N, K, F = case
+    if act in ("tanh", "softplus") and case not in (DENSE[1], DENSE[5]):
+        pytest.skip("the other activations on two of the shapes")
+    gen = hp.rng(1200 + K + F)
+    x = hp.normal(gen, (N, K), dtype)
+    w = hp.normal(gen, (K, F), dtype, std=1.0 / np.sqrt(K))
+    b = hp.normal(gen, (1, F), dtype)
+    g = hp.normal(gen, (N, F), dtype)
+    dense = ch.DenseKernelLayer(dtype, (K,), F)
+    wp, bp = dense.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    layers = [dense]
+    if act:
+        layers.append(ch.ActivationLayer(dtype, act, (F,)))
+    layers = ch.fuse_layers(layers)
+    t = ch.DeviceTensor.from_host(x)
+    for l in layers:
+        t = l.pass_forward(t, True)
+    y = t.to_host()
+    d = ch.DeviceTensor.from_host(g)
+    for l in reversed(layers):
+        d = l.pass_back(d)
+    dx = d.to_host()
+    x64, w64, b64, g64 = (np.asarray(a, np.float64) for a in (x, w, b, g))
+    z_ref = oracle.dense_forward(x64, w64, b64)
+    if act:
+        y_ref = oracle.act_forward(act, z_ref)
+        dz_ref = oracle.act_backward(act, z_ref, y_ref, g64)
+    else:
+        y_ref, dz_ref = z_ref, g64
+    dx_ref, dw_ref, db_ref = oracle.dense_backward(x64, w64, dz_ref)
+    tol = TOL[np.dtype(dtype)]
+    label = "small gemm dense %s %s %s" % ("x".join(str(v) for v in case), act, np.dtype(dtype).name)
+    assert hp.rel_err(y.reshape(y_ref.shape), y_ref, label=label + " y") < tol
+    assert hp.rel_err(dx.reshape(dx_ref.shape), dx_ref, label=label + " dx") < tol
+    assert hp.rel_err(wp.get_grad(), dw_ref) < tol
+    assert hp.rel_err(bp.get_grad(), db_ref) < tol
+    # the same pass again: bit for bit
+    t = ch.DeviceTensor.from_host(x)
+    for l in layers:
+        t = l.pass_forward(t, True)
+    assert np.array_equal(t.to_host(), y)
+
+
+# N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh: few output tiles in one or both passes
+CONV = [
+    (32, 16, 16, 128, 32, 3, 3, 1, 1, 1, 1, 0, 0),       # forward: 8192 x 1152 x 32, the shape of an LSTM's recurrent input gradient
+    (32, 16, 16, 32, 128, 3, 3, 1, 1, 1, 1, 0, 0),       # its input gradient is that problem
+    (128, 16, 16, 32, 64, 3, 3, 1, 1, 1, 1, 0, 0),       # input gradient 32768 x 576 x 32
+    (24, 9, 7, 16, 24, 3, 2, 2, 1, 1, 1, 0, 0),          # padding wider than one, partial tiles in both directions
+    (16, 12, 12, 8, 40, 5, 5, 2, 2, 1, 1, 0, 0),         # eight channels: half a batch of steps per tap
+    (20, 10, 10, 36, 20, 3, 3, 0, 0, 1, 1, 1, 1),        # dilated receptor, no padding
+    (32, 13, 13, 16, 48, 3, 3, 1, 1, 2, 2, 0, 0),        # strided: the input gradient tests divisibility per tap
+    (8, 6, 6, 64, 16, 1, 1, 0, 0, 1, 1, 0, 0),           # 1 x 1 receptor
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", CONV, ids=lambda c: "x".join(str(v) for v in c))
+def test_convolutions_with_few_tiles(case, dtype):
+    N, H, W, C, F, RH, RW, pv, ph, sv, sh, dv, dh = case
+    geom = dict(RH=RH, RW=RW, pv=pv, ph=ph, sv=sv, sh=sh, dv=dv, dh=dh)
+    gen = hp.rng(1300 + H + C + F)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (RH * RW * C, F), dtype, std=1.0 / np.sqrt(RH * RW * C))
+    b = hp.normal(gen, (1, F), dtype)
+    OH, OW = hp.conv_dims(H, W, RH, RW, pv, ph, sv, sh, dv, dh)
+    g = hp.normal(gen, (N, OH, OW, F), dtype)
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F, RH, RW, pv, ph, sv, sh, dv, dh)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    xd, gd = ch.DeviceTensor.from_host(x), ch.DeviceTensor.from_host(g)
+    out = layer.pass_forward(xd, True).to_host()
+    dx = layer.pass_back(gd).to_host()
+    x64, w64, b64, g64 = (np.asarray(a, np.float64) for a in (x, w, b, g))
+    o_ref, cache = oracle.conv_forward(x64, w64, b64, return_cache=True, **geom)
+    dx_ref, dw_ref, db_ref = oracle.conv_backward(x.shape, cache, w64, g64, **geom)
+    tol = TOL[np.dtype(dtype)]
+    label = "small gemm conv %s %s" % ("x".join(str(v) for v in case), np.dtype(dtype).name)
+    assert hp.rel_err(out, o_ref, label=label + " y") < tol
+    assert hp.rel_err(dx, dx_ref, label=label + " dx") < tol
+    assert hp.rel_err(wp.get_grad(), dw_ref) < tol
+    assert hp.rel_err(bp.get_grad(), db_ref) < tol
+    layer.pass_forward(xd, True)
+    assert np.array_equal(layer.pass_back(gd).to_host(), dx)
+
+
+def test_non_finite_inputs_stay_where_they_are():
+    """Lanes in the padding and steps past the end of a wavefront's share read valid memory and must drop what they read:
+    an infinite input element may only reach the outputs whose receptor holds it."""
+    dtype = np.float32
+    N, H, W, C, F = 32, 8, 8, 32, 32
+    geom = dict(RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0)
+    gen = hp.rng(1400)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    x[0, 0, 0, 0] = np.inf              # element 0 of the tensor: what lanes in the padding read
+    x[5, 3, 4, 7] = np.inf
+    w = np.abs(hp.normal(gen, (9 * C, F), dtype, std=0.1)) + 0.01
+    b = hp.normal(gen, (1, F), dtype)
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F, 3, 3, 1, 1, 1, 1, 0, 0)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    out = layer.pass_forward(ch.DeviceTensor.from_host(x), False).to_host()
+    ref = oracle.conv_forward(np.asarray(x, np.float64), np.asarray(w, np.float64), np.asarray(b, np.float64), **geom)
+    assert np.array_equal(np.isfinite(out), np.isfinite(ref))
+    assert not np.isnan(out).any()
+    fin = np.isfinite(ref)
+    assert np.max(np.abs(out[fin] - ref[fin])) < 1e-3
