@@ -220,6 +220,34 @@ __device__ __forceinline__ size_t out_row(const GatherGeom& g, int m) {
 	return (size_t) n + (size_t) g.N * (size_t) ((g.out_a0 + g.out_sa * a) + g.out_OA * (g.out_b0 + g.out_sb * b));
 }
 
+/* Sum of v over a group of TL consecutive lanes (TL = 16: a row of the wavefront; TL = 32: two rows) with data-parallel
+ * primitives of the vector ALU - lane exchanges inside quads, mirrored halves of a row, the last lane of a row broadcast to
+ * the next row - so that no step goes through the LDS crossbar, which the wavefronts of a CU share (a butterfly of
+ * ds_bpermute over the 64 column sums of a lane was most of the moments epilogue's time). The total is valid in the
+ * last lane of the group (for TL = 16 in all of them). */
+template<int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v) {
+	return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+template<int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_move(double v) {
+	const long long bits = __builtin_bit_cast(long long, v);
+	const int lo = __builtin_amdgcn_update_dpp(0, (int) (bits & 0xffffffffll), CTRL, ROW_MASK, 0xF, false);
+	const int hi = __builtin_amdgcn_update_dpp(0, (int) (bits >> 32), CTRL, ROW_MASK, 0xF, false);
+	return __builtin_bit_cast(double, ((long long) hi << 32) | (long long) (unsigned) lo);
+}
+template<typename T, int TL>
+__device__ __forceinline__ T lane_group_sum(T v) {
+	static_assert(TL == 16 || TL == 32, "a row or two rows of the wavefront");
+	v += dpp_move<0xB1, 0xF>(v);            /* quad_perm [1, 0, 3, 2] */
+	v += dpp_move<0x4E, 0xF>(v);            /* quad_perm [2, 3, 0, 1] */
+	v += dpp_move<0x141, 0xF>(v);           /* row_half_mirror */
+	v += dpp_move<0x140, 0xF>(v);           /* row_mirror */
+	if constexpr (TL == 32)
+		v += dpp_move<0x142, 0xA>(v);       /* row_bcast:15 into rows 1 and 3 (the other rows receive zero) */
+	return v;
+}
+
 /* Several gathered GEMMs of one source and one result tensor in a single launch (the residue classes of a strided
  * input gradient): blockIdx.z picks the problem, whose geometry, tile walk and prepared weights come from this table
  * instead of the kernel's own arguments. No cut reductions: every tile is whole. */
@@ -718,9 +746,8 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 		 * m merged in ascending order by the update of Chan et al. */
 		T* const red = &As[0][0][0];                    /* [WAVES_M][BF][4]: count, shift, sum, sum of squares */
 		static_assert(WAVES_M * (WAVES_F * WT_F) * 4 <= 2 * KC * LDA, "the moment partials reuse the A operand buffers");
-		/* The cross-lane steps are written level by level over all of a lane's FB * NACC columns: the shuffles of a
-		 * level do not depend on one another, so they go out together and are waited for once (a butterfly per column,
-		 * one after the other, is a chain of a few hundred LDS-crossbar round trips). */
+		/* The cross-lane sums stay inside the vector ALU (lane_group_sum), and the shift, one value per column from the
+		 * first lane of each group, is read as a scalar (fp32; fp64 has few columns per lane and shuffles it). */
 		T c[FB][MF::NACC], s1[FB][MF::NACC], s2[FB][MF::NACC];
 		#pragma unroll
 		for (int i = 0; i < FB; ++i)
@@ -730,8 +757,16 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 		#pragma unroll
 		for (int i = 0; i < FB; ++i)
 			#pragma unroll
-			for (int r = 0; r < MF::NACC; ++r)
-				c[i][r] = __shfl(c[i][r], lane & ~(TL - 1), 64);
+			for (int r = 0; r < MF::NACC; ++r) {
+				if constexpr (std::is_same<T, float>::value) {
+					/* the first lane of each half of the wavefront, read as scalars */
+					const int bits = __builtin_bit_cast(int, c[i][r]);
+					const int lo = __builtin_amdgcn_readlane(bits, 0), hi = __builtin_amdgcn_readlane(bits, 32);
+					c[i][r] = __builtin_bit_cast(float, lk == 0 ? lo : hi);
+				} else {
+					c[i][r] = __shfl(c[i][r], lane & ~(TL - 1), 64);
+				}
+			}
 		#pragma unroll
 		for (int i = 0; i < FB; ++i)
 			#pragma unroll
@@ -747,26 +782,15 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 				}
 			}
 		#pragma unroll
-		for (int off = 1; off < TL; off <<= 1) {
-			T t1[FB][MF::NACC], t2[FB][MF::NACC];
+		for (int i = 0; i < FB; ++i)
 			#pragma unroll
-			for (int i = 0; i < FB; ++i)
-				#pragma unroll
-				for (int r = 0; r < MF::NACC; ++r) {
-					t1[i][r] = __shfl_xor(s1[i][r], off, 64);
-					t2[i][r] = __shfl_xor(s2[i][r], off, 64);
-				}
-			#pragma unroll
-			for (int i = 0; i < FB; ++i)
-				#pragma unroll
-				for (int r = 0; r < MF::NACC; ++r) {
-					s1[i][r] += t1[i][r];
-					s2[i][r] += t2[i][r];
-				}
-		}
+			for (int r = 0; r < MF::NACC; ++r) {
+				s1[i][r] = lane_group_sum<T, TL>(s1[i][r]);
+				s2[i][r] = lane_group_sum<T, TL>(s2[i][r]);
+			}
 		/* rows of this wave that exist: all of them in the blocked order, else what is left of M */
 		const int wave_rows = L.sample_blocks > 0 ? WT_M : max(0, min(WT_M, g.M - (tile * BM + wm * WT_M)));
-		if (lc == 0) {
+		if (lc == TL - 1) {                  /* the lane that holds the group's totals */
 			#pragma unroll
 			for (int i = 0; i < FB; ++i)
 				#pragma unroll

@@ -1400,10 +1400,67 @@ __device__ __forceinline__ void merge_tile_moments(const T* __restrict__ stats, 
 	m2 = lds[2][0];
 }
 
+/* (sample, pooled row, pooled column) of element i of a channel's pooled slab, kept up to date as i advances by a fixed
+ * step: the divisions happen once per thread, each step costs two additions with carry (64-bit divisions per iteration
+ * were most of the instructions of these loops). */
+struct PooledWalk {
+	int n, a, b;            /* i = n + N * (a + OHp * b) */
+	int dn, da, db;         /* the step, decomposed the same way */
+};
+__device__ __forceinline__ PooledWalk pooled_walk(size_t i, unsigned step, int N, int OHp) {
+	PooledWalk w;
+	const unsigned i32 = (unsigned) i;      /* a slab has fewer than 2^31 elements */
+	w.n = (int) (i32 % (unsigned) N);
+	const unsigned t = i32 / (unsigned) N;
+	w.a = (int) (t % (unsigned) OHp);
+	w.b = (int) (t / (unsigned) OHp);
+	w.dn = (int) (step % (unsigned) N);
+	const unsigned dt = step / (unsigned) N;
+	w.da = (int) (dt % (unsigned) OHp);
+	w.db = (int) (dt / (unsigned) OHp);
+	return w;
+}
+__device__ __forceinline__ void pooled_walk_next(PooledWalk& w, int N, int OHp) {
+	w.n += w.dn;
+	const int c1 = w.n >= N;
+	w.n -= c1 ? N : 0;
+	w.a += w.da + c1;
+	const int c2 = w.a >= OHp;
+	w.a -= c2 ? OHp : 0;
+	w.b += w.db + c2;
+}
+
 struct ChainBn {
 	int mtiles;             /* rows of the per-tile moments (training) */
 	int training, stats_init;
+	int merged;             /* training: mean_cache and inv_sd_cache already hold the batch moments (bn_merge_moments_kernel) */
 };
+
+/* Mean and inverse standard deviation of every channel from the per-tile moments, and the running averages' update
+ * (BatchNormLayer.hpp:229-243), one block per channel: for launches with so many tiles that merging them in every block
+ * of bn_chain_forward_kernel (a chain of dependent loads per thread, repeated by all blocks of a channel) would take
+ * longer than a launch of its own. */
+template<typename T>
+__global__ __launch_bounds__(256)
+void bn_merge_moments_kernel(const T* __restrict__ stats, int mtiles, int C, size_t L, T* __restrict__ avg_mean,
+		T* __restrict__ avg_inv_sd, int stats_init, T decay, T eps, T* __restrict__ mean_cache, T* __restrict__ inv_sd_cache) {
+	__shared__ T lds[3][256];
+	const int c = blockIdx.x;
+	T mean, m2;
+	merge_tile_moments<T>(stats, mtiles, C, c, lds, mean, m2);
+	if (threadIdx.x == 0) {
+		const T inv_sd = (T) 1 / dev_sqrt(m2 / (T) L + eps);
+		mean_cache[c] = mean;
+		inv_sd_cache[c] = inv_sd;
+		if (stats_init) {
+			avg_mean[c] = ((T) 1 - decay) * avg_mean[c] + decay * mean;
+			avg_inv_sd[c] = ((T) 1 - decay) * avg_inv_sd[c] + decay * inv_sd;
+		} else {
+			avg_mean[c] = mean;
+			avg_inv_sd[c] = inv_sd;
+		}
+	}
+}
 
 /* Forward pass behind the kernel layer with batch norm: channel moments (training: merged from the tiles' moments;
  * inference: the running statistics), then y = act(gamma * (z - mean) * inv_sd + beta), pooled when POOL. The
@@ -1419,7 +1476,10 @@ void bn_chain_forward_kernel(ChainShape s, int N, size_t span, ChainBn bn, const
 	const int OHp = s.H / s.prh, OWp = s.W / s.prw;
 	const size_t L = (size_t) N * s.H * s.W, Lp = (size_t) N * OHp * OWp;
 	T mean, inv_sd;
-	if (bn.training) {
+	if (bn.training && bn.merged) {
+		mean = mean_cache[c];
+		inv_sd = inv_sd_cache[c];
+	} else if (bn.training) {
 		T m2;
 		merge_tile_moments<T>(stats, bn.mtiles, s.C, c, lds, mean, m2);
 		inv_sd = (T) 1 / dev_sqrt(m2 / (T) L + eps);
@@ -1444,10 +1504,9 @@ void bn_chain_forward_kernel(ChainShape s, int N, size_t span, ChainBn bn, const
 	T* oc = out + (size_t) c * Lp;
 	act_dispatch(s.kind, [&](auto kc) {
 		constexpr int KIND = decltype(kc)::value;
-		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
-			const int n = (int) (i % (size_t) N);
-			const size_t t = i / (size_t) N;
-			const int a_p = (int) (t % (size_t) OHp), b_p = (int) (t / (size_t) OHp);
+		PooledWalk walk = pooled_walk(begin + (size_t) threadIdx.x * V, 256u * V, N, OHp);
+		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V, pooled_walk_next(walk, N, OHp)) {
+			const int n = walk.n, a_p = walk.a, b_p = walk.b;
 			const T* base = zc + n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw));
 			T res[V];
 			unsigned bi[V];
@@ -1537,10 +1596,9 @@ void bn_chain_sums_kernel(ChainShape s, int N, size_t span, const T* __restrict_
 	T s1 = (T) 0, s2 = (T) 0;
 	act_dispatch(s.kind, [&](auto kc) {
 		constexpr int KIND = decltype(kc)::value;
-		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
-			const int n = (int) (i % (size_t) N);
-			const size_t t = i / (size_t) N;
-			const int a_p = (int) (t % (size_t) OHp), b_p = (int) (t / (size_t) OHp);
+		PooledWalk walk = pooled_walk(begin + (size_t) threadIdx.x * V, 256u * V, N, OHp);
+		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V, pooled_walk_next(walk, N, OHp)) {
+			const int n = walk.n, a_p = walk.a, b_p = walk.b;
 			const T* base = zc + n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw));
 			T gv[V];
 			unsigned iv[V];
@@ -1592,10 +1650,9 @@ void bn_chain_apply_kernel(ChainShape s, int N, size_t span, const T* __restrict
 	T* dc = dz + (size_t) c * L;
 	act_dispatch(s.kind, [&](auto kc) {
 		constexpr int KIND = decltype(kc)::value;
-		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V) {
-			const int n = (int) (i % (size_t) N);
-			const size_t t = i / (size_t) N;
-			const int a_p = (int) (t % (size_t) OHp), b_p = (int) (t / (size_t) OHp);
+		PooledWalk walk = pooled_walk(begin + (size_t) threadIdx.x * V, 256u * V, N, OHp);
+		for (size_t i = begin + (size_t) threadIdx.x * V; i < end; i += (size_t) 256 * V, pooled_walk_next(walk, N, OHp)) {
+			const int n = walk.n, a_p = walk.a, b_p = walk.b;
 			const size_t off = n + (size_t) N * ((size_t) a_p * s.prh + (size_t) s.H * ((size_t) b_p * s.prw));
 			T gv[V];
 			unsigned iv[V];
@@ -1654,6 +1711,10 @@ void chain_backward(const ChainShape& s, int N, const T* g, const unsigned* inds
 	check_launch();
 }
 
+/* From this many tiles on the tiles' moments are merged by bn_merge_moments_kernel: measured on 256 x 56 x 56 x 64 (1568
+ * tiles), merging inside bn_chain_forward_kernel took 26 of its 82 us; at 512 tiles it is two loads per thread. */
+constexpr int BN_CHAIN_MERGE_TILES = 1024;
+
 size_t bn_chain_workspace(int channels) {
 	return (size_t) 2 * channels * BN_MAX_SPLITS;
 }
@@ -1664,7 +1725,14 @@ void bn_chain_forward_launch(const ChainShape& s, int N, int mtiles, bool traini
 		unsigned* inds) {
 	const size_t Lp = (size_t) N * (s.H / s.prh) * (s.W / s.prw);
 	const int splits = bn_splits(s.C, Lp);
-	const ChainBn bn = { mtiles, training ? 1 : 0, stats_init ? 1 : 0 };
+	/* many tiles: their moments are merged once per channel by a launch of its own rather than by every block */
+	const bool merged = training && mtiles >= BN_CHAIN_MERGE_TILES;
+	if (merged) {
+		bn_merge_moments_kernel<T><<<(unsigned) s.C, 256, 0, stream()>>>(stats, mtiles, s.C, (size_t) N * s.H * s.W, avg_mean, avg_inv_sd,
+				stats_init ? 1 : 0, decay, eps, mean_cache, inv_sd_cache);
+		check_launch();
+	}
+	const ChainBn bn = { mtiles, training ? 1 : 0, stats_init ? 1 : 0, merged ? 1 : 0 };
 	bn_chain_forward_kernel<T, V, POOL><<<dim3((unsigned) s.C, (unsigned) splits), 256, 0, stream()>>>(s, N, bn_span(Lp, splits), bn, z,
 			stats, gamma, beta, avg_mean, avg_inv_sd, decay, eps, mean_cache, inv_sd_cache, out, inds);
 	check_launch();

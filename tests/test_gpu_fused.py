@@ -412,6 +412,8 @@ BN_CASES = [
     (32, 6, 10, 4, 9, ("tanh", 0.0), ("max", 2, 2, 2, 2), False),
     (8, 9, 9, 3, 5, ("softplus", 0.0), ("max", 3, 3, 2, 2), False),          # overlapping windows behind the chain pass
     (64, 1, 1, 48, 24, ("relu", 0.0), None, True),
+    # more than a thousand GEMM tiles: their moments are merged by a launch of its own in front of the chain's forward pass
+    (64, 96, 96, 3, 8, ("relu", 0.0), ("max", 2, 2, 2, 2), False),
 ]
 
 
