@@ -1511,7 +1511,10 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES;
 	constexpr int TL = MF::TL, KS = MF::KS;
-	constexpr int B = 16;                   /* reduction steps per batch of loads */
+	/* Reduction steps per batch of loads: 48 operand registers (a block of sixteen wavefronts has 128 registers per lane;
+	 * batches of 32 steps spilled), 32 in the blocks of four wavefronts, of which a CU must hold four (measured: at 136
+	 * registers it held three, and 1024 tiles took a second round) */
+	constexpr int B = (WAVES == 4 ? 16 : 24) / (int) (sizeof(T) / 4);
 	__shared__ T red[WAVES * TL * TL];
 
 	const int mtile = xcd_tile(blockIdx.x, mtiles);
@@ -1561,7 +1564,7 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 		ok = ok && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
 		const int c_first = cg0 * KS + lk;
 		/* 32-bit byte offsets from the kernel's own pointers: a load then needs one address register, not two, and
-		 * sixteen steps' worth of loads fit beside the accumulators. Lanes in the padding read element 0 and drop it. */
+		 * a whole batch of loads fits beside the accumulators. Lanes in the padding read element 0 and drop it. */
 		unsigned aoff = ok ? (unsigned) (n + g.NS * (ya + g.LH * yb) + plane * c_first) * (unsigned) sizeof(T) : 0u;
 		const unsigned ainc = ok ? astep : 0u;
 		unsigned boff = (unsigned) ((tap + taps * c_first) * g.ldw + f0 + lc) * (unsigned) sizeof(T);
@@ -1601,9 +1604,14 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 				wb[u] = load_b(boff + uu * bstep);
 			}
 			__builtin_amdgcn_sched_barrier(0);
+			/* (in groups of four, so that a short remainder does not pay for a whole batch of matrix instructions) */
 			#pragma unroll
-			for (int u = 0; u < B; ++u)
-				acc[u & 1] = MF::mma(wb[u], (ok && u < rem) ? xa[u] : (T) 0, acc[u & 1]);
+			for (int u0 = 0; u0 < B; u0 += 4)
+				if (u0 < rem) {
+					#pragma unroll
+					for (int u = u0; u < u0 + 4; ++u)
+						acc[u & 1] = MF::mma(wb[u], (ok && u < rem) ? xa[u] : (T) 0, acc[u & 1]);
+				}
 			__builtin_amdgcn_sched_barrier(0);
 		}
 		s0 += count;
@@ -2010,9 +2018,9 @@ int wave_split_waves(const GatherGeom& g) {
 	int waves = 16;
 	while (waves > 4 && (tiles * waves > slots || steps < 8 * waves))
 		waves /= 2;
-	/* A wavefront's share of the reduction is a chain of batches of sixteen steps, each a round trip to memory of two
-	 * microseconds or more: three batches where the wavefronts are few (their round trips coincide), five where the chip
-	 * is full of them (blocks at different points of their chains overlap). Longer reductions are cut across blocks
+	/* A wavefront's share of the reduction is a chain of batches of loads, each a round trip to memory of two
+	 * microseconds or more: 48 steps (two or three batches) where the wavefronts are few and their round trips coincide, 80
+	 * where the chip is full of them (blocks at different points of their chains overlap). Longer reductions are cut across blocks
 	 * (measured: a dense layer 4096 -> 10 at batch 128, four tiles, 23 us this way, 12 us cut across blocks). */
 	const int per_wave = (steps + waves - 1) / waves;
 	if (per_wave > (tiles * waves * 2 <= slots ? 48 : 80))
