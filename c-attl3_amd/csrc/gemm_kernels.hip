@@ -2244,12 +2244,13 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		launch(0, (int) std::min<long>(std::min<long>(slots / total, nchunks / 2), 32));
 		return true;
 	}
-	const int rem = mtiles % slots;
-	if (!no_split && ftiles == 1 && mtiles > slots && rem > 0 && rem * 2 <= slots && nchunks >= 8) {
+	/* (a round of the chip holds slots / ftiles rows of tiles) */
+	const int round_m = std::max(1, slots / ftiles), rem = mtiles % round_m;
+	if (!no_split && mtiles > round_m && rem > 0 && rem * 2 <= round_m && nchunks >= 8) {
 		/* The tiles left over after whole rounds would keep a fraction of the chip busy for a whole tile time.
 		 * Their reduction is cut into parts instead; the part blocks come last in the grid and fill the
 		 * chip as the last round of whole tiles drains. */
-		launch(mtiles - rem, (int) std::min<long>(std::min(slots / rem, nchunks / 4), 16));
+		launch(mtiles - rem, (int) std::min<long>(std::min(round_m / rem, nchunks / 4), 16));
 		return true;
 	}
 	launch(mtiles, 1);

@@ -139,3 +139,36 @@ def test_non_finite_inputs_stay_where_they_are():
     assert not np.isnan(out).any()
     fin = np.isfinite(ref)
     assert np.max(np.abs(out[fin] - ref[fin])) < 1e-3
+
+
+# ---- many tiles in several column blocks: the tiles left over after whole rounds of the chip are cut into parts ------------
+
+@pytest.mark.parametrize("N", [96, 144])
+@pytest.mark.parametrize("wide_side", ["forward", "input gradient"])
+def test_left_over_tiles_with_several_column_blocks(N, wide_side):
+    """Launches whose tiles form more than one column block and do not fill whole rounds of the chip: the left-over rows of
+    tiles have their reduction cut into parts that a second launch adds (which batch size leaves such rows depends on how
+    many blocks a CU holds, so two are tried). 192 output columns are two column blocks of the widest tile; the wide side
+    is the forward pass of a 16 -> 192 layer or the input gradient of a 192 -> 16 layer."""
+    dtype = np.float32
+    H = W = 28
+    C, F = (16, 192) if wide_side == "forward" else (192, 16)
+    geom = dict(RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0)
+    gen = hp.rng(1500 + N + C)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (9 * C, F), dtype, std=1.0 / np.sqrt(9 * C))
+    b = hp.normal(gen, (1, F), dtype)
+    g = hp.normal(gen, (N, H, W, F), dtype)
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F, 3, 3, 1, 1, 1, 1, 0, 0)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    out = layer.pass_forward(ch.DeviceTensor.from_host(x), True).to_host()
+    dx = layer.pass_back(ch.DeviceTensor.from_host(g)).to_host()
+    x64, w64, b64, g64 = (np.asarray(a, np.float64) for a in (x, w, b, g))
+    o_ref, cache = oracle.conv_forward(x64, w64, b64, return_cache=True, **geom)
+    dx_ref, dw_ref, db_ref = oracle.conv_backward(x.shape, cache, w64, g64, **geom)
+    label = "left-over tiles %s N=%d" % (wide_side, N)
+    assert hp.rel_err(out, o_ref, label=label + " y") < 1e-4
+    assert hp.rel_err(dx, dx_ref, label=label + " dx") < 1e-4
+    assert hp.rel_err(wp.get_grad(), dw_ref) < 1e-4
