@@ -1233,6 +1233,10 @@ __device__ __forceinline__ void reduce_partials_block(const T* __restrict__ part
 template<typename T>
 __device__ __forceinline__ void reduce_partials_wide_block(const T* __restrict__ partials, T* __restrict__ dst, size_t count, int blk,
 		int splits) {
+	/* Neighbouring outputs share the cache lines of every slice: the blocks of one XCD take a contiguous range of outputs,
+	 * so that a line is fetched by one L2, not by all eight (the entry's blocks start at a multiple of 8 and are a
+	 * multiple of 8, see reduce_partials_many). */
+	blk = xcd_tile(blk, (int) (((count + 3) / 4 + 7) / 8 * 8));
 	const size_t i = (size_t) blk * 4 + threadIdx.x / 64;
 	if (i >= count)
 		return;
@@ -2610,8 +2614,10 @@ WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 	const int tiles = p.ktiles * p.ftiles;
 	const int chunks = (M + v.mc - 1) / v.mc;
 	int want = std::max(1, slots / tiles);
-	const int min_chunks = tune.wgrad_min_chunks > 0 ? tune.wgrad_min_chunks : (short_m ? 2 : 4);
-	want = std::min(want, std::max(1, chunks / min_chunks));  /* at least four chunks per block */
+	/* at least four chunks per block; two where the chunks are 128 rows long (measured on 32768 x 288 x 64: 128 slices of
+	 * two chunks 49.9 us for the backward pass, 64 slices of four 53.0 us) */
+	const int min_chunks = tune.wgrad_min_chunks > 0 ? tune.wgrad_min_chunks : (short_m || v.mc >= 128 ? 2 : 4);
+	want = std::min(want, std::max(1, chunks / min_chunks));
 	if (tune.wgrad_splits > 0)
 		want = std::min(tune.wgrad_splits, chunks);
 	p.chunks_per_split = (chunks + want - 1) / want;
@@ -2797,7 +2803,7 @@ void reduce_partials_many(ReduceBatch<T> batch) {
 		ReduceEntry<T>& q = batch.e[i];
 		q.first_block = blocks;
 		const size_t per = q.wide ? 4 : 64;
-		const size_t need = (q.count + per - 1) / per;
+		const size_t need = ((q.count + per - 1) / per + 7) / 8 * 8;      /* whole groups of eight: a block's XCD is its number modulo 8 */
 		CATTLE_HIP_REQUIRE(need + (size_t) blocks <= 2147483647u, "gradients too large for one reduce launch");
 		blocks += (int) need;
 	}
