@@ -1515,10 +1515,10 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES;
 	constexpr int TL = MF::TL, KS = MF::KS;
-	/* Reduction steps per batch of loads: 48 operand registers (a block of sixteen wavefronts has 128 registers per lane;
-	 * batches of 32 steps spilled), 32 in the blocks of four wavefronts, of which a CU must hold four (measured: at 136
-	 * registers it held three, and 1024 tiles took a second round) */
-	constexpr int B = (WAVES == 4 ? 16 : 24) / (int) (sizeof(T) / 4);
+	/* Reduction steps per batch of loads: 64 operand registers in fp32, 48 in fp64 (a block of sixteen wavefronts has 128
+	 * registers per lane; more spilled), 32 in the blocks of four wavefronts, of which a CU must hold four (measured: at
+	 * 136 registers it held three, and 1024 tiles took a second round) */
+	constexpr int B = sizeof(T) == 4 ? (WAVES == 4 ? 16 : 32) : (WAVES == 4 ? 8 : 12);
 	__shared__ T red[WAVES * TL * TL];
 
 	const int mtile = xcd_tile(blockIdx.x, mtiles);
@@ -1546,12 +1546,12 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 	const int s_begin = wave * per, s_end = min(total, s_begin + per);
 	const unsigned astep = (unsigned) (plane * KS) * (unsigned) sizeof(T), bstep = (unsigned) (taps * KS * g.ldw) * (unsigned) sizeof(T);   /* bytes */
 
-	typename MF::acc_t acc[2];
+	/* one accumulator: a SIMD's matrix pipe runs one instruction at a time, so a chain of dependent instructions costs
+	 * nothing, and a second accumulator's registers are worth more as loads in flight */
+	typename MF::acc_t acc;
 	#pragma unroll
-	for (int i = 0; i < 2; ++i)
-		#pragma unroll
-		for (int r = 0; r < MF::NACC; ++r)
-			acc[i][r] = (T) 0;
+	for (int r = 0; r < MF::NACC; ++r)
+		acc[r] = (T) 0;
 
 	for (int s0 = s_begin; s0 < s_end;) {
 		const int tap = s0 / spt, cg0 = s0 - tap * spt;
@@ -1594,7 +1594,7 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 			__builtin_amdgcn_sched_barrier(0);
 			#pragma unroll
 			for (int u = 0; u < B; ++u)
-				acc[u & 1] = MF::mma(wb[u], ok ? xa[u] : (T) 0, acc[u & 1]);
+				acc = MF::mma(wb[u], ok ? xa[u] : (T) 0, acc);
 			__builtin_amdgcn_sched_barrier(0);
 		}
 		if (i < count) {
@@ -1614,7 +1614,7 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 				if (u0 < rem) {
 					#pragma unroll
 					for (int u = u0; u < u0 + 4; ++u)
-						acc[u & 1] = MF::mma(wb[u], (ok && u < rem) ? xa[u] : (T) 0, acc[u & 1]);
+						acc = MF::mma(wb[u], (ok && u < rem) ? xa[u] : (T) 0, acc);
 				}
 			__builtin_amdgcn_sched_barrier(0);
 		}
@@ -1622,7 +1622,7 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 	}
 	#pragma unroll
 	for (int r = 0; r < MF::NACC; ++r)
-		red[(wave * TL + acc_row<T>(r, lk)) * TL + lc] = acc[0][r] + acc[1][r];
+		red[(wave * TL + acc_row<T>(r, lk)) * TL + lc] = acc[r];
 	__syncthreads();
 	for (int o = tid; o < TL * TL; o += THREADS) {
 		T v = red[o];
