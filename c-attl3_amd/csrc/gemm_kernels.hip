@@ -1242,8 +1242,21 @@ __device__ __forceinline__ void reduce_partials_wide_block(const T* __restrict__
 		return;
 	const int lane = threadIdx.x % 64;
 	T s = (T) 0;
-	for (int p = lane; p < splits; p += 64)
-		s += partials[(size_t) p * count + i];
+	/* eight slices' loads are issued before the first of their additions (one after the other they are a chain of memory
+	 * round trips); the additions keep their order */
+	constexpr int AHEAD = 8;
+	for (int p0 = lane; p0 < splits; p0 += 64 * AHEAD) {
+		T v[AHEAD];
+		#pragma unroll
+		for (int j = 0; j < AHEAD; ++j) {
+			const int p = p0 + 64 * j;
+			v[j] = p < splits ? partials[(size_t) p * count + i] : (T) 0;
+		}
+		#pragma unroll
+		for (int j = 0; j < AHEAD; ++j)
+			if (p0 + 64 * j < splits)
+				s += v[j];
+	}
 	#pragma unroll
 	for (int off = 32; off > 0; off >>= 1)
 		s += __shfl_down(s, off, 64);
