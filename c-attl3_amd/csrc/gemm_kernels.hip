@@ -258,15 +258,25 @@ template<typename T> struct GatherClasses {
 	const T* wt[MAX_GATHER_CLASSES];
 };
 
+/* A block's place in the launch as the GEMM bodies see it: the kernels that run a body alone pass the hardware's block
+ * index, a kernel that runs two problems in one launch passes each its own numbering. */
+struct BlockPlace {
+	int x, y, ny;           /* block index along x and y, blocks along y */
+};
+__device__ __forceinline__ BlockPlace own_block_place() {
+	return BlockPlace{ (int) blockIdx.x, (int) blockIdx.y, (int) gridDim.y };
+}
+
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI, int PF>
 __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom& g, const GatherLaunch& L, T* __restrict__ partials, const Epilogue<T>& E);
+		T* __restrict__ out, const GatherGeom& g, const GatherLaunch& L, T* __restrict__ partials, const Epilogue<T>& E,
+		const BlockPlace bp);
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI = EPI_NONE, int PF = 1>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
 void gather_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom g, const GatherLaunch L, T* __restrict__ partials, const Epilogue<T> E) {
-	gather_gemm_body<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, DIVS, EPI, PF>(src, wt, bias, out, g, L, partials, E);
+	gather_gemm_body<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, DIVS, EPI, PF>(src, wt, bias, out, g, L, partials, E, own_block_place());
 }
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC>
@@ -276,12 +286,13 @@ void gather_gemm_classes_kernel(const T* __restrict__ src, T* __restrict__ out, 
 	const GatherLaunch L = classes.L[blockIdx.z];
 	const Epilogue<T> none = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr, {} };
 	gather_gemm_body<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_NONE, 1>(src, classes.wt[blockIdx.z], (const T*) nullptr, out, g, L,
-			(T*) nullptr, none);
+			(T*) nullptr, none, own_block_place());
 }
 
 template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC, bool DIVS, int EPI, int PF>
 __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom& g, const GatherLaunch& L, T* __restrict__ partials, const Epilogue<T>& E) {
+		T* __restrict__ out, const GatherGeom& g, const GatherLaunch& L, T* __restrict__ partials, const Epilogue<T>& E,
+		const BlockPlace bp) {
 	typedef Mfma<T> MF;
 	constexpr int THREADS = 64 * WAVES_M * WAVES_F;
 	constexpr int BM = WAVES_M * WT_M, BF = WAVES_F * WT_F;
@@ -306,13 +317,13 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 	__shared__ int4 ktab[NSLOT][KC];     /* per reduction index: element offset, ya term, yb term, channel offset */
 
 	int local, part = 0;
-	const bool split = (int) blockIdx.x >= L.main_blocks;
+	const bool split = bp.x >= L.main_blocks;
 	if (!split) {
-		local = xcd_tile(blockIdx.x, L.main_count);
+		local = xcd_tile(bp.x, L.main_count);
 		if (local >= L.main_count)
 			return;
 	} else {
-		const int r = (int) blockIdx.x - L.main_blocks;
+		const int r = bp.x - L.main_blocks;
 		local = r / L.ksplit;
 		part = r - local * L.ksplit;
 		if (local >= L.split_count)
@@ -322,7 +333,7 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 	if (L.tile_rows > 0)
 		tile = swizzle_tile(tile, L.tile_rows, L.mtiles / L.tile_rows);
 	const int tid = threadIdx.x;
-	const int f0 = blockIdx.y * BF;
+	const int f0 = bp.y * BF;
 	/* The bias values of the tile's columns go through LDS: fetched now, read in the epilogue, many barriers later.
 	 * Read from global memory there, each of a lane's FB * NACC values was a load with a wait of its own in front
 	 * of its store: sixteen to thirty-two memory round trips in a row at the end of every block. */
@@ -347,7 +358,7 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 		for (int it = 0; it < LSTM_ELEMS; ++it) {
 			const int idx = tid + it * THREADS, row = idx % BM, cl = idx / BM;
 			const int mrow = tile_row_m(L, g, tile, BM, row);
-			lstm_e[it] = mrow < g.M ? (unsigned) mrow + (unsigned) g.M * (unsigned) (blockIdx.y * CB + cl) : 0xffffffffu;
+			lstm_e[it] = mrow < g.M ? (unsigned) mrow + (unsigned) g.M * (unsigned) (bp.y * CB + cl) : 0xffffffffu;
 			/* (every element of the array assigned: a partly initialised register array ends up in scratch memory) */
 			lstm_in[it] = lstm_forward_load<T>(E.lstm, lstm_e[it] != 0xffffffffu ? lstm_e[it] : 0u);
 		}
@@ -546,7 +557,7 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 	constexpr int VS = MB * (int) sizeof(T) > 16 ? 16 / (int) sizeof(T) : MB;
 	if (split) {
 		/* partial sums of this part: a dense BF x BM tile (m fastest), always whole and aligned */
-		T* ptile = partials + ((size_t) (local * (int) gridDim.y + (int) blockIdx.y) * L.ksplit + part) * (BM * BF);
+		T* ptile = partials + ((size_t) (local * bp.ny + bp.y) * L.ksplit + part) * (BM * BF);
 		#pragma unroll
 		for (int i = 0; i < FB; ++i)
 			#pragma unroll
@@ -875,11 +886,10 @@ struct WgradSplit {
  * grid = tiles * splits blocks (1-D). Bias rows are dealt out over the k tiles (row f belongs to the
  * block with f % ktiles == k-tile index) so that every block does the same amount of extra work.
  * ---------------------------------------------------------------------------------------------- */
-template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, int MIN_WAVES, bool ACTG = false>
-__global__ __launch_bounds__(64 * WAVES_K * WAVES_F, MIN_WAVES)      /* MIN_WAVES: wavefronts per SIMD the registers must allow */
-void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
-		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan, const T* __restrict__ act_y,
-		T* __restrict__ act_dz, T act_p0, T act_p1) {
+template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, bool ACTG>
+__device__ __forceinline__ void wgrad_body(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
+		T* __restrict__ bias_partials, const GatherGeom& g, const WgradSplit& plan, const T* __restrict__ act_y,
+		T* __restrict__ act_dz, T act_p0, T act_p1, int bid) {
 	/* (the activation's tensors as parameters of their own: pointers inside a structure are not known to point to global
 	 * memory, and flat loads count against the LDS counter as well, see vec_load_global) */
 	typedef Mfma<T> MF;
@@ -903,7 +913,7 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 	const int tid = threadIdx.x;
 	/* blocks of one slice (its k and f tiles) get consecutive positions on one XCD: they read the same
 	 * rows of G, which then come out of that XCD's L2 instead of HBM */
-	const int pos = xcd_tile(blockIdx.x, plan.tiles * plan.splits);
+	const int pos = xcd_tile(bid, plan.tiles * plan.splits);
 	if (pos >= plan.tiles * plan.splits)
 		return;
 	const int split = pos / plan.tiles, tile = pos - split * plan.tiles;
@@ -1187,6 +1197,39 @@ void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __rest
 			s += bred[tid * Q + q];
 		T* o = bias_partials + ((size_t) split * g.F + f0 + tid);
 		*o = direct ? *o + s : s;
+	}
+}
+
+template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, int MIN_WAVES, bool ACTG = false>
+__global__ __launch_bounds__(64 * WAVES_K * WAVES_F, MIN_WAVES)      /* MIN_WAVES: wavefronts per SIMD the registers must allow */
+void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
+		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan, const T* __restrict__ act_y,
+		T* __restrict__ act_dz, T act_p0, T act_p1) {
+	wgrad_body<T, WAVES_K, WAVES_F, WT_K, WT_F, MC, VEC, ACTG>(src, og, partials, bias_partials, g, plan, act_y, act_dz, act_p0, act_p1,
+			(int) blockIdx.x);
+}
+
+/* A layer's input gradient and its weight gradient in one launch, for layers whose two launches are a few microseconds
+ * each and wait for nothing but the same upstream gradient (the last layers of a network: a dependent launch costs 4-5 us
+ * however little it does). The gather GEMM's blocks keep their places (x below gather_x); the weight gradient's blocks,
+ * one wavefront each (the 32 x 32 tile), are the blocks with x from gather_x on, numbered row by row of the grid. */
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC, int VEC>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_F)
+void gather_with_wgrad_kernel(const T* __restrict__ src, const T* __restrict__ wt, T* __restrict__ out, const GatherGeom g,
+		const GatherLaunch L, int gather_x, const T* __restrict__ w_src, const T* __restrict__ w_og, T* __restrict__ w_partials,
+		T* __restrict__ w_bias_partials, const GatherGeom w_g, const WgradSplit w_plan) {
+	if ((int) blockIdx.x < gather_x) {
+		const Epilogue<T> none = { 0, (T) 0, nullptr, nullptr, 1, 1, 1, 1, nullptr, {} };
+		gather_gemm_body<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, VEC, false, EPI_NONE, 1>(src, wt, (const T*) nullptr, out, g, L, (T*) nullptr, none,
+				BlockPlace{ (int) blockIdx.x, (int) blockIdx.y, (int) gridDim.y });
+	} else {
+		if (threadIdx.x >= 64)
+			return;
+		const int bid = ((int) blockIdx.x - gather_x) + ((int) gridDim.x - gather_x) * (int) blockIdx.y;
+		if (bid >= (w_plan.tiles * w_plan.splits + 7) / 8 * 8)
+			return;
+		wgrad_body<T, 1, 1, 32, 32, 32, VEC, false>(w_src, w_og, w_partials, w_bias_partials, w_g, w_plan,
+				(const T*) nullptr, (T*) nullptr, (T) 0, (T) 0, bid);
 	}
 }
 
@@ -1777,6 +1820,17 @@ void split_reduce_lstm_backward_kernel(const T* __restrict__ partials, const Gat
 		lstm_backward_element<T, false>(A, (unsigned) m + (unsigned) g.M * (unsigned) f, true, acc);
 }
 
+/* A weight-gradient launch of one-wavefront 32 x 32 tiles (fp32) that may ride in an input-gradient launch
+ * (gather_with_wgrad_kernel) instead of being a launch of its own; `done` says whether it did. */
+template<typename T>
+struct WgradRider {
+	const T *x, *og;
+	T *partials, *bias_partials;
+	GatherGeom g;
+	WgradSplit plan;
+	bool done;
+};
+
 /* One instantiation of gather_gemm_kernel and what the tile chooser needs to know about it. */
 template<typename T>
 struct GatherVariant {
@@ -1785,6 +1839,9 @@ struct GatherVariant {
 	void (*launch)(dim3 grid, size_t dyn_lds, const T*, const T*, const T*, T*, const GatherGeom&, const GatherLaunch&,
 			T* partials, bool vec, bool divs, int epi, const Epilogue<T>&);
 	void (*launch_classes)(dim3 grid, const T* src, T* out, const GatherClasses<T>&);      /* 16-byte loads, no divisors, no epilogue */
+	/* whole tiles, 16-byte loads, no divisors, no bias, no epilogue, with a small weight gradient in the same launch; null
+	 * where that kernel does not exist */
+	void (*launch_with_wgrad)(const GatherLaunch&, int ftiles, const T* src, const T* wt, T* out, const GatherGeom&, const WgradRider<T>&);
 	int (*blocks_per_cu)(size_t dyn_lds, bool vec, bool divs, int epi);       /* what the runtime says fits on a CU */
 };
 
@@ -1815,6 +1872,17 @@ void launch_gather_variant(dim3 grid, size_t dyn, const T* src, const T* wt, con
 		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, false, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
 	else
 		gather_gemm_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, 1, true, EPI_NONE, PF><<<grid, block, dyn, stream()>>>(src, wt, bias, out, g, L, partials, E);
+	CATTLE_HIP_CHECK(hipGetLastError());
+}
+
+template<typename T, int WAVES_M, int WAVES_F, int WT_M, int WT_F, int KC>
+void launch_gather_with_wgrad_variant(const GatherLaunch& L, int ftiles, const T* src, const T* wt, T* out, const GatherGeom& g,
+		const WgradRider<T>& r) {
+	const int gather_x = L.main_blocks;
+	const int w_blocks = round_up(r.plan.tiles * r.plan.splits, 8);
+	const dim3 grid((unsigned) (gather_x + (w_blocks + ftiles - 1) / ftiles), (unsigned) ftiles), block(64 * WAVES_M * WAVES_F);
+	gather_with_wgrad_kernel<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, GemmCfg<T>::VEC><<<grid, block, 0, stream()>>>(src, wt, out, g, L, gather_x,
+			r.x, r.og, r.partials, r.bias_partials, r.g, r.plan);
 	CATTLE_HIP_CHECK(hipGetLastError());
 }
 
@@ -1872,6 +1940,9 @@ GatherVariant<T> gather_variant() {
 	v.kc = KC;
 	v.launch = &launch_gather_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, PF>;
 	v.launch_classes = &launch_gather_classes_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC>;
+	v.launch_with_wgrad = nullptr;
+	if constexpr (std::is_same<T, float>::value && WAVES_M * WT_M <= 64 && PF == 1)      /* the short tiles, fp32 */
+		v.launch_with_wgrad = &launch_gather_with_wgrad_variant<T, WAVES_M, WAVES_F, WT_M, WT_F, KC>;
 	v.blocks_per_cu = &gather_variant_occupancy<T, WAVES_M, WAVES_F, WT_M, WT_F, KC, PF>;
 	return v;
 }
@@ -2068,7 +2139,7 @@ void launch_wave_split_variant(const T* src, const T* wt, const T* bias, T* out,
 template<typename T>
 bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const GatherGeom& g, ScratchArena* arena = nullptr,
 		int epi = EPI_NONE, const Epilogue<T>* E = nullptr, int* mtiles_out = nullptr, const LstmBackwardStep<T>* then = nullptr,
-		bool* then_done = nullptr, const std::function<void(int bf)>* before_launch = nullptr) {
+		bool* then_done = nullptr, const std::function<void(int bf)>* before_launch = nullptr, WgradRider<T>* rider = nullptr) {
 	const bool vec = g.N % GemmCfg<T>::VEC == 0 && g.NS % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
 	const bool divs = g.DA != 1 || g.DB != 1;
 	if (epi != EPI_NONE && (!vec || divs || (reinterpret_cast<uintptr_t>(out) & 15) != 0))
@@ -2268,6 +2339,14 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		 * Their reduction is cut into parts instead; the part blocks come last in the grid and fill the
 		 * chip as the last round of whole tiles drains. */
 		launch(mtiles - rem, (int) std::min<long>(std::min(round_m / rem, nchunks / 4), 16));
+		return true;
+	}
+	if (rider && v.launch_with_wgrad && epi == EPI_NONE && bias == nullptr && then == nullptr && vec && !divs && dyn == 0 &&
+			g.out_sa == 1 && g.out_sb == 1 && g.out_a0 == 0 && g.out_b0 == 0 && g.out_OA == g.OA && g.out_M == g.M) {
+		/* whole tiles only, and a small weight gradient that waits for the same upstream gradient: one launch for both */
+		const GatherLaunch L = { mtiles, tile_rows, mtiles, round_up(mtiles, 8), 0, 1, nchunks, sample_blocks, pos_b, sb_shift };
+		v.launch_with_wgrad(L, ftiles, src, wt, out, g, *rider);
+		rider->done = true;
 		return true;
 	}
 	launch(mtiles, 1);
@@ -2765,8 +2844,23 @@ void conv_forward_static(const ConvShape& s, int N, const T* x, const T* w, cons
 }
 
 template<typename T>
+void conv_weight_gradient_with(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials,
+		const WgradAct<T>* act, ReduceBatch<T>* deferred, const std::function<bool(WgradRider<T>&)>* elsewhere);
+template<typename T>
+bool conv_input_gradient_with(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad, T* wt_dgrad, bool wt_ready,
+		const LstmBackwardStep<T>* then, int og_batch, WgradRider<T>* rider);
+
+template<typename T>
 void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials,
 		const WgradAct<T>* act, ReduceBatch<T>* deferred) {
+	conv_weight_gradient_with<T>(s, N, x, out_grad, wgrad, bgrad, partials, act, deferred, nullptr);
+}
+
+/* `elsewhere`, if given, is offered the kernel launch when it is one that can ride in another launch (WgradRider) and
+ * says whether it ran it; the sums of the slices follow here either way. */
+template<typename T>
+void conv_weight_gradient_with(const ConvShape& s, int N, const T* x, const T* out_grad, T* wgrad, T* bgrad, T* partials,
+		const WgradAct<T>* act, ReduceBatch<T>* deferred, const std::function<bool(WgradRider<T>&)>* elsewhere) {
 	check_sizes(s, N);
 	if (deferred)
 		deferred->count = 0;
@@ -2779,14 +2873,25 @@ void conv_weight_gradient(const ConvShape& s, int N, const T* x, const T* out_gr
 	const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
 	const size_t count = (size_t) g.K * g.F;
 	T* bias_partials = partials + (size_t) p.splits * count;
+	static_assert(WGRAD_MC == 32, "the chunk length gather_with_wgrad_kernel is built with");
+	const bool can_ride = elsewhere != nullptr && std::is_same<T, float>::value && !act && vec && v.bk == 32 && v.bf == 32 &&
+			v.waves == 1 && v.mc == WGRAD_MC;
+	auto run = [&](T* to_w, T* to_b, const WgradSplit& how) {
+		if (can_ride) {
+			WgradRider<T> rider = { x, out_grad, to_w, to_b, g, how, false };
+			if ((*elsewhere)(rider))
+				return;
+		}
+		v.launch(x, out_grad, to_w, to_b, g, how, vec, act);
+	};
 	if (p.splits == 1) {
 		/* one slice: every block owns its tile of the gradient and adds to it directly, no second launch */
 		const WgradSplit direct = { p.ktiles, p.ktiles * p.ftiles, 1, p.chunks_per_split, p.pixel_mode, 1 };
-		v.launch(x, out_grad, wgrad, bgrad, g, direct, vec, act);
+		run(wgrad, bgrad, direct);
 		return;
 	}
 	const WgradSplit split = { p.ktiles, p.ktiles * p.ftiles, p.splits, p.chunks_per_split, p.pixel_mode, 0 };
-	v.launch(x, out_grad, partials, bias_partials, g, split, vec, act);
+	run(partials, bias_partials, split);
 	/* a few thousand outputs cut into many partials: a wavefront per output; else 64 outputs per block, 16-byte loads
 	 * where counts and alignment allow */
 	constexpr int V = 16 / (int) sizeof(T);
@@ -2829,6 +2934,13 @@ void reduce_partials_many(ReduceBatch<T> batch) {
 template<typename T>
 bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad, T* wt_dgrad, bool wt_ready,
 		const LstmBackwardStep<T>* then, int og_batch) {
+	return conv_input_gradient_with<T>(s, N, w, out_grad, in_grad, wt_dgrad, wt_ready, then, og_batch, nullptr);
+}
+
+/* (`rider`: a small weight-gradient launch that may run inside this one, see WgradRider) */
+template<typename T>
+bool conv_input_gradient_with(const ConvShape& s, int N, const T* w, const T* out_grad, T* in_grad, T* wt_dgrad, bool wt_ready,
+		const LstmBackwardStep<T>* then, int og_batch, WgradRider<T>* rider) {
 	check_sizes(s, std::max(N, og_batch));
 	if (then == nullptr && use_strided_classes(s, N)) {
 		std::vector<StridedClass> classes;
@@ -2895,7 +3007,7 @@ bool conv_input_gradient(const ConvShape& s, int N, const T* w, const T* out_gra
 		CATTLE_HIP_CHECK(hipGetLastError());
 	}
 	bool then_done = false;
-	launch_gather<T>(out_grad, wt_dgrad, (const T*) nullptr, in_grad, d, nullptr, EPI_NONE, nullptr, nullptr, then, &then_done);
+	launch_gather<T>(out_grad, wt_dgrad, (const T*) nullptr, in_grad, d, nullptr, EPI_NONE, nullptr, nullptr, then, &then_done, nullptr, rider);
 	return then_done;
 }
 
@@ -2903,8 +3015,16 @@ template<typename T>
 void conv_backward(const ConvShape& s, int N, const T* x, const T* w, const T* out_grad, T* wgrad, T* bgrad,
 		T* in_grad, T* wt_dgrad, bool wt_ready, T* partials, const WgradAct<T>* act, ReduceBatch<T>* deferred) {
 	CATTLE_HIP_REQUIRE(!act || !in_grad || act->dz != nullptr, "the input gradient needs the gradient before the activation");
-	conv_weight_gradient<T>(s, N, x, out_grad, wgrad, bgrad, partials, act, deferred);
-	if (in_grad)
+	/* Without an activation to undo, the two gradients wait for the same upstream gradient only: where the weight gradient
+	 * is a launch of one-wavefront tiles, the input-gradient launch takes its blocks along. */
+	bool in_grad_done = false;
+	const std::function<bool(WgradRider<T>&)> with_input_gradient = [&](WgradRider<T>& rider) {
+		conv_input_gradient_with<T>(s, N, w, out_grad, in_grad, wt_dgrad, wt_ready, nullptr, 0, &rider);
+		in_grad_done = true;
+		return rider.done;
+	};
+	conv_weight_gradient_with<T>(s, N, x, out_grad, wgrad, bgrad, partials, act, deferred, in_grad && !act ? &with_input_gradient : nullptr);
+	if (in_grad && !in_grad_done)
 		conv_input_gradient<T>(s, N, w, act ? (const T*) act->dz : out_grad, in_grad, wt_dgrad, wt_ready, nullptr, 0);
 }
 
