@@ -172,3 +172,34 @@ def test_left_over_tiles_with_several_column_blocks(N, wide_side):
     assert hp.rel_err(out, o_ref, label=label + " y") < 1e-4
     assert hp.rel_err(dx, dx_ref, label=label + " dx") < 1e-4
     assert hp.rel_err(wp.get_grad(), dw_ref) < 1e-4
+
+
+@pytest.mark.parametrize("case", [(256, 256, 10), (128, 4096, 10), (64, 96, 24), (32, 40, 5)], ids=lambda c: "x".join(str(v) for v in c))
+def test_weight_gradient_riding_in_the_input_gradient_launch(case):
+    """A last layer's weight gradient (one-wavefront tiles) runs inside its input-gradient launch when both wait for the
+    same upstream gradient only. Riding or launched alone (the same layer as a network's first layer, which has no input
+    gradient), its slices and their order are the same: the gradients must agree bit for bit, and with the oracle."""
+    N, K, F = case
+    dtype = np.float32
+    gen = hp.rng(1600 + K + F)
+    x = hp.normal(gen, (N, K), dtype)
+    w = hp.normal(gen, (K, F), dtype, std=1.0 / np.sqrt(K))
+    b = hp.normal(gen, (1, F), dtype)
+    g = hp.normal(gen, (N, F), dtype)
+    grads = []
+    for first_layer in (False, True):
+        dense = ch.DenseKernelLayer(dtype, (K,), F)
+        dense.set_input_layer(first_layer)
+        wp, bp = dense.get_params()
+        wp.set_values(w)
+        bp.set_values(b)
+        dense.pass_forward(ch.DeviceTensor.from_host(x), True)
+        dx = dense.pass_back(ch.DeviceTensor.from_host(g))
+        grads.append((wp.get_grad().copy(), bp.get_grad().copy(), None if first_layer else dx.to_host()))
+    assert np.array_equal(grads[0][0], grads[1][0])
+    assert np.array_equal(grads[0][1], grads[1][1])
+    x64, w64, g64 = (np.asarray(a, np.float64) for a in (x, w, g))
+    dx_ref, dw_ref, db_ref = oracle.dense_backward(x64, w64, g64)
+    assert hp.rel_err(grads[0][2].reshape(dx_ref.shape), dx_ref, label="riding weight gradient %s dx" % "x".join(str(v) for v in case)) < 1e-4
+    assert hp.rel_err(grads[0][0], dw_ref) < 1e-4
+    assert hp.rel_err(grads[0][1], db_ref) < 1e-4
