@@ -1574,7 +1574,8 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 	/* Reduction steps per batch of loads: 64 operand registers in fp32, 48 in fp64 (a block of sixteen wavefronts has 128
 	 * registers per lane; more spilled), 32 in the blocks of four wavefronts, of which a CU must hold four (measured: at
 	 * 136 registers it held three, and 1024 tiles took a second round) */
-	constexpr int B = sizeof(T) == 4 ? (WAVES == 4 ? 16 : 32) : (WAVES == 4 ? 8 : 12);
+	/* (the LSTM tail keeps nine preloaded values per lane through the loop: shorter batches make room for them) */
+	constexpr int B = sizeof(T) == 4 ? (WAVES == 4 ? 16 : (TAIL == WS_LSTM_BACKWARD ? 24 : 32)) : (WAVES == 4 ? 8 : 12);
 	__shared__ T red[WAVES * TL * TL];
 
 	const int mtile = xcd_tile(blockIdx.x, mtiles);
@@ -1602,6 +1603,17 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 	const int s_begin = wave * per, s_end = min(total, s_begin + per);
 	const unsigned astep = (unsigned) (plane * KS) * (unsigned) sizeof(T), bstep = (unsigned) (taps * KS * g.ldw) * (unsigned) sizeof(T);   /* bytes */
 
+	/* LSTM tail: what the backward step of this thread's first output element reads is fetched now and used after the
+	 * reduction, so that the kernel does not end with a round trip to memory */
+	const int o_first = tid;
+	const int mo_first = m0 + o_first % TL, f_first = f0 + o_first / TL;
+	bool preloaded = false;
+	LstmBackwardInputs<T> pre = {};
+	if constexpr (TAIL == WS_LSTM_BACKWARD) {
+		preloaded = lstm_backward_can_preload(then);
+		const bool mine = o_first < TL * TL && mo_first < g.M && f_first < g.F;
+		pre = lstm_backward_load<T>(then, preloaded && mine ? (unsigned) mo_first + (unsigned) g.M * (unsigned) f_first : 0u, true);
+	}
 	/* one accumulator: a SIMD's matrix pipe runs one instruction at a time, so a chain of dependent instructions costs
 	 * nothing, and a second accumulator's registers are worth more as loads in flight */
 	typename MF::acc_t acc;
@@ -1689,10 +1701,16 @@ void wave_split_gemm_kernel(const T* __restrict__ src, const T* __restrict__ wt,
 		if (mo >= g.M || f >= g.F)
 			continue;
 		if constexpr (TAIL == WS_LSTM_BACKWARD) {
-			if (lstm_standard_acts(then.a))
-				lstm_backward_element<T, true>(then, (unsigned) mo + (unsigned) g.M * (unsigned) f, true, v);
+			const unsigned e = (unsigned) mo + (unsigned) g.M * (unsigned) f;
+			if (preloaded && o == o_first) {
+				if (lstm_standard_acts(then.a))
+					lstm_backward_finish<T, true>(then, e, true, v, pre);
+				else
+					lstm_backward_finish<T, false>(then, e, true, v, pre);
+			} else if (lstm_standard_acts(then.a))
+				lstm_backward_element<T, true>(then, e, true, v);
 			else
-				lstm_backward_element<T, false>(then, (unsigned) mo + (unsigned) g.M * (unsigned) f, true, v);
+				lstm_backward_element<T, false>(then, e, true, v);
 		} else {
 			v += bias ? bias[f] : (T) 0;
 			if constexpr (TAIL == WS_ACT) {

@@ -176,6 +176,60 @@ __device__ __forceinline__ void lstm_forward_element(const LstmForwardStep<T>& A
 	lstm_forward_store<T>(A, e, lstm_forward_compute<T, STD>(A, in, has_zh, zh4));
 }
 
+/* What the backward step of element e reads, for the usual cell (no kept pre-activation values, no multiplicative
+ * integration): a kernel that knows its elements early can fetch these before its own work and run the step on them later
+ * (lstm_backward_finish), instead of paying a round trip to memory at its end. */
+template<typename T>
+struct LstmBackwardInputs {
+	T og, gates[4], as, sgrad, state, prev;
+};
+template<typename T>
+__device__ __forceinline__ bool lstm_backward_can_preload(const LstmBackwardStep<T>& A) {
+	return A.z == nullptr && A.zx_fwd == nullptr;
+}
+template<typename T>
+__device__ __forceinline__ LstmBackwardInputs<T> lstm_backward_load(const LstmBackwardStep<T>& A, unsigned e, bool has_dh) {
+	const unsigned N = (unsigned) A.N, P = (unsigned) A.P;
+	const unsigned rest = e / N, n = e - rest * N;
+	LstmBackwardInputs<T> in;
+	in.og = A.out_grad ? lstm_ld<T>(A.out_grad, seq_offset(n, rest, A.N, A.og_T, A.og_t)) : (T) 0;
+	#pragma unroll
+	for (int g = 0; g < 4; ++g)
+		in.gates[g] = lstm_ld<T>(A.gates, (unsigned) g * P + e);
+	in.as = lstm_ld<T>(A.act_state, e);
+	in.sgrad = has_dh ? lstm_ld<T>(A.state_grad, e) : (T) 0;
+	in.state = lstm_ld<T>(A.state, e);
+	in.prev = A.prev_state ? lstm_ld<T>(A.prev_state, e) : (T) 0;
+	return in;
+}
+/* The step itself on preloaded inputs: the same arithmetic, in the same order, as lstm_backward_element below. */
+template<typename T, bool STD = false>
+__device__ __forceinline__ void lstm_backward_finish(const LstmBackwardStep<T>& A, unsigned e, bool has_dh, T dh,
+		const LstmBackwardInputs<T>& in) {
+	const unsigned N = (unsigned) A.N, P = (unsigned) A.P;
+	const unsigned slab_rows = P / N;
+	const unsigned rest = e / N, n = e - rest * N;
+	T hg = has_dh ? dh : (T) 0;
+	if (A.out_grad)
+		hg += in.og;
+	const T f = in.gates[0], w = in.gates[1], c = in.gates[2], r = in.gates[3];
+	const T as = in.as;
+	const T sg = in.sgrad + lstm_act_b<T, STD, 3>(A.a, in.state, as, r * hg);
+	T d[4];
+	d[3] = lstm_act_b<T, STD, 4>(A.a, (T) 0, r, as * hg);
+	d[2] = lstm_act_b<T, STD, 2>(A.a, (T) 0, c, w * sg);
+	d[1] = lstm_act_b<T, STD, 1>(A.a, (T) 0, w, c * sg);
+	d[0] = lstm_act_b<T, STD, 0>(A.a, (T) 0, f, in.prev * sg);
+	lstm_st<T>(A.state_grad, e, sg * f);
+	#pragma unroll
+	for (int g = 0; g < 4; ++g) {
+		if (A.dzx_all)
+			lstm_st<T>(A.dzx_all, seq_offset(n, rest + g * slab_rows, A.N, A.x_T, A.x_t), d[g]);
+		if (A.dzh_all)
+			lstm_st<T>(A.dzh_all, seq_offset(n, rest + g * slab_rows, A.N, A.h_T, A.h_t), A.prev_state ? d[g] : (T) 0);
+	}
+}
+
 /* Backward step of element e. dh: the gradient of the element's hidden output that came back through the next
  * step's output-side kernels; has_dh is false at the last time step, where there is none and the state gradient
  * starts at zero (:422-425). */
