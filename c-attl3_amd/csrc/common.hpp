@@ -123,6 +123,12 @@ template<typename T> struct WgradAct {
 	T* dz;
 	int kind;
 	T p;
+	/* pool_inds != null: the gradient handed to the weight-gradient launch and `y` are the tensors behind a max pool
+	 * whose windows of 2^pool_sh_a x 2^pool_sh_b (height x width, stride = receptor) tile the kernel layer's output, and
+	 * pool_inds is the pool's arg-max cache; dz must be null (the full-size gradient is never formed in memory), the
+	 * launch needs 16-byte loads, and kind may be -1 for no activation. */
+	const unsigned* pool_inds;
+	int pool_sh_a, pool_sh_b;
 };
 /* Partial sums that wait to be added to their gradients: entry e is `splits` matrices of `count` values each, one
  * after the other at `partials`, to be added to dst in the fixed order of reduce_partials_many (first_block is filled in

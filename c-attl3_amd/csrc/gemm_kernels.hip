@@ -886,10 +886,19 @@ struct WgradSplit {
  * grid = tiles * splits blocks (1-D). Bias rows are dealt out over the k tiles (row f belongs to the
  * block with f % ktiles == k-tile index) so that every block does the same amount of extra work.
  * ---------------------------------------------------------------------------------------------- */
-template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, bool ACTG>
+/* GMODE: where the G operand comes from. 0: `og` is it. 1 (WgradAct): og is the gradient behind a rectifier whose coded
+ * outputs are act_y; the derivative is applied as a chunk goes into LDS, and the blocks of the first k tile write the
+ * product to act_dz (if given). 2: og is the gradient behind a rectifier and a max pool whose windows tile the output
+ * (2^pool_sh_a x 2^pool_sh_b, stride = receptor): og and act_y are pooled tensors, pool_inds the pool's arg-max cache in
+ * the layout of MaxPoolLayer; an element of G is the pooled gradient times the derivative where the arg-max names its
+ * position in the window and zero elsewhere, formed as the chunk goes into LDS - the full-size gradient is never
+ * written (for layers whose input gradient nobody needs). */
+template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC, int GMODE>
 __device__ __forceinline__ void wgrad_body(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
 		T* __restrict__ bias_partials, const GatherGeom& g, const WgradSplit& plan, const T* __restrict__ act_y,
-		T* __restrict__ act_dz, T act_p0, T act_p1, int bid) {
+		T* __restrict__ act_dz, T act_p0, T act_p1, int bid, const unsigned* __restrict__ pool_inds = nullptr, int pool_sh_a = 0,
+		int pool_sh_b = 0) {
+	constexpr bool ACTG = GMODE != 0;
 	/* (the activation's tensors as parameters of their own: pointers inside a structure are not known to point to global
 	 * memory, and flat loads count against the LDS counter as well, see vec_load_global) */
 	typedef Mfma<T> MF;
@@ -973,6 +982,8 @@ __device__ __forceinline__ void wgrad_body(const T* __restrict__ src, const T* _
 	/* ACTG: the activation outputs beside the gradient values, and where both came from; the derivative is applied
 	 * when the chunk is stored to LDS, a chunk after its loads were issued, so that nothing waits for them here */
 	T yreg[ACTG ? GSLOTS : 1][VEC];
+	unsigned ireg[GMODE == 2 ? GSLOTS : 1][VEC];        /* GMODE 2: the windows' arg-max positions */
+	unsigned pos_loaded = 0;                            /* ... and the position of the loaded rows in their window */
 	int gm_loaded = 0;
 	bool gvalid_loaded = false;
 
@@ -994,23 +1005,36 @@ __device__ __forceinline__ void wgrad_body(const T* __restrict__ src, const T* _
 					xreg[s][v] = (T) 0;
 			}
 		}
+		/* GMODE 2: the rows' window (ap, bp) of the pooled tensors, whose rows are mp = n + N (ap + OAp bp) */
+		const int ap = a >> pool_sh_a, bp = b >> pool_sh_b, oap = g.OA >> pool_sh_a;
+		const size_t mp = (size_t) n + (size_t) g.N * (ap + oap * bp), pooled_rows = (size_t) g.M >> (pool_sh_a + pool_sh_b);
 		#pragma unroll
 		for (int s = 0; s < GSLOTS; ++s) {
 			const int row = row0 + s * RP;
 			const int f = f0 + row;
 			if (mvalid && f < g.F && (BF % RP == 0 || row < BF)) {
-				vec_load<T, VEC>(greg[s], og + ((size_t) m + (size_t) g.M * f));
-				if constexpr (ACTG)
-					vec_load<T, VEC>(yreg[s], act_y + ((size_t) m + (size_t) g.M * f));
+				if constexpr (GMODE == 2) {
+					vec_load<T, VEC>(greg[s], og + (mp + pooled_rows * f));
+					vec_load<T, VEC>(yreg[s], act_y + (mp + pooled_rows * f));
+					vec_load<unsigned, VEC>(ireg[s], pool_inds + ((size_t) (bp * oap + ap) * ((size_t) g.F * g.N) + (size_t) f * g.N + n));
+				} else {
+					vec_load<T, VEC>(greg[s], og + ((size_t) m + (size_t) g.M * f));
+					if constexpr (ACTG)
+						vec_load<T, VEC>(yreg[s], act_y + ((size_t) m + (size_t) g.M * f));
+				}
 			} else {
 				#pragma unroll
 				for (int v = 0; v < VEC; ++v) {
 					greg[s][v] = (T) 0;
 					if constexpr (ACTG)
 						yreg[s][v] = (T) 0;
+					if constexpr (GMODE == 2)
+						ireg[s][v] = 0xffffffffu;
 				}
 			}
 		}
+		if constexpr (GMODE == 2)
+			pos_loaded = (unsigned) (((b - (bp << pool_sh_b)) << pool_sh_a) + (a - (ap << pool_sh_a)));
 		gm_loaded = m;
 		gvalid_loaded = mvalid;
 		if (pixel_mode) {
@@ -1054,11 +1078,14 @@ __device__ __forceinline__ void wgrad_body(const T* __restrict__ src, const T* _
 					#pragma unroll
 					for (int v = 0; v < VEC; ++v) {
 						const T slope = sign_bit(yreg[s][v]) ? act_p1 * yreg[s][v] + act_p0 : (T) 1;
-						dzv[v] = live ? slope * greg[s][v] : (T) 0;
+						if constexpr (GMODE == 2)
+							dzv[v] = live && ireg[s][v] == pos_loaded ? slope * greg[s][v] : (T) 0;
+						else
+							dzv[v] = live ? slope * greg[s][v] : (T) 0;
 					}
 					vec_store<T, VEC>(&Gs[row0 + s * RP][col * VEC], dzv);
 					/* each element of G belongs to one (slice, f tile): the blocks of the first k tile write it */
-					if (act_dz != nullptr && kt == 0 && live)
+					if (GMODE == 1 && act_dz != nullptr && kt == 0 && live)
 						vec_store<T, VEC>(act_dz + ((size_t) gm_loaded + (size_t) g.M * (f0 + row0 + s * RP)), dzv);
 				}
 			}
@@ -1205,8 +1232,18 @@ __global__ __launch_bounds__(64 * WAVES_K * WAVES_F, MIN_WAVES)      /* MIN_WAVE
 void wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
 		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan, const T* __restrict__ act_y,
 		T* __restrict__ act_dz, T act_p0, T act_p1) {
-	wgrad_body<T, WAVES_K, WAVES_F, WT_K, WT_F, MC, VEC, ACTG>(src, og, partials, bias_partials, g, plan, act_y, act_dz, act_p0, act_p1,
+	wgrad_body<T, WAVES_K, WAVES_F, WT_K, WT_F, MC, VEC, ACTG ? 1 : 0>(src, og, partials, bias_partials, g, plan, act_y, act_dz, act_p0, act_p1,
 			(int) blockIdx.x);
+}
+
+/* The weight gradient of a layer behind a rectifier and a max pool, from the pooled gradient (wgrad_body, GMODE 2). */
+template<typename T, int WAVES_K, int WAVES_F, int WT_K, int WT_F, int MC, int VEC>
+__global__ __launch_bounds__(64 * WAVES_K * WAVES_F)
+void wgrad_pooled_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
+		T* __restrict__ bias_partials, const GatherGeom g, const WgradSplit plan, const T* __restrict__ act_y, T act_p0, T act_p1,
+		const unsigned* __restrict__ pool_inds, int pool_sh_a, int pool_sh_b) {
+	wgrad_body<T, WAVES_K, WAVES_F, WT_K, WT_F, MC, VEC, 2>(src, og, partials, bias_partials, g, plan, act_y, (T*) nullptr, act_p0, act_p1,
+			(int) blockIdx.x, pool_inds, pool_sh_a, pool_sh_b);
 }
 
 /* A layer's input gradient and its weight gradient in one launch, for layers whose two launches are a few microseconds
@@ -1228,7 +1265,7 @@ void gather_with_wgrad_kernel(const T* __restrict__ src, const T* __restrict__ w
 		const int bid = ((int) blockIdx.x - gather_x) + ((int) gridDim.x - gather_x) * (int) blockIdx.y;
 		if (bid >= (w_plan.tiles * w_plan.splits + 7) / 8 * 8)
 			return;
-		wgrad_body<T, 1, 1, 32, 32, 32, VEC, false>(w_src, w_og, w_partials, w_bias_partials, w_g, w_plan,
+		wgrad_body<T, 1, 1, 32, 32, 32, VEC, 0>(w_src, w_og, w_partials, w_bias_partials, w_g, w_plan,
 				(const T*) nullptr, (T*) nullptr, (T) 0, (T) 0, bid);
 	}
 }
@@ -2564,12 +2601,18 @@ void launch_wgrad_variant(const T* x, const T* og, T* partials, T* bias_partials
 	dim3 block(64 * WK * WF), grid((unsigned) round_up(plan.tiles * plan.splits, 8));
 	/* derivative on the negative side: p0 + p1 * y */
 	T p0 = (T) 0, p1 = (T) 0;
-	if (act) {
+	if (act && act->pool_inds && act->kind < 0) {
+		p0 = (T) 1;             /* no activation behind the pool: slope one on either side */
+	} else if (act) {
 		CATTLE_HIP_REQUIRE(act_sign_coded(act->kind) && act->p >= (T) 0, "only a rectifier can be undone while the gradient is loaded");
 		p0 = act->kind == ACT_RELU ? (T) 0 : act->p;
 		p1 = act->kind == ACT_ELU ? (T) 1 : (T) 0;
 	}
-	if (vec) {
+	if (act && act->pool_inds) {
+		CATTLE_HIP_REQUIRE(vec && act->dz == nullptr, "the weight gradient from a pooled gradient needs 16-byte loads and forms no full-size gradient");
+		wgrad_pooled_kernel<T, WK, WF, TK, TF, MC, VEC><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan, act->y, p0, p1,
+				act->pool_inds, act->pool_sh_a, act->pool_sh_b);
+	} else if (vec) {
 		if (act)        /* the extra operand registers do not fit a register cap: MIN_WAVES 1 */
 			wgrad_kernel<T, WK, WF, TK, TF, MC, VEC, 1, true><<<grid, block, 0, stream()>>>(x, og, partials, bias_partials, g, plan, act->y, act->dz, p0, p1);
 		else
@@ -2886,7 +2929,8 @@ void conv_weight_gradient_with(const ConvShape& s, int N, const T* x, const T* o
 	/* split-M partials, then a fixed-order reduction that accumulates */
 	const bool vec = N % GemmCfg<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
 			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0 &&
-			(!act || ((reinterpret_cast<uintptr_t>(act->y) & 15) == 0 && (reinterpret_cast<uintptr_t>(act->dz) & 15) == 0));
+			(!act || ((reinterpret_cast<uintptr_t>(act->y) & 15) == 0 && (reinterpret_cast<uintptr_t>(act->dz) & 15) == 0 &&
+					(reinterpret_cast<uintptr_t>(act->pool_inds) & 15) == 0));
 	const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N, vec);
 	const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
 	const size_t count = (size_t) g.K * g.F;

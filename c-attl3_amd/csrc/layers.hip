@@ -1277,6 +1277,8 @@ struct FusedLayer : LayerBase {
 			chain_backward<T>(chain_shape(true), n, g, nullptr, needs_pre() ? nullptr : y_cache, needs_pre() ? y_cache : nullptr, dz);
 		} else if (mode == MODE_POOL) {
 			CATTLE_HIP_REQUIRE(pool->inds_count == N * pool->out_volume(), "pass_back without cached max indices");
+			if (pooled_weight_gradient(g, n, in_grad))
+				return;
 			chain_backward<T>(chain_shape(true), n, g, (const unsigned*) pool->inds.p, y_cache, needs_pre() ? (const T*) pre_buf.p : nullptr, dz);
 		} else {
 			if (pool) {
@@ -1288,7 +1290,7 @@ struct FusedLayer : LayerBase {
 				/* a rectifier, whose derivative the sign bit of the coded output names: applied by the weight-gradient
 				 * launch while it loads the gradient, which also leaves dz behind for the input-gradient launch - no
 				 * pass of its own */
-				const WgradAct<T> through = { y_cache, in_grad ? dz : nullptr, act->kind, (T) act->p };
+				const WgradAct<T> through = { y_cache, in_grad ? dz : nullptr, act->kind, (T) act->p, nullptr, 0, 0 };
 				conv->backward_through(g, N, in_grad, &through);
 				return;
 			}
@@ -1298,6 +1300,29 @@ struct FusedLayer : LayerBase {
 	}
 	bool needs_pre() const {
 		return act && !act_backward_from_output(act->kind, (double) act->p);
+	}
+	/* MODE_POOL with max pooling, nobody needing the input gradient (a network's first layer), no activation or a
+	 * rectifier, windows whose sides are powers of two, 16-byte loads: the weight-gradient launch forms the gradient
+	 * of the kernel layer's output from the pooled gradient, the arg-max cache and the coded outputs as it loads its
+	 * operand, and the pass over the full-size tensor that scatters it (chain_backward_kernel) does not run. */
+	bool pooled_weight_gradient(const T* g, int n, void* in_grad) {
+		auto log2_exact = [](int v) {
+			int s = 0;
+			while ((1 << s) < v)
+				++s;
+			return (1 << s) == v ? s : -1;
+		};
+		const PoolShape& ps = pool->shape;
+		const int sh_a = log2_exact(ps.RH), sh_b = log2_exact(ps.RW);
+		constexpr int V = 16 / (int) sizeof(T);
+		auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+		if (in_grad != nullptr || sh_a < 0 || sh_b < 0 || n % V != 0 || !aligned(g) || !aligned(y_cache) || !aligned(pool->inds.p))
+			return false;
+		if (act && !(act_sign_coded(act->kind) && act->p >= 0))
+			return false;
+		const WgradAct<T> through = { y_cache, nullptr, act ? act->kind : -1, act ? (T) act->p : (T) 0, (const unsigned*) pool->inds.p, sh_a, sh_b };
+		conv->backward_through(g, (size_t) n, nullptr, &through);
+		return true;
 	}
 	void empty_cache() override {
 		LayerBase::empty_cache();

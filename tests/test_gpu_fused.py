@@ -566,6 +566,48 @@ def test_fused_input_layer_skips_the_input_gradient():
     assert np.array_equal(members["conv"].get_params()[0].get_grad(), grads["dw"])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act", [("relu", 0.0), ("leaky_relu", 0.125), ("elu", 0.5), None, ("tanh", 0.0)])
+@pytest.mark.parametrize("window", [(2, 2), (4, 2), (1, 2), (3, 3)])
+def test_first_layer_weight_gradient_from_the_pooled_gradient(window, act, dtype):
+    """A fused first layer (nobody needs its input gradient) with a rectifier or no activation and a max pool whose window
+    sides are powers of two forms the gradient of the convolution output inside the weight-gradient launch, from the pooled
+    gradient, the arg-max cache and the coded outputs; the pass that scatters it does not run. The gradients must equal, bit
+    for bit, those of the same layer when it is not the first (where that pass runs), and agree with the oracle's chain.
+    Other activations and windows (3 x 3) take the usual path either way."""
+    prh, prw = window
+    N, H, W, C, F = 16, 12, 12, 3, 10
+    pool = ("max", prh, prw, prh, prw)
+    gen = hp.rng(77 + prh * 8 + prw)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (9 * C, F), dtype, std=0.3)
+    b = hp.uniform(gen, (1, F), -0.5, 0.5, dtype)
+    g = hp.normal(gen, (N, H // prh, W // prw, F), dtype)
+    runs = []
+    for first in (False, True):
+        fused, members, kdims = _build(dtype, N, H, W, C, F, conv=GEOM_3X3, act=act, pool=pool)
+        fused.set_input_layer(first)
+        out, dx, mode = _run_fused(fused, members, x, w, b, g)
+        assert mode == "pool" or window == (3, 3)
+        assert (dx is None) == first or mode == "unfused"
+        wp, bp = members["conv"].get_params()
+        runs.append((wp.get_grad().copy(), bp.get_grad().copy(), members["pool"].max_indices(N), out))
+    assert np.array_equal(runs[0][0], runs[1][0])
+    assert np.array_equal(runs[0][1], runs[1][1])
+    assert np.array_equal(runs[0][2], runs[1][2])
+    dw, db, dev_inds, out = runs[1]
+    chain = Chain(GEOM_3X3, act=act, pool=pool)
+    x64, w64, b64 = (np.asarray(a, np.float64) for a in (x, w, b))
+    chain.forward(x64, w64, b64)
+    assert _compare_selections(chain, dev_inds, dtype, pool) < 1e-3
+    ref = chain.backward(x64, w64, np.asarray(g, np.float64), inds=dev_inds,
+                         pre_act=_pre_act_at_device_sides(chain, out, dev_inds, dtype))
+    tol = TOL[np.dtype(dtype)]
+    label = "first layer %dx%d %s %s" % (prh, prw, act[0] if act else "-", np.dtype(dtype).name)
+    assert hp.rel_err(dw, ref["dw"], label=label + " dw") < tol
+    assert hp.rel_err(db, ref["db"].reshape(1, -1), label=label + " db") < tol
+
+
 # ---- a seeded sweep of fused groups over geometries nobody chose by hand ------------------------------------------------
 
 def _sweep_cases(count, seed):
