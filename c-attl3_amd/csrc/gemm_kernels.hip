@@ -626,8 +626,11 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 		/* Pre-activation values of a group of output columns go through LDS (the operand buffers are free now), so
 		 * that the threads can be dealt out over (column, window, sample): a window's positions lie in different
 		 * lanes and waves. A pass stages, for one accumulator block i, the RG accumulator rows of group q of every
-		 * wave: FP = WAVES_F * RG columns x BM rows. */
-		constexpr int RG = std::is_same<T, float>::value ? 8 : 4, GROUPS = TL / RG, FP = WAVES_F * RG, LROW = BM + 4;
+		 * wave: FP = WAVES_F * RG columns x BM rows, as many as the buffers hold (every barrier between passes is a
+		 * stall of the whole block). */
+		constexpr int LROW = BM + 4, ROOM = 2 * KC * LDA / (WAVES_F * LROW), RG_MIN = std::is_same<T, float>::value ? 8 : 4;
+		constexpr int RG = ROOM >= TL ? TL : ROOM >= TL / 2 ? TL / 2 : RG_MIN, GROUPS = TL / RG, FP = WAVES_F * RG;
+		constexpr int REGS_PER_GROUP = MF::NACC / GROUPS;
 		static_assert(FP * LROW <= 2 * KC * LDA, "the staging tile of the pooling epilogue reuses the A operand buffers");
 		T* const stage = &As[0][0][0];
 		const int SB = 1 << sb_shift, P = BM >> sb_shift, pa = P / L.pos_b;
@@ -635,6 +638,28 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 		const int strip = tile / L.tile_rows, trow = tile - strip * L.tile_rows;
 		const int ab = trow / L.sample_blocks, nb = trow - ab * L.sample_blocks;
 		const int a_p0 = ab * wa_n, b_p0 = strip * (L.pos_b / E.prw);
+		/* What an output's place asks of index arithmetic: the window's first value in a staged column, and the element
+		 * offsets of column 0 in the pooled tensors, the arg-max cache and the full-size tensor. */
+		struct Spot {
+			int col;
+			size_t pooled, ind, full;
+		};
+		const auto spot = [&](int s_i, int w) {
+			const int wb = w / wa_n, wa = w - wb * wa_n;
+			const int n = (nb << sb_shift) + s_i, a_p = a_p0 + wa, b_p = b_p0 + wb;
+			return Spot { s_i + (((wa * E.prh) + pa * (wb * E.prw)) << sb_shift), (size_t) n + (size_t) g.N * (a_p + (size_t) E.OHp * b_p),
+					((size_t) b_p * E.OHp + a_p) * ((size_t) g.F * g.N) + n,
+					(size_t) n + (size_t) g.N * (a_p * E.prh + (size_t) g.OA * (b_p * E.prw)) };
+		};
+		/* The threads walk (sample, window, column), samples first. When the windows of a pass divide the threads of a
+		 * sample block evenly, a thread keeps its sample and window through every pass and only its column moves on. */
+		const int tps = THREADS >> sb_shift, outputs = (FP * W * SB + THREADS - 1) / THREADS;
+		const bool fixed_spot = tps % W == 0;
+		const int fl0 = (tid >> sb_shift) / W, fl_step = tps / W;
+		Spot sp = spot(tid & (SB - 1), (tid >> sb_shift) % W);
+		const int kstep = pa << sb_shift;
+		const bool two_by_two = E.prh == 2 && E.prw == 2;
+		const size_t pooled_plane = (size_t) g.N * E.OHp * E.OWp;
 		act_dispatch(E.kind, [&](auto kc) {
 			constexpr int KIND = decltype(kc)::value;
 			#pragma unroll
@@ -644,7 +669,7 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 					__syncthreads();
 					#pragma unroll
 					for (int r = 0; r < MF::NACC; ++r) {
-						if ((std::is_same<T, float>::value ? r / 4 : r) != q)
+						if (r / REGS_PER_GROUP != q)
 							continue;
 						const int arow = acc_row<T>(r, lk);
 						const T bv = bias_s[wf * WT_F + FB * arow + i];
@@ -658,49 +683,66 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 							vec_store<T, VS>(dst + j0, *reinterpret_cast<T (*)[VS]>(&v[j0]));
 					}
 					__syncthreads();
-					for (int it = tid; it < FP * W * SB; it += THREADS) {
-						const int s_i = it & (SB - 1), t2 = it >> sb_shift;
-						const int fl = t2 / W, w = t2 - fl * W;
+					for (int pass = 0; pass < outputs; ++pass) {
+						int fl;
+						if (fixed_spot) {
+							fl = fl0 + pass * fl_step;
+							if (fl >= FP)
+								break;
+						} else {
+							const int it = tid + pass * THREADS;
+							if (it >= FP * W * SB)
+								break;
+							const int t2 = it >> sb_shift;
+							fl = t2 / W;
+							sp = spot(it & (SB - 1), t2 - fl * W);
+						}
 						const int f = f0 + (fl / RG) * WT_F + FB * (RG * q + fl % RG) + i;
 						if (f >= g.F)
 							continue;
-						const int wb = w / wa_n, wa = w - wb * wa_n;
-						const T* col = stage + fl * LROW + s_i;
+						const T* col = stage + fl * LROW + sp.col;
 						if (E.pool_mean) {
 							/* the mean of the window, summed width-major / height-minor as the layer of its own does
 							 * (MeanPoolLayer.hpp:35-41); what the backward pass needs goes out at every position */
-							const int n = (nb << sb_shift) + s_i, a_p = a_p0 + wa, b_p = b_p0 + wb;
 							T sum = (T) 0;
 							for (int k = 0; k < E.prw; ++k)
 								for (int l = 0; l < E.prh; ++l) {
-									const T z = col[((wa * E.prh + l) + pa * (wb * E.prw + k)) << sb_shift];
+									const T z = col[k * kstep + l * SB];
 									const T y = act_f_coded<T, KIND>(z, E.p);
 									sum += y;
 									if (E.pre)
-										E.pre[(size_t) n + (size_t) g.N * ((a_p * E.prh + l) + (size_t) g.OA * ((b_p * E.prw + k) + (size_t) g.OB * f))] =
-												E.keep_input ? z : y;
+										E.pre[sp.full + (size_t) g.N * (l + (size_t) g.OA * (k + (size_t) g.OB * f))] = E.keep_input ? z : y;
 								}
-							out[(size_t) n + (size_t) g.N * (a_p + (size_t) E.OHp * (b_p + (size_t) E.OWp * f))] = sum / (T) (E.prh * E.prw);
+							out[sp.pooled + pooled_plane * f] = sum / (T) (E.prh * E.prw);
 							continue;
 						}
 						/* strict '>' from lowest(), width-major / height-minor scan (MaxPoolLayer.hpp:45-56) */
-						T best = std::numeric_limits<T>::lowest(), best_pre = col[((wa * E.prh) + pa * (wb * E.prw)) << sb_shift];
+						T best = std::numeric_limits<T>::lowest(), best_pre = col[0];
 						unsigned bi = 0;
-						for (int k = 0; k < E.prw; ++k)
-							for (int l = 0; l < E.prh; ++l) {
-								const T z = col[((wa * E.prh + l) + pa * (wb * E.prw + k)) << sb_shift];
-								const T y = act_f_coded<T, KIND>(z, E.p);
-								if (y > best) {
-									best = y;
-									best_pre = z;
-									bi = (unsigned) (k * E.prh + l);
-								}
+						const auto consider = [&](T z, unsigned at) {
+							const T y = act_f_coded<T, KIND>(z, E.p);
+							if (y > best) {
+								best = y;
+								best_pre = z;
+								bi = at;
 							}
-						const int n = (nb << sb_shift) + s_i, a_p = a_p0 + wa, b_p = b_p0 + wb;
-						out[(size_t) n + (size_t) g.N * (a_p + (size_t) E.OHp * (b_p + (size_t) E.OWp * f))] = best;
-						E.inds[((size_t) b_p * E.OHp + a_p) * ((size_t) g.F * g.N) + (size_t) f * g.N + n] = bi;
+						};
+						if (two_by_two) {
+							/* the usual window: its four values fetched together, then scanned in the same order */
+							const T z0 = best_pre, z1 = col[SB], z2 = col[kstep], z3 = col[kstep + SB];
+							consider(z0, 0u);
+							consider(z1, 1u);
+							consider(z2, 2u);
+							consider(z3, 3u);
+						} else {
+							for (int k = 0; k < E.prw; ++k)
+								for (int l = 0; l < E.prh; ++l)
+									consider(col[k * kstep + l * SB], (unsigned) (k * E.prh + l));
+						}
+						out[sp.pooled + pooled_plane * f] = best;
+						E.inds[sp.ind + (size_t) f * g.N] = bi;
 						if (E.pre)
-							E.pre[(size_t) n + (size_t) g.N * (a_p + (size_t) E.OHp * (b_p + (size_t) E.OWp * f))] = best_pre;
+							E.pre[sp.pooled + pooled_plane * f] = best_pre;
 					}
 				}
 			}
