@@ -1532,14 +1532,13 @@ void* g_scratch_ptr[MAX_DEVICES] = { nullptr };
  * wave order: the summation order depends on the geometry only.
  * ---------------------------------------------------------------------------------------------- */
 constexpr int FEW_COLUMNS = 4;
-template<typename T, int VEC, bool DIVS>
-__global__ __launch_bounds__(256)
-void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom g) {
+template<typename T, int VEC, bool DIVS, int UNROLL>
+__device__ __forceinline__ void few_columns_body(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
+		T* __restrict__ out, const GatherGeom& g, int block) {
 	constexpr int WAVES = 4, ROWS = 64 * VEC;
 	const int lane = threadIdx.x % 64;
 	const int wave = __builtin_amdgcn_readfirstlane((int) threadIdx.x / 64);
-	const int m = (int) blockIdx.x * ROWS + lane * VEC;
+	const int m = block * ROWS + lane * VEC;
 	const bool mvalid = m < g.M;             /* whole vectors: M is a multiple of VEC */
 	int n, ya0, yb0;
 	{
@@ -1550,8 +1549,6 @@ void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ 
 		yb0 = b * g.SB + g.PB;
 	}
 	const int plane = g.NS * g.LH * g.LW;
-	const int per = (g.LC + WAVES - 1) / WAVES;
-	const int c0 = wave * per, c1 = min(g.LC, c0 + per);
 	const int taps = g.R * g.S;
 	T acc[FEW_COLUMNS][VEC];
 	#pragma unroll
@@ -1559,6 +1556,10 @@ void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ 
 		#pragma unroll
 		for (int i = 0; i < VEC; ++i)
 			acc[c][i] = (T) 0;
+	/* the source channels are dealt over the waves; a tap that reaches none of a wavefront's rows (zero padding, or a
+	 * stride that does not divide: its rows share an output position or a few) is skipped whole */
+	const int per = (g.LC + WAVES - 1) / WAVES;
+	const int c0 = wave * per, c1 = min(g.LC, c0 + per);
 	for (int sb = 0; sb < g.S; ++sb)
 		for (int r = 0; r < g.R; ++r) {
 			int ya = ya0 + r * g.RA, yb = yb0 + sb * g.RB;
@@ -1570,13 +1571,14 @@ void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ 
 				yb = qb;
 			}
 			ok = ok && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
-			if (__builtin_amdgcn_ballot_w64(ok) == 0)        /* the tap reaches none of the wave's rows */
+			if (__builtin_amdgcn_ballot_w64(ok) == 0)
 				continue;
 			const T* p = src + (ok ? n + g.NS * (ya + g.LH * yb) + plane * c0 : 0);
 			/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded to four) first in its row */
 			const T* w = wt + (size_t) (r + g.R * (sb + g.S * c0)) * g.ldw;
 			const size_t wstep = (size_t) taps * g.ldw;
-			#pragma unroll 8
+			/* UNROLL loads in flight per wait; what is left over of a wave's channels goes one load at a time */
+			#pragma unroll UNROLL
 			for (int ch = c0; ch < c1; ++ch) {
 				T v[VEC];
 				if (ok) {
@@ -1623,6 +1625,31 @@ void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ 
 				vec_store<T, VEC>(out + (out_row(g, m) + (size_t) g.out_M * c), acc[c]);
 			}
 		}
+	}
+}
+
+template<typename T, int VEC, bool DIVS, int UNROLL>
+__global__ __launch_bounds__(256)
+void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
+		T* __restrict__ out, const GatherGeom g) {
+	few_columns_body<T, VEC, DIVS, UNROLL>(src, wt, bias, out, g, (int) blockIdx.x);
+}
+
+/* An input gradient of a few columns and the layer's weight gradient in one launch (see gather_with_wgrad_kernel: both
+ * wait for the same upstream gradient only, and a dependent launch costs 4-5 us however little it does): blocks below
+ * gather_blocks form the input gradient, the others are the weight gradient's one-wavefront blocks. */
+template<typename T, int VEC, int UNROLL>
+__global__ __launch_bounds__(256)
+void few_columns_with_wgrad_kernel(const T* __restrict__ src, const T* __restrict__ wt, T* __restrict__ out, const GatherGeom g,
+		int gather_blocks, const T* __restrict__ w_src, const T* __restrict__ w_og, T* __restrict__ w_partials,
+		T* __restrict__ w_bias_partials, const GatherGeom w_g, const WgradSplit w_plan) {
+	if ((int) blockIdx.x < gather_blocks) {
+		few_columns_body<T, VEC, false, UNROLL>(src, wt, (const T*) nullptr, out, g, (int) blockIdx.x);
+	} else {
+		if (threadIdx.x >= 64)
+			return;
+		wgrad_body<T, 1, 1, 32, 32, 32, VEC, 0>(w_src, w_og, w_partials, w_bias_partials, w_g, w_plan,
+				(const T*) nullptr, (T*) nullptr, (T) 0, (T) 0, (int) blockIdx.x - gather_blocks);
 	}
 }
 
@@ -2248,14 +2275,27 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		 * the load instructions beats four times the waves (9 against 19 us on a 200,704 x 48 x 1 problem) */
 		const bool wide = vec && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 		const unsigned blocks = (unsigned) ((g.M + (wide ? 64 * V : 64) - 1) / (wide ? 64 * V : 64));
-		if (wide && divs)
-			few_columns_gather_kernel<T, V, true><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		/* a wave's share of the channels in whole batches of loads: eight to a batch if that divides it, else four */
+		const bool by8 = ((g.LC + 3) / 4) % 8 == 0;
+		if (rider && wide && !divs && bias == nullptr) {
+			const unsigned w_blocks = (unsigned) round_up(rider->plan.tiles * rider->plan.splits, 8);
+			if (by8)
+				few_columns_with_wgrad_kernel<T, V, 8><<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks, rider->x, rider->og,
+						rider->partials, rider->bias_partials, rider->g, rider->plan);
+			else
+				few_columns_with_wgrad_kernel<T, V, 4><<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks, rider->x, rider->og,
+						rider->partials, rider->bias_partials, rider->g, rider->plan);
+			rider->done = true;
+		} else if (wide && divs)
+			few_columns_gather_kernel<T, V, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		else if (wide && by8)
+			few_columns_gather_kernel<T, V, false, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else if (wide)
-			few_columns_gather_kernel<T, V, false><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+			few_columns_gather_kernel<T, V, false, 4><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else if (divs)
-			few_columns_gather_kernel<T, 1, true><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+			few_columns_gather_kernel<T, 1, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else
-			few_columns_gather_kernel<T, 1, false><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+			few_columns_gather_kernel<T, 1, false, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		CATTLE_HIP_CHECK(hipGetLastError());
 		if (mtiles_out)
 			*mtiles_out = 0;

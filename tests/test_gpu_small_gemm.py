@@ -203,3 +203,41 @@ def test_weight_gradient_riding_in_the_input_gradient_launch(case):
     assert hp.rel_err(grads[0][2].reshape(dx_ref.shape), dx_ref, label="riding weight gradient %s dx" % "x".join(str(v) for v in case)) < 1e-4
     assert hp.rel_err(grads[0][0], dw_ref) < 1e-4
     assert hp.rel_err(grads[0][1], db_ref) < 1e-4
+
+
+@pytest.mark.parametrize("case", [(64, 32, 32, 3, 16, 3, 1), (128, 32, 32, 3, 32, 3, 1), (32, 12, 10, 1, 8, 5, 2), (16, 9, 9, 4, 20, 3, 0),
+                                  (12, 8, 8, 2, 6, 3, 1)],
+                         ids=lambda c: "x".join(str(v) for v in c))
+def test_weight_gradient_riding_in_an_input_gradient_of_few_columns(case):
+    """The input gradient of a convolution over one to four channels (no matrix tiles: a lane owns rows and multiplies by
+    wave-uniform weights) carries the layer's weight gradient in its launch when that is one of one-wavefront tiles.
+    Riding or alone (the same layer as a network's first layer), the weight and bias gradients agree bit for bit; all
+    three gradients agree with the oracle. The first two cases are the first layers of BASELINE configs[0] and [2]."""
+    N, H, W, C, F, R, pad = case
+    dtype = np.float32
+    geom = dict(RH=R, RW=R, pv=pad, ph=pad, sv=1, sh=1, dv=0, dh=0)
+    gen = hp.rng(1700 + N + F)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (R * R * C, F), dtype, std=1.0 / np.sqrt(R * R * C))
+    b = hp.normal(gen, (1, F), dtype)
+    OH, OW = hp.conv_dims(H, W, R, R, pad, pad, 1, 1, 0, 0)
+    g = hp.normal(gen, (N, OH, OW, F), dtype)
+    grads = []
+    for first_layer in (False, True):
+        layer = ch.ConvKernelLayer(dtype, (H, W, C), F, R, R, pad, pad, 1, 1, 0, 0)
+        layer.set_input_layer(first_layer)
+        wp, bp = layer.get_params()
+        wp.set_values(w)
+        bp.set_values(b)
+        layer.pass_forward(ch.DeviceTensor.from_host(x), True)
+        dx = layer.pass_back(ch.DeviceTensor.from_host(g))
+        grads.append((wp.get_grad().copy(), bp.get_grad().copy(), None if first_layer else dx.to_host()))
+    assert np.array_equal(grads[0][0], grads[1][0])
+    assert np.array_equal(grads[0][1], grads[1][1])
+    x64, w64, b64, g64 = (np.asarray(a, np.float64) for a in (x, w, b, g))
+    o_ref, cache = oracle.conv_forward(x64, w64, b64, return_cache=True, **geom)
+    dx_ref, dw_ref, db_ref = oracle.conv_backward(x.shape, cache, w64, g64, **geom)
+    label = "few columns with weight gradient %s" % "x".join(str(v) for v in case)
+    assert hp.rel_err(grads[0][2], dx_ref, label=label + " dx") < 1e-4
+    assert hp.rel_err(grads[0][0], dw_ref, label=label + " dw") < 1e-4
+    assert hp.rel_err(grads[0][1], db_ref.reshape(1, -1), label=label + " db") < 1e-4
