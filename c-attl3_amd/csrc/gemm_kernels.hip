@@ -1556,49 +1556,94 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 		#pragma unroll
 		for (int i = 0; i < VEC; ++i)
 			acc[c][i] = (T) 0;
-	/* the source channels are dealt over the waves; a tap that reaches none of a wavefront's rows (zero padding, or a
-	 * stride that does not divide: its rows share an output position or a few) is skipped whole */
-	const int per = (g.LC + WAVES - 1) / WAVES;
-	const int c0 = wave * per, c1 = min(g.LC, c0 + per);
-	for (int sb = 0; sb < g.S; ++sb)
-		for (int r = 0; r < g.R; ++r) {
-			int ya = ya0 + r * g.RA, yb = yb0 + sb * g.RB;
-			bool ok = mvalid;
-			if (DIVS) {
-				const int qa = ya / g.DA, qb = yb / g.DB;
-				ok = ok && qa * g.DA == ya && qb * g.DB == yb;
-				ya = qa;
-				yb = qb;
-			}
-			ok = ok && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
-			if (__builtin_amdgcn_ballot_w64(ok) == 0)
-				continue;
-			const T* p = src + (ok ? n + g.NS * (ya + g.LH * yb) + plane * c0 : 0);
-			/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded to four) first in its row */
-			const T* w = wt + (size_t) (r + g.R * (sb + g.S * c0)) * g.ldw;
-			const size_t wstep = (size_t) taps * g.ldw;
-			/* UNROLL loads in flight per wait; what is left over of a wave's channels goes one load at a time */
-			#pragma unroll UNROLL
-			for (int ch = c0; ch < c1; ++ch) {
-				T v[VEC];
-				if (ok) {
-					vec_load_global<T, VEC>(v, p);
-				} else {
+	if constexpr (UNROLL == 0) {
+		/* Few source channels (a first layer's forward pass, a transposed convolution that ends in an image): the loop over
+		 * taps below would wait for memory once per tap with a load or two in flight. Here the reduction steps (tap-major,
+		 * channels within a tap) are dealt over the waves in contiguous shares and a wave takes its share in batches whose
+		 * loads are all in flight together: a step that does not reach a row (zero padding) or lies past the share reads a
+		 * block of zeros instead of branching. The address arithmetic is paid per step, not per tap: with many channels
+		 * per tap the loop below is the faster one (4 x 4 x 3 -> 3 on 25,600 rows 6.9 -> 4.7 us; 3 x 3 x 32 -> 3 on 131,072
+		 * rows 14.7 -> 22.7 us). */
+		constexpr int BATCH = sizeof(T) == 4 ? 12 : 8;
+		const int total = taps * g.LC, per = (total + WAVES - 1) / WAVES;
+		const int s0 = wave * per, s1 = min(total, s0 + per);
+		int tap = s0 / g.LC, ch = s0 - tap * g.LC;
+		int sb = tap / g.R, r = tap - sb * g.R;
+		const T* const zeros = reinterpret_cast<const T*>(g_zero_block);
+		const int base = n + g.NS * (ya0 + g.LH * yb0);
+		for (int s = s0; s < s1; s += BATCH) {
+			T v[BATCH][VEC], wk[BATCH][FEW_COLUMNS];
+			#pragma unroll
+			for (int j = 0; j < BATCH; ++j) {
+				const bool live = s + j < s1;        /* wave-uniform */
+				const int da = r * g.RA, db = sb * g.RB;
+				const bool ok = mvalid && live && (unsigned) (ya0 + da) < (unsigned) g.LH && (unsigned) (yb0 + db) < (unsigned) g.LW;
+				vec_load_global<T, VEC>(v[j], ok ? src + (base + g.NS * (da + g.LH * db) + plane * ch) : zeros);
+				/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded to four) first in its row */
+				vec_load_global<T, FEW_COLUMNS>(wk[j], wt + (size_t) (live ? r + g.R * (sb + g.S * ch) : 0) * g.ldw);
+				if (!live) {
 					#pragma unroll
-					for (int i = 0; i < VEC; ++i)
-						v[i] = (T) 0;
+					for (int c = 0; c < FEW_COLUMNS; ++c)
+						wk[j][c] = (T) 0;
 				}
-				T wk[FEW_COLUMNS];
-				vec_load_global<T, FEW_COLUMNS>(wk, w);
+				const bool last_ch = ch + 1 == g.LC, last_r = r + 1 == g.R;
+				ch = last_ch ? 0 : ch + 1;
+				sb += last_ch && last_r ? 1 : 0;
+				r = last_ch ? (last_r ? 0 : r + 1) : r;
+			}
+			#pragma unroll
+			for (int j = 0; j < BATCH; ++j)
 				#pragma unroll
 				for (int c = 0; c < FEW_COLUMNS; ++c)
 					#pragma unroll
 					for (int i = 0; i < VEC; ++i)
-						acc[c][i] += v[i] * wk[c];
-				p += ok ? plane : 0;
-				w += wstep;
-			}
+						acc[c][i] += v[j][i] * wk[j][c];
 		}
+	} else {
+		/* the source channels are dealt over the waves; a tap that reaches none of a wavefront's rows (zero padding, or a
+		 * stride that does not divide: its rows share an output position or a few) is skipped whole */
+		const int per = (g.LC + WAVES - 1) / WAVES;
+		const int c0 = wave * per, c1 = min(g.LC, c0 + per);
+		for (int sb = 0; sb < g.S; ++sb)
+			for (int r = 0; r < g.R; ++r) {
+				int ya = ya0 + r * g.RA, yb = yb0 + sb * g.RB;
+				bool ok = mvalid;
+				if (DIVS) {
+					const int qa = ya / g.DA, qb = yb / g.DB;
+					ok = ok && qa * g.DA == ya && qb * g.DB == yb;
+					ya = qa;
+					yb = qb;
+				}
+				ok = ok && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
+				if (__builtin_amdgcn_ballot_w64(ok) == 0)
+					continue;
+				const T* p = src + (ok ? n + g.NS * (ya + g.LH * yb) + plane * c0 : 0);
+				/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded to four) first in its row */
+				const T* w = wt + (size_t) (r + g.R * (sb + g.S * c0)) * g.ldw;
+				const size_t wstep = (size_t) taps * g.ldw;
+				/* UNROLL loads in flight per wait; what is left over of a wave's channels goes one load at a time */
+				#pragma unroll (UNROLL > 0 ? UNROLL : 1)
+				for (int ch = c0; ch < c1; ++ch) {
+					T v[VEC];
+					if (ok) {
+						vec_load_global<T, VEC>(v, p);
+					} else {
+						#pragma unroll
+						for (int i = 0; i < VEC; ++i)
+							v[i] = (T) 0;
+					}
+					T wk[FEW_COLUMNS];
+					vec_load_global<T, FEW_COLUMNS>(wk, w);
+					#pragma unroll
+					for (int c = 0; c < FEW_COLUMNS; ++c)
+						#pragma unroll
+						for (int i = 0; i < VEC; ++i)
+							acc[c][i] += v[i] * wk[c];
+					p += ok ? plane : 0;
+					w += wstep;
+				}
+			}
+	}
 	__shared__ T red[WAVES - 1][FEW_COLUMNS][ROWS];
 	if (wave > 0) {
 		#pragma unroll
@@ -1633,6 +1678,13 @@ __global__ __launch_bounds__(256)
 void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom g) {
 	few_columns_body<T, VEC, DIVS, UNROLL>(src, wt, bias, out, g, (int) blockIdx.x);
+}
+
+template<typename T, int VEC, int UNROLL>
+__global__ __launch_bounds__(256)
+void few_columns_plain_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
+		T* __restrict__ out, const GatherGeom g) {
+	few_columns_body<T, VEC, false, UNROLL>(src, wt, bias, out, g, (int) blockIdx.x);
 }
 
 /* An input gradient of a few columns and the layer's weight gradient in one launch (see gather_with_wgrad_kernel: both
@@ -2275,27 +2327,30 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		 * the load instructions beats four times the waves (9 against 19 us on a 200,704 x 48 x 1 problem) */
 		const bool wide = vec && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 		const unsigned blocks = (unsigned) ((g.M + (wide ? 64 * V : 64) - 1) / (wide ? 64 * V : 64));
-		/* a wave's share of the channels in whole batches of loads: eight to a batch if that divides it, else four */
-		const bool by8 = ((g.LC + 3) / 4) % 8 == 0;
+		/* how a wave walks the reduction (few_columns_body): with up to eight source channels, steps of all taps in batches
+		 * (0); else tap by tap with a wave's share of the channels in whole batches of loads, eight to a batch if that
+		 * divides the share, else four */
+		const int walk = !divs && wide && g.LC <= 8 ? 0 : ((g.LC + 3) / 4) % 8 == 0 ? 8 : 4;
+		#define CATTLE_HIP_FEW_COLUMNS(KERNEL, ...) \
+			do { \
+				if (walk == 0) KERNEL<T, V, 0> __VA_ARGS__; \
+				else if (walk == 8) KERNEL<T, V, 8> __VA_ARGS__; \
+				else KERNEL<T, V, 4> __VA_ARGS__; \
+			} while (0)
 		if (rider && wide && !divs && bias == nullptr) {
 			const unsigned w_blocks = (unsigned) round_up(rider->plan.tiles * rider->plan.splits, 8);
-			if (by8)
-				few_columns_with_wgrad_kernel<T, V, 8><<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks, rider->x, rider->og,
-						rider->partials, rider->bias_partials, rider->g, rider->plan);
-			else
-				few_columns_with_wgrad_kernel<T, V, 4><<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks, rider->x, rider->og,
-						rider->partials, rider->bias_partials, rider->g, rider->plan);
+			CATTLE_HIP_FEW_COLUMNS(few_columns_with_wgrad_kernel, <<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks,
+					rider->x, rider->og, rider->partials, rider->bias_partials, rider->g, rider->plan));
 			rider->done = true;
 		} else if (wide && divs)
 			few_columns_gather_kernel<T, V, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
-		else if (wide && by8)
-			few_columns_gather_kernel<T, V, false, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else if (wide)
-			few_columns_gather_kernel<T, V, false, 4><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+			CATTLE_HIP_FEW_COLUMNS(few_columns_plain_kernel, <<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g));
 		else if (divs)
 			few_columns_gather_kernel<T, 1, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else
 			few_columns_gather_kernel<T, 1, false, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		#undef CATTLE_HIP_FEW_COLUMNS
 		CATTLE_HIP_CHECK(hipGetLastError());
 		if (mtiles_out)
 			*mtiles_out = 0;
@@ -2853,6 +2908,11 @@ WgradPlan wgrad_plan(int M, int K, int F, int N, bool vec) {
 	 * two chunks 49.9 us for the backward pass, 64 slices of four 53.0 us) */
 	const int min_chunks = tune.wgrad_min_chunks > 0 ? tune.wgrad_min_chunks : (short_m || v.mc >= 128 ? 2 : 4);
 	want = std::min(want, std::max(1, chunks / min_chunks));
+	/* a short reduction whose tiles already give every CU a block is not cut: the slices of a large gradient cost more to
+	 * write, read back and add than the shorter chains save (dense 4096 -> 1024 at batch 512: two slices of 16.8 MB,
+	 * 50 us + 33 us for the launch that adds them) */
+	if (short_m && tiles >= device_shape().cus)
+		want = 1;
 	if (tune.wgrad_splits > 0)
 		want = std::min(tune.wgrad_splits, chunks);
 	p.chunks_per_split = (chunks + want - 1) / want;
