@@ -608,6 +608,36 @@ def test_first_layer_weight_gradient_from_the_pooled_gradient(window, act, dtype
     assert hp.rel_err(db, ref["db"].reshape(1, -1), label=label + " db") < tol
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N", [6, 7, 2, 36])
+def test_first_layer_weight_gradient_with_ragged_batches(N, dtype):
+    """Batches that are not whole 16-byte vectors of samples (or only in fp64) take the path with the scatter pass; a first
+    layer's gradients must not depend on which path ran."""
+    H, W, C, F = 8, 8, 3, 6
+    act, pool = ("relu", 0.0), ("max", 2, 2, 2, 2)
+    gen = hp.rng(900 + N)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (9 * C, F), dtype, std=0.3)
+    b = hp.uniform(gen, (1, F), -0.5, 0.5, dtype)
+    g = hp.normal(gen, (N, H // 2, W // 2, F), dtype)
+    runs = []
+    for first in (False, True):
+        fused, members, kdims = _build(dtype, N, H, W, C, F, conv=GEOM_3X3, act=act, pool=pool)
+        fused.set_input_layer(first)
+        out, dx, mode = _run_fused(fused, members, x, w, b, g)
+        wp, bp = members["conv"].get_params()
+        runs.append((wp.get_grad().copy(), bp.get_grad().copy(), mode))
+    assert runs[0][2] == runs[1][2]
+    assert np.array_equal(runs[0][0], runs[1][0])
+    assert np.array_equal(runs[0][1], runs[1][1])
+    chain = Chain(GEOM_3X3, act=act, pool=pool)
+    x64, w64, b64 = (np.asarray(a, np.float64) for a in (x, w, b))
+    chain.forward(x64, w64, b64)
+    ref = chain.backward(x64, w64, np.asarray(g, np.float64))
+    tol = TOL[np.dtype(dtype)]
+    assert hp.rel_err(runs[1][0], ref["dw"], label="first layer N=%d %s dw" % (N, np.dtype(dtype).name)) < tol
+
+
 # ---- a seeded sweep of fused groups over geometries nobody chose by hand ------------------------------------------------
 
 def _sweep_cases(count, seed):
