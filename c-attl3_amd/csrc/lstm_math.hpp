@@ -58,7 +58,7 @@ __device__ __forceinline__ T lstm_ld(const T* p, unsigned i) {
 }
 template<typename T>
 __device__ __forceinline__ void lstm_st(T* p, unsigned i, T v) {
-	((__attribute__((address_space(1))) T*) p)[i] = v;
+	__builtin_nontemporal_store(v, (__attribute__((address_space(1))) T*) p + i);
 }
 
 /* The usual cell: sigmoid gates, tanh on the candidates and on the state. Kernels test for it once and run the
