@@ -125,6 +125,22 @@ __device__ __forceinline__ void vec_store(T* p, const T (&src)[V]) {
 	}
 }
 
+/* The same as a streaming store to global memory: results that the storing XCD will not read again need no place in
+ * its L2, and a kernel's end does not wait for them to be written back from there. */
+template<typename T, int V>
+__device__ __forceinline__ void vec_store_stream(T* p, const T (&src)[V]) {
+	if constexpr (V == 1) {
+		__builtin_nontemporal_store(src[0], (__attribute__((address_space(1))) T*) p);
+	} else {
+		typedef typename VecOf<T, V>::type vt;
+		vt v;
+		#pragma unroll
+		for (int i = 0; i < V; ++i)
+			v[i] = src[i];
+		__builtin_nontemporal_store(v, (__attribute__((address_space(1))) vt*) p);
+	}
+}
+
 /* fn(std::integral_constant<int, 0>()) ... fn(std::integral_constant<int, N - 1>()): a loop whose index is a
  * compile-time constant in the body (register arrays indexed by it stay registers) */
 template<int N, typename Fn>
@@ -739,10 +755,10 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 								for (int l = 0; l < E.prh; ++l)
 									consider(col[k * kstep + l * SB], (unsigned) (k * E.prh + l));
 						}
-						out[sp.pooled + pooled_plane * f] = best;
-						E.inds[sp.ind + (size_t) f * g.N] = bi;
+						__builtin_nontemporal_store(best, (__attribute__((address_space(1))) T*) out + (sp.pooled + pooled_plane * f));
+						__builtin_nontemporal_store(bi, (__attribute__((address_space(1))) unsigned*) E.inds + (sp.ind + (size_t) f * g.N));
 						if (E.pre)
-							E.pre[sp.pooled + pooled_plane * f] = best_pre;
+							__builtin_nontemporal_store(best_pre, (__attribute__((address_space(1))) T*) E.pre + (sp.pooled + pooled_plane * f));
 					}
 				}
 			}
@@ -773,9 +789,9 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 						if (mm < g.M) {
 							#pragma unroll
 							for (int j0 = 0; j0 < MB; j0 += VS) {
-								vec_store<T, VS>(out + o + j0, *reinterpret_cast<T (*)[VS]>(&y[j0]));
+								vec_store_stream<T, VS>(out + o + j0, *reinterpret_cast<T (*)[VS]>(&y[j0]));
 								if (E.pre)
-									vec_store<T, VS>(E.pre + o + j0, *reinterpret_cast<T (*)[VS]>(&z[j0]));
+									vec_store_stream<T, VS>(E.pre + o + j0, *reinterpret_cast<T (*)[VS]>(&z[j0]));
 							}
 						}
 					} else {
@@ -897,7 +913,7 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 							#pragma unroll
 							for (int j = 0; j < VS; ++j)
 								v[j] = acc[i][j0 + j][r] + bv;
-							vec_store<T, VS>(dst + j0, v);
+							vec_store_stream<T, VS>(dst + j0, v);
 						}
 					}
 				} else {
@@ -1943,10 +1959,10 @@ void split_reduce_kernel(const T* __restrict__ partials, const T* __restrict__ b
 	const size_t o = ACT ? (size_t) m + (size_t) M * f : out_row(g, min(m, M - 1)) + (size_t) g.out_M * f;
 	T* dst = out + o;
 	if (m + V <= M && (reinterpret_cast<uintptr_t>(dst) & 15) == 0 && (!ACT || !E.pre || (reinterpret_cast<uintptr_t>(E.pre + o) & 15) == 0)) {
-		vec_store<T, V>(dst, acc);
+		vec_store_stream<T, V>(dst, acc);
 		if constexpr (ACT)
 			if (E.pre)
-				vec_store<T, V>(E.pre + o, pre);
+				vec_store_stream<T, V>(E.pre + o, pre);
 	} else {
 		#pragma unroll
 		for (int i = 0; i < V; ++i)
