@@ -363,20 +363,22 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 	const int chunk0 = split ? part * L.chunks_per_part : 0;
 	const int nchunks = split ? min(L.chunks_per_part, (g.K + KC - 1) / KC - chunk0) : (g.K + KC - 1) / KC;
 
-	/* EPI_LSTM: this thread's state elements (row idx % BM of the tile, hidden channel idx / BM of the tile's CB) and
-	 * what their forward step reads besides this kernel's own sums, fetched now and used in the epilogue */
+	/* EPI_LSTM: this thread's state elements - LV consecutive rows (samples) of one hidden channel of the tile's CB per
+	 * group, so that every tensor of the step is read and written LV elements at a time - and what their forward step
+	 * reads besides this kernel's own sums, fetched now and used in the epilogue */
 	constexpr int CB = BF / 4, LSTM_ELEMS = EPI == EPI_LSTM ? BM * CB / THREADS : 1;
-	unsigned lstm_e[LSTM_ELEMS];
-	LstmForwardInputs<T> lstm_in[LSTM_ELEMS];
+	constexpr int LV = EPI == EPI_LSTM && BM * CB % (THREADS * VEC) == 0 ? VEC : 1, LSTM_GROUPS = LSTM_ELEMS / LV;
+	unsigned lstm_e[LSTM_GROUPS];
+	LstmForwardInputs<T> lstm_in[LSTM_GROUPS][LV];
 	if constexpr (EPI == EPI_LSTM) {
 		static_assert(BM * CB % THREADS == 0, "whole rounds of threads over a tile's state elements");
 		#pragma unroll
-		for (int it = 0; it < LSTM_ELEMS; ++it) {
-			const int idx = tid + it * THREADS, row = idx % BM, cl = idx / BM;
+		for (int gi = 0; gi < LSTM_GROUPS; ++gi) {
+			const int idx = tid + gi * THREADS, row = (idx % (BM / LV)) * LV, cl = idx / (BM / LV);
 			const int mrow = tile_row_m(L, g, tile, BM, row);
-			lstm_e[it] = mrow < g.M ? (unsigned) mrow + (unsigned) g.M * (unsigned) (bp.y * CB + cl) : 0xffffffffu;
+			lstm_e[gi] = mrow < g.M ? (unsigned) mrow + (unsigned) g.M * (unsigned) (bp.y * CB + cl) : 0xffffffffu;
 			/* (every element of the array assigned: a partly initialised register array ends up in scratch memory) */
-			lstm_in[it] = lstm_forward_load<T>(E.lstm, lstm_e[it] != 0xffffffffu ? lstm_e[it] : 0u);
+			lstm_forward_load_vec<T, LV>(E.lstm, lstm_e[gi] != 0xffffffffu ? lstm_e[gi] : 0u, lstm_in[gi]);
 		}
 	}
 
@@ -614,28 +616,37 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 		__syncthreads();
 		/* the arithmetic of all of a thread's elements before the first store: independent chains that the compiler
 		 * may interleave (stores in between would keep them apart), which matters with a wavefront per SIMD */
-		LstmForwardOutputs<T> res[LSTM_ELEMS];
-		T zh4[LSTM_ELEMS][4];
+		LstmForwardOutputs<T> res[LSTM_GROUPS][LV];
+		T zh4[LSTM_GROUPS][LV][4];
 		#pragma unroll
-		for (int it = 0; it < LSTM_ELEMS; ++it) {
-			const int idx = tid + it * THREADS, row = idx % BM, cl = idx / BM;
+		for (int gi = 0; gi < LSTM_GROUPS; ++gi) {
+			const int idx = tid + gi * THREADS, row = (idx % (BM / LV)) * LV, cl = idx / (BM / LV);
 			#pragma unroll
-			for (int gt = 0; gt < 4; ++gt)
-				zh4[it][gt] = lstm_stage[(gt * CB + cl) * LROW + row];
+			for (int gt = 0; gt < 4; ++gt) {
+				T zv[LV];
+				vec_load<T, LV>(zv, &lstm_stage[(gt * CB + cl) * LROW + row]);
+				#pragma unroll
+				for (int k = 0; k < LV; ++k)
+					zh4[gi][k][gt] = zv[k];
+			}
 		}
 		if (lstm_standard_acts(E.lstm.a)) {
 			#pragma unroll
-			for (int it = 0; it < LSTM_ELEMS; ++it)
-				res[it] = lstm_forward_compute<T, true>(E.lstm, lstm_in[it], true, zh4[it]);
+			for (int gi = 0; gi < LSTM_GROUPS; ++gi)
+				#pragma unroll
+				for (int k = 0; k < LV; ++k)
+					res[gi][k] = lstm_forward_compute<T, true>(E.lstm, lstm_in[gi][k], true, zh4[gi][k]);
 		} else {
 			#pragma unroll
-			for (int it = 0; it < LSTM_ELEMS; ++it)
-				res[it] = lstm_forward_compute<T, false>(E.lstm, lstm_in[it], true, zh4[it]);
+			for (int gi = 0; gi < LSTM_GROUPS; ++gi)
+				#pragma unroll
+				for (int k = 0; k < LV; ++k)
+					res[gi][k] = lstm_forward_compute<T, false>(E.lstm, lstm_in[gi][k], true, zh4[gi][k]);
 		}
 		#pragma unroll
-		for (int it = 0; it < LSTM_ELEMS; ++it)
-			if (lstm_e[it] != 0xffffffffu)
-				lstm_forward_store<T>(E.lstm, lstm_e[it], res[it]);
+		for (int gi = 0; gi < LSTM_GROUPS; ++gi)
+			if (lstm_e[gi] != 0xffffffffu)
+				lstm_forward_store_vec<T, LV>(E.lstm, lstm_e[gi], res[gi]);
 		return;
 	}
 	if constexpr (EPI == EPI_POOL) {
@@ -667,12 +678,15 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 					((size_t) b_p * E.OHp + a_p) * ((size_t) g.F * g.N) + n,
 					(size_t) n + (size_t) g.N * (a_p * E.prh + (size_t) g.OA * (b_p * E.prw)) };
 		};
-		/* The threads walk (sample, window, column), samples first. When the windows of a pass divide the threads of a
-		 * sample block evenly, a thread keeps its sample and window through every pass and only its column moves on. */
-		const int tps = THREADS >> sb_shift, outputs = (FP * W * SB + THREADS - 1) / THREADS;
+		/* The threads walk (samples, window, column), samples first and PV of them (one 16-byte access) per thread. When
+		 * the windows of a pass divide the threads of a sample block evenly, a thread keeps its samples and window through
+		 * every pass and only its column moves on. */
+		constexpr int PV = VEC, PV_SHIFT = PV == 4 ? 2 : PV == 2 ? 1 : 0;
+		const int sbv_shift = sb_shift - PV_SHIFT, SBV = 1 << sbv_shift;          /* the planner keeps SB >= PV */
+		const int tps = THREADS >> sbv_shift, outputs = (FP * W * SBV + THREADS - 1) / THREADS;
 		const bool fixed_spot = tps % W == 0;
-		const int fl0 = (tid >> sb_shift) / W, fl_step = tps / W;
-		Spot sp = spot(tid & (SB - 1), (tid >> sb_shift) % W);
+		const int fl0 = (tid >> sbv_shift) / W, fl_step = tps / W;
+		Spot sp = spot((tid & (SBV - 1)) << PV_SHIFT, (tid >> sbv_shift) % W);
 		const int kstep = pa << sb_shift;
 		const bool two_by_two = E.prh == 2 && E.prw == 2;
 		const size_t pooled_plane = (size_t) g.N * E.OHp * E.OWp;
@@ -707,58 +721,85 @@ __device__ __forceinline__ void gather_gemm_body(const T* __restrict__ src, cons
 								break;
 						} else {
 							const int it = tid + pass * THREADS;
-							if (it >= FP * W * SB)
+							if (it >= FP * W * SBV)
 								break;
-							const int t2 = it >> sb_shift;
+							const int t2 = it >> sbv_shift;
 							fl = t2 / W;
-							sp = spot(it & (SB - 1), t2 - fl * W);
+							sp = spot((it & (SBV - 1)) << PV_SHIFT, t2 - fl * W);
 						}
 						const int f = f0 + (fl / RG) * WT_F + FB * (RG * q + fl % RG) + i;
 						if (f >= g.F)
 							continue;
 						const T* col = stage + fl * LROW + sp.col;
+						T zv[PV];
 						if (E.pool_mean) {
 							/* the mean of the window, summed width-major / height-minor as the layer of its own does
 							 * (MeanPoolLayer.hpp:35-41); what the backward pass needs goes out at every position */
-							T sum = (T) 0;
+							T sum[PV];
+							#pragma unroll
+							for (int e = 0; e < PV; ++e)
+								sum[e] = (T) 0;
 							for (int k = 0; k < E.prw; ++k)
 								for (int l = 0; l < E.prh; ++l) {
-									const T z = col[k * kstep + l * SB];
-									const T y = act_f_coded<T, KIND>(z, E.p);
-									sum += y;
+									vec_load<T, PV>(zv, col + k * kstep + l * SB);
+									T y[PV];
+									#pragma unroll
+									for (int e = 0; e < PV; ++e) {
+										y[e] = act_f_coded<T, KIND>(zv[e], E.p);
+										sum[e] += y[e];
+									}
 									if (E.pre)
-										E.pre[sp.full + (size_t) g.N * (l + (size_t) g.OA * (k + (size_t) g.OB * f))] = E.keep_input ? z : y;
+										vec_store_stream<T, PV>(E.pre + (sp.full + (size_t) g.N * (l + (size_t) g.OA * (k + (size_t) g.OB * f))),
+												E.keep_input ? zv : y);
 								}
-							out[sp.pooled + pooled_plane * f] = sum / (T) (E.prh * E.prw);
+							#pragma unroll
+							for (int e = 0; e < PV; ++e)
+								sum[e] = sum[e] / (T) (E.prh * E.prw);
+							vec_store_stream<T, PV>(out + (sp.pooled + pooled_plane * f), sum);
 							continue;
 						}
 						/* strict '>' from lowest(), width-major / height-minor scan (MaxPoolLayer.hpp:45-56) */
-						T best = std::numeric_limits<T>::lowest(), best_pre = col[0];
-						unsigned bi = 0;
-						const auto consider = [&](T z, unsigned at) {
-							const T y = act_f_coded<T, KIND>(z, E.p);
-							if (y > best) {
-								best = y;
-								best_pre = z;
-								bi = at;
+						T best[PV], best_pre[PV];
+						unsigned bi[PV];
+						vec_load<T, PV>(zv, col);
+						#pragma unroll
+						for (int e = 0; e < PV; ++e) {
+							best[e] = std::numeric_limits<T>::lowest();
+							best_pre[e] = zv[e];
+							bi[e] = 0;
+						}
+						const auto consider = [&](const T (&z)[PV], unsigned at) {
+							#pragma unroll
+							for (int e = 0; e < PV; ++e) {
+								const T y = act_f_coded<T, KIND>(z[e], E.p);
+								if (y > best[e]) {
+									best[e] = y;
+									best_pre[e] = z[e];
+									bi[e] = at;
+								}
 							}
 						};
 						if (two_by_two) {
-							/* the usual window: its four values fetched together, then scanned in the same order */
-							const T z0 = best_pre, z1 = col[SB], z2 = col[kstep], z3 = col[kstep + SB];
-							consider(z0, 0u);
+							/* the usual window: its four positions fetched together, then scanned in the same order */
+							T z1[PV], z2[PV], z3[PV];
+							vec_load<T, PV>(z1, col + SB);
+							vec_load<T, PV>(z2, col + kstep);
+							vec_load<T, PV>(z3, col + kstep + SB);
+							consider(zv, 0u);
 							consider(z1, 1u);
 							consider(z2, 2u);
 							consider(z3, 3u);
 						} else {
 							for (int k = 0; k < E.prw; ++k)
-								for (int l = 0; l < E.prh; ++l)
-									consider(col[k * kstep + l * SB], (unsigned) (k * E.prh + l));
+								for (int l = 0; l < E.prh; ++l) {
+									vec_load<T, PV>(zv, col + k * kstep + l * SB);
+									consider(zv, (unsigned) (k * E.prh + l));
+								}
 						}
-						__builtin_nontemporal_store(best, (__attribute__((address_space(1))) T*) out + (sp.pooled + pooled_plane * f));
-						__builtin_nontemporal_store(bi, (__attribute__((address_space(1))) unsigned*) E.inds + (sp.ind + (size_t) f * g.N));
+						vec_store_stream<T, PV>(out + (sp.pooled + pooled_plane * f), best);
+						vec_store_stream<unsigned, PV>(E.inds + (sp.ind + (size_t) f * g.N), bi);
 						if (E.pre)
-							__builtin_nontemporal_store(best_pre, (__attribute__((address_space(1))) T*) E.pre + (sp.pooled + pooled_plane * f));
+							vec_store_stream<T, PV>(E.pre + (sp.pooled + pooled_plane * f), best_pre);
 					}
 				}
 			}
@@ -2450,7 +2491,8 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	if (epi == EPI_LSTM) {
 		/* a short tile (it stages itself whole) whose column groups are whole gate groups of the hidden channels */
 		const int hidden = g.F / 4;
-		if (v.bm > 128 || g.F % 4 != 0 || hidden % (v.bf / 4) != 0 || (size_t) g.M * hidden != E->lstm.P)
+		if (v.bm > 128 || g.F % 4 != 0 || hidden % (v.bf / 4) != 0 || (size_t) g.M * hidden != E->lstm.P ||
+				!lstm_forward_vectors<T>(E->lstm, GemmCfg<T>::VEC))
 			return false;
 	}
 	if (before_launch)
@@ -3022,6 +3064,9 @@ bool conv_forward_fused(const ConvShape& s, int N, const T* x, const T* w, const
 	}
 	/* the staging pass deals threads over windows of at most a tile's positions */
 	if (epi == EPI_POOL && E.prh * E.prw > 64)
+		return false;
+	/* it writes 16 bytes of consecutive samples at a time */
+	if (epi == EPI_POOL && (((reinterpret_cast<uintptr_t>(E.inds) | reinterpret_cast<uintptr_t>(E.pre)) & 15) != 0))
 		return false;
 	return launch_gather<T>(x, wt, b, out, g, nullptr, epi, &E, mtiles);
 }

@@ -168,6 +168,107 @@ __device__ __forceinline__ void lstm_forward_store(const LstmForwardStep<T>& A, 
 		lstm_st<T>(A.out, seq_offset(n, rest, A.N, A.out_T, A.out_t), o.h);
 }
 
+/* The same for V consecutive elements e0 .. e0 + V - 1 (e0 and N multiples of V, so they are V consecutive samples of
+ * one place and consecutive in every tensor of the step; tensors aligned to V elements): one access of V elements per
+ * tensor instead of V accesses, and the index arithmetic once. */
+template<typename T, int V>
+__device__ __forceinline__ void lstm_ldv(T (&dst)[V], const T* p, unsigned i) {
+	if constexpr (V == 1) {
+		dst[0] = lstm_ld<T>(p, i);
+	} else {
+		typedef T vt __attribute__((ext_vector_type(V)));
+		const vt v = *(const __attribute__((address_space(1))) vt*) (p + i);
+		#pragma unroll
+		for (int k = 0; k < V; ++k)
+			dst[k] = v[k];
+	}
+}
+template<typename T, int V>
+__device__ __forceinline__ void lstm_stv(T* p, unsigned i, const T (&src)[V]) {
+	if constexpr (V == 1) {
+		lstm_st<T>(p, i, src[0]);
+	} else {
+		typedef T vt __attribute__((ext_vector_type(V)));
+		vt v;
+		#pragma unroll
+		for (int k = 0; k < V; ++k)
+			v[k] = src[k];
+		__builtin_nontemporal_store(v, (__attribute__((address_space(1))) vt*) (p + i));
+	}
+}
+template<typename T, int V>
+__device__ __forceinline__ void lstm_forward_load_vec(const LstmForwardStep<T>& A, unsigned e0, LstmForwardInputs<T> (&in)[V]) {
+	const unsigned N = (unsigned) A.N, slab_rows = (unsigned) A.P / N;
+	const unsigned rest = e0 / N, n = e0 - rest * N;
+	T v[V];
+	#pragma unroll
+	for (int g = 0; g < 4; ++g) {
+		if (A.zx)
+			lstm_ldv<T, V>(v, A.zx, seq_offset(n, rest + g * slab_rows, A.N, A.zx_T, A.zx_t));
+		#pragma unroll
+		for (int k = 0; k < V; ++k)
+			in[k].zx[g] = A.zx ? v[k] : (T) 0;
+	}
+	if (A.prev_state)
+		lstm_ldv<T, V>(v, A.prev_state, e0);
+	#pragma unroll
+	for (int k = 0; k < V; ++k)
+		in[k].prev = A.prev_state ? v[k] : (T) 0;
+}
+template<typename T, int V>
+__device__ __forceinline__ void lstm_forward_store_vec(const LstmForwardStep<T>& A, unsigned e0, const LstmForwardOutputs<T> (&o)[V]) {
+	const unsigned N = (unsigned) A.N, P = (unsigned) A.P;
+	const unsigned rest = e0 / N, n = e0 - rest * N;
+	T v[V];
+	#pragma unroll
+	for (int g = 0; g < 4; ++g) {
+		if (A.z) {
+			#pragma unroll
+			for (int k = 0; k < V; ++k)
+				v[k] = o[k].v[g];
+			lstm_stv<T, V>(A.z, (unsigned) g * P + e0, v);
+		}
+		#pragma unroll
+		for (int k = 0; k < V; ++k)
+			v[k] = o[k].y[g];
+		lstm_stv<T, V>(A.gates, (unsigned) g * P + e0, v);
+	}
+	#pragma unroll
+	for (int k = 0; k < V; ++k)
+		v[k] = o[k].s;
+	lstm_stv<T, V>(A.state, e0, v);
+	#pragma unroll
+	for (int k = 0; k < V; ++k)
+		v[k] = o[k].as;
+	lstm_stv<T, V>(A.act_state, e0, v);
+	#pragma unroll
+	for (int k = 0; k < V; ++k)
+		v[k] = o[k].h;
+	if (A.hprev_all) {
+		if (A.h_t < A.h_T)
+			lstm_stv<T, V>(A.hprev_all, seq_offset(n, rest, A.N, A.h_T, A.h_t), v);
+		if (!A.prev_state) {                                    /* first step: no previous output, slab 0 is zero */
+			T zero[V];
+			#pragma unroll
+			for (int k = 0; k < V; ++k)
+				zero[k] = (T) 0;
+			lstm_stv<T, V>(A.hprev_all, seq_offset(n, rest, A.N, A.h_T, 0), zero);
+		}
+	}
+	if (A.out)
+		lstm_stv<T, V>(A.out, seq_offset(n, rest, A.N, A.out_T, A.out_t), v);
+}
+/* Whether the step's tensors allow accesses of V elements. */
+template<typename T>
+inline bool lstm_forward_vectors(const LstmForwardStep<T>& A, int V) {
+	const uintptr_t mask = (uintptr_t) V * sizeof(T) - 1;
+	const void* const ptrs[8] = { A.zx, A.prev_state, A.z, A.gates, A.state, A.act_state, A.hprev_all, A.out };
+	for (const void* q : ptrs)
+		if ((reinterpret_cast<uintptr_t>(q) & mask) != 0)
+			return false;
+	return A.N % V == 0 && A.P % (size_t) V == 0;
+}
+
 /* Every load of the element comes before its first store: the tensors are not declared free of aliases, and a store
  * between two loads would make the second wait for the first. */
 template<typename T, bool STD = false>
