@@ -1605,6 +1605,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 		ya0 = a * g.SA + g.PA;
 		yb0 = b * g.SB + g.PB;
 	}
+	constexpr int LOADS_IN_FLIGHT = UNROLL > 0 ? UNROLL : 1;
 	const int plane = g.NS * g.LH * g.LW;
 	const int taps = g.R * g.S;
 	T acc[FEW_COLUMNS][VEC];
@@ -1679,7 +1680,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 				const T* w = wt + (size_t) (r + g.R * (sb + g.S * c0)) * g.ldw;
 				const size_t wstep = (size_t) taps * g.ldw;
 				/* UNROLL loads in flight per wait; what is left over of a wave's channels goes one load at a time */
-				#pragma unroll (UNROLL > 0 ? UNROLL : 1)
+				#pragma unroll LOADS_IN_FLIGHT
 				for (int ch = c0; ch < c1; ++ch) {
 					T v[VEC];
 					if (ok) {
