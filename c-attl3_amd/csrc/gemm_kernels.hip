@@ -1576,7 +1576,10 @@ constexpr int MAX_DEVICES = 64;
 void* g_scratch_ptr[MAX_DEVICES] = { nullptr };
 
 /* ------------------------------------------------------------------------------------------------
- * The same gathered GEMM, out[M x F] = gather(src)[M x K] * wt[K x F] (+ bias), for F <= 4 output columns: the input
+ * The same gathered GEMM, out[M x F] = gather(src)[M x K] * wt[K x F] (+ bias), for F <= 4 output columns (NC = 8: five to
+ * eight, unstrided problems with 16-byte accesses: at 8 columns the vector ALU still beats 32-column matrix tiles that
+ * are three quarters padding, 81 -> 61 us on an 81,920 x 1152 x 8 input gradient; eight waves per block sharing the
+ * reduction instead of four were slower on every problem tried): the input
  * gradient of a network's first convolution (its columns are the image's channels), a transposed convolution that
  * ends in one or three channels, a convolution with a handful of filters. On 32 x 32 matrix tiles such a problem is
  * seven eighths padding (measured on a 3 x 3 x 32 -> 3 input gradient: the matrix pipes busy half of the kernel's
@@ -1588,8 +1591,8 @@ void* g_scratch_ptr[MAX_DEVICES] = { nullptr };
  * source channels are dealt over the four waves of a block, whose sums meet in LDS and are added in ascending
  * wave order: the summation order depends on the geometry only.
  * ---------------------------------------------------------------------------------------------- */
-constexpr int FEW_COLUMNS = 4;
-template<typename T, int VEC, bool DIVS, int UNROLL>
+constexpr int FEW_COLUMNS = 4, SOME_COLUMNS = 8;
+template<typename T, int VEC, bool DIVS, int UNROLL, int NC = FEW_COLUMNS>
 __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom& g, int block) {
 	constexpr int WAVES = 4, ROWS = 64 * VEC;
@@ -1608,9 +1611,9 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 	constexpr int LOADS_IN_FLIGHT = UNROLL > 0 ? UNROLL : 1;
 	const int plane = g.NS * g.LH * g.LW;
 	const int taps = g.R * g.S;
-	T acc[FEW_COLUMNS][VEC];
+	T acc[NC][VEC];
 	#pragma unroll
-	for (int c = 0; c < FEW_COLUMNS; ++c)
+	for (int c = 0; c < NC; ++c)
 		#pragma unroll
 		for (int i = 0; i < VEC; ++i)
 			acc[c][i] = (T) 0;
@@ -1630,18 +1633,18 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 		const T* const zeros = reinterpret_cast<const T*>(g_zero_block);
 		const int base = n + g.NS * (ya0 + g.LH * yb0);
 		for (int s = s0; s < s1; s += BATCH) {
-			T v[BATCH][VEC], wk[BATCH][FEW_COLUMNS];
+			T v[BATCH][VEC], wk[BATCH][NC];
 			#pragma unroll
 			for (int j = 0; j < BATCH; ++j) {
 				const bool live = s + j < s1;        /* wave-uniform */
 				const int da = r * g.RA, db = sb * g.RB;
 				const bool ok = mvalid && live && (unsigned) (ya0 + da) < (unsigned) g.LH && (unsigned) (yb0 + db) < (unsigned) g.LW;
 				vec_load_global<T, VEC>(v[j], ok ? src + (base + g.NS * (da + g.LH * db) + plane * ch) : zeros);
-				/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded to four) first in its row */
-				vec_load_global<T, FEW_COLUMNS>(wk[j], wt + (size_t) (live ? r + g.R * (sb + g.S * ch) : 0) * g.ldw);
+				/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded) first in its row */
+				vec_load_global<T, NC>(wk[j], wt + (size_t) (live ? r + g.R * (sb + g.S * ch) : 0) * g.ldw);
 				if (!live) {
 					#pragma unroll
-					for (int c = 0; c < FEW_COLUMNS; ++c)
+					for (int c = 0; c < NC; ++c)
 						wk[j][c] = (T) 0;
 				}
 				const bool last_ch = ch + 1 == g.LC, last_r = r + 1 == g.R;
@@ -1652,7 +1655,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 			#pragma unroll
 			for (int j = 0; j < BATCH; ++j)
 				#pragma unroll
-				for (int c = 0; c < FEW_COLUMNS; ++c)
+				for (int c = 0; c < NC; ++c)
 					#pragma unroll
 					for (int i = 0; i < VEC; ++i)
 						acc[c][i] += v[j][i] * wk[j][c];
@@ -1676,7 +1679,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 				if (__builtin_amdgcn_ballot_w64(ok) == 0)
 					continue;
 				const T* p = src + (ok ? n + g.NS * (ya + g.LH * yb) + plane * c0 : 0);
-				/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded to four) first in its row */
+				/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded) first in its row */
 				const T* w = wt + (size_t) (r + g.R * (sb + g.S * c0)) * g.ldw;
 				const size_t wstep = (size_t) taps * g.ldw;
 				/* UNROLL loads in flight per wait; what is left over of a wave's channels goes one load at a time */
@@ -1690,10 +1693,10 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 						for (int i = 0; i < VEC; ++i)
 							v[i] = (T) 0;
 					}
-					T wk[FEW_COLUMNS];
-					vec_load_global<T, FEW_COLUMNS>(wk, w);
+					T wk[NC];
+					vec_load_global<T, NC>(wk, w);
 					#pragma unroll
-					for (int c = 0; c < FEW_COLUMNS; ++c)
+					for (int c = 0; c < NC; ++c)
 						#pragma unroll
 						for (int i = 0; i < VEC; ++i)
 							acc[c][i] += v[i] * wk[c];
@@ -1702,16 +1705,16 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 				}
 			}
 	}
-	__shared__ T red[WAVES - 1][FEW_COLUMNS][ROWS];
+	__shared__ T red[WAVES - 1][NC][ROWS];
 	if (wave > 0) {
 		#pragma unroll
-		for (int c = 0; c < FEW_COLUMNS; ++c)
+		for (int c = 0; c < NC; ++c)
 			vec_store<T, VEC>(&red[wave - 1][c][lane * VEC], acc[c]);
 	}
 	__syncthreads();
 	if (wave == 0 && mvalid) {
 		#pragma unroll
-		for (int c = 0; c < FEW_COLUMNS; ++c) {
+		for (int c = 0; c < NC; ++c) {
 			if (c < g.F) {
 				#pragma unroll
 				for (int q = 0; q < WAVES - 1; ++q) {
@@ -1738,11 +1741,11 @@ void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ 
 	few_columns_body<T, VEC, DIVS, UNROLL>(src, wt, bias, out, g, (int) blockIdx.x);
 }
 
-template<typename T, int VEC, int UNROLL>
+template<typename T, int VEC, int UNROLL, int NC = FEW_COLUMNS>
 __global__ __launch_bounds__(256)
 void few_columns_plain_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom g) {
-	few_columns_body<T, VEC, false, UNROLL>(src, wt, bias, out, g, (int) blockIdx.x);
+	few_columns_body<T, VEC, false, UNROLL, NC>(src, wt, bias, out, g, (int) blockIdx.x);
 }
 
 /* An input gradient of a few columns and the layer's weight gradient in one launch (see gather_with_wgrad_kernel: both
@@ -2378,12 +2381,13 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	const bool divs = g.DA != 1 || g.DB != 1;
 	if (epi != EPI_NONE && (!vec || divs || (reinterpret_cast<uintptr_t>(out) & 15) != 0))
 		return false;
-	if (epi == EPI_NONE && then == nullptr && g.F <= FEW_COLUMNS) {
-		/* a handful of output columns: no matrix tiles (few_columns_gather_kernel) */
+	/* 16-byte loads wherever alignment allows, even where they leave a SIMD a wave or two: measured, a quarter of
+	 * the load instructions beats four times the waves (9 against 19 us on a 200,704 x 48 x 1 problem) */
+	const bool wide = vec && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+	if (epi == EPI_NONE && then == nullptr && (g.F <= FEW_COLUMNS || (g.F <= SOME_COLUMNS && wide && !divs))) {
+		/* a handful of output columns: no matrix tiles (few_columns_gather_kernel); five to eight of them in the
+		 * vectorised forward form only */
 		constexpr int V = GemmCfg<T>::VEC;
-		/* 16-byte loads wherever alignment allows, even where they leave a SIMD a wave or two: measured, a quarter of
-		 * the load instructions beats four times the waves (9 against 19 us on a 200,704 x 48 x 1 problem) */
-		const bool wide = vec && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 		const unsigned blocks = (unsigned) ((g.M + (wide ? 64 * V : 64) - 1) / (wide ? 64 * V : 64));
 		/* how a wave walks the reduction (few_columns_body): with up to eight source channels, steps of all taps in batches
 		 * (0); else tap by tap with a wave's share of the channels in whole batches of loads, eight to a batch if that
@@ -2395,7 +2399,11 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 				else if (walk == 8) KERNEL<T, V, 8> __VA_ARGS__; \
 				else KERNEL<T, V, 4> __VA_ARGS__; \
 			} while (0)
-		if (rider && wide && !divs && bias == nullptr) {
+		if (g.F > FEW_COLUMNS) {
+			if (walk == 0) few_columns_plain_kernel<T, V, 0, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+			else if (walk == 8) few_columns_plain_kernel<T, V, 8, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+			else few_columns_plain_kernel<T, V, 4, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
+		} else if (rider && wide && !divs && bias == nullptr) {
 			const unsigned w_blocks = (unsigned) round_up(rider->plan.tiles * rider->plan.splits, 8);
 			CATTLE_HIP_FEW_COLUMNS(few_columns_with_wgrad_kernel, <<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks,
 					rider->x, rider->og, rider->partials, rider->bias_partials, rider->g, rider->plan));

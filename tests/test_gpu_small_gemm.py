@@ -241,3 +241,37 @@ def test_weight_gradient_riding_in_an_input_gradient_of_few_columns(case):
     assert hp.rel_err(grads[0][2], dx_ref, label=label + " dx") < 1e-4
     assert hp.rel_err(grads[0][0], dw_ref, label=label + " dw") < 1e-4
     assert hp.rel_err(grads[0][1], db_ref.reshape(1, -1), label=label + " db") < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", [(32, 16, 16, 8, 128, 3, 1), (16, 10, 12, 5, 7, 3, 1), (8, 9, 9, 6, 6, 5, 2), (12, 8, 8, 40, 8, 3, 0),
+                                  (6, 8, 8, 8, 5, 3, 1)],
+                         ids=lambda c: "x".join(str(v) for v in c))
+def test_five_to_eight_columns_without_matrix_tiles(case, dtype):
+    """Products with five to eight output columns (a forward pass with that many filters, an input gradient to that many
+    channels) run on the vector ALU like those with up to four when their accesses can be 16 bytes wide. The first case is
+    the input-side convolution of BASELINE configs[4] at one time step's batch; the last has a batch that only fp64 can
+    take in whole vectors."""
+    N, H, W, C, F, R, pad = case
+    geom = dict(RH=R, RW=R, pv=pad, ph=pad, sv=1, sh=1, dv=0, dh=0)
+    gen = hp.rng(1800 + N + C + F)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (R * R * C, F), dtype, std=1.0 / np.sqrt(R * R * C))
+    b = hp.normal(gen, (1, F), dtype)
+    OH, OW = hp.conv_dims(H, W, R, R, pad, pad, 1, 1, 0, 0)
+    g = hp.normal(gen, (N, OH, OW, F), dtype)
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F, R, R, pad, pad, 1, 1, 0, 0)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    out = layer.pass_forward(ch.DeviceTensor.from_host(x), True).to_host()
+    dx = layer.pass_back(ch.DeviceTensor.from_host(g)).to_host()
+    x64, w64, b64, g64 = (np.asarray(a, np.float64) for a in (x, w, b, g))
+    o_ref, cache = oracle.conv_forward(x64, w64, b64, return_cache=True, **geom)
+    dx_ref, dw_ref, db_ref = oracle.conv_backward(x.shape, cache, w64, g64, **geom)
+    tol = 1e-4 if dtype == np.float32 else 1e-10
+    label = "five to eight columns %s %s" % ("x".join(str(v) for v in case), np.dtype(dtype).name)
+    assert hp.rel_err(out, o_ref, label=label + " y") < tol
+    assert hp.rel_err(dx, dx_ref, label=label + " dx") < tol
+    assert hp.rel_err(wp.get_grad(), dw_ref, label=label + " dw") < tol
+    assert hp.rel_err(bp.get_grad(), db_ref.reshape(1, -1), label=label + " db") < tol
