@@ -1734,18 +1734,26 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 	}
 }
 
+/* Which 64 VEC rows block `bid` of a grid of (blocks rounded up to eight) takes: every XCD a contiguous range of the rows,
+ * so that the blocks of neighbouring output positions, which read the same source rows through different taps, share an
+ * L2 (dealt round-robin, an 81,920 x 1152 x 8 input gradient fetched its 42 MB source eight times over: 349 MB). */
+template<int VEC>
+__device__ __forceinline__ int few_columns_block(const GatherGeom& g, int bid) {
+	return xcd_tile(bid, (g.M + 64 * VEC - 1) / (64 * VEC));
+}
+
 template<typename T, int VEC, bool DIVS, int UNROLL>
 __global__ __launch_bounds__(256)
 void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom g) {
-	few_columns_body<T, VEC, DIVS, UNROLL>(src, wt, bias, out, g, (int) blockIdx.x);
+	few_columns_body<T, VEC, DIVS, UNROLL>(src, wt, bias, out, g, few_columns_block<VEC>(g, (int) blockIdx.x));
 }
 
 template<typename T, int VEC, int UNROLL, int NC = FEW_COLUMNS>
 __global__ __launch_bounds__(256)
 void few_columns_plain_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
 		T* __restrict__ out, const GatherGeom g) {
-	few_columns_body<T, VEC, false, UNROLL, NC>(src, wt, bias, out, g, (int) blockIdx.x);
+	few_columns_body<T, VEC, false, UNROLL, NC>(src, wt, bias, out, g, few_columns_block<VEC>(g, (int) blockIdx.x));
 }
 
 /* An input gradient of a few columns and the layer's weight gradient in one launch (see gather_with_wgrad_kernel: both
@@ -1757,7 +1765,7 @@ void few_columns_with_wgrad_kernel(const T* __restrict__ src, const T* __restric
 		int gather_blocks, const T* __restrict__ w_src, const T* __restrict__ w_og, T* __restrict__ w_partials,
 		T* __restrict__ w_bias_partials, const GatherGeom w_g, const WgradSplit w_plan) {
 	if ((int) blockIdx.x < gather_blocks) {
-		few_columns_body<T, VEC, false, UNROLL>(src, wt, (const T*) nullptr, out, g, (int) blockIdx.x);
+		few_columns_body<T, VEC, false, UNROLL>(src, wt, (const T*) nullptr, out, g, few_columns_block<VEC>(g, (int) blockIdx.x));
 	} else {
 		if (threadIdx.x >= 64)
 			return;
@@ -2388,7 +2396,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		/* a handful of output columns: no matrix tiles (few_columns_gather_kernel); five to eight of them in the
 		 * vectorised forward form only */
 		constexpr int V = GemmCfg<T>::VEC;
-		const unsigned blocks = (unsigned) ((g.M + (wide ? 64 * V : 64) - 1) / (wide ? 64 * V : 64));
+		const unsigned blocks = (unsigned) round_up((g.M + (wide ? 64 * V : 64) - 1) / (wide ? 64 * V : 64), 8);   /* few_columns_block */
 		/* how a wave walks the reduction (few_columns_body): with up to eight source channels, steps of all taps in batches
 		 * (0); else tap by tap with a wave's share of the channels in whole batches of loads, eight to a batch if that
 		 * divides the share, else four */
