@@ -1316,7 +1316,8 @@ struct FusedLayer : LayerBase {
 		const int sh_a = log2_exact(ps.RH), sh_b = log2_exact(ps.RW);
 		constexpr int V = 16 / (int) sizeof(T);
 		auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-		if (in_grad != nullptr || sh_a < 0 || sh_b < 0 || n % V != 0 || !aligned(g) || !aligned(y_cache) || !aligned(pool->inds.p))
+		if (in_grad != nullptr || sh_a < 0 || sh_b < 0 || n % V != 0 || !aligned(g) || !aligned(y_cache) || !aligned(pool->inds.p) ||
+				!aligned(conv->x_cache))
 			return false;
 		if (act && !(act_sign_coded(act->kind) && act->p >= 0))
 			return false;
