@@ -281,6 +281,8 @@ def conv_shapes_run(args, dtype):
         ("autoencoder transposed conv 4x4 10x10x3 -> 3, batch 256", "transconv", 256, 10, 10, 3, 3, 4, 4, 0, 0, 1, 1, 0, 0, False),
         ("autoencoder transposed conv 4x4 stride 2 13x13x3 -> 1, batch 256", "transconv", 256, 13, 13, 3, 1, 4, 4, 0, 0, 2, 2, 0, 0, False),
         ("transposed conv 3x3 stride 2 14x14x128 -> 64 pad 1, batch 64", "transconv", 64, 14, 14, 128, 64, 3, 3, 1, 1, 2, 2, 0, 0, False),
+        # the last layer of an image decoder: many channels in, an image out
+        ("conv 3x3 64x64x64 -> 3, batch 64", "conv", 64, 64, 64, 64, 3, 3, 3, 1, 1, 1, 1, 0, 0, False),
     ]
     if args.only:
         shapes = [sh for sh in shapes if args.only in sh[0]]

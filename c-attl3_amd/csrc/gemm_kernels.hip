@@ -1598,10 +1598,31 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 	constexpr int WAVES = 4, ROWS = 64 * VEC;
 	const int lane = threadIdx.x % 64;
 	const int wave = __builtin_amdgcn_readfirstlane((int) threadIdx.x / 64);
-	const int m = block * ROWS + lane * VEC;
-	const bool mvalid = m < g.M;             /* whole vectors: M is a multiple of VEC */
-	int n, ya0, yb0;
-	{
+	/* The block's rows: 64 VEC consecutive m (samples of one output position, mostly), or - unstrided problems whose batch is
+	 * a multiple of 32 and whose output divides into patches - 32 samples of a patch of 2 x (64 VEC / 64) positions: the
+	 * taps of neighbouring positions read the same source rows, so a block of a patch touches a third of the source
+	 * bytes that a block of one position's samples does, and the rest comes out of the caches (a 3 x 3 x 64 -> 3
+	 * convolution over 262,144 rows fetched its 67 MB source six times over). */
+	constexpr int LPS = 32 / VEC, PATCH_A = 2, PATCH_B = 64 / LPS / PATCH_A;
+	/* (where fetches rather than arithmetic bound the kernel: up to four columns, and a source that the L2 caches
+	 * together do not hold - with eight columns, or a source of 17 and 42 MB, patches were 10-14 % slower: their loads
+	 * are 128-byte pieces where the other order reads a kilobyte at a stretch) */
+	const bool patches = !DIVS && VEC > 1 && NC == FEW_COLUMNS && g.N % 32 == 0 && g.OA % PATCH_A == 0 && g.OB % PATCH_B == 0 &&
+			(size_t) g.NS * g.LH * g.LW * g.LC * sizeof(T) > ((size_t) 48 << 20);
+	int m, n, ya0, yb0;
+	bool mvalid;
+	if (patches) {
+		const int sbs = g.N / 32, pas = g.OA / PATCH_A;
+		const int patch = block / sbs, pb_i = patch / pas, pos = lane / LPS;
+		const int a = (patch - pb_i * pas) * PATCH_A + pos % PATCH_A, b = pb_i * PATCH_B + pos / PATCH_A;
+		n = (block - patch * sbs) * 32 + (lane % LPS) * VEC;
+		m = n + g.N * (a + g.OA * b);
+		mvalid = b < g.OB;                       /* (blocks past the last one: the grid is rounded up) */
+		ya0 = a * g.SA + g.PA;
+		yb0 = b * g.SB + g.PB;
+	} else {
+		m = block * ROWS + lane * VEC;
+		mvalid = m < g.M;                        /* whole vectors: M is a multiple of VEC */
 		n = m % g.N;
 		const int t = m / g.N;
 		const int a = t % g.OA, b = t / g.OA;
@@ -1664,7 +1685,14 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 		/* the source channels are dealt over the waves; a tap that reaches none of a wavefront's rows (zero padding, or a
 		 * stride that does not divide: its rows share an output position or a few) is skipped whole */
 		const int per = (g.LC + WAVES - 1) / WAVES;
-		const int c0 = wave * per, c1 = min(g.LC, c0 + per);
+		const int w0 = wave * per, w1 = min(g.LC, w0 + per);
+		/* With patches, whole batches of channels outermost and the taps inside: what a tap's loads bring into the caches
+		 * is what the next taps of the same channels read at the neighbouring positions, a few kilobytes later instead
+		 * of after all of the wave's channels. Otherwise (and for a share that is not whole batches) tap by tap over all
+		 * of the wave's channels: the per-tap arithmetic once. */
+		const int group = patches && per % LOADS_IN_FLIGHT == 0 ? LOADS_IN_FLIGHT : max(per, 1);
+		for (int c0 = w0; c0 < w1; c0 += group) {
+		const int c1 = min(w1, c0 + group);
 		for (int sb = 0; sb < g.S; ++sb)
 			for (int r = 0; r < g.R; ++r) {
 				int ya = ya0 + r * g.RA, yb = yb0 + sb * g.RB;
@@ -1704,6 +1732,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 					w += wstep;
 				}
 			}
+		}
 	}
 	__shared__ T red[WAVES - 1][NC][ROWS];
 	if (wave > 0) {

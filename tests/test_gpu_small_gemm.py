@@ -275,3 +275,26 @@ def test_five_to_eight_columns_without_matrix_tiles(case, dtype):
     assert hp.rel_err(dx, dx_ref, label=label + " dx") < tol
     assert hp.rel_err(wp.get_grad(), dw_ref, label=label + " dw") < tol
     assert hp.rel_err(bp.get_grad(), db_ref.reshape(1, -1), label=label + " db") < tol
+
+
+@pytest.mark.parametrize("case", [(np.float32, 32, 64, 100, 64, 3), (np.float64, 32, 64, 64, 52, 2), (np.float32, 64, 48, 40, 136, 4)],
+                         ids=["f32-3", "f64-2", "f32-4"])
+def test_few_columns_over_a_large_source(case):
+    """A convolution to a few channels whose source is larger than the L2 caches together (the last layer of an image
+    decoder) deals its blocks over patches of output positions instead of runs of samples; padding, patch borders and the
+    blocks past the last patch must come out as in the plain order. Forward pass against the oracle."""
+    dtype, N, H, W, C, F = case
+    geom = dict(RH=3, RW=3, pv=1, ph=1, sv=1, sh=1, dv=0, dh=0)
+    gen = hp.rng(1900 + C + F)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (9 * C, F), dtype, std=1.0 / np.sqrt(9 * C))
+    b = hp.normal(gen, (1, F), dtype)
+    assert x.nbytes > 48 << 20
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F, 3, 3, 1, 1, 1, 1, 0, 0)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    out = layer.pass_forward(ch.DeviceTensor.from_host(x), False).to_host()
+    ref = oracle.conv_forward(np.asarray(x, np.float64), np.asarray(w, np.float64), np.asarray(b, np.float64), **geom)
+    tol = 1e-4 if dtype == np.float32 else 1e-10
+    assert hp.rel_err(out, ref, label="few columns, large source %s" % "-".join(str(v) for v in case[1:])) < tol
