@@ -1804,6 +1804,113 @@ void few_columns_with_wgrad_kernel(const T* __restrict__ src, const T* __restric
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * The weight gradient of a convolution with up to four filters (the last layer of an image decoder: many channels in, an
+ * image out), dW[K x F] = patches(x)^T [K x M] * G[M x F], without matrix tiles: a 32 x 32 tile would be seven eighths
+ * padding along F and the matrix pipes would spend the kernel's time on zeros (114 us for K = 576, F = 3 over 262,144
+ * rows). A wavefront owns one source channel and a lane VEC consecutive rows m (samples of one output position): per
+ * row vector it loads the F gradient vectors once and the channel's value at each of the TAPS receptor positions, and
+ * adds their products into TAPS x F sums of its own; the sums of a slice of M are then added over the 64 lanes (a
+ * butterfly of lane exchanges, so every run adds in the same order) and written as the slice's partial [k + K f], k = tap +
+ * taps * channel, like the partials of wgrad_body, for the same launch to add. The column sums of G (the bias gradient)
+ * come from the first wavefront of every slice. grid = (channels / 4 rounded up, slices).
+ * ---------------------------------------------------------------------------------------------- */
+template<typename T, int VEC, int MAXT>
+__global__ __launch_bounds__(256)
+void few_filters_wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
+		T* __restrict__ bias_partials, const GatherGeom g, int splits, int direct) {
+	constexpr int NC = FEW_COLUMNS, ROWS = 64 * VEC;
+	const int lane = threadIdx.x % 64;
+	const int wave = __builtin_amdgcn_readfirstlane((int) threadIdx.x / 64);
+	const int ch = (int) blockIdx.x * 4 + wave, split = (int) blockIdx.y;
+	const int taps = g.R * g.S;
+	const bool sums_bias = blockIdx.x == 0 && wave == 0 && bias_partials != nullptr;
+	if (ch >= g.LC)
+		return;                                  /* (no barrier below) */
+	const int total = (g.M + ROWS - 1) / ROWS, per = (total + splits - 1) / splits;
+	const int it0 = split * per, it1 = min(total, it0 + per);
+	/* the displacement of receptor position t along both axes (wave-uniform, kept in scalar registers) */
+	int dya[MAXT], dyb[MAXT];
+	#pragma unroll
+	for (int t = 0; t < MAXT; ++t) {
+		const int tt = min(t, taps - 1);
+		dya[t] = (tt % g.R) * g.RA;
+		dyb[t] = (tt / g.R) * g.RB;
+	}
+	T acc[MAXT][NC], bacc[NC];
+	#pragma unroll
+	for (int t = 0; t < MAXT; ++t)
+		#pragma unroll
+		for (int f = 0; f < NC; ++f)
+			acc[t][f] = (T) 0;
+	#pragma unroll
+	for (int f = 0; f < NC; ++f)
+		bacc[f] = (T) 0;
+	const T* const zeros = reinterpret_cast<const T*>(g_zero_block);
+	const T* const plane = src + (size_t) g.NS * g.LH * g.LW * ch;
+	for (int it = it0; it < it1; ++it) {
+		const int m = it * ROWS + lane * VEC;
+		const bool valid = m < g.M;              /* whole vectors: M is a multiple of VEC */
+		const int n = m % g.N, pos = m / g.N;
+		const int a = pos % g.OA, b = pos / g.OA;
+		const int ya0 = a * g.SA + g.PA, yb0 = b * g.SB + g.PB;
+		T gv[NC][VEC], xv[MAXT][VEC];
+		#pragma unroll
+		for (int f = 0; f < NC; ++f)
+			vec_load_global<T, VEC>(gv[f], valid && f < g.F ? og + ((size_t) m + (size_t) g.M * f) : zeros);
+		#pragma unroll
+		for (int t = 0; t < MAXT; ++t) {
+			const int ya = ya0 + dya[t], yb = yb0 + dyb[t];
+			const bool ok = valid && t < taps && (unsigned) ya < (unsigned) g.LH && (unsigned) yb < (unsigned) g.LW;
+			vec_load_global<T, VEC>(xv[t], ok ? plane + (n + g.NS * (ya + g.LH * yb)) : zeros);
+		}
+		#pragma unroll
+		for (int t = 0; t < MAXT; ++t)
+			#pragma unroll
+			for (int f = 0; f < NC; ++f)
+				#pragma unroll
+				for (int i = 0; i < VEC; ++i)
+					acc[t][f] += xv[t][i] * gv[f][i];
+		if (sums_bias) {
+			#pragma unroll
+			for (int f = 0; f < NC; ++f)
+				#pragma unroll
+				for (int i = 0; i < VEC; ++i)
+					bacc[f] += gv[f][i];
+		}
+	}
+	/* the lanes' sums: a butterfly, after which every lane holds the total */
+	#pragma unroll
+	for (int off = 32; off >= 1; off >>= 1) {
+		#pragma unroll
+		for (int t = 0; t < MAXT; ++t)
+			#pragma unroll
+			for (int f = 0; f < NC; ++f)
+				acc[t][f] += __shfl_xor(acc[t][f], off, 64);
+		#pragma unroll
+		for (int f = 0; f < NC; ++f)
+			bacc[f] += __shfl_xor(bacc[f], off, 64);
+	}
+	/* lane t * NC + f writes sum (t, f) */
+	T* dst = partials + (size_t) split * ((size_t) g.K * g.F);
+	#pragma unroll
+	for (int t = 0; t < MAXT; ++t)
+		#pragma unroll
+		for (int f = 0; f < NC; ++f)
+			if (lane == (t * NC + f) % 64 && t < taps && f < g.F) {
+				T* o = dst + ((size_t) (t + taps * ch) + (size_t) g.K * f);
+				*o = direct ? *o + acc[t][f] : acc[t][f];
+			}
+	if (sums_bias) {
+		#pragma unroll
+		for (int f = 0; f < NC; ++f)
+			if (lane == f && f < g.F) {
+				T* o = bias_partials + ((size_t) split * g.F + f);
+				*o = direct ? *o + bacc[f] : bacc[f];
+			}
+	}
+}
+
+/* ------------------------------------------------------------------------------------------------
  * The same product for problems with far fewer output tiles than the chip has wavefront slots, as one launch without
  * partial sums in memory: a block owns one TL x TL tile of the result (one matrix-instruction tile) and its WAVES
  * wavefronts each take a contiguous share of the reduction; their partial tiles meet in LDS and are added in ascending
@@ -3180,14 +3287,32 @@ void conv_weight_gradient_with(const ConvShape& s, int N, const T* x, const T* o
 			(reinterpret_cast<uintptr_t>(out_grad) & 15) == 0 &&
 			(!act || ((reinterpret_cast<uintptr_t>(act->y) & 15) == 0 && (reinterpret_cast<uintptr_t>(act->dz) & 15) == 0 &&
 					(reinterpret_cast<uintptr_t>(act->pool_inds) & 15) == 0));
-	const WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N, vec);
+	WgradPlan p = wgrad_plan<T>(g.M, g.K, g.F, N, vec);
 	const WgradVariant<T>& v = WgradVariants<T>::get()[p.variant];
 	const size_t count = (size_t) g.K * g.F;
+	/* up to four filters over a long M: no matrix tiles (few_filters_wgrad_kernel). Its blocks are four source channels
+	 * by a slice of M; slices so that the chip holds four of its wavefronts per SIMD and a wavefront still walks four
+	 * row vectors or more before it adds up its lanes - never more than the plan's, whose partials the caller has room for. */
+	const int taps = g.R * g.S;
+	const bool few_filters = !act && vec && g.F <= FEW_COLUMNS && taps <= 16 && (long) g.M * g.K >= (16L << 20);
+	if (few_filters) {
+		const int channel_blocks = (g.LC + 3) / 4, row_vectors = (g.M + 64 * GemmCfg<T>::VEC - 1) / (64 * GemmCfg<T>::VEC);
+		p.splits = std::max(1, std::min(p.splits, std::min(device_shape().cus * 4 / channel_blocks, row_vectors / 4)));
+	}
 	T* bias_partials = partials + (size_t) p.splits * count;
 	static_assert(WGRAD_MC == 32, "the chunk length gather_with_wgrad_kernel is built with");
 	const bool can_ride = elsewhere != nullptr && std::is_same<T, float>::value && !act && vec && v.bk == 32 && v.bf == 32 &&
 			v.waves == 1 && v.mc == WGRAD_MC;
 	auto run = [&](T* to_w, T* to_b, const WgradSplit& how) {
+		if (few_filters) {
+			const dim3 grid((unsigned) ((g.LC + 3) / 4), (unsigned) how.splits);
+			if (taps <= 9)
+				few_filters_wgrad_kernel<T, GemmCfg<T>::VEC, 9><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
+			else
+				few_filters_wgrad_kernel<T, GemmCfg<T>::VEC, 16><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
+			CATTLE_HIP_CHECK(hipGetLastError());
+			return;
+		}
 		if (can_ride) {
 			WgradRider<T> rider = { x, out_grad, to_w, to_b, g, how, false };
 			if ((*elsewhere)(rider))

@@ -298,3 +298,38 @@ def test_few_columns_over_a_large_source(case):
     ref = oracle.conv_forward(np.asarray(x, np.float64), np.asarray(w, np.float64), np.asarray(b, np.float64), **geom)
     tol = 1e-4 if dtype == np.float32 else 1e-10
     assert hp.rel_err(out, ref, label="few columns, large source %s" % "-".join(str(v) for v in case[1:])) < tol
+
+
+@pytest.mark.parametrize("case", [(np.float32, 32, 32, 32, 64, 3, 3, 1, 1, 0), (np.float32, 24, 40, 36, 30, 4, 4, 2, 1, 0),
+                                  (np.float64, 32, 32, 32, 66, 2, 3, 1, 1, 0), (np.float32, 128, 33, 33, 64, 3, 3, 1, 2, 0),
+                                  (np.float32, 64, 30, 30, 40, 1, 3, 2, 1, 1), (np.float32, 20, 48, 48, 64, 3, 3, 1, 1, 0)],
+                         ids=lambda c: "-".join(str(v) for v in c[1:]))
+def test_weight_gradient_of_few_filters(case):
+    """The weight and bias gradients of a convolution with up to four filters over many rows (no matrix tiles: a wavefront
+    per source channel, sums over lanes at the end of a slice): 3 x 3 and 4 x 4 receptors, a channel count that leaves the
+    last block partly empty, stride and dilation, both precisions, and two passes whose gradients accumulate. All three
+    gradients against the oracle."""
+    dtype, N, H, W, C, F, R, pad, stride, dil = case
+    geom = dict(RH=R, RW=R, pv=pad, ph=pad, sv=stride, sh=stride, dv=dil, dh=dil)
+    gen = hp.rng(2000 + C + F + R)
+    x = hp.normal(gen, (N, H, W, C), dtype)
+    w = hp.normal(gen, (R * R * C, F), dtype, std=1.0 / np.sqrt(R * R * C))
+    b = hp.normal(gen, (1, F), dtype)
+    OH, OW = hp.conv_dims(H, W, R, R, pad, pad, stride, stride, dil, dil)
+    assert N * OH * OW * R * R * C >= 16 << 20
+    g = hp.normal(gen, (N, OH, OW, F), dtype)
+    layer = ch.ConvKernelLayer(dtype, (H, W, C), F, R, R, pad, pad, stride, stride, dil, dil)
+    wp, bp = layer.get_params()
+    wp.set_values(w)
+    bp.set_values(b)
+    for _ in range(2):                      # gradients accumulate until they are reset
+        layer.pass_forward(ch.DeviceTensor.from_host(x), True)
+        dx = layer.pass_back(ch.DeviceTensor.from_host(g)).to_host()
+    x64, w64, b64, g64 = (np.asarray(a, np.float64) for a in (x, w, b, g))
+    o_ref, cache = oracle.conv_forward(x64, w64, b64, return_cache=True, **geom)
+    dx_ref, dw_ref, db_ref = oracle.conv_backward(x.shape, cache, w64, g64, **geom)
+    tol = 1e-4 if dtype == np.float32 else 1e-10
+    label = "few filters %s" % "-".join(str(v) for v in case[1:])
+    assert hp.rel_err(dx, dx_ref, label=label + " dx") < tol
+    assert hp.rel_err(wp.get_grad(), 2 * dw_ref, label=label + " dw") < tol
+    assert hp.rel_err(bp.get_grad(), 2 * db_ref.reshape(1, -1), label=label + " db") < tol
