@@ -2583,6 +2583,12 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		if (blocks >= device_shape().cus && blocks * 2 <= 3 * device_shape().cus)
 			best_v = 1;
 	}
+	/* (the same one step further down: 86,400 x 216 x 48 on 338 tiles of 256 x 64, 46.6 us; on 676 of 256 x 32, 36.4) */
+	if (best_v == 1 && vars[2].bm == vars[1].bm && vars[1].bf > vars[2].bf && g.F > vars[2].bf) {
+		const long blocks = (long) ((g.M + vars[1].bm - 1) / vars[1].bm) * ((g.F + vars[1].bf - 1) / vars[1].bf);
+		if (blocks >= device_shape().cus && blocks * 2 <= 3 * device_shape().cus)
+			best_v = 2;
+	}
 	/* Too few tiles of that shape to give every CU one: a narrower tile of the same height first, if that does and the
 	 * reduction is short. Such a launch is one round of blocks whose time is latency, so two half-width blocks on a CU
 	 * overlap each other's waits (50,176 x 576 x 128: 109 -> 96 us), while with a long reduction the matrix pipes are
