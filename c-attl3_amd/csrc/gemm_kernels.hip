@@ -1594,7 +1594,7 @@ void* g_scratch_ptr[MAX_DEVICES] = { nullptr };
 constexpr int FEW_COLUMNS = 4, SOME_COLUMNS = 8;
 template<typename T, int VEC, bool DIVS, int UNROLL, int NC = FEW_COLUMNS>
 __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom& g, int block) {
+		T* __restrict__ out, const GatherGeom& g, int block, int act_kind = -1, T act_p = (T) 0, T* __restrict__ act_pre = nullptr) {
 	constexpr int WAVES = 4, ROWS = 64 * VEC;
 	const int lane = threadIdx.x % 64;
 	const int wave = __builtin_amdgcn_readfirstlane((int) threadIdx.x / 64);
@@ -1757,9 +1757,27 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 				#pragma unroll
 				for (int i = 0; i < VEC; ++i)
 					acc[c][i] += bv;
-				vec_store<T, VEC>(out + (out_row(g, m) + (size_t) g.out_M * c), acc[c]);
+				if (act_kind < 0)
+					vec_store<T, VEC>(out + (out_row(g, m) + (size_t) g.out_M * c), acc[c]);
 			}
 		}
+		/* an element-wise activation on the way out (the fused forward pass of a kernel layer and its activation: coded
+		 * outputs, and the inputs too where the backward pass needs them; 16-byte accesses, plain output map) */
+		if (act_kind >= 0)
+			act_dispatch(act_kind, [&](auto kc) {
+				#pragma unroll
+				for (int c = 0; c < NC; ++c)
+					if (c < g.F) {
+						T y[VEC];
+						#pragma unroll
+						for (int i = 0; i < VEC; ++i)
+							y[i] = act_f_coded<T, decltype(kc)::value>(acc[c][i], act_p);
+						const size_t o = (size_t) m + (size_t) g.M * c;
+						vec_store_stream<T, VEC>(out + o, y);
+						if (act_pre)
+							vec_store_stream<T, VEC>(act_pre + o, acc[c]);
+					}
+			});
 	}
 }
 
@@ -1781,8 +1799,8 @@ void few_columns_gather_kernel(const T* __restrict__ src, const T* __restrict__ 
 template<typename T, int VEC, int UNROLL, int NC = FEW_COLUMNS>
 __global__ __launch_bounds__(256)
 void few_columns_plain_kernel(const T* __restrict__ src, const T* __restrict__ wt, const T* __restrict__ bias,
-		T* __restrict__ out, const GatherGeom g) {
-	few_columns_body<T, VEC, false, UNROLL, NC>(src, wt, bias, out, g, few_columns_block<VEC>(g, (int) blockIdx.x));
+		T* __restrict__ out, const GatherGeom g, int act_kind, T act_p, T* __restrict__ act_pre) {
+	few_columns_body<T, VEC, false, UNROLL, NC>(src, wt, bias, out, g, few_columns_block<VEC>(g, (int) blockIdx.x), act_kind, act_p, act_pre);
 }
 
 /* An input gradient of a few columns and the layer's weight gradient in one launch (see gather_with_wgrad_kernel: both
@@ -2528,7 +2546,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 	/* 16-byte loads wherever alignment allows, even where they leave a SIMD a wave or two: measured, a quarter of
 	 * the load instructions beats four times the waves (9 against 19 us on a 200,704 x 48 x 1 problem) */
 	const bool wide = vec && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
-	if (epi == EPI_NONE && then == nullptr && (g.F <= FEW_COLUMNS || (g.F <= SOME_COLUMNS && wide && !divs))) {
+	if ((epi == EPI_NONE || epi == EPI_ACT) && then == nullptr && (g.F <= FEW_COLUMNS || (g.F <= SOME_COLUMNS && wide && !divs))) {
 		/* a handful of output columns: no matrix tiles (few_columns_gather_kernel); five to eight of them in the
 		 * vectorised forward form only */
 		constexpr int V = GemmCfg<T>::VEC;
@@ -2543,11 +2561,17 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 				else if (walk == 8) KERNEL<T, V, 8> __VA_ARGS__; \
 				else KERNEL<T, V, 4> __VA_ARGS__; \
 			} while (0)
+		/* the activation epilogue (it comes with 16-byte accesses and without divisors, see above) */
+		const int act_kind = epi == EPI_ACT ? E->kind : -1;
+		const T act_p = epi == EPI_ACT ? E->p : (T) 0;
+		T* const act_pre = epi == EPI_ACT ? E->pre : nullptr;
+		if (epi == EPI_ACT && (reinterpret_cast<uintptr_t>(act_pre) & 15) != 0)
+			return false;
 		if (g.F > FEW_COLUMNS) {
-			if (walk == 0) few_columns_plain_kernel<T, V, 0, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
-			else if (walk == 8) few_columns_plain_kernel<T, V, 8, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
-			else few_columns_plain_kernel<T, V, 4, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
-		} else if (rider && wide && !divs && bias == nullptr) {
+			if (walk == 0) few_columns_plain_kernel<T, V, 0, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre);
+			else if (walk == 8) few_columns_plain_kernel<T, V, 8, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre);
+			else few_columns_plain_kernel<T, V, 4, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre);
+		} else if (epi == EPI_NONE && rider && wide && !divs && bias == nullptr) {
 			const unsigned w_blocks = (unsigned) round_up(rider->plan.tiles * rider->plan.splits, 8);
 			CATTLE_HIP_FEW_COLUMNS(few_columns_with_wgrad_kernel, <<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks,
 					rider->x, rider->og, rider->partials, rider->bias_partials, rider->g, rider->plan));
@@ -2555,7 +2579,7 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		} else if (wide && divs)
 			few_columns_gather_kernel<T, V, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else if (wide)
-			CATTLE_HIP_FEW_COLUMNS(few_columns_plain_kernel, <<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g));
+			CATTLE_HIP_FEW_COLUMNS(few_columns_plain_kernel, <<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre));
 		else if (divs)
 			few_columns_gather_kernel<T, 1, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else

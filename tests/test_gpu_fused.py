@@ -638,6 +638,36 @@ def test_first_layer_weight_gradient_with_ragged_batches(N, dtype):
     assert hp.rel_err(runs[1][0], ref["dw"], label="first layer N=%d %s dw" % (N, np.dtype(dtype).name)) < tol
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("F", [1, 3, 4, 6, 8])
+@pytest.mark.parametrize("act", [("tanh", 0.0), ("sigmoid", 0.0), ("relu", 0.0), ("leaky_relu", 0.125), ("softplus", 0.0)],
+                         ids=lambda a: a[0])
+def test_fused_activation_behind_a_few_filters(act, F, dtype):
+    """A kernel layer with one to eight filters and its activation as one fused layer (the output layer of an image decoder):
+    the product runs without matrix tiles and applies the activation as it stores. Forward and all gradients against the
+    oracle's layers behind one another."""
+    N, H, W, C = 16, 12, 10, 24
+    fused, members, kdims = _build(dtype, N, H, W, C, F, conv=GEOM_3X3, act=act)
+    chain = Chain(GEOM_3X3, act=act)
+    gen = hp.rng(300 + F)
+    x = hp.uniform(gen, (N, H, W, C), -1, 1, dtype)
+    w = hp.uniform(gen, (9 * C, F), -0.3, 0.3, dtype)
+    b = hp.uniform(gen, (1, F), -0.5, 0.5, dtype)
+    x64, w64, b64 = (np.asarray(a, np.float64) for a in (x, w, b))
+    ref = chain.forward(x64, w64, b64)
+    g = hp.uniform(gen, ref.shape, -1, 1, dtype)
+    out, dx, mode = _run_fused(fused, members, x, w, b, g)
+    assert mode == "act"
+    tol = TOL[np.dtype(dtype)]
+    label = "fused %s behind %d filters %s" % (act[0], F, np.dtype(dtype).name)
+    assert hp.rel_err(out, ref, label=label + " forward") < tol
+    grads = chain.backward(x64, w64, np.asarray(g, np.float64), pre_act=_pre_act_at_device_sides(chain, out, None, dtype))
+    wp, bp = members["conv"].get_params()
+    assert hp.rel_err(dx, grads["dx"], label=label + " dx") < tol
+    assert hp.rel_err(wp.get_grad(), grads["dw"], label=label + " dw") < tol
+    assert hp.rel_err(bp.get_grad(), grads["db"].reshape(1, -1), label=label + " db") < tol
+
+
 # ---- a seeded sweep of fused groups over geometries nobody chose by hand ------------------------------------------------
 
 def _sweep_cases(count, seed):
