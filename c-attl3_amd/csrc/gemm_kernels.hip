@@ -1607,7 +1607,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 	/* (where fetches rather than arithmetic bound the kernel: up to four columns, and a source that the L2 caches
 	 * together do not hold - with eight columns, or a source of 17 and 42 MB, patches were 10-14 % slower: their loads
 	 * are 128-byte pieces where the other order reads a kilobyte at a stretch) */
-	const bool patches = !DIVS && VEC > 1 && NC == FEW_COLUMNS && g.N % 32 == 0 && g.OA % PATCH_A == 0 && g.OB % PATCH_B == 0 &&
+	const bool patches = !DIVS && VEC > 1 && NC <= FEW_COLUMNS && g.N % 32 == 0 && g.OA % PATCH_A == 0 && g.OB % PATCH_B == 0 &&
 			(size_t) g.NS * g.LH * g.LW * g.LC * sizeof(T) > ((size_t) 48 << 20);
 	int m, n, ya0, yb0;
 	bool mvalid;
@@ -1630,6 +1630,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 		yb0 = b * g.SB + g.PB;
 	}
 	constexpr int LOADS_IN_FLIGHT = UNROLL > 0 ? UNROLL : 1;
+	constexpr int WL = NC == 3 ? 4 : NC;     /* a reduction row's weights are loaded as one, two, four or eight values */
 	const int plane = g.NS * g.LH * g.LW;
 	const int taps = g.R * g.S;
 	T acc[NC][VEC];
@@ -1654,7 +1655,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 		const T* const zeros = reinterpret_cast<const T*>(g_zero_block);
 		const int base = n + g.NS * (ya0 + g.LH * yb0);
 		for (int s = s0; s < s1; s += BATCH) {
-			T v[BATCH][VEC], wk[BATCH][NC];
+			T v[BATCH][VEC], wk[BATCH][WL];
 			#pragma unroll
 			for (int j = 0; j < BATCH; ++j) {
 				const bool live = s + j < s1;        /* wave-uniform */
@@ -1662,7 +1663,7 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 				const bool ok = mvalid && live && (unsigned) (ya0 + da) < (unsigned) g.LH && (unsigned) (yb0 + db) < (unsigned) g.LW;
 				vec_load_global<T, VEC>(v[j], ok ? src + (base + g.NS * (da + g.LH * db) + plane * ch) : zeros);
 				/* reduction row k = r + R (s + S ch); the prepared weights hold its F values (zero-padded) first in its row */
-				vec_load_global<T, NC>(wk[j], wt + (size_t) (live ? r + g.R * (sb + g.S * ch) : 0) * g.ldw);
+				vec_load_global<T, WL>(wk[j], wt + (size_t) (live ? r + g.R * (sb + g.S * ch) : 0) * g.ldw);
 				if (!live) {
 					#pragma unroll
 					for (int c = 0; c < NC; ++c)
@@ -1721,8 +1722,8 @@ __device__ __forceinline__ void few_columns_body(const T* __restrict__ src, cons
 						for (int i = 0; i < VEC; ++i)
 							v[i] = (T) 0;
 					}
-					T wk[NC];
-					vec_load_global<T, NC>(wk, w);
+					T wk[WL];
+					vec_load_global<T, WL>(wk, w);
 					#pragma unroll
 					for (int c = 0; c < NC; ++c)
 						#pragma unroll
@@ -1806,13 +1807,13 @@ void few_columns_plain_kernel(const T* __restrict__ src, const T* __restrict__ w
 /* An input gradient of a few columns and the layer's weight gradient in one launch (see gather_with_wgrad_kernel: both
  * wait for the same upstream gradient only, and a dependent launch costs 4-5 us however little it does): blocks below
  * gather_blocks form the input gradient, the others are the weight gradient's one-wavefront blocks. */
-template<typename T, int VEC, int UNROLL>
+template<typename T, int VEC, int UNROLL, int NC>
 __global__ __launch_bounds__(256)
 void few_columns_with_wgrad_kernel(const T* __restrict__ src, const T* __restrict__ wt, T* __restrict__ out, const GatherGeom g,
 		int gather_blocks, const T* __restrict__ w_src, const T* __restrict__ w_og, T* __restrict__ w_partials,
 		T* __restrict__ w_bias_partials, const GatherGeom w_g, const WgradSplit w_plan) {
 	if ((int) blockIdx.x < gather_blocks) {
-		few_columns_body<T, VEC, false, UNROLL>(src, wt, (const T*) nullptr, out, g, few_columns_block<VEC>(g, (int) blockIdx.x));
+		few_columns_body<T, VEC, false, UNROLL, NC>(src, wt, (const T*) nullptr, out, g, few_columns_block<VEC>(g, (int) blockIdx.x));
 	} else {
 		if (threadIdx.x >= 64)
 			return;
@@ -1832,11 +1833,11 @@ void few_columns_with_wgrad_kernel(const T* __restrict__ src, const T* __restric
  * taps * channel, like the partials of wgrad_body, for the same launch to add. The column sums of G (the bias gradient)
  * come from the first wavefront of every slice. grid = (channels / 4 rounded up, slices).
  * ---------------------------------------------------------------------------------------------- */
-template<typename T, int VEC, int MAXT>
+template<typename T, int VEC, int MAXT, int NC>
 __global__ __launch_bounds__(256)
 void few_filters_wgrad_kernel(const T* __restrict__ src, const T* __restrict__ og, T* __restrict__ partials,
 		T* __restrict__ bias_partials, const GatherGeom g, int splits, int direct) {
-	constexpr int NC = FEW_COLUMNS, ROWS = 64 * VEC;
+	constexpr int ROWS = 64 * VEC;            /* (NC: accumulators per receptor position, three for an image's, else four) */
 	const int lane = threadIdx.x % 64;
 	const int wave = __builtin_amdgcn_readfirstlane((int) threadIdx.x / 64);
 	const int ch = (int) blockIdx.x * 4 + wave, split = (int) blockIdx.y;
@@ -2555,36 +2556,49 @@ bool launch_gather(const T* src, const T* wt, const T* bias, T* out, const Gathe
 		 * (0); else tap by tap with a wave's share of the channels in whole batches of loads, eight to a batch if that
 		 * divides the share, else four */
 		const int walk = !divs && wide && g.LC <= 8 ? 0 : ((g.LC + 3) / 4) % 8 == 0 ? 8 : 4;
-		#define CATTLE_HIP_FEW_COLUMNS(KERNEL, ...) \
-			do { \
-				if (walk == 0) KERNEL<T, V, 0> __VA_ARGS__; \
-				else if (walk == 8) KERNEL<T, V, 8> __VA_ARGS__; \
-				else KERNEL<T, V, 4> __VA_ARGS__; \
-			} while (0)
+		/* as many accumulators per row as there are columns, for the counts that images have (one, three), else four or
+		 * eight: a fourth accumulator for three columns is a third more multiply-adds */
+		const auto with_walk = [&](auto fn) {
+			if (walk == 0) fn(std::integral_constant<int, 0>());
+			else if (walk == 8) fn(std::integral_constant<int, 8>());
+			else fn(std::integral_constant<int, 4>());
+		};
+		const auto with_columns = [&](auto fn) {
+			if (g.F > FEW_COLUMNS) fn(std::integral_constant<int, SOME_COLUMNS>());
+			else if (g.F == 3) fn(std::integral_constant<int, 3>());
+			else if (g.F == 1) fn(std::integral_constant<int, 1>());
+			else fn(std::integral_constant<int, FEW_COLUMNS>());
+		};
 		/* the activation epilogue (it comes with 16-byte accesses and without divisors, see above) */
 		const int act_kind = epi == EPI_ACT ? E->kind : -1;
 		const T act_p = epi == EPI_ACT ? E->p : (T) 0;
 		T* const act_pre = epi == EPI_ACT ? E->pre : nullptr;
 		if (epi == EPI_ACT && (reinterpret_cast<uintptr_t>(act_pre) & 15) != 0)
 			return false;
-		if (g.F > FEW_COLUMNS) {
-			if (walk == 0) few_columns_plain_kernel<T, V, 0, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre);
-			else if (walk == 8) few_columns_plain_kernel<T, V, 8, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre);
-			else few_columns_plain_kernel<T, V, 4, SOME_COLUMNS><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre);
-		} else if (epi == EPI_NONE && rider && wide && !divs && bias == nullptr) {
+		if (epi == EPI_NONE && g.F <= FEW_COLUMNS && rider && wide && !divs && bias == nullptr) {
 			const unsigned w_blocks = (unsigned) round_up(rider->plan.tiles * rider->plan.splits, 8);
-			CATTLE_HIP_FEW_COLUMNS(few_columns_with_wgrad_kernel, <<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks,
-					rider->x, rider->og, rider->partials, rider->bias_partials, rider->g, rider->plan));
+			with_walk([&](auto w) {
+				if (g.F == 3)
+					few_columns_with_wgrad_kernel<T, V, decltype(w)::value, 3><<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g, (int) blocks,
+							rider->x, rider->og, rider->partials, rider->bias_partials, rider->g, rider->plan);
+				else
+					few_columns_with_wgrad_kernel<T, V, decltype(w)::value, FEW_COLUMNS><<<blocks + w_blocks, 256, 0, stream()>>>(src, wt, out, g,
+							(int) blocks, rider->x, rider->og, rider->partials, rider->bias_partials, rider->g, rider->plan);
+			});
 			rider->done = true;
 		} else if (wide && divs)
 			few_columns_gather_kernel<T, V, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else if (wide)
-			CATTLE_HIP_FEW_COLUMNS(few_columns_plain_kernel, <<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g, act_kind, act_p, act_pre));
+			with_walk([&](auto w) {
+				with_columns([&](auto c) {
+					few_columns_plain_kernel<T, V, decltype(w)::value, decltype(c)::value><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g,
+							act_kind, act_p, act_pre);
+				});
+			});
 		else if (divs)
 			few_columns_gather_kernel<T, 1, true, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
 		else
 			few_columns_gather_kernel<T, 1, false, 8><<<blocks, 256, 0, stream()>>>(src, wt, bias, out, g);
-		#undef CATTLE_HIP_FEW_COLUMNS
 		CATTLE_HIP_CHECK(hipGetLastError());
 		if (mtiles_out)
 			*mtiles_out = 0;
@@ -3336,10 +3350,15 @@ void conv_weight_gradient_with(const ConvShape& s, int N, const T* x, const T* o
 	auto run = [&](T* to_w, T* to_b, const WgradSplit& how) {
 		if (few_filters) {
 			const dim3 grid((unsigned) ((g.LC + 3) / 4), (unsigned) how.splits);
-			if (taps <= 9)
-				few_filters_wgrad_kernel<T, GemmCfg<T>::VEC, 9><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
+			constexpr int V = GemmCfg<T>::VEC;
+			if (taps <= 9 && g.F == 3)
+				few_filters_wgrad_kernel<T, V, 9, 3><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
+			else if (taps <= 9)
+				few_filters_wgrad_kernel<T, V, 9, FEW_COLUMNS><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
+			else if (g.F == 3)
+				few_filters_wgrad_kernel<T, V, 16, 3><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
 			else
-				few_filters_wgrad_kernel<T, GemmCfg<T>::VEC, 16><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
+				few_filters_wgrad_kernel<T, V, 16, FEW_COLUMNS><<<grid, 256, 0, stream()>>>(x, out_grad, to_w, to_b, g, how.splits, how.direct);
 			CATTLE_HIP_CHECK(hipGetLastError());
 			return;
 		}
